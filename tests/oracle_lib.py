@@ -1,0 +1,235 @@
+"""ctypes bindings for the CPU oracle (oracle/libsampler_oracle.so) and, where it has been built,
+the reference library driver (oracle/_ref/libref_sampler.so).  Test infrastructure only."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_SO = os.path.join(ORACLE_DIR, "libsampler_oracle.so")
+REF_SO = os.path.join(ORACLE_DIR, "_ref", "libref_sampler.so")
+
+STATUS_OK = 0
+STATUS_EMPTY_LOGITS = 1
+STATUS_BAD_TEMPERATURE = 2
+STATUS_BAD_TOP_P = 3
+STATUS_BAD_MIN_P = 4
+STATUS_NO_FINITE_LOGIT = 5
+STATUS_INVALID_DISTRIBUTION = 6
+
+STATUS_MESSAGES = {
+    STATUS_EMPTY_LOGITS: "cannot sample empty logits",
+    STATUS_BAD_TEMPERATURE: "temperature must be finite and non-negative",
+    STATUS_BAD_TOP_P: "top_p must be in the range (0, 1]",
+    STATUS_BAD_MIN_P: "min_p must be in the range [0, 1]",
+    STATUS_NO_FINITE_LOGIT: "sampling requires at least one finite logit",
+    STATUS_INVALID_DISTRIBUTION: "sampling distribution is invalid",
+}
+
+
+class SamplingOptions(ctypes.Structure):
+    _fields_ = [("temperature", ctypes.c_float), ("top_k", ctypes.c_uint32),
+                ("top_p", ctypes.c_float), ("min_p", ctypes.c_float)]
+
+
+ROW_PARAMS_DTYPE = np.dtype([("temperature", "<f4"), ("top_k", "<u4"), ("top_p", "<f4"),
+                             ("min_p", "<f4"), ("stop_begin", "<u4"), ("stop_count", "<u4")])
+
+ORACLE_RESULT_DTYPE = np.dtype([("token_id", "<i4"), ("probability", "<f4"), ("kept_count", "<u4"),
+                                ("status", "u1"), ("is_stop", "u1"), ("draw_consumed", "u1"),
+                                ("has_nan", "u1"), ("cdf_gap", "<f4"), ("top_p_gap", "<f4")])
+
+
+def build_oracle():
+    subprocess.run(["make", "-C", ORACLE_DIR, "oracle"], check=True, stdout=subprocess.DEVNULL)
+
+
+_oracle = None
+
+
+def oracle():
+    global _oracle
+    if _oracle is not None:
+        return _oracle
+    if not os.path.exists(ORACLE_SO):
+        build_oracle()
+    lib = ctypes.CDLL(ORACLE_SO)
+    f32p = ctypes.POINTER(ctypes.c_float)
+    lib.oracle_status_message.restype = ctypes.c_char_p
+    lib.oracle_status_message.argtypes = [ctypes.c_int]
+    lib.oracle_validate_sampling_options.argtypes = [ctypes.POINTER(SamplingOptions)]
+    lib.oracle_sampling_distribution.argtypes = [
+        ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(SamplingOptions),
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)]
+    lib.oracle_sample.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(SamplingOptions),
+                                  ctypes.c_float, ctypes.c_void_p]
+    lib.oracle_sample_batch.argtypes = [
+        ctypes.c_void_p, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64,
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+    lib.oracle_bfloat16_to_float.restype = ctypes.c_float
+    lib.oracle_bfloat16_to_float.argtypes = [ctypes.c_uint16]
+    lib.oracle_float_to_bfloat16.restype = ctypes.c_uint16
+    lib.oracle_float_to_bfloat16.argtypes = [ctypes.c_float]
+    lib.oracle_quantize_bfloat16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+    lib.oracle_rng_create.restype = ctypes.c_void_p
+    lib.oracle_rng_create.argtypes = [ctypes.c_uint64]
+    lib.oracle_rng_destroy.argtypes = [ctypes.c_void_p]
+    lib.oracle_rng_uniform.restype = ctypes.c_float
+    lib.oracle_rng_uniform.argtypes = [ctypes.c_void_p]
+    lib.oracle_expf_libm.restype = ctypes.c_float
+    lib.oracle_expf_libm.argtypes = [ctypes.c_float]
+    lib.oracle_expf_restated.restype = ctypes.c_float
+    lib.oracle_expf_restated.argtypes = [ctypes.c_float]
+    lib.oracle_expf_compare_range.restype = ctypes.c_uint64
+    lib.oracle_expf_compare_range.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
+    _oracle = lib
+    return lib
+
+
+def oracle_distribution(logits, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
+    """Returns (status, ids, probabilities) for one fp32 row."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    options = SamplingOptions(temperature, top_k, top_p, min_p)
+    cap = max(1, logits.size)
+    ids = np.empty(cap, dtype=np.int32)
+    probs = np.empty(cap, dtype=np.float32)
+    count = ctypes.c_size_t(0)
+    status = oracle().oracle_sampling_distribution(
+        logits.ctypes.data, logits.size, ctypes.byref(options),
+        ids.ctypes.data, probs.ctypes.data, cap, ctypes.byref(count))
+    return status, ids[:count.value].copy(), probs[:count.value].copy()
+
+
+def oracle_sample(logits, uniform, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
+    """Returns a 1-element ORACLE_RESULT_DTYPE record for one fp32 row."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    options = SamplingOptions(temperature, top_k, top_p, min_p)
+    result = np.zeros(1, dtype=ORACLE_RESULT_DTYPE)
+    oracle().oracle_sample(logits.ctypes.data, logits.size, ctypes.byref(options),
+                           ctypes.c_float(uniform), result.ctypes.data)
+    return result[0]
+
+
+def oracle_sample_batch(logits, params, uniforms, stop_ids=None, threads=1, vocab=None):
+    """logits: [rows, stride] float32 or uint16 (bf16 bits); params: ROW_PARAMS_DTYPE[rows]."""
+    logits = np.ascontiguousarray(logits)
+    assert logits.ndim == 2 and logits.dtype in (np.float32, np.uint16)
+    rows, stride = logits.shape
+    vocab = stride if vocab is None else vocab
+    params = np.ascontiguousarray(params, dtype=ROW_PARAMS_DTYPE)
+    uniforms = np.ascontiguousarray(uniforms, dtype=np.float32)
+    assert params.shape == (rows,) and uniforms.shape == (rows,)
+    stops = None if stop_ids is None else np.ascontiguousarray(stop_ids, dtype=np.int32)
+    results = np.zeros(rows, dtype=ORACLE_RESULT_DTYPE)
+    rc = oracle().oracle_sample_batch(
+        logits.ctypes.data, 0 if logits.dtype == np.float32 else 1, rows, vocab, stride,
+        params.ctypes.data, uniforms.ctypes.data,
+        None if stops is None else stops.ctypes.data, results.ctypes.data, threads)
+    assert rc == 0
+    return results
+
+
+def quantize_bf16(values):
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty(values.shape, dtype=np.uint16)
+    oracle().oracle_quantize_bfloat16(values.ctypes.data, out.ctypes.data, values.size)
+    return out
+
+
+def widen_bf16(bits):
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+class OracleRng:
+    """std::mt19937_64(seed) + std::uniform_real_distribution<float>(0, 1), one draw per call."""
+
+    def __init__(self, seed):
+        self._handle = oracle().oracle_rng_create(seed)
+
+    def uniform(self):
+        return float(oracle().oracle_rng_uniform(self._handle))
+
+    def __del__(self):
+        if getattr(self, "_handle", None):
+            oracle().oracle_rng_destroy(self._handle)
+            self._handle = None
+
+
+_ref = None
+
+
+def reference_available():
+    return os.path.exists(REF_SO)
+
+
+def reference():
+    """The reference library driver; only present where the reference checkout was built."""
+    global _ref
+    if _ref is not None:
+        return _ref
+    lib = ctypes.CDLL(REF_SO)
+    lib.ref_session_create.restype = ctypes.c_void_p
+    lib.ref_session_create.argtypes = [ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t]
+    lib.ref_session_destroy.argtypes = [ctypes.c_void_p]
+    lib.ref_session_sample.argtypes = [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_uint32,
+        ctypes.c_float, ctypes.c_float, ctypes.POINTER(ctypes.c_int32),
+        ctypes.POINTER(ctypes.c_float), ctypes.c_char_p, ctypes.c_size_t]
+    lib.ref_sampling_distribution.argtypes = [
+        ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_uint32, ctypes.c_float,
+        ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+        ctypes.POINTER(ctypes.c_size_t), ctypes.c_char_p, ctypes.c_size_t]
+    lib.ref_sample_rows.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_uint32, ctypes.c_uint32,
+                                                            ctypes.c_uint64] + [ctypes.c_void_p] * 11 + [ctypes.c_int]
+    lib.ref_bfloat16_to_float.restype = ctypes.c_float
+    lib.ref_bfloat16_to_float.argtypes = [ctypes.c_uint16]
+    lib.ref_float_to_bfloat16.restype = ctypes.c_uint16
+    lib.ref_float_to_bfloat16.argtypes = [ctypes.c_float]
+    _ref = lib
+    return lib
+
+
+class ReferenceSession:
+    """A real reference Session (seeded) whose sample() is called on arbitrary rows."""
+
+    def __init__(self, seed):
+        message = ctypes.create_string_buffer(256)
+        self._handle = reference().ref_session_create(seed, message, 256)
+        if not self._handle:
+            raise RuntimeError("reference session: " + message.value.decode())
+
+    @property
+    def handle(self):
+        return self._handle
+
+    def sample(self, logits, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
+        """Returns (error_code_plus_one_or_zero, token_id, probability, message)."""
+        logits = np.ascontiguousarray(logits, dtype=np.float32)
+        token = ctypes.c_int32(-1)
+        prob = ctypes.c_float(0.0)
+        message = ctypes.create_string_buffer(256)
+        rc = reference().ref_session_sample(
+            self._handle, logits.ctypes.data, logits.size, temperature, top_k, top_p, min_p,
+            ctypes.byref(token), ctypes.byref(prob), message, 256)
+        return rc, token.value, prob.value, message.value.decode()
+
+    def __del__(self):
+        if getattr(self, "_handle", None):
+            reference().ref_session_destroy(self._handle)
+            self._handle = None
+
+
+def reference_distribution(logits, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
+    """Returns (rc, ids, probabilities, message) from the reference's own sampling_distribution."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    cap = max(1, logits.size)
+    ids = np.empty(cap, dtype=np.int32)
+    probs = np.empty(cap, dtype=np.float32)
+    count = ctypes.c_size_t(0)
+    message = ctypes.create_string_buffer(256)
+    rc = reference().ref_sampling_distribution(
+        logits.ctypes.data, logits.size, temperature, top_k, top_p, min_p,
+        ids.ctypes.data, probs.ctypes.data, cap, ctypes.byref(count), message, 256)
+    return rc, ids[:count.value].copy(), probs[:count.value].copy(), message.value.decode()
