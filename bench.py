@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X generation sampler: sampled rows/s and HBM GB/s on the logits read.
+
+A step is one pass of the sampler (ncnn_moe_hip_sampler_sample_device, every kernel of the path) over
+one batch of synthetic logits that is already resident in HBM.  The workload is configuration 2 of
+BASELINE.json: B=64, V=151,936 fp32 logits N(0, 3^2) with 8 spikes at +12 per row, temperature 0.7,
+Top-K 20, Top-P 0.8.  Steps rotate over several distinct logits buffers whose total size exceeds the
+256 MB Infinity Cache, so the logits come from HBM and not from a cache warmed by the previous step.
+
+Prints ONE JSON line.  `roofline` prices the dominant kernel (the one HBM pass over the logits)
+against the 8 TB/s HBM peak using the algorithmic bytes of a launch and the average step time
+measured with HIP events on the launch stream.  `cpu_baseline` times the reference's own
+Session::sample loop (oracle/_ref, kind "reference") or, where that library is absent, the CPU
+oracle (kind "port") on the host cores, on the same rows.
+"""
+import argparse
+import ctypes
+import importlib.util
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PACKAGE_DIR = os.path.join(ROOT, "ncnn-moe-runtime_amd")
+HBM_PEAK_BYTES_PER_S = 8.0e12
+
+
+def load_package():
+    if "ncnn_moe_runtime_amd" in sys.modules:
+        return sys.modules["ncnn_moe_runtime_amd"]
+    spec = importlib.util.spec_from_file_location(
+        "ncnn_moe_runtime_amd", os.path.join(PACKAGE_DIR, "__init__.py"),
+        submodule_search_locations=[PACKAGE_DIR])
+    module = importlib.util.module_from_spec(spec)
+    sys.modules["ncnn_moe_runtime_amd"] = module
+    spec.loader.exec_module(module)
+    return module
+
+
+def algorithmic_bytes(rows, vocab, element_bytes):
+    """Logits read once, parameters (24 B) and uniform (4 B) in, result (16 B) out, per row."""
+    return rows * vocab * element_bytes + rows * (24 + 4) + rows * 16
+
+
+def cpu_baseline(workload, host_threads, sample_rows):
+    """Times the CPU sampler on the first sample_rows rows of the workload."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+
+    rows = min(sample_rows, workload["rows"])
+    logits = workload["logits"][:rows]
+    params = workload["params"][:rows]
+    uniforms = workload["uniforms"][:rows]
+    fp32 = logits if workload["dtype"] == "f32" else oracle_lib.widen_bf16(logits)
+    fp32 = np.ascontiguousarray(fp32, dtype=np.float32)
+
+    if oracle_lib.reference_available():
+        kind = "reference"
+        sessions = [oracle_lib.ReferenceSession(seed) for seed in range(rows)]
+        handles = (ctypes.c_void_p * rows)(*[s.handle for s in sessions])
+        temperature = np.ascontiguousarray(params["temperature"])
+        top_k = np.ascontiguousarray(params["top_k"])
+        top_p = np.ascontiguousarray(params["top_p"])
+        min_p = np.ascontiguousarray(params["min_p"])
+        stop_begin = np.ascontiguousarray(params["stop_begin"])
+        stop_count = np.ascontiguousarray(params["stop_count"])
+        stops = workload["stop_ids"]
+        tokens = np.zeros(rows, dtype=np.int32)
+        probabilities = np.zeros(rows, dtype=np.float32)
+        is_stop = np.zeros(rows, dtype=np.uint8)
+        status = np.zeros(rows, dtype=np.int32)
+
+        def run(threads):
+            oracle_lib.reference().ref_sample_rows(
+                handles, fp32.ctypes.data, rows, fp32.shape[1], fp32.shape[1],
+                temperature.ctypes.data, top_k.ctypes.data, top_p.ctypes.data, min_p.ctypes.data,
+                None if stops is None else stops.ctypes.data, stop_begin.ctypes.data, stop_count.ctypes.data,
+                tokens.ctypes.data, probabilities.ctypes.data, is_stop.ctypes.data, status.ctypes.data, threads)
+    else:
+        kind = "port"
+
+        def run(threads):
+            oracle_lib.oracle_sample_batch(fp32, params, uniforms, workload["stop_ids"], threads=threads)
+
+    def best_of(threads, repetitions):
+        best = float("inf")
+        for _ in range(repetitions):
+            start = time.perf_counter()
+            run(threads)
+            best = min(best, time.perf_counter() - start)
+        return best
+
+    single = best_of(1, 2)
+    multi = best_of(host_threads, 3) if host_threads > 1 else single
+    return {
+        "value": rows / multi,
+        "unit": "rows/s",
+        "cores": host_threads,
+        "kind": kind,
+        "sample": "%d rows of the benchmark batch, best of 3 passes on %d threads (one Session per row); "
+                  "1 thread: %.1f rows/s" % (rows, host_threads, rows / single),
+        "single_thread_value": rows / single,
+    }
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=2000)
+    parser.add_argument("--warmup", type=int, default=200)
+    parser.add_argument("--workload", default="cfg2_topk_topp")
+    parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
+    parser.add_argument("--cpu-rows", type=int, default=64)
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: every box of this build has one MI355X; run with --gpus 1")
+
+    load_package()
+    from ncnn_moe_runtime_amd import hip_sampler, workloads
+    import torch
+
+    if not torch.cuda.is_available() or hip_sampler.device_count() < 1:
+        sys.exit("bench.py needs a GPU: no HIP device is visible")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    workload = workloads.make_workload(args.workload)
+    rows, vocab = workload["rows"], workload["vocab"]
+    element_bytes = 4 if workload["dtype"] == "f32" else 2
+    dtype_code = hip_sampler.LOGITS_F32 if workload["dtype"] == "f32" else hip_sampler.LOGITS_BF16
+    batch_bytes = rows * vocab * element_bytes
+    buffers = args.buffers if args.buffers > 0 else max(2, -(-320 * 1024 * 1024 // batch_bytes))
+
+    # buffer 0 holds the seeded host workload (checked against the oracle); the others hold rows of the
+    # same distribution generated on the device, so that consecutive steps read different HBM lines
+    host_logits = torch.from_numpy(workload["logits"].view(np.int16) if element_bytes == 2 else workload["logits"])
+    logits = [host_logits.to(device)]
+    generator = torch.Generator(device=device)
+    generator.manual_seed(1234)
+    for _ in range(buffers - 1):
+        permutation = torch.randperm(vocab, device=device, generator=generator)
+        logits.append(logits[0][:, permutation].contiguous())
+    params = torch.from_numpy(workload["params"].view(np.uint8).reshape(rows, -1)).to(device)
+    uniforms = torch.from_numpy(workload["uniforms"]).to(device)
+    stop_ids = None if workload["stop_ids"] is None else torch.from_numpy(workload["stop_ids"]).to(device)
+    results = torch.zeros((rows, 16), dtype=torch.uint8, device=device)
+
+    sampler = hip_sampler.HipSampler(rows, vocab)
+    stream = torch.cuda.Stream(device=device)
+    stream_pointer = stream.cuda_stream
+
+    def step(index):
+        sampler.sample_device(
+            logits[index % buffers].data_ptr(), dtype_code, rows, vocab, vocab,
+            params.data_ptr(), uniforms.data_ptr(), None if stop_ids is None else stop_ids.data_ptr(),
+            results.data_ptr(), stream_pointer)
+
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        # parity of the measured path on buffer 0 against the CPU oracle
+        step(0)
+        stream.synchronize()
+        gpu = results.cpu().numpy().view(hip_sampler.RESULT_DTYPE).reshape(rows)
+        for index in range(args.warmup):
+            step(index)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        start_event = torch.cuda.Event(enable_timing=True)
+        stop_event = torch.cuda.Event(enable_timing=True)
+        wall_start = time.perf_counter()
+        start_event.record(stream)
+        for index in range(args.steps):
+            step(index)
+        stop_event.record(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        wall_seconds = time.perf_counter() - wall_start
+    event_seconds = start_event.elapsed_time(stop_event) * 1e-3
+    seconds_per_step = event_seconds / args.steps
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+    import parity_util
+    host_threads = min(16, os.cpu_count() or 1)
+    cpu = oracle_lib.oracle_sample_batch(workload["logits"], workload["params"], workload["uniforms"],
+                                         workload["stop_ids"], threads=host_threads)
+    parity = parity_util.parity_counters(gpu, cpu)
+    parity["status_mismatches"] = int(np.count_nonzero(gpu["status"] != cpu["status"]))
+    parity["kept_count_mismatches"] = int(np.count_nonzero(gpu["kept_count"] != cpu["kept_count"]))
+
+    bytes_per_launch = algorithmic_bytes(rows, vocab, element_bytes)
+    achieved = bytes_per_launch / seconds_per_step
+    line = {
+        "metric": "sampled rows/sec + HBM GB/s (% peak), B=64 V=151936 fp32 temp+topk+topp",
+        "value": rows / seconds_per_step,
+        "unit": "rows/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": seconds_per_step * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if element_bytes == 4 else "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": workload["description"],
+            "name": workload["name"],
+            "rows": rows,
+            "vocab": vocab,
+            "logits_buffers_rotated": buffers,
+            "logits_bytes_per_step": batch_bytes,
+            "entry_point": "ncnn_moe_hip_sampler_sample_device",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved / 1e9,
+            "peak": HBM_PEAK_BYTES_PER_S / 1e9,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_BYTES_PER_S,
+            "traffic": None,
+            "kernel": "scan_select_kernel",
+            "algorithmic_bytes_per_launch": bytes_per_launch,
+        },
+        "parity": parity,
+        "wall_ms_per_step": wall_seconds / args.steps * 1e3,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(workload, host_threads, args.cpu_rows)
+    sampler.close()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

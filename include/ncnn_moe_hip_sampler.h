@@ -1,0 +1,160 @@
+/*
+ * C ABI of the MI355X (gfx950) generation sampler.
+ *
+ * This is the boundary a maintainer of the runtime binds from src/backends/hip: plain pointers and
+ * sizes, POD structs, no exceptions.  One handle serves one device; a handle is not re-entrant
+ * (use one handle per scheduler worker, or serialise calls), matching the per-Session mutex of the
+ * CPU sampler (src/engine/session.cpp:452-456).
+ *
+ * The sampler computes, per row of a [rows, vocab] logits matrix, exactly what the CPU path
+ * Session::sample computes for one Session (src/engine/session.cpp:393-443, :76-136): option
+ * validation, greedy argmax over finite logits, or the stable (logit descending, index ascending)
+ * ordering, Top-K, softmax in that order with sequential fp32 sums, Min-P, Top-P, renormalisation
+ * and the inverse-CDF draw, plus the stop-token test of the callers
+ * (src/engine/session.cpp:60-63, examples/internal/run_model.cpp:790).  The uniform draw is
+ * supplied per row by the caller, which owns the Session RNG (include/ncnn/moe/session.h:303).
+ */
+#ifndef NCNN_MOE_HIP_SAMPLER_H
+#define NCNN_MOE_HIP_SAMPLER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ncnn_moe_hip_sampler ncnn_moe_hip_sampler;
+
+/* Logits element type.  The runtime's logits tensor is fp32 (src/compiler/graph_builder.cpp:586-594);
+ * bf16 rows are widened with bits << 16 (src/kernels/cpu_ops.cpp:26-32) before any arithmetic. */
+enum ncnn_moe_logits_dtype
+{
+    NCNN_MOE_LOGITS_F32 = 0,
+    NCNN_MOE_LOGITS_BF16 = 1
+};
+
+/* Call-level return codes.  Errors map to ErrorCode::InternalError (include/ncnn/moe/result.h:12-25)
+ * except NCNN_MOE_SAMPLER_INVALID_ARGUMENT, which maps to ErrorCode::InvalidArgument. */
+enum ncnn_moe_sampler_rc
+{
+    NCNN_MOE_SAMPLER_SUCCESS = 0,
+    NCNN_MOE_SAMPLER_INVALID_ARGUMENT = 1,
+    NCNN_MOE_SAMPLER_HIP_ERROR = 2,
+    NCNN_MOE_SAMPLER_NO_DEVICE = 3
+};
+
+/* Per-row status: one value per fixed InvalidArgument message of the CPU sampler
+ * (src/engine/session.cpp:68, :70, :72, :85 and :421, :103, :399).  A bad row does not fail the batch. */
+enum ncnn_moe_row_status
+{
+    NCNN_MOE_ROW_OK = 0,
+    NCNN_MOE_ROW_EMPTY_LOGITS = 1,
+    NCNN_MOE_ROW_BAD_TEMPERATURE = 2,
+    NCNN_MOE_ROW_BAD_TOP_P = 3,
+    NCNN_MOE_ROW_BAD_MIN_P = 4,
+    NCNN_MOE_ROW_NO_FINITE_LOGIT = 5,
+    NCNN_MOE_ROW_INVALID_DISTRIBUTION = 6
+};
+
+/* Bits of ncnn_moe_sample_result::flags. */
+enum ncnn_moe_row_flags
+{
+    NCNN_MOE_ROW_FLAG_HAS_NAN = 1,       /* the row held a NaN; NaN logits are skipped, as greedy does */
+    NCNN_MOE_ROW_FLAG_GENERAL_PATH = 2,  /* served by the full-order path rather than the Top-K select */
+    NCNN_MOE_ROW_FLAG_FALLBACK = 4       /* the Top-K select overflowed its candidate buffers (heavy ties) */
+};
+
+/* SamplingOptions (include/ncnn/moe/session.h:49-55) plus the row's slice of the stop-id array
+ * (GenerationOptions::stop_tokens, include/ncnn/moe/session.h:76-84). */
+typedef struct ncnn_moe_sample_params
+{
+    float temperature;
+    uint32_t top_k;
+    float top_p;
+    float min_p;
+    uint32_t stop_begin;
+    uint32_t stop_count;
+} ncnn_moe_sample_params;
+
+/* SampledToken (include/ncnn/moe/session.h:57-61) plus StreamToken::is_stop_token (:63-72). */
+typedef struct ncnn_moe_sample_result
+{
+    int32_t token_id;      /* -1 unless status is NCNN_MOE_ROW_OK */
+    float probability;
+    uint32_t kept_count;   /* candidates left after Top-K, Min-P and Top-P; 1 for greedy */
+    uint8_t status;        /* enum ncnn_moe_row_status */
+    uint8_t is_stop;
+    uint8_t draw_consumed; /* 1 iff the CPU sampler would have advanced the Session RNG (session.cpp:429-433) */
+    uint8_t flags;         /* enum ncnn_moe_row_flags */
+} ncnn_moe_sample_result;
+
+/* Replaces nothing on the CPU side (the CPU sampler holds no state); plays the role of the static
+ * create() of the runtime's backend operators (src/backends/ncnn/ncnn_linear.h:45-71).  Allocates the
+ * device logits buffer and every scratch buffer up front for max_rows x max_vocab, so that sampling
+ * itself allocates nothing. */
+int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_vocab, ncnn_moe_hip_sampler** out);
+void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* sampler);
+
+/* Device-resident hand-off replacing the host copy of the LM-head output
+ * (src/engine/cpu_executor.cpp:2449-2455, :2978-2999; src/kernels/cpu_ops.cpp:1166-1172): the decode
+ * step writes [rows, vocab] logits of `dtype` at *device_logits with *row_stride elements per row. */
+int ncnn_moe_hip_sampler_logits_buffer(
+    ncnn_moe_hip_sampler* sampler, int dtype, uint32_t rows, uint32_t vocab,
+    void** device_logits, uint64_t* row_stride);
+
+/* Host rows -> the handle's logits buffer (LogitsOutput::values, include/ncnn/moe/session.h:30-33),
+ * for callers whose logits still live on the host.  row_stride is in elements. */
+int ncnn_moe_hip_sampler_upload_logits(
+    ncnn_moe_hip_sampler* sampler, const void* host_logits, int dtype,
+    uint32_t rows, uint32_t vocab, uint64_t row_stride);
+
+/* The batched form of Session::sample (include/ncnn/moe/session.h:326, src/engine/session.cpp:452-456)
+ * over the handle's logits buffer: replaces the serial per-session loop of
+ * examples/internal/run_model.cpp:776-809.  All pointers are host memory; the call returns when
+ * results[] is filled.  uniforms[row] is the draw the row's Session RNG would produce next. */
+int ncnn_moe_hip_sampler_sample(
+    ncnn_moe_hip_sampler* sampler, uint32_t rows,
+    const ncnn_moe_sample_params* params, const float* uniforms,
+    const int32_t* stop_ids, uint32_t stop_id_count,
+    ncnn_moe_sample_result* results);
+
+/* Same computation with every operand already in device memory and no host synchronisation:
+ * kernels are enqueued on `stream` (a hipStream_t, or null for the default stream) and the call
+ * returns at once.  device_logits may be any device matrix (row_stride in elements), not only the
+ * handle's buffer.  This is the entry the decode step calls in its own stream. */
+int ncnn_moe_hip_sampler_sample_device(
+    ncnn_moe_hip_sampler* sampler,
+    const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
+    const ncnn_moe_sample_params* device_params, const float* device_uniforms,
+    const int32_t* device_stop_ids,
+    ncnn_moe_sample_result* device_results, void* stream);
+
+/* sampling_distribution (src/engine/session.cpp:76-136) for one row of the handle's logits buffer:
+ * the filtered, renormalised (token id, probability) list in the CPU order.  Writes min(*count, cap)
+ * entries.  Used by parity tests and by speculative verification (src/engine/session.cpp:799-804).
+ * Returns the row status in *status (a greedy row yields NCNN_MOE_ROW_OK with its single token). */
+int ncnn_moe_hip_sampler_distribution(
+    ncnn_moe_hip_sampler* sampler, uint32_t row, const ncnn_moe_sample_params* params,
+    uint32_t cap, int32_t* ids, float* probabilities, uint32_t* count, uint32_t* status);
+
+/* Error text of the last failed call on this handle (Error::message, include/ncnn/moe/result.h:21-25). */
+const char* ncnn_moe_hip_sampler_last_error(const ncnn_moe_hip_sampler* sampler);
+
+/* The CPU sampler's fixed message for a row status (src/engine/session.cpp:68,70,72,85,103,399). */
+const char* ncnn_moe_hip_sampler_status_message(int row_status);
+
+/* Number of HIP devices visible, 0 if none (no counterpart: the CPU sampler needs no device). */
+int ncnn_moe_hip_sampler_device_count(void);
+
+/* Test hooks (no counterpart in the runtime).  force_general routes every non-greedy row through
+ * the full-order path; expf evaluates the device exponential on n host values. */
+int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* sampler, int enabled);
+int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* sampler, const float* in, float* out, size_t n);
+void ncnn_moe_hip_sampler_debug_exp2_table(uint64_t out[32]);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NCNN_MOE_HIP_SAMPLER_H */

@@ -1,0 +1,493 @@
+// C ABI of the gfx950 generation sampler: handle, device buffers and kernel launches.
+#include "ncnn_moe_hip_sampler.h"
+
+#include "sampler_kernels.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+using namespace ncnn_moe_hip;
+
+struct ncnn_moe_hip_sampler
+{
+    int device = 0;
+    uint32_t max_rows = 0;
+    uint32_t max_vocab = 0;
+    uint32_t max_segments = 0;
+    uint64_t logits_stride_f32 = 0; // elements per row of the handle's logits buffer, fp32 view
+    int force_general = 0;
+    hipStream_t stream = nullptr;
+
+    void* logits = nullptr;
+    int logits_dtype = NCNN_MOE_LOGITS_F32;
+    uint32_t logits_rows = 0;
+    uint32_t logits_vocab = 0;
+    uint64_t logits_stride = 0;
+
+    ncnn_moe_sample_params* params = nullptr;
+    float* uniforms = nullptr;
+    ncnn_moe_sample_result* results = nullptr;
+    int32_t* stop_ids = nullptr;
+    uint32_t stop_capacity = 0;
+
+    float* segment_values = nullptr;
+    int32_t* segment_indices = nullptr;
+    uint32_t* segment_counts = nullptr;
+    uint32_t* row_counter = nullptr;
+    uint32_t* row_flags = nullptr;
+    uint32_t* row_state = nullptr;
+
+    uint32_t* sort_keys[2] = {nullptr, nullptr};
+    uint32_t* sort_indices[2] = {nullptr, nullptr};
+    uint64_t sort_stride = 0;
+
+    int32_t* distribution_ids = nullptr;
+    float* distribution_probabilities = nullptr;
+    uint32_t* distribution_count = nullptr;
+    ncnn_moe_sample_params* single_params = nullptr;
+    float* single_uniform = nullptr;
+    ncnn_moe_sample_result* single_result = nullptr;
+
+    std::string last_error;
+};
+
+namespace {
+
+uint64_t round_up(uint64_t value, uint64_t multiple)
+{
+    return (value + multiple - 1) / multiple * multiple;
+}
+
+int fail(ncnn_moe_hip_sampler* s, int rc, const std::string& message)
+{
+    if (s != nullptr)
+        s->last_error = message;
+    return rc;
+}
+
+int hip_fail(ncnn_moe_hip_sampler* s, hipError_t error, const char* what)
+{
+    return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, std::string(what) + ": " + hipGetErrorString(error));
+}
+
+#define SAMPLER_HIP_CHECK(s, call)                   \
+    do                                               \
+    {                                                \
+        const hipError_t error_ = (call);            \
+        if (error_ != hipSuccess)                    \
+            return hip_fail((s), error_, #call);     \
+    } while (0)
+
+uint32_t segments_for(uint32_t vocab, int dtype, const void* logits, uint64_t row_stride)
+{
+    const uint32_t width = dtype == NCNN_MOE_LOGITS_F32 ? 4u : 8u;
+    const uint32_t element = dtype == NCNN_MOE_LOGITS_F32 ? 4u : 2u;
+    const bool aligned = (reinterpret_cast<uintptr_t>(logits) & 15u) == 0 && (row_stride * element) % 16u == 0;
+    const uint64_t span = static_cast<uint64_t>(vocab) + (aligned ? 0u : width - 1u);
+    return static_cast<uint32_t>((span + kSegmentValues - 1) / kSegmentValues);
+}
+
+// Enqueues the whole sampling path for `rows` rows.
+int launch_sampler(
+    ncnn_moe_hip_sampler* s, const void* logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
+    const ncnn_moe_sample_params* params, const float* uniforms, const int32_t* stop_ids,
+    ncnn_moe_sample_result* results, bool want_distribution, hipStream_t stream)
+{
+    SamplerArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.logits = logits;
+    a.row_stride = row_stride;
+    a.rows = rows;
+    a.vocab = vocab;
+    a.segments = segments_for(vocab, dtype, logits, row_stride);
+    a.force_general = s->force_general;
+    a.params = params;
+    a.uniforms = uniforms;
+    a.stop_ids = stop_ids;
+    a.results = results;
+    a.segment_values = s->segment_values;
+    a.segment_indices = s->segment_indices;
+    a.segment_counts = s->segment_counts;
+    a.row_counter = s->row_counter;
+    a.row_flags = s->row_flags;
+    a.row_state = s->row_state;
+    a.sort_keys[0] = s->sort_keys[0];
+    a.sort_keys[1] = s->sort_keys[1];
+    a.sort_indices[0] = s->sort_indices[0];
+    a.sort_indices[1] = s->sort_indices[1];
+    a.sort_stride = s->sort_stride;
+    if (want_distribution)
+    {
+        a.distribution_ids = s->distribution_ids;
+        a.distribution_probabilities = s->distribution_probabilities;
+        a.distribution_cap = s->max_vocab;
+        a.distribution_count = s->distribution_count;
+    }
+    if (a.segments > s->max_segments)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab exceeds the handle's max_vocab");
+
+    const dim3 scan_grid(a.segments, rows, 1);
+    if (dtype == NCNN_MOE_LOGITS_F32)
+    {
+        hipLaunchKernelGGL(scan_select_kernel<NCNN_MOE_LOGITS_F32>, scan_grid, dim3(kScanThreads), 0, stream, a);
+        hipLaunchKernelGGL(general_sort_kernel<NCNN_MOE_LOGITS_F32>, dim3(rows), dim3(kSortThreads), 0, stream, a);
+    }
+    else
+    {
+        hipLaunchKernelGGL(scan_select_kernel<NCNN_MOE_LOGITS_BF16>, scan_grid, dim3(kScanThreads), 0, stream, a);
+        hipLaunchKernelGGL(general_sort_kernel<NCNN_MOE_LOGITS_BF16>, dim3(rows), dim3(kSortThreads), 0, stream, a);
+    }
+    hipLaunchKernelGGL(general_replay_kernel, dim3(rows), dim3(kReplayThreads), 0, stream, a);
+    SAMPLER_HIP_CHECK(s, hipGetLastError());
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int check_shape(ncnn_moe_hip_sampler* s, int dtype, uint32_t rows, uint32_t vocab)
+{
+    if (dtype != NCNN_MOE_LOGITS_F32 && dtype != NCNN_MOE_LOGITS_BF16)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "unknown logits dtype");
+    if (rows == 0 || rows > s->max_rows)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "rows must be in [1, max_rows]");
+    if (vocab > s->max_vocab)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab exceeds the handle's max_vocab");
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+} // namespace
+
+extern "C" {
+
+int ncnn_moe_hip_sampler_device_count(void)
+{
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess)
+        return 0;
+    return count;
+}
+
+int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_vocab, ncnn_moe_hip_sampler** out)
+{
+    if (out == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    *out = nullptr;
+    if (max_rows == 0 || max_vocab == 0)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count == 0)
+        return NCNN_MOE_SAMPLER_NO_DEVICE;
+    if (device < 0 || device >= count)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+
+    ncnn_moe_hip_sampler* s = new (std::nothrow) ncnn_moe_hip_sampler();
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_HIP_ERROR;
+    s->device = device;
+    s->max_rows = max_rows;
+    s->max_vocab = max_vocab;
+    s->max_segments = static_cast<uint32_t>((static_cast<uint64_t>(max_vocab) + 7 + kSegmentValues - 1) / kSegmentValues);
+    s->logits_stride_f32 = round_up(max_vocab, 8);
+    s->sort_stride = round_up(max_vocab, 4);
+
+    auto destroy_and_return = [&](hipError_t error, const char* what) {
+        std::fprintf(stderr, "ncnn_moe_hip_sampler_create: %s: %s\n", what, hipGetErrorString(error));
+        ncnn_moe_hip_sampler_destroy(s);
+        return NCNN_MOE_SAMPLER_HIP_ERROR;
+    };
+#define CREATE_CHECK(call)                            \
+    do                                                \
+    {                                                 \
+        const hipError_t error_ = (call);             \
+        if (error_ != hipSuccess)                     \
+            return destroy_and_return(error_, #call); \
+    } while (0)
+
+    CREATE_CHECK(hipSetDevice(device));
+    CREATE_CHECK(hipStreamCreate(&s->stream));
+    const size_t rows = max_rows;
+    const size_t slots = rows * s->max_segments;
+    CREATE_CHECK(hipMalloc(&s->logits, rows * s->logits_stride_f32 * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->params, rows * sizeof(ncnn_moe_sample_params)));
+    CREATE_CHECK(hipMalloc(&s->uniforms, rows * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->results, rows * sizeof(ncnn_moe_sample_result)));
+    s->stop_capacity = static_cast<uint32_t>(rows * 16);
+    CREATE_CHECK(hipMalloc(&s->stop_ids, static_cast<size_t>(s->stop_capacity) * sizeof(int32_t)));
+    CREATE_CHECK(hipMalloc(&s->segment_values, slots * kFastTopK * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->segment_indices, slots * kFastTopK * sizeof(int32_t)));
+    CREATE_CHECK(hipMalloc(&s->segment_counts, slots * sizeof(uint32_t)));
+    CREATE_CHECK(hipMalloc(&s->row_counter, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMalloc(&s->row_flags, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMalloc(&s->row_state, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMemset(s->row_counter, 0, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMemset(s->row_flags, 0, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMemset(s->row_state, 0, rows * sizeof(uint32_t)));
+    for (int i = 0; i < 2; ++i)
+    {
+        CREATE_CHECK(hipMalloc(&s->sort_keys[i], rows * s->sort_stride * sizeof(uint32_t)));
+        CREATE_CHECK(hipMalloc(&s->sort_indices[i], rows * s->sort_stride * sizeof(uint32_t)));
+    }
+    CREATE_CHECK(hipMalloc(&s->distribution_ids, static_cast<size_t>(max_vocab) * sizeof(int32_t)));
+    CREATE_CHECK(hipMalloc(&s->distribution_probabilities, static_cast<size_t>(max_vocab) * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->distribution_count, sizeof(uint32_t)));
+    CREATE_CHECK(hipMalloc(&s->single_params, sizeof(ncnn_moe_sample_params)));
+    CREATE_CHECK(hipMalloc(&s->single_uniform, sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->single_result, sizeof(ncnn_moe_sample_result)));
+    CREATE_CHECK(hipDeviceSynchronize());
+#undef CREATE_CHECK
+    *out = s;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
+{
+    if (s == nullptr)
+        return;
+    (void)hipSetDevice(s->device);
+    if (s->stream != nullptr)
+    {
+        (void)hipStreamSynchronize(s->stream);
+        (void)hipStreamDestroy(s->stream);
+    }
+    void* buffers[] = {
+        s->logits, s->params, s->uniforms, s->results, s->stop_ids, s->segment_values, s->segment_indices,
+        s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->sort_keys[0], s->sort_keys[1],
+        s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
+        s->distribution_count, s->single_params, s->single_uniform, s->single_result};
+    for (void* buffer : buffers)
+    {
+        if (buffer != nullptr)
+            (void)hipFree(buffer);
+    }
+    delete s;
+}
+
+int ncnn_moe_hip_sampler_logits_buffer(
+    ncnn_moe_hip_sampler* s, int dtype, uint32_t rows, uint32_t vocab,
+    void** device_logits, uint64_t* row_stride)
+{
+    if (s == nullptr || device_logits == nullptr || row_stride == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    const int rc = check_shape(s, dtype, rows, vocab);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return rc;
+    s->logits_dtype = dtype;
+    s->logits_rows = rows;
+    s->logits_vocab = vocab;
+    // rows start on 16-byte boundaries: 4 fp32 or 8 bf16 elements
+    s->logits_stride = round_up(vocab, dtype == NCNN_MOE_LOGITS_F32 ? 4 : 8);
+    *device_logits = s->logits;
+    *row_stride = s->logits_stride;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_upload_logits(
+    ncnn_moe_hip_sampler* s, const void* host_logits, int dtype,
+    uint32_t rows, uint32_t vocab, uint64_t row_stride)
+{
+    if (s == nullptr || host_logits == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    void* device_logits = nullptr;
+    uint64_t device_stride = 0;
+    const int rc = ncnn_moe_hip_sampler_logits_buffer(s, dtype, rows, vocab, &device_logits, &device_stride);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return rc;
+    if (row_stride < vocab)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "row_stride is smaller than vocab");
+    if (vocab == 0)
+        return NCNN_MOE_SAMPLER_SUCCESS;
+    const size_t element = dtype == NCNN_MOE_LOGITS_F32 ? 4 : 2;
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
+    SAMPLER_HIP_CHECK(s, hipMemcpy2DAsync(
+        device_logits, device_stride * element, host_logits, row_stride * element,
+        static_cast<size_t>(vocab) * element, rows, hipMemcpyHostToDevice, s->stream));
+    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_sample(
+    ncnn_moe_hip_sampler* s, uint32_t rows,
+    const ncnn_moe_sample_params* params, const float* uniforms,
+    const int32_t* stop_ids, uint32_t stop_id_count,
+    ncnn_moe_sample_result* results)
+{
+    if (s == nullptr || params == nullptr || uniforms == nullptr || results == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    if (rows == 0 || rows > s->logits_rows)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "rows exceeds the rows of the logits buffer");
+    for (uint32_t row = 0; row < rows; ++row)
+    {
+        const uint64_t end = static_cast<uint64_t>(params[row].stop_begin) + params[row].stop_count;
+        if (params[row].stop_count != 0 && (stop_ids == nullptr || end > stop_id_count))
+            return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "a row's stop-id slice lies outside stop_ids");
+    }
+    if (s->logits_vocab == 0)
+    {
+        // src/engine/session.cpp:397-400
+        for (uint32_t row = 0; row < rows; ++row)
+        {
+            results[row] = ncnn_moe_sample_result{-1, 0.0f, 0u, NCNN_MOE_ROW_EMPTY_LOGITS, 0, 0, 0};
+        }
+        return NCNN_MOE_SAMPLER_SUCCESS;
+    }
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
+    if (stop_id_count > s->stop_capacity)
+    {
+        SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+        SAMPLER_HIP_CHECK(s, hipFree(s->stop_ids));
+        s->stop_ids = nullptr;
+        s->stop_capacity = 0;
+        SAMPLER_HIP_CHECK(s, hipMalloc(&s->stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t)));
+        s->stop_capacity = stop_id_count;
+    }
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->params, params, rows * sizeof(ncnn_moe_sample_params), hipMemcpyHostToDevice, s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->uniforms, uniforms, rows * sizeof(float), hipMemcpyHostToDevice, s->stream));
+    if (stop_id_count > 0)
+        SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->stop_ids, stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t), hipMemcpyHostToDevice, s->stream));
+    const int rc = launch_sampler(
+        s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
+        s->params, s->uniforms, stop_id_count > 0 ? s->stop_ids : nullptr, s->results, false, s->stream);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return rc;
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
+    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_sample_device(
+    ncnn_moe_hip_sampler* s,
+    const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
+    const ncnn_moe_sample_params* device_params, const float* device_uniforms,
+    const int32_t* device_stop_ids,
+    ncnn_moe_sample_result* device_results, void* stream)
+{
+    if (s == nullptr || device_logits == nullptr || device_params == nullptr || device_uniforms == nullptr ||
+        device_results == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    const int rc = check_shape(s, dtype, rows, vocab);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return rc;
+    if (vocab == 0)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab must be positive");
+    if (row_stride < vocab)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "row_stride is smaller than vocab");
+    return launch_sampler(
+        s, device_logits, dtype, rows, vocab, row_stride, device_params, device_uniforms, device_stop_ids,
+        device_results, false, static_cast<hipStream_t>(stream));
+}
+
+int ncnn_moe_hip_sampler_distribution(
+    ncnn_moe_hip_sampler* s, uint32_t row, const ncnn_moe_sample_params* params,
+    uint32_t cap, int32_t* ids, float* probabilities, uint32_t* count, uint32_t* status)
+{
+    if (s == nullptr || params == nullptr || count == nullptr || status == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    if (cap > 0 && (ids == nullptr || probabilities == nullptr))
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    if (row >= s->logits_rows)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "row lies outside the logits buffer");
+    *count = 0;
+    if (s->logits_vocab == 0)
+    {
+        *status = NCNN_MOE_ROW_EMPTY_LOGITS;
+        return NCNN_MOE_SAMPLER_SUCCESS;
+    }
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
+    ncnn_moe_sample_params single = *params;
+    single.stop_begin = 0;
+    single.stop_count = 0;
+    const float uniform = 0.5f;
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->single_params, &single, sizeof(single), hipMemcpyHostToDevice, s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->single_uniform, &uniform, sizeof(uniform), hipMemcpyHostToDevice, s->stream));
+    const size_t element = s->logits_dtype == NCNN_MOE_LOGITS_F32 ? 4 : 2;
+    const char* row_logits = static_cast<const char*>(s->logits) + static_cast<size_t>(row) * s->logits_stride * element;
+    const int rc = launch_sampler(
+        s, row_logits, s->logits_dtype, 1, s->logits_vocab, s->logits_stride,
+        s->single_params, s->single_uniform, nullptr, s->single_result, true, s->stream);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return rc;
+    ncnn_moe_sample_result result;
+    uint32_t kept = 0;
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(&result, s->single_result, sizeof(result), hipMemcpyDeviceToHost, s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(&kept, s->distribution_count, sizeof(kept), hipMemcpyDeviceToHost, s->stream));
+    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    *status = result.status;
+    *count = kept;
+    const uint32_t n = kept < cap ? kept : cap;
+    if (n > 0)
+    {
+        SAMPLER_HIP_CHECK(s, hipMemcpy(ids, s->distribution_ids, static_cast<size_t>(n) * sizeof(int32_t), hipMemcpyDeviceToHost));
+        SAMPLER_HIP_CHECK(s, hipMemcpy(probabilities, s->distribution_probabilities, static_cast<size_t>(n) * sizeof(float), hipMemcpyDeviceToHost));
+    }
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+const char* ncnn_moe_hip_sampler_last_error(const ncnn_moe_hip_sampler* s)
+{
+    return s == nullptr ? "" : s->last_error.c_str();
+}
+
+const char* ncnn_moe_hip_sampler_status_message(int row_status)
+{
+    switch (row_status)
+    {
+    case NCNN_MOE_ROW_OK: return "";
+    case NCNN_MOE_ROW_EMPTY_LOGITS: return "cannot sample empty logits";
+    case NCNN_MOE_ROW_BAD_TEMPERATURE: return "temperature must be finite and non-negative";
+    case NCNN_MOE_ROW_BAD_TOP_P: return "top_p must be in the range (0, 1]";
+    case NCNN_MOE_ROW_BAD_MIN_P: return "min_p must be in the range [0, 1]";
+    case NCNN_MOE_ROW_NO_FINITE_LOGIT: return "sampling requires at least one finite logit";
+    case NCNN_MOE_ROW_INVALID_DISTRIBUTION: return "sampling distribution is invalid";
+    default: return "unknown row status";
+    }
+}
+
+int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* s, int enabled)
+{
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    s->force_general = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* s, const float* in, float* out, size_t n)
+{
+    if (s == nullptr || in == nullptr || out == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    if (n == 0)
+        return NCNN_MOE_SAMPLER_SUCCESS;
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
+    float* device_in = nullptr;
+    float* device_out = nullptr;
+    SAMPLER_HIP_CHECK(s, hipMalloc(&device_in, n * sizeof(float)));
+    hipError_t error = hipMalloc(&device_out, n * sizeof(float));
+    if (error == hipSuccess)
+        error = hipMemcpy(device_in, in, n * sizeof(float), hipMemcpyHostToDevice);
+    if (error == hipSuccess)
+    {
+        const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+        hipLaunchKernelGGL(expf_probe_kernel, dim3(blocks), dim3(256), 0, s->stream, device_in, device_out, n);
+        error = hipGetLastError();
+    }
+    if (error == hipSuccess)
+        error = hipStreamSynchronize(s->stream);
+    if (error == hipSuccess)
+        error = hipMemcpy(out, device_out, n * sizeof(float), hipMemcpyDeviceToHost);
+    (void)hipFree(device_in);
+    if (device_out != nullptr)
+        (void)hipFree(device_out);
+    if (error != hipSuccess)
+        return hip_fail(s, error, "debug_expf");
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+void ncnn_moe_hip_sampler_debug_exp2_table(uint64_t out[32])
+{
+    static const uint64_t table[32] = {NCNN_MOE_EXP2_TABLE_VALUES};
+    std::memcpy(out, table, sizeof(table));
+}
+
+} // extern "C"

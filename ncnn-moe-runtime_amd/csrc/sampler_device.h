@@ -1,0 +1,231 @@
+// Device-side building blocks of the gfx950 generation sampler: row-mode resolution, the
+// exponential that reproduces libm expf bit for bit, order-preserving sort keys and wave64 helpers.
+#ifndef NCNN_MOE_HIP_SAMPLER_DEVICE_H
+#define NCNN_MOE_HIP_SAMPLER_DEVICE_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ncnn_moe_hip_sampler.h"
+
+namespace ncnn_moe_hip {
+
+constexpr int kWaveSize = 64;
+
+// Top-K select ("fast") path geometry: a workgroup of 256 threads owns a segment of
+// 256 * 40 = 10240 consecutive logits, 40 per lane, loaded with 16-byte loads.
+constexpr int kScanThreads = 256;
+constexpr int kScanWaves = kScanThreads / kWaveSize;
+constexpr int kValuesPerLane = 40;
+constexpr int kSegmentValues = kScanThreads * kValuesPerLane;
+constexpr int kFastTopK = 64;         // largest effective Top-K served by the select path
+constexpr int kWaveCandidateCap = 128; // candidates one wave may emit for its segment
+constexpr int kSurvivorCap = 512;      // candidates that may survive the row-level prune
+constexpr int kMaxSegments = 4096;
+
+// Full-order ("general") path geometry.
+constexpr int kSortThreads = 1024;
+constexpr int kSortWaves = kSortThreads / kWaveSize;
+constexpr int kReplayThreads = 256;
+constexpr int kReplayChunk = 1024;
+
+enum RowMode : int
+{
+    kModeInvalid = 0,
+    kModeGreedy = 1,
+    kModeTopK = 2,
+    kModeGeneral = 3
+};
+
+enum RowState : uint32_t
+{
+    kRowDone = 0,
+    kRowNeedsGeneral = 1
+};
+
+// Bits accumulated per row while its segments are scanned.
+enum ScanFlags : uint32_t
+{
+    kScanSawNan = 1u,
+    kScanSawPositiveInfinity = 2u,
+    kScanOverflow = 4u
+};
+
+__device__ __forceinline__ bool is_finite_f32(float value)
+{
+    return (__float_as_uint(value) & 0x7f800000u) != 0x7f800000u;
+}
+
+// validate_sampling_options, src/engine/session.cpp:65-74 of the reference.
+__device__ __forceinline__ int validate_params(const ncnn_moe_sample_params& p)
+{
+    if (!is_finite_f32(p.temperature) || p.temperature < 0.0f)
+        return NCNN_MOE_ROW_BAD_TEMPERATURE;
+    if (!is_finite_f32(p.top_p) || p.top_p <= 0.0f || p.top_p > 1.0f)
+        return NCNN_MOE_ROW_BAD_TOP_P;
+    if (!is_finite_f32(p.min_p) || p.min_p < 0.0f || p.min_p > 1.0f)
+        return NCNN_MOE_ROW_BAD_MIN_P;
+    return NCNN_MOE_ROW_OK;
+}
+
+// Which path serves the row.  effective_k is the length of the Top-K window (vocab when Top-K is off,
+// session.cpp:86-87), 1 for greedy.
+__device__ __forceinline__ int resolve_row_mode(
+    const ncnn_moe_sample_params& p, uint32_t vocab, uint32_t segments, int force_general,
+    uint32_t& effective_k, int& status)
+{
+    status = validate_params(p);
+    effective_k = 0;
+    if (status != NCNN_MOE_ROW_OK)
+        return kModeInvalid;
+    if (p.temperature == 0.0f)
+    {
+        effective_k = 1;
+        return kModeGreedy;
+    }
+    effective_k = (p.top_k == 0u || p.top_k >= vocab) ? vocab : p.top_k;
+    if (!force_general && effective_k <= static_cast<uint32_t>(kFastTopK) && segments <= static_cast<uint32_t>(kMaxSegments))
+        return kModeTopK;
+    return kModeGeneral;
+}
+
+// 2^(i/32) as double bits with i << 47 subtracted, i = 0..31 (correctly rounded).
+#define NCNN_MOE_EXP2_TABLE_VALUES \
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull, \
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull, \
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull, \
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull, \
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull, \
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull, \
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull, \
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull,
+
+__device__ __constant__ const uint64_t kExp2Table[32] = {NCNN_MOE_EXP2_TABLE_VALUES};
+
+// expf with the results of glibc 2.35 expf on x86-64 with FMA (the CPU sampler's std::exp,
+// src/engine/session.cpp:98): x * 32/ln2 = k + r, exp(x) = 2^(k/32) * (1 + c2 r + c1 r^2 + c0 r^3),
+// all in double, one rounding to float at the end.  The reduction uses fma(32/ln2, x, -k), as the
+// FMA build of that routine does; the polynomial rounds identically with or without fused steps.
+__device__ __forceinline__ float expf_libm(float x)
+{
+    const uint32_t bits = __float_as_uint(x);
+    const uint32_t abstop = (bits >> 20) & 0x7ffu;
+    if (abstop >= 0x42bu) // |x| >= 88 or not finite
+    {
+        if (bits == 0xff800000u)
+            return 0.0f;
+        if (abstop >= 0x7f8u)
+            return x + x;
+        if (x > 0x1.62e42ep6f)
+            return __uint_as_float(0x7f800000u);
+        if (x < -0x1.9fe368p6f)
+            return 0.0f;
+    }
+    const double inverse_ln2_scaled = 0x1.71547652b82fep+0 * 32.0;
+    const double shift = 0x1.8p+52;
+    const double c0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
+    const double c1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;
+    const double c2 = 0x1.62e42ff0c52d6p-1 / 32.0;
+    const double xd = static_cast<double>(x);
+    const double z = inverse_ln2_scaled * xd;
+    double kd = z + shift;
+    const uint64_t ki = static_cast<uint64_t>(__double_as_longlong(kd));
+    kd -= shift;
+    const double r = fma(inverse_ln2_scaled, xd, -kd);
+    const uint64_t scale_bits = kExp2Table[ki & 31u] + (ki << 47);
+    const double scale = __longlong_as_double(static_cast<long long>(scale_bits));
+    const double p = fma(c0, r, c1);
+    const double r2 = r * r;
+    double y = fma(c2, r, 1.0);
+    y = fma(p, r2, y);
+    y = y * scale;
+    return static_cast<float>(y);
+}
+
+// Ascending sort key for the order (logit descending, index ascending under a stable sort):
+// the complement of the usual order-preserving float key, with -0 folded onto +0 so that the two
+// tie (LogitOrder compares with ==, src/engine/session.cpp:30-35) and NaN mapped to the last key.
+__device__ __forceinline__ uint32_t descending_key(float value)
+{
+    uint32_t bits = __float_as_uint(value);
+    if (value != value)
+        return 0xffffffffu;
+    if (bits == 0x80000000u)
+        bits = 0u;
+    const uint32_t ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+    return ~ordered;
+}
+
+__device__ __forceinline__ float value_from_descending_key(uint32_t key)
+{
+    const uint32_t ordered = ~key;
+    const uint32_t bits = (ordered & 0x80000000u) ? (ordered & 0x7fffffffu) : ~ordered;
+    return __uint_as_float(bits);
+}
+
+constexpr uint32_t kLastFiniteKey = 0xff7fffffu;   // key of -FLT_MAX
+constexpr uint32_t kPositiveInfinityKey = 0x007fffffu;
+
+__device__ __forceinline__ int lane_id()
+{
+    return static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+}
+
+// Number of set bits of mask below the calling lane.
+__device__ __forceinline__ int lanes_below(uint64_t mask)
+{
+    return static_cast<int>(__builtin_amdgcn_mbcnt_hi(
+        static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)));
+}
+
+__device__ __forceinline__ float read_lane(float value, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(value), lane));
+}
+
+__device__ __forceinline__ int read_lane(int value, int lane)
+{
+    return __builtin_amdgcn_readlane(value, lane);
+}
+
+// One compare-exchange stage across lanes at distance j; keep_max selects which partner value stays.
+__device__ __forceinline__ float exchange_stage(float value, int j, bool keep_max)
+{
+    const float other = __shfl_xor(value, j, kWaveSize);
+    return keep_max ? fmaxf(value, other) : fminf(value, other);
+}
+
+// Sorts one value per lane into descending order across the wave (lane 0 holds the largest).
+__device__ __forceinline__ float wave_sort_descending(float value, int lane)
+{
+#pragma unroll
+    for (int k = 2; k <= kWaveSize; k <<= 1)
+    {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1)
+        {
+            const bool descending_block = (lane & k) == 0 || k == kWaveSize;
+            const bool lower_lane = (lane & j) == 0;
+            value = exchange_stage(value, j, lower_lane == descending_block);
+        }
+    }
+    return value;
+}
+
+// value is bitonic across the wave; returns it sorted descending.
+__device__ __forceinline__ float wave_bitonic_merge_descending(float value, int lane)
+{
+#pragma unroll
+    for (int j = kWaveSize >> 1; j > 0; j >>= 1)
+        value = exchange_stage(value, j, (lane & j) == 0);
+    return value;
+}
+
+__device__ __forceinline__ bool candidate_before(float a_value, int a_index, float b_value, int b_index)
+{
+    return a_value > b_value || (a_value == b_value && a_index < b_index);
+}
+
+} // namespace ncnn_moe_hip
+
+#endif // NCNN_MOE_HIP_SAMPLER_DEVICE_H

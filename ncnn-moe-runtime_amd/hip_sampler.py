@@ -1,0 +1,214 @@
+"""ctypes binding of libncnn_moe_hip_sampler.so (include/ncnn_moe_hip_sampler.h).
+
+There is no CPU fallback: if the library is missing or no GPU is visible, calls raise.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(PACKAGE_DIR, "libncnn_moe_hip_sampler.so")
+
+LOGITS_F32 = 0
+LOGITS_BF16 = 1
+
+RC_SUCCESS = 0
+RC_INVALID_ARGUMENT = 1
+RC_HIP_ERROR = 2
+RC_NO_DEVICE = 3
+
+ROW_OK = 0
+ROW_EMPTY_LOGITS = 1
+ROW_BAD_TEMPERATURE = 2
+ROW_BAD_TOP_P = 3
+ROW_BAD_MIN_P = 4
+ROW_NO_FINITE_LOGIT = 5
+ROW_INVALID_DISTRIBUTION = 6
+
+FLAG_HAS_NAN = 1
+FLAG_GENERAL_PATH = 2
+FLAG_FALLBACK = 4
+
+PARAMS_DTYPE = np.dtype([("temperature", "<f4"), ("top_k", "<u4"), ("top_p", "<f4"),
+                         ("min_p", "<f4"), ("stop_begin", "<u4"), ("stop_count", "<u4")])
+RESULT_DTYPE = np.dtype([("token_id", "<i4"), ("probability", "<f4"), ("kept_count", "<u4"),
+                         ("status", "u1"), ("is_stop", "u1"), ("draw_consumed", "u1"), ("flags", "u1")])
+
+EXPORTED_SYMBOLS = [
+    "ncnn_moe_hip_sampler_create",
+    "ncnn_moe_hip_sampler_destroy",
+    "ncnn_moe_hip_sampler_logits_buffer",
+    "ncnn_moe_hip_sampler_upload_logits",
+    "ncnn_moe_hip_sampler_sample",
+    "ncnn_moe_hip_sampler_sample_device",
+    "ncnn_moe_hip_sampler_distribution",
+    "ncnn_moe_hip_sampler_last_error",
+    "ncnn_moe_hip_sampler_status_message",
+    "ncnn_moe_hip_sampler_device_count",
+    "ncnn_moe_hip_sampler_debug_force_general",
+    "ncnn_moe_hip_sampler_debug_expf",
+    "ncnn_moe_hip_sampler_debug_exp2_table",
+]
+
+
+class SamplerError(RuntimeError):
+    pass
+
+
+_library = None
+
+
+def load_library():
+    """Loads the C-ABI library; raises if it has not been built."""
+    global _library
+    if _library is not None:
+        return _library
+    if not os.path.exists(LIBRARY_PATH):
+        raise SamplerError(
+            "%s is missing: build it with `make -C %s` (or __graft_entry__.build())" % (LIBRARY_PATH, PACKAGE_DIR))
+    lib = ctypes.CDLL(LIBRARY_PATH)
+    vp = ctypes.c_void_p
+    lib.ncnn_moe_hip_sampler_create.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(vp)]
+    lib.ncnn_moe_hip_sampler_destroy.argtypes = [vp]
+    lib.ncnn_moe_hip_sampler_destroy.restype = None
+    lib.ncnn_moe_hip_sampler_logits_buffer.argtypes = [
+        vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(vp), ctypes.POINTER(ctypes.c_uint64)]
+    lib.ncnn_moe_hip_sampler_upload_logits.argtypes = [vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64]
+    lib.ncnn_moe_hip_sampler_sample.argtypes = [vp, ctypes.c_uint32, vp, vp, vp, ctypes.c_uint32, vp]
+    lib.ncnn_moe_hip_sampler_sample_device.argtypes = [
+        vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp, vp, vp, vp, vp]
+    lib.ncnn_moe_hip_sampler_distribution.argtypes = [
+        vp, ctypes.c_uint32, vp, ctypes.c_uint32, vp, vp, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32)]
+    lib.ncnn_moe_hip_sampler_last_error.argtypes = [vp]
+    lib.ncnn_moe_hip_sampler_last_error.restype = ctypes.c_char_p
+    lib.ncnn_moe_hip_sampler_status_message.argtypes = [ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_status_message.restype = ctypes.c_char_p
+    lib.ncnn_moe_hip_sampler_device_count.argtypes = []
+    lib.ncnn_moe_hip_sampler_debug_force_general.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_expf.argtypes = [vp, vp, vp, ctypes.c_size_t]
+    lib.ncnn_moe_hip_sampler_debug_exp2_table.argtypes = [vp]
+    lib.ncnn_moe_hip_sampler_debug_exp2_table.restype = None
+    _library = lib
+    return lib
+
+
+def status_message(row_status):
+    return load_library().ncnn_moe_hip_sampler_status_message(int(row_status)).decode()
+
+
+def exp2_table():
+    out = np.zeros(32, dtype=np.uint64)
+    load_library().ncnn_moe_hip_sampler_debug_exp2_table(out.ctypes.data)
+    return out
+
+
+def make_params(rows, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
+    params = np.zeros(rows, dtype=PARAMS_DTYPE)
+    params["temperature"] = temperature
+    params["top_k"] = top_k
+    params["top_p"] = top_p
+    params["min_p"] = min_p
+    return params
+
+
+class HipSampler:
+    """One sampler handle on one device."""
+
+    def __init__(self, max_rows, max_vocab, device=0):
+        self._lib = load_library()
+        self._handle = ctypes.c_void_p()
+        rc = self._lib.ncnn_moe_hip_sampler_create(device, max_rows, max_vocab, ctypes.byref(self._handle))
+        if rc != RC_SUCCESS:
+            self._handle = ctypes.c_void_p()
+            raise SamplerError("ncnn_moe_hip_sampler_create failed with code %d (no GPU or out of memory?)" % rc)
+        self.max_rows = max_rows
+        self.max_vocab = max_vocab
+
+    def close(self):
+        if getattr(self, "_handle", None) and self._handle.value:
+            self._lib.ncnn_moe_hip_sampler_destroy(self._handle)
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):
+        self.close()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    @property
+    def handle(self):
+        return self._handle
+
+    def _check(self, rc):
+        if rc != RC_SUCCESS:
+            raise SamplerError("rc=%d: %s" % (rc, self._lib.ncnn_moe_hip_sampler_last_error(self._handle).decode()))
+
+    def logits_buffer(self, dtype, rows, vocab):
+        pointer = ctypes.c_void_p()
+        stride = ctypes.c_uint64()
+        self._check(self._lib.ncnn_moe_hip_sampler_logits_buffer(
+            self._handle, dtype, rows, vocab, ctypes.byref(pointer), ctypes.byref(stride)))
+        return pointer.value, stride.value
+
+    def upload_logits(self, logits, vocab=None):
+        """logits: [rows, stride] float32, or uint16 holding bf16 bit patterns."""
+        logits = np.ascontiguousarray(logits)
+        if logits.ndim != 2 or logits.dtype not in (np.float32, np.uint16):
+            raise ValueError("logits must be a 2-D float32 or uint16 (bf16 bits) array")
+        rows, stride = logits.shape
+        vocab = stride if vocab is None else vocab
+        dtype = LOGITS_F32 if logits.dtype == np.float32 else LOGITS_BF16
+        pointer = logits.ctypes.data if logits.size else ctypes.c_void_p(8)
+        self._check(self._lib.ncnn_moe_hip_sampler_upload_logits(self._handle, pointer, dtype, rows, vocab, stride))
+
+    def sample(self, params, uniforms, stop_ids=None):
+        params = np.ascontiguousarray(params, dtype=PARAMS_DTYPE)
+        uniforms = np.ascontiguousarray(uniforms, dtype=np.float32)
+        rows = params.shape[0]
+        if uniforms.shape != (rows,):
+            raise ValueError("one uniform per row is required")
+        stops = None if stop_ids is None else np.ascontiguousarray(stop_ids, dtype=np.int32)
+        results = np.zeros(rows, dtype=RESULT_DTYPE)
+        self._check(self._lib.ncnn_moe_hip_sampler_sample(
+            self._handle, rows, params.ctypes.data, uniforms.ctypes.data,
+            None if stops is None or stops.size == 0 else stops.ctypes.data,
+            0 if stops is None else stops.size, results.ctypes.data))
+        return results
+
+    def sample_device(self, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr,
+                      stop_ids_ptr, results_ptr, stream=None):
+        """All pointers are device addresses (ints); enqueues and returns."""
+        self._check(self._lib.ncnn_moe_hip_sampler_sample_device(
+            self._handle, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr,
+            stop_ids_ptr, results_ptr, stream))
+
+    def distribution(self, row, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, cap=None):
+        """Returns (row_status, ids, probabilities) for one row of the uploaded logits."""
+        params = make_params(1, temperature, top_k, top_p, min_p)
+        cap = self.max_vocab if cap is None else cap
+        ids = np.empty(max(cap, 1), dtype=np.int32)
+        probabilities = np.empty(max(cap, 1), dtype=np.float32)
+        count = ctypes.c_uint32()
+        status = ctypes.c_uint32()
+        self._check(self._lib.ncnn_moe_hip_sampler_distribution(
+            self._handle, row, params.ctypes.data, cap, ids.ctypes.data, probabilities.ctypes.data,
+            ctypes.byref(count), ctypes.byref(status)))
+        n = min(count.value, cap)
+        return status.value, ids[:n].copy(), probabilities[:n].copy(), count.value
+
+    def force_general(self, enabled):
+        self._check(self._lib.ncnn_moe_hip_sampler_debug_force_general(self._handle, 1 if enabled else 0))
+
+    def expf(self, values):
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        out = np.empty_like(values)
+        self._check(self._lib.ncnn_moe_hip_sampler_debug_expf(self._handle, values.ctypes.data, out.ctypes.data, values.size))
+        return out
+
+
+def device_count():
+    return load_library().ncnn_moe_hip_sampler_device_count()

@@ -426,6 +426,12 @@ float oracle_expf_libm(float x)
     return std::exp(x);
 }
 
+void oracle_expf_libm_array(const float* in, float* out, size_t n)
+{
+    for (size_t i = 0; i < n; ++i)
+        out[i] = std::exp(in[i]);
+}
+
 float oracle_expf_restated(float x)
 {
     const uint32_t bits = float_bits(x);

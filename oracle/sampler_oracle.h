@@ -108,6 +108,7 @@ float oracle_rng_uniform(void* rng);
 /* libm expf, and the table-driven restatement the device code uses; must agree bit for bit. */
 float oracle_expf_libm(float x);
 float oracle_expf_restated(float x);
+void oracle_expf_libm_array(const float* in, float* out, size_t n);
 /* Returns the number of mismatching bit patterns in [first_bits, last_bits]. */
 uint64_t oracle_expf_compare_range(uint32_t first_bits, uint32_t last_bits, uint32_t stride);
 

@@ -82,6 +82,7 @@ def oracle():
     lib.oracle_expf_libm.argtypes = [ctypes.c_float]
     lib.oracle_expf_restated.restype = ctypes.c_float
     lib.oracle_expf_restated.argtypes = [ctypes.c_float]
+    lib.oracle_expf_libm_array.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
     lib.oracle_expf_compare_range.restype = ctypes.c_uint64
     lib.oracle_expf_compare_range.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
     _oracle = lib
@@ -129,6 +130,13 @@ def oracle_sample_batch(logits, params, uniforms, stop_ids=None, threads=1, voca
         None if stops is None else stops.ctypes.data, results.ctypes.data, threads)
     assert rc == 0
     return results
+
+
+def expf_libm(values):
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty_like(values)
+    oracle().oracle_expf_libm_array(values.ctypes.data, out.ctypes.data, values.size)
+    return out
 
 
 def quantize_bf16(values):

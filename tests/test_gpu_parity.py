@@ -1,0 +1,261 @@
+"""GPU parity: the HIP sampler, called through its C ABI, against the CPU oracle on identical seeded
+inputs.  Token ids, statuses, kept counts and flags must match bit for bit."""
+import numpy as np
+import pytest
+
+import oracle_lib
+import parity_util
+from ncnn_moe_runtime_amd import hip_sampler, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _announce(text):
+    print("[case] " + text, flush=True)
+
+
+@pytest.fixture(scope="module")
+def small_sampler():
+    sampler = hip_sampler.HipSampler(64, 40000)
+    yield sampler
+    sampler.close()
+
+
+def _check_rows(sampler, logits, params, uniforms, stop_ids=None, dtype="f32", context="", general=False, vocab=None):
+    _announce(context + (" [general]" if general else ""))
+    sampler.force_general(general)
+    try:
+        sampler.upload_logits(logits, vocab=vocab)
+        gpu = sampler.sample(params, uniforms, stop_ids)
+    finally:
+        sampler.force_general(False)
+    cpu = parity_util.run_oracle(logits, params, uniforms, stop_ids, vocab=vocab)
+    parity_util.assert_results_match(gpu, cpu, dtype, context)
+    return gpu, cpu
+
+
+def test_device_expf_matches_libm(small_sampler):
+    _announce("device expf vs libm expf")
+    # every 53rd float in [-110, -0.0], every 997th positive float up to 90, and special values
+    negative = np.arange(0x80000000, 0xC2DC0000, 53, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    positive = np.arange(0, 0x42B40000, 997, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, -88.0, -87.5, -103.0, -103.9, -104.0, -150.0,
+                        88.7, 88.8, 1e-30, -1e-30], dtype=np.float32)
+    values = np.concatenate([negative, positive, special])
+    device = small_sampler.expf(values)
+    host = oracle_lib.expf_libm(values)
+    both_nan = np.isnan(device) & np.isnan(host)
+    mismatch = (device.view(np.uint32) != host.view(np.uint32)) & ~both_nan
+    assert not mismatch.any(), "first mismatch at x=%r" % values[np.nonzero(mismatch)[0][:4]]
+
+
+# logf of {0.4, 0.3, 0.2, 0.1} in fp32, as bit patterns (the inputs of the recorded reference answers)
+LN_4321 = np.array([3211432455, 3214547912, 3217949200, 3222494606], dtype=np.uint32).view(np.float32).tolist()
+
+KNOWN = [
+    # logits, options, expected kept ids, expected probabilities (recorded from the reference)
+    (LN_4321, dict(min_p=0.45, top_p=0.75), [0, 1, 2], [0.444444478, 0.333333313, 0.222222209]),
+    (LN_4321, dict(min_p=0.5, top_p=0.75), [0, 1], [0.571428597, 0.428571403]),
+    (LN_4321, dict(top_p=0.5), [0, 1], [0.571428597, 0.428571403]),
+    ([1, 2, 3], dict(top_k=7), [2, 1, 0], [0.665240943, 0.244728476, 0.0900305733]),
+    ([1, 2, 3, 4, 5], dict(temperature=0.5, top_k=3, top_p=0.9, min_p=0.05), [4, 3], [0.880797088, 0.119202919]),
+    ([2, 2, 1], dict(min_p=1.0), [0, 1], [0.5, 0.5]),
+    ([5, 7, 7, 7], dict(top_k=2), [1, 2], [0.5, 0.5]),
+    ([1, 1], dict(top_p=0.5), [0], [1.0]),
+    ([3, -np.inf, -np.inf], dict(top_k=2), [0], [1.0]),
+]
+
+
+@pytest.mark.parametrize("general", [False, True])
+def test_known_answers_distribution(small_sampler, general):
+    small_sampler.force_general(general)
+    try:
+        for logits, options, ids, probabilities in KNOWN:
+            _announce("known answer %s %s general=%s" % (logits, options, general))
+            row = np.array([logits], dtype=np.float32)
+            small_sampler.upload_logits(row)
+            status, got_ids, got_probabilities, count = small_sampler.distribution(0, **options)
+            assert status == 0
+            assert count == len(ids)
+            assert got_ids.tolist() == ids
+            np.testing.assert_allclose(got_probabilities, np.array(probabilities, dtype=np.float32), rtol=2e-7)
+            oracle_status, oracle_ids, oracle_probabilities = oracle_lib.oracle_distribution(row[0], **options)
+            assert oracle_status == 0 and oracle_ids.tolist() == ids
+            assert np.array_equal(got_probabilities.view(np.uint32), oracle_probabilities.view(np.uint32))
+    finally:
+        small_sampler.force_general(False)
+
+
+@pytest.mark.parametrize("general", [False, True])
+def test_reference_test_vectors_and_errors(small_sampler, general):
+    """The reference's own sampler checks (tests/test_runtime.cpp:4332-4362) and its error cases."""
+    nan, inf = np.nan, np.inf
+    cases = [
+        ([1, 2, 3], dict(temperature=0.0), 0, 2, 1.0),
+        ([3, nan, 3], dict(temperature=0.0), 0, 0, 1.0),
+        ([nan, inf], dict(temperature=0.0), hip_sampler.ROW_NO_FINITE_LOGIT, -1, 0.0),
+        ([1, 2, 3], dict(top_k=1), 0, 2, 1.0),
+        ([1, 2, 3], dict(top_p=0.0), hip_sampler.ROW_BAD_TOP_P, -1, 0.0),
+        ([1, 2, 3], dict(top_p=1.5), hip_sampler.ROW_BAD_TOP_P, -1, 0.0),
+        ([1, 2, 3], dict(temperature=-1.0), hip_sampler.ROW_BAD_TEMPERATURE, -1, 0.0),
+        ([1, 2, 3], dict(temperature=inf), hip_sampler.ROW_BAD_TEMPERATURE, -1, 0.0),
+        ([1, 2, 3], dict(temperature=nan), hip_sampler.ROW_BAD_TEMPERATURE, -1, 0.0),
+        ([1, 2, 3], dict(min_p=-0.1), hip_sampler.ROW_BAD_MIN_P, -1, 0.0),
+        ([1, 2, 3], dict(min_p=1.1), hip_sampler.ROW_BAD_MIN_P, -1, 0.0),
+        ([0.0, -0.0], dict(top_k=1), 0, 0, 1.0),
+        ([-0.0, 0.0], dict(top_k=1), 0, 0, 1.0),
+        ([-inf, -inf], dict(temperature=0.0), hip_sampler.ROW_NO_FINITE_LOGIT, -1, 0.0),
+        ([-inf, -inf], dict(temperature=1.0), hip_sampler.ROW_NO_FINITE_LOGIT, -1, 0.0),
+        ([1, inf, 2], dict(temperature=0.7, top_k=20, top_p=0.8), hip_sampler.ROW_NO_FINITE_LOGIT, -1, 0.0),
+        ([1, inf, 2], dict(temperature=0.0), 0, 2, 1.0),
+        ([1, 2], dict(temperature=1e-39), hip_sampler.ROW_INVALID_DISTRIBUTION, -1, 0.0),
+        ([1, 2], dict(temperature=1e-30), 0, 1, 1.0),
+        ([1, 3, 2], dict(temperature=-0.0), 0, 1, 1.0),
+    ]
+    small_sampler.force_general(general)
+    try:
+        for logits, options, status, token, probability in cases:
+            _announce("reference vector %s %s general=%s" % (logits, options, general))
+            row = np.array([logits], dtype=np.float32)
+            params = hip_sampler.make_params(1, **options)
+            small_sampler.upload_logits(row)
+            got = small_sampler.sample(params, np.array([0.25], dtype=np.float32))[0]
+            assert got["status"] == status, (logits, options, got)
+            assert got["token_id"] == token, (logits, options, got)
+            assert got["probability"] == np.float32(probability)
+            cpu = oracle_lib.oracle_sample(row[0], 0.25, **options)
+            assert cpu["status"] == status and cpu["token_id"] == token
+            if status != 0:
+                assert hip_sampler.status_message(status) == oracle_lib.STATUS_MESSAGES[status]
+    finally:
+        small_sampler.force_general(False)
+
+
+def test_empty_logits(small_sampler):
+    _announce("empty logits")
+    small_sampler.upload_logits(np.zeros((2, 0), dtype=np.float32))
+    got = small_sampler.sample(hip_sampler.make_params(2), np.zeros(2, dtype=np.float32))
+    assert (got["status"] == hip_sampler.ROW_EMPTY_LOGITS).all() and (got["token_id"] == -1).all()
+    assert hip_sampler.status_message(hip_sampler.ROW_EMPTY_LOGITS) == "cannot sample empty logits"
+
+
+def test_rng_lockstep_draws(small_sampler):
+    """{0,5,5,-1}, Top-K 2, uniforms from mt19937_64(1234): token = u < 0.5 ? 1 : 2 (reference probe)."""
+    _announce("rng lock-step")
+    rng = oracle_lib.OracleRng(1234)
+    uniforms = np.array([rng.uniform() for _ in range(64)], dtype=np.float32)
+    logits = np.tile(np.array([0, 5, 5, -1], dtype=np.float32), (64, 1))
+    small_sampler.upload_logits(logits)
+    got = small_sampler.sample(hip_sampler.make_params(64, top_k=2), uniforms)
+    assert np.array_equal(got["token_id"], np.where(uniforms < 0.5, 1, 2))
+    assert (got["probability"] == 0.5).all() and (got["draw_consumed"] == 1).all() and (got["kept_count"] == 2).all()
+
+
+@pytest.mark.parametrize("general", [False, True])
+def test_cfg1_plumbing(small_sampler, general):
+    w = workloads.make_workload("cfg1_plumbing", rows=8)
+    greedy = w["params"].copy()
+    greedy["temperature"] = 0.0
+    _check_rows(small_sampler, w["logits"], greedy, w["uniforms"], context="cfg1 greedy", general=general)
+    _check_rows(small_sampler, w["logits"], w["params"], w["uniforms"], context="cfg1 T.8 K50 P.9", general=general)
+    status, ids, probabilities, count = small_sampler.distribution(0, 0.8, 50, 0.9, 0.0)
+    oracle_status, oracle_ids, oracle_probabilities = oracle_lib.oracle_distribution(w["logits"][0], 0.8, 50, 0.9, 0.0)
+    assert status == oracle_status == 0 and count == oracle_ids.size
+    assert np.array_equal(ids, oracle_ids)
+    np.testing.assert_allclose(probabilities, oracle_probabilities, rtol=1e-5)
+
+
+def test_uniform_sweep_hits_every_cdf_boundary(small_sampler):
+    """One row, 64 uniforms spread over [0, 1): the draw must agree with the oracle everywhere."""
+    w = workloads.make_workload("cfg1_plumbing", rows=1, seed=5)
+    logits = np.tile(w["logits"], (64, 1))
+    uniforms = ((np.arange(64, dtype=np.float32) + 0.5) / 64).astype(np.float32)
+    uniforms[-1] = np.float32(1.0) - np.float32(2.0 ** -24)
+    uniforms[0] = 0.0
+    _check_rows(small_sampler, logits, hip_sampler.make_params(64, 0.8, 50, 0.9), uniforms, context="uniform sweep")
+
+
+def test_edge_rows(small_sampler):
+    """Ties across the Top-K boundary, NaN / inf rows, one-token vocabularies, misaligned strides."""
+    rng = np.random.default_rng(11)
+    vocab = 12345
+    rows = 16
+    logits = rng.standard_normal((rows, vocab)).astype(np.float32)
+    logits[0, :] = 1.0                       # every logit tied
+    logits[1, ::3] = 2.5                     # a third of the row tied at the top
+    logits[2, 100:200] = np.nan
+    logits[3, 5] = np.nan
+    logits[3, 0] = 9.0
+    logits[4, :] = -np.inf
+    logits[4, 777] = -3.0
+    logits[5, :] = np.nan
+    logits[6, 10] = np.inf
+    logits[7, :] = np.round(logits[7, :] * 2) / 2   # heavy ties
+    logits[8, :] = -0.0
+    logits[8, ::2] = 0.0
+    logits[9, 4000:] = -np.inf
+    params = hip_sampler.make_params(rows, 0.9, 20, 0.95, 0.0)
+    params["top_k"][10] = 1
+    params["top_k"][11] = 64
+    params["top_k"][12] = 0
+    params["top_k"][13] = 65
+    params["temperature"][14] = 0.0
+    params["min_p"][15] = 0.3
+    uniforms = rng.random(rows).astype(np.float32)
+    _check_rows(small_sampler, logits, params, uniforms, context="edge rows")
+    greedy = params.copy()
+    greedy["temperature"] = 0.0
+    _check_rows(small_sampler, logits, greedy, uniforms, context="edge rows greedy")
+    # stride wider than the vocabulary and not a multiple of four: rows start misaligned
+    wide = np.full((rows, vocab + 3), 50.0, dtype=np.float32)
+    wide[:, :vocab] = logits
+    _check_rows(small_sampler, wide, params, uniforms, context="edge rows, misaligned stride", vocab=vocab)
+    for tiny in (1, 2, 3, 63, 64, 65):
+        small = rng.standard_normal((4, tiny)).astype(np.float32)
+        _check_rows(small_sampler, small, hip_sampler.make_params(4, 1.1, 0, 0.9, 0.01), uniforms[:4],
+                    context="vocab %d" % tiny)
+
+
+def test_bf16_rows(small_sampler):
+    rng = np.random.default_rng(3)
+    logits = workloads.float32_to_bf16_bits(rng.standard_normal((8, 30011)).astype(np.float32) * 2)
+    params = hip_sampler.make_params(8, 0.6, 64, 0.9, 0.02)
+    uniforms = rng.random(8).astype(np.float32)
+    _check_rows(small_sampler, logits, params, uniforms, dtype="bf16", context="bf16 rows K64")
+    _check_rows(small_sampler, logits, params, uniforms, dtype="bf16", context="bf16 rows K64", general=True)
+    params["top_k"] = 0
+    _check_rows(small_sampler, logits, params, uniforms, dtype="bf16", context="bf16 rows no Top-K")
+
+
+def test_stop_tokens(small_sampler):
+    w = workloads.make_workload("cfg4_service_mix", rows=32, vocab=20000)
+    _check_rows(small_sampler, w["logits"], w["params"], w["uniforms"], w["stop_ids"], context="service mix, small")
+
+
+def _full_config(name, dtype):
+    w = workloads.make_workload(name)
+    _announce("%s full size: %s" % (name, w["description"]))
+    gpu = parity_util.run_workload_on_gpu(w)
+    cpu = parity_util.run_oracle(w["logits"], w["params"], w["uniforms"], w["stop_ids"])
+    counters = parity_util.parity_counters(gpu, cpu)
+    print("[parity] %s %s" % (name, counters), flush=True)
+    parity_util.assert_results_match(gpu, cpu, dtype, name)
+    return gpu, cpu
+
+
+def test_cfg2_full():
+    gpu, _ = _full_config("cfg2_topk_topp", "f32")
+    assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH == 0).all()
+
+
+def test_cfg3_full():
+    _full_config("cfg3_full_nucleus", "bf16")
+
+
+def test_cfg4_full():
+    _full_config("cfg4_service_mix", "f32")
+
+
+def test_cfg5_full():
+    gpu, _ = _full_config("cfg5_tie_stress", "bf16")
+    assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH == 0).all()
