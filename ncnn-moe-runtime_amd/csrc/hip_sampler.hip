@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -106,6 +107,7 @@ int launch_sampler(
     a.vocab = vocab;
     a.segments = segments_for(vocab, dtype, logits, row_stride);
     a.force_general = s->force_general;
+    a.debug_stage = getenv("NCNN_MOE_SAMPLER_DEBUG_STAGE") ? atoi(getenv("NCNN_MOE_SAMPLER_DEBUG_STAGE")) : 0;
     a.params = params;
     a.uniforms = uniforms;
     a.stop_ids = stop_ids;

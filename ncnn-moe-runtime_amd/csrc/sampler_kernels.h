@@ -23,6 +23,7 @@ struct SamplerArgs
     uint32_t vocab;
     uint32_t segments;
     int force_general;
+    int debug_stage; // TEMPORARY profiling knob
 
     const ncnn_moe_sample_params* params;
     const float* uniforms;
@@ -344,6 +345,12 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
     if (lane_max == __uint_as_float(0x7f800000u))
         local_flags |= kScanSawPositiveInfinity;
 
+    if (a.debug_stage == 1)
+    {
+        if (lane_max == 12345.678f)
+            a.segment_values[0] = lane_max;
+        return;
+    }
     // ---- K-th largest lane maximum of the workgroup: a lower bound for the K-th best logit of the
     // row, because the lanes above it each hold a distinct logit at least that large.
     const float sorted_max = wave_sort_descending(lane_max, lane);
@@ -360,6 +367,12 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
     float threshold = read_lane(merged, top_k - 1);
     threshold = fmaxf(threshold, -3.402823466e+38f); // -inf and padding never qualify
 
+    if (a.debug_stage == 2)
+    {
+        if (threshold == 12345.678f)
+            a.segment_values[0] = threshold;
+        return;
+    }
     // ---- collect the lane values at or above the bound into this wave's LDS region
     int wave_count = 0;
 #pragma unroll
@@ -387,6 +400,12 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
         atomicOr(&block_flags, local_flags);
     __syncthreads();
 
+    if (a.debug_stage == 3)
+    {
+        if (candidate_counts[0] == 12345)
+            a.segment_values[0] = 1.0f;
+        return;
+    }
     // ---- exact rank of every candidate among the workgroup's candidates; the best K go to HBM
     int counts[kScanWaves];
     int total = 0;
@@ -428,6 +447,8 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
             atomicOr(&a.row_flags[row], flags);
     }
 
+    if (a.debug_stage == 4)
+        return;
     // ---- the last workgroup of the row merges the segments
     __threadfence();
     __syncthreads();
@@ -441,6 +462,15 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
     if (!block_is_last)
         return;
     __threadfence();
+    if (a.debug_stage == 5)
+    {
+        if (tid == 0)
+        {
+            a.row_counter[row] = 0;
+            a.row_flags[row] = 0;
+        }
+        return;
+    }
 
     const uint32_t row_flags = __hip_atomic_load(&a.row_flags[row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     uint8_t result_flags = (row_flags & kScanSawNan) ? NCNN_MOE_ROW_FLAG_HAS_NAN : 0;
