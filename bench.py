@@ -153,11 +153,17 @@ def main():
     stream = torch.cuda.Stream(device=device)
     stream_pointer = stream.cuda_stream
 
+    # the scheduler holds every Session's SamplingOptions on the host, so it knows whether a batch can
+    # need the full-order kernels (no Top-K window, or one wider than 64)
+    effective_k = np.where((workload["params"]["top_k"] == 0) | (workload["params"]["top_k"] >= vocab),
+                           vocab, workload["params"]["top_k"])
+    may_need_full_order = bool(np.any((workload["params"]["temperature"] != 0) & (effective_k > 64)))
+
     def step(index):
         sampler.sample_device(
             logits[index % buffers].data_ptr(), dtype_code, rows, vocab, vocab,
             params.data_ptr(), uniforms.data_ptr(), None if stop_ids is None else stop_ids.data_ptr(),
-            results.data_ptr(), stream_pointer)
+            results.data_ptr(), may_need_full_order, stream_pointer)
 
     torch.cuda.synchronize()
     with torch.cuda.stream(stream):

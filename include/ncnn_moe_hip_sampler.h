@@ -54,7 +54,12 @@ enum ncnn_moe_row_status
     NCNN_MOE_ROW_BAD_TOP_P = 3,
     NCNN_MOE_ROW_BAD_MIN_P = 4,
     NCNN_MOE_ROW_NO_FINITE_LOGIT = 5,
-    NCNN_MOE_ROW_INVALID_DISTRIBUTION = 6
+    NCNN_MOE_ROW_INVALID_DISTRIBUTION = 6,
+    /* Not a CPU-sampler error.  Only ncnn_moe_hip_sampler_sample_device called with
+     * may_need_full_order = 0 reports it, for a row that cannot be served by the Top-K select path:
+     * its Top-K window is absent or wider than 64, or its ties overflowed the select buffers.
+     * Call again with may_need_full_order = 1. */
+    NCNN_MOE_ROW_NEEDS_FULL_ORDER = 7
 };
 
 /* Bits of ncnn_moe_sample_result::flags. */
@@ -122,13 +127,16 @@ int ncnn_moe_hip_sampler_sample(
 /* Same computation with every operand already in device memory and no host synchronisation:
  * kernels are enqueued on `stream` (a hipStream_t, or null for the default stream) and the call
  * returns at once.  device_logits may be any device matrix (row_stride in elements), not only the
- * handle's buffer.  This is the entry the decode step calls in its own stream. */
+ * handle's buffer.  This is the entry the decode step calls in its own stream.
+ * may_need_full_order: pass 0 when the caller knows from its host-side SamplingOptions that every
+ * row is greedy or has 1 <= top_k <= 64 (then one kernel is enqueued); pass 1 otherwise (the
+ * full-order kernels are enqueued as well and pick up the rows that need them). */
 int ncnn_moe_hip_sampler_sample_device(
     ncnn_moe_hip_sampler* sampler,
     const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
     const ncnn_moe_sample_params* device_params, const float* device_uniforms,
     const int32_t* device_stop_ids,
-    ncnn_moe_sample_result* device_results, void* stream);
+    ncnn_moe_sample_result* device_results, int may_need_full_order, void* stream);
 
 /* sampling_distribution (src/engine/session.cpp:76-136) for one row of the handle's logits buffer:
  * the filtered, renormalised (token id, probability) list in the CPU order.  Writes min(*count, cap)

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -84,20 +85,50 @@ int hip_fail(ncnn_moe_hip_sampler* s, hipError_t error, const char* what)
             return hip_fail((s), error_, #call);     \
     } while (0)
 
-uint32_t segments_for(uint32_t vocab, int dtype, const void* logits, uint64_t row_stride)
+uint64_t logits_span(uint32_t vocab, int dtype, const void* logits, uint64_t row_stride)
 {
     const uint32_t width = dtype == NCNN_MOE_LOGITS_F32 ? 4u : 8u;
     const uint32_t element = dtype == NCNN_MOE_LOGITS_F32 ? 4u : 2u;
     const bool aligned = (reinterpret_cast<uintptr_t>(logits) & 15u) == 0 && (row_stride * element) % 16u == 0;
-    const uint64_t span = static_cast<uint64_t>(vocab) + (aligned ? 0u : width - 1u);
-    return static_cast<uint32_t>((span + kSegmentValues - 1) / kSegmentValues);
+    return static_cast<uint64_t>(vocab) + (aligned ? 0u : width - 1u);
+}
+
+uint64_t segment_values(int dtype, int chunks)
+{
+    return static_cast<uint64_t>(dtype == NCNN_MOE_LOGITS_F32 ? kSegmentValuesF32 : kSegmentValuesBF16) * chunks;
+}
+
+// Chunks of vectors one lane keeps in registers (1, 2 or 4).  One chunk streams fastest; longer
+// rows take more so that a row has at most kMaxSegments segments, which the row merge can stage.
+int chunks_for(int dtype, uint64_t span)
+{
+    if (const char* forced = getenv("NCNN_MOE_SAMPLER_CHUNKS")) // TEMPORARY tuning knob
+        return atoi(forced);
+    for (int chunks = 1; chunks < 4; chunks <<= 1)
+    {
+        if ((span + segment_values(dtype, chunks) - 1) / segment_values(dtype, chunks) <= static_cast<uint64_t>(kMaxSegments))
+            return chunks;
+    }
+    return 4;
+}
+
+template <int DTYPE>
+void launch_scan(int chunks, dim3 grid, hipStream_t stream, const SamplerArgs& a)
+{
+    if (chunks == 4)
+        hipLaunchKernelGGL((scan_select_kernel<DTYPE, 4>), grid, dim3(kScanThreads), 0, stream, a);
+    else if (chunks == 2)
+        hipLaunchKernelGGL((scan_select_kernel<DTYPE, 2>), grid, dim3(kScanThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((scan_select_kernel<DTYPE, 1>), grid, dim3(kScanThreads), 0, stream, a);
 }
 
 // Enqueues the whole sampling path for `rows` rows.
 int launch_sampler(
     ncnn_moe_hip_sampler* s, const void* logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
     const ncnn_moe_sample_params* params, const float* uniforms, const int32_t* stop_ids,
-    ncnn_moe_sample_result* results, bool want_distribution, hipStream_t stream)
+    ncnn_moe_sample_result* results, bool want_distribution, bool select_pass, bool full_order_pass,
+    hipStream_t stream)
 {
     SamplerArgs a;
     std::memset(&a, 0, sizeof(a));
@@ -105,7 +136,9 @@ int launch_sampler(
     a.row_stride = row_stride;
     a.rows = rows;
     a.vocab = vocab;
-    a.segments = segments_for(vocab, dtype, logits, row_stride);
+    const uint64_t span = logits_span(vocab, dtype, logits, row_stride);
+    const int chunks = chunks_for(dtype, span);
+    a.segments = static_cast<uint32_t>((span + segment_values(dtype, chunks) - 1) / segment_values(dtype, chunks));
     a.force_general = s->force_general;
     a.debug_stage = getenv("NCNN_MOE_SAMPLER_DEBUG_STAGE") ? atoi(getenv("NCNN_MOE_SAMPLER_DEBUG_STAGE")) : 0;
     a.params = params;
@@ -134,19 +167,34 @@ int launch_sampler(
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab exceeds the handle's max_vocab");
 
     const dim3 scan_grid(a.segments, rows, 1);
-    if (dtype == NCNN_MOE_LOGITS_F32)
+    if (select_pass)
     {
-        hipLaunchKernelGGL(scan_select_kernel<NCNN_MOE_LOGITS_F32>, scan_grid, dim3(kScanThreads), 0, stream, a);
-        hipLaunchKernelGGL(general_sort_kernel<NCNN_MOE_LOGITS_F32>, dim3(rows), dim3(kSortThreads), 0, stream, a);
+        if (dtype == NCNN_MOE_LOGITS_F32)
+            launch_scan<NCNN_MOE_LOGITS_F32>(chunks, scan_grid, stream, a);
+        else
+            launch_scan<NCNN_MOE_LOGITS_BF16>(chunks, scan_grid, stream, a);
     }
-    else
+    if (full_order_pass)
     {
-        hipLaunchKernelGGL(scan_select_kernel<NCNN_MOE_LOGITS_BF16>, scan_grid, dim3(kScanThreads), 0, stream, a);
-        hipLaunchKernelGGL(general_sort_kernel<NCNN_MOE_LOGITS_BF16>, dim3(rows), dim3(kSortThreads), 0, stream, a);
+        if (dtype == NCNN_MOE_LOGITS_F32)
+            hipLaunchKernelGGL(general_sort_kernel<NCNN_MOE_LOGITS_F32>, dim3(rows), dim3(kSortThreads), 0, stream, a);
+        else
+            hipLaunchKernelGGL(general_sort_kernel<NCNN_MOE_LOGITS_BF16>, dim3(rows), dim3(kSortThreads), 0, stream, a);
+        hipLaunchKernelGGL(general_replay_kernel, dim3(rows), dim3(kReplayThreads), 0, stream, a);
     }
-    hipLaunchKernelGGL(general_replay_kernel, dim3(rows), dim3(kReplayThreads), 0, stream, a);
     SAMPLER_HIP_CHECK(s, hipGetLastError());
     return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+// Host-side twin of resolve_row_mode: does the row's SamplingOptions send it to the full-order path?
+bool row_needs_full_order(const ncnn_moe_sample_params& p, uint32_t vocab)
+{
+    const bool valid = std::isfinite(p.temperature) && p.temperature >= 0.0f && std::isfinite(p.top_p) &&
+        p.top_p > 0.0f && p.top_p <= 1.0f && std::isfinite(p.min_p) && p.min_p >= 0.0f && p.min_p <= 1.0f;
+    if (!valid || p.temperature == 0.0f)
+        return false;
+    const uint32_t effective_k = (p.top_k == 0u || p.top_k >= vocab) ? vocab : p.top_k;
+    return effective_k > static_cast<uint32_t>(kFastTopK);
 }
 
 int check_shape(ncnn_moe_hip_sampler* s, int dtype, uint32_t rows, uint32_t vocab)
@@ -191,7 +239,7 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     s->device = device;
     s->max_rows = max_rows;
     s->max_vocab = max_vocab;
-    s->max_segments = static_cast<uint32_t>((static_cast<uint64_t>(max_vocab) + 7 + kSegmentValues - 1) / kSegmentValues);
+    s->max_segments = static_cast<uint32_t>((static_cast<uint64_t>(max_vocab) + 7 + kSegmentValuesF32 - 1) / kSegmentValuesF32);
     s->logits_stride_f32 = round_up(max_vocab, 8);
     s->sort_stride = round_up(max_vocab, 4);
 
@@ -218,8 +266,8 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->results, rows * sizeof(ncnn_moe_sample_result)));
     s->stop_capacity = static_cast<uint32_t>(rows * 16);
     CREATE_CHECK(hipMalloc(&s->stop_ids, static_cast<size_t>(s->stop_capacity) * sizeof(int32_t)));
-    CREATE_CHECK(hipMalloc(&s->segment_values, slots * kFastTopK * sizeof(float)));
-    CREATE_CHECK(hipMalloc(&s->segment_indices, slots * kFastTopK * sizeof(int32_t)));
+    CREATE_CHECK(hipMalloc(&s->segment_values, slots * kSegmentRecordSlots * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->segment_indices, slots * kSegmentRecordSlots * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->segment_counts, slots * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->row_counter, rows * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->row_flags, rows * sizeof(uint32_t)));
@@ -349,13 +397,35 @@ int ncnn_moe_hip_sampler_sample(
     SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->uniforms, uniforms, rows * sizeof(float), hipMemcpyHostToDevice, s->stream));
     if (stop_id_count > 0)
         SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->stop_ids, stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t), hipMemcpyHostToDevice, s->stream));
-    const int rc = launch_sampler(
+    // the host sees the options: the full-order kernels are enqueued only if some row needs them
+    bool full_order = s->force_general != 0;
+    for (uint32_t row = 0; row < rows && !full_order; ++row)
+        full_order = row_needs_full_order(params[row], s->logits_vocab);
+    const int32_t* device_stops = stop_id_count > 0 ? s->stop_ids : nullptr;
+    int rc = launch_sampler(
         s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-        s->params, s->uniforms, stop_id_count > 0 ? s->stop_ids : nullptr, s->results, false, s->stream);
+        s->params, s->uniforms, device_stops, s->results, false, true, full_order, s->stream);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return rc;
     SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
     SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    if (!full_order)
+    {
+        // a row whose ties overflowed the select buffers is finished by the full-order kernels
+        bool pending = false;
+        for (uint32_t row = 0; row < rows && !pending; ++row)
+            pending = results[row].status == NCNN_MOE_ROW_NEEDS_FULL_ORDER;
+        if (pending)
+        {
+            rc = launch_sampler(
+                s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
+                s->params, s->uniforms, device_stops, s->results, false, false, true, s->stream);
+            if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+                return rc;
+            SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
+            SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+        }
+    }
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 
@@ -364,7 +434,7 @@ int ncnn_moe_hip_sampler_sample_device(
     const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
     const ncnn_moe_sample_params* device_params, const float* device_uniforms,
     const int32_t* device_stop_ids,
-    ncnn_moe_sample_result* device_results, void* stream)
+    ncnn_moe_sample_result* device_results, int may_need_full_order, void* stream)
 {
     if (s == nullptr || device_logits == nullptr || device_params == nullptr || device_uniforms == nullptr ||
         device_results == nullptr)
@@ -378,7 +448,7 @@ int ncnn_moe_hip_sampler_sample_device(
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "row_stride is smaller than vocab");
     return launch_sampler(
         s, device_logits, dtype, rows, vocab, row_stride, device_params, device_uniforms, device_stop_ids,
-        device_results, false, static_cast<hipStream_t>(stream));
+        device_results, false, true, may_need_full_order != 0 || s->force_general != 0, static_cast<hipStream_t>(stream));
 }
 
 int ncnn_moe_hip_sampler_distribution(
@@ -408,7 +478,7 @@ int ncnn_moe_hip_sampler_distribution(
     const char* row_logits = static_cast<const char*>(s->logits) + static_cast<size_t>(row) * s->logits_stride * element;
     const int rc = launch_sampler(
         s, row_logits, s->logits_dtype, 1, s->logits_vocab, s->logits_stride,
-        s->single_params, s->single_uniform, nullptr, s->single_result, true, s->stream);
+        s->single_params, s->single_uniform, nullptr, s->single_result, true, true, true, s->stream);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return rc;
     ncnn_moe_sample_result result;

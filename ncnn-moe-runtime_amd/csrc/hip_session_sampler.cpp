@@ -1,0 +1,296 @@
+// Host-side C++ face of the gfx950 generation sampler (see hip_session_sampler.h).
+#include "hip_session_sampler.h"
+
+#include "ncnn_moe_hip_sampler.h"
+
+#include <algorithm>
+#include <cmath>
+
+namespace ncnn {
+namespace moe {
+
+namespace {
+
+Error invalid_argument(const char* message)
+{
+    return Error{ErrorCode::InvalidArgument, message};
+}
+
+// Row status -> the CPU sampler's Error (src/engine/session.cpp:68,70,72,85,103,399).
+Error error_of_row_status(int status)
+{
+    return Error{ErrorCode::InvalidArgument, ncnn_moe_hip_sampler_status_message(status)};
+}
+
+Error error_of_call(int rc, const ncnn_moe_hip_sampler* handle)
+{
+    const char* text = handle != nullptr ? ncnn_moe_hip_sampler_last_error(handle) : "";
+    if (rc == NCNN_MOE_SAMPLER_INVALID_ARGUMENT)
+        return Error{ErrorCode::InvalidArgument, std::string("hip sampler: ") + text};
+    return Error{ErrorCode::InternalError, std::string("hip sampler: ") + text};
+}
+
+template <typename T>
+std::vector<Result<T>> every_row(size_t rows, const Error& error)
+{
+    std::vector<Result<T>> results;
+    results.reserve(rows);
+    for (size_t i = 0; i < rows; ++i)
+        results.emplace_back(error);
+    return results;
+}
+
+} // namespace
+
+Result<bool> validate_sampling_options(const SamplingOptions& options)
+{
+    if (!std::isfinite(options.temperature) || options.temperature < 0.0f)
+        return invalid_argument("temperature must be finite and non-negative");
+    if (!std::isfinite(options.top_p) || options.top_p <= 0.0f || options.top_p > 1.0f)
+        return invalid_argument("top_p must be in the range (0, 1]");
+    if (!std::isfinite(options.min_p) || options.min_p < 0.0f || options.min_p > 1.0f)
+        return invalid_argument("min_p must be in the range [0, 1]");
+    return true;
+}
+
+float peek_uniform(const std::mt19937_64& generator, std::mt19937_64& advanced)
+{
+    advanced = generator;
+    std::uniform_real_distribution<float> distribution(0.0f, 1.0f);
+    return distribution(advanced);
+}
+
+struct HipSampler::Impl
+{
+    ncnn_moe_hip_sampler* handle = nullptr;
+    uint32_t max_rows = 0;
+    uint32_t max_vocab = 0;
+    std::vector<float> staging;
+    std::vector<ncnn_moe_sample_params> params;
+    std::vector<int32_t> stop_ids;
+    std::vector<ncnn_moe_sample_result> results;
+
+    ~Impl()
+    {
+        if (handle != nullptr)
+            ncnn_moe_hip_sampler_destroy(handle);
+    }
+};
+
+HipSampler::HipSampler() : impl_(std::make_unique<Impl>()) {}
+
+HipSampler::~HipSampler() = default;
+
+std::shared_ptr<HipSampler> HipSampler::create(int device, uint32_t max_rows, uint32_t max_vocab)
+{
+    std::shared_ptr<HipSampler> sampler(new HipSampler());
+    if (ncnn_moe_hip_sampler_create(device, max_rows, max_vocab, &sampler->impl_->handle) != NCNN_MOE_SAMPLER_SUCCESS)
+        return nullptr;
+    sampler->impl_->max_rows = max_rows;
+    sampler->impl_->max_vocab = max_vocab;
+    return sampler;
+}
+
+uint32_t HipSampler::max_rows() const noexcept
+{
+    return impl_->max_rows;
+}
+
+uint32_t HipSampler::max_vocab() const noexcept
+{
+    return impl_->max_vocab;
+}
+
+std::vector<Result<BatchSampledToken>> HipSampler::sample(
+    std::span<const std::span<const float>> logits,
+    std::span<const SamplingOptions> options,
+    std::span<const float> uniforms,
+    std::span<const std::vector<int32_t>> stop_tokens,
+    std::vector<uint8_t>& draw_consumed)
+{
+    const size_t rows = logits.size();
+    draw_consumed.assign(rows, 0);
+    if (rows == 0 || options.size() != rows || uniforms.size() != rows || (!stop_tokens.empty() && stop_tokens.size() != rows))
+        return every_row<BatchSampledToken>(rows, invalid_argument("sample batch operands differ in length"));
+    if (rows > impl_->max_rows)
+        return every_row<BatchSampledToken>(rows, invalid_argument("sample batch exceeds the sampler's max_rows"));
+    const size_t vocab = logits[0].size();
+    for (const std::span<const float>& row : logits)
+    {
+        if (row.size() != vocab)
+            return every_row<BatchSampledToken>(rows, invalid_argument("sample batch rows differ in length"));
+    }
+    if (vocab > impl_->max_vocab)
+        return every_row<BatchSampledToken>(rows, invalid_argument("logits exceed the sampler's max_vocab"));
+
+    const std::lock_guard<std::mutex> lock(mutex_);
+    Impl& impl = *impl_;
+    impl.staging.resize(rows * vocab);
+    for (size_t row = 0; row < rows; ++row)
+        std::copy(logits[row].begin(), logits[row].end(), impl.staging.begin() + row * vocab);
+    impl.params.resize(rows);
+    impl.stop_ids.clear();
+    for (size_t row = 0; row < rows; ++row)
+    {
+        ncnn_moe_sample_params& p = impl.params[row];
+        p.temperature = options[row].temperature;
+        p.top_k = options[row].top_k;
+        p.top_p = options[row].top_p;
+        p.min_p = options[row].min_p;
+        p.stop_begin = static_cast<uint32_t>(impl.stop_ids.size());
+        p.stop_count = 0;
+        if (!stop_tokens.empty())
+        {
+            p.stop_count = static_cast<uint32_t>(stop_tokens[row].size());
+            impl.stop_ids.insert(impl.stop_ids.end(), stop_tokens[row].begin(), stop_tokens[row].end());
+        }
+    }
+    impl.results.resize(rows);
+
+    int rc = ncnn_moe_hip_sampler_upload_logits(
+        impl.handle, impl.staging.data(), NCNN_MOE_LOGITS_F32, static_cast<uint32_t>(rows), static_cast<uint32_t>(vocab), vocab);
+    if (rc == NCNN_MOE_SAMPLER_SUCCESS)
+    {
+        rc = ncnn_moe_hip_sampler_sample(
+            impl.handle, static_cast<uint32_t>(rows), impl.params.data(), uniforms.data(),
+            impl.stop_ids.empty() ? nullptr : impl.stop_ids.data(), static_cast<uint32_t>(impl.stop_ids.size()),
+            impl.results.data());
+    }
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return every_row<BatchSampledToken>(rows, error_of_call(rc, impl.handle));
+
+    std::vector<Result<BatchSampledToken>> out;
+    out.reserve(rows);
+    for (size_t row = 0; row < rows; ++row)
+    {
+        const ncnn_moe_sample_result& r = impl.results[row];
+        if (r.status != NCNN_MOE_ROW_OK)
+        {
+            out.emplace_back(error_of_row_status(r.status));
+            continue;
+        }
+        draw_consumed[row] = r.draw_consumed;
+        BatchSampledToken token;
+        token.token.token_id = r.token_id;
+        token.token.probability = r.probability;
+        token.is_stop_token = r.is_stop != 0;
+        token.kept_count = r.kept_count;
+        out.emplace_back(token);
+    }
+    return out;
+}
+
+Result<std::vector<TokenProbability>> HipSampler::distribution(std::span<const float> logits, const SamplingOptions& options)
+{
+    if (logits.empty())
+        return invalid_argument("cannot sample empty logits");
+    if (logits.size() > impl_->max_vocab)
+        return invalid_argument("logits exceed the sampler's max_vocab");
+    const std::lock_guard<std::mutex> lock(mutex_);
+    Impl& impl = *impl_;
+    int rc = ncnn_moe_hip_sampler_upload_logits(
+        impl.handle, logits.data(), NCNN_MOE_LOGITS_F32, 1, static_cast<uint32_t>(logits.size()), logits.size());
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return error_of_call(rc, impl.handle);
+    ncnn_moe_sample_params p{options.temperature, options.top_k, options.top_p, options.min_p, 0, 0};
+    std::vector<int32_t> ids(logits.size());
+    std::vector<float> probabilities(logits.size());
+    uint32_t count = 0;
+    uint32_t status = 0;
+    rc = ncnn_moe_hip_sampler_distribution(
+        impl.handle, 0, &p, static_cast<uint32_t>(logits.size()), ids.data(), probabilities.data(), &count, &status);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return error_of_call(rc, impl.handle);
+    if (status != NCNN_MOE_ROW_OK)
+        return error_of_row_status(static_cast<int>(status));
+    std::vector<TokenProbability> candidates(count);
+    for (uint32_t i = 0; i < count; ++i)
+        candidates[i] = TokenProbability{ids[i], probabilities[i]};
+    return candidates;
+}
+
+SamplingSession::SamplingSession(HipSamplerPtr sampler, const SamplingSessionOptions& options)
+    : sampler_(std::move(sampler)), random_generator_(options.sampling_seed)
+{
+}
+
+Result<SampledToken> SamplingSession::sample(const LogitsOutput& logits, const SamplingOptions& options)
+{
+    const std::lock_guard<std::mutex> lock(mutex_);
+    if (logits.values.empty())
+        return invalid_argument("cannot sample empty logits");
+    if (!sampler_)
+        return Error{ErrorCode::InternalError, "hip sampler is unavailable (no GPU, or create() failed)"};
+    std::mt19937_64 advanced;
+    const float uniform = peek_uniform(random_generator_, advanced);
+    const std::span<const float> row(logits.values);
+    std::vector<uint8_t> draw_consumed;
+    auto results = sampler_->sample(
+        std::span<const std::span<const float>>(&row, 1), std::span<const SamplingOptions>(&options, 1),
+        std::span<const float>(&uniform, 1), {}, draw_consumed);
+    if (!results[0])
+        return results[0].error();
+    if (draw_consumed[0])
+        random_generator_ = advanced;
+    return results[0].value().token;
+}
+
+std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample(
+    const HipSamplerPtr& sampler, std::span<const SampleBatchRequest> requests)
+{
+    const size_t rows = requests.size();
+    if (rows == 0)
+        return {};
+    if (!sampler)
+        return every_row<BatchSampledToken>(rows, Error{ErrorCode::InternalError, "hip sampler is unavailable (no GPU, or create() failed)"});
+    std::vector<SamplingSession*> ordered;
+    ordered.reserve(rows);
+    for (const SampleBatchRequest& request : requests)
+    {
+        if (request.session == nullptr || request.logits == nullptr)
+            return every_row<BatchSampledToken>(rows, invalid_argument("sample batch contains a null session or logits"));
+        ordered.push_back(request.session);
+    }
+    std::sort(ordered.begin(), ordered.end());
+    if (std::adjacent_find(ordered.begin(), ordered.end()) != ordered.end())
+        return every_row<BatchSampledToken>(rows, invalid_argument("sample batch contains duplicate sessions"));
+    std::vector<std::unique_lock<std::mutex>> locks;
+    locks.reserve(rows);
+    for (SamplingSession* session : ordered)
+        locks.emplace_back(session->mutex_);
+
+    // rows with empty logits fail on their own (session.cpp:397-400); the others go to the device together
+    std::vector<size_t> active;
+    std::vector<std::span<const float>> logits;
+    std::vector<SamplingOptions> options;
+    std::vector<float> uniforms;
+    std::vector<std::mt19937_64> advanced;
+    std::vector<std::vector<int32_t>> stop_tokens;
+    for (size_t i = 0; i < rows; ++i)
+    {
+        if (requests[i].logits->values.empty())
+            continue;
+        active.push_back(i);
+        logits.emplace_back(requests[i].logits->values);
+        options.push_back(requests[i].sampling);
+        advanced.emplace_back();
+        uniforms.push_back(peek_uniform(requests[i].session->random_generator_, advanced.back()));
+        stop_tokens.push_back(requests[i].stop_tokens);
+    }
+    std::vector<Result<BatchSampledToken>> out = every_row<BatchSampledToken>(rows, invalid_argument("cannot sample empty logits"));
+    if (active.empty())
+        return out;
+    std::vector<uint8_t> draw_consumed;
+    auto sampled = sampler->sample(logits, options, uniforms, stop_tokens, draw_consumed);
+    for (size_t j = 0; j < active.size(); ++j)
+    {
+        const size_t i = active[j];
+        out[i] = sampled[j];
+        if (sampled[j] && draw_consumed[j])
+            requests[i].session->random_generator_ = advanced[j];
+    }
+    return out;
+}
+
+} // namespace moe
+} // namespace ncnn

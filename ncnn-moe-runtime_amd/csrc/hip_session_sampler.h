@@ -1,0 +1,194 @@
+// Host-side C++ face of the gfx950 generation sampler, shaped like the runtime's own Session
+// sampling interface so that it can stand in for the CPU sampler:
+//
+//   SamplingOptions / SampledToken / LogitsOutput / Result<T> / Error   the runtime's public types
+//       (include/ncnn/moe/session.h:30-61, include/ncnn/moe/result.h:12-71).  When this header is
+//       compiled inside the runtime (NCNN_MOE_SESSION_H already defined) the runtime's own types
+//       are used; a stand-alone build defines equivalents with the same names and defaults.
+//   HipSampler           backend operator in the style of src/backends/ncnn/ncnn_linear.h:45-71:
+//       pimpl, static create() returning a shared_ptr that is null on failure.
+//   SamplingSession      the sampling slice of Session (include/ncnn/moe/session.h:288-342): the
+//       seeded std::mt19937_64 (session.cpp:291), the per-Session mutex, sample().
+//   SessionBatchSampler  the batched entry beside SessionBatchAccess::decode
+//       (src/engine/session_batch.h:32-42): locks the Sessions in ascending pointer order and
+//       rejects duplicates (src/engine/session.cpp:1249-1265), draws one uniform per row from a COPY
+//       of each Session's generator, samples every row in one device call, and commits the copy back
+//       only for rows whose draw was consumed (session.cpp:429-433).
+//
+// Everything here runs on the device through the C ABI of include/ncnn_moe_hip_sampler.h.  There is
+// no CPU fallback: without a usable GPU create() returns null and sample() reports InternalError.
+#ifndef NCNN_MOE_HIP_SESSION_SAMPLER_H
+#define NCNN_MOE_HIP_SESSION_SAMPLER_H
+
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <random>
+#include <span>
+#include <string>
+#include <utility>
+#include <variant>
+#include <vector>
+
+#ifndef NCNN_MOE_SESSION_H
+
+namespace ncnn {
+namespace moe {
+
+enum class ErrorCode
+{
+    InvalidArgument,
+    IoError,
+    InvalidModel,
+    UnsupportedModel,
+    InternalError
+};
+
+struct Error
+{
+    ErrorCode code = ErrorCode::InternalError;
+    std::string message;
+};
+
+// Value-or-error carrier with the accessors the runtime's callers use: bool conversion, value(), error().
+template <typename T>
+class Result
+{
+public:
+    Result(T value) : storage_(std::in_place_index<0>, std::move(value)) {}
+    Result(Error error) : storage_(std::in_place_index<1>, std::move(error)) {}
+
+    explicit operator bool() const noexcept { return storage_.index() == 0; }
+    T& value() { return std::get<0>(storage_); }
+    const T& value() const { return std::get<0>(storage_); }
+    const Error& error() const { return std::get<1>(storage_); }
+
+private:
+    std::variant<T, Error> storage_;
+};
+
+struct LogitsOutput
+{
+    std::vector<float> values;
+};
+
+struct SamplingOptions
+{
+    float temperature = 1.0f;
+    uint32_t top_k = 0;
+    float top_p = 1.0f;
+    float min_p = 0.0f;
+};
+
+struct SampledToken
+{
+    int32_t token_id = -1;
+    float probability = 0.0f;
+};
+
+} // namespace moe
+} // namespace ncnn
+
+#endif // NCNN_MOE_SESSION_H
+
+namespace ncnn {
+namespace moe {
+
+// One sampled row of a batch: the token plus the stop flag the generation loops derive from it
+// (StreamToken::is_stop_token, include/ncnn/moe/session.h:63-72).
+struct BatchSampledToken
+{
+    SampledToken token;
+    bool is_stop_token = false;
+    uint32_t kept_count = 0;
+};
+
+// A candidate of the filtered distribution (sampling_distribution, src/engine/session.cpp:76-136).
+struct TokenProbability
+{
+    int32_t token_id = -1;
+    float probability = 0.0f;
+};
+
+class HipSampler
+{
+public:
+    // Null when no GPU is usable or the device buffers for max_rows x max_vocab cannot be allocated.
+    static std::shared_ptr<HipSampler> create(int device, uint32_t max_rows, uint32_t max_vocab);
+    ~HipSampler();
+    HipSampler(const HipSampler&) = delete;
+    HipSampler& operator=(const HipSampler&) = delete;
+
+    uint32_t max_rows() const noexcept;
+    uint32_t max_vocab() const noexcept;
+
+    // Samples rows.size() rows; logits[i] is row i (all rows must have the same length).  uniforms[i]
+    // is the draw row i would consume.  draw_consumed[i] reports whether it did.  One Result per row:
+    // a bad row does not fail the others.  A call-level failure yields that Error for every row.
+    std::vector<Result<BatchSampledToken>> sample(
+        std::span<const std::span<const float>> logits,
+        std::span<const SamplingOptions> options,
+        std::span<const float> uniforms,
+        std::span<const std::vector<int32_t>> stop_tokens,
+        std::vector<uint8_t>& draw_consumed);
+
+    // sampling_distribution for one row.
+    Result<std::vector<TokenProbability>> distribution(std::span<const float> logits, const SamplingOptions& options);
+
+private:
+    HipSampler();
+    struct Impl;
+    std::unique_ptr<Impl> impl_;
+    std::mutex mutex_;
+};
+
+using HipSamplerPtr = std::shared_ptr<HipSampler>;
+
+struct SamplingSessionOptions
+{
+    uint64_t sampling_seed = 0; // SessionOptions::sampling_seed, include/ncnn/moe/session.h:280-286
+};
+
+class SamplingSession
+{
+public:
+    SamplingSession(HipSamplerPtr sampler, const SamplingSessionOptions& options = {});
+
+    // Session::sample, include/ncnn/moe/session.h:326.
+    [[nodiscard]] Result<SampledToken> sample(const LogitsOutput& logits, const SamplingOptions& options = {});
+
+private:
+    friend class SessionBatchSampler;
+    HipSamplerPtr sampler_;
+    std::mt19937_64 random_generator_;
+    mutable std::mutex mutex_;
+};
+
+struct SampleBatchRequest
+{
+    SamplingSession* session = nullptr;
+    const LogitsOutput* logits = nullptr;
+    SamplingOptions sampling;
+    std::vector<int32_t> stop_tokens; // GenerationOptions::stop_tokens
+};
+
+class SessionBatchSampler
+{
+public:
+    // One device call for the whole batch; replaces the serial loop of
+    // examples/internal/run_model.cpp:776-809.  Rejects empty batches, null or duplicate Sessions and
+    // rows of different lengths with InvalidArgument for every row.
+    static std::vector<Result<BatchSampledToken>> sample(const HipSamplerPtr& sampler, std::span<const SampleBatchRequest> requests);
+};
+
+// validate_sampling_options (src/engine/session.cpp:65-74) on the host, with the same messages.
+Result<bool> validate_sampling_options(const SamplingOptions& options);
+
+// The uniform std::uniform_real_distribution<float>(0, 1) would draw next from `generator`,
+// without advancing it.  `advanced` receives the generator state after the draw.
+float peek_uniform(const std::mt19937_64& generator, std::mt19937_64& advanced);
+
+} // namespace moe
+} // namespace ncnn
+
+#endif // NCNN_MOE_HIP_SESSION_SAMPLER_H

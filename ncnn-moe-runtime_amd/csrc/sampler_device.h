@@ -12,16 +12,21 @@ namespace ncnn_moe_hip {
 
 constexpr int kWaveSize = 64;
 
-// Top-K select ("fast") path geometry: a workgroup of 256 threads owns a segment of
-// 256 * 40 = 10240 consecutive logits, 40 per lane, loaded with 16-byte loads.
-constexpr int kScanThreads = 256;
+// Top-K select ("fast") path geometry: a workgroup of 512 threads (8 waves) owns a segment of
+// consecutive logits, a few 16-byte vectors per lane (5 fp32 vectors = 20 logits, 3 bf16 vectors =
+// 24 logits) times the chunk count.  Few loads per lane and many waves per CU stream fastest.
+constexpr int kScanThreads = 512;
 constexpr int kScanWaves = kScanThreads / kWaveSize;
-constexpr int kValuesPerLane = 40;
-constexpr int kSegmentValues = kScanThreads * kValuesPerLane;
-constexpr int kFastTopK = 64;         // largest effective Top-K served by the select path
-constexpr int kWaveCandidateCap = 128; // candidates one wave may emit for its segment
-constexpr int kSurvivorCap = 512;      // candidates that may survive the row-level prune
-constexpr int kMaxSegments = 4096;
+constexpr int kVectorsPerLaneF32 = 5;
+constexpr int kVectorsPerLaneBF16 = 3;
+constexpr int kSegmentValuesF32 = kScanThreads * kVectorsPerLaneF32 * 4;   // 10240 logits per chunk
+constexpr int kSegmentValuesBF16 = kScanThreads * kVectorsPerLaneBF16 * 8; // 12288 logits per chunk
+constexpr int kFastTopK = 64;            // largest effective Top-K served by the select path
+constexpr int kWaveCandidateCap = 64;    // candidates one wave may collect for its segment
+constexpr int kSegmentRecordSlots = 256; // candidate slots of a segment's record in HBM
+constexpr int kMaxSegments = 16;         // segments per row the row merge can stage in one trip
+constexpr int kMergeStageSlots = 4096;   // record slots of a row loaded in one trip (8 per thread)
+constexpr int kMergeSurvivorCap = 512;   // candidates that may survive the row-level prune
 
 // Full-order ("general") path geometry.
 constexpr int kSortThreads = 1024;
@@ -87,6 +92,14 @@ __device__ __forceinline__ int resolve_row_mode(
     if (!force_general && effective_k <= static_cast<uint32_t>(kFastTopK) && segments <= static_cast<uint32_t>(kMaxSegments))
         return kModeTopK;
     return kModeGeneral;
+}
+
+// Entries of a segment's record that the row merge reads: twice the Top-K window plus 16 (the bound
+// admits K logits and a few more; ties beyond that overflow to the full-order path).
+__host__ __device__ __forceinline__ uint32_t segment_record_entries(uint32_t effective_k)
+{
+    const uint32_t entries = effective_k * 2u + 16u;
+    return entries > static_cast<uint32_t>(kSegmentRecordSlots) ? static_cast<uint32_t>(kSegmentRecordSlots) : entries;
 }
 
 // 2^(i/32) as double bits with i << 47 subtracted, i = 0..31 (correctly rounded).

@@ -77,6 +77,20 @@ __device__ __forceinline__ void write_error(const SamplerArgs& a, uint32_t row, 
         *a.distribution_count = 0;
 }
 
+// Marks a row that still has to go through the full-order kernels.
+__device__ __forceinline__ void write_pending(const SamplerArgs& a, uint32_t row)
+{
+    ncnn_moe_sample_result r;
+    r.token_id = -1;
+    r.probability = 0.0f;
+    r.kept_count = 0;
+    r.status = NCNN_MOE_ROW_NEEDS_FULL_ORDER;
+    r.is_stop = 0;
+    r.draw_consumed = 0;
+    r.flags = 0;
+    a.results[row] = r;
+}
+
 __device__ __forceinline__ void write_token(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
     int32_t token, float probability, uint32_t kept, uint8_t draw_consumed, uint8_t flags)
@@ -197,6 +211,7 @@ struct LogitsVector<NCNN_MOE_LOGITS_F32>
 {
     static constexpr int kWidth = 4;
     static constexpr int kElementBytes = 4;
+    static constexpr int kVectorsPerLane = kVectorsPerLaneF32;
     __device__ static __forceinline__ void unpack(const uint4& raw, float* out)
     {
         out[0] = __uint_as_float(raw.x);
@@ -211,6 +226,7 @@ struct LogitsVector<NCNN_MOE_LOGITS_BF16>
 {
     static constexpr int kWidth = 8;
     static constexpr int kElementBytes = 2;
+    static constexpr int kVectorsPerLane = kVectorsPerLaneBF16;
     // bf16 -> fp32 is bits << 16 (src/kernels/cpu_ops.cpp:26-32); element 2i is the low half of word i.
     __device__ static __forceinline__ void unpack(const uint4& raw, float* out)
     {
@@ -225,13 +241,248 @@ struct LogitsVector<NCNN_MOE_LOGITS_BF16>
     }
 };
 
-template <int DTYPE>
-__global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a)
+// Agent-scope relaxed accesses: they write through / read around the per-XCD L2, so data handed from
+// one workgroup to another needs no L2 write-back or invalidate, only a wait for the stores to land.
+__device__ __forceinline__ void store_agent(uint32_t* address, uint32_t value)
+{
+    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ uint32_t load_agent(const uint32_t* address)
+{
+    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Ascending integer key of a float for bitwise selection (larger logit, larger key); never 0 for a
+// finite logit, so 0 can mark an empty slot.
+__device__ __forceinline__ uint32_t ascending_key(float value)
+{
+    uint32_t bits = __float_as_uint(value);
+    if (bits == 0x80000000u)
+        bits = 0u; // -0 ties with +0
+    return (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+}
+
+__device__ __forceinline__ float value_from_ascending_key(uint32_t key)
+{
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+// The quota-th largest of the wave's 64 keys (one per lane), found bit by bit with wave-wide counts.
+__device__ __forceinline__ uint32_t wave_select_key(uint32_t key, int quota)
+{
+    uint32_t prefix = 0;
+#pragma unroll
+    for (int bit = 31; bit >= 0; --bit)
+    {
+        const uint32_t trial = prefix | (1u << bit);
+        if (__popcll(__ballot(key >= trial)) >= quota)
+            prefix = trial;
+    }
+    return prefix;
+}
+
+// The top_k-th largest of m <= 64 * R keys in LDS (0 if fewer than top_k are non-zero), by one wave:
+// keys in registers, the answer built bit by bit from wave-wide counts.
+template <int R>
+__device__ __forceinline__ uint32_t select_kth_key(const uint32_t* keys_in_lds, int m, int top_k, int lane)
+{
+    uint32_t keys[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        const int q = r * kWaveSize + lane;
+        keys[r] = q < m ? keys_in_lds[q] : 0u;
+    }
+    uint32_t prefix = 0;
+    for (int bit = 31; bit >= 0; --bit)
+    {
+        const uint32_t trial = prefix | (1u << bit);
+        int count = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            count += __popcll(__ballot(keys[r] >= trial));
+        if (count >= top_k)
+            prefix = trial;
+    }
+    return prefix;
+}
+
+__device__ __forceinline__ uint32_t select_kth_key_dispatch(const uint32_t* keys_in_lds, int m, int top_k, int lane)
+{
+    if (m <= kWaveSize)
+        return select_kth_key<1>(keys_in_lds, m, top_k, lane);
+    if (m <= 2 * kWaveSize)
+        return select_kth_key<2>(keys_in_lds, m, top_k, lane);
+    if (m <= 4 * kWaveSize)
+        return select_kth_key<4>(keys_in_lds, m, top_k, lane);
+    return select_kth_key<8>(keys_in_lds, m, top_k, lane);
+}
+
+struct BoundScratch
+{
+    uint32_t wave_bounds[kScanWaves];
+    uint32_t hot_keys[kScanThreads];
+    uint32_t hot_total;
+    uint32_t result;
+};
+
+// The exact top_k-th largest of the workgroup's per-thread keys (one key per thread, 0 = no key);
+// 0 when fewer than top_k threads hold a key.  All threads of the workgroup must call it.
+//   A  every wave finds a lower bound of the ceil(top_k/8)-th largest of its 64 keys (upper 16 bits
+//      only); the smallest of the eight bounds is reached by at least top_k keys of the workgroup;
+//   B  the keys at or above that bound (a few dozen) are gathered in LDS;
+//   C  wave 0 selects the exact top_k-th largest of the gathered keys.
+__device__ __forceinline__ uint32_t workgroup_kth_largest_key(uint32_t key, int top_k, int tid, BoundScratch& scratch)
+{
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const int quota = (top_k + kScanWaves - 1) / kScanWaves;
+    uint32_t prefix = 0;
+#pragma unroll
+    for (int bit = 31; bit >= 16; --bit)
+    {
+        const uint32_t trial = prefix | (1u << bit);
+        if (__popcll(__ballot(key >= trial)) >= quota)
+            prefix = trial;
+    }
+    if (lane == 0)
+        scratch.wave_bounds[wave] = prefix;
+    if (tid == 0)
+        scratch.hot_total = 0;
+    __syncthreads();
+    uint32_t loose_bound = scratch.wave_bounds[0];
+#pragma unroll
+    for (int w = 1; w < kScanWaves; ++w)
+        loose_bound = min(loose_bound, scratch.wave_bounds[w]);
+    const bool hot = key != 0u && key >= loose_bound;
+    const uint64_t hot_mask = __ballot(hot);
+    if (hot_mask != 0)
+    {
+        uint32_t base = 0;
+        if (lane == 0)
+            base = atomicAdd(&scratch.hot_total, static_cast<uint32_t>(__popcll(hot_mask)));
+        base = __builtin_amdgcn_readfirstlane(base);
+        if (hot)
+            scratch.hot_keys[base + lanes_below(hot_mask)] = key;
+    }
+    __syncthreads();
+    if (wave == 0)
+    {
+        const uint32_t kth = select_kth_key_dispatch(scratch.hot_keys, static_cast<int>(scratch.hot_total), top_k, lane);
+        if (lane == 0)
+            scratch.result = kth;
+    }
+    __syncthreads();
+    return scratch.result;
+}
+
+// Exact best-K selection over m <= 64 * R candidates in LDS by one wave; keys live in registers.
+// Selected candidates (at most top_k) are written, unordered, to final_values / final_indices.
+template <int R>
+__device__ __forceinline__ int select_best_wave(
+    const uint32_t* staged_keys, const int32_t* staged_indices, int m, int top_k, int lane,
+    float* final_values, int32_t* final_indices)
+{
+    uint32_t keys[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        const int q = r * kWaveSize + lane;
+        keys[r] = q < m ? staged_keys[q] : 0u;
+    }
+    uint32_t key_cut = 1u; // every staged key qualifies
+    uint32_t index_cut = 0xffffffffu;
+    if (m > top_k)
+    {
+        uint32_t prefix = 0;
+        for (int bit = 31; bit >= 0; --bit)
+        {
+            const uint32_t trial = prefix | (1u << bit);
+            int count = 0;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                count += __popcll(__ballot(keys[r] >= trial));
+            if (count >= top_k)
+                prefix = trial;
+        }
+        key_cut = prefix;
+        int above = 0;
+        int ties = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+        {
+            above += __popcll(__ballot(keys[r] > key_cut));
+            ties += __popcll(__ballot(keys[r] == key_cut));
+        }
+        const int needed = top_k - above; // of the ties, the `needed` lowest indices stay
+        if (ties > needed)
+        {
+            uint32_t index_prefix = 0;
+            for (int bit = 31; bit >= 0; --bit)
+            {
+                const uint32_t trial = index_prefix | (1u << bit);
+                int count = 0;
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                {
+                    const int q = r * kWaveSize + lane;
+                    const bool tie = keys[r] == key_cut && key_cut != 0u && q < m;
+                    const uint32_t index = tie ? static_cast<uint32_t>(staged_indices[q]) : 0xffffffffu;
+                    count += __popcll(__ballot(tie && index < trial));
+                }
+                if (count < needed)
+                    index_prefix = trial;
+            }
+            index_cut = index_prefix;
+        }
+    }
+    int n = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        const int q = r * kWaveSize + lane;
+        const uint32_t key = keys[r];
+        bool selected = key != 0u && key >= key_cut;
+        int32_t index = 0;
+        if (selected)
+        {
+            index = staged_indices[q];
+            if (key == key_cut && static_cast<uint32_t>(index) > index_cut)
+                selected = false;
+        }
+        const uint64_t mask = __ballot(selected);
+        if (mask != 0)
+        {
+            const int position = n + lanes_below(mask);
+            if (selected && position < kFastTopK)
+            {
+                final_values[position] = value_from_ascending_key(key);
+                final_indices[position] = index;
+            }
+            n += __popcll(mask);
+        }
+    }
+    return n < kFastTopK ? n : kFastTopK;
+}
+
+// One HBM pass of the select path.  CHUNKS * (5 fp32 | 3 bf16) vectors per lane are held in registers.
+//
+// Every workgroup: 16-byte loads -> per-vector and per-lane maxima -> the exact K-th largest lane
+// maximum of the workgroup, a bound that at least K logits of the segment reach -> the logits at
+// or above the bound (K and a few) go to the segment's record in HBM.  The last workgroup to finish
+// a row loads every record of the row, prunes the candidates with the same kind of bound, selects
+// the exact best K by (logit descending, index ascending), and runs the CPU sampler's epilogue.
+template <int DTYPE, int CHUNKS>
+__global__ __launch_bounds__(kScanThreads, (CHUNKS == 1 && DTYPE == NCNN_MOE_LOGITS_F32) ? 8 : 1) void scan_select_kernel(SamplerArgs a)
 {
     using Vector = LogitsVector<DTYPE>;
     constexpr int kWidth = Vector::kWidth;
-    constexpr int kVectors = kValuesPerLane / kWidth;
+    constexpr int kVectors = Vector::kVectorsPerLane * CHUNKS;
+    constexpr int kLaneValues = kVectors * kWidth;
+    constexpr uint32_t kSegment = static_cast<uint32_t>(kScanThreads) * kLaneValues;
     constexpr uint32_t kNegativeInfinity = 0xff800000u;
+    constexpr uint32_t kPositiveInfinity = 0x7f800000u;
 
     const uint32_t row = blockIdx.y;
     const uint32_t segment = blockIdx.x;
@@ -239,16 +490,15 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
 
-    __shared__ float lane_maxima[kScanWaves][kWaveSize];
+    __shared__ BoundScratch bound_scratch;
     __shared__ float candidate_values[kScanWaves][kWaveCandidateCap];
     __shared__ int32_t candidate_indices[kScanWaves][kWaveCandidateCap];
     __shared__ int candidate_counts[kScanWaves];
     __shared__ uint32_t block_flags;
     __shared__ int block_is_last;
-    __shared__ float survivor_values[kSurvivorCap];
-    __shared__ int32_t survivor_indices[kSurvivorCap];
-    __shared__ int survivor_count;
-    __shared__ float reduce_scratch[kScanWaves];
+    __shared__ uint32_t survivor_keys[kMergeSurvivorCap];
+    __shared__ int32_t survivor_indices[kMergeSurvivorCap];
+    __shared__ uint32_t survivor_total;
     __shared__ float final_values[kFastTopK];
     __shared__ int32_t final_indices[kFastTopK];
 
@@ -267,6 +517,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
             }
             else
             {
+                write_pending(a, row);
                 a.row_state[row] = kRowNeedsGeneral;
             }
         }
@@ -274,9 +525,13 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
     }
     const bool greedy = mode == kModeGreedy;
     const int top_k = static_cast<int>(effective_k);
+    const uint32_t record_entries = segment_record_entries(effective_k);
 
     if (tid == 0)
+    {
         block_flags = 0;
+        survivor_total = 0;
+    }
 
     // ---- load the segment: 16-byte loads from the 16-byte aligned address at or below the row start
     const char* row_pointer = static_cast<const char*>(a.logits) +
@@ -286,31 +541,36 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
     const char* aligned_base = row_pointer - static_cast<size_t>(misalignment) * Vector::kElementBytes;
     const uint32_t valid_begin = misalignment;
     const uint32_t valid_end = misalignment + a.vocab;
-    const uint32_t segment_base = segment * static_cast<uint32_t>(kSegmentValues);
+    const uint32_t segment_base = segment * kSegment;
 
-    float values[kValuesPerLane];
+    float values[kLaneValues];
     uint4 raw[kVectors];
 #pragma unroll
-    for (int it = 0; it < kVectors; ++it)
+    for (int v = 0; v < kVectors; ++v)
     {
-        const uint32_t first = segment_base + static_cast<uint32_t>(it * kScanThreads + tid) * kWidth;
+        const uint32_t first = segment_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth;
         if (first < valid_end && first + kWidth > valid_begin)
-            raw[it] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(first) * Vector::kElementBytes);
+            raw[v] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(first) * Vector::kElementBytes);
         else
-            raw[it] = make_uint4(kNegativeInfinity, kNegativeInfinity, kNegativeInfinity, kNegativeInfinity);
+            raw[v] = make_uint4(kNegativeInfinity, kNegativeInfinity, kNegativeInfinity, kNegativeInfinity);
     }
+
+    // ---- per-vector maxima, per-lane maximum (NaN ignored), NaN / +inf detection
+    float group_max[kVectors];
+    float lane_max = __uint_as_float(kNegativeInfinity);
+    bool saw_nan = false;
 #pragma unroll
-    for (int it = 0; it < kVectors; ++it)
+    for (int v = 0; v < kVectors; ++v)
     {
-        const uint32_t first = segment_base + static_cast<uint32_t>(it * kScanThreads + tid) * kWidth;
+        const uint32_t first = segment_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth;
         const bool any_valid = first < valid_end && first + kWidth > valid_begin;
         if (any_valid)
-            Vector::unpack(raw[it], &values[it * kWidth]);
+            Vector::unpack(raw[v], &values[v * kWidth]);
         else
         {
 #pragma unroll
             for (int c = 0; c < kWidth; ++c)
-                values[it * kWidth + c] = __uint_as_float(kNegativeInfinity);
+                values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
         }
         if (any_valid && (first < valid_begin || first + kWidth > valid_end))
         {
@@ -319,79 +579,78 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
             {
                 const uint32_t position = first + c;
                 if (position < valid_begin || position >= valid_end)
-                    values[it * kWidth + c] = __uint_as_float(kNegativeInfinity);
+                    values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
             }
         }
-    }
-
-    // ---- per-lane maximum (NaN ignored), NaN / +inf detection
-    uint32_t local_flags = 0;
-    float lane_max = __uint_as_float(kNegativeInfinity);
-    bool saw_nan = false;
+        float vector_max = __uint_as_float(kNegativeInfinity);
 #pragma unroll
-    for (int i = 0; i < kValuesPerLane; ++i)
-    {
-        float v = values[i];
-        saw_nan = saw_nan || (v != v);
-        if (greedy && v == __uint_as_float(0x7f800000u))
+        for (int c = 0; c < kWidth; ++c)
         {
-            v = __uint_as_float(kNegativeInfinity); // greedy skips every non-finite logit (session.cpp:411-412)
-            values[i] = v;
+            float x = values[v * kWidth + c];
+            saw_nan = saw_nan || (x != x);
+            if (greedy && x == __uint_as_float(kPositiveInfinity))
+            {
+                x = __uint_as_float(kNegativeInfinity); // greedy skips every non-finite logit (session.cpp:411-412)
+                values[v * kWidth + c] = x;
+            }
+            vector_max = fmaxf(vector_max, x);
         }
-        lane_max = fmaxf(lane_max, v);
+        group_max[v] = vector_max;
+        lane_max = fmaxf(lane_max, vector_max);
     }
+    uint32_t local_flags = 0;
     if (saw_nan)
         local_flags |= kScanSawNan;
-    if (lane_max == __uint_as_float(0x7f800000u))
+    if (lane_max == __uint_as_float(kPositiveInfinity))
         local_flags |= kScanSawPositiveInfinity;
-
     if (a.debug_stage == 1)
     {
         if (lane_max == 12345.678f)
             a.segment_values[0] = lane_max;
         return;
     }
-    // ---- K-th largest lane maximum of the workgroup: a lower bound for the K-th best logit of the
-    // row, because the lanes above it each hold a distinct logit at least that large.
-    const float sorted_max = wave_sort_descending(lane_max, lane);
-    lane_maxima[wave][lane] = sorted_max;
-    __syncthreads();
-    float merged = sorted_max;
-#pragma unroll
-    for (int other = 1; other < kScanWaves; ++other)
-    {
-        const int source = (wave + other) & (kScanWaves - 1);
-        const float reversed = lane_maxima[source][kWaveSize - 1 - lane];
-        merged = wave_bitonic_merge_descending(fmaxf(merged, reversed), lane);
-    }
-    float threshold = read_lane(merged, top_k - 1);
-    threshold = fmaxf(threshold, -3.402823466e+38f); // -inf and padding never qualify
 
+    // ---- bound: the exact K-th largest lane maximum of the workgroup.  The lanes at or above it each
+    // hold a distinct logit at least that large, so the K-th best logit of the row is no smaller.
+    const uint32_t lane_key = lane_max == __uint_as_float(kNegativeInfinity) ? 0u : ascending_key(lane_max);
+    const uint32_t bound_key = workgroup_kth_largest_key(lane_key, top_k, tid, bound_scratch);
+    // fewer than K lanes hold a finite logit: every finite logit of the segment is a candidate
+    const float threshold = bound_key == 0u ? -3.402823466e+38f : fmaxf(value_from_ascending_key(bound_key), -3.402823466e+38f);
     if (a.debug_stage == 2)
     {
         if (threshold == 12345.678f)
             a.segment_values[0] = threshold;
         return;
     }
-    // ---- collect the lane values at or above the bound into this wave's LDS region
+
+    // ---- collect the values at or above the bound into this wave's LDS region; only vectors whose
+    // maximum reaches the bound are looked at
     int wave_count = 0;
 #pragma unroll
-    for (int i = 0; i < kValuesPerLane; ++i)
+    for (int v = 0; v < kVectors; ++v)
     {
-        const bool hit = values[i] >= threshold;
-        const uint64_t hits = __ballot(hit);
-        if (hits != 0)
+        const bool vector_hit = group_max[v] >= threshold;
+        if (__ballot(vector_hit) != 0)
         {
-            const int position = wave_count + lanes_below(hits);
-            if (hit && position < kWaveCandidateCap)
+#pragma unroll
+            for (int c = 0; c < kWidth; ++c)
             {
-                const int it = i / kWidth;
-                const int c = i % kWidth;
-                const uint32_t element = segment_base + static_cast<uint32_t>(it * kScanThreads + tid) * kWidth + c - misalignment;
-                candidate_values[wave][position] = values[i];
-                candidate_indices[wave][position] = static_cast<int32_t>(element);
+                const float x = values[v * kWidth + c];
+                const bool hit = vector_hit && x >= threshold;
+                const uint64_t hits = __ballot(hit);
+                if (hits != 0)
+                {
+                    const int position = wave_count + lanes_below(hits);
+                    if (hit && position < kWaveCandidateCap)
+                    {
+                        const uint32_t element =
+                            segment_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth + c - misalignment;
+                        candidate_values[wave][position] = x;
+                        candidate_indices[wave][position] = static_cast<int32_t>(element);
+                    }
+                    wave_count += __popcll(hits);
+                }
             }
-            wave_count += __popcll(hits);
         }
     }
     if (lane == 0)
@@ -399,69 +658,62 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
     if (local_flags != 0)
         atomicOr(&block_flags, local_flags);
     __syncthreads();
-
     if (a.debug_stage == 3)
     {
         if (candidate_counts[0] == 12345)
             a.segment_values[0] = 1.0f;
         return;
     }
-    // ---- exact rank of every candidate among the workgroup's candidates; the best K go to HBM
-    int counts[kScanWaves];
+
+    // ---- hand the candidates over: compact copy of the wave regions into the segment's record
+    uint32_t* const out_values = reinterpret_cast<uint32_t*>(a.segment_values);
+    uint32_t* const out_indices = reinterpret_cast<uint32_t*>(a.segment_indices);
+    const size_t segment_slot = (static_cast<size_t>(row) * a.segments + segment);
+    int offset = 0;
     int total = 0;
     bool overflow = false;
 #pragma unroll
     for (int w = 0; w < kScanWaves; ++w)
     {
-        counts[w] = candidate_counts[w];
-        overflow = overflow || counts[w] > kWaveCandidateCap;
-        total += counts[w];
+        const int count = candidate_counts[w];
+        overflow = overflow || count > kWaveCandidateCap;
+        if (w < wave)
+            offset += count;
+        total += count;
     }
-    const size_t segment_slot = (static_cast<size_t>(row) * a.segments + segment);
+    overflow = overflow || static_cast<uint32_t>(total) > record_entries;
     if (!overflow)
     {
-        for (int slot = lane; slot < counts[wave]; slot += kWaveSize)
+        for (int j = lane; j < wave_count; j += kWaveSize)
         {
-            const float my_value = candidate_values[wave][slot];
-            const int32_t my_index = candidate_indices[wave][slot];
-            int rank = 0;
-            for (int w = 0; w < kScanWaves; ++w)
-            {
-                for (int j = 0; j < counts[w]; ++j)
-                    rank += candidate_before(candidate_values[w][j], candidate_indices[w][j], my_value, my_index) ? 1 : 0;
-            }
-            if (rank < top_k)
-            {
-                a.segment_values[segment_slot * kFastTopK + rank] = my_value;
-                a.segment_indices[segment_slot * kFastTopK + rank] = my_index;
-            }
+            store_agent(&out_values[segment_slot * kSegmentRecordSlots + offset + j], __float_as_uint(candidate_values[wave][j]));
+            store_agent(&out_indices[segment_slot * kSegmentRecordSlots + offset + j], static_cast<uint32_t>(candidate_indices[wave][j]));
         }
     }
     if (tid == 0)
     {
-        a.segment_counts[segment_slot] = overflow ? 0u : static_cast<uint32_t>(total < top_k ? total : top_k);
+        store_agent(&a.segment_counts[segment_slot], overflow ? 0u : static_cast<uint32_t>(total));
         uint32_t flags = block_flags;
         if (overflow)
             flags |= kScanOverflow;
         if (flags != 0)
             atomicOr(&a.row_flags[row], flags);
     }
-
     if (a.debug_stage == 4)
         return;
-    // ---- the last workgroup of the row merges the segments
-    __threadfence();
+
+    // ---- the last workgroup of the row merges the segments.  The barrier waits for this workgroup's
+    // agent-scope stores; the counter is bumped only after that.
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (tid == 0)
     {
-        const uint32_t previous = atomicAdd(&a.row_counter[row], 1u);
+        const uint32_t previous = __hip_atomic_fetch_add(&a.row_counter[row], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         block_is_last = previous == a.segments - 1 ? 1 : 0;
-        survivor_count = 0;
     }
     __syncthreads();
     if (!block_is_last)
         return;
-    __threadfence();
     if (a.debug_stage == 5)
     {
         if (tid == 0)
@@ -472,7 +724,31 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
         return;
     }
 
-    const uint32_t row_flags = __hip_atomic_load(&a.row_flags[row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // every load of the merge is issued before any is used: one trip to memory
+    const size_t row_slot = static_cast<size_t>(row) * a.segments;
+    const uint32_t row_entries = a.segments * record_entries;
+    constexpr int kPerThread = kMergeStageSlots / kScanThreads;
+    uint32_t loaded_keys[kPerThread];
+    uint32_t loaded_indices[kPerThread];
+    uint32_t loaded_counts[kPerThread];
+    const uint32_t row_flags = load_agent(&a.row_flags[row]);
+    const bool stageable = row_entries <= static_cast<uint32_t>(kMergeStageSlots);
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+    {
+        const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
+        loaded_keys[j] = 0;
+        loaded_indices[j] = 0;
+        loaded_counts[j] = 0;
+        if (stageable && q < row_entries)
+        {
+            const uint32_t s = q / record_entries;
+            const uint32_t r = q - s * record_entries;
+            loaded_keys[j] = load_agent(&out_values[(row_slot + s) * kSegmentRecordSlots + r]);
+            loaded_indices[j] = load_agent(&out_indices[(row_slot + s) * kSegmentRecordSlots + r]);
+            loaded_counts[j] = load_agent(&a.segment_counts[row_slot + s]);
+        }
+    }
     uint8_t result_flags = (row_flags & kScanSawNan) ? NCNN_MOE_ROW_FLAG_HAS_NAN : 0;
     __syncthreads();
     if (tid == 0)
@@ -480,10 +756,14 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
         a.row_counter[row] = 0;
         a.row_flags[row] = 0;
     }
-    if (row_flags & kScanOverflow)
+    if ((row_flags & kScanOverflow) || !stageable)
     {
+        // ties (or a very long row) left more candidates than the records hold: the full-order kernels take the row
         if (tid == 0)
+        {
+            write_pending(a, row);
             a.row_state[row] = kRowNeedsGeneral;
+        }
         return;
     }
     if (!greedy && (row_flags & kScanSawPositiveInfinity))
@@ -496,67 +776,78 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
         }
         return;
     }
-
-    const size_t row_slot = static_cast<size_t>(row) * a.segments;
-    // prune bound: the best K-th value of any segment that holds K candidates
-    float bound = __uint_as_float(kNegativeInfinity);
-    for (uint32_t s = tid; s < a.segments; s += kScanThreads)
-    {
-        if (a.segment_counts[row_slot + s] == static_cast<uint32_t>(top_k))
-            bound = fmaxf(bound, a.segment_values[(row_slot + s) * kFastTopK + top_k - 1]);
-    }
+    // per-thread best key; slots past a segment's count hold nothing
+    uint32_t thread_key = 0;
 #pragma unroll
-    for (int j = kWaveSize >> 1; j > 0; j >>= 1)
-        bound = fmaxf(bound, __shfl_xor(bound, j, kWaveSize));
-    if (lane == 0)
-        reduce_scratch[wave] = bound;
-    __syncthreads();
-    bound = fmaxf(fmaxf(reduce_scratch[0], reduce_scratch[1]), fmaxf(reduce_scratch[2], reduce_scratch[3]));
-
-    const uint32_t slots = a.segments * kFastTopK;
-    for (uint32_t slot = tid; slot < slots; slot += kScanThreads)
+    for (int j = 0; j < kPerThread; ++j)
     {
-        const uint32_t s = slot / kFastTopK;
-        const uint32_t r = slot % kFastTopK;
-        if (r < a.segment_counts[row_slot + s])
+        const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
+        const uint32_t r = q % record_entries;
+        loaded_keys[j] = (q < row_entries && r < loaded_counts[j]) ? ascending_key(__uint_as_float(loaded_keys[j])) : 0u;
+        thread_key = max(thread_key, loaded_keys[j]);
+    }
+    if (a.debug_stage == 6)
+        return;
+    // prune: at least K candidates reach the K-th largest per-thread best
+    const uint32_t prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, bound_scratch);
+    {
+        int survivors_here = 0;
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j)
+            survivors_here += (loaded_keys[j] != 0u && loaded_keys[j] >= prune_key) ? 1 : 0;
+        // wave-aggregated reservation of survivor slots
+        int prefix = survivors_here;
+#pragma unroll
+        for (int step = 1; step < kWaveSize; step <<= 1)
         {
-            const float v = a.segment_values[(row_slot + s) * kFastTopK + r];
-            if (v >= bound)
+            const int up = __shfl_up(prefix, step, kWaveSize);
+            if (lane >= step)
+                prefix += up;
+        }
+        const int wave_total = __shfl(prefix, kWaveSize - 1, kWaveSize);
+        uint32_t base = 0;
+        if (lane == 0 && wave_total > 0)
+            base = atomicAdd(&survivor_total, static_cast<uint32_t>(wave_total));
+        base = __builtin_amdgcn_readfirstlane(base);
+        uint32_t position = base + static_cast<uint32_t>(prefix - survivors_here);
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j)
+        {
+            if (loaded_keys[j] != 0u && loaded_keys[j] >= prune_key)
             {
-                const int position = atomicAdd(&survivor_count, 1);
-                if (position < kSurvivorCap)
+                if (position < static_cast<uint32_t>(kMergeSurvivorCap))
                 {
-                    survivor_values[position] = v;
-                    survivor_indices[position] = a.segment_indices[(row_slot + s) * kFastTopK + r];
+                    survivor_keys[position] = loaded_keys[j];
+                    survivor_indices[position] = static_cast<int32_t>(loaded_indices[j]);
                 }
+                ++position;
             }
         }
     }
     __syncthreads();
-    const int survivors = survivor_count;
-    if (survivors > kSurvivorCap)
+    const int survivors = static_cast<int>(survivor_total);
+    if (survivors > kMergeSurvivorCap)
     {
         if (tid == 0)
+        {
+            write_pending(a, row);
             a.row_state[row] = kRowNeedsGeneral;
+        }
         return;
     }
-    for (int slot = tid; slot < survivors; slot += kScanThreads)
-    {
-        const float my_value = survivor_values[slot];
-        const int32_t my_index = survivor_indices[slot];
-        int rank = 0;
-        for (int j = 0; j < survivors; ++j)
-            rank += candidate_before(survivor_values[j], survivor_indices[j], my_value, my_index) ? 1 : 0;
-        if (rank < top_k)
-        {
-            final_values[rank] = my_value;
-            final_indices[rank] = my_index;
-        }
-    }
-    __syncthreads();
     if (wave != 0)
         return;
-    const int n = survivors < top_k ? survivors : top_k;
+
+    // ---- wave 0: exact best K of the survivors, then their order, then the epilogue
+    int n = 0;
+    if (survivors <= kWaveSize)
+        n = select_best_wave<1>(survivor_keys, survivor_indices, survivors, top_k, lane, final_values, final_indices);
+    else if (survivors <= 2 * kWaveSize)
+        n = select_best_wave<2>(survivor_keys, survivor_indices, survivors, top_k, lane, final_values, final_indices);
+    else
+        n = select_best_wave<8>(survivor_keys, survivor_indices, survivors, top_k, lane, final_values, final_indices);
+    if (a.debug_stage == 7)
+        return;
     if (lane == 0)
         a.row_state[row] = kRowDone;
     if (n == 0)
@@ -565,8 +856,18 @@ __global__ __launch_bounds__(kScanThreads) void scan_select_kernel(SamplerArgs a
             write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
         return;
     }
-    const float value = lane < n ? final_values[lane] : 0.0f;
-    const int32_t index = lane < n ? final_indices[lane] : -1;
+    float value = lane < n ? final_values[lane] : 0.0f;
+    int32_t index = lane < n ? final_indices[lane] : -1;
+    int rank = 0;
+    for (int j = 0; j < n; ++j)
+        rank += candidate_before(read_lane(value, j), read_lane(index, j), value, index) ? 1 : 0;
+    if (lane < n)
+    {
+        final_values[rank] = value;
+        final_indices[rank] = index;
+    }
+    value = lane < n ? final_values[lane] : 0.0f;
+    index = lane < n ? final_indices[lane] : -1;
     if (greedy)
     {
         if (lane == 0)

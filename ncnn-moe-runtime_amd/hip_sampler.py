@@ -25,6 +25,7 @@ ROW_BAD_TOP_P = 3
 ROW_BAD_MIN_P = 4
 ROW_NO_FINITE_LOGIT = 5
 ROW_INVALID_DISTRIBUTION = 6
+ROW_NEEDS_FULL_ORDER = 7
 
 FLAG_HAS_NAN = 1
 FLAG_GENERAL_PATH = 2
@@ -77,7 +78,7 @@ def load_library():
     lib.ncnn_moe_hip_sampler_upload_logits.argtypes = [vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64]
     lib.ncnn_moe_hip_sampler_sample.argtypes = [vp, ctypes.c_uint32, vp, vp, vp, ctypes.c_uint32, vp]
     lib.ncnn_moe_hip_sampler_sample_device.argtypes = [
-        vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp, vp, vp, vp, vp]
+        vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp, vp, vp, vp, ctypes.c_int, vp]
     lib.ncnn_moe_hip_sampler_distribution.argtypes = [
         vp, ctypes.c_uint32, vp, ctypes.c_uint32, vp, vp, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32)]
     lib.ncnn_moe_hip_sampler_last_error.argtypes = [vp]
@@ -180,11 +181,11 @@ class HipSampler:
         return results
 
     def sample_device(self, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr,
-                      stop_ids_ptr, results_ptr, stream=None):
+                      stop_ids_ptr, results_ptr, may_need_full_order=True, stream=None):
         """All pointers are device addresses (ints); enqueues and returns."""
         self._check(self._lib.ncnn_moe_hip_sampler_sample_device(
             self._handle, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr,
-            stop_ids_ptr, results_ptr, stream))
+            stop_ids_ptr, results_ptr, 1 if may_need_full_order else 0, stream))
 
     def distribution(self, row, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, cap=None):
         """Returns (row_status, ids, probabilities) for one row of the uploaded logits."""

@@ -1,0 +1,83 @@
+"""The C-ABI library loads without a GPU and exports every function include/*.h declares;
+the C++ host mirror's host-only tests pass."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from ncnn_moe_runtime_amd import hip_sampler
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PACKAGE_DIR = os.path.join(ROOT, "ncnn-moe-runtime_amd")
+TEST_PROGRAM = os.path.join(PACKAGE_DIR, "test_session_sampler")
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "ncnn_moe_hip_sampler.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ncnn_moe_hip_sampler_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert declared_functions() == sorted(hip_sampler.EXPORTED_SYMBOLS)
+
+
+def test_library_exports_every_declared_function():
+    library = hip_sampler.load_library()
+    for name in declared_functions():
+        assert getattr(library, name) is not None
+
+
+def test_status_messages_are_the_cpu_sampler_messages():
+    expected = {
+        1: "cannot sample empty logits",
+        2: "temperature must be finite and non-negative",
+        3: "top_p must be in the range (0, 1]",
+        4: "min_p must be in the range [0, 1]",
+        5: "sampling requires at least one finite logit",
+        6: "sampling distribution is invalid",
+    }
+    for status, message in expected.items():
+        assert hip_sampler.status_message(status) == message
+    assert hip_sampler.status_message(0) == ""
+
+
+def test_struct_layouts():
+    assert hip_sampler.PARAMS_DTYPE.itemsize == 24
+    assert hip_sampler.RESULT_DTYPE.itemsize == 16
+
+
+def test_exp2_table_is_correctly_rounded():
+    """2^(i/32) as double bits minus i << 47, recomputed with 80-digit decimal arithmetic."""
+    from decimal import Decimal, getcontext
+    import struct
+    getcontext().prec = 80
+    table = hip_sampler.exp2_table()
+    for i in range(32):
+        value = float(Decimal(2) ** (Decimal(i) / Decimal(32)))
+        bits = struct.unpack("<Q", struct.pack("<d", value))[0] - (i << 47)
+        assert int(table[i]) == bits
+
+
+def test_create_without_gpu_fails_loudly():
+    if hip_sampler.device_count() > 0:
+        pytest.skip("a GPU is visible")
+    with pytest.raises(hip_sampler.SamplerError):
+        hip_sampler.HipSampler(4, 1000)
+
+
+def test_host_mirror_host_only_tests():
+    assert os.path.exists(TEST_PROGRAM), "build it with make -C ncnn-moe-runtime_amd"
+    done = subprocess.run([TEST_PROGRAM, "--host"], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "all host-side session sampler tests passed" in done.stdout
+
+
+@pytest.mark.gpu
+def test_host_mirror_on_gpu():
+    print("[case] C++ host mirror test program", flush=True)
+    done = subprocess.run([TEST_PROGRAM], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "all session sampler tests passed" in done.stdout
