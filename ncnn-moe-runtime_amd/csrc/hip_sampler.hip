@@ -7,7 +7,6 @@
 
 #include <cmath>
 #include <cstdio>
-#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -102,8 +101,6 @@ uint64_t segment_values(int dtype, int chunks)
 // rows take more so that a row has at most kMaxSegments segments, which the row merge can stage.
 int chunks_for(int dtype, uint64_t span)
 {
-    if (const char* forced = getenv("NCNN_MOE_SAMPLER_CHUNKS")) // TEMPORARY tuning knob
-        return atoi(forced);
     for (int chunks = 1; chunks < 4; chunks <<= 1)
     {
         if ((span + segment_values(dtype, chunks) - 1) / segment_values(dtype, chunks) <= static_cast<uint64_t>(kMaxSegments))
@@ -140,7 +137,6 @@ int launch_sampler(
     const int chunks = chunks_for(dtype, span);
     a.segments = static_cast<uint32_t>((span + segment_values(dtype, chunks) - 1) / segment_values(dtype, chunks));
     a.force_general = s->force_general;
-    a.debug_stage = getenv("NCNN_MOE_SAMPLER_DEBUG_STAGE") ? atoi(getenv("NCNN_MOE_SAMPLER_DEBUG_STAGE")) : 0;
     a.params = params;
     a.uniforms = uniforms;
     a.stop_ids = stop_ids;

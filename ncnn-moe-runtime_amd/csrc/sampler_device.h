@@ -31,8 +31,9 @@ constexpr int kMergeSurvivorCap = 512;   // candidates that may survive the row-
 // Full-order ("general") path geometry.
 constexpr int kSortThreads = 1024;
 constexpr int kSortWaves = kSortThreads / kWaveSize;
-constexpr int kReplayThreads = 256;
-constexpr int kReplayChunk = 1024;
+constexpr int kReplayThreads = 512;
+constexpr int kReplayPerThread = 8;
+constexpr int kReplayChunk = kReplayThreads * kReplayPerThread;
 
 enum RowMode : int
 {

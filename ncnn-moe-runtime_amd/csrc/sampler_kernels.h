@@ -23,7 +23,6 @@ struct SamplerArgs
     uint32_t vocab;
     uint32_t segments;
     int force_general;
-    int debug_stage; // TEMPORARY profiling knob
 
     const ncnn_moe_sample_params* params;
     const float* uniforms;
@@ -603,12 +602,6 @@ __global__ __launch_bounds__(kScanThreads, (CHUNKS == 1 && DTYPE == NCNN_MOE_LOG
         local_flags |= kScanSawNan;
     if (lane_max == __uint_as_float(kPositiveInfinity))
         local_flags |= kScanSawPositiveInfinity;
-    if (a.debug_stage == 1)
-    {
-        if (lane_max == 12345.678f)
-            a.segment_values[0] = lane_max;
-        return;
-    }
 
     // ---- bound: the exact K-th largest lane maximum of the workgroup.  The lanes at or above it each
     // hold a distinct logit at least that large, so the K-th best logit of the row is no smaller.
@@ -616,12 +609,6 @@ __global__ __launch_bounds__(kScanThreads, (CHUNKS == 1 && DTYPE == NCNN_MOE_LOG
     const uint32_t bound_key = workgroup_kth_largest_key(lane_key, top_k, tid, bound_scratch);
     // fewer than K lanes hold a finite logit: every finite logit of the segment is a candidate
     const float threshold = bound_key == 0u ? -3.402823466e+38f : fmaxf(value_from_ascending_key(bound_key), -3.402823466e+38f);
-    if (a.debug_stage == 2)
-    {
-        if (threshold == 12345.678f)
-            a.segment_values[0] = threshold;
-        return;
-    }
 
     // ---- collect the values at or above the bound into this wave's LDS region; only vectors whose
     // maximum reaches the bound are looked at
@@ -658,12 +645,6 @@ __global__ __launch_bounds__(kScanThreads, (CHUNKS == 1 && DTYPE == NCNN_MOE_LOG
     if (local_flags != 0)
         atomicOr(&block_flags, local_flags);
     __syncthreads();
-    if (a.debug_stage == 3)
-    {
-        if (candidate_counts[0] == 12345)
-            a.segment_values[0] = 1.0f;
-        return;
-    }
 
     // ---- hand the candidates over: compact copy of the wave regions into the segment's record
     uint32_t* const out_values = reinterpret_cast<uint32_t*>(a.segment_values);
@@ -699,8 +680,6 @@ __global__ __launch_bounds__(kScanThreads, (CHUNKS == 1 && DTYPE == NCNN_MOE_LOG
         if (flags != 0)
             atomicOr(&a.row_flags[row], flags);
     }
-    if (a.debug_stage == 4)
-        return;
 
     // ---- the last workgroup of the row merges the segments.  The barrier waits for this workgroup's
     // agent-scope stores; the counter is bumped only after that.
@@ -714,15 +693,6 @@ __global__ __launch_bounds__(kScanThreads, (CHUNKS == 1 && DTYPE == NCNN_MOE_LOG
     __syncthreads();
     if (!block_is_last)
         return;
-    if (a.debug_stage == 5)
-    {
-        if (tid == 0)
-        {
-            a.row_counter[row] = 0;
-            a.row_flags[row] = 0;
-        }
-        return;
-    }
 
     // every load of the merge is issued before any is used: one trip to memory
     const size_t row_slot = static_cast<size_t>(row) * a.segments;
@@ -786,8 +756,6 @@ __global__ __launch_bounds__(kScanThreads, (CHUNKS == 1 && DTYPE == NCNN_MOE_LOG
         loaded_keys[j] = (q < row_entries && r < loaded_counts[j]) ? ascending_key(__uint_as_float(loaded_keys[j])) : 0u;
         thread_key = max(thread_key, loaded_keys[j]);
     }
-    if (a.debug_stage == 6)
-        return;
     // prune: at least K candidates reach the K-th largest per-thread best
     const uint32_t prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, bound_scratch);
     {
@@ -846,8 +814,6 @@ __global__ __launch_bounds__(kScanThreads, (CHUNKS == 1 && DTYPE == NCNN_MOE_LOG
         n = select_best_wave<2>(survivor_keys, survivor_indices, survivors, top_k, lane, final_values, final_indices);
     else
         n = select_best_wave<8>(survivor_keys, survivor_indices, survivors, top_k, lane, final_values, final_indices);
-    if (a.debug_stage == 7)
-        return;
     if (lane == 0)
         a.row_state[row] = kRowDone;
     if (n == 0)
@@ -1032,8 +998,310 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
     }
 }
 
-// Walks the sorted row as the CPU sampler does (src/engine/session.cpp:84-134, :429-442).
-// Terms are computed by the whole workgroup a chunk at a time; thread 0 adds them in order.
+// ---------------------------------------------------------------------------------------------
+// Exact sequential fp32 sums, computed in parallel.
+//
+// The CPU sampler adds probabilities one at a time in sorted order (session.cpp:100, :123, :131,
+// :437), so every partial sum is rounded to fp32 before the next term is added.  While the running
+// sum s stays inside one binade [2^k, 2^(k+1)) its 24-bit mantissa N is an integer in units of
+// ulp(s), and adding a non-negative term t moves it by
+//     floor(t/ulp) + [frac > 1/2] + [frac == 1/2 and N + floor(t/ulp) is odd]      (round to nearest even)
+// which depends on the sum only through the parity of N.  A term is therefore a pair
+// (step if N is even, step if N is odd); pairs compose associatively, so a block-wide scan gives
+// every partial sum of a chunk exactly.  The first step that would leave the binade is carried
+// out as one real fp32 addition and the scan restarts behind it with the wider ulp.
+// ---------------------------------------------------------------------------------------------
+
+struct ParityStep
+{
+    uint32_t even; // mantissa increment when the mantissa is even before the step
+    uint32_t odd;  // ... when it is odd
+};
+
+constexpr uint32_t kBinadeFull = 1u << 24;
+constexpr uint32_t kStepCap = 1u << 28; // sums past the binade are only compared against 2^24
+
+__device__ __forceinline__ ParityStep compose_steps(const ParityStep& first, const ParityStep& second)
+{
+    ParityStep r;
+    r.even = first.even + ((first.even & 1u) ? second.odd : second.even);
+    r.odd = first.odd + ((first.odd & 1u) ? second.even : second.odd);
+    r.even = min(r.even, kStepCap);
+    r.odd = min(r.odd, kStepCap);
+    return r;
+}
+
+// Biased exponent (denormals and zero share exponent 1) and integer mantissa of a non-negative float:
+// value = mantissa * 2^(exponent - 150).
+__device__ __forceinline__ void decode_sum(float value, int& exponent, uint32_t& mantissa)
+{
+    const uint32_t bits = __float_as_uint(value);
+    exponent = static_cast<int>(bits >> 23);
+    mantissa = bits & 0x7fffffu;
+    if (exponent == 0)
+        exponent = 1;
+    else
+        mantissa |= 0x800000u;
+}
+
+__device__ __forceinline__ float encode_sum(int exponent, uint32_t mantissa)
+{
+    return __uint_as_float((static_cast<uint32_t>(exponent - 1) << 23) + mantissa);
+}
+
+// The step a term causes on a sum with biased exponent `exponent`.
+__device__ __forceinline__ ParityStep step_of_term(float term, int exponent)
+{
+    int term_exponent;
+    uint32_t term_mantissa;
+    decode_sum(term, term_exponent, term_mantissa);
+    ParityStep step;
+    const int shift = exponent - term_exponent;
+    if (term_mantissa == 0u || shift >= 25)
+    {
+        step.even = 0u;
+        step.odd = 0u;
+    }
+    else if (shift <= 0)
+    {
+        step.even = kBinadeFull; // at least half the sum: the addition leaves the binade
+        step.odd = kBinadeFull;
+    }
+    else
+    {
+        const uint32_t whole = term_mantissa >> shift;
+        const uint32_t rest = term_mantissa & ((1u << shift) - 1u);
+        const uint32_t half = 1u << (shift - 1);
+        if (rest > half)
+        {
+            step.even = whole + 1u;
+            step.odd = whole + 1u;
+        }
+        else if (rest < half)
+        {
+            step.even = whole;
+            step.odd = whole;
+        }
+        else
+        {
+            step.even = whole + (whole & 1u);
+            step.odd = whole + 1u - (whole & 1u);
+        }
+    }
+    return step;
+}
+
+enum StopMode : int
+{
+    kStopNever = 0,
+    kStopAtOrAbove = 1, // first partial sum s with s >= bound
+    kStopAbove = 2      // first partial sum s with s > bound
+};
+
+// Smallest mantissa (at biased exponent `exponent`) whose sum satisfies the stop condition.
+__device__ __forceinline__ uint32_t stop_mantissa(int mode, float bound, int exponent)
+{
+    if (mode == kStopNever)
+        return 0xffffffffu;
+    int bound_exponent;
+    uint32_t bound_mantissa;
+    decode_sum(bound, bound_exponent, bound_mantissa);
+    if (bound_exponent > exponent)
+        return 0xffffffffu; // not inside this binade
+    const int shift = exponent - bound_exponent;
+    if (shift == 0)
+        return mode == kStopAtOrAbove ? bound_mantissa : bound_mantissa + 1u;
+    if (shift >= 25)
+        return (mode == kStopAtOrAbove && bound_mantissa == 0u) ? 0u : 1u;
+    const uint32_t whole = bound_mantissa >> shift;
+    const uint32_t rest = bound_mantissa & ((1u << shift) - 1u);
+    if (mode == kStopAtOrAbove)
+        return whole + (rest != 0u ? 1u : 0u);
+    return whole + 1u;
+}
+
+constexpr int kReplayWaves = kReplayThreads / kWaveSize;
+
+struct ReplayScratch
+{
+    ParityStep wave_totals[kReplayWaves];
+    uint32_t first_event; // (index << 1 | kind) of the earliest event of the round, kind 0 = leaves the binade, 1 = stop
+    uint32_t final_mantissa;
+    float event_sum;
+    int absorbed;
+};
+
+struct RunningSum
+{
+    float sum;          // the sum after the last term processed (after the stopping term if stopped)
+    uint32_t stop_index; // index of the term at which the stop condition first held
+    bool stopped;
+};
+
+// One sorted row seen as a sequence of terms; `phase` selects what the CPU loop adds:
+//   0  exp(logit/T - maximum)                                  (session.cpp:98-100)
+//   1  the above divided by the normaliser                     (session.cpp:105, :123)
+//   2  the above divided by the renormaliser                   (session.cpp:134, :437)
+struct SortedRow
+{
+    const uint32_t* keys;
+    float temperature;
+    float maximum;
+    float normalizer;
+    float renormalizer;
+};
+
+template <int PHASE>
+__device__ __forceinline__ float row_term(const SortedRow& row, uint32_t i)
+{
+    float t = expf_libm(value_from_descending_key(row.keys[i]) / row.temperature - row.maximum);
+    if (PHASE >= 1)
+        t = t / row.normalizer;
+    if (PHASE >= 2)
+        t = t / row.renormalizer;
+    return t;
+}
+
+// The running fp32 sum of terms [0, count) of the row, starting from 0, exactly as a sequential
+// loop produces it.  PHASE 0 also stops (without `stopped`) once the sum no longer moves, which
+// is final because the terms are non-increasing.  Every thread of the workgroup must call it.
+template <int PHASE>
+__device__ __forceinline__ RunningSum exact_running_sum(
+    const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
+{
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    float sum = 0.0f;
+    for (uint32_t base = 0; base < count; base += kReplayChunk)
+    {
+        const uint32_t chunk_end = min(count, base + static_cast<uint32_t>(kReplayChunk));
+        const uint32_t thread_first = base + static_cast<uint32_t>(tid) * kReplayPerThread;
+        float terms[kReplayPerThread];
+#pragma unroll
+        for (int j = 0; j < kReplayPerThread; ++j)
+        {
+            const uint32_t i = thread_first + j;
+            terms[j] = i < chunk_end ? row_term<PHASE>(row, i) : 0.0f;
+        }
+        uint32_t start = base;
+        while (start < chunk_end)
+        {
+            int exponent;
+            uint32_t mantissa;
+            decode_sum(sum, exponent, mantissa);
+            const uint32_t stop_at = stop_mantissa(mode, bound, exponent);
+
+            ParityStep thread_total{0u, 0u};
+            ParityStep first_step{0u, 0u};
+#pragma unroll
+            for (int j = 0; j < kReplayPerThread; ++j)
+            {
+                const uint32_t i = thread_first + j;
+                ParityStep step{0u, 0u};
+                if (i >= start && i < chunk_end)
+                    step = step_of_term(terms[j], exponent);
+                if (j == 0)
+                    first_step = step;
+                thread_total = compose_steps(thread_total, step);
+            }
+            if (tid == 0)
+            {
+                scratch.first_event = 0xffffffffu;
+                // the largest remaining term of the row does not move the sum: nothing later can
+                scratch.absorbed = (PHASE == 0 && start == base && base > 0 && first_step.even == 0u && first_step.odd == 0u) ? 1 : 0;
+            }
+            // inclusive scan of the per-thread totals across the wave, then across waves
+            ParityStep inclusive = thread_total;
+#pragma unroll
+            for (int step = 1; step < kWaveSize; step <<= 1)
+            {
+                ParityStep earlier;
+                earlier.even = __shfl_up(inclusive.even, step, kWaveSize);
+                earlier.odd = __shfl_up(inclusive.odd, step, kWaveSize);
+                if (lane >= step)
+                    inclusive = compose_steps(earlier, inclusive);
+            }
+            ParityStep exclusive;
+            exclusive.even = __shfl_up(inclusive.even, 1, kWaveSize);
+            exclusive.odd = __shfl_up(inclusive.odd, 1, kWaveSize);
+            if (lane == 0)
+                exclusive = ParityStep{0u, 0u};
+            if (lane == kWaveSize - 1)
+                scratch.wave_totals[wave] = inclusive;
+            __syncthreads();
+            if (scratch.absorbed)
+                return RunningSum{sum, 0u, false};
+            ParityStep before{0u, 0u};
+            for (int w = 0; w < wave; ++w)
+                before = compose_steps(before, scratch.wave_totals[w]);
+            before = compose_steps(before, exclusive);
+            uint32_t current = mantissa + ((mantissa & 1u) ? before.odd : before.even);
+
+            // walk this thread's terms with the true mantissa; remember the first event
+            bool have_event = false;
+            uint32_t event_key = 0;
+            uint32_t event_mantissa = 0;
+            float event_term = 0.0f;
+#pragma unroll
+            for (int j = 0; j < kReplayPerThread; ++j)
+            {
+                const uint32_t i = thread_first + j;
+                const bool active = i >= start && i < chunk_end;
+                ParityStep step{0u, 0u};
+                if (active)
+                    step = step_of_term(terms[j], exponent);
+                const uint32_t next = current + ((current & 1u) ? step.odd : step.even);
+                if (active && !have_event)
+                {
+                    if (next >= kBinadeFull)
+                    {
+                        have_event = true;
+                        event_key = i << 1;
+                        event_mantissa = current;
+                        event_term = terms[j];
+                    }
+                    else if (next >= stop_at)
+                    {
+                        have_event = true;
+                        event_key = (i << 1) | 1u;
+                        event_mantissa = next;
+                    }
+                }
+                current = next;
+            }
+            if (have_event)
+                atomicMin(&scratch.first_event, event_key);
+            if (tid == kReplayThreads - 1)
+                scratch.final_mantissa = current;
+            __syncthreads();
+            const uint32_t event = scratch.first_event;
+            if (event == 0xffffffffu)
+            {
+                sum = encode_sum(exponent, scratch.final_mantissa);
+                __syncthreads();
+                break;
+            }
+            if (have_event && event_key == event)
+            {
+                const float at_event = encode_sum(exponent, event_mantissa);
+                scratch.event_sum = (event & 1u) ? at_event : at_event + event_term;
+            }
+            __syncthreads();
+            sum = scratch.event_sum;
+            const uint32_t event_index = event >> 1;
+            __syncthreads();
+            if (event & 1u)
+                return RunningSum{sum, event_index, true};
+            if ((mode == kStopAtOrAbove && sum >= bound) || (mode == kStopAbove && sum > bound))
+                return RunningSum{sum, event_index, true};
+            start = event_index + 1u;
+        }
+    }
+    return RunningSum{sum, 0u, false};
+}
+
+// Walks the sorted row as the CPU sampler does (src/engine/session.cpp:84-134, :429-442), with
+// every running sum reproduced exactly by exact_running_sum.  One workgroup per row.
 __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerArgs a)
 {
     const uint32_t row = blockIdx.x;
@@ -1045,18 +1313,13 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     const uint32_t* indices = a.sort_indices[1] + row * a.sort_stride;
     const uint32_t vocab = a.vocab;
 
-    __shared__ float chunk[kReplayChunk];
-    __shared__ float shared_value;
-    __shared__ float shared_cumulative;
-    __shared__ uint32_t shared_count;
-    __shared__ int shared_stop;
-    __shared__ int shared_selected;
+    __shared__ ReplayScratch scratch;
 
     uint8_t flags = NCNN_MOE_ROW_FLAG_GENERAL_PATH;
     {
         uint32_t effective_k = 0;
         int status = 0;
-        if (resolve_row_mode(p, vocab, a.segments, 0, effective_k, status) == kModeTopK && !a.force_general)
+        if (resolve_row_mode(p, vocab, a.segments, 0, effective_k, status) != kModeGeneral)
             flags |= NCNN_MOE_ROW_FLAG_FALLBACK;
     }
     if (keys[vocab - 1] == 0xffffffffu)
@@ -1108,119 +1371,55 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     if (p.top_k > 0 && p.top_k < vocab && n > p.top_k)
         n = p.top_k;
 
-    const float temperature = p.temperature;
-    const float maximum = value_from_descending_key(first_key) / temperature;
+    SortedRow sorted;
+    sorted.keys = keys;
+    sorted.temperature = p.temperature;
+    sorted.maximum = value_from_descending_key(first_key) / p.temperature;
+    sorted.normalizer = 1.0f;
+    sorted.renormalizer = 1.0f;
 
-    // ---- normaliser: sequential sum in sorted order; stops once the sum no longer moves, which is
-    // exact because the terms are non-increasing
-    if (tid == 0)
-    {
-        shared_value = 0.0f;
-        shared_stop = 0;
-    }
-    __syncthreads();
-    for (uint32_t base = 0; base < n; base += kReplayChunk)
-    {
-        for (int j = tid; j < kReplayChunk; j += kReplayThreads)
-        {
-            const uint32_t i = base + j;
-            chunk[j] = i < n ? expf_libm(value_from_descending_key(keys[i]) / temperature - maximum) : 0.0f;
-        }
-        __syncthreads();
-        if (tid == 0)
-        {
-            float sum = shared_value;
-            const uint32_t count = n - base < kReplayChunk ? n - base : kReplayChunk;
-            if (base > 0 && sum + chunk[0] == sum)
-            {
-                shared_stop = 1;
-            }
-            else
-            {
-                for (uint32_t j = 0; j < count; ++j)
-                    sum += chunk[j];
-                shared_value = sum;
-            }
-        }
-        __syncthreads();
-        if (shared_stop)
-            break;
-    }
-    const float normalizer = shared_value;
+    // ---- normaliser (session.cpp:92-103).  A first term that is not finite poisons the sum.
+    const float first_term = row_term<0>(sorted, 0);
+    float normalizer = first_term;
+    if (is_finite_f32(first_term))
+        normalizer = exact_running_sum<0>(sorted, n, kStopNever, 0.0f, scratch, tid).sum;
     if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
     {
         if (tid == 0)
             write_error(a, row, NCNN_MOE_ROW_INVALID_DISTRIBUTION, flags);
         return;
     }
+    sorted.normalizer = normalizer;
 
-    // ---- Min-P and Top-P: probabilities are non-increasing, so both keep a prefix
-    const float top_probability = expf_libm(value_from_descending_key(first_key) / temperature - maximum) / normalizer;
-    const float min_p_threshold = top_probability * p.min_p;
-    const bool use_min_p = p.min_p > 0.0f;
-    __syncthreads();
-    if (tid == 0)
+    // ---- Min-P (session.cpp:107-117): probabilities are non-increasing, so the survivors are a prefix
+    uint32_t candidates = n;
+    if (p.min_p > 0.0f)
     {
-        shared_cumulative = 0.0f;
-        shared_count = 0;
-        shared_stop = 0;
-    }
-    __syncthreads();
-    for (uint32_t base = 0; base < n; base += kReplayChunk)
-    {
-        for (int j = tid; j < kReplayChunk; j += kReplayThreads)
+        const float threshold = row_term<1>(sorted, 0) * p.min_p;
+        uint32_t first = 0, last = n; // first position whose probability is below the threshold
+        while (first < last)
         {
-            const uint32_t i = base + j;
-            float probability = -1.0f;
-            if (i < n)
-            {
-                probability = expf_libm(value_from_descending_key(keys[i]) / temperature - maximum) / normalizer;
-                if (use_min_p && !(probability >= min_p_threshold))
-                    probability = -1.0f;
-            }
-            chunk[j] = probability;
+            const uint32_t middle = (first + last) >> 1;
+            if (row_term<1>(sorted, middle) >= threshold)
+                first = middle + 1;
+            else
+                last = middle;
         }
-        __syncthreads();
-        if (tid == 0)
-        {
-            float cumulative = shared_cumulative;
-            uint32_t count = shared_count;
-            int stop = 0;
-            for (int j = 0; j < kReplayChunk; ++j)
-            {
-                const float probability = chunk[j];
-                if (probability < 0.0f)
-                {
-                    stop = 1; // end of the row or first candidate under the Min-P threshold
-                    break;
-                }
-                cumulative += probability;
-                ++count;
-                if (cumulative >= p.top_p)
-                {
-                    stop = 1;
-                    break;
-                }
-            }
-            shared_cumulative = cumulative;
-            shared_count = count;
-            shared_stop = stop;
-        }
-        __syncthreads();
-        if (shared_stop)
-            break;
+        candidates = first;
     }
-    const uint32_t kept = shared_count;
-    const float renormalizer = shared_cumulative;
+
+    // ---- Top-P (session.cpp:119-128) and the renormaliser (:130-132), which adds the same values
+    const RunningSum nucleus = exact_running_sum<1>(sorted, candidates, kStopAtOrAbove, p.top_p, scratch, tid);
+    const uint32_t kept = nucleus.stopped ? nucleus.stop_index + 1u : candidates;
+    sorted.renormalizer = nucleus.sum;
 
     if (a.distribution_count != nullptr && row == 0)
     {
         const uint32_t limit = kept < a.distribution_cap ? kept : a.distribution_cap;
         for (uint32_t i = tid; i < limit; i += kReplayThreads)
         {
-            const float probability = expf_libm(value_from_descending_key(keys[i]) / temperature - maximum) / normalizer;
             a.distribution_ids[i] = static_cast<int32_t>(indices[i]);
-            a.distribution_probabilities[i] = probability / renormalizer;
+            a.distribution_probabilities[i] = row_term<2>(sorted, i);
         }
         if (tid == 0)
             *a.distribution_count = kept;
@@ -1233,51 +1432,12 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
         return;
     }
 
-    // ---- inverse-CDF draw over the kept prefix
-    const float uniform = a.uniforms[row];
-    __syncthreads();
+    // ---- inverse-CDF draw over the kept prefix (session.cpp:432-442)
+    const RunningSum draw = exact_running_sum<2>(sorted, kept, kStopAbove, a.uniforms[row], scratch, tid);
     if (tid == 0)
     {
-        shared_cumulative = 0.0f;
-        shared_selected = -1;
-    }
-    __syncthreads();
-    for (uint32_t base = 0; base < kept; base += kReplayChunk)
-    {
-        for (int j = tid; j < kReplayChunk; j += kReplayThreads)
-        {
-            const uint32_t i = base + j;
-            float probability = 0.0f;
-            if (i < kept)
-                probability = (expf_libm(value_from_descending_key(keys[i]) / temperature - maximum) / normalizer) / renormalizer;
-            chunk[j] = probability;
-        }
-        __syncthreads();
-        if (tid == 0)
-        {
-            float cumulative = shared_cumulative;
-            const uint32_t count = kept - base < kReplayChunk ? kept - base : kReplayChunk;
-            for (uint32_t j = 0; j < count; ++j)
-            {
-                cumulative += chunk[j];
-                if (uniform < cumulative)
-                {
-                    shared_selected = static_cast<int>(base + j);
-                    break;
-                }
-            }
-            shared_cumulative = cumulative;
-        }
-        __syncthreads();
-        if (shared_selected >= 0)
-            break;
-    }
-    if (tid == 0)
-    {
-        const uint32_t selected = shared_selected >= 0 ? static_cast<uint32_t>(shared_selected) : kept - 1;
-        const float probability =
-            (expf_libm(value_from_descending_key(keys[selected]) / temperature - maximum) / normalizer) / renormalizer;
-        write_token(a, row, p, static_cast<int32_t>(indices[selected]), probability, kept, 1, flags);
+        const uint32_t selected = draw.stopped ? draw.stop_index : kept - 1u;
+        write_token(a, row, p, static_cast<int32_t>(indices[selected]), row_term<2>(sorted, selected), kept, 1, flags);
     }
 }
 
