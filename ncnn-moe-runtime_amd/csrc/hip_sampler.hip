@@ -172,11 +172,23 @@ int launch_sampler(
     }
     if (full_order_pass)
     {
+        // the token indices ride along with the keys only when the whole distribution is exported
         if (dtype == NCNN_MOE_LOGITS_F32)
-            hipLaunchKernelGGL(general_sort_kernel<NCNN_MOE_LOGITS_F32>, dim3(rows), dim3(kSortThreads), 0, stream, a);
+        {
+            if (want_distribution)
+                hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_F32, true>), dim3(rows), dim3(kSortThreads), 0, stream, a);
+            else
+                hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_F32, false>), dim3(rows), dim3(kSortThreads), 0, stream, a);
+            hipLaunchKernelGGL(general_replay_kernel<NCNN_MOE_LOGITS_F32>, dim3(rows), dim3(kReplayThreads), 0, stream, a);
+        }
         else
-            hipLaunchKernelGGL(general_sort_kernel<NCNN_MOE_LOGITS_BF16>, dim3(rows), dim3(kSortThreads), 0, stream, a);
-        hipLaunchKernelGGL(general_replay_kernel, dim3(rows), dim3(kReplayThreads), 0, stream, a);
+        {
+            if (want_distribution)
+                hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kSortThreads), 0, stream, a);
+            else
+                hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_BF16, false>), dim3(rows), dim3(kSortThreads), 0, stream, a);
+            hipLaunchKernelGGL(general_replay_kernel<NCNN_MOE_LOGITS_BF16>, dim3(rows), dim3(kReplayThreads), 0, stream, a);
+        }
     }
     SAMPLER_HIP_CHECK(s, hipGetLastError());
     return NCNN_MOE_SAMPLER_SUCCESS;

@@ -31,6 +31,8 @@ constexpr int kMergeSurvivorCap = 512;   // candidates that may survive the row-
 // Full-order ("general") path geometry.
 constexpr int kSortThreads = 1024;
 constexpr int kSortWaves = kSortThreads / kWaveSize;
+constexpr int kSortPerThread = 8;
+constexpr int kSortTile = kSortThreads * kSortPerThread;
 constexpr int kReplayThreads = 512;
 constexpr int kReplayPerThread = 8;
 constexpr int kReplayChunk = kReplayThreads * kReplayPerThread;

@@ -875,8 +875,10 @@ __device__ __forceinline__ float load_logit<NCNN_MOE_LOGITS_BF16>(const void* ro
 
 // Stable LSD radix sort (8-bit digits) of one row by descending_key; one workgroup per row.
 // fp32 rows take four passes; bf16 keys only differ in their upper 16 bits and take two.
-// The sorted keys and indices end in sort_keys[1] / sort_indices[1].
-template <int DTYPE>
+// The sorted keys end in sort_keys[1].  With PAIRS the token indices travel with the keys and end in
+// sort_indices[1] (needed only when the whole filtered distribution is exported); sampling sorts the
+// keys alone and recovers the one index it needs from the logits afterwards.
+template <int DTYPE, bool PAIRS>
 __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs a)
 {
     constexpr int kPasses = DTYPE == NCNN_MOE_LOGITS_F32 ? 4 : 2;
@@ -931,6 +933,10 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
     }
     __syncthreads();
 
+    // Every pass walks the row in tiles of 1024 x 8 elements.  A wave owns 512 consecutive elements of
+    // the tile and ranks them in 8 rounds of 64 (one element per lane), so that the order inside the
+    // wave is the input order; its per-digit running counts live in LDS.  A prefix over the 16 waves
+    // and the digit bases then turns the ranks into output positions.
     for (int pass = 0; pass < kPasses; ++pass)
     {
         const int shift = 8 * (pass + kFirstDigit);
@@ -940,37 +946,55 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
         uint32_t* target_indices = indices[pass & 1];
         if (tid < 256)
             digit_base[tid] = histogram[pass][tid];
-        for (uint32_t tile = 0; tile < n; tile += kSortThreads)
+        for (uint32_t tile = 0; tile < n; tile += kSortTile)
         {
             for (int i = tid; i < kSortWaves * 256; i += kSortThreads)
                 (&wave_counts[0][0])[i] = 0;
-            const uint32_t i = tile + tid;
-            const bool valid = i < n;
-            uint32_t key = 0xffffffffu;
-            uint32_t index = i;
-            if (valid)
+            uint32_t tile_keys[kSortPerThread];
+            uint32_t tile_indices[kSortPerThread];
+            uint32_t tile_ranks[kSortPerThread];
+            const uint32_t wave_first = tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread);
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
             {
-                if (pass == 0)
-                    key = descending_key(load_logit<DTYPE>(row_pointer, i));
-                else
+                const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+                tile_keys[e] = 0xffffffffu;
+                tile_indices[e] = i;
+                if (i < n)
                 {
-                    key = source_keys[i];
-                    index = source_indices[i];
+                    if (pass == 0)
+                        tile_keys[e] = descending_key(load_logit<DTYPE>(row_pointer, i));
+                    else
+                    {
+                        tile_keys[e] = source_keys[i];
+                        if (PAIRS)
+                            tile_indices[e] = source_indices[i];
+                    }
                 }
             }
-            const uint32_t digit = (key >> shift) & 255u;
-            uint64_t peers = __ballot(valid);
-#pragma unroll
-            for (int b = 0; b < 8; ++b)
-            {
-                const bool bit = (digit >> b) & 1u;
-                const uint64_t set = __ballot(valid && bit);
-                peers &= bit ? set : ~set;
-            }
-            const int rank_in_wave = lanes_below(peers);
             __syncthreads();
-            if (valid && rank_in_wave == 0)
-                wave_counts[wave][digit] = static_cast<uint32_t>(__popcll(peers));
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
+            {
+                const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+                const bool valid = i < n;
+                const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+                uint64_t peers = __ballot(valid);
+#pragma unroll
+                for (int b = 0; b < 8; ++b)
+                {
+                    const bool bit = (digit >> b) & 1u;
+                    const uint64_t set = __ballot(valid && bit);
+                    peers &= bit ? set : ~set;
+                }
+                const int rank_in_round = lanes_below(peers);
+                uint32_t seen = 0;
+                if (valid)
+                    seen = wave_counts[wave][digit];
+                tile_ranks[e] = seen + static_cast<uint32_t>(rank_in_round);
+                if (valid && rank_in_round == 0)
+                    wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popcll(peers));
+            }
             __syncthreads();
             if (tid < 256)
             {
@@ -985,11 +1009,18 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
                 digit_base[tid] = running;
             }
             __syncthreads();
-            if (valid)
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
             {
-                const uint32_t position = wave_counts[wave][digit] + static_cast<uint32_t>(rank_in_wave);
-                target_keys[position] = key;
-                target_indices[position] = index;
+                const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+                if (i < n)
+                {
+                    const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+                    const uint32_t position = wave_counts[wave][digit] + tile_ranks[e];
+                    target_keys[position] = tile_keys[e];
+                    if (PAIRS)
+                        target_indices[position] = tile_indices[e];
+                }
             }
             __syncthreads();
         }
@@ -1300,8 +1331,99 @@ __device__ __forceinline__ RunningSum exact_running_sum(
     return RunningSum{sum, 0u, false};
 }
 
+struct RecoverScratch
+{
+    uint32_t wave_counts[kReplayWaves];
+    int32_t found;
+};
+
+// Token index of position `rank` of the sorted row, from the logits: the sort is stable, so it is
+// the (rank - first position of that key)-th element, in index order, whose key equals keys[rank].
+// Every thread of the workgroup must call it.
+template <int DTYPE>
+__device__ __forceinline__ int32_t recover_token_index(
+    const void* row_pointer, uint32_t vocab, const uint32_t* keys, uint32_t rank, RecoverScratch& scratch, int tid)
+{
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const uint32_t key = keys[rank];
+    uint32_t low = 0, high = rank; // first position holding this key
+    while (low < high)
+    {
+        const uint32_t middle = (low + high) >> 1;
+        if (keys[middle] < key)
+            low = middle + 1;
+        else
+            high = middle;
+    }
+    const uint32_t ordinal = rank - low;
+    uint32_t passed = 0; // matches before the current chunk
+    if (tid == 0)
+        scratch.found = -1;
+    __syncthreads();
+    for (uint32_t base = 0; base < vocab; base += kReplayChunk)
+    {
+        const uint32_t first = base + static_cast<uint32_t>(tid) * kReplayPerThread;
+        uint32_t matches = 0;
+        uint32_t count = 0;
+#pragma unroll
+        for (int j = 0; j < kReplayPerThread; ++j)
+        {
+            const uint32_t i = first + j;
+            if (i < vocab && descending_key(load_logit<DTYPE>(row_pointer, i)) == key)
+            {
+                matches |= 1u << j;
+                ++count;
+            }
+        }
+        uint32_t inclusive = count;
+#pragma unroll
+        for (int step = 1; step < kWaveSize; step <<= 1)
+        {
+            const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
+            if (lane >= step)
+                inclusive += up;
+        }
+        if (lane == kWaveSize - 1)
+            scratch.wave_counts[wave] = inclusive;
+        __syncthreads();
+        uint32_t before = passed;
+        uint32_t chunk_total = 0;
+        for (int w = 0; w < kReplayWaves; ++w)
+        {
+            const uint32_t c = scratch.wave_counts[w];
+            if (w < wave)
+                before += c;
+            chunk_total += c;
+        }
+        before += inclusive - count;
+        if (ordinal >= before && ordinal < before + count)
+        {
+            uint32_t skip = ordinal - before;
+#pragma unroll
+            for (int j = 0; j < kReplayPerThread; ++j)
+            {
+                if (matches & (1u << j))
+                {
+                    if (skip == 0)
+                        scratch.found = static_cast<int32_t>(first + j);
+                    --skip;
+                }
+            }
+        }
+        __syncthreads();
+        if (scratch.found >= 0)
+            break;
+        passed += chunk_total;
+    }
+    const int32_t found = scratch.found;
+    __syncthreads();
+    return found;
+}
+
 // Walks the sorted row as the CPU sampler does (src/engine/session.cpp:84-134, :429-442), with
 // every running sum reproduced exactly by exact_running_sum.  One workgroup per row.
+template <int DTYPE>
 __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerArgs a)
 {
     const uint32_t row = blockIdx.x;
@@ -1310,10 +1432,14 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     const int tid = threadIdx.x;
     const ncnn_moe_sample_params p = a.params[row];
     const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
-    const uint32_t* indices = a.sort_indices[1] + row * a.sort_stride;
+    const uint32_t* indices = a.sort_indices[1] + row * a.sort_stride; // valid only when the distribution is exported
+    const bool have_indices = a.distribution_count != nullptr;
     const uint32_t vocab = a.vocab;
+    const char* row_pointer = static_cast<const char*>(a.logits) +
+        static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
 
     __shared__ ReplayScratch scratch;
+    __shared__ RecoverScratch recover_scratch;
 
     uint8_t flags = NCNN_MOE_ROW_FLAG_GENERAL_PATH;
     {
@@ -1340,10 +1466,15 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
             else
                 high = middle;
         }
+        const bool any_finite = low < vocab && keys[low] <= kLastFiniteKey;
+        int32_t token = -1;
+        if (any_finite)
+            token = have_indices ? static_cast<int32_t>(indices[low])
+                                 : recover_token_index<DTYPE>(row_pointer, vocab, keys, low, recover_scratch, tid);
         if (tid == 0)
         {
-            if (low < vocab && keys[low] <= kLastFiniteKey)
-                write_token(a, row, p, static_cast<int32_t>(indices[low]), 1.0f, 1u, 0, flags);
+            if (any_finite)
+                write_token(a, row, p, token, 1.0f, 1u, 0, flags);
             else
                 write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, flags);
         }
@@ -1427,18 +1558,20 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
 
     if (kept == 1)
     {
+        const int32_t token = have_indices ? static_cast<int32_t>(indices[0])
+                                           : recover_token_index<DTYPE>(row_pointer, vocab, keys, 0, recover_scratch, tid);
         if (tid == 0)
-            write_token(a, row, p, static_cast<int32_t>(indices[0]), 1.0f, 1u, 0, flags);
+            write_token(a, row, p, token, 1.0f, 1u, 0, flags);
         return;
     }
 
     // ---- inverse-CDF draw over the kept prefix (session.cpp:432-442)
     const RunningSum draw = exact_running_sum<2>(sorted, kept, kStopAbove, a.uniforms[row], scratch, tid);
+    const uint32_t selected = draw.stopped ? draw.stop_index : kept - 1u;
+    const int32_t token = have_indices ? static_cast<int32_t>(indices[selected])
+                                       : recover_token_index<DTYPE>(row_pointer, vocab, keys, selected, recover_scratch, tid);
     if (tid == 0)
-    {
-        const uint32_t selected = draw.stopped ? draw.stop_index : kept - 1u;
-        write_token(a, row, p, static_cast<int32_t>(indices[selected]), row_term<2>(sorted, selected), kept, 1, flags);
-    }
+        write_token(a, row, p, token, row_term<2>(sorted, selected), kept, 1, flags);
 }
 
 // Evaluates expf_libm on n values (test hook).
