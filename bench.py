@@ -45,6 +45,16 @@ def algorithmic_bytes(rows, vocab, element_bytes):
     return rows * vocab * element_bytes + rows * (24 + 4) + rows * 16
 
 
+def measured_traffic(workload_name):
+    """HBM bytes per launch of the dominant kernel as measured with rocprofv3 --pmc FETCH_SIZE and
+    WRITE_SIZE (each scaled by the reading of a 256 MiB copy), recorded beside the profile summaries."""
+    path = os.path.join(ROOT, "profiles", "scan_select_%s_traffic.json" % workload_name)
+    if not os.path.exists(path):
+        return None
+    with open(path) as handle:
+        return json.load(handle).get("hbm_bytes_per_launch")
+
+
 def cpu_baseline(workload, host_threads, sample_rows):
     """Times the CPU sampler on the first sample_rows rows of the workload."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -115,6 +125,9 @@ def main():
     parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
     parser.add_argument("--cpu-rows", type=int, default=64)
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--copy-calibration", type=int, default=0,
+                        help="after the timed steps, copy a 256 MiB buffer this many times (a kernel of known "
+                             "traffic for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every box of this build has one MI355X; run with --gpus 1")
@@ -187,6 +200,12 @@ def main():
         wall_seconds = time.perf_counter() - wall_start
     event_seconds = start_event.elapsed_time(stop_event) * 1e-3
     seconds_per_step = event_seconds / args.steps
+    if args.copy_calibration > 0:
+        source = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=device)
+        target = torch.empty_like(source)
+        for _ in range(args.copy_calibration):
+            target.copy_(source)
+        torch.cuda.synchronize()
 
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib
@@ -228,7 +247,7 @@ def main():
             "peak": HBM_PEAK_BYTES_PER_S / 1e9,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_BYTES_PER_S,
-            "traffic": None,
+            "traffic": measured_traffic(workload["name"]),
             "kernel": "scan_select_kernel",
             "algorithmic_bytes_per_launch": bytes_per_launch,
         },
