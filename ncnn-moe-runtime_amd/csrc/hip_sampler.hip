@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -92,40 +93,69 @@ uint64_t logits_span(uint32_t vocab, int dtype, const void* logits, uint64_t row
     return static_cast<uint64_t>(vocab) + (aligned ? 0u : width - 1u);
 }
 
-uint64_t segment_values(int dtype, int chunks)
+// How the select kernel covers a row: `segments` workgroups, each streaming `chunks_per_segment`
+// chunks.  A workgroup that sees the whole row finishes it itself and serves Top-K windows up to
+// kSelectTopK; rows split over several workgroups (small batches, so that every CU streams) are
+// merged by the last workgroup to arrive and serve windows up to kFastTopK.
+struct SelectGeometry
 {
-    return static_cast<uint64_t>(dtype == NCNN_MOE_LOGITS_F32 ? kSegmentValuesF32 : kSegmentValuesBF16) * chunks;
+    uint32_t segments = 1;
+    uint32_t chunks_per_segment = 1;
+    bool looped = true;
+    uint32_t max_top_k = kSelectTopK;
+};
+
+uint64_t chunk_values(int dtype)
+{
+    return dtype == NCNN_MOE_LOGITS_F32 ? kSegmentValuesF32 : kSegmentValuesBF16;
 }
 
-// Chunks of vectors one lane keeps in registers (1, 2 or 4).  One chunk streams fastest; longer
-// rows take more so that a row has at most kMaxSegments segments, which the row merge can stage.
-int chunks_for(int dtype, uint64_t span)
+SelectGeometry select_geometry(int dtype, uint64_t span, uint32_t rows, bool whole_row)
 {
-    for (int chunks = 1; chunks < 4; chunks <<= 1)
+    SelectGeometry g;
+    const uint64_t total_chunks = std::max<uint64_t>(1, (span + chunk_values(dtype) - 1) / chunk_values(dtype));
+    uint64_t segments = 1;
+    if (!whole_row && rows < static_cast<uint32_t>(kWholeRowBatch))
     {
-        if ((span + segment_values(dtype, chunks) - 1) / segment_values(dtype, chunks) <= static_cast<uint64_t>(kMaxSegments))
-            return chunks;
+        const uint64_t wanted = (static_cast<uint64_t>(kSelectWorkgroupTarget) + rows - 1) / rows;
+        segments = std::min<uint64_t>(std::min<uint64_t>(wanted, total_chunks), static_cast<uint64_t>(kMaxSegments));
     }
-    return 4;
+    const uint64_t chunks_per_segment = (total_chunks + segments - 1) / segments;
+    segments = (total_chunks + chunks_per_segment - 1) / chunks_per_segment;
+    g.segments = static_cast<uint32_t>(segments);
+    g.chunks_per_segment = static_cast<uint32_t>(chunks_per_segment);
+    g.looped = chunks_per_segment > 1 || segments == 1;
+    g.max_top_k = segments == 1 ? static_cast<uint32_t>(kSelectTopK) : static_cast<uint32_t>(kFastTopK);
+    return g;
 }
 
 template <int DTYPE>
-void launch_scan(int chunks, dim3 grid, hipStream_t stream, const SamplerArgs& a)
+void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, SamplerArgs a, bool only_pending)
 {
-    if (chunks == 4)
-        hipLaunchKernelGGL((scan_select_kernel<DTYPE, 4>), grid, dim3(kScanThreads), 0, stream, a);
-    else if (chunks == 2)
-        hipLaunchKernelGGL((scan_select_kernel<DTYPE, 2>), grid, dim3(kScanThreads), 0, stream, a);
+    a.segments = g.segments;
+    a.chunks_per_segment = g.chunks_per_segment;
+    a.max_select_top_k = g.max_top_k;
+    a.only_pending = only_pending ? 1 : 0;
+    const dim3 grid(g.segments, rows, 1);
+    if (g.looped)
+        hipLaunchKernelGGL((scan_select_kernel<DTYPE, true>), grid, dim3(kScanThreads), 0, stream, a);
     else
-        hipLaunchKernelGGL((scan_select_kernel<DTYPE, 1>), grid, dim3(kScanThreads), 0, stream, a);
+        hipLaunchKernelGGL((scan_select_kernel<DTYPE, false>), grid, dim3(kScanThreads), 0, stream, a);
 }
 
-// Enqueues the whole sampling path for `rows` rows.
+// Which kernels a call enqueues.  Rows a pass cannot serve are marked pending and taken by the next.
+struct SamplerPasses
+{
+    bool select = true;      // the batch-shaped select kernel
+    bool wide_select = false; // one workgroup per pending row: Top-K windows up to kSelectTopK
+    bool full_order = false; // sort + replay for every row still pending
+};
+
+// Enqueues the sampling path for `rows` rows.
 int launch_sampler(
     ncnn_moe_hip_sampler* s, const void* logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
     const ncnn_moe_sample_params* params, const float* uniforms, const int32_t* stop_ids,
-    ncnn_moe_sample_result* results, bool want_distribution, bool select_pass, bool full_order_pass,
-    hipStream_t stream)
+    ncnn_moe_sample_result* results, bool want_distribution, SamplerPasses passes, hipStream_t stream)
 {
     SamplerArgs a;
     std::memset(&a, 0, sizeof(a));
@@ -134,8 +164,6 @@ int launch_sampler(
     a.rows = rows;
     a.vocab = vocab;
     const uint64_t span = logits_span(vocab, dtype, logits, row_stride);
-    const int chunks = chunks_for(dtype, span);
-    a.segments = static_cast<uint32_t>((span + segment_values(dtype, chunks) - 1) / segment_values(dtype, chunks));
     a.force_general = s->force_general;
     a.params = params;
     a.uniforms = uniforms;
@@ -159,18 +187,26 @@ int launch_sampler(
         a.distribution_cap = s->max_vocab;
         a.distribution_count = s->distribution_count;
     }
-    if (a.segments > s->max_segments)
+    const SelectGeometry batch_geometry = select_geometry(dtype, span, rows, false);
+    if (batch_geometry.segments > s->max_segments)
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab exceeds the handle's max_vocab");
 
-    const dim3 scan_grid(a.segments, rows, 1);
-    if (select_pass)
+    if (passes.select)
     {
         if (dtype == NCNN_MOE_LOGITS_F32)
-            launch_scan<NCNN_MOE_LOGITS_F32>(chunks, scan_grid, stream, a);
+            launch_select<NCNN_MOE_LOGITS_F32>(batch_geometry, rows, stream, a, false);
         else
-            launch_scan<NCNN_MOE_LOGITS_BF16>(chunks, scan_grid, stream, a);
+            launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, a, false);
     }
-    if (full_order_pass)
+    if (passes.wide_select && batch_geometry.segments > 1)
+    {
+        const SelectGeometry row_geometry = select_geometry(dtype, span, rows, true);
+        if (dtype == NCNN_MOE_LOGITS_F32)
+            launch_select<NCNN_MOE_LOGITS_F32>(row_geometry, rows, stream, a, true);
+        else
+            launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, stream, a, true);
+    }
+    if (passes.full_order)
     {
         // the token indices ride along with the keys only when the whole distribution is exported
         if (dtype == NCNN_MOE_LOGITS_F32)
@@ -194,15 +230,12 @@ int launch_sampler(
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 
-// Host-side twin of resolve_row_mode: does the row's SamplingOptions send it to the full-order path?
-bool row_needs_full_order(const ncnn_moe_sample_params& p, uint32_t vocab)
+// Would a select kernel serving windows up to max_top_k leave the row to a later pass?
+bool row_left_pending(const ncnn_moe_sample_params& p, uint32_t vocab, uint32_t max_top_k)
 {
-    const bool valid = std::isfinite(p.temperature) && p.temperature >= 0.0f && std::isfinite(p.top_p) &&
-        p.top_p > 0.0f && p.top_p <= 1.0f && std::isfinite(p.min_p) && p.min_p >= 0.0f && p.min_p <= 1.0f;
-    if (!valid || p.temperature == 0.0f)
-        return false;
-    const uint32_t effective_k = (p.top_k == 0u || p.top_k >= vocab) ? vocab : p.top_k;
-    return effective_k > static_cast<uint32_t>(kFastTopK);
+    uint32_t effective_k = 0;
+    int status = NCNN_MOE_ROW_OK;
+    return resolve_row_mode(p, vocab, max_top_k, 0, effective_k, status) == kModeGeneral;
 }
 
 int check_shape(ncnn_moe_hip_sampler* s, int dtype, uint32_t rows, uint32_t vocab)
@@ -247,7 +280,8 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     s->device = device;
     s->max_rows = max_rows;
     s->max_vocab = max_vocab;
-    s->max_segments = static_cast<uint32_t>((static_cast<uint64_t>(max_vocab) + 7 + kSegmentValuesF32 - 1) / kSegmentValuesF32);
+    s->max_segments = static_cast<uint32_t>(std::min<uint64_t>(
+        static_cast<uint64_t>(kMaxSegments), (static_cast<uint64_t>(max_vocab) + 7 + kSegmentValuesF32 - 1) / kSegmentValuesF32));
     s->logits_stride_f32 = round_up(max_vocab, 8);
     s->sort_stride = round_up(max_vocab, 4);
 
@@ -405,14 +439,19 @@ int ncnn_moe_hip_sampler_sample(
     SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->uniforms, uniforms, rows * sizeof(float), hipMemcpyHostToDevice, s->stream));
     if (stop_id_count > 0)
         SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->stop_ids, stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t), hipMemcpyHostToDevice, s->stream));
-    // the host sees the options: the full-order kernels are enqueued only if some row needs them
-    bool full_order = s->force_general != 0;
-    for (uint32_t row = 0; row < rows && !full_order; ++row)
-        full_order = row_needs_full_order(params[row], s->logits_vocab);
+    // the host sees the options: the later passes are enqueued only if some row needs them
+    SamplerPasses passes;
+    passes.full_order = s->force_general != 0;
+    for (uint32_t row = 0; row < rows; ++row)
+    {
+        passes.wide_select = passes.wide_select || row_left_pending(params[row], s->logits_vocab, kFastTopK);
+        passes.full_order = passes.full_order || row_left_pending(params[row], s->logits_vocab, kSelectTopK);
+    }
+    const bool full_order = passes.full_order;
     const int32_t* device_stops = stop_id_count > 0 ? s->stop_ids : nullptr;
     int rc = launch_sampler(
         s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-        s->params, s->uniforms, device_stops, s->results, false, true, full_order, s->stream);
+        s->params, s->uniforms, device_stops, s->results, false, passes, s->stream);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return rc;
     SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
@@ -425,9 +464,12 @@ int ncnn_moe_hip_sampler_sample(
             pending = results[row].status == NCNN_MOE_ROW_NEEDS_FULL_ORDER;
         if (pending)
         {
+            SamplerPasses retry;
+            retry.select = false;
+            retry.full_order = true;
             rc = launch_sampler(
                 s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-                s->params, s->uniforms, device_stops, s->results, false, false, true, s->stream);
+                s->params, s->uniforms, device_stops, s->results, false, retry, s->stream);
             if (rc != NCNN_MOE_SAMPLER_SUCCESS)
                 return rc;
             SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
@@ -454,9 +496,12 @@ int ncnn_moe_hip_sampler_sample_device(
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab must be positive");
     if (row_stride < vocab)
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "row_stride is smaller than vocab");
+    SamplerPasses passes;
+    passes.wide_select = may_need_full_order != 0;
+    passes.full_order = may_need_full_order != 0 || s->force_general != 0;
     return launch_sampler(
         s, device_logits, dtype, rows, vocab, row_stride, device_params, device_uniforms, device_stop_ids,
-        device_results, false, true, may_need_full_order != 0 || s->force_general != 0, static_cast<hipStream_t>(stream));
+        device_results, false, passes, static_cast<hipStream_t>(stream));
 }
 
 int ncnn_moe_hip_sampler_distribution(
@@ -484,9 +529,11 @@ int ncnn_moe_hip_sampler_distribution(
     SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->single_uniform, &uniform, sizeof(uniform), hipMemcpyHostToDevice, s->stream));
     const size_t element = s->logits_dtype == NCNN_MOE_LOGITS_F32 ? 4 : 2;
     const char* row_logits = static_cast<const char*>(s->logits) + static_cast<size_t>(row) * s->logits_stride * element;
+    SamplerPasses distribution_passes;
+    distribution_passes.full_order = true;
     const int rc = launch_sampler(
         s, row_logits, s->logits_dtype, 1, s->logits_vocab, s->logits_stride,
-        s->single_params, s->single_uniform, nullptr, s->single_result, true, true, true, s->stream);
+        s->single_params, s->single_uniform, nullptr, s->single_result, true, distribution_passes, s->stream);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return rc;
     ncnn_moe_sample_result result;

@@ -1,0 +1,519 @@
+// Shared pieces of the sampler kernels: launch arguments, result writers, logits vector traits,
+// agent-scope accesses, integer keys, wave-level selection, and the one-wave epilogue.
+#ifndef NCNN_MOE_HIP_SAMPLER_COMMON_H
+#define NCNN_MOE_HIP_SAMPLER_COMMON_H
+
+#include "sampler_device.h"
+
+namespace ncnn_moe_hip {
+
+struct SamplerArgs
+{
+    const void* logits;
+    uint64_t row_stride; // elements
+    uint32_t rows;
+    uint32_t vocab;
+    uint32_t segments;           // workgroups per row in the select kernel
+    uint32_t chunks_per_segment; // chunks (512 x 5 fp32 / 3 bf16 vectors) one workgroup streams
+    uint32_t max_select_top_k;   // widest Top-K window the select kernel of this launch serves
+    int force_general;
+    int only_pending;            // serve only rows an earlier launch of the call left pending
+
+    const ncnn_moe_sample_params* params;
+    const float* uniforms;
+    const int32_t* stop_ids;
+    ncnn_moe_sample_result* results;
+
+    // select-path scratch
+    float* segment_values;     // [rows][segments][kSegmentRecordSlots]
+    int32_t* segment_indices;  // [rows][segments][kSegmentRecordSlots]
+    uint32_t* segment_counts;  // [rows][segments]
+    uint32_t* row_counter;     // [rows], zero between launches
+    uint32_t* row_flags;       // [rows], zero between launches
+    uint32_t* row_state;       // [rows], written by every launch
+
+    // general-path scratch, [rows][sort_stride] each
+    uint32_t* sort_keys[2];
+    uint32_t* sort_indices[2];
+    uint64_t sort_stride;
+
+    // optional filtered-distribution output for row 0 of the launch
+    int32_t* distribution_ids;
+    float* distribution_probabilities;
+    uint32_t distribution_cap;
+    uint32_t* distribution_count;
+};
+
+__device__ __forceinline__ uint8_t stop_flag(const SamplerArgs& a, const ncnn_moe_sample_params& p, int32_t token)
+{
+    if (a.stop_ids == nullptr)
+        return 0;
+    for (uint32_t i = 0; i < p.stop_count; ++i)
+    {
+        if (a.stop_ids[p.stop_begin + i] == token)
+            return 1;
+    }
+    return 0;
+}
+
+__device__ __forceinline__ void write_error(const SamplerArgs& a, uint32_t row, int status, uint8_t flags)
+{
+    ncnn_moe_sample_result r;
+    r.token_id = -1;
+    r.probability = 0.0f;
+    r.kept_count = 0;
+    r.status = static_cast<uint8_t>(status);
+    r.is_stop = 0;
+    r.draw_consumed = 0;
+    r.flags = flags;
+    a.results[row] = r;
+    if (a.distribution_count != nullptr && row == 0)
+        *a.distribution_count = 0;
+}
+
+// Marks a row that still has to go through the full-order kernels.
+__device__ __forceinline__ void write_pending(const SamplerArgs& a, uint32_t row)
+{
+    ncnn_moe_sample_result r;
+    r.token_id = -1;
+    r.probability = 0.0f;
+    r.kept_count = 0;
+    r.status = NCNN_MOE_ROW_NEEDS_FULL_ORDER;
+    r.is_stop = 0;
+    r.draw_consumed = 0;
+    r.flags = 0;
+    a.results[row] = r;
+}
+
+__device__ __forceinline__ void write_token(
+    const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
+    int32_t token, float probability, uint32_t kept, uint8_t draw_consumed, uint8_t flags)
+{
+    ncnn_moe_sample_result r;
+    r.token_id = token;
+    r.probability = probability;
+    r.kept_count = kept;
+    r.status = NCNN_MOE_ROW_OK;
+    r.is_stop = stop_flag(a, p, token);
+    r.draw_consumed = draw_consumed;
+    r.flags = flags;
+    a.results[row] = r;
+}
+
+// The CPU sampler from the sorted Top-K window onwards (src/engine/session.cpp:89-134, :429-442),
+// executed by one wave: lane i holds candidate i of n <= 64 candidates in (logit descending, index
+// ascending) order.  Sums run in candidate order on every lane redundantly.
+__device__ __forceinline__ void finish_row_wave(
+    const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
+    float value, int32_t index, int n, int lane, uint8_t flags)
+{
+    const float temperature = p.temperature;
+    const float top_value = read_lane(value, 0);
+    const float maximum = top_value / temperature;
+    float term = 0.0f;
+    if (lane < n)
+        term = expf_libm(value / temperature - maximum);
+
+    float normalizer = 0.0f;
+    for (int i = 0; i < n; ++i)
+        normalizer += read_lane(term, i);
+    if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
+    {
+        if (lane == 0)
+            write_error(a, row, NCNN_MOE_ROW_INVALID_DISTRIBUTION, flags);
+        return;
+    }
+    const float probability = term / normalizer;
+
+    bool keep = lane < n;
+    if (p.min_p > 0.0f)
+    {
+        const float threshold = read_lane(probability, 0) * p.min_p;
+        keep = keep && (probability >= threshold);
+    }
+    uint64_t pending = __ballot(keep);
+
+    float cumulative = 0.0f;
+    uint64_t kept_mask = 0;
+    int kept = 0;
+    while (pending != 0)
+    {
+        const int i = __builtin_ctzll(pending);
+        pending &= pending - 1;
+        cumulative += read_lane(probability, i);
+        kept_mask |= 1ull << i;
+        ++kept;
+        if (cumulative >= p.top_p)
+            break;
+    }
+    // The renormaliser of session.cpp:130-132 adds the same values in the same order as the Top-P scan.
+    const float renormalizer = cumulative;
+    const float final_probability = probability / renormalizer;
+
+    if (a.distribution_count != nullptr && row == 0)
+    {
+        if ((kept_mask >> lane) & 1ull)
+        {
+            const int position = lanes_below(kept_mask);
+            if (static_cast<uint32_t>(position) < a.distribution_cap)
+            {
+                a.distribution_ids[position] = index;
+                a.distribution_probabilities[position] = final_probability;
+            }
+        }
+        if (lane == 0)
+            *a.distribution_count = static_cast<uint32_t>(kept);
+    }
+
+    int selected = 0;
+    uint8_t draw_consumed = 0;
+    float selected_probability = 1.0f;
+    if (kept == 1)
+    {
+        selected = __builtin_ctzll(kept_mask);
+    }
+    else
+    {
+        draw_consumed = 1;
+        const float uniform = a.uniforms[row];
+        float running = 0.0f;
+        uint64_t walk = kept_mask;
+        selected = 63 - __builtin_clzll(kept_mask);
+        while (walk != 0)
+        {
+            const int i = __builtin_ctzll(walk);
+            walk &= walk - 1;
+            running += read_lane(final_probability, i);
+            if (uniform < running)
+            {
+                selected = i;
+                break;
+            }
+        }
+        selected_probability = read_lane(final_probability, selected);
+    }
+    const int32_t token = read_lane(index, selected);
+    if (lane == 0)
+        write_token(a, row, p, token, selected_probability, static_cast<uint32_t>(kept), draw_consumed, flags);
+}
+
+template <int DTYPE>
+struct LogitsVector;
+
+template <>
+struct LogitsVector<NCNN_MOE_LOGITS_F32>
+{
+    static constexpr int kWidth = 4;
+    static constexpr int kElementBytes = 4;
+    static constexpr int kVectorsPerLane = kVectorsPerLaneF32;
+    __device__ static __forceinline__ void unpack(const uint4& raw, float* out)
+    {
+        out[0] = __uint_as_float(raw.x);
+        out[1] = __uint_as_float(raw.y);
+        out[2] = __uint_as_float(raw.z);
+        out[3] = __uint_as_float(raw.w);
+    }
+};
+
+template <>
+struct LogitsVector<NCNN_MOE_LOGITS_BF16>
+{
+    static constexpr int kWidth = 8;
+    static constexpr int kElementBytes = 2;
+    static constexpr int kVectorsPerLane = kVectorsPerLaneBF16;
+    // bf16 -> fp32 is bits << 16 (src/kernels/cpu_ops.cpp:26-32); element 2i is the low half of word i.
+    __device__ static __forceinline__ void unpack(const uint4& raw, float* out)
+    {
+        out[0] = __uint_as_float(raw.x << 16);
+        out[1] = __uint_as_float(raw.x & 0xffff0000u);
+        out[2] = __uint_as_float(raw.y << 16);
+        out[3] = __uint_as_float(raw.y & 0xffff0000u);
+        out[4] = __uint_as_float(raw.z << 16);
+        out[5] = __uint_as_float(raw.z & 0xffff0000u);
+        out[6] = __uint_as_float(raw.w << 16);
+        out[7] = __uint_as_float(raw.w & 0xffff0000u);
+    }
+};
+
+// Agent-scope relaxed accesses: they write through / read around the per-XCD L2, so data handed from
+// one workgroup to another needs no L2 write-back or invalidate, only a wait for the stores to land.
+__device__ __forceinline__ void store_agent(uint32_t* address, uint32_t value)
+{
+    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ uint32_t load_agent(const uint32_t* address)
+{
+    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Ascending integer key of a float for bitwise selection (larger logit, larger key); never 0 for a
+// finite logit, so 0 can mark an empty slot.
+__device__ __forceinline__ uint32_t ascending_key(float value)
+{
+    uint32_t bits = __float_as_uint(value);
+    if (bits == 0x80000000u)
+        bits = 0u; // -0 ties with +0
+    return (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+}
+
+__device__ __forceinline__ float value_from_ascending_key(uint32_t key)
+{
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+// The quota-th largest of the wave's 64 keys (one per lane), found bit by bit with wave-wide counts.
+__device__ __forceinline__ uint32_t wave_select_key(uint32_t key, int quota)
+{
+    uint32_t prefix = 0;
+#pragma unroll
+    for (int bit = 31; bit >= 0; --bit)
+    {
+        const uint32_t trial = prefix | (1u << bit);
+        if (__popcll(__ballot(key >= trial)) >= quota)
+            prefix = trial;
+    }
+    return prefix;
+}
+
+// The top_k-th largest of m <= 64 * R keys in LDS (0 if fewer than top_k are non-zero), by one wave:
+// keys in registers, the answer built bit by bit from wave-wide counts.
+template <int R>
+__device__ __forceinline__ uint32_t select_kth_key(const uint32_t* keys_in_lds, int m, int top_k, int lane)
+{
+    uint32_t keys[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        const int q = r * kWaveSize + lane;
+        keys[r] = q < m ? keys_in_lds[q] : 0u;
+    }
+    uint32_t prefix = 0;
+    for (int bit = 31; bit >= 0; --bit)
+    {
+        const uint32_t trial = prefix | (1u << bit);
+        int count = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            count += __popcll(__ballot(keys[r] >= trial));
+        if (count >= top_k)
+            prefix = trial;
+    }
+    return prefix;
+}
+
+__device__ __forceinline__ uint32_t select_kth_key_dispatch(const uint32_t* keys_in_lds, int m, int top_k, int lane)
+{
+    if (m <= kWaveSize)
+        return select_kth_key<1>(keys_in_lds, m, top_k, lane);
+    if (m <= 2 * kWaveSize)
+        return select_kth_key<2>(keys_in_lds, m, top_k, lane);
+    if (m <= 4 * kWaveSize)
+        return select_kth_key<4>(keys_in_lds, m, top_k, lane);
+    if (m <= 8 * kWaveSize)
+        return select_kth_key<8>(keys_in_lds, m, top_k, lane);
+    return select_kth_key<16>(keys_in_lds, m, top_k, lane);
+}
+
+struct BoundScratch
+{
+    uint32_t wave_bounds[kScanWaves];
+    uint32_t hot_keys[2 * kScanThreads];
+    uint32_t hot_total;
+    uint32_t result;
+};
+
+// The top_k-th largest of the workgroup's keys (KEYS per thread, each standing for a distinct
+// logit; 0 = no key), or with exact == false a lower bound of it that at least top_k keys still
+// reach; 0 when fewer than top_k keys exist.  top_k <= 512 * KEYS.  All threads of the workgroup must call it.
+//   A  every wave finds a lower bound of the ceil(top_k/8)-th largest of its 64 * KEYS keys (upper 16 bits
+//      only); the smallest of the eight bounds is reached by at least top_k keys of the workgroup;
+//   B  the keys at or above that bound are gathered in LDS;
+//   C  wave 0 selects the exact top_k-th largest of the gathered keys.
+template <int KEYS>
+__device__ __forceinline__ uint32_t workgroup_kth_largest_key(
+    const uint32_t (&keys)[KEYS], int top_k, int tid, BoundScratch& scratch, bool exact)
+{
+    static_assert(KEYS == 1 || KEYS == 2, "the gather buffer holds two keys per thread");
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const int quota = (top_k + kScanWaves - 1) / kScanWaves;
+    uint32_t prefix = 0;
+#pragma unroll
+    for (int bit = 31; bit >= 16; --bit)
+    {
+        const uint32_t trial = prefix | (1u << bit);
+        int reached = 0;
+#pragma unroll
+        for (int slot = 0; slot < KEYS; ++slot)
+            reached += __popcll(__ballot(keys[slot] >= trial));
+        if (reached >= quota)
+            prefix = trial;
+    }
+    if (lane == 0)
+        scratch.wave_bounds[wave] = prefix;
+    if (tid == 0)
+        scratch.hot_total = 0;
+    __syncthreads();
+    uint32_t loose_bound = scratch.wave_bounds[0];
+#pragma unroll
+    for (int w = 1; w < kScanWaves; ++w)
+        loose_bound = min(loose_bound, scratch.wave_bounds[w]);
+    if (!exact)
+    {
+        __syncthreads();
+        return loose_bound;
+    }
+#pragma unroll
+    for (int slot = 0; slot < KEYS; ++slot)
+    {
+        const uint32_t key = keys[slot];
+        const bool hot = key != 0u && key >= loose_bound;
+        const uint64_t hot_mask = __ballot(hot);
+        if (hot_mask != 0)
+        {
+            uint32_t base = 0;
+            if (lane == 0)
+                base = atomicAdd(&scratch.hot_total, static_cast<uint32_t>(__popcll(hot_mask)));
+            base = __builtin_amdgcn_readfirstlane(base);
+            if (hot)
+                scratch.hot_keys[base + lanes_below(hot_mask)] = key;
+        }
+    }
+    __syncthreads();
+    if (wave == 0)
+    {
+        const uint32_t kth = select_kth_key_dispatch(scratch.hot_keys, static_cast<int>(scratch.hot_total), top_k, lane);
+        if (lane == 0)
+            scratch.result = kth;
+    }
+    __syncthreads();
+    return scratch.result;
+}
+
+// A lower bound of the top_k-th largest of the workgroup's N values per thread (NaN and -inf do not
+// count), exact in the upper 16 bits of the key; 0 when fewer than top_k values count.  At least top_k
+// values reach the bound, and only as many more as share those 16 bits with the top_k-th largest.
+// All threads of the workgroup must call it.
+template <int N>
+__device__ __forceinline__ uint32_t workgroup_loose_kth_of_values(
+    const float (&values)[N], int top_k, int tid, BoundScratch& scratch)
+{
+    uint32_t keys[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+        keys[i] = values[i] > -__builtin_inff() ? ascending_key(values[i]) : 0u; // false for NaN as well
+    // one counter per bit in scratch.hot_keys
+    if (tid < 16)
+        scratch.hot_keys[tid] = 0;
+    __syncthreads();
+    uint32_t prefix = 0;
+    for (int bit = 31; bit >= 16; --bit)
+    {
+        const uint32_t trial = prefix | (1u << bit);
+        int wave_count = 0;
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+            wave_count += __popcll(__ballot(keys[i] >= trial));
+        if ((tid & (kWaveSize - 1)) == 0)
+            atomicAdd(&scratch.hot_keys[31 - bit], static_cast<uint32_t>(wave_count));
+        __syncthreads();
+        if (scratch.hot_keys[31 - bit] >= static_cast<uint32_t>(top_k))
+            prefix = trial;
+    }
+    __syncthreads();
+    return prefix;
+}
+
+// Exact best-K selection over m <= 64 * R candidates in LDS by one wave; keys live in registers.
+// Selected candidates (at most top_k) are written, unordered, to final_values / final_indices.
+template <int R>
+__device__ __forceinline__ int select_best_wave(
+    const uint32_t* staged_keys, const int32_t* staged_indices, int m, int top_k, int lane,
+    float* final_values, int32_t* final_indices)
+{
+    uint32_t keys[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        const int q = r * kWaveSize + lane;
+        keys[r] = q < m ? staged_keys[q] : 0u;
+    }
+    uint32_t key_cut = 1u; // every staged key qualifies
+    uint32_t index_cut = 0xffffffffu;
+    if (m > top_k)
+    {
+        uint32_t prefix = 0;
+        for (int bit = 31; bit >= 0; --bit)
+        {
+            const uint32_t trial = prefix | (1u << bit);
+            int count = 0;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                count += __popcll(__ballot(keys[r] >= trial));
+            if (count >= top_k)
+                prefix = trial;
+        }
+        key_cut = prefix;
+        int above = 0;
+        int ties = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+        {
+            above += __popcll(__ballot(keys[r] > key_cut));
+            ties += __popcll(__ballot(keys[r] == key_cut));
+        }
+        const int needed = top_k - above; // of the ties, the `needed` lowest indices stay
+        if (ties > needed)
+        {
+            uint32_t index_prefix = 0;
+            for (int bit = 31; bit >= 0; --bit)
+            {
+                const uint32_t trial = index_prefix | (1u << bit);
+                int count = 0;
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                {
+                    const int q = r * kWaveSize + lane;
+                    const bool tie = keys[r] == key_cut && key_cut != 0u && q < m;
+                    const uint32_t index = tie ? static_cast<uint32_t>(staged_indices[q]) : 0xffffffffu;
+                    count += __popcll(__ballot(tie && index < trial));
+                }
+                if (count < needed)
+                    index_prefix = trial;
+            }
+            index_cut = index_prefix;
+        }
+    }
+    int n = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        const int q = r * kWaveSize + lane;
+        const uint32_t key = keys[r];
+        bool selected = key != 0u && key >= key_cut;
+        int32_t index = 0;
+        if (selected)
+        {
+            index = staged_indices[q];
+            if (key == key_cut && static_cast<uint32_t>(index) > index_cut)
+                selected = false;
+        }
+        const uint64_t mask = __ballot(selected);
+        if (mask != 0)
+        {
+            const int position = n + lanes_below(mask);
+            if (selected && position < kFastTopK)
+            {
+                final_values[position] = value_from_ascending_key(key);
+                final_indices[position] = index;
+            }
+            n += __popcll(mask);
+        }
+    }
+    return n < kFastTopK ? n : kFastTopK;
+}
+
+} // namespace ncnn_moe_hip
+
+#endif // NCNN_MOE_HIP_SAMPLER_COMMON_H

@@ -21,12 +21,16 @@ constexpr int kVectorsPerLaneF32 = 5;
 constexpr int kVectorsPerLaneBF16 = 3;
 constexpr int kSegmentValuesF32 = kScanThreads * kVectorsPerLaneF32 * 4;   // 10240 logits per chunk
 constexpr int kSegmentValuesBF16 = kScanThreads * kVectorsPerLaneBF16 * 8; // 12288 logits per chunk
-constexpr int kFastTopK = 64;            // largest effective Top-K served by the select path
-constexpr int kWaveCandidateCap = 64;    // candidates one wave may collect for its segment
+constexpr int kFastTopK = 64;            // widest Top-K window finished by one wave
+constexpr int kSelectTopK = 1024;
+constexpr int kTwoKeyBoundTopK = 512; // wider windows bound their first chunk by a select over all its values         // widest Top-K window of the select path (rows of one segment)
+constexpr int kSingleListCap = 512;      // candidate list of a workgroup that streams a single chunk
+constexpr int kLoopedListCap = 4096;     // candidate list of a workgroup that streams several chunks
 constexpr int kSegmentRecordSlots = 256; // candidate slots of a segment's record in HBM
-constexpr int kMaxSegments = 16;         // segments per row the row merge can stage in one trip
+constexpr int kMaxSegments = 16;
+constexpr int kWholeRowBatch = 256;          // from this many rows on, one workgroup streams a whole row
+constexpr int kSelectWorkgroupTarget = 1024; // workgroups a smaller batch is split into (4 per CU)         // segments per row the row merge can stage in one trip
 constexpr int kMergeStageSlots = 4096;   // record slots of a row loaded in one trip (8 per thread)
-constexpr int kMergeSurvivorCap = 512;   // candidates that may survive the row-level prune
 
 // Full-order ("general") path geometry.
 constexpr int kSortThreads = 1024;
@@ -59,13 +63,19 @@ enum ScanFlags : uint32_t
     kScanOverflow = 4u
 };
 
-__device__ __forceinline__ bool is_finite_f32(float value)
+__host__ __device__ __forceinline__ bool is_finite_f32(float value)
 {
-    return (__float_as_uint(value) & 0x7f800000u) != 0x7f800000u;
+    union
+    {
+        float f;
+        uint32_t u;
+    } bits;
+    bits.f = value;
+    return (bits.u & 0x7f800000u) != 0x7f800000u;
 }
 
 // validate_sampling_options, src/engine/session.cpp:65-74 of the reference.
-__device__ __forceinline__ int validate_params(const ncnn_moe_sample_params& p)
+__host__ __device__ __forceinline__ int validate_params(const ncnn_moe_sample_params& p)
 {
     if (!is_finite_f32(p.temperature) || p.temperature < 0.0f)
         return NCNN_MOE_ROW_BAD_TEMPERATURE;
@@ -77,9 +87,10 @@ __device__ __forceinline__ int validate_params(const ncnn_moe_sample_params& p)
 }
 
 // Which path serves the row.  effective_k is the length of the Top-K window (vocab when Top-K is off,
-// session.cpp:86-87), 1 for greedy.
-__device__ __forceinline__ int resolve_row_mode(
-    const ncnn_moe_sample_params& p, uint32_t vocab, uint32_t segments, int force_general,
+// session.cpp:86-87), 1 for greedy.  max_select_top_k is the widest window the launch's select kernel
+// handles: kFastTopK when rows are split into segments, kSelectTopK when a workgroup sees a whole row.
+__host__ __device__ __forceinline__ int resolve_row_mode(
+    const ncnn_moe_sample_params& p, uint32_t vocab, uint32_t max_select_top_k, int force_general,
     uint32_t& effective_k, int& status)
 {
     status = validate_params(p);
@@ -92,16 +103,16 @@ __device__ __forceinline__ int resolve_row_mode(
         return kModeGreedy;
     }
     effective_k = (p.top_k == 0u || p.top_k >= vocab) ? vocab : p.top_k;
-    if (!force_general && effective_k <= static_cast<uint32_t>(kFastTopK) && segments <= static_cast<uint32_t>(kMaxSegments))
+    if (!force_general && effective_k <= max_select_top_k)
         return kModeTopK;
     return kModeGeneral;
 }
 
-// Entries of a segment's record that the row merge reads: twice the Top-K window plus 16 (the bound
-// admits K logits and a few more; ties beyond that overflow to the full-order path).
+// Entries of a segment's record that the row merge reads: twice the Top-K window plus 64 (a list is
+// tightened when it grows past that; ties beyond it overflow to the full-order path).
 __host__ __device__ __forceinline__ uint32_t segment_record_entries(uint32_t effective_k)
 {
-    const uint32_t entries = effective_k * 2u + 16u;
+    const uint32_t entries = effective_k * 2u + 64u;
     return entries > static_cast<uint32_t>(kSegmentRecordSlots) ? static_cast<uint32_t>(kSegmentRecordSlots) : entries;
 }
 

@@ -1,0 +1,374 @@
+// Full-order path: rows with no Top-K window (or one too wide for the select path) need the complete
+// stable order, because the CPU sampler's sums run over it sequentially.
+//   general_sort_kernel    stable LSD radix sort of one row by descending key, one workgroup per row
+//   general_replay_kernel  the sampler's walk over the sorted row
+#ifndef NCNN_MOE_HIP_SAMPLER_FULL_ORDER_H
+#define NCNN_MOE_HIP_SAMPLER_FULL_ORDER_H
+
+#include "sampler_exact_sum.h"
+
+namespace ncnn_moe_hip {
+
+template <int DTYPE>
+__device__ __forceinline__ float load_logit(const void* row_pointer, uint32_t i);
+
+template <>
+__device__ __forceinline__ float load_logit<NCNN_MOE_LOGITS_F32>(const void* row_pointer, uint32_t i)
+{
+    return static_cast<const float*>(row_pointer)[i];
+}
+
+template <>
+__device__ __forceinline__ float load_logit<NCNN_MOE_LOGITS_BF16>(const void* row_pointer, uint32_t i)
+{
+    return __uint_as_float(static_cast<uint32_t>(static_cast<const uint16_t*>(row_pointer)[i]) << 16);
+}
+
+// Stable LSD radix sort (8-bit digits) of one row by descending_key; one workgroup per row.
+// fp32 rows take four passes; bf16 keys only differ in their upper 16 bits and take two.
+// The sorted keys end in sort_keys[1].  With PAIRS the token indices travel with the keys and end in
+// sort_indices[1] (needed only when the whole filtered distribution is exported); sampling sorts the
+// keys alone and recovers the one index it needs from the logits afterwards.
+template <int DTYPE, bool PAIRS>
+__global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs a)
+{
+    constexpr int kPasses = DTYPE == NCNN_MOE_LOGITS_F32 ? 4 : 2;
+    constexpr int kFirstDigit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0 : 2;
+    const uint32_t row = blockIdx.x;
+    if (a.row_state[row] != kRowNeedsGeneral)
+        return;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const uint32_t n = a.vocab;
+
+    __shared__ uint32_t histogram[kPasses][256];
+    __shared__ uint32_t digit_base[256];
+    __shared__ uint32_t wave_counts[kSortWaves][256];
+
+    const char* row_pointer = static_cast<const char*>(a.logits) +
+        static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
+    uint32_t* keys[2] = {a.sort_keys[0] + row * a.sort_stride, a.sort_keys[1] + row * a.sort_stride};
+    uint32_t* indices[2] = {a.sort_indices[0] + row * a.sort_stride, a.sort_indices[1] + row * a.sort_stride};
+
+    for (int i = tid; i < kPasses * 256; i += kSortThreads)
+        (&histogram[0][0])[i] = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < n; i += kSortThreads)
+    {
+        const uint32_t key = descending_key(load_logit<DTYPE>(row_pointer, i));
+#pragma unroll
+        for (int pass = 0; pass < kPasses; ++pass)
+            atomicAdd(&histogram[pass][(key >> (8 * (pass + kFirstDigit))) & 255u], 1u);
+    }
+    __syncthreads();
+    // exclusive scan of each histogram by one wave (4 bins per lane)
+    if (wave < kPasses)
+    {
+        uint32_t* h = histogram[wave];
+        const uint32_t c0 = h[lane * 4 + 0], c1 = h[lane * 4 + 1], c2 = h[lane * 4 + 2], c3 = h[lane * 4 + 3];
+        const uint32_t lane_total = c0 + c1 + c2 + c3;
+        uint32_t inclusive = lane_total;
+#pragma unroll
+        for (int j = 1; j < kWaveSize; j <<= 1)
+        {
+            const uint32_t up = __shfl_up(inclusive, j, kWaveSize);
+            if (lane >= j)
+                inclusive += up;
+        }
+        const uint32_t exclusive = inclusive - lane_total;
+        h[lane * 4 + 0] = exclusive;
+        h[lane * 4 + 1] = exclusive + c0;
+        h[lane * 4 + 2] = exclusive + c0 + c1;
+        h[lane * 4 + 3] = exclusive + c0 + c1 + c2;
+    }
+    __syncthreads();
+
+    // Every pass walks the row in tiles of 1024 x 8 elements.  A wave owns 512 consecutive elements of
+    // the tile and ranks them in 8 rounds of 64 (one element per lane), so that the order inside the
+    // wave is the input order; its per-digit running counts live in LDS.  A prefix over the 16 waves
+    // and the digit bases then turns the ranks into output positions.
+    for (int pass = 0; pass < kPasses; ++pass)
+    {
+        const int shift = 8 * (pass + kFirstDigit);
+        const uint32_t* source_keys = keys[(pass + 1) & 1];   // pass 0 reads the logits instead
+        const uint32_t* source_indices = indices[(pass + 1) & 1];
+        uint32_t* target_keys = keys[pass & 1];
+        uint32_t* target_indices = indices[pass & 1];
+        if (tid < 256)
+            digit_base[tid] = histogram[pass][tid];
+        for (uint32_t tile = 0; tile < n; tile += kSortTile)
+        {
+            for (int i = tid; i < kSortWaves * 256; i += kSortThreads)
+                (&wave_counts[0][0])[i] = 0;
+            uint32_t tile_keys[kSortPerThread];
+            uint32_t tile_indices[kSortPerThread];
+            uint32_t tile_ranks[kSortPerThread];
+            const uint32_t wave_first = tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread);
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
+            {
+                const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+                tile_keys[e] = 0xffffffffu;
+                tile_indices[e] = i;
+                if (i < n)
+                {
+                    if (pass == 0)
+                        tile_keys[e] = descending_key(load_logit<DTYPE>(row_pointer, i));
+                    else
+                    {
+                        tile_keys[e] = source_keys[i];
+                        if (PAIRS)
+                            tile_indices[e] = source_indices[i];
+                    }
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
+            {
+                const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+                const bool valid = i < n;
+                const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+                uint64_t peers = __ballot(valid);
+#pragma unroll
+                for (int b = 0; b < 8; ++b)
+                {
+                    const bool bit = (digit >> b) & 1u;
+                    const uint64_t set = __ballot(valid && bit);
+                    peers &= bit ? set : ~set;
+                }
+                const int rank_in_round = lanes_below(peers);
+                uint32_t seen = 0;
+                if (valid)
+                    seen = wave_counts[wave][digit];
+                tile_ranks[e] = seen + static_cast<uint32_t>(rank_in_round);
+                if (valid && rank_in_round == 0)
+                    wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popcll(peers));
+            }
+            __syncthreads();
+            if (tid < 256)
+            {
+                uint32_t running = digit_base[tid];
+#pragma unroll
+                for (int w = 0; w < kSortWaves; ++w)
+                {
+                    const uint32_t c = wave_counts[w][tid];
+                    wave_counts[w][tid] = running;
+                    running += c;
+                }
+                digit_base[tid] = running;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
+            {
+                const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+                if (i < n)
+                {
+                    const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+                    const uint32_t position = wave_counts[wave][digit] + tile_ranks[e];
+                    target_keys[position] = tile_keys[e];
+                    if (PAIRS)
+                        target_indices[position] = tile_indices[e];
+                }
+            }
+            __syncthreads();
+        }
+        __threadfence_block();
+        __syncthreads();
+    }
+}
+
+struct RecoverScratch
+{
+    uint32_t wave_counts[kReplayWaves];
+    int32_t found;
+};
+
+// Token index of position `rank` of the sorted row, from the logits: the sort is stable, so it is
+// the (rank - first position of that key)-th element, in index order, whose key equals keys[rank].
+// Every thread of the workgroup must call it.
+template <int DTYPE>
+__device__ __forceinline__ int32_t recover_token_index(
+    const void* row_pointer, uint32_t vocab, const uint32_t* keys, uint32_t rank, RecoverScratch& scratch, int tid)
+{
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const uint32_t key = keys[rank];
+    uint32_t low = 0, high = rank; // first position holding this key
+    while (low < high)
+    {
+        const uint32_t middle = (low + high) >> 1;
+        if (keys[middle] < key)
+            low = middle + 1;
+        else
+            high = middle;
+    }
+    const uint32_t ordinal = rank - low;
+    uint32_t passed = 0; // matches before the current chunk
+    if (tid == 0)
+        scratch.found = -1;
+    __syncthreads();
+    for (uint32_t base = 0; base < vocab; base += kReplayChunk)
+    {
+        const uint32_t first = base + static_cast<uint32_t>(tid) * kReplayPerThread;
+        uint32_t matches = 0;
+        uint32_t count = 0;
+#pragma unroll
+        for (int j = 0; j < kReplayPerThread; ++j)
+        {
+            const uint32_t i = first + j;
+            if (i < vocab && descending_key(load_logit<DTYPE>(row_pointer, i)) == key)
+            {
+                matches |= 1u << j;
+                ++count;
+            }
+        }
+        uint32_t inclusive = count;
+#pragma unroll
+        for (int step = 1; step < kWaveSize; step <<= 1)
+        {
+            const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
+            if (lane >= step)
+                inclusive += up;
+        }
+        if (lane == kWaveSize - 1)
+            scratch.wave_counts[wave] = inclusive;
+        __syncthreads();
+        uint32_t before = passed;
+        uint32_t chunk_total = 0;
+        for (int w = 0; w < kReplayWaves; ++w)
+        {
+            const uint32_t c = scratch.wave_counts[w];
+            if (w < wave)
+                before += c;
+            chunk_total += c;
+        }
+        before += inclusive - count;
+        if (ordinal >= before && ordinal < before + count)
+        {
+            uint32_t skip = ordinal - before;
+#pragma unroll
+            for (int j = 0; j < kReplayPerThread; ++j)
+            {
+                if (matches & (1u << j))
+                {
+                    if (skip == 0)
+                        scratch.found = static_cast<int32_t>(first + j);
+                    --skip;
+                }
+            }
+        }
+        __syncthreads();
+        if (scratch.found >= 0)
+            break;
+        passed += chunk_total;
+    }
+    const int32_t found = scratch.found;
+    __syncthreads();
+    return found;
+}
+
+// Full-order rows: walks the sorted row as the CPU sampler does (src/engine/session.cpp:84-134,
+// :429-442).  One workgroup per row.
+template <int DTYPE>
+__global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerArgs a)
+{
+    const uint32_t row = blockIdx.x;
+    if (a.row_state[row] != kRowNeedsGeneral)
+        return;
+    const int tid = threadIdx.x;
+    const ncnn_moe_sample_params p = a.params[row];
+    const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
+    const bool have_indices = a.distribution_count != nullptr; // the pair sort ran: indices are valid
+    const uint32_t* indices = have_indices ? a.sort_indices[1] + row * a.sort_stride : nullptr;
+    const uint32_t vocab = a.vocab;
+    const char* row_pointer = static_cast<const char*>(a.logits) +
+        static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
+
+    __shared__ ReplayScratch scratch;
+    __shared__ RecoverScratch recover_scratch;
+
+    uint8_t flags = NCNN_MOE_ROW_FLAG_GENERAL_PATH;
+    {
+        uint32_t effective_k = 0;
+        int status = 0;
+        if (resolve_row_mode(p, vocab, a.max_select_top_k, 0, effective_k, status) != kModeGeneral)
+            flags |= NCNN_MOE_ROW_FLAG_FALLBACK;
+    }
+    if (keys[vocab - 1] == 0xffffffffu)
+        flags |= NCNN_MOE_ROW_FLAG_HAS_NAN;
+    if (tid == 0)
+        a.row_state[row] = kRowDone;
+
+    auto token_at = [&](uint32_t rank) -> int32_t {
+        if (have_indices)
+            return static_cast<int32_t>(indices[rank]);
+        return recover_token_index<DTYPE>(row_pointer, vocab, keys, rank, recover_scratch, tid);
+    };
+
+    if (p.temperature == 0.0f)
+    {
+        // a greedy row whose select overflowed (every logit tied): first finite logit in sorted order,
+        // non-finite logits skipped (src/engine/session.cpp:404-424)
+        uint32_t low = 0, high = vocab;
+        while (low < high)
+        {
+            const uint32_t middle = (low + high) >> 1;
+            if (keys[middle] <= kPositiveInfinityKey)
+                low = middle + 1;
+            else
+                high = middle;
+        }
+        const bool any_finite = low < vocab && keys[low] <= kLastFiniteKey;
+        int32_t token = -1;
+        if (any_finite)
+            token = token_at(low);
+        if (tid == 0)
+        {
+            if (any_finite)
+            {
+                write_token(a, row, p, token, 1.0f, 1u, 0, flags);
+                if (a.distribution_count != nullptr && row == 0)
+                {
+                    *a.distribution_count = 1;
+                    if (a.distribution_cap > 0)
+                    {
+                        a.distribution_ids[0] = token;
+                        a.distribution_probabilities[0] = 1.0f;
+                    }
+                }
+            }
+            else
+                write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, flags);
+        }
+        return;
+    }
+
+    // finite logits form a prefix of the sorted row, after any +inf (which rejects the row)
+    const uint32_t first_key = keys[0];
+    if (first_key <= kPositiveInfinityKey || first_key > kLastFiniteKey)
+    {
+        if (tid == 0)
+            write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, flags);
+        return;
+    }
+    uint32_t low = 0, high = vocab; // first position whose key is not finite
+    while (low < high)
+    {
+        const uint32_t middle = (low + high) >> 1;
+        if (keys[middle] <= kLastFiniteKey)
+            low = middle + 1;
+        else
+            high = middle;
+    }
+    uint32_t n = low;
+    if (p.top_k > 0 && p.top_k < vocab && n > p.top_k)
+        n = p.top_k;
+    replay_sorted_window(a, row, p, keys, n, indices, flags, scratch, tid, token_at);
+}
+
+} // namespace ncnn_moe_hip
+
+#endif // NCNN_MOE_HIP_SAMPLER_FULL_ORDER_H

@@ -1,0 +1,594 @@
+// Select path: the one HBM pass over the logits for greedy rows and rows with a Top-K window.
+//
+// A workgroup of 512 threads streams a contiguous range of chunks of one row (a chunk is 512 lanes x
+// 5 fp32 or 3 bf16 16-byte vectors) and keeps the row's Top-K candidates of that range:
+//   * per-vector and per-lane maxima of the chunk;
+//   * a bound that at least K logits reach: for the first chunk the exact K-th largest of the 512
+//     lane maxima, later the K-th best candidate collected so far (the list is tightened whenever
+//     it grows past 2K + 64 entries);
+//   * the logits at or above the bound are appended to a candidate list in LDS.
+// One segment per row (large batches): the workgroup finishes the row itself.  Several segments per
+// row (small batches, so that every CU streams): each hands its list over through HBM and the last
+// workgroup to arrive merges them.  Either way the candidates are reduced to the exact best K by
+// (logit descending, index ascending) and the CPU sampler's epilogue runs on them.
+#ifndef NCNN_MOE_HIP_SAMPLER_SELECT_H
+#define NCNN_MOE_HIP_SAMPLER_SELECT_H
+
+#include "sampler_exact_sum.h"
+
+namespace ncnn_moe_hip {
+
+template <bool LOOPED>
+struct SelectShared
+{
+    static constexpr int kListCap = LOOPED ? kLoopedListCap : kSingleListCap;
+    static constexpr int kSortedCap = LOOPED ? kSelectTopK : 1;
+    BoundScratch bound;
+    uint32_t list_keys[kListCap];
+    int32_t list_indices[kListCap];
+    uint32_t list_count;
+    uint32_t block_flags;
+    int block_is_last;
+    float final_values[kFastTopK];
+    int32_t final_indices[kFastTopK];
+    uint32_t sorted_keys[kSortedCap];    // descending keys of the ordered window when K > 64
+    uint32_t sorted_indices[kSortedCap];
+    ReplayScratch replay;
+};
+
+// Appends the caller's candidate (if `hit`) to the workgroup's list.  Positions are reserved per
+// wave with one LDS atomic; the order inside the list is irrelevant.  Called by whole waves.
+template <bool LOOPED>
+__device__ __forceinline__ void append_candidate(SelectShared<LOOPED>& shared, bool hit, uint32_t key, int32_t index, int lane)
+{
+    const uint64_t hits = __ballot(hit);
+    if (hits == 0)
+        return;
+    uint32_t base = 0;
+    if (lane == __builtin_ctzll(hits))
+        base = atomicAdd(&shared.list_count, static_cast<uint32_t>(__popcll(hits)));
+    base = __builtin_amdgcn_readlane(base, __builtin_ctzll(hits));
+    const uint32_t position = base + static_cast<uint32_t>(lanes_below(hits));
+    if (hit && position < static_cast<uint32_t>(SelectShared<LOOPED>::kListCap))
+    {
+        shared.list_keys[position] = key;
+        shared.list_indices[position] = index;
+    }
+}
+
+// Raises the bound to (a lower bound of) the K-th best candidate of the list and drops the
+// candidates below it.  All threads call it; returns the new bound key.
+template <bool LOOPED>
+__device__ __forceinline__ uint32_t tighten_list(SelectShared<LOOPED>& shared, uint32_t bound_key, int top_k, int tid)
+{
+    constexpr int kPerThread = SelectShared<LOOPED>::kListCap / kScanThreads;
+    const int lane = tid & (kWaveSize - 1);
+    const uint32_t count = min(shared.list_count, static_cast<uint32_t>(SelectShared<LOOPED>::kListCap));
+    uint32_t keys[kPerThread];
+    int32_t indices[kPerThread];
+    uint32_t best = 0, second = 0; // the thread's two best candidates: two distinct logits
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+    {
+        const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
+        keys[j] = q < count ? shared.list_keys[q] : 0u;
+        indices[j] = q < count ? shared.list_indices[q] : 0;
+        second = max(second, min(best, keys[j]));
+        best = max(best, keys[j]);
+    }
+    // at least K candidates reach the K-th largest of the per-thread best and second-best keys
+    const uint32_t thread_keys[2] = {best, second};
+    const uint32_t kth = workgroup_kth_largest_key(thread_keys, top_k, tid, shared.bound, true);
+    bound_key = max(bound_key, kth);
+    if (tid == 0)
+        shared.list_count = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+        append_candidate(shared, keys[j] != 0u && keys[j] >= bound_key, keys[j], indices[j], lane);
+    __syncthreads();
+    return bound_key;
+}
+
+// From the candidate list to the sampled token: exact best K, their order, the epilogue.
+// All threads of the workgroup call it; n_list <= kListCap.
+template <bool LOOPED>
+__device__ __forceinline__ void finish_from_list(
+    const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p, bool greedy, int top_k,
+    SelectShared<LOOPED>& shared, uint8_t result_flags, int tid)
+{
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    int n_list = static_cast<int>(shared.list_count);
+    if (top_k <= kFastTopK)
+    {
+        if constexpr (LOOPED)
+        {
+            if (n_list > 8 * kWaveSize)
+            {
+                tighten_list(shared, 0u, top_k, tid);
+                n_list = static_cast<int>(shared.list_count);
+            }
+        }
+        if (n_list > 8 * kWaveSize)
+        {
+            // ties left more candidates than one wave orders: the full-order kernels take the row
+            if (tid == 0)
+            {
+                write_pending(a, row);
+                a.row_state[row] = kRowNeedsGeneral;
+            }
+            return;
+        }
+        if (wave != 0)
+            return;
+        int n = 0;
+        if (n_list <= kWaveSize)
+            n = select_best_wave<1>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
+        else if (n_list <= 2 * kWaveSize)
+            n = select_best_wave<2>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
+        else if (n_list <= 4 * kWaveSize)
+            n = select_best_wave<4>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
+        else
+            n = select_best_wave<8>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
+        if (lane == 0)
+            a.row_state[row] = kRowDone;
+        if (n == 0)
+        {
+            if (lane == 0)
+                write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
+            return;
+        }
+        float value = lane < n ? shared.final_values[lane] : 0.0f;
+        int32_t index = lane < n ? shared.final_indices[lane] : -1;
+        int rank = 0;
+        for (int j = 0; j < n; ++j)
+            rank += candidate_before(read_lane(value, j), read_lane(index, j), value, index) ? 1 : 0;
+        if (lane < n)
+        {
+            shared.final_values[rank] = value;
+            shared.final_indices[rank] = index;
+        }
+        value = lane < n ? shared.final_values[lane] : 0.0f;
+        index = lane < n ? shared.final_indices[lane] : -1;
+        if (greedy)
+        {
+            if (lane == 0)
+            {
+                write_token(a, row, p, index, 1.0f, 1u, 0, result_flags);
+                if (a.distribution_count != nullptr && row == 0)
+                {
+                    *a.distribution_count = 1;
+                    if (a.distribution_cap > 0)
+                    {
+                        a.distribution_ids[0] = index;
+                        a.distribution_probabilities[0] = 1.0f;
+                    }
+                }
+            }
+            return;
+        }
+        finish_row_wave(a, row, p, value, index, n, lane, result_flags);
+        return;
+    }
+    if constexpr (LOOPED)
+    {
+        // ---- a window wider than one wave: exact K-th best key, then ranks by counting, then the
+        // walk over the ordered window with exact running sums
+        constexpr int kPerThread = SelectShared<LOOPED>::kListCap / kScanThreads;
+        if (n_list > top_k + 64)
+            tighten_list(shared, 0u, top_k, tid); // fewer candidates to rank
+        const int n_ranked = static_cast<int>(shared.list_count);
+        uint32_t keys[kPerThread];
+        int32_t indices[kPerThread];
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j)
+        {
+            const int q = j * kScanThreads + tid;
+            keys[j] = q < n_ranked ? shared.list_keys[q] : 0u;
+            indices[j] = q < n_ranked ? shared.list_indices[q] : 0;
+        }
+        // rank of every candidate among all candidates; the best top_k go, in order, to sorted_*
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j)
+        {
+            if (keys[j] == 0u)
+                continue;
+            int rank = 0;
+#pragma unroll 8
+            for (int q = 0; q < n_ranked; ++q)
+            {
+                const uint32_t other_key = shared.list_keys[q];
+                const int32_t other_index = shared.list_indices[q];
+                rank += (other_key > keys[j] || (other_key == keys[j] && other_index < indices[j])) ? 1 : 0;
+            }
+            if (rank < top_k)
+            {
+                shared.sorted_keys[rank] = descending_key(value_from_ascending_key(keys[j]));
+                shared.sorted_indices[rank] = static_cast<uint32_t>(indices[j]);
+            }
+        }
+        __syncthreads();
+        const uint32_t n = static_cast<uint32_t>(n_ranked < top_k ? n_ranked : top_k);
+        if (tid == 0)
+            a.row_state[row] = kRowDone;
+        if (n == 0)
+        {
+            if (tid == 0)
+                write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
+            return;
+        }
+        const uint32_t* sorted_indices = shared.sorted_indices;
+        auto token_at = [&](uint32_t rank) -> int32_t { return static_cast<int32_t>(sorted_indices[rank]); };
+        replay_sorted_window(a, row, p, shared.sorted_keys, n, shared.sorted_indices, result_flags, shared.replay, tid, token_at);
+    }
+}
+
+template <int DTYPE, int VECTORS>
+__device__ __forceinline__ void load_chunk(
+    uint4 (&raw)[VECTORS], const char* aligned_base, uint32_t chunk_base, uint32_t valid_begin, uint32_t valid_end, int tid)
+{
+    using Vector = LogitsVector<DTYPE>;
+    constexpr uint32_t kNegativeInfinity = 0xff800000u;
+#pragma unroll
+    for (int v = 0; v < VECTORS; ++v)
+    {
+        const uint32_t first = chunk_base + static_cast<uint32_t>(v * kScanThreads + tid) * Vector::kWidth;
+        if (first < valid_end && first + Vector::kWidth > valid_begin)
+            raw[v] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(first) * Vector::kElementBytes);
+        else
+            raw[v] = make_uint4(kNegativeInfinity, kNegativeInfinity, kNegativeInfinity, kNegativeInfinity);
+    }
+}
+
+template <int DTYPE, bool LOOPED>
+__global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_F32) ? 8 : 1) void scan_select_kernel(SamplerArgs a)
+{
+    using Vector = LogitsVector<DTYPE>;
+    using Shared = SelectShared<LOOPED>;
+    constexpr int kWidth = Vector::kWidth;
+    constexpr int kVectors = Vector::kVectorsPerLane;
+    constexpr int kLaneValues = kVectors * kWidth;
+    constexpr uint32_t kChunk = static_cast<uint32_t>(kScanThreads) * kLaneValues;
+    constexpr uint32_t kNegativeInfinity = 0xff800000u;
+    constexpr uint32_t kPositiveInfinity = 0x7f800000u;
+
+    const uint32_t row = blockIdx.y;
+    const uint32_t segment = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+
+    __shared__ Shared shared;
+
+    if (a.only_pending && a.row_state[row] != kRowNeedsGeneral)
+        return;
+    const ncnn_moe_sample_params p = a.params[row];
+    uint32_t effective_k = 0;
+    int status = NCNN_MOE_ROW_OK;
+    const int mode = resolve_row_mode(p, a.vocab, a.max_select_top_k, a.force_general, effective_k, status);
+    if (mode == kModeInvalid || mode == kModeGeneral)
+    {
+        if (segment == 0 && tid == 0)
+        {
+            if (mode == kModeInvalid)
+            {
+                write_error(a, row, status, 0);
+                a.row_state[row] = kRowDone;
+            }
+            else
+            {
+                write_pending(a, row);
+                a.row_state[row] = kRowNeedsGeneral;
+            }
+        }
+        return;
+    }
+    const bool greedy = mode == kModeGreedy;
+    const int top_k = static_cast<int>(effective_k);
+    const uint32_t tighten_limit = static_cast<uint32_t>(2 * top_k + 64);
+
+    if (tid == 0)
+    {
+        shared.block_flags = 0;
+        shared.list_count = 0;
+    }
+
+    const char* row_pointer = static_cast<const char*>(a.logits) +
+        static_cast<size_t>(row) * a.row_stride * Vector::kElementBytes;
+    const uint32_t misalignment =
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row_pointer) & 15u) / Vector::kElementBytes;
+    const char* aligned_base = row_pointer - static_cast<size_t>(misalignment) * Vector::kElementBytes;
+    const uint32_t valid_begin = misalignment;
+    const uint32_t valid_end = misalignment + a.vocab;
+    const uint32_t first_chunk = segment * a.chunks_per_segment;
+    const uint32_t total_chunks = (valid_end + kChunk - 1) / kChunk;
+    const uint32_t end_chunk = min(total_chunks, first_chunk + a.chunks_per_segment);
+
+    uint32_t bound_key = 0; // ascending key every Top-K member is known to reach; 0: none yet
+    uint32_t local_flags = 0;
+    bool overflow = false;
+
+    uint4 raw[2][kVectors];
+    if (first_chunk < end_chunk)
+        load_chunk<DTYPE, kVectors>(raw[0], aligned_base, first_chunk * kChunk, valid_begin, valid_end, tid);
+    __syncthreads();
+
+    // Processes the chunk held in `buffer`; all indexing is static after unrolling.
+    auto process = [&](uint4 (&buffer)[kVectors], uint32_t chunk, bool first_of_segment) {
+        const uint32_t chunk_base = chunk * kChunk;
+        float values[kLaneValues];
+        float group_max[kVectors];
+        float lane_max = __uint_as_float(kNegativeInfinity);
+        float half_max[2] = {__uint_as_float(kNegativeInfinity), __uint_as_float(kNegativeInfinity)};
+        bool saw_nan = false;
+#pragma unroll
+        for (int v = 0; v < kVectors; ++v)
+        {
+            const uint32_t first = chunk_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth;
+            const bool any_valid = first < valid_end && first + kWidth > valid_begin;
+            if (any_valid)
+                Vector::unpack(buffer[v], &values[v * kWidth]);
+            else
+            {
+#pragma unroll
+                for (int c = 0; c < kWidth; ++c)
+                    values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
+            }
+            if (any_valid && (first < valid_begin || first + kWidth > valid_end))
+            {
+#pragma unroll
+                for (int c = 0; c < kWidth; ++c)
+                {
+                    const uint32_t position = first + c;
+                    if (position < valid_begin || position >= valid_end)
+                        values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
+                }
+            }
+            float vector_max = __uint_as_float(kNegativeInfinity);
+#pragma unroll
+            for (int c = 0; c < kWidth; ++c)
+            {
+                float x = values[v * kWidth + c];
+                saw_nan = saw_nan || (x != x);
+                if (greedy && x == __uint_as_float(kPositiveInfinity))
+                {
+                    x = __uint_as_float(kNegativeInfinity); // greedy skips every non-finite logit (session.cpp:411-412)
+                    values[v * kWidth + c] = x;
+                }
+                vector_max = fmaxf(vector_max, x);
+            }
+            group_max[v] = vector_max;
+            lane_max = fmaxf(lane_max, vector_max);
+            if constexpr (LOOPED)
+                half_max[v < (kVectors + 1) / 2 ? 0 : 1] = fmaxf(half_max[v < (kVectors + 1) / 2 ? 0 : 1], vector_max);
+        }
+        if (saw_nan)
+            local_flags |= kScanSawNan;
+        if (lane_max == __uint_as_float(kPositiveInfinity))
+            local_flags |= kScanSawPositiveInfinity;
+
+        // ---- bound of the first chunk: the exact K-th largest lane maximum.  The lanes at or above it
+        // each hold a distinct logit at least that large, so the K-th best logit of the row is no smaller.
+        if (first_of_segment)
+        {
+            if (LOOPED && top_k > kTwoKeyBoundTopK)
+            {
+                // a wide window: the lane maxima bound too loosely, so select over every value of the chunk
+                bound_key = max(bound_key, workgroup_loose_kth_of_values(values, top_k, tid, shared.bound));
+            }
+            else if constexpr (LOOPED)
+            {
+                // two keys per lane (the maxima of the two halves of its vectors): 1024 distinct logits
+                const uint32_t lane_keys[2] = {
+                    half_max[0] == __uint_as_float(kNegativeInfinity) ? 0u : ascending_key(half_max[0]),
+                    half_max[1] == __uint_as_float(kNegativeInfinity) ? 0u : ascending_key(half_max[1])};
+                bound_key = max(bound_key, workgroup_kth_largest_key(lane_keys, top_k, tid, shared.bound, true));
+            }
+            else
+            {
+                const uint32_t lane_keys[1] = {lane_max == __uint_as_float(kNegativeInfinity) ? 0u : ascending_key(lane_max)};
+                bound_key = max(bound_key, workgroup_kth_largest_key(lane_keys, top_k, tid, shared.bound, true));
+            }
+        }
+        // no bound yet (fewer than K lanes hold a finite logit): every finite logit is a candidate
+        const float threshold = bound_key == 0u ? -3.402823466e+38f : fmaxf(value_from_ascending_key(bound_key), -3.402823466e+38f);
+
+        // ---- collect the values at or above the bound; only vectors whose maximum reaches it are looked at
+#pragma unroll
+        for (int v = 0; v < kVectors; ++v)
+        {
+            const bool vector_hit = group_max[v] >= threshold;
+            if (__ballot(vector_hit) != 0)
+            {
+#pragma unroll
+                for (int c = 0; c < kWidth; ++c)
+                {
+                    const float x = values[v * kWidth + c];
+                    const uint32_t element = chunk_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth + c - misalignment;
+                    append_candidate(shared, vector_hit && x >= threshold, ascending_key(x), static_cast<int32_t>(element), lane);
+                }
+            }
+        }
+        __syncthreads();
+        if (shared.list_count > static_cast<uint32_t>(Shared::kListCap))
+            overflow = true; // candidates were dropped: only the full-order path can serve the row
+        else if (LOOPED && shared.list_count > tighten_limit)
+            bound_key = tighten_list(shared, bound_key, top_k, tid);
+    };
+
+    if constexpr (LOOPED)
+    {
+        for (uint32_t chunk = first_chunk; chunk < end_chunk; chunk += 2)
+        {
+            if (chunk + 1 < end_chunk)
+                load_chunk<DTYPE, kVectors>(raw[1], aligned_base, (chunk + 1) * kChunk, valid_begin, valid_end, tid);
+            process(raw[0], chunk, chunk == first_chunk);
+            if (chunk + 1 < end_chunk)
+            {
+                if (chunk + 2 < end_chunk)
+                    load_chunk<DTYPE, kVectors>(raw[0], aligned_base, (chunk + 2) * kChunk, valid_begin, valid_end, tid);
+                process(raw[1], chunk + 1, false);
+            }
+        }
+    }
+    else
+    {
+        if (first_chunk < end_chunk)
+            process(raw[0], first_chunk, true);
+    }
+
+    if (local_flags != 0)
+        atomicOr(&shared.block_flags, local_flags);
+    __syncthreads();
+
+    if (a.segments == 1)
+    {
+        // ---- the workgroup saw the whole row: finish it here
+        const uint32_t flags = shared.block_flags;
+        const uint8_t result_flags = (flags & kScanSawNan) ? NCNN_MOE_ROW_FLAG_HAS_NAN : 0;
+        if (overflow)
+        {
+            if (tid == 0)
+            {
+                write_pending(a, row);
+                a.row_state[row] = kRowNeedsGeneral;
+            }
+            return;
+        }
+        if (!greedy && (flags & kScanSawPositiveInfinity))
+        {
+            // the stable order puts +inf first and the CPU sampler rejects the row (session.cpp:84-85)
+            if (tid == 0)
+            {
+                write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
+                a.row_state[row] = kRowDone;
+            }
+            return;
+        }
+        finish_from_list(a, row, p, greedy, top_k, shared, result_flags, tid);
+        return;
+    }
+
+    // ---- several segments per row: hand the list over through the segment's record in HBM
+    uint32_t* const out_values = reinterpret_cast<uint32_t*>(a.segment_values);
+    uint32_t* const out_indices = reinterpret_cast<uint32_t*>(a.segment_indices);
+    const size_t segment_slot = static_cast<size_t>(row) * a.segments + segment;
+    const uint32_t record_entries = segment_record_entries(effective_k);
+    if (LOOPED && !overflow && shared.list_count > record_entries)
+        bound_key = tighten_list(shared, bound_key, top_k, tid);
+    const uint32_t handed = shared.list_count;
+    overflow = overflow || handed > record_entries;
+    if (!overflow)
+    {
+        for (uint32_t j = tid; j < handed; j += kScanThreads)
+        {
+            store_agent(&out_values[segment_slot * kSegmentRecordSlots + j], shared.list_keys[j]);
+            store_agent(&out_indices[segment_slot * kSegmentRecordSlots + j], static_cast<uint32_t>(shared.list_indices[j]));
+        }
+    }
+    if (tid == 0)
+    {
+        store_agent(&a.segment_counts[segment_slot], overflow ? 0u : handed);
+        uint32_t flags = shared.block_flags;
+        if (overflow)
+            flags |= kScanOverflow;
+        if (flags != 0)
+            atomicOr(&a.row_flags[row], flags);
+    }
+    // The barrier waits for this workgroup's agent-scope stores; the counter is bumped only after that.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0)
+    {
+        const uint32_t previous = __hip_atomic_fetch_add(&a.row_counter[row], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        shared.block_is_last = previous == a.segments - 1 ? 1 : 0;
+        shared.list_count = 0;
+    }
+    __syncthreads();
+    if (!shared.block_is_last)
+        return;
+
+    // ---- last workgroup of the row: every load of the merge is issued before any is used (one trip)
+    const size_t row_slot = static_cast<size_t>(row) * a.segments;
+    const uint32_t row_entries = a.segments * record_entries;
+    constexpr int kPerThread = kMergeStageSlots / kScanThreads;
+    uint32_t loaded_keys[kPerThread];
+    uint32_t loaded_indices[kPerThread];
+    uint32_t loaded_counts[kPerThread];
+    const uint32_t row_flags = load_agent(&a.row_flags[row]);
+    const bool stageable = row_entries <= static_cast<uint32_t>(kMergeStageSlots);
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+    {
+        const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
+        loaded_keys[j] = 0;
+        loaded_indices[j] = 0;
+        loaded_counts[j] = 0;
+        if (stageable && q < row_entries)
+        {
+            const uint32_t s = q / record_entries;
+            const uint32_t r = q - s * record_entries;
+            loaded_keys[j] = load_agent(&out_values[(row_slot + s) * kSegmentRecordSlots + r]);
+            loaded_indices[j] = load_agent(&out_indices[(row_slot + s) * kSegmentRecordSlots + r]);
+            loaded_counts[j] = load_agent(&a.segment_counts[row_slot + s]);
+        }
+    }
+    const uint8_t result_flags = (row_flags & kScanSawNan) ? NCNN_MOE_ROW_FLAG_HAS_NAN : 0;
+    __syncthreads();
+    if (tid == 0)
+    {
+        a.row_counter[row] = 0;
+        a.row_flags[row] = 0;
+    }
+    bool too_many = (row_flags & kScanOverflow) || !stageable;
+    uint32_t thread_key[1] = {0u};
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+    {
+        const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
+        const uint32_t r = q % record_entries;
+        loaded_keys[j] = (q < row_entries && r < loaded_counts[j]) ? loaded_keys[j] : 0u;
+        thread_key[0] = max(thread_key[0], loaded_keys[j]);
+    }
+    if (__syncthreads_or(too_many ? 1 : 0))
+    {
+        // ties (or a very long row) left more candidates than the merge holds: the full-order kernels take the row
+        if (tid == 0)
+        {
+            write_pending(a, row);
+            a.row_state[row] = kRowNeedsGeneral;
+        }
+        return;
+    }
+    if (!greedy && (row_flags & kScanSawPositiveInfinity))
+    {
+        if (tid == 0)
+        {
+            write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
+            a.row_state[row] = kRowDone;
+        }
+        return;
+    }
+    // prune: at least K candidates reach the K-th largest per-thread best (K <= 64 on this path)
+    const uint32_t prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, shared.bound, true);
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+        append_candidate(shared, loaded_keys[j] != 0u && loaded_keys[j] >= prune_key, loaded_keys[j],
+                         static_cast<int32_t>(loaded_indices[j]), lane);
+    __syncthreads();
+    if (shared.list_count > static_cast<uint32_t>(Shared::kListCap))
+    {
+        if (tid == 0)
+        {
+            write_pending(a, row);
+            a.row_state[row] = kRowNeedsGeneral;
+        }
+        return;
+    }
+    finish_from_list(a, row, p, greedy, top_k, shared, result_flags, tid);
+}
+
+} // namespace ncnn_moe_hip
+
+#endif // NCNN_MOE_HIP_SAMPLER_SELECT_H

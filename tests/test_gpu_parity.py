@@ -259,3 +259,100 @@ def test_cfg4_full():
 def test_cfg5_full():
     gpu, _ = _full_config("cfg5_tie_stress", "bf16")
     assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH == 0).all()
+
+
+WINDOW_SIZES = [1, 2, 20, 64, 65, 100, 257, 512, 513, 1000, 1024, 1025, 0]
+
+
+def _mixed_params(rows, rng):
+    params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+    params["top_k"] = np.array([WINDOW_SIZES[i % len(WINDOW_SIZES)] for i in range(rows)], dtype=np.uint32)
+    params["temperature"] = rng.uniform(0.3, 1.6, size=rows).astype(np.float32)
+    params["temperature"][rng.random(rows) < 0.08] = 0.0
+    params["top_p"] = np.where(rng.random(rows) < 0.3, 1.0, rng.uniform(0.4, 1.0, size=rows)).astype(np.float32)
+    params["min_p"] = np.where(rng.random(rows) < 0.5, 0.0, rng.uniform(0.0, 0.05, size=rows)).astype(np.float32)
+    return params
+
+
+def _plant_edge_rows(logits, first):
+    """Tie-heavy, NaN, infinite and nearly empty rows starting at row `first`; returns the rows used."""
+    vocab = logits.shape[1]
+    logits[first + 0, :] = 1.0                         # every logit tied: candidate lists overflow
+    logits[first + 1, ::3] = 2.5                       # a third of the row tied at the top
+    logits[first + 2, 100:200] = np.nan
+    logits[first + 3, :] = -np.inf
+    logits[first + 3, vocab // 2] = -3.0               # one finite logit
+    logits[first + 4, :] = np.nan
+    logits[first + 5, 10] = np.inf
+    logits[first + 6, :] = np.round(logits[first + 6, :] * 4) / 4   # heavy ties at every level
+    logits[first + 7, vocab // 3:] = -np.inf           # the tail of the row carries nothing
+    logits[first + 8, :] = -np.inf
+    logits[first + 8, :700] = np.linspace(0, -5, 700, dtype=np.float32)   # fewer finite logits than most windows
+    return 9
+
+
+@pytest.fixture(scope="module")
+def batch_sampler():
+    sampler = hip_sampler.HipSampler(320, 110000)
+    yield sampler
+    sampler.close()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_whole_row_workgroups(batch_sampler, dtype):
+    """From 256 rows on one workgroup streams a whole row and serves Top-K windows up to 1024."""
+    rng = np.random.default_rng(71)
+    rows, vocab = 300, 33333
+    logits = (rng.standard_normal((rows, vocab)) * 2.5).astype(np.float32)
+    for block in range(0, rows, 13 * 9):
+        _plant_edge_rows(logits, block)
+    _plant_edge_rows(logits, 150)
+    params = _mixed_params(rows, rng)
+    uniforms = rng.random(rows).astype(np.float32)
+    if dtype == "bf16":
+        logits = workloads.float32_to_bf16_bits(logits)
+    _check_rows(batch_sampler, logits, params, uniforms, dtype=dtype, context="whole-row workgroups " + dtype)
+
+
+def test_whole_row_long_rows(batch_sampler):
+    """Eleven chunks per workgroup: the running bound and the list tightening see many chunks."""
+    rng = np.random.default_rng(72)
+    rows, vocab = 256, 109999
+    logits = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    logits.sort(axis=1)                                 # ascending: every chunk beats the bound so far
+    logits[1::2] = logits[1::2, ::-1]                   # and descending rows
+    _plant_edge_rows(logits, 40)
+    params = _mixed_params(rows, rng)
+    uniforms = rng.random(rows).astype(np.float32)
+    _check_rows(batch_sampler, logits, params, uniforms, context="whole-row workgroups, long sorted rows")
+
+
+@pytest.mark.parametrize("rows", [200, 130, 90])
+def test_multi_chunk_segments(batch_sampler, rows):
+    """Between 65 and 255 rows of a long vocabulary a segment streams several chunks before the hand-over."""
+    rng = np.random.default_rng(73 + rows)
+    vocab = 109000
+    logits = (rng.standard_normal((rows, vocab)) * 2).astype(np.float32)
+    logits[::4] = np.sort(logits[::4], axis=1)
+    _plant_edge_rows(logits, 20)
+    params = _mixed_params(rows, rng)
+    uniforms = rng.random(rows).astype(np.float32)
+    _check_rows(batch_sampler, logits, params, uniforms, context="multi-chunk segments, %d rows" % rows)
+    bf16 = workloads.float32_to_bf16_bits(logits)
+    _check_rows(batch_sampler, bf16, params, uniforms, dtype="bf16", context="multi-chunk segments bf16, %d rows" % rows)
+
+
+def test_wide_windows_small_batch(small_sampler):
+    """A small batch is split over segments (windows up to 64); wider windows take the second select launch."""
+    rng = np.random.default_rng(74)
+    rows, vocab = 26, 39999
+    logits = (rng.standard_normal((rows, vocab)) * 2).astype(np.float32)
+    _plant_edge_rows(logits, 13)
+    params = _mixed_params(rows, rng)
+    uniforms = rng.random(rows).astype(np.float32)
+    gpu, _ = _check_rows(small_sampler, logits, params, uniforms, context="wide windows, small batch")
+    served_by_select = (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH) == 0
+    plain = np.ones(rows, dtype=bool)
+    plain[13:22] = False
+    wide = plain & (params["top_k"] >= 1) & (params["top_k"] <= 1024)
+    assert served_by_select[wide].all(), "rows with Top-K <= 1024 must not need the sort"
