@@ -94,15 +94,15 @@ uint64_t logits_span(uint32_t vocab, int dtype, const void* logits, uint64_t row
 }
 
 // How the select kernel covers a row: `segments` workgroups, each streaming `chunks_per_segment`
-// chunks.  A workgroup that sees the whole row finishes it itself and serves Top-K windows up to
-// kSelectTopK; rows split over several workgroups (small batches, so that every CU streams) are
-// merged by the last workgroup to arrive and serve windows up to kFastTopK.
+// chunks.  Small batches are split so that every CU streams; the last workgroup of a row to arrive
+// merges the segments.  From kWholeRowBatch rows on a workgroup streams the whole row and finishes it.
+// The wide variant (Top-K windows up to kSelectTopK) always takes whole rows.
 struct SelectGeometry
 {
     uint32_t segments = 1;
     uint32_t chunks_per_segment = 1;
     bool looped = true;
-    uint32_t max_top_k = kSelectTopK;
+    bool wide = false;
 };
 
 uint64_t chunk_values(int dtype)
@@ -110,22 +110,31 @@ uint64_t chunk_values(int dtype)
     return dtype == NCNN_MOE_LOGITS_F32 ? kSegmentValuesF32 : kSegmentValuesBF16;
 }
 
-SelectGeometry select_geometry(int dtype, uint64_t span, uint32_t rows, bool whole_row)
+SelectGeometry select_geometry(int dtype, uint64_t span, uint32_t rows, bool wide)
 {
     SelectGeometry g;
+    g.wide = wide;
     const uint64_t total_chunks = std::max<uint64_t>(1, (span + chunk_values(dtype) - 1) / chunk_values(dtype));
-    uint64_t segments = 1;
-    if (!whole_row && rows < static_cast<uint32_t>(kWholeRowBatch))
+    auto split = [&](int workgroups) {
+        const uint64_t wanted = (static_cast<uint64_t>(workgroups) + rows - 1) / rows;
+        uint64_t segments = std::min<uint64_t>(std::min<uint64_t>(wanted, total_chunks), static_cast<uint64_t>(kMaxSegments));
+        const uint64_t chunks_per_segment = (total_chunks + segments - 1) / segments;
+        segments = (total_chunks + chunks_per_segment - 1) / chunks_per_segment;
+        g.segments = static_cast<uint32_t>(segments);
+        g.chunks_per_segment = static_cast<uint32_t>(chunks_per_segment);
+    };
+    if (wide || rows >= static_cast<uint32_t>(kWholeRowBatch))
     {
-        const uint64_t wanted = (static_cast<uint64_t>(kSelectWorkgroupTarget) + rows - 1) / rows;
-        segments = std::min<uint64_t>(std::min<uint64_t>(wanted, total_chunks), static_cast<uint64_t>(kMaxSegments));
+        g.segments = 1;
+        g.chunks_per_segment = static_cast<uint32_t>(total_chunks);
     }
-    const uint64_t chunks_per_segment = (total_chunks + segments - 1) / segments;
-    segments = (total_chunks + chunks_per_segment - 1) / chunks_per_segment;
-    g.segments = static_cast<uint32_t>(segments);
-    g.chunks_per_segment = static_cast<uint32_t>(chunks_per_segment);
-    g.looped = chunks_per_segment > 1 || segments == 1;
-    g.max_top_k = segments == 1 ? static_cast<uint32_t>(kSelectTopK) : static_cast<uint32_t>(kFastTopK);
+    else
+    {
+        split(kSingleChunkWorkgroups);
+        if (g.chunks_per_segment > 1)
+            split(kLoopedWorkgroups); // the looped kernel keeps two workgroups per CU resident
+    }
+    g.looped = g.chunks_per_segment > 1 || g.segments == 1;
     return g;
 }
 
@@ -134,20 +143,22 @@ void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, S
 {
     a.segments = g.segments;
     a.chunks_per_segment = g.chunks_per_segment;
-    a.max_select_top_k = g.max_top_k;
+    a.max_select_top_k = g.wide ? kSelectTopK : kFastTopK;
     a.only_pending = only_pending ? 1 : 0;
     const dim3 grid(g.segments, rows, 1);
-    if (g.looped)
-        hipLaunchKernelGGL((scan_select_kernel<DTYPE, true>), grid, dim3(kScanThreads), 0, stream, a);
+    if (g.wide)
+        hipLaunchKernelGGL((scan_select_kernel<DTYPE, true, true>), grid, dim3(kScanThreads), 0, stream, a);
+    else if (g.looped)
+        hipLaunchKernelGGL((scan_select_kernel<DTYPE, true, false>), grid, dim3(kScanThreads), 0, stream, a);
     else
-        hipLaunchKernelGGL((scan_select_kernel<DTYPE, false>), grid, dim3(kScanThreads), 0, stream, a);
+        hipLaunchKernelGGL((scan_select_kernel<DTYPE, false, false>), grid, dim3(kScanThreads), 0, stream, a);
 }
 
 // Which kernels a call enqueues.  Rows a pass cannot serve are marked pending and taken by the next.
 struct SamplerPasses
 {
     bool select = true;      // the batch-shaped select kernel
-    bool wide_select = false; // one workgroup per pending row: Top-K windows up to kSelectTopK
+    bool wide_select = false; // one workgroup per row still pending: Top-K windows up to kSelectTopK
     bool full_order = false; // sort + replay for every row still pending
 };
 
@@ -198,7 +209,7 @@ int launch_sampler(
         else
             launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, a, false);
     }
-    if (passes.wide_select && batch_geometry.segments > 1)
+    if (passes.wide_select)
     {
         const SelectGeometry row_geometry = select_geometry(dtype, span, rows, true);
         if (dtype == NCNN_MOE_LOGITS_F32)

@@ -302,6 +302,8 @@ __device__ __forceinline__ uint32_t select_kth_key(const uint32_t* keys_in_lds, 
     return prefix;
 }
 
+// MAX_SLOTS: keys per lane the caller can have (m <= 64 * MAX_SLOTS).
+template <int MAX_SLOTS>
 __device__ __forceinline__ uint32_t select_kth_key_dispatch(const uint32_t* keys_in_lds, int m, int top_k, int lane)
 {
     if (m <= kWaveSize)
@@ -310,7 +312,7 @@ __device__ __forceinline__ uint32_t select_kth_key_dispatch(const uint32_t* keys
         return select_kth_key<2>(keys_in_lds, m, top_k, lane);
     if (m <= 4 * kWaveSize)
         return select_kth_key<4>(keys_in_lds, m, top_k, lane);
-    if (m <= 8 * kWaveSize)
+    if (MAX_SLOTS <= 8 || m <= 8 * kWaveSize)
         return select_kth_key<8>(keys_in_lds, m, top_k, lane);
     return select_kth_key<16>(keys_in_lds, m, top_k, lane);
 }
@@ -383,7 +385,7 @@ __device__ __forceinline__ uint32_t workgroup_kth_largest_key(
     __syncthreads();
     if (wave == 0)
     {
-        const uint32_t kth = select_kth_key_dispatch(scratch.hot_keys, static_cast<int>(scratch.hot_total), top_k, lane);
+        const uint32_t kth = select_kth_key_dispatch<8 * KEYS>(scratch.hot_keys, static_cast<int>(scratch.hot_total), top_k, lane);
         if (lane == 0)
             scratch.result = kth;
     }

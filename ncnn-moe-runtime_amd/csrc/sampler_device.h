@@ -24,12 +24,14 @@ constexpr int kSegmentValuesBF16 = kScanThreads * kVectorsPerLaneBF16 * 8; // 12
 constexpr int kFastTopK = 64;            // widest Top-K window finished by one wave
 constexpr int kSelectTopK = 1024;
 constexpr int kTwoKeyBoundTopK = 512; // wider windows bound their first chunk by a select over all its values         // widest Top-K window of the select path (rows of one segment)
-constexpr int kSingleListCap = 512;      // candidate list of a workgroup that streams a single chunk
-constexpr int kLoopedListCap = 4096;     // candidate list of a workgroup that streams several chunks
+constexpr int kNarrowListCap = 512;      // candidate list for Top-K windows up to kFastTopK
+constexpr int kWideListCap = 4096;       // candidate list for Top-K windows up to kSelectTopK
 constexpr int kSegmentRecordSlots = 256; // candidate slots of a segment's record in HBM
 constexpr int kMaxSegments = 16;
 constexpr int kWholeRowBatch = 256;          // from this many rows on, one workgroup streams a whole row
-constexpr int kSelectWorkgroupTarget = 1024; // workgroups a smaller batch is split into (4 per CU)         // segments per row the row merge can stage in one trip
+constexpr int kSingleChunkWorkgroups = 1024;  // workgroups a smaller batch is split into when each streams one chunk (4 per CU)
+constexpr int kLoopedWorkgroups = 512;        // ... and when each streams several chunks (2 per CU)
+         // segments per row the row merge can stage in one trip
 constexpr int kMergeStageSlots = 4096;   // record slots of a row loaded in one trip (8 per thread)
 
 // Full-order ("general") path geometry.
@@ -108,11 +110,11 @@ __host__ __device__ __forceinline__ int resolve_row_mode(
     return kModeGeneral;
 }
 
-// Entries of a segment's record that the row merge reads: twice the Top-K window plus 64 (a list is
-// tightened when it grows past that; ties beyond it overflow to the full-order path).
+// Entries of a segment's record that the row merge reads: twice the Top-K window plus 16 (a segment
+// hands over K candidates and a few more; ties beyond that overflow to the full-order path).
 __host__ __device__ __forceinline__ uint32_t segment_record_entries(uint32_t effective_k)
 {
-    const uint32_t entries = effective_k * 2u + 64u;
+    const uint32_t entries = effective_k * 2u + 16u;
     return entries > static_cast<uint32_t>(kSegmentRecordSlots) ? static_cast<uint32_t>(kSegmentRecordSlots) : entries;
 }
 

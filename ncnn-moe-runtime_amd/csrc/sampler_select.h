@@ -18,11 +18,11 @@
 
 namespace ncnn_moe_hip {
 
-template <bool LOOPED>
+template <bool WIDE>
 struct SelectShared
 {
-    static constexpr int kListCap = LOOPED ? kLoopedListCap : kSingleListCap;
-    static constexpr int kSortedCap = LOOPED ? kSelectTopK : 1;
+    static constexpr int kListCap = WIDE ? kWideListCap : kNarrowListCap;
+    static constexpr int kSortedCap = WIDE ? kSelectTopK : 1;
     BoundScratch bound;
     uint32_t list_keys[kListCap];
     int32_t list_indices[kListCap];
@@ -38,8 +38,8 @@ struct SelectShared
 
 // Appends the caller's candidate (if `hit`) to the workgroup's list.  Positions are reserved per
 // wave with one LDS atomic; the order inside the list is irrelevant.  Called by whole waves.
-template <bool LOOPED>
-__device__ __forceinline__ void append_candidate(SelectShared<LOOPED>& shared, bool hit, uint32_t key, int32_t index, int lane)
+template <bool WIDE>
+__device__ __forceinline__ void append_candidate(SelectShared<WIDE>& shared, bool hit, uint32_t key, int32_t index, int lane)
 {
     const uint64_t hits = __ballot(hit);
     if (hits == 0)
@@ -49,7 +49,7 @@ __device__ __forceinline__ void append_candidate(SelectShared<LOOPED>& shared, b
         base = atomicAdd(&shared.list_count, static_cast<uint32_t>(__popcll(hits)));
     base = __builtin_amdgcn_readlane(base, __builtin_ctzll(hits));
     const uint32_t position = base + static_cast<uint32_t>(lanes_below(hits));
-    if (hit && position < static_cast<uint32_t>(SelectShared<LOOPED>::kListCap))
+    if (hit && position < static_cast<uint32_t>(SelectShared<WIDE>::kListCap))
     {
         shared.list_keys[position] = key;
         shared.list_indices[position] = index;
@@ -58,12 +58,12 @@ __device__ __forceinline__ void append_candidate(SelectShared<LOOPED>& shared, b
 
 // Raises the bound to (a lower bound of) the K-th best candidate of the list and drops the
 // candidates below it.  All threads call it; returns the new bound key.
-template <bool LOOPED>
-__device__ __forceinline__ uint32_t tighten_list(SelectShared<LOOPED>& shared, uint32_t bound_key, int top_k, int tid)
+template <bool WIDE>
+__device__ __forceinline__ uint32_t tighten_list(SelectShared<WIDE>& shared, uint32_t bound_key, int top_k, int tid)
 {
-    constexpr int kPerThread = SelectShared<LOOPED>::kListCap / kScanThreads;
+    constexpr int kPerThread = SelectShared<WIDE>::kListCap / kScanThreads;
     const int lane = tid & (kWaveSize - 1);
-    const uint32_t count = min(shared.list_count, static_cast<uint32_t>(SelectShared<LOOPED>::kListCap));
+    const uint32_t count = min(shared.list_count, static_cast<uint32_t>(SelectShared<WIDE>::kListCap));
     uint32_t keys[kPerThread];
     int32_t indices[kPerThread];
     uint32_t best = 0, second = 0; // the thread's two best candidates: two distinct logits
@@ -77,8 +77,17 @@ __device__ __forceinline__ uint32_t tighten_list(SelectShared<LOOPED>& shared, u
         best = max(best, keys[j]);
     }
     // at least K candidates reach the K-th largest of the per-thread best and second-best keys
-    const uint32_t thread_keys[2] = {best, second};
-    const uint32_t kth = workgroup_kth_largest_key(thread_keys, top_k, tid, shared.bound, true);
+    uint32_t kth;
+    if constexpr (kPerThread > 1)
+    {
+        const uint32_t thread_keys[2] = {best, second};
+        kth = workgroup_kth_largest_key(thread_keys, top_k, tid, shared.bound, true);
+    }
+    else
+    {
+        const uint32_t thread_keys[1] = {best};
+        kth = workgroup_kth_largest_key(thread_keys, top_k, tid, shared.bound, true);
+    }
     bound_key = max(bound_key, kth);
     if (tid == 0)
         shared.list_count = 0;
@@ -90,19 +99,44 @@ __device__ __forceinline__ uint32_t tighten_list(SelectShared<LOOPED>& shared, u
     return bound_key;
 }
 
+// The ordered window (lane i holds candidate i of n <= 64) to the row's result; one wave.
+__device__ __forceinline__ void finish_ordered_wave(
+    const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p, bool greedy,
+    float value, int32_t index, int n, int lane, uint8_t result_flags)
+{
+    if (greedy)
+    {
+        if (lane == 0)
+        {
+            write_token(a, row, p, index, 1.0f, 1u, 0, result_flags);
+            if (a.distribution_count != nullptr && row == 0)
+            {
+                *a.distribution_count = 1;
+                if (a.distribution_cap > 0)
+                {
+                    a.distribution_ids[0] = index;
+                    a.distribution_probabilities[0] = 1.0f;
+                }
+            }
+        }
+        return;
+    }
+    finish_row_wave(a, row, p, value, index, n, lane, result_flags);
+}
+
 // From the candidate list to the sampled token: exact best K, their order, the epilogue.
 // All threads of the workgroup call it; n_list <= kListCap.
-template <bool LOOPED>
+template <bool WIDE>
 __device__ __forceinline__ void finish_from_list(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p, bool greedy, int top_k,
-    SelectShared<LOOPED>& shared, uint8_t result_flags, int tid)
+    SelectShared<WIDE>& shared, uint8_t result_flags, int tid)
 {
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
     int n_list = static_cast<int>(shared.list_count);
     if (top_k <= kFastTopK)
     {
-        if constexpr (LOOPED)
+        if constexpr (WIDE)
         {
             if (n_list > 8 * kWaveSize)
             {
@@ -124,8 +158,37 @@ __device__ __forceinline__ void finish_from_list(
             return;
         int n = 0;
         if (n_list <= kWaveSize)
-            n = select_best_wave<1>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
-        else if (n_list <= 2 * kWaveSize)
+        {
+            // one candidate per lane: its rank among all of them is its place in the window
+            const uint32_t key = lane < n_list ? shared.list_keys[lane] : 0u;
+            const int32_t candidate_index = lane < n_list ? shared.list_indices[lane] : 0;
+            int before = 0;
+            for (int j = 0; j < n_list; ++j)
+            {
+                const uint32_t other_key = static_cast<uint32_t>(read_lane(static_cast<int>(key), j));
+                const int32_t other_index = read_lane(candidate_index, j);
+                before += (other_key > key || (other_key == key && other_index < candidate_index)) ? 1 : 0;
+            }
+            if (lane < n_list && before < top_k)
+            {
+                shared.final_values[before] = value_from_ascending_key(key);
+                shared.final_indices[before] = candidate_index;
+            }
+            n = n_list < top_k ? n_list : top_k;
+            if (lane == 0)
+                a.row_state[row] = kRowDone;
+            if (n == 0)
+            {
+                if (lane == 0)
+                    write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
+                return;
+            }
+            const float value = lane < n ? shared.final_values[lane] : 0.0f;
+            const int32_t index = lane < n ? shared.final_indices[lane] : -1;
+            finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags);
+            return;
+        }
+        if (n_list <= 2 * kWaveSize)
             n = select_best_wave<2>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
         else if (n_list <= 4 * kWaveSize)
             n = select_best_wave<4>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
@@ -151,31 +214,14 @@ __device__ __forceinline__ void finish_from_list(
         }
         value = lane < n ? shared.final_values[lane] : 0.0f;
         index = lane < n ? shared.final_indices[lane] : -1;
-        if (greedy)
-        {
-            if (lane == 0)
-            {
-                write_token(a, row, p, index, 1.0f, 1u, 0, result_flags);
-                if (a.distribution_count != nullptr && row == 0)
-                {
-                    *a.distribution_count = 1;
-                    if (a.distribution_cap > 0)
-                    {
-                        a.distribution_ids[0] = index;
-                        a.distribution_probabilities[0] = 1.0f;
-                    }
-                }
-            }
-            return;
-        }
-        finish_row_wave(a, row, p, value, index, n, lane, result_flags);
+        finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags);
         return;
     }
-    if constexpr (LOOPED)
+    if constexpr (WIDE)
     {
         // ---- a window wider than one wave: exact K-th best key, then ranks by counting, then the
         // walk over the ordered window with exact running sums
-        constexpr int kPerThread = SelectShared<LOOPED>::kListCap / kScanThreads;
+        constexpr int kPerThread = SelectShared<WIDE>::kListCap / kScanThreads;
         if (n_list > top_k + 64)
             tighten_list(shared, 0u, top_k, tid); // fewer candidates to rank
         const int n_ranked = static_cast<int>(shared.list_count);
@@ -242,11 +288,14 @@ __device__ __forceinline__ void load_chunk(
     }
 }
 
-template <int DTYPE, bool LOOPED>
-__global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_F32) ? 8 : 1) void scan_select_kernel(SamplerArgs a)
+// LOOPED: a workgroup streams several chunks (double-buffered).  WIDE: Top-K windows up to kSelectTopK
+// (a long candidate list, more registers and LDS); otherwise up to kFastTopK.
+template <int DTYPE, bool LOOPED, bool WIDE>
+__global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_F32) ? 8 : (WIDE ? 1 : 4)) void scan_select_kernel(SamplerArgs a)
 {
     using Vector = LogitsVector<DTYPE>;
-    using Shared = SelectShared<LOOPED>;
+    static_assert(LOOPED || !WIDE, "wide windows are served by whole-row workgroups");
+    using Shared = SelectShared<WIDE>;
     constexpr int kWidth = Vector::kWidth;
     constexpr int kVectors = Vector::kVectorsPerLane;
     constexpr int kLaneValues = kVectors * kWidth;
@@ -349,19 +398,37 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
 #pragma unroll
             for (int c = 0; c < kWidth; ++c)
             {
-                float x = values[v * kWidth + c];
+                const float x = values[v * kWidth + c];
                 saw_nan = saw_nan || (x != x);
-                if (greedy && x == __uint_as_float(kPositiveInfinity))
-                {
-                    x = __uint_as_float(kNegativeInfinity); // greedy skips every non-finite logit (session.cpp:411-412)
-                    values[v * kWidth + c] = x;
-                }
                 vector_max = fmaxf(vector_max, x);
             }
             group_max[v] = vector_max;
             lane_max = fmaxf(lane_max, vector_max);
-            if constexpr (LOOPED)
-                half_max[v < (kVectors + 1) / 2 ? 0 : 1] = fmaxf(half_max[v < (kVectors + 1) / 2 ? 0 : 1], vector_max);
+        }
+        if (greedy && __ballot(lane_max == __uint_as_float(kPositiveInfinity)) != 0)
+        {
+            // greedy skips every non-finite logit (session.cpp:411-412): rare, so redone out of line
+            lane_max = __uint_as_float(kNegativeInfinity);
+#pragma unroll
+            for (int v = 0; v < kVectors; ++v)
+            {
+                float vector_max = __uint_as_float(kNegativeInfinity);
+#pragma unroll
+                for (int c = 0; c < kWidth; ++c)
+                {
+                    if (values[v * kWidth + c] == __uint_as_float(kPositiveInfinity))
+                        values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
+                    vector_max = fmaxf(vector_max, values[v * kWidth + c]);
+                }
+                group_max[v] = vector_max;
+                lane_max = fmaxf(lane_max, vector_max);
+            }
+        }
+        if constexpr (WIDE)
+        {
+#pragma unroll
+            for (int v = 0; v < kVectors; ++v)
+                half_max[v < (kVectors + 1) / 2 ? 0 : 1] = fmaxf(half_max[v < (kVectors + 1) / 2 ? 0 : 1], group_max[v]);
         }
         if (saw_nan)
             local_flags |= kScanSawNan;
@@ -372,12 +439,12 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         // each hold a distinct logit at least that large, so the K-th best logit of the row is no smaller.
         if (first_of_segment)
         {
-            if (LOOPED && top_k > kTwoKeyBoundTopK)
+            if (WIDE && top_k > kTwoKeyBoundTopK)
             {
                 // a wide window: the lane maxima bound too loosely, so select over every value of the chunk
                 bound_key = max(bound_key, workgroup_loose_kth_of_values(values, top_k, tid, shared.bound));
             }
-            else if constexpr (LOOPED)
+            else if constexpr (WIDE)
             {
                 // two keys per lane (the maxima of the two halves of its vectors): 1024 distinct logits
                 const uint32_t lane_keys[2] = {
@@ -406,7 +473,9 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
                 {
                     const float x = values[v * kWidth + c];
                     const uint32_t element = chunk_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth + c - misalignment;
-                    append_candidate(shared, vector_hit && x >= threshold, ascending_key(x), static_cast<int32_t>(element), lane);
+                    const bool hit = vector_hit && x >= threshold;
+                    if (__ballot(hit) != 0)
+                        append_candidate(shared, hit, ascending_key(x), static_cast<int32_t>(element), lane);
                 }
             }
         }
@@ -570,7 +639,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         }
         return;
     }
-    // prune: at least K candidates reach the K-th largest per-thread best (K <= 64 on this path)
+    // prune: at least K candidates reach this lower bound of the K-th largest per-thread best
     const uint32_t prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, shared.bound, true);
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
