@@ -302,7 +302,7 @@ __device__ __forceinline__ uint32_t select_kth_key(const uint32_t* keys_in_lds, 
     return prefix;
 }
 
-// MAX_SLOTS: keys per lane the caller can have (m <= 64 * MAX_SLOTS).
+// Exact top_k-th largest of m keys in LDS, by one wave; m <= 64 * MAX_SLOTS (MAX_SLOTS 8 or 16).
 template <int MAX_SLOTS>
 __device__ __forceinline__ uint32_t select_kth_key_dispatch(const uint32_t* keys_in_lds, int m, int top_k, int lane)
 {

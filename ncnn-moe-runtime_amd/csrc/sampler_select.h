@@ -271,20 +271,23 @@ __device__ __forceinline__ void finish_from_list(
     }
 }
 
+// Issues the chunk's loads.  A vector with no valid element reads the row's last vector instead (and is
+// ignored later): the loads stay free of branches, so the next chunk's loads can be in flight while
+// this chunk is processed.  vocab >= 1.
 template <int DTYPE, int VECTORS>
 __device__ __forceinline__ void load_chunk(
-    uint4 (&raw)[VECTORS], const char* aligned_base, uint32_t chunk_base, uint32_t valid_begin, uint32_t valid_end, int tid)
+    uint4 (&raw)[VECTORS], const char* aligned_base, uint32_t chunk_base, uint32_t valid_begin, uint32_t segment_end,
+    uint32_t valid_end, int tid)
 {
     using Vector = LogitsVector<DTYPE>;
-    constexpr uint32_t kNegativeInfinity = 0xff800000u;
+    const uint32_t last_vector = (valid_end - 1u) / Vector::kWidth * Vector::kWidth;
 #pragma unroll
     for (int v = 0; v < VECTORS; ++v)
     {
         const uint32_t first = chunk_base + static_cast<uint32_t>(v * kScanThreads + tid) * Vector::kWidth;
-        if (first < valid_end && first + Vector::kWidth > valid_begin)
-            raw[v] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(first) * Vector::kElementBytes);
-        else
-            raw[v] = make_uint4(kNegativeInfinity, kNegativeInfinity, kNegativeInfinity, kNegativeInfinity);
+        const bool any_valid = first < segment_end && first + Vector::kWidth > valid_begin;
+        const uint32_t source = any_valid ? first : last_vector;
+        raw[v] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(source) * Vector::kElementBytes);
     }
 }
 
@@ -335,7 +338,11 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     }
     const bool greedy = mode == kModeGreedy;
     const int top_k = static_cast<int>(effective_k);
-    const uint32_t tighten_limit = static_cast<uint32_t>(2 * top_k + 64);
+    // the list is tightened when it grows past this; a wide list keeps room for a chunk's additions
+    const uint32_t tighten_limit = WIDE ? static_cast<uint32_t>(2 * top_k + 64) : static_cast<uint32_t>(kNarrowListCap - 192);
+    uint32_t next_check = 0;      // chunk at which the list is looked at next
+    uint32_t count_at_check = 0;  // list length at the last look
+    uint32_t chunk_at_check = 0;  // first chunk after the last look
 
     if (tid == 0)
     {
@@ -353,14 +360,16 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     const uint32_t first_chunk = segment * a.chunks_per_segment;
     const uint32_t total_chunks = (valid_end + kChunk - 1) / kChunk;
     const uint32_t end_chunk = min(total_chunks, first_chunk + a.chunks_per_segment);
+    // positions this workgroup covers end here; a chunk past end_chunk holds nothing valid
+    const uint32_t segment_end = min(valid_end, end_chunk * kChunk);
+    chunk_at_check = first_chunk;
 
     uint32_t bound_key = 0; // ascending key every Top-K member is known to reach; 0: none yet
     uint32_t local_flags = 0;
     bool overflow = false;
 
     uint4 raw[2][kVectors];
-    if (first_chunk < end_chunk)
-        load_chunk<DTYPE, kVectors>(raw[0], aligned_base, first_chunk * kChunk, valid_begin, valid_end, tid);
+    load_chunk<DTYPE, kVectors>(raw[0], aligned_base, first_chunk * kChunk, valid_begin, segment_end, valid_end, tid);
     __syncthreads();
 
     // Processes the chunk held in `buffer`; all indexing is static after unrolling.
@@ -375,7 +384,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         for (int v = 0; v < kVectors; ++v)
         {
             const uint32_t first = chunk_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth;
-            const bool any_valid = first < valid_end && first + kWidth > valid_begin;
+            const bool any_valid = first < segment_end && first + kWidth > valid_begin;
             if (any_valid)
                 Vector::unpack(buffer[v], &values[v * kWidth]);
             else
@@ -384,13 +393,13 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
                 for (int c = 0; c < kWidth; ++c)
                     values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
             }
-            if (any_valid && (first < valid_begin || first + kWidth > valid_end))
+            if (any_valid && (first < valid_begin || first + kWidth > segment_end))
             {
 #pragma unroll
                 for (int c = 0; c < kWidth; ++c)
                 {
                     const uint32_t position = first + c;
-                    if (position < valid_begin || position >= valid_end)
+                    if (position < valid_begin || position >= segment_end)
                         values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
                 }
             }
@@ -465,7 +474,12 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
 #pragma unroll
         for (int v = 0; v < kVectors; ++v)
         {
-            const bool vector_hit = group_max[v] >= threshold;
+            // the vector's maximum is recomputed here rather than kept across the bound computation
+            float vector_max = values[v * kWidth];
+#pragma unroll
+            for (int c = 1; c < kWidth; ++c)
+                vector_max = fmaxf(vector_max, values[v * kWidth + c]);
+            const bool vector_hit = (LOOPED ? group_max[v] : vector_max) >= threshold;
             if (__ballot(vector_hit) != 0)
             {
 #pragma unroll
@@ -479,32 +493,54 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
                 }
             }
         }
-        __syncthreads();
-        if (shared.list_count > static_cast<uint32_t>(Shared::kListCap))
-            overflow = true; // candidates were dropped: only the full-order path can serve the row
-        else if (LOOPED && shared.list_count > tighten_limit)
-            bound_key = tighten_list(shared, bound_key, top_k, tid);
+        if constexpr (!LOOPED)
+        {
+            __syncthreads();
+            if (shared.list_count > static_cast<uint32_t>(Shared::kListCap))
+                overflow = true; // candidates were dropped: only the full-order path can serve the row
+        }
+        else if (first_of_segment || chunk >= next_check)
+        {
+            // The list is looked at (a barrier) only as often as its growth asks for: once the bound is
+            // tight a chunk adds next to nothing and the waves stream on without waiting for each other.
+            __syncthreads();
+            const uint32_t count = shared.list_count;
+            if (count > static_cast<uint32_t>(Shared::kListCap))
+                overflow = true;
+            else
+            {
+                const uint32_t chunks = chunk - chunk_at_check + 1u;
+                const uint32_t rate = (count - count_at_check + chunks - 1u) / chunks; // candidates per chunk
+                if (count > tighten_limit)
+                    bound_key = tighten_list(shared, bound_key, top_k, tid);
+                count_at_check = shared.list_count;
+                chunk_at_check = chunk + 1u;
+                const uint32_t slack = static_cast<uint32_t>(Shared::kListCap) - count_at_check;
+                const uint32_t interval = slack / (2u * rate + 16u);
+                next_check = chunk + (interval < 1u ? 1u : (interval > 8u ? 8u : interval));
+            }
+        }
     };
 
     if constexpr (LOOPED)
     {
+        // Two chunks per trip, the loads of the next chunk always in flight while one is processed.  The
+        // loop is free of branches around loads: a chunk past end_chunk reads the row's last vector and
+        // counts nothing.
         for (uint32_t chunk = first_chunk; chunk < end_chunk; chunk += 2)
         {
-            if (chunk + 1 < end_chunk)
-                load_chunk<DTYPE, kVectors>(raw[1], aligned_base, (chunk + 1) * kChunk, valid_begin, valid_end, tid);
+            load_chunk<DTYPE, kVectors>(raw[1], aligned_base, (chunk + 1) * kChunk, valid_begin, segment_end, valid_end, tid);
             process(raw[0], chunk, chunk == first_chunk);
-            if (chunk + 1 < end_chunk)
-            {
-                if (chunk + 2 < end_chunk)
-                    load_chunk<DTYPE, kVectors>(raw[0], aligned_base, (chunk + 2) * kChunk, valid_begin, valid_end, tid);
-                process(raw[1], chunk + 1, false);
-            }
+            load_chunk<DTYPE, kVectors>(raw[0], aligned_base, (chunk + 2) * kChunk, valid_begin, segment_end, valid_end, tid);
+            process(raw[1], chunk + 1, false);
         }
+        __syncthreads();
+        if (shared.list_count > static_cast<uint32_t>(Shared::kListCap))
+            overflow = true;
     }
     else
     {
-        if (first_chunk < end_chunk)
-            process(raw[0], first_chunk, true);
+        process(raw[0], first_chunk, true);
     }
 
     if (local_flags != 0)

@@ -21,7 +21,9 @@ def small_sampler():
     sampler.close()
 
 
-def _check_rows(sampler, logits, params, uniforms, stop_ids=None, dtype="f32", context="", general=False, vocab=None):
+def _check_rows(sampler, logits, params, uniforms, stop_ids=None, dtype="f32", context="", general=False, vocab=None,
+                select_rows=None):
+    """select_rows: rows that the select kernels must serve themselves (no sort)."""
     _announce(context + (" [general]" if general else ""))
     sampler.force_general(general)
     try:
@@ -31,6 +33,9 @@ def _check_rows(sampler, logits, params, uniforms, stop_ids=None, dtype="f32", c
         sampler.force_general(False)
     cpu = parity_util.run_oracle(logits, params, uniforms, stop_ids, vocab=vocab)
     parity_util.assert_results_match(gpu, cpu, dtype, context)
+    if select_rows is not None:
+        sorted_rows = np.nonzero(select_rows & ((gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH) != 0))[0]
+        assert sorted_rows.size == 0, "%s: rows %s took the full-order path" % (context, sorted_rows[:8])
     return gpu, cpu
 
 
@@ -156,8 +161,14 @@ def test_cfg1_plumbing(small_sampler, general):
     w = workloads.make_workload("cfg1_plumbing", rows=8)
     greedy = w["params"].copy()
     greedy["temperature"] = 0.0
-    _check_rows(small_sampler, w["logits"], greedy, w["uniforms"], context="cfg1 greedy", general=general)
-    _check_rows(small_sampler, w["logits"], w["params"], w["uniforms"], context="cfg1 T.8 K50 P.9", general=general)
+    select_rows = None if general else np.ones(8, dtype=bool)
+    _check_rows(small_sampler, w["logits"], greedy, w["uniforms"], context="cfg1 greedy", general=general,
+                select_rows=select_rows)
+    _check_rows(small_sampler, w["logits"], w["params"], w["uniforms"], context="cfg1 T.8 K50 P.9", general=general,
+                select_rows=select_rows)
+    if not general:
+        _check_rows(small_sampler, w["logits"][:1], w["params"][:1], w["uniforms"][:1], context="cfg1, one row",
+                    select_rows=select_rows[:1])
     status, ids, probabilities, count = small_sampler.distribution(0, 0.8, 50, 0.9, 0.0)
     oracle_status, oracle_ids, oracle_probabilities = oracle_lib.oracle_distribution(w["logits"][0], 0.8, 50, 0.9, 0.0)
     assert status == oracle_status == 0 and count == oracle_ids.size
@@ -291,6 +302,14 @@ def _plant_edge_rows(logits, first):
     return 9
 
 
+def _select_rows(params, edge_blocks):
+    """Rows the select kernels must serve without the sort: greedy or 1 <= Top-K <= 1024, outside the edge rows."""
+    mask = (params["temperature"] == 0.0) | ((params["top_k"] >= 1) & (params["top_k"] <= 1024))
+    for first in edge_blocks:
+        mask[first:first + 9] = False
+    return mask
+
+
 @pytest.fixture(scope="module")
 def batch_sampler():
     sampler = hip_sampler.HipSampler(320, 110000)
@@ -311,7 +330,8 @@ def test_whole_row_workgroups(batch_sampler, dtype):
     uniforms = rng.random(rows).astype(np.float32)
     if dtype == "bf16":
         logits = workloads.float32_to_bf16_bits(logits)
-    _check_rows(batch_sampler, logits, params, uniforms, dtype=dtype, context="whole-row workgroups " + dtype)
+    _check_rows(batch_sampler, logits, params, uniforms, dtype=dtype, context="whole-row workgroups " + dtype,
+                select_rows=_select_rows(params, list(range(0, rows, 13 * 9)) + [150]))
 
 
 def test_whole_row_long_rows(batch_sampler):
@@ -337,7 +357,10 @@ def test_multi_chunk_segments(batch_sampler, rows):
     _plant_edge_rows(logits, 20)
     params = _mixed_params(rows, rng)
     uniforms = rng.random(rows).astype(np.float32)
-    _check_rows(batch_sampler, logits, params, uniforms, context="multi-chunk segments, %d rows" % rows)
+    select_rows = _select_rows(params, [20])
+    select_rows[::4] = False   # ascending rows may overflow the candidate list: every chunk beats the bound
+    _check_rows(batch_sampler, logits, params, uniforms, context="multi-chunk segments, %d rows" % rows,
+                select_rows=select_rows)
     bf16 = workloads.float32_to_bf16_bits(logits)
     _check_rows(batch_sampler, bf16, params, uniforms, dtype="bf16", context="multi-chunk segments bf16, %d rows" % rows)
 
