@@ -122,6 +122,7 @@ def main():
     parser.add_argument("--steps", type=int, default=2000)
     parser.add_argument("--warmup", type=int, default=200)
     parser.add_argument("--workload", default="cfg2_topk_topp")
+    parser.add_argument("--rows", type=int, default=0, help="batch rows (0: the configuration's own)")
     parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
     parser.add_argument("--cpu-rows", type=int, default=64)
     parser.add_argument("--no-cpu-baseline", action="store_true")
@@ -141,7 +142,7 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    workload = workloads.make_workload(args.workload)
+    workload = workloads.make_workload(args.workload, rows=args.rows if args.rows > 0 else None)
     rows, vocab = workload["rows"], workload["vocab"]
     element_bytes = 4 if workload["dtype"] == "f32" else 2
     dtype_code = hip_sampler.LOGITS_F32 if workload["dtype"] == "f32" else hip_sampler.LOGITS_BF16
