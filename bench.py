@@ -201,6 +201,35 @@ def main():
         wall_seconds = time.perf_counter() - wall_start
     event_seconds = start_event.elapsed_time(stop_event) * 1e-3
     seconds_per_step = event_seconds / args.steps
+
+    # Beside the headline: the spread of single launches (one event pair per launch, which adds the
+    # event's own cost to each) and the same loop on ONE buffer, which the 256 MB Infinity Cache holds.
+    detail_steps = min(args.steps, 200)
+    with torch.cuda.stream(stream):
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(detail_steps)]
+        for index, (first, last) in enumerate(pairs):
+            first.record(stream)
+            step(index)
+            last.record(stream)
+        stream.synchronize()
+        single_launch_us = np.array([first.elapsed_time(last) * 1e3 for first, last in pairs])
+        resident_start = torch.cuda.Event(enable_timing=True)
+        resident_stop = torch.cuda.Event(enable_timing=True)
+        for _ in range(10):
+            step(0)
+        resident_start.record(stream)
+        for _ in range(detail_steps):
+            step(0)
+        resident_stop.record(stream)
+        stream.synchronize()
+    torch.cuda.synchronize()
+    detail = {
+        "single_launch_us_p10_median_p90": [float(np.percentile(single_launch_us, q)) for q in (10, 50, 90)],
+        "single_launch_note": "one HIP event pair per launch, %d launches; includes the events' own cost" % detail_steps,
+        "cache_resident_ms_per_step": resident_start.elapsed_time(resident_stop) / detail_steps,
+        "cache_resident_note": "same loop on one logits buffer (%.1f MB), held by the Infinity Cache where it fits; "
+                               "not the reported value" % (batch_bytes / 1e6),
+    }
     if args.copy_calibration > 0:
         source = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=device)
         target = torch.empty_like(source)
@@ -248,12 +277,13 @@ def main():
             "peak": HBM_PEAK_BYTES_PER_S / 1e9,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_BYTES_PER_S,
-            "traffic": measured_traffic(workload["name"]),
+            "traffic": measured_traffic(workload["name"]) if args.rows == 0 else None,
             "kernel": "scan_select_kernel",
             "algorithmic_bytes_per_launch": bytes_per_launch,
         },
         "parity": parity,
         "wall_ms_per_step": wall_seconds / args.steps * 1e3,
+        "detail": detail,
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(workload, host_threads, args.cpu_rows)
