@@ -315,6 +315,26 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
 
     if (a.only_pending && a.row_state[row] != kRowNeedsGeneral)
         return;
+    // The first chunk's loads go out before anything that waits for the row's options.
+    const char* row_pointer = static_cast<const char*>(a.logits) +
+        static_cast<size_t>(row) * a.row_stride * Vector::kElementBytes;
+    const uint32_t misalignment =
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row_pointer) & 15u) / Vector::kElementBytes;
+    const char* aligned_base = row_pointer - static_cast<size_t>(misalignment) * Vector::kElementBytes;
+    const uint32_t valid_begin = misalignment;
+    const uint32_t valid_end = misalignment + a.vocab;
+    const uint32_t first_chunk = segment * a.chunks_per_segment;
+    const uint32_t total_chunks = (valid_end + kChunk - 1) / kChunk;
+    const uint32_t end_chunk = min(total_chunks, first_chunk + a.chunks_per_segment);
+    // positions this workgroup covers end here; a chunk past end_chunk holds nothing valid
+    const uint32_t segment_end = min(valid_end, end_chunk * kChunk);
+
+    uint32_t bound_key = 0; // ascending key every Top-K member is known to reach; 0: none yet
+    uint32_t local_flags = 0;
+    bool overflow = false;
+
+    uint4 raw[2][kVectors];
+    load_chunk<DTYPE, kVectors>(raw[0], aligned_base, first_chunk * kChunk, valid_begin, segment_end, valid_end, tid);
     const ncnn_moe_sample_params p = a.params[row];
     uint32_t effective_k = 0;
     int status = NCNN_MOE_ROW_OK;
@@ -342,7 +362,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     const uint32_t tighten_limit = WIDE ? static_cast<uint32_t>(2 * top_k + 64) : static_cast<uint32_t>(kNarrowListCap - 192);
     uint32_t next_check = 0;      // chunk at which the list is looked at next
     uint32_t count_at_check = 0;  // list length at the last look
-    uint32_t chunk_at_check = 0;  // first chunk after the last look
+    uint32_t chunk_at_check = first_chunk;  // first chunk after the last look
 
     if (tid == 0)
     {
@@ -350,26 +370,6 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         shared.list_count = 0;
     }
 
-    const char* row_pointer = static_cast<const char*>(a.logits) +
-        static_cast<size_t>(row) * a.row_stride * Vector::kElementBytes;
-    const uint32_t misalignment =
-        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row_pointer) & 15u) / Vector::kElementBytes;
-    const char* aligned_base = row_pointer - static_cast<size_t>(misalignment) * Vector::kElementBytes;
-    const uint32_t valid_begin = misalignment;
-    const uint32_t valid_end = misalignment + a.vocab;
-    const uint32_t first_chunk = segment * a.chunks_per_segment;
-    const uint32_t total_chunks = (valid_end + kChunk - 1) / kChunk;
-    const uint32_t end_chunk = min(total_chunks, first_chunk + a.chunks_per_segment);
-    // positions this workgroup covers end here; a chunk past end_chunk holds nothing valid
-    const uint32_t segment_end = min(valid_end, end_chunk * kChunk);
-    chunk_at_check = first_chunk;
-
-    uint32_t bound_key = 0; // ascending key every Top-K member is known to reach; 0: none yet
-    uint32_t local_flags = 0;
-    bool overflow = false;
-
-    uint4 raw[2][kVectors];
-    load_chunk<DTYPE, kVectors>(raw[0], aligned_base, first_chunk * kChunk, valid_begin, segment_end, valid_end, tid);
     __syncthreads();
 
     // Processes the chunk held in `buffer`; all indexing is static after unrolling.
