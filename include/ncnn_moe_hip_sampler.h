@@ -146,6 +146,52 @@ int ncnn_moe_hip_sampler_distribution(
     ncnn_moe_hip_sampler* sampler, uint32_t row, const ncnn_moe_sample_params* params,
     uint32_t cap, int32_t* ids, float* probabilities, uint32_t* count, uint32_t* status);
 
+/* Outcome of one speculative verification step. */
+enum ncnn_moe_verify_status
+{
+    NCNN_MOE_VERIFY_OK = 0,
+    /* a sampling error of a row that the accept loop reached; row_status holds the ncnn_moe_row_status
+     * (the target row's error wins over the draft row's, src/engine/session.cpp:805-813) */
+    NCNN_MOE_VERIFY_ROW_ERROR = 1,
+    NCNN_MOE_VERIFY_ZERO_DRAFT_PROBABILITY = 2, /* "sampled draft token has zero probability" (:822-830) */
+    NCNN_MOE_VERIFY_RESIDUAL_EMPTY = 3,         /* "speculative residual distribution is empty" (:170-175) */
+    NCNN_MOE_VERIFY_RESIDUAL_FAILED = 4,        /* "speculative residual sampling failed" (:199-201) */
+    /* Not a CPU-sampler error: with temperature > 0 this entry serves Top-K windows of 1..64 only. */
+    NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW = 5
+};
+
+typedef struct ncnn_moe_verify_result
+{
+    uint32_t accepted;            /* draft tokens accepted, 0..draft_count */
+    int32_t next_token_id;        /* the token emitted after them; -1 unless status is NCNN_MOE_VERIFY_OK */
+    float next_probability;
+    uint32_t status;              /* enum ncnn_moe_verify_status */
+    uint32_t row_status;          /* enum ncnn_moe_row_status when status is NCNN_MOE_VERIFY_ROW_ERROR */
+    uint32_t accept_draws;        /* uniforms[0 .. accept_draws) were consumed by the accept tests (:833-837) */
+    uint32_t final_draw_consumed; /* 1 iff uniforms[accept_draws] was consumed by the last token's draw */
+    uint32_t next_is_residual;    /* 1 iff the last token came from the residual distribution (:865-869) */
+} ncnn_moe_verify_result;
+
+enum { NCNN_MOE_MAX_DRAFT_TOKENS = 16 };
+
+/* The verification step of speculative generation (src/engine/session.cpp:776-874 with
+ * candidate_probability :138-148 and sample_residual_distribution :150-202) in one device pass.
+ * The handle's logits buffer holds 2 * draft_count + 1 rows: rows [0, draft_count] are the target
+ * model's logits after the anchor and after each proposed token, rows [draft_count + 1,
+ * 2 * draft_count] the draft model's logits that proposed_token_ids[i] was sampled from.
+ * options: one SamplingOptions for every row (the stop slice is ignored).  uniforms: the next
+ * draft_count + 1 draws of the Session RNG in order; the accept test of position i uses uniforms[i],
+ * the last token's draw uses the one after the last accept test.  accepted_probabilities receives
+ * the probability reported for each accepted token (:839-841, 1.0 for greedy :795).
+ * 1 <= draft_count <= NCNN_MOE_MAX_DRAFT_TOKENS.  All pointers are host memory. */
+int ncnn_moe_hip_sampler_speculative_verify(
+    ncnn_moe_hip_sampler* sampler, uint32_t draft_count,
+    const ncnn_moe_sample_params* options, const int32_t* proposed_token_ids, const float* uniforms,
+    float* accepted_probabilities, ncnn_moe_verify_result* result);
+
+/* The fixed message of a verification status (src/engine/session.cpp:174, :201, :829). */
+const char* ncnn_moe_hip_sampler_verify_status_message(int verify_status);
+
 /* Error text of the last failed call on this handle (Error::message, include/ncnn/moe/result.h:21-25). */
 const char* ncnn_moe_hip_sampler_last_error(const ncnn_moe_hip_sampler* sampler);
 

@@ -2,6 +2,7 @@
 #include "ncnn_moe_hip_sampler.h"
 
 #include "sampler_kernels.h"
+#include "sampler_verify.h"
 
 #include <hip/hip_runtime.h>
 
@@ -51,6 +52,15 @@ struct ncnn_moe_hip_sampler
     int32_t* distribution_ids = nullptr;
     float* distribution_probabilities = nullptr;
     uint32_t* distribution_count = nullptr;
+    // speculative verification: exported distributions of 2 * kMaxDrafts + 1 rows and the small operands
+    int32_t* verify_ids = nullptr;
+    float* verify_probabilities = nullptr;
+    uint32_t* verify_counts = nullptr;
+    int32_t* verify_proposed = nullptr;
+    float* verify_uniforms = nullptr;
+    float* verify_accepted = nullptr;
+    ncnn_moe_verify_result* verify_result = nullptr;
+
     ncnn_moe_sample_params* single_params = nullptr;
     float* single_uniform = nullptr;
     ncnn_moe_sample_result* single_result = nullptr;
@@ -154,6 +164,15 @@ void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, S
         hipLaunchKernelGGL((scan_select_kernel<DTYPE, false, false>), grid, dim3(kScanThreads), 0, stream, a);
 }
 
+// Where a launch writes the rows' filtered distributions (cap entries per row); count == nullptr: nowhere.
+struct DistributionExport
+{
+    int32_t* ids = nullptr;
+    float* probabilities = nullptr;
+    uint32_t* count = nullptr;
+    uint32_t cap = 0;
+};
+
 // Which kernels a call enqueues.  Rows a pass cannot serve are marked pending and taken by the next.
 struct SamplerPasses
 {
@@ -166,8 +185,9 @@ struct SamplerPasses
 int launch_sampler(
     ncnn_moe_hip_sampler* s, const void* logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
     const ncnn_moe_sample_params* params, const float* uniforms, const int32_t* stop_ids,
-    ncnn_moe_sample_result* results, bool want_distribution, SamplerPasses passes, hipStream_t stream)
+    ncnn_moe_sample_result* results, DistributionExport export_to, SamplerPasses passes, hipStream_t stream)
 {
+    const bool want_distribution = export_to.count != nullptr;
     SamplerArgs a;
     std::memset(&a, 0, sizeof(a));
     a.logits = logits;
@@ -193,10 +213,10 @@ int launch_sampler(
     a.sort_stride = s->sort_stride;
     if (want_distribution)
     {
-        a.distribution_ids = s->distribution_ids;
-        a.distribution_probabilities = s->distribution_probabilities;
-        a.distribution_cap = s->max_vocab;
-        a.distribution_count = s->distribution_count;
+        a.distribution_ids = export_to.ids;
+        a.distribution_probabilities = export_to.probabilities;
+        a.distribution_cap = export_to.cap;
+        a.distribution_count = export_to.count;
     }
     const SelectGeometry batch_geometry = select_geometry(dtype, span, rows, false);
     if (batch_geometry.segments > s->max_segments)
@@ -336,6 +356,14 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->distribution_ids, static_cast<size_t>(max_vocab) * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->distribution_probabilities, static_cast<size_t>(max_vocab) * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->distribution_count, sizeof(uint32_t)));
+    constexpr size_t kVerifyRows = 2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1;
+    CREATE_CHECK(hipMalloc(&s->verify_ids, kVerifyRows * kFastTopK * sizeof(int32_t)));
+    CREATE_CHECK(hipMalloc(&s->verify_probabilities, kVerifyRows * kFastTopK * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->verify_counts, kVerifyRows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMalloc(&s->verify_proposed, NCNN_MOE_MAX_DRAFT_TOKENS * sizeof(int32_t)));
+    CREATE_CHECK(hipMalloc(&s->verify_uniforms, (NCNN_MOE_MAX_DRAFT_TOKENS + 1) * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->verify_accepted, NCNN_MOE_MAX_DRAFT_TOKENS * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->verify_result, sizeof(ncnn_moe_verify_result)));
     CREATE_CHECK(hipMalloc(&s->single_params, sizeof(ncnn_moe_sample_params)));
     CREATE_CHECK(hipMalloc(&s->single_uniform, sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->single_result, sizeof(ncnn_moe_sample_result)));
@@ -359,7 +387,9 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
         s->logits, s->params, s->uniforms, s->results, s->stop_ids, s->segment_values, s->segment_indices,
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->sort_keys[0], s->sort_keys[1],
         s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
-        s->distribution_count, s->single_params, s->single_uniform, s->single_result};
+        s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
+        s->verify_probabilities, s->verify_counts, s->verify_proposed, s->verify_uniforms, s->verify_accepted,
+        s->verify_result};
     for (void* buffer : buffers)
     {
         if (buffer != nullptr)
@@ -462,7 +492,7 @@ int ncnn_moe_hip_sampler_sample(
     const int32_t* device_stops = stop_id_count > 0 ? s->stop_ids : nullptr;
     int rc = launch_sampler(
         s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-        s->params, s->uniforms, device_stops, s->results, false, passes, s->stream);
+        s->params, s->uniforms, device_stops, s->results, DistributionExport{}, passes, s->stream);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return rc;
     SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
@@ -480,7 +510,7 @@ int ncnn_moe_hip_sampler_sample(
             retry.full_order = true;
             rc = launch_sampler(
                 s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-                s->params, s->uniforms, device_stops, s->results, false, retry, s->stream);
+                s->params, s->uniforms, device_stops, s->results, DistributionExport{}, retry, s->stream);
             if (rc != NCNN_MOE_SAMPLER_SUCCESS)
                 return rc;
             SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
@@ -512,7 +542,7 @@ int ncnn_moe_hip_sampler_sample_device(
     passes.full_order = may_need_full_order != 0 || s->force_general != 0;
     return launch_sampler(
         s, device_logits, dtype, rows, vocab, row_stride, device_params, device_uniforms, device_stop_ids,
-        device_results, false, passes, static_cast<hipStream_t>(stream));
+        device_results, DistributionExport{}, passes, static_cast<hipStream_t>(stream));
 }
 
 int ncnn_moe_hip_sampler_distribution(
@@ -542,9 +572,14 @@ int ncnn_moe_hip_sampler_distribution(
     const char* row_logits = static_cast<const char*>(s->logits) + static_cast<size_t>(row) * s->logits_stride * element;
     SamplerPasses distribution_passes;
     distribution_passes.full_order = true;
+    DistributionExport single_row_export;
+    single_row_export.ids = s->distribution_ids;
+    single_row_export.probabilities = s->distribution_probabilities;
+    single_row_export.count = s->distribution_count;
+    single_row_export.cap = s->max_vocab;
     const int rc = launch_sampler(
         s, row_logits, s->logits_dtype, 1, s->logits_vocab, s->logits_stride,
-        s->single_params, s->single_uniform, nullptr, s->single_result, true, distribution_passes, s->stream);
+        s->single_params, s->single_uniform, nullptr, s->single_result, single_row_export, distribution_passes, s->stream);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return rc;
     ncnn_moe_sample_result result;
@@ -561,6 +596,95 @@ int ncnn_moe_hip_sampler_distribution(
         SAMPLER_HIP_CHECK(s, hipMemcpy(probabilities, s->distribution_probabilities, static_cast<size_t>(n) * sizeof(float), hipMemcpyDeviceToHost));
     }
     return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_speculative_verify(
+    ncnn_moe_hip_sampler* s, uint32_t draft_count,
+    const ncnn_moe_sample_params* options, const int32_t* proposed_token_ids, const float* uniforms,
+    float* accepted_probabilities, ncnn_moe_verify_result* result)
+{
+    if (s == nullptr || options == nullptr || proposed_token_ids == nullptr || uniforms == nullptr ||
+        accepted_probabilities == nullptr || result == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    if (draft_count == 0 || draft_count > NCNN_MOE_MAX_DRAFT_TOKENS)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "draft_count must be in [1, NCNN_MOE_MAX_DRAFT_TOKENS]");
+    const uint32_t rows = 2u * draft_count + 1u;
+    if (s->logits_rows != rows)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "the logits buffer must hold 2 * draft_count + 1 rows");
+    *result = ncnn_moe_verify_result{0u, -1, 0.0f, NCNN_MOE_VERIFY_OK, NCNN_MOE_ROW_OK, 0u, 0u, 0u};
+    if (s->logits_vocab == 0)
+    {
+        // every row reports "cannot sample empty logits" (src/engine/session.cpp:397-400)
+        result->status = NCNN_MOE_VERIFY_ROW_ERROR;
+        result->row_status = NCNN_MOE_ROW_EMPTY_LOGITS;
+        return NCNN_MOE_SAMPLER_SUCCESS;
+    }
+    ncnn_moe_sample_params row_options = *options;
+    row_options.stop_begin = 0;
+    row_options.stop_count = 0;
+    // the exported distributions hold one Top-K window of at most kFastTopK candidates per row
+    uint32_t effective_k = 0;
+    int status = NCNN_MOE_ROW_OK;
+    if (resolve_row_mode(row_options, s->logits_vocab, kFastTopK, 0, effective_k, status) == kModeGeneral)
+    {
+        result->status = NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW;
+        return NCNN_MOE_SAMPLER_SUCCESS;
+    }
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
+    std::vector<ncnn_moe_sample_params> row_params(rows, row_options);
+    std::vector<float> row_uniforms(rows, 0.0f);
+    row_uniforms[draft_count] = uniforms[draft_count]; // the draw of the row after the last drafted token
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->params, row_params.data(), rows * sizeof(ncnn_moe_sample_params), hipMemcpyHostToDevice, s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->uniforms, row_uniforms.data(), rows * sizeof(float), hipMemcpyHostToDevice, s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_proposed, proposed_token_ids, draft_count * sizeof(int32_t), hipMemcpyHostToDevice, s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_uniforms, uniforms, (draft_count + 1) * sizeof(float), hipMemcpyHostToDevice, s->stream));
+    // the copies above read pageable host memory that lives only until this function returns
+    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+
+    DistributionExport export_to;
+    export_to.ids = s->verify_ids;
+    export_to.probabilities = s->verify_probabilities;
+    export_to.count = s->verify_counts;
+    export_to.cap = kFastTopK;
+    SamplerPasses passes;
+    passes.full_order = true; // rows whose ties overflow the select lists still get their distribution
+    const int rc = launch_sampler(
+        s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
+        s->params, s->uniforms, nullptr, s->results, export_to, passes, s->stream);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return rc;
+    VerifyArgs v;
+    v.draft_count = draft_count;
+    v.temperature = row_options.temperature;
+    v.row_results = s->results;
+    v.distribution_ids = s->verify_ids;
+    v.distribution_probabilities = s->verify_probabilities;
+    v.distribution_count = s->verify_counts;
+    v.distribution_cap = kFastTopK;
+    v.proposed = s->verify_proposed;
+    v.uniforms = s->verify_uniforms;
+    v.accepted_probabilities = s->verify_accepted;
+    v.result = s->verify_result;
+    hipLaunchKernelGGL(speculative_verify_kernel, dim3(1), dim3(kWaveSize), 0, s->stream, v);
+    SAMPLER_HIP_CHECK(s, hipGetLastError());
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(result, s->verify_result, sizeof(*result), hipMemcpyDeviceToHost, s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(accepted_probabilities, s->verify_accepted, draft_count * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+const char* ncnn_moe_hip_sampler_verify_status_message(int verify_status)
+{
+    switch (verify_status)
+    {
+    case NCNN_MOE_VERIFY_OK: return "";
+    case NCNN_MOE_VERIFY_ROW_ERROR: return "a sampled row failed";
+    case NCNN_MOE_VERIFY_ZERO_DRAFT_PROBABILITY: return "sampled draft token has zero probability";
+    case NCNN_MOE_VERIFY_RESIDUAL_EMPTY: return "speculative residual distribution is empty";
+    case NCNN_MOE_VERIFY_RESIDUAL_FAILED: return "speculative residual sampling failed";
+    case NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW: return "speculative verification on the device needs temperature 0 or 1 <= top_k <= 64";
+    default: return "unknown verification status";
+    }
 }
 
 const char* ncnn_moe_hip_sampler_last_error(const ncnn_moe_hip_sampler* s)

@@ -37,7 +37,8 @@ struct SamplerArgs
     uint32_t* sort_indices[2];
     uint64_t sort_stride;
 
-    // optional filtered-distribution output for row 0 of the launch
+    // optional filtered-distribution output: row r writes at most distribution_cap (id, probability)
+    // entries from r * distribution_cap on, and its full kept length to distribution_count[r]
     int32_t* distribution_ids;
     float* distribution_probabilities;
     uint32_t distribution_cap;
@@ -67,8 +68,8 @@ __device__ __forceinline__ void write_error(const SamplerArgs& a, uint32_t row, 
     r.draw_consumed = 0;
     r.flags = flags;
     a.results[row] = r;
-    if (a.distribution_count != nullptr && row == 0)
-        *a.distribution_count = 0;
+    if (a.distribution_count != nullptr)
+        a.distribution_count[row] = 0;
 }
 
 // Marks a row that still has to go through the full-order kernels.
@@ -150,19 +151,20 @@ __device__ __forceinline__ void finish_row_wave(
     const float renormalizer = cumulative;
     const float final_probability = probability / renormalizer;
 
-    if (a.distribution_count != nullptr && row == 0)
+    if (a.distribution_count != nullptr)
     {
+        const size_t first = static_cast<size_t>(row) * a.distribution_cap;
         if ((kept_mask >> lane) & 1ull)
         {
             const int position = lanes_below(kept_mask);
             if (static_cast<uint32_t>(position) < a.distribution_cap)
             {
-                a.distribution_ids[position] = index;
-                a.distribution_probabilities[position] = final_probability;
+                a.distribution_ids[first + position] = index;
+                a.distribution_probabilities[first + position] = final_probability;
             }
         }
         if (lane == 0)
-            *a.distribution_count = static_cast<uint32_t>(kept);
+            a.distribution_count[row] = static_cast<uint32_t>(kept);
     }
 
     int selected = 0;

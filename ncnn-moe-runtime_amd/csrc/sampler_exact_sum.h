@@ -363,16 +363,17 @@ __device__ __forceinline__ void replay_sorted_window(
     const uint32_t kept = nucleus.stopped ? nucleus.stop_index + 1u : candidates;
     sorted.renormalizer = nucleus.sum;
 
-    if (a.distribution_count != nullptr && row == 0 && sorted_indices != nullptr)
+    if (a.distribution_count != nullptr && sorted_indices != nullptr)
     {
+        const size_t first = static_cast<size_t>(row) * a.distribution_cap;
         const uint32_t limit = kept < a.distribution_cap ? kept : a.distribution_cap;
         for (uint32_t i = tid; i < limit; i += kReplayThreads)
         {
-            a.distribution_ids[i] = static_cast<int32_t>(sorted_indices[i]);
-            a.distribution_probabilities[i] = row_term<2>(sorted, i);
+            a.distribution_ids[first + i] = static_cast<int32_t>(sorted_indices[i]);
+            a.distribution_probabilities[first + i] = row_term<2>(sorted, i);
         }
         if (tid == 0)
-            *a.distribution_count = kept;
+            a.distribution_count[row] = kept;
     }
 
     if (kept == 1)

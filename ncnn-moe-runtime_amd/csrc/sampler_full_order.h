@@ -330,13 +330,13 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
             if (any_finite)
             {
                 write_token(a, row, p, token, 1.0f, 1u, 0, flags);
-                if (a.distribution_count != nullptr && row == 0)
+                if (a.distribution_count != nullptr)
                 {
-                    *a.distribution_count = 1;
+                    a.distribution_count[row] = 1;
                     if (a.distribution_cap > 0)
                     {
-                        a.distribution_ids[0] = token;
-                        a.distribution_probabilities[0] = 1.0f;
+                        a.distribution_ids[static_cast<size_t>(row) * a.distribution_cap] = token;
+                        a.distribution_probabilities[static_cast<size_t>(row) * a.distribution_cap] = 1.0f;
                     }
                 }
             }

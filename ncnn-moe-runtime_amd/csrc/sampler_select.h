@@ -109,13 +109,13 @@ __device__ __forceinline__ void finish_ordered_wave(
         if (lane == 0)
         {
             write_token(a, row, p, index, 1.0f, 1u, 0, result_flags);
-            if (a.distribution_count != nullptr && row == 0)
+            if (a.distribution_count != nullptr)
             {
-                *a.distribution_count = 1;
+                a.distribution_count[row] = 1;
                 if (a.distribution_cap > 0)
                 {
-                    a.distribution_ids[0] = index;
-                    a.distribution_probabilities[0] = 1.0f;
+                    a.distribution_ids[static_cast<size_t>(row) * a.distribution_cap] = index;
+                    a.distribution_probabilities[static_cast<size_t>(row) * a.distribution_cap] = 1.0f;
                 }
             }
         }

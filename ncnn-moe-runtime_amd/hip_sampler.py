@@ -27,6 +27,14 @@ ROW_NO_FINITE_LOGIT = 5
 ROW_INVALID_DISTRIBUTION = 6
 ROW_NEEDS_FULL_ORDER = 7
 
+VERIFY_OK = 0
+VERIFY_ROW_ERROR = 1
+VERIFY_ZERO_DRAFT_PROBABILITY = 2
+VERIFY_RESIDUAL_EMPTY = 3
+VERIFY_RESIDUAL_FAILED = 4
+VERIFY_UNSUPPORTED_WINDOW = 5
+MAX_DRAFT_TOKENS = 16
+
 FLAG_HAS_NAN = 1
 FLAG_GENERAL_PATH = 2
 FLAG_FALLBACK = 4
@@ -35,6 +43,9 @@ PARAMS_DTYPE = np.dtype([("temperature", "<f4"), ("top_k", "<u4"), ("top_p", "<f
                          ("min_p", "<f4"), ("stop_begin", "<u4"), ("stop_count", "<u4")])
 RESULT_DTYPE = np.dtype([("token_id", "<i4"), ("probability", "<f4"), ("kept_count", "<u4"),
                          ("status", "u1"), ("is_stop", "u1"), ("draw_consumed", "u1"), ("flags", "u1")])
+VERIFY_RESULT_DTYPE = np.dtype([("accepted", "<u4"), ("next_token_id", "<i4"), ("next_probability", "<f4"),
+                                ("status", "<u4"), ("row_status", "<u4"), ("accept_draws", "<u4"),
+                                ("final_draw_consumed", "<u4"), ("next_is_residual", "<u4")])
 
 EXPORTED_SYMBOLS = [
     "ncnn_moe_hip_sampler_create",
@@ -44,6 +55,8 @@ EXPORTED_SYMBOLS = [
     "ncnn_moe_hip_sampler_sample",
     "ncnn_moe_hip_sampler_sample_device",
     "ncnn_moe_hip_sampler_distribution",
+    "ncnn_moe_hip_sampler_speculative_verify",
+    "ncnn_moe_hip_sampler_verify_status_message",
     "ncnn_moe_hip_sampler_last_error",
     "ncnn_moe_hip_sampler_status_message",
     "ncnn_moe_hip_sampler_device_count",
@@ -81,6 +94,9 @@ def load_library():
         vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp, vp, vp, vp, ctypes.c_int, vp]
     lib.ncnn_moe_hip_sampler_distribution.argtypes = [
         vp, ctypes.c_uint32, vp, ctypes.c_uint32, vp, vp, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32)]
+    lib.ncnn_moe_hip_sampler_speculative_verify.argtypes = [vp, ctypes.c_uint32, vp, vp, vp, vp, vp]
+    lib.ncnn_moe_hip_sampler_verify_status_message.argtypes = [ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_verify_status_message.restype = ctypes.c_char_p
     lib.ncnn_moe_hip_sampler_last_error.argtypes = [vp]
     lib.ncnn_moe_hip_sampler_last_error.restype = ctypes.c_char_p
     lib.ncnn_moe_hip_sampler_status_message.argtypes = [ctypes.c_int]
@@ -96,6 +112,10 @@ def load_library():
 
 def status_message(row_status):
     return load_library().ncnn_moe_hip_sampler_status_message(int(row_status)).decode()
+
+
+def verify_status_message(verify_status):
+    return load_library().ncnn_moe_hip_sampler_verify_status_message(int(verify_status)).decode()
 
 
 def exp2_table():
@@ -200,6 +220,21 @@ class HipSampler:
             ctypes.byref(count), ctypes.byref(status)))
         n = min(count.value, cap)
         return status.value, ids[:n].copy(), probabilities[:n].copy(), count.value
+
+    def speculative_verify(self, proposed_token_ids, uniforms, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
+        """One verification step over the uploaded logits (rows [0, D]: target, rows [D + 1, 2 D]: draft).
+        uniforms: D + 1 canonical draws.  Returns (VERIFY_RESULT_DTYPE record, accepted probabilities[D])."""
+        proposed = np.ascontiguousarray(proposed_token_ids, dtype=np.int32)
+        uniforms = np.ascontiguousarray(uniforms, dtype=np.float32)
+        drafts = proposed.size
+        assert uniforms.shape == (drafts + 1,)
+        options = make_params(1, temperature, top_k, top_p, min_p)
+        accepted = np.zeros(max(drafts, 1), dtype=np.float32)
+        result = np.zeros(1, dtype=VERIFY_RESULT_DTYPE)
+        self._check(self._lib.ncnn_moe_hip_sampler_speculative_verify(
+            self._handle, drafts, options.ctypes.data, proposed.ctypes.data, uniforms.ctypes.data,
+            accepted.ctypes.data, result.ctypes.data))
+        return result[0], accepted[:drafts]
 
     def force_general(self, enabled):
         self._check(self._lib.ncnn_moe_hip_sampler_debug_force_general(self._handle, 1 if enabled else 0))

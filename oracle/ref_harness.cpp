@@ -244,6 +244,64 @@ int ref_sample_rows(
     return 0;
 }
 
+/* candidate_probability, file-static at src/engine/session.cpp:138-148. */
+float ref_candidate_probability(const int32_t* ids, const float* probabilities, size_t count, int32_t token_id)
+{
+    std::vector<SamplingCandidate> candidates(count);
+    for (size_t i = 0; i < count; ++i)
+    {
+        candidates[i].token_id = ids[i];
+        candidates[i].probability = probabilities[i];
+    }
+    return candidate_probability(candidates, token_id);
+}
+
+/*
+ * sample_residual_distribution, file-static at src/engine/session.cpp:150-202, driven by a
+ * std::mt19937_64 seeded with `seed` and advanced by `discard` draws first.  *draws receives the
+ * number of 64-bit outputs the call consumed.
+ */
+int ref_sample_residual_distribution(
+    const int32_t* target_ids, const float* target_probabilities, size_t target_count,
+    const int32_t* draft_ids, const float* draft_probabilities, size_t draft_count,
+    size_t vocab, uint64_t seed, uint64_t discard,
+    int32_t* token_id, float* probability, uint64_t* draws,
+    char* message, size_t message_cap)
+{
+    std::vector<SamplingCandidate> target(target_count), draft(draft_count);
+    for (size_t i = 0; i < target_count; ++i)
+    {
+        target[i].token_id = target_ids[i];
+        target[i].probability = target_probabilities[i];
+    }
+    for (size_t i = 0; i < draft_count; ++i)
+    {
+        draft[i].token_id = draft_ids[i];
+        draft[i].probability = draft_probabilities[i];
+    }
+    std::mt19937_64 generator(seed);
+    generator.discard(discard);
+    std::mt19937_64 shadow = generator;
+    *token_id = -1;
+    *probability = 0.0f;
+    auto sampled = sample_residual_distribution(target, draft, vocab, generator);
+    uint64_t consumed = 0;
+    while (!(shadow == generator) && consumed < 16)
+    {
+        shadow.discard(1);
+        ++consumed;
+    }
+    *draws = consumed;
+    if (!sampled)
+    {
+        copy_message(sampled.error().message, message, message_cap);
+        return 1 + static_cast<int>(sampled.error().code);
+    }
+    *token_id = sampled.value().token_id;
+    *probability = sampled.value().probability;
+    return 0;
+}
+
 float ref_bfloat16_to_float(uint16_t value)
 {
     return bfloat16_to_float(value);

@@ -17,6 +17,13 @@
  *                                      the reference's file-static function itself (where it builds).
  *   oracle_sample (draw)               inverse-CDF definition; the reference's Session::sample in
  *                                      RNG lock-step (where it builds); committed golden vectors.
+ *   oracle_candidate_probability,      the reference's file-static functions themselves (where it builds):
+ *   oracle_sample_residual_distribution  random distributions with a real mt19937_64 in lock-step; brute force
+ *                                      in fp64 on small cases; committed golden vectors.
+ *   oracle_speculative_verify          the accept loop is inline in the reference's generate(): pinned by the
+ *                                      two functions above plus the identity that fixes the algorithm (the
+ *                                      emitted token follows the target distribution whatever the draft is),
+ *                                      integrated over a grid of uniforms; greedy reduces to arg-max equality.
  *   oracle_rng_uniform                 2000-draw lock-step against the reference Session; golden draws.
  *   oracle_*_bfloat16                  exhaustive 65536-value round trip and round-to-nearest-even
  *                                      checks against the definition.
@@ -226,6 +233,55 @@ int sample_row(
     return ORACLE_OK;
 }
 
+/* src/engine/session.cpp:138-148 */
+float candidate_probability(const std::vector<Candidate>& candidates, int32_t token_id)
+{
+    for (const Candidate& candidate : candidates)
+    {
+        if (candidate.token_id == token_id)
+            return candidate.probability;
+    }
+    return 0.0f;
+}
+
+/* src/engine/session.cpp:150-202.  The reference draws uniform_real_distribution<float>(0, normalizer),
+ * which libstdc++ evaluates as canonical * (normalizer - 0) + 0 in fp32. */
+int sample_residual_distribution(
+    const std::vector<Candidate>& target, const std::vector<Candidate>& draft, size_t vocab,
+    float canonical_uniform, int32_t& token_id, float& probability)
+{
+    std::vector<float> residual(vocab, 0.0f);
+    for (const Candidate& candidate : target)
+        residual[candidate.token_id] = candidate.probability;
+    for (const Candidate& candidate : draft)
+        residual[candidate.token_id] = std::max(0.0f, residual[candidate.token_id] - candidate.probability);
+    const float normalizer = std::accumulate(residual.begin(), residual.end(), 0.0f);
+    if (!std::isfinite(normalizer) || normalizer <= 0.0f)
+        return ORACLE_VERIFY_RESIDUAL_EMPTY;
+    const float sample_value = canonical_uniform * (normalizer - 0.0f) + 0.0f;
+    float cumulative = 0.0f;
+    for (size_t id = 0; id < residual.size(); ++id)
+    {
+        cumulative += residual[id];
+        if (sample_value < cumulative)
+        {
+            token_id = static_cast<int32_t>(id);
+            probability = residual[id] / normalizer;
+            return ORACLE_VERIFY_OK;
+        }
+    }
+    for (size_t id = residual.size(); id != 0; --id)
+    {
+        if (residual[id - 1] > 0.0f)
+        {
+            token_id = static_cast<int32_t>(id - 1);
+            probability = residual[id - 1] / normalizer;
+            return ORACLE_VERIFY_OK;
+        }
+    }
+    return ORACLE_VERIFY_RESIDUAL_FAILED;
+}
+
 /* Table-driven expf: 2^(k/32) table, degree-3 polynomial evaluated in double, one final rounding. */
 struct Exp2fTable
 {
@@ -378,6 +434,128 @@ int oracle_sample_batch(
     for (std::thread& worker : pool)
         worker.join();
     return 0;
+}
+
+float oracle_candidate_probability(const int32_t* ids, const float* probabilities, size_t count, int32_t token_id)
+{
+    std::vector<Candidate> candidates(count);
+    for (size_t i = 0; i < count; ++i)
+        candidates[i] = Candidate{ids[i], probabilities[i]};
+    return candidate_probability(candidates, token_id);
+}
+
+int oracle_sample_residual_distribution(
+    const int32_t* target_ids, const float* target_probabilities, size_t target_count,
+    const int32_t* draft_ids, const float* draft_probabilities, size_t draft_count,
+    size_t vocab, float canonical_uniform, int32_t* token_id, float* probability)
+{
+    std::vector<Candidate> target(target_count), draft(draft_count);
+    for (size_t i = 0; i < target_count; ++i)
+        target[i] = Candidate{target_ids[i], target_probabilities[i]};
+    for (size_t i = 0; i < draft_count; ++i)
+        draft[i] = Candidate{draft_ids[i], draft_probabilities[i]};
+    *token_id = -1;
+    *probability = 0.0f;
+    return sample_residual_distribution(target, draft, vocab, canonical_uniform, *token_id, *probability);
+}
+
+/* src/engine/session.cpp:776-874 */
+int oracle_speculative_verify(
+    const float* target_logits, const float* draft_logits, size_t vocab, uint32_t draft_count,
+    const oracle_sampling_options* options, const int32_t* proposed_token_ids, const float* uniforms,
+    float* accepted_probabilities, oracle_verify_result* result)
+{
+    oracle_verify_result r;
+    std::memset(&r, 0, sizeof(r));
+    r.next_token_id = -1;
+    auto fail_row = [&](int row_status) {
+        r.status = ORACLE_VERIFY_ROW_ERROR;
+        r.row_status = static_cast<uint32_t>(row_status);
+        *result = r;
+        return static_cast<int>(r.status);
+    };
+    std::vector<Candidate> rejected_target, rejected_draft;
+    uint32_t accepted = 0;
+    while (accepted < draft_count)
+    {
+        const float* target_row = target_logits + static_cast<size_t>(accepted) * vocab;
+        const float* draft_row = draft_logits + static_cast<size_t>(accepted) * vocab;
+        if (options->temperature == 0.0f)
+        {
+            oracle_row_result target_token;
+            if (sample_row(target_row, vocab, *options, 0.0f, target_token) != ORACLE_OK)
+            {
+                r.accepted = accepted;
+                return fail_row(target_token.status);
+            }
+            if (target_token.token_id != proposed_token_ids[accepted])
+                break;
+            accepted_probabilities[accepted] = 1.0f;
+        }
+        else
+        {
+            /* sampling_distribution is reached only with options that an earlier sample() call of the
+             * generation loop has validated; the oracle reports unvalidated ones as the row's error */
+            const int valid = vocab == 0 ? ORACLE_EMPTY_LOGITS : oracle_validate_sampling_options(options);
+            std::vector<Candidate> target_distribution, draft_distribution;
+            const int target_status = valid != ORACLE_OK ? valid
+                : sampling_distribution(target_row, vocab, *options, target_distribution, nullptr);
+            const int draft_status = valid != ORACLE_OK ? valid
+                : sampling_distribution(draft_row, vocab, *options, draft_distribution, nullptr);
+            if (target_status != ORACLE_OK || draft_status != ORACLE_OK)
+            {
+                r.accepted = accepted;
+                return fail_row(target_status != ORACLE_OK ? target_status : draft_status);
+            }
+            const int32_t token_id = proposed_token_ids[accepted];
+            const float target_probability = candidate_probability(target_distribution, token_id);
+            const float draft_probability = candidate_probability(draft_distribution, token_id);
+            if (draft_probability <= 0.0f)
+            {
+                r.accepted = accepted;
+                r.status = ORACLE_VERIFY_ZERO_DRAFT_PROBABILITY;
+                *result = r;
+                return static_cast<int>(r.status);
+            }
+            const float acceptance_probability = std::min(1.0f, target_probability / draft_probability);
+            const float uniform = uniforms[r.accept_draws++];
+            if (uniform >= acceptance_probability)
+            {
+                rejected_target = std::move(target_distribution);
+                rejected_draft = std::move(draft_distribution);
+                break;
+            }
+            accepted_probabilities[accepted] = target_probability;
+        }
+        ++accepted;
+    }
+    r.accepted = accepted;
+    if (accepted < draft_count && options->temperature > 0.0f)
+    {
+        r.next_is_residual = 1;
+        int32_t token_id = -1;
+        float probability = 0.0f;
+        const int status = sample_residual_distribution(
+            rejected_target, rejected_draft, vocab, uniforms[r.accept_draws], token_id, probability);
+        r.status = static_cast<uint32_t>(status);
+        /* the reference draws before the walk: the draw is consumed unless the distribution was empty */
+        r.final_draw_consumed = status == ORACLE_VERIFY_RESIDUAL_EMPTY ? 0u : 1u;
+        if (status == ORACLE_VERIFY_OK)
+        {
+            r.next_token_id = token_id;
+            r.next_probability = probability;
+        }
+        *result = r;
+        return status;
+    }
+    oracle_row_result next;
+    if (sample_row(target_logits + static_cast<size_t>(accepted) * vocab, vocab, *options, uniforms[r.accept_draws], next) != ORACLE_OK)
+        return fail_row(next.status);
+    r.next_token_id = next.token_id;
+    r.next_probability = next.probability;
+    r.final_draw_consumed = next.draw_consumed;
+    *result = r;
+    return ORACLE_VERIFY_OK;
 }
 
 /* src/kernels/cpu_ops.cpp:26-32 */

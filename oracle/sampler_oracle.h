@@ -92,6 +92,46 @@ int oracle_sample_batch(
     const int32_t* stop_ids,
     oracle_row_result* results, int threads);
 
+/* Speculative verification.  Statuses beyond the row statuses of the accept loop. */
+enum oracle_verify_status
+{
+    ORACLE_VERIFY_OK = 0,
+    ORACLE_VERIFY_ROW_ERROR = 1,              /* row_status holds the failing row's oracle_status */
+    ORACLE_VERIFY_ZERO_DRAFT_PROBABILITY = 2, /* "sampled draft token has zero probability" */
+    ORACLE_VERIFY_RESIDUAL_EMPTY = 3,         /* "speculative residual distribution is empty" */
+    ORACLE_VERIFY_RESIDUAL_FAILED = 4         /* "speculative residual sampling failed" */
+};
+
+typedef struct oracle_verify_result
+{
+    uint32_t accepted;
+    int32_t next_token_id;
+    float next_probability;
+    uint32_t status;
+    uint32_t row_status;
+    uint32_t accept_draws;
+    uint32_t final_draw_consumed;
+    uint32_t next_is_residual;
+} oracle_verify_result;
+
+/* src/engine/session.cpp:138-148 */
+float oracle_candidate_probability(const int32_t* ids, const float* probabilities, size_t count, int32_t token_id);
+
+/* src/engine/session.cpp:150-202 with the canonical draw in [0, 1) supplied by the caller
+ * (uniform_real_distribution<float>(0, normalizer) returns canonical * normalizer). */
+int oracle_sample_residual_distribution(
+    const int32_t* target_ids, const float* target_probabilities, size_t target_count,
+    const int32_t* draft_ids, const float* draft_probabilities, size_t draft_count,
+    size_t vocab, float canonical_uniform, int32_t* token_id, float* probability);
+
+/* src/engine/session.cpp:776-874: the accept loop over draft_count proposed tokens and the token
+ * that follows.  target_logits holds draft_count + 1 rows, draft_logits draft_count rows, uniforms
+ * the next draft_count + 1 canonical draws of the Session RNG. */
+int oracle_speculative_verify(
+    const float* target_logits, const float* draft_logits, size_t vocab, uint32_t draft_count,
+    const oracle_sampling_options* options, const int32_t* proposed_token_ids, const float* uniforms,
+    float* accepted_probabilities, oracle_verify_result* result);
+
 /* src/kernels/cpu_ops.cpp:26-40 */
 float oracle_bfloat16_to_float(uint16_t value);
 uint16_t oracle_float_to_bfloat16(float value);

@@ -37,6 +37,15 @@ class SamplingOptions(ctypes.Structure):
 ROW_PARAMS_DTYPE = np.dtype([("temperature", "<f4"), ("top_k", "<u4"), ("top_p", "<f4"),
                              ("min_p", "<f4"), ("stop_begin", "<u4"), ("stop_count", "<u4")])
 
+VERIFY_RESULT_DTYPE = np.dtype([("accepted", "<u4"), ("next_token_id", "<i4"), ("next_probability", "<f4"),
+                                ("status", "<u4"), ("row_status", "<u4"), ("accept_draws", "<u4"),
+                                ("final_draw_consumed", "<u4"), ("next_is_residual", "<u4")])
+VERIFY_MESSAGES = {
+    2: "sampled draft token has zero probability",
+    3: "speculative residual distribution is empty",
+    4: "speculative residual sampling failed",
+}
+
 ORACLE_RESULT_DTYPE = np.dtype([("token_id", "<i4"), ("probability", "<f4"), ("kept_count", "<u4"),
                                 ("status", "u1"), ("is_stop", "u1"), ("draw_consumed", "u1"),
                                 ("has_nan", "u1"), ("cdf_gap", "<f4"), ("top_p_gap", "<f4")])
@@ -68,6 +77,14 @@ def oracle():
     lib.oracle_sample_batch.argtypes = [
         ctypes.c_void_p, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64,
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+    lib.oracle_candidate_probability.restype = ctypes.c_float
+    lib.oracle_candidate_probability.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32]
+    lib.oracle_sample_residual_distribution.argtypes = [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+        ctypes.c_size_t, ctypes.c_float, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_float)]
+    lib.oracle_speculative_verify.argtypes = [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32, ctypes.POINTER(SamplingOptions),
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.oracle_bfloat16_to_float.restype = ctypes.c_float
     lib.oracle_bfloat16_to_float.argtypes = [ctypes.c_uint16]
     lib.oracle_float_to_bfloat16.restype = ctypes.c_uint16
@@ -132,6 +149,45 @@ def oracle_sample_batch(logits, params, uniforms, stop_ids=None, threads=1, voca
     return results
 
 
+def oracle_candidate_probability(ids, probabilities, token_id):
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    probabilities = np.ascontiguousarray(probabilities, dtype=np.float32)
+    return oracle().oracle_candidate_probability(ids.ctypes.data, probabilities.ctypes.data, ids.size, int(token_id))
+
+
+def oracle_sample_residual(target_ids, target_probabilities, draft_ids, draft_probabilities, vocab, canonical_uniform):
+    """Returns (status, token_id, probability)."""
+    target_ids = np.ascontiguousarray(target_ids, dtype=np.int32)
+    target_probabilities = np.ascontiguousarray(target_probabilities, dtype=np.float32)
+    draft_ids = np.ascontiguousarray(draft_ids, dtype=np.int32)
+    draft_probabilities = np.ascontiguousarray(draft_probabilities, dtype=np.float32)
+    token = ctypes.c_int32(-1)
+    probability = ctypes.c_float(0.0)
+    status = oracle().oracle_sample_residual_distribution(
+        target_ids.ctypes.data, target_probabilities.ctypes.data, target_ids.size,
+        draft_ids.ctypes.data, draft_probabilities.ctypes.data, draft_ids.size,
+        vocab, ctypes.c_float(canonical_uniform), ctypes.byref(token), ctypes.byref(probability))
+    return status, token.value, probability.value
+
+
+def oracle_speculative_verify(target_logits, draft_logits, proposed_token_ids, uniforms,
+                              temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
+    """target_logits [D + 1, V], draft_logits [D, V] fp32.  Returns (VERIFY_RESULT_DTYPE record, accepted[D])."""
+    target_logits = np.ascontiguousarray(target_logits, dtype=np.float32)
+    draft_logits = np.ascontiguousarray(draft_logits, dtype=np.float32)
+    proposed = np.ascontiguousarray(proposed_token_ids, dtype=np.int32)
+    uniforms = np.ascontiguousarray(uniforms, dtype=np.float32)
+    drafts = proposed.size
+    assert target_logits.shape[0] == drafts + 1 and draft_logits.shape[0] == drafts and uniforms.size == drafts + 1
+    options = SamplingOptions(temperature, top_k, top_p, min_p)
+    accepted = np.zeros(max(drafts, 1), dtype=np.float32)
+    result = np.zeros(1, dtype=VERIFY_RESULT_DTYPE)
+    oracle().oracle_speculative_verify(
+        target_logits.ctypes.data, draft_logits.ctypes.data, target_logits.shape[1], drafts,
+        ctypes.byref(options), proposed.ctypes.data, uniforms.ctypes.data, accepted.ctypes.data, result.ctypes.data)
+    return result[0], accepted[:drafts]
+
+
 def expf_libm(values):
     values = np.ascontiguousarray(values, dtype=np.float32)
     out = np.empty_like(values)
@@ -191,6 +247,12 @@ def reference():
         ctypes.POINTER(ctypes.c_size_t), ctypes.c_char_p, ctypes.c_size_t]
     lib.ref_sample_rows.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_uint32, ctypes.c_uint32,
                                                             ctypes.c_uint64] + [ctypes.c_void_p] * 11 + [ctypes.c_int]
+    lib.ref_candidate_probability.restype = ctypes.c_float
+    lib.ref_candidate_probability.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32]
+    lib.ref_sample_residual_distribution.argtypes = [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+        ctypes.c_size_t, ctypes.c_uint64, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int32),
+        ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_uint64), ctypes.c_char_p, ctypes.c_size_t]
     lib.ref_bfloat16_to_float.restype = ctypes.c_float
     lib.ref_bfloat16_to_float.argtypes = [ctypes.c_uint16]
     lib.ref_float_to_bfloat16.restype = ctypes.c_uint16
@@ -241,3 +303,27 @@ def reference_distribution(logits, temperature=1.0, top_k=0, top_p=1.0, min_p=0.
         logits.ctypes.data, logits.size, temperature, top_k, top_p, min_p,
         ids.ctypes.data, probs.ctypes.data, cap, ctypes.byref(count), message, 256)
     return rc, ids[:count.value].copy(), probs[:count.value].copy(), message.value.decode()
+
+
+def reference_sample_residual(target_ids, target_probabilities, draft_ids, draft_probabilities, vocab, seed, discard=0):
+    """The reference's own sample_residual_distribution with mt19937_64(seed) advanced by `discard`.
+    Returns (rc, token_id, probability, draws consumed, message)."""
+    target_ids = np.ascontiguousarray(target_ids, dtype=np.int32)
+    target_probabilities = np.ascontiguousarray(target_probabilities, dtype=np.float32)
+    draft_ids = np.ascontiguousarray(draft_ids, dtype=np.int32)
+    draft_probabilities = np.ascontiguousarray(draft_probabilities, dtype=np.float32)
+    token = ctypes.c_int32(-1)
+    probability = ctypes.c_float(0.0)
+    draws = ctypes.c_uint64(0)
+    message = ctypes.create_string_buffer(256)
+    rc = reference().ref_sample_residual_distribution(
+        target_ids.ctypes.data, target_probabilities.ctypes.data, target_ids.size,
+        draft_ids.ctypes.data, draft_probabilities.ctypes.data, draft_ids.size,
+        vocab, seed, discard, ctypes.byref(token), ctypes.byref(probability), ctypes.byref(draws), message, 256)
+    return rc, token.value, probability.value, draws.value, message.value.decode()
+
+
+def reference_candidate_probability(ids, probabilities, token_id):
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    probabilities = np.ascontiguousarray(probabilities, dtype=np.float32)
+    return reference().ref_candidate_probability(ids.ctypes.data, probabilities.ctypes.data, ids.size, int(token_id))
