@@ -209,6 +209,79 @@ Result<std::vector<TokenProbability>> HipSampler::distribution(std::span<const f
     return candidates;
 }
 
+Result<SpeculativeVerification> HipSampler::verify_speculative(
+    std::span<const std::span<const float>> target_logits,
+    std::span<const std::span<const float>> draft_logits,
+    std::span<const int32_t> proposed_token_ids,
+    const SamplingOptions& options,
+    std::span<const float> uniforms,
+    uint32_t& draws_consumed)
+{
+    draws_consumed = 0;
+    const size_t drafts = proposed_token_ids.size();
+    if (drafts == 0 || drafts > NCNN_MOE_MAX_DRAFT_TOKENS)
+        return invalid_argument("speculative verification takes 1 to 16 proposed tokens");
+    if (target_logits.size() != drafts + 1 || draft_logits.size() != drafts || uniforms.size() != drafts + 1)
+        return invalid_argument("speculative verification operands differ in length");
+    const size_t rows = 2 * drafts + 1;
+    if (rows > impl_->max_rows)
+        return invalid_argument("speculative verification exceeds the sampler's max_rows");
+    const size_t vocab = target_logits[0].size();
+    if (vocab == 0)
+        return invalid_argument("cannot sample empty logits");
+    if (vocab > impl_->max_vocab)
+        return invalid_argument("logits exceed the sampler's max_vocab");
+    for (const std::span<const float>& row : target_logits)
+    {
+        if (row.size() != vocab)
+            return invalid_argument("speculative verification rows differ in length");
+    }
+    for (const std::span<const float>& row : draft_logits)
+    {
+        if (row.size() != vocab)
+            return invalid_argument("speculative verification rows differ in length");
+    }
+
+    const std::lock_guard<std::mutex> lock(mutex_);
+    Impl& impl = *impl_;
+    impl.staging.resize(rows * vocab);
+    for (size_t row = 0; row <= drafts; ++row)
+        std::copy(target_logits[row].begin(), target_logits[row].end(), impl.staging.begin() + row * vocab);
+    for (size_t row = 0; row < drafts; ++row)
+        std::copy(draft_logits[row].begin(), draft_logits[row].end(), impl.staging.begin() + (drafts + 1 + row) * vocab);
+    int rc = ncnn_moe_hip_sampler_upload_logits(
+        impl.handle, impl.staging.data(), NCNN_MOE_LOGITS_F32, static_cast<uint32_t>(rows), static_cast<uint32_t>(vocab), vocab);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return error_of_call(rc, impl.handle);
+    const ncnn_moe_sample_params p{options.temperature, options.top_k, options.top_p, options.min_p, 0, 0};
+    std::vector<float> accepted_probabilities(drafts, 0.0f);
+    ncnn_moe_verify_result verified{};
+    rc = ncnn_moe_hip_sampler_speculative_verify(
+        impl.handle, static_cast<uint32_t>(drafts), &p, proposed_token_ids.data(), uniforms.data(),
+        accepted_probabilities.data(), &verified);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return error_of_call(rc, impl.handle);
+    draws_consumed = verified.accept_draws + verified.final_draw_consumed;
+    switch (verified.status)
+    {
+    case NCNN_MOE_VERIFY_OK:
+        break;
+    case NCNN_MOE_VERIFY_ROW_ERROR:
+        return error_of_row_status(static_cast<int>(verified.row_status));
+    case NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW:
+        return Error{ErrorCode::InvalidArgument, ncnn_moe_hip_sampler_verify_status_message(static_cast<int>(verified.status))};
+    default: // the reference reports these three as InternalError (src/engine/session.cpp:172-175, :199-201, :826-830)
+        return Error{ErrorCode::InternalError, ncnn_moe_hip_sampler_verify_status_message(static_cast<int>(verified.status))};
+    }
+    SpeculativeVerification out;
+    out.accepted.reserve(verified.accepted);
+    for (uint32_t i = 0; i < verified.accepted; ++i)
+        out.accepted.push_back(SampledToken{proposed_token_ids[i], accepted_probabilities[i]});
+    out.next = SampledToken{verified.next_token_id, verified.next_probability};
+    out.next_from_residual = verified.next_is_residual != 0;
+    return out;
+}
+
 SamplingSession::SamplingSession(HipSamplerPtr sampler, const SamplingSessionOptions& options)
     : sampler_(std::move(sampler)), random_generator_(options.sampling_seed)
 {
@@ -233,6 +306,33 @@ Result<SampledToken> SamplingSession::sample(const LogitsOutput& logits, const S
     if (draw_consumed[0])
         random_generator_ = advanced;
     return results[0].value().token;
+}
+
+Result<SpeculativeVerification> SamplingSession::verify_speculative(
+    std::span<const LogitsOutput> target_logits, std::span<const LogitsOutput> draft_logits,
+    std::span<const int32_t> proposed_token_ids, const SamplingOptions& options)
+{
+    const std::lock_guard<std::mutex> lock(mutex_);
+    if (!sampler_)
+        return Error{ErrorCode::InternalError, "hip sampler is unavailable (no GPU, or create() failed)"};
+    std::vector<std::span<const float>> target_rows, draft_rows;
+    for (const LogitsOutput& row : target_logits)
+        target_rows.emplace_back(row.values);
+    for (const LogitsOutput& row : draft_logits)
+        draft_rows.emplace_back(row.values);
+    // the draws the loop could consume, in the generator's order; only the consumed ones are committed
+    std::mt19937_64 shadow = random_generator_;
+    std::vector<float> uniforms(proposed_token_ids.size() + 1);
+    for (float& uniform : uniforms)
+    {
+        std::mt19937_64 advanced;
+        uniform = peek_uniform(shadow, advanced);
+        shadow = advanced;
+    }
+    uint32_t draws_consumed = 0;
+    auto verified = sampler_->verify_speculative(target_rows, draft_rows, proposed_token_ids, options, uniforms, draws_consumed);
+    random_generator_.discard(draws_consumed); // one 64-bit output per uniform_real_distribution<float> draw
+    return verified;
 }
 
 std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample(

@@ -110,6 +110,14 @@ struct TokenProbability
     float probability = 0.0f;
 };
 
+// Outcome of one verification step of speculative generation (src/engine/session.cpp:776-874).
+struct SpeculativeVerification
+{
+    std::vector<SampledToken> accepted; // the proposed tokens that stand, each with its reported probability
+    SampledToken next;                  // the token emitted after them (residual draw, or the target's own sample)
+    bool next_from_residual = false;
+};
+
 class HipSampler
 {
 public:
@@ -135,6 +143,18 @@ public:
     // sampling_distribution for one row.
     Result<std::vector<TokenProbability>> distribution(std::span<const float> logits, const SamplingOptions& options);
 
+    // The accept loop and the following token of src/engine/session.cpp:776-874 in one device pass.
+    // target_logits: proposed.size() + 1 rows (after the anchor and after each proposed token);
+    // draft_logits: the rows the proposed tokens were sampled from; uniforms: the Session RNG's next
+    // proposed.size() + 1 draws.  draws_consumed receives how many of them the step used, in order.
+    Result<SpeculativeVerification> verify_speculative(
+        std::span<const std::span<const float>> target_logits,
+        std::span<const std::span<const float>> draft_logits,
+        std::span<const int32_t> proposed_token_ids,
+        const SamplingOptions& options,
+        std::span<const float> uniforms,
+        uint32_t& draws_consumed);
+
 private:
     HipSampler();
     struct Impl;
@@ -156,6 +176,12 @@ public:
 
     // Session::sample, include/ncnn/moe/session.h:326.
     [[nodiscard]] Result<SampledToken> sample(const LogitsOutput& logits, const SamplingOptions& options = {});
+
+    // The verification step of Session::generate's speculative loop (src/engine/session.cpp:776-874):
+    // draws from this Session's generator exactly as that loop would.
+    [[nodiscard]] Result<SpeculativeVerification> verify_speculative(
+        std::span<const LogitsOutput> target_logits, std::span<const LogitsOutput> draft_logits,
+        std::span<const int32_t> proposed_token_ids, const SamplingOptions& options = {});
 
 private:
     friend class SessionBatchSampler;

@@ -309,6 +309,109 @@ static void test_batch_rejects_bad_requests(const HipSamplerPtr& sampler)
     check(SessionBatchSampler::sample(sampler, {}).empty());
 }
 
+// The verification step of speculative generation (src/engine/session.cpp:776-874): what is accepted,
+// what follows, which error text comes back, and that the Session's generator advances by exactly the
+// draws the step consumed.
+static void test_speculative_verification(const HipSamplerPtr& sampler)
+{
+    const std::vector<float> ramp = {0.0f, 1.0f, 2.0f, 3.0f, 2.5f, -1.0f};
+    // greedy: the first two proposals are the target's own choices, the third is not
+    {
+        SamplingSession session(sampler, SamplingSessionOptions{7});
+        std::vector<LogitsOutput> target = {logits_of(ramp), logits_of({5, 0, 0, 0, 0, 0}), logits_of({0, 0, 9, 0, 0, 0}),
+                                            logits_of({0, 7, 0, 0, 0, 0})};
+        std::vector<LogitsOutput> draft = {logits_of(ramp), logits_of(ramp), logits_of(ramp)};
+        const std::vector<int32_t> proposed = {3, 0, 4};
+        SamplingOptions greedy;
+        greedy.temperature = 0.0f;
+        auto verified = session.verify_speculative(target, draft, proposed, greedy);
+        check(static_cast<bool>(verified));
+        check(verified.value().accepted.size() == 2);
+        check(verified.value().accepted[0].token_id == 3 && verified.value().accepted[0].probability == 1.0f);
+        check(verified.value().accepted[1].token_id == 0);
+        check(verified.value().next.token_id == 2 && verified.value().next.probability == 1.0f);
+        check(!verified.value().next_from_residual);
+        // no draw was consumed: the next sampled token is decided by the generator's first output
+        std::mt19937_64 shadow(7);
+        const float u = std::uniform_real_distribution<float>(0.0f, 1.0f)(shadow);
+        SamplingOptions two;
+        two.top_k = 2;
+        auto sampled = session.sample(logits_of({0, 5, 5, -1}), two);
+        check(static_cast<bool>(sampled));
+        check(sampled.value().token_id == (u < 0.5f ? 1 : 2));
+    }
+    // identical target and draft distributions: every proposal stands (ratio 1), D accept draws and
+    // one draw for the row behind the last proposal
+    {
+        SamplingSession session(sampler, SamplingSessionOptions{11});
+        std::vector<LogitsOutput> target = {logits_of(ramp), logits_of(ramp), logits_of({0, 5, 5, -1, -1, -1})};
+        std::vector<LogitsOutput> draft = {logits_of(ramp), logits_of(ramp)};
+        SamplingOptions options;
+        options.top_k = 4;
+        auto verified = session.verify_speculative(target, draft, std::vector<int32_t>{2, 4}, options);
+        check(static_cast<bool>(verified));
+        check(verified.value().accepted.size() == 2 && !verified.value().next_from_residual);
+        std::mt19937_64 shadow(11);
+        std::uniform_real_distribution<float> canonical(0.0f, 1.0f);
+        canonical(shadow);
+        canonical(shadow);
+        const float u_final = canonical(shadow);
+        check(verified.value().next.token_id == (u_final < 0.5f ? 1 : 2));
+        const float u_next = canonical(shadow);
+        SamplingOptions two;
+        two.top_k = 2;
+        auto sampled = session.sample(logits_of({0, 5, 5, -1}), two);
+        check(sampled.value().token_id == (u_next < 0.5f ? 1 : 2));
+    }
+    // a draft that is sure of a token the target rates low: rejected, the next token comes from the residual
+    {
+        std::vector<float> sure = ramp;
+        sure[5] = 40.0f;
+        int rejected = 0;
+        for (uint64_t seed = 0; seed < 8; ++seed)
+        {
+            SamplingSession session(sampler, SamplingSessionOptions{seed});
+            std::vector<LogitsOutput> target = {logits_of(ramp), logits_of(ramp)};
+            std::vector<LogitsOutput> draft = {logits_of(sure)};
+            SamplingOptions options;
+            options.top_k = 6;
+            auto verified = session.verify_speculative(target, draft, std::vector<int32_t>{5}, options);
+            check(static_cast<bool>(verified));
+            if (verified.value().accepted.empty())
+            {
+                ++rejected;
+                check(verified.value().next_from_residual);
+                check(verified.value().next.token_id != 5 && verified.value().next.probability > 0.0f);
+            }
+        }
+        check(rejected >= 7); // the target gives token 5 about 0.8 % of the mass
+    }
+    // error text
+    {
+        SamplingSession session(sampler);
+        std::vector<LogitsOutput> target = {logits_of(ramp), logits_of(ramp)};
+        std::vector<LogitsOutput> draft = {logits_of(ramp)};
+        SamplingOptions options;
+        options.top_k = 2;
+        auto outside = session.verify_speculative(target, draft, std::vector<int32_t>{0}, options);
+        check(!outside && outside.error().code == ErrorCode::InternalError);
+        check(outside.error().message == "sampled draft token has zero probability");
+        // no Top-K window over a vocabulary longer than 64: not served by this entry
+        std::vector<LogitsOutput> long_target = {logits_of(std::vector<float>(100, 0.5f)), logits_of(std::vector<float>(100, 0.5f))};
+        std::vector<LogitsOutput> long_draft = {logits_of(std::vector<float>(100, 0.5f))};
+        auto window = session.verify_speculative(long_target, long_draft, std::vector<int32_t>{3}, SamplingOptions{});
+        check(!window && window.error().code == ErrorCode::InvalidArgument);
+        // the same options over a short vocabulary are a window of its whole length
+        auto whole = session.verify_speculative(target, draft, std::vector<int32_t>{3}, SamplingOptions{});
+        check(static_cast<bool>(whole));
+        std::vector<LogitsOutput> broken = {logits_of(std::vector<float>(6, -std::numeric_limits<float>::infinity())), logits_of(ramp)};
+        auto no_finite = session.verify_speculative(broken, draft, std::vector<int32_t>{3}, options);
+        check(!no_finite && no_finite.error().message == "sampling requires at least one finite logit");
+        auto lengths = session.verify_speculative(target, draft, std::vector<int32_t>{3, 3}, options);
+        check(!lengths && lengths.error().code == ErrorCode::InvalidArgument);
+    }
+}
+
 int main(int argc, char** argv)
 {
     const bool host_only = argc > 1 && std::strcmp(argv[1], "--host") == 0;
@@ -334,6 +437,7 @@ int main(int argc, char** argv)
         test_distribution_known_answers(sampler);
         test_batch_equals_serial(sampler);
         test_batch_rejects_bad_requests(sampler);
+        test_speculative_verification(sampler);
     }
     catch (const std::exception& error)
     {
