@@ -116,6 +116,66 @@ def cpu_baseline(workload, host_threads, sample_rows):
     }
 
 
+def bench_speculative_verify(args, hip_sampler):
+    """One verification step of speculative generation per step: 2 D + 1 rows of V = 151,936 fp32 logits
+    resident in the handle's buffer, the small operands and the result crossing PCIe as the host entry
+    does.  Not the headline metric; printed in the same JSON shape."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+
+    if hip_sampler.device_count() < 1:
+        sys.exit("bench.py needs a GPU: no HIP device is visible")
+    drafts, vocab = args.drafts, 151936
+    options = dict(temperature=0.7, top_k=20, top_p=0.8, min_p=0.0)
+    rng = np.random.Generator(np.random.PCG64(77))
+    target = (rng.standard_normal((drafts + 1, vocab), dtype=np.float32) * np.float32(3.0))
+    draft = target[:drafts] + rng.standard_normal((drafts, vocab), dtype=np.float32) * np.float32(0.5)
+    proposed = [int(oracle_lib.oracle_sample(row, 0.37, **options)["token_id"]) for row in draft]
+    uniform_sets = [rng.random(drafts + 1, dtype=np.float32) for _ in range(64)]
+    sampler = hip_sampler.HipSampler(2 * drafts + 1, vocab)
+    sampler.upload_logits(np.concatenate([target, draft], axis=0))
+    mismatches = 0
+    accepted_total = 0
+    for uniforms in uniform_sets[:16]:
+        gpu, gpu_accepted = sampler.speculative_verify(proposed, uniforms, **options)
+        cpu, cpu_accepted = oracle_lib.oracle_speculative_verify(target, draft, proposed, uniforms, **options)
+        same = all(gpu[f] == cpu[f] for f in ("status", "accepted", "next_token_id", "accept_draws", "final_draw_consumed"))
+        same = same and np.float32(gpu["next_probability"]).view(np.uint32) == np.float32(cpu["next_probability"]).view(np.uint32)
+        same = same and np.array_equal(gpu_accepted[:cpu["accepted"]].view(np.uint32), cpu_accepted[:cpu["accepted"]].view(np.uint32))
+        mismatches += 0 if same else 1
+        accepted_total += int(cpu["accepted"])
+    for index in range(args.warmup):
+        sampler.speculative_verify(proposed, uniform_sets[index % 64], **options)
+    start = time.perf_counter()
+    for index in range(args.steps):
+        sampler.speculative_verify(proposed, uniform_sets[index % 64], **options)
+    seconds_per_step = (time.perf_counter() - start) / args.steps
+    cpu_start = time.perf_counter()
+    cpu_steps = 3
+    for index in range(cpu_steps):
+        oracle_lib.oracle_speculative_verify(target, draft, proposed, uniform_sets[index], **options)
+    cpu_seconds = (time.perf_counter() - cpu_start) / cpu_steps
+    bytes_per_step = (2 * drafts + 1) * vocab * 4
+    line = {
+        "metric": "speculative verification steps/sec, D=%d V=151936 fp32 temp+topk+topp" % drafts,
+        "value": 1.0 / seconds_per_step, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": seconds_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "speculative verification, %d drafted tokens, %d x %d fp32 logits resident in HBM; "
+                               "T 0.7, Top-K 20, Top-P 0.8" % (drafts, 2 * drafts + 1, vocab),
+                   "entry_point": "ncnn_moe_hip_sampler_speculative_verify (host operands, synchronous)"},
+        "roofline": {"bound": "hbm", "achieved": bytes_per_step / seconds_per_step / 1e9, "peak": HBM_PEAK_BYTES_PER_S / 1e9,
+                     "unit": "GB/s", "frac": bytes_per_step / seconds_per_step / HBM_PEAK_BYTES_PER_S, "traffic": None,
+                     "kernel": "scan_select_kernel + speculative_verify_kernel, wall clock of the synchronous call",
+                     "algorithmic_bytes_per_launch": bytes_per_step},
+        "parity": {"steps_checked": 16, "step_mismatches": mismatches, "mean_accepted": accepted_total / 16.0},
+        "cpu_baseline": {"value": 1.0 / cpu_seconds, "unit": "steps/s", "cores": 1, "kind": "port",
+                         "sample": "%d steps of the CPU oracle's verification (two full sorts per tested position)" % cpu_steps},
+    }
+    sampler.close()
+    print(json.dumps(line))
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -123,6 +183,7 @@ def main():
     parser.add_argument("--warmup", type=int, default=200)
     parser.add_argument("--workload", default="cfg2_topk_topp")
     parser.add_argument("--rows", type=int, default=0, help="batch rows (0: the configuration's own)")
+    parser.add_argument("--drafts", type=int, default=5, help="drafted tokens per step of --workload speculative_verify")
     parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
     parser.add_argument("--cpu-rows", type=int, default=64)
     parser.add_argument("--no-cpu-baseline", action="store_true")
@@ -135,6 +196,8 @@ def main():
 
     load_package()
     from ncnn_moe_runtime_amd import hip_sampler, workloads
+    if args.workload == "speculative_verify":
+        return bench_speculative_verify(args, hip_sampler)
     import torch
 
     if not torch.cuda.is_available() or hip_sampler.device_count() < 1:

@@ -56,10 +56,23 @@ struct ncnn_moe_hip_sampler
     int32_t* verify_ids = nullptr;
     float* verify_probabilities = nullptr;
     uint32_t* verify_counts = nullptr;
-    int32_t* verify_proposed = nullptr;
-    float* verify_uniforms = nullptr;
-    float* verify_accepted = nullptr;
-    ncnn_moe_verify_result* verify_result = nullptr;
+    // operands and outcome of a step travel as one block each, through pinned host memory
+    struct VerifyInput
+    {
+        ncnn_moe_sample_params params[2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1];
+        float row_uniforms[2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1];
+        int32_t proposed[NCNN_MOE_MAX_DRAFT_TOKENS];
+        float uniforms[NCNN_MOE_MAX_DRAFT_TOKENS + 1];
+    };
+    struct VerifyOutput
+    {
+        ncnn_moe_verify_result result;
+        float accepted[NCNN_MOE_MAX_DRAFT_TOKENS];
+    };
+    VerifyInput* verify_input = nullptr;        // device
+    VerifyOutput* verify_output = nullptr;      // device
+    VerifyInput* verify_input_host = nullptr;   // pinned
+    VerifyOutput* verify_output_host = nullptr; // pinned
 
     ncnn_moe_sample_params* single_params = nullptr;
     float* single_uniform = nullptr;
@@ -360,10 +373,10 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->verify_ids, kVerifyRows * kFastTopK * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->verify_probabilities, kVerifyRows * kFastTopK * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->verify_counts, kVerifyRows * sizeof(uint32_t)));
-    CREATE_CHECK(hipMalloc(&s->verify_proposed, NCNN_MOE_MAX_DRAFT_TOKENS * sizeof(int32_t)));
-    CREATE_CHECK(hipMalloc(&s->verify_uniforms, (NCNN_MOE_MAX_DRAFT_TOKENS + 1) * sizeof(float)));
-    CREATE_CHECK(hipMalloc(&s->verify_accepted, NCNN_MOE_MAX_DRAFT_TOKENS * sizeof(float)));
-    CREATE_CHECK(hipMalloc(&s->verify_result, sizeof(ncnn_moe_verify_result)));
+    CREATE_CHECK(hipMalloc(&s->verify_input, sizeof(ncnn_moe_hip_sampler::VerifyInput)));
+    CREATE_CHECK(hipMalloc(&s->verify_output, sizeof(ncnn_moe_hip_sampler::VerifyOutput)));
+    CREATE_CHECK(hipHostMalloc(&s->verify_input_host, sizeof(ncnn_moe_hip_sampler::VerifyInput), hipHostMallocDefault));
+    CREATE_CHECK(hipHostMalloc(&s->verify_output_host, sizeof(ncnn_moe_hip_sampler::VerifyOutput), hipHostMallocDefault));
     CREATE_CHECK(hipMalloc(&s->single_params, sizeof(ncnn_moe_sample_params)));
     CREATE_CHECK(hipMalloc(&s->single_uniform, sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->single_result, sizeof(ncnn_moe_sample_result)));
@@ -388,13 +401,16 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->sort_keys[0], s->sort_keys[1],
         s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
-        s->verify_probabilities, s->verify_counts, s->verify_proposed, s->verify_uniforms, s->verify_accepted,
-        s->verify_result};
+        s->verify_probabilities, s->verify_counts, s->verify_input, s->verify_output};
     for (void* buffer : buffers)
     {
         if (buffer != nullptr)
             (void)hipFree(buffer);
     }
+    if (s->verify_input_host != nullptr)
+        (void)hipHostFree(s->verify_input_host);
+    if (s->verify_output_host != nullptr)
+        (void)hipHostFree(s->verify_output_host);
     delete s;
 }
 
@@ -631,15 +647,16 @@ int ncnn_moe_hip_sampler_speculative_verify(
         return NCNN_MOE_SAMPLER_SUCCESS;
     }
     SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
-    std::vector<ncnn_moe_sample_params> row_params(rows, row_options);
-    std::vector<float> row_uniforms(rows, 0.0f);
-    row_uniforms[draft_count] = uniforms[draft_count]; // the draw of the row after the last drafted token
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->params, row_params.data(), rows * sizeof(ncnn_moe_sample_params), hipMemcpyHostToDevice, s->stream));
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->uniforms, row_uniforms.data(), rows * sizeof(float), hipMemcpyHostToDevice, s->stream));
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_proposed, proposed_token_ids, draft_count * sizeof(int32_t), hipMemcpyHostToDevice, s->stream));
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_uniforms, uniforms, (draft_count + 1) * sizeof(float), hipMemcpyHostToDevice, s->stream));
-    // the copies above read pageable host memory that lives only until this function returns
-    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    ncnn_moe_hip_sampler::VerifyInput& in = *s->verify_input_host;
+    for (uint32_t row = 0; row < rows; ++row)
+    {
+        in.params[row] = row_options;
+        in.row_uniforms[row] = 0.0f;
+    }
+    in.row_uniforms[draft_count] = uniforms[draft_count]; // the draw of the row after the last drafted token
+    std::memcpy(in.proposed, proposed_token_ids, draft_count * sizeof(int32_t));
+    std::memcpy(in.uniforms, uniforms, (draft_count + 1) * sizeof(float));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_input, s->verify_input_host, sizeof(in), hipMemcpyHostToDevice, s->stream));
 
     DistributionExport export_to;
     export_to.ids = s->verify_ids;
@@ -650,7 +667,7 @@ int ncnn_moe_hip_sampler_speculative_verify(
     passes.full_order = true; // rows whose ties overflow the select lists still get their distribution
     const int rc = launch_sampler(
         s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-        s->params, s->uniforms, nullptr, s->results, export_to, passes, s->stream);
+        s->verify_input->params, s->verify_input->row_uniforms, nullptr, s->results, export_to, passes, s->stream);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return rc;
     VerifyArgs v;
@@ -661,15 +678,16 @@ int ncnn_moe_hip_sampler_speculative_verify(
     v.distribution_probabilities = s->verify_probabilities;
     v.distribution_count = s->verify_counts;
     v.distribution_cap = kFastTopK;
-    v.proposed = s->verify_proposed;
-    v.uniforms = s->verify_uniforms;
-    v.accepted_probabilities = s->verify_accepted;
-    v.result = s->verify_result;
+    v.proposed = s->verify_input->proposed;
+    v.uniforms = s->verify_input->uniforms;
+    v.accepted_probabilities = s->verify_output->accepted;
+    v.result = &s->verify_output->result;
     hipLaunchKernelGGL(speculative_verify_kernel, dim3(1), dim3(kWaveSize), 0, s->stream, v);
     SAMPLER_HIP_CHECK(s, hipGetLastError());
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(result, s->verify_result, sizeof(*result), hipMemcpyDeviceToHost, s->stream));
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(accepted_probabilities, s->verify_accepted, draft_count * sizeof(float), hipMemcpyDeviceToHost, s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_output_host, s->verify_output, sizeof(ncnn_moe_hip_sampler::VerifyOutput), hipMemcpyDeviceToHost, s->stream));
     SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    *result = s->verify_output_host->result;
+    std::memcpy(accepted_probabilities, s->verify_output_host->accepted, draft_count * sizeof(float));
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 
