@@ -199,6 +199,148 @@ __device__ __forceinline__ void finish_row_wave(
         write_token(a, row, p, token, selected_probability, static_cast<uint32_t>(kept), draw_consumed, flags);
 }
 
+// The same walk for an ordered window of up to 64 * SLOTS candidates held by one wave: candidate i
+// sits in slot i / 64 of lane i % 64.  The sums are the CPU loops themselves, one fp32 addition per
+// candidate in order (a wave-uniform v_readlane feeds each addition), so nothing has to be proved
+// about them; a 1024-candidate window costs about 10,000 cycles per pass.
+template <int SLOTS>
+__device__ __forceinline__ void finish_row_wave_wide(
+    const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
+    const float (&value)[SLOTS], const int32_t (&index)[SLOTS], int n, int lane, uint8_t flags)
+{
+    const float temperature = p.temperature;
+    const float maximum = read_lane(value[0], 0) / temperature;
+    float term[SLOTS];
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+        term[s] = (s * kWaveSize + lane) < n ? expf_libm(value[s] / temperature - maximum) : 0.0f;
+
+    float normalizer = 0.0f;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+    {
+        const int slot_count = min(kWaveSize, n - s * kWaveSize);
+        for (int l = 0; l < slot_count; ++l)
+            normalizer += read_lane(term[s], l);
+    }
+    if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
+    {
+        if (lane == 0)
+            write_error(a, row, NCNN_MOE_ROW_INVALID_DISTRIBUTION, flags);
+        return;
+    }
+    float probability[SLOTS];
+    uint64_t keep[SLOTS];
+    const float threshold = (term[0] / normalizer) * p.min_p; // lane 0 holds the first candidate
+    const float first_threshold = read_lane(threshold, 0);
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+    {
+        probability[s] = term[s] / normalizer;
+        bool kept = (s * kWaveSize + lane) < n;
+        if (p.min_p > 0.0f)
+            kept = kept && probability[s] >= first_threshold;
+        keep[s] = __ballot(kept);
+    }
+
+    // Top-P (session.cpp:119-128); the renormaliser of :130-132 adds the same values in the same order
+    float cumulative = 0.0f;
+    int kept_count = 0;
+    int last_slot = 0, last_lane = 0;
+    bool reached = false;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+    {
+        uint64_t pending = reached ? 0ull : keep[s];
+        uint64_t taken = 0;
+        while (pending != 0)
+        {
+            const int l = __builtin_ctzll(pending);
+            pending &= pending - 1;
+            cumulative += read_lane(probability[s], l);
+            taken |= 1ull << l;
+            ++kept_count;
+            last_slot = s;
+            last_lane = l;
+            if (cumulative >= p.top_p)
+            {
+                reached = true;
+                break;
+            }
+        }
+        keep[s] = taken;
+    }
+    const float renormalizer = cumulative;
+    float final_probability[SLOTS];
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+        final_probability[s] = probability[s] / renormalizer;
+
+    if (a.distribution_count != nullptr)
+    {
+        const size_t first = static_cast<size_t>(row) * a.distribution_cap;
+        uint32_t before = 0;
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s)
+        {
+            if ((keep[s] >> lane) & 1ull)
+            {
+                const uint32_t position = before + static_cast<uint32_t>(lanes_below(keep[s]));
+                if (position < a.distribution_cap)
+                {
+                    a.distribution_ids[first + position] = index[s];
+                    a.distribution_probabilities[first + position] = final_probability[s];
+                }
+            }
+            before += static_cast<uint32_t>(__popcll(keep[s]));
+        }
+        if (lane == 0)
+            a.distribution_count[row] = static_cast<uint32_t>(kept_count);
+    }
+
+    int selected_slot = last_slot, selected_lane = last_lane; // the draw falls through to the last candidate
+    uint8_t draw_consumed = 0;
+    if (kept_count > 1)
+    {
+        draw_consumed = 1;
+        const float uniform = a.uniforms[row];
+        float running = 0.0f;
+        bool found = false;
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s)
+        {
+            uint64_t walk = found ? 0ull : keep[s];
+            while (walk != 0)
+            {
+                const int l = __builtin_ctzll(walk);
+                walk &= walk - 1;
+                running += read_lane(final_probability[s], l);
+                if (uniform < running)
+                {
+                    selected_slot = s;
+                    selected_lane = l;
+                    found = true;
+                    break;
+                }
+            }
+        }
+    }
+    float selected_probability = 1.0f;
+    int32_t token = -1;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+    {
+        if (s == selected_slot)
+        {
+            token = read_lane(index[s], selected_lane);
+            if (kept_count > 1)
+                selected_probability = read_lane(final_probability[s], selected_lane);
+        }
+    }
+    if (lane == 0)
+        write_token(a, row, p, token, selected_probability, static_cast<uint32_t>(kept_count), draw_consumed, flags);
+}
+
 template <int DTYPE>
 struct LogitsVector;
 
@@ -395,24 +537,20 @@ __device__ __forceinline__ uint32_t workgroup_kth_largest_key(
     return scratch.result;
 }
 
-// A lower bound of the top_k-th largest of the workgroup's N values per thread (NaN and -inf do not
-// count), exact in the upper 16 bits of the key; 0 when fewer than top_k values count.  At least top_k
-// values reach the bound, and only as many more as share those 16 bits with the top_k-th largest.
-// All threads of the workgroup must call it.
-template <int N>
-__device__ __forceinline__ uint32_t workgroup_loose_kth_of_values(
-    const float (&values)[N], int top_k, int tid, BoundScratch& scratch)
+// The top_k-th largest of the workgroup's N keys per thread (0 = no key), found bit by bit over the
+// upper BITS bits of the key with workgroup-wide counts: BITS == 32 gives the exact key, fewer bits a
+// lower bound that at least top_k keys reach (and only as many more as share those bits with the
+// top_k-th largest).  0 when fewer than top_k keys exist.  All threads of the workgroup must call it.
+template <int BITS, int N>
+__device__ __forceinline__ uint32_t workgroup_kth_of_keys(
+    const uint32_t (&keys)[N], int top_k, int tid, BoundScratch& scratch)
 {
-    uint32_t keys[N];
-#pragma unroll
-    for (int i = 0; i < N; ++i)
-        keys[i] = values[i] > -__builtin_inff() ? ascending_key(values[i]) : 0u; // false for NaN as well
-    // one counter per bit in scratch.hot_keys
-    if (tid < 16)
-        scratch.hot_keys[tid] = 0;
+    static_assert(BITS >= 1 && BITS <= 32, "one counter per bit lives in the gather buffer");
+    if (tid < BITS)
+        scratch.hot_keys[tid] = 0; // one counter per bit
     __syncthreads();
     uint32_t prefix = 0;
-    for (int bit = 31; bit >= 16; --bit)
+    for (int bit = 31; bit > 31 - BITS; --bit)
     {
         const uint32_t trial = prefix | (1u << bit);
         int wave_count = 0;

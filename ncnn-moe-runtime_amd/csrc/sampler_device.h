@@ -207,6 +207,13 @@ __device__ __forceinline__ int lanes_below(uint64_t mask)
         static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)));
 }
 
+// Workgroup barrier that orders LDS traffic only: waits for this wave's LDS operations, not for its
+// outstanding global loads and stores (which __syncthreads() would also wait for).
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 __device__ __forceinline__ float read_lane(float value, int lane)
 {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(value), lane));

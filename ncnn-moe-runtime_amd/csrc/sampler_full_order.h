@@ -97,33 +97,43 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
         uint32_t* target_indices = indices[pass & 1];
         if (tid < 256)
             digit_base[tid] = histogram[pass][tid];
-        for (uint32_t tile = 0; tile < n; tile += kSortTile)
-        {
-            for (int i = tid; i < kSortWaves * 256; i += kSortThreads)
-                (&wave_counts[0][0])[i] = 0;
-            uint32_t tile_keys[kSortPerThread];
-            uint32_t tile_indices[kSortPerThread];
-            uint32_t tile_ranks[kSortPerThread];
+        // The next tile's keys are loaded while this tile is ranked, and the barriers inside the loop
+        // order LDS traffic only: a tile reads one global buffer and writes the other, so nothing in the
+        // loop has to wait for its scattered stores.
+        auto load_tile = [&](uint32_t tile, uint32_t (&out_keys)[kSortPerThread], uint32_t (&out_indices)[kSortPerThread]) {
             const uint32_t wave_first = tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread);
 #pragma unroll
             for (int e = 0; e < kSortPerThread; ++e)
             {
                 const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
-                tile_keys[e] = 0xffffffffu;
-                tile_indices[e] = i;
-                if (i < n)
+                const uint32_t source = i < n ? i : n - 1u; // always a valid address; masked below
+                uint32_t key;
+                uint32_t index = i;
+                if (pass == 0)
+                    key = descending_key(load_logit<DTYPE>(row_pointer, source));
+                else
                 {
-                    if (pass == 0)
-                        tile_keys[e] = descending_key(load_logit<DTYPE>(row_pointer, i));
-                    else
-                    {
-                        tile_keys[e] = source_keys[i];
-                        if (PAIRS)
-                            tile_indices[e] = source_indices[i];
-                    }
+                    key = source_keys[source];
+                    if (PAIRS)
+                        index = source_indices[source];
                 }
+                out_keys[e] = i < n ? key : 0xffffffffu;
+                out_indices[e] = i < n ? index : i;
             }
-            __syncthreads();
+        };
+        uint32_t tile_keys[kSortPerThread];
+        uint32_t tile_indices[kSortPerThread];
+        load_tile(0, tile_keys, tile_indices);
+        for (uint32_t tile = 0; tile < n; tile += kSortTile)
+        {
+            uint32_t next_keys[kSortPerThread];
+            uint32_t next_indices[kSortPerThread];
+            load_tile(tile + kSortTile < n ? tile + kSortTile : tile, next_keys, next_indices);
+            for (int i = tid; i < kSortWaves * 256; i += kSortThreads)
+                (&wave_counts[0][0])[i] = 0;
+            uint32_t tile_ranks[kSortPerThread];
+            const uint32_t wave_first = tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread);
+            lds_barrier();
 #pragma unroll
             for (int e = 0; e < kSortPerThread; ++e)
             {
@@ -146,7 +156,7 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
                 if (valid && rank_in_round == 0)
                     wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popcll(peers));
             }
-            __syncthreads();
+            lds_barrier();
             if (tid < 256)
             {
                 uint32_t running = digit_base[tid];
@@ -159,7 +169,7 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
                 }
                 digit_base[tid] = running;
             }
-            __syncthreads();
+            lds_barrier();
 #pragma unroll
             for (int e = 0; e < kSortPerThread; ++e)
             {
@@ -173,7 +183,13 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
                         target_indices[position] = tile_indices[e];
                 }
             }
-            __syncthreads();
+            lds_barrier();
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
+            {
+                tile_keys[e] = next_keys[e];
+                tile_indices[e] = next_indices[e];
+            }
         }
         __threadfence_block();
         __syncthreads();

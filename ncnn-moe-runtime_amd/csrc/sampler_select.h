@@ -66,22 +66,21 @@ __device__ __forceinline__ uint32_t tighten_list(SelectShared<WIDE>& shared, uin
     const uint32_t count = min(shared.list_count, static_cast<uint32_t>(SelectShared<WIDE>::kListCap));
     uint32_t keys[kPerThread];
     int32_t indices[kPerThread];
-    uint32_t best = 0, second = 0; // the thread's two best candidates: two distinct logits
+    uint32_t best = 0;
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
     {
         const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
         keys[j] = q < count ? shared.list_keys[q] : 0u;
         indices[j] = q < count ? shared.list_indices[q] : 0;
-        second = max(second, min(best, keys[j]));
         best = max(best, keys[j]);
     }
-    // at least K candidates reach the K-th largest of the per-thread best and second-best keys
     uint32_t kth;
     if constexpr (kPerThread > 1)
     {
-        const uint32_t thread_keys[2] = {best, second};
-        kth = workgroup_kth_largest_key(thread_keys, top_k, tid, shared.bound, true);
+        // a long list: the exact K-th best of all its entries (a bound from per-thread maxima would keep
+        // most of a list whose threads hold several members of a wide window each)
+        kth = workgroup_kth_of_keys<32>(keys, top_k, tid, shared.bound);
     }
     else
     {
@@ -256,7 +255,7 @@ __device__ __forceinline__ void finish_from_list(
             }
         }
         __syncthreads();
-        const uint32_t n = static_cast<uint32_t>(n_ranked < top_k ? n_ranked : top_k);
+        const int n = n_ranked < top_k ? n_ranked : top_k;
         if (tid == 0)
             a.row_state[row] = kRowDone;
         if (n == 0)
@@ -265,9 +264,20 @@ __device__ __forceinline__ void finish_from_list(
                 write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
             return;
         }
-        const uint32_t* sorted_indices = shared.sorted_indices;
-        auto token_at = [&](uint32_t rank) -> int32_t { return static_cast<int32_t>(sorted_indices[rank]); };
-        replay_sorted_window(a, row, p, shared.sorted_keys, n, shared.sorted_indices, result_flags, shared.replay, tid, token_at);
+        if (wave != 0)
+            return;
+        // wave 0 walks the ordered window: candidate i in slot i / 64 of lane i % 64
+        constexpr int kSlots = kSelectTopK / kWaveSize;
+        float values[kSlots];
+        int32_t tokens[kSlots];
+#pragma unroll
+        for (int s = 0; s < kSlots; ++s)
+        {
+            const int i = s * kWaveSize + lane;
+            values[s] = i < n ? value_from_descending_key(shared.sorted_keys[i]) : 0.0f;
+            tokens[s] = i < n ? static_cast<int32_t>(shared.sorted_indices[i]) : -1;
+        }
+        finish_row_wave_wide<kSlots>(a, row, p, values, tokens, n, lane, result_flags);
     }
 }
 
@@ -451,7 +461,11 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
             if (WIDE && top_k > kTwoKeyBoundTopK)
             {
                 // a wide window: the lane maxima bound too loosely, so select over every value of the chunk
-                bound_key = max(bound_key, workgroup_loose_kth_of_values(values, top_k, tid, shared.bound));
+                uint32_t value_keys[kLaneValues];
+#pragma unroll
+                for (int i = 0; i < kLaneValues; ++i)
+                    value_keys[i] = values[i] > -__builtin_inff() ? ascending_key(values[i]) : 0u; // false for NaN as well
+                bound_key = max(bound_key, workgroup_kth_of_keys<32>(value_keys, top_k, tid, shared.bound));
             }
             else if constexpr (WIDE)
             {
