@@ -43,8 +43,13 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
     const uint32_t n = a.vocab;
 
     __shared__ uint32_t histogram[kPasses][256];
-    __shared__ uint32_t digit_base[256];
+    __shared__ uint32_t digit_base[256];          // output position of the next key of each digit
     __shared__ uint32_t wave_counts[kSortWaves][256];
+    __shared__ uint32_t tile_start[256];          // first slot of each digit in the staged tile
+    __shared__ uint32_t global_offset[256];       // output position minus staged slot, per digit
+    __shared__ uint32_t scan_partial[4];
+    __shared__ uint32_t staged_keys[kSortTile];   // the tile ordered by digit, written out in runs
+    __shared__ uint32_t staged_indices[PAIRS ? kSortTile : 1];
 
     const char* row_pointer = static_cast<const char*>(a.logits) +
         static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
@@ -54,6 +59,8 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
     for (int i = tid; i < kPasses * 256; i += kSortThreads)
         (&histogram[0][0])[i] = 0;
     __syncthreads();
+    // Digit histograms of every pass (plain LDS atomics: matching equal digits with ballots first, to
+    // spare the same-address conflicts of the upper digits, was measured and costs more than it saves).
     for (uint32_t i = tid; i < n; i += kSortThreads)
     {
         const uint32_t key = descending_key(load_logit<DTYPE>(row_pointer, i));
@@ -157,19 +164,41 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
                     wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popcll(peers));
             }
             lds_barrier();
+            // per digit: slots of the waves inside the digit's run, the run's length, then the runs' starts
+            uint32_t digit_total = 0;
+            uint32_t inclusive = 0;
             if (tid < 256)
             {
-                uint32_t running = digit_base[tid];
 #pragma unroll
                 for (int w = 0; w < kSortWaves; ++w)
                 {
                     const uint32_t c = wave_counts[w][tid];
-                    wave_counts[w][tid] = running;
-                    running += c;
+                    wave_counts[w][tid] = digit_total;
+                    digit_total += c;
                 }
-                digit_base[tid] = running;
+                inclusive = digit_total;
+#pragma unroll
+                for (int step = 1; step < kWaveSize; step <<= 1)
+                {
+                    const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
+                    if (lane >= step)
+                        inclusive += up;
+                }
+                if (lane == kWaveSize - 1)
+                    scan_partial[wave] = inclusive;
             }
             lds_barrier();
+            if (tid < 256)
+            {
+                uint32_t start = inclusive - digit_total;
+                for (int w = 0; w < wave; ++w)
+                    start += scan_partial[w];
+                tile_start[tid] = start;
+                global_offset[tid] = digit_base[tid] - start;
+                digit_base[tid] += digit_total;
+            }
+            lds_barrier();
+            // stage the tile in digit order (stable: waves in order, ranks in order) ...
 #pragma unroll
             for (int e = 0; e < kSortPerThread; ++e)
             {
@@ -177,10 +206,27 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
                 if (i < n)
                 {
                     const uint32_t digit = (tile_keys[e] >> shift) & 255u;
-                    const uint32_t position = wave_counts[wave][digit] + tile_ranks[e];
-                    target_keys[position] = tile_keys[e];
+                    const uint32_t slot = tile_start[digit] + wave_counts[wave][digit] + tile_ranks[e];
+                    staged_keys[slot] = tile_keys[e];
                     if (PAIRS)
-                        target_indices[position] = tile_indices[e];
+                        staged_indices[slot] = tile_indices[e];
+                }
+            }
+            lds_barrier();
+            // ... and write it out: consecutive threads hold consecutive slots, so a digit's run goes to
+            // consecutive addresses
+            const uint32_t tile_count = min(static_cast<uint32_t>(kSortTile), n - tile);
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
+            {
+                const uint32_t slot = static_cast<uint32_t>(e * kSortThreads + tid);
+                if (slot < tile_count)
+                {
+                    const uint32_t key = staged_keys[slot];
+                    const uint32_t position = global_offset[(key >> shift) & 255u] + slot;
+                    target_keys[position] = key;
+                    if (PAIRS)
+                        target_indices[position] = staged_indices[slot];
                 }
             }
             lds_barrier();
