@@ -56,7 +56,7 @@ enum ncnn_moe_row_status
     NCNN_MOE_ROW_NO_FINITE_LOGIT = 5,
     NCNN_MOE_ROW_INVALID_DISTRIBUTION = 6,
     /* Not a CPU-sampler error.  Only ncnn_moe_hip_sampler_sample_device called with
-     * may_need_full_order = 0 reports it, for a row that cannot be served by the Top-K select path:
+     * may_need_full_order = 0 reports it, for a row that the first select kernel cannot serve:
      * its Top-K window is absent or wider than 64, or its ties overflowed the select buffers.
      * Call again with may_need_full_order = 1. */
     NCNN_MOE_ROW_NEEDS_FULL_ORDER = 7
@@ -129,8 +129,9 @@ int ncnn_moe_hip_sampler_sample(
  * returns at once.  device_logits may be any device matrix (row_stride in elements), not only the
  * handle's buffer.  This is the entry the decode step calls in its own stream.
  * may_need_full_order: pass 0 when the caller knows from its host-side SamplingOptions that every
- * row is greedy or has 1 <= top_k <= 64 (then one kernel is enqueued); pass 1 otherwise (the
- * full-order kernels are enqueued as well and pick up the rows that need them). */
+ * row is greedy or has 1 <= top_k <= 64 (then one kernel is enqueued); pass 1 otherwise (a select
+ * kernel for Top-K windows up to 1024 and the full-order kernels are enqueued as well and pick up
+ * the rows that need them).  Calls on one handle share its scratch memory and must not overlap. */
 int ncnn_moe_hip_sampler_sample_device(
     ncnn_moe_hip_sampler* sampler,
     const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,

@@ -1,0 +1,79 @@
+"""ncnn_moe_hip_sampler_sample_device through the C ABI with every operand in device memory (torch only
+allocates the buffers and owns the stream): the entry the decode step calls.  Checks the three
+passes (batch-shaped select, wide select, full order), the may_need_full_order contract and that the
+call does not need the handle's own logits buffer."""
+import numpy as np
+import pytest
+
+import parity_util
+from ncnn_moe_runtime_amd import hip_sampler
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _device(array):
+    return torch.from_numpy(np.ascontiguousarray(array).view(np.uint8).reshape(-1)).to("cuda:0")
+
+
+def _run(sampler, logits, params, uniforms, may_need_full_order, stream):
+    rows, vocab = logits.shape
+    dtype = hip_sampler.LOGITS_F32 if logits.dtype == np.float32 else hip_sampler.LOGITS_BF16
+    d_logits, d_params, d_uniforms = _device(logits), _device(params), _device(uniforms)
+    d_results = torch.zeros(rows * 16, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    sampler.sample_device(d_logits.data_ptr(), dtype, rows, vocab, vocab, d_params.data_ptr(), d_uniforms.data_ptr(),
+                          None, d_results.data_ptr(), may_need_full_order, stream.cuda_stream)
+    stream.synchronize()
+    return d_results.cpu().numpy().view(hip_sampler.RESULT_DTYPE).reshape(rows)
+
+
+@pytest.mark.parametrize("rows", [24, 300])
+def test_three_passes_on_a_caller_stream(rows):
+    print("[case] sample_device, %d rows, mixed windows" % rows, flush=True)
+    rng = np.random.default_rng(rows)
+    vocab = 50021
+    logits = (rng.standard_normal((rows, vocab)) * 2.5).astype(np.float32)
+    params = hip_sampler.make_params(rows, 0.8, 0, 0.92, 0.0)
+    params["top_k"] = np.array([(1, 20, 64, 65, 700, 1024, 1025, 0)[i % 8] for i in range(rows)], dtype=np.uint32)
+    params["temperature"][::11] = 0.0
+    uniforms = rng.random(rows).astype(np.float32)
+    cpu = parity_util.run_oracle(logits, params, uniforms)
+    stream = torch.cuda.Stream(device="cuda:0")
+    with hip_sampler.HipSampler(rows, vocab) as sampler:
+        full = _run(sampler, logits, params, uniforms, True, stream)
+        parity_util.assert_results_match(full, cpu, "f32", "sample_device, all passes")
+        served_by_select = (params["temperature"] == 0.0) | ((params["top_k"] >= 1) & (params["top_k"] <= 1024))
+        assert ((full["flags"][served_by_select] & hip_sampler.FLAG_GENERAL_PATH) == 0).all()
+        # one kernel only: rows that need a later pass say so, the others are final
+        first = _run(sampler, logits, params, uniforms, False, stream)
+        narrow = (params["temperature"] == 0.0) | ((params["top_k"] >= 1) & (params["top_k"] <= 64))
+        assert (first["status"][~narrow] == hip_sampler.ROW_NEEDS_FULL_ORDER).all()
+        assert (first["token_id"][~narrow] == -1).all()
+        parity_util.assert_results_match(first[narrow], cpu[narrow], "f32", "sample_device, select pass only")
+        # and a second call with every pass finishes them
+        again = _run(sampler, logits, params, uniforms, True, stream)
+        parity_util.assert_results_match(again, cpu, "f32", "sample_device, repeated")
+
+
+def test_bf16_strided_rows_on_the_default_stream():
+    print("[case] sample_device, bf16, stride wider than the vocabulary", flush=True)
+    from ncnn_moe_runtime_amd import workloads
+    rng = np.random.default_rng(5)
+    rows, vocab, stride = 70, 40001, 40008
+    values = (rng.standard_normal((rows, stride)) * 2).astype(np.float32)
+    bits = workloads.float32_to_bf16_bits(values)
+    bits[:, vocab:] = workloads.float32_to_bf16_bits(np.full((rows, stride - vocab), 60.0, dtype=np.float32))  # never read
+    params = hip_sampler.make_params(rows, 0.7, 40, 0.9, 0.01)
+    uniforms = rng.random(rows).astype(np.float32)
+    cpu = parity_util.run_oracle(np.ascontiguousarray(bits[:, :vocab]), params, uniforms)
+    d_logits, d_params, d_uniforms = _device(bits), _device(params), _device(uniforms)
+    d_results = torch.zeros(rows * 16, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    with hip_sampler.HipSampler(rows, vocab) as sampler:
+        sampler.sample_device(d_logits.data_ptr(), hip_sampler.LOGITS_BF16, rows, vocab, stride, d_params.data_ptr(),
+                              d_uniforms.data_ptr(), None, d_results.data_ptr(), False, None)
+        torch.cuda.synchronize()
+    gpu = d_results.cpu().numpy().view(hip_sampler.RESULT_DTYPE).reshape(rows)
+    parity_util.assert_results_match(gpu, cpu, "bf16", "sample_device, bf16 strided")
