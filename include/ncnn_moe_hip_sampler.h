@@ -157,7 +157,8 @@ enum ncnn_moe_verify_status
     NCNN_MOE_VERIFY_ZERO_DRAFT_PROBABILITY = 2, /* "sampled draft token has zero probability" (:822-830) */
     NCNN_MOE_VERIFY_RESIDUAL_EMPTY = 3,         /* "speculative residual distribution is empty" (:170-175) */
     NCNN_MOE_VERIFY_RESIDUAL_FAILED = 4,        /* "speculative residual sampling failed" (:199-201) */
-    /* Not a CPU-sampler error: with temperature > 0 this entry serves Top-K windows of 1..64 only. */
+    /* Not a CPU-sampler error: a filtered distribution (after Top-K, Min-P, Top-P) that the accept loop
+     * reached holds more than 1024 candidates, which is what this entry keeps per row. */
     NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW = 5
 };
 

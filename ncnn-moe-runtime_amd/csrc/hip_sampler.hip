@@ -370,8 +370,8 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->distribution_probabilities, static_cast<size_t>(max_vocab) * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->distribution_count, sizeof(uint32_t)));
     constexpr size_t kVerifyRows = 2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1;
-    CREATE_CHECK(hipMalloc(&s->verify_ids, kVerifyRows * kFastTopK * sizeof(int32_t)));
-    CREATE_CHECK(hipMalloc(&s->verify_probabilities, kVerifyRows * kFastTopK * sizeof(float)));
+    CREATE_CHECK(hipMalloc(&s->verify_ids, kVerifyRows * kVerifyCap * sizeof(int32_t)));
+    CREATE_CHECK(hipMalloc(&s->verify_probabilities, kVerifyRows * kVerifyCap * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->verify_counts, kVerifyRows * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->verify_input, sizeof(ncnn_moe_hip_sampler::VerifyInput)));
     CREATE_CHECK(hipMalloc(&s->verify_output, sizeof(ncnn_moe_hip_sampler::VerifyOutput)));
@@ -638,14 +638,6 @@ int ncnn_moe_hip_sampler_speculative_verify(
     ncnn_moe_sample_params row_options = *options;
     row_options.stop_begin = 0;
     row_options.stop_count = 0;
-    // the exported distributions hold one Top-K window of at most kFastTopK candidates per row
-    uint32_t effective_k = 0;
-    int status = NCNN_MOE_ROW_OK;
-    if (resolve_row_mode(row_options, s->logits_vocab, kFastTopK, 0, effective_k, status) == kModeGeneral)
-    {
-        result->status = NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW;
-        return NCNN_MOE_SAMPLER_SUCCESS;
-    }
     SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
     ncnn_moe_hip_sampler::VerifyInput& in = *s->verify_input_host;
     for (uint32_t row = 0; row < rows; ++row)
@@ -662,9 +654,10 @@ int ncnn_moe_hip_sampler_speculative_verify(
     export_to.ids = s->verify_ids;
     export_to.probabilities = s->verify_probabilities;
     export_to.count = s->verify_counts;
-    export_to.cap = kFastTopK;
+    export_to.cap = kVerifyCap;
     SamplerPasses passes;
-    passes.full_order = true; // rows whose ties overflow the select lists still get their distribution
+    passes.wide_select = row_left_pending(row_options, s->logits_vocab, kFastTopK);
+    passes.full_order = true; // also serves rows whose ties overflow the select lists
     const int rc = launch_sampler(
         s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
         s->verify_input->params, s->verify_input->row_uniforms, nullptr, s->results, export_to, passes, s->stream);
@@ -677,12 +670,11 @@ int ncnn_moe_hip_sampler_speculative_verify(
     v.distribution_ids = s->verify_ids;
     v.distribution_probabilities = s->verify_probabilities;
     v.distribution_count = s->verify_counts;
-    v.distribution_cap = kFastTopK;
     v.proposed = s->verify_input->proposed;
     v.uniforms = s->verify_input->uniforms;
     v.accepted_probabilities = s->verify_output->accepted;
     v.result = &s->verify_output->result;
-    hipLaunchKernelGGL(speculative_verify_kernel, dim3(1), dim3(kWaveSize), 0, s->stream, v);
+    hipLaunchKernelGGL(speculative_verify_kernel, dim3(1), dim3(kVerifyThreads), 0, s->stream, v);
     SAMPLER_HIP_CHECK(s, hipGetLastError());
     SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_output_host, s->verify_output, sizeof(ncnn_moe_hip_sampler::VerifyOutput), hipMemcpyDeviceToHost, s->stream));
     SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
@@ -700,7 +692,7 @@ const char* ncnn_moe_hip_sampler_verify_status_message(int verify_status)
     case NCNN_MOE_VERIFY_ZERO_DRAFT_PROBABILITY: return "sampled draft token has zero probability";
     case NCNN_MOE_VERIFY_RESIDUAL_EMPTY: return "speculative residual distribution is empty";
     case NCNN_MOE_VERIFY_RESIDUAL_FAILED: return "speculative residual sampling failed";
-    case NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW: return "speculative verification on the device needs temperature 0 or 1 <= top_k <= 64";
+    case NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW: return "speculative verification on the device holds filtered distributions of up to 1024 candidates";
     default: return "unknown verification status";
     }
 }

@@ -1,6 +1,6 @@
 // Speculative verification (src/engine/session.cpp:776-874): the accept loop over the drafted
 // tokens and the draw of the token that follows them, from the filtered distributions that the
-// sampling kernels exported for the target and draft rows.  One wave.
+// sampling kernels exported for the target and draft rows.  One workgroup.
 #ifndef NCNN_MOE_HIP_SAMPLER_VERIFY_H
 #define NCNN_MOE_HIP_SAMPLER_VERIFY_H
 
@@ -8,15 +8,18 @@
 
 namespace ncnn_moe_hip {
 
+constexpr int kVerifyThreads = 512;
+constexpr int kVerifyCap = kSelectTopK; // candidates of a row's filtered distribution the step can use
+constexpr int kVerifySlots = kVerifyCap / kWaveSize;
+
 struct VerifyArgs
 {
     uint32_t draft_count;
     float temperature;
     const ncnn_moe_sample_result* row_results; // [2 * draft_count + 1]: target rows, then draft rows
-    const int32_t* distribution_ids;           // [rows][distribution_cap], cap <= 64
+    const int32_t* distribution_ids;           // [rows][kVerifyCap]
     const float* distribution_probabilities;
-    const uint32_t* distribution_count;        // [rows]
-    uint32_t distribution_cap;
+    const uint32_t* distribution_count;        // [rows]: the full kept length, which may exceed kVerifyCap
     const int32_t* proposed;                   // [draft_count]
     const float* uniforms;                     // [draft_count + 1]
     float* accepted_probabilities;             // [draft_count]
@@ -25,19 +28,14 @@ struct VerifyArgs
 
 struct VerifyShared
 {
-    float residual[kWaveSize];
-    int32_t token[kWaveSize];
+    int32_t target_ids[kVerifyCap];
+    float target_probabilities[kVerifyCap];
+    int32_t draft_ids[kVerifyCap];
+    float draft_probabilities[kVerifyCap];
+    float ordered_residual[kVerifyCap]; // the residual in token-id order
+    int32_t ordered_token[kVerifyCap];
+    float found[2];                     // candidate_probability of the proposed token: target, draft
 };
-
-// candidate_probability (src/engine/session.cpp:138-148): the probability the row's filtered
-// distribution gives `token`, 0 when it is not a candidate.  Lane l holds candidate l of the row.
-__device__ __forceinline__ float candidate_probability_wave(int32_t candidate_id, float probability, bool valid, int32_t token)
-{
-    const uint64_t match = __ballot(valid && candidate_id == token);
-    if (match == 0)
-        return 0.0f;
-    return read_lane(probability, __builtin_ctzll(match));
-}
 
 __device__ __forceinline__ void write_verify_result(
     const VerifyArgs& v, uint32_t accepted, int32_t token, float probability, uint32_t status, uint32_t row_status,
@@ -55,10 +53,12 @@ __device__ __forceinline__ void write_verify_result(
     *v.result = r;
 }
 
-__global__ __launch_bounds__(kWaveSize) void speculative_verify_kernel(VerifyArgs v)
+__global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(VerifyArgs v)
 {
     __shared__ VerifyShared shared;
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
     const uint32_t drafts = v.draft_count;
     uint32_t accepted = 0;
     uint32_t accept_draws = 0;
@@ -71,13 +71,13 @@ __global__ __launch_bounds__(kWaveSize) void speculative_verify_kernel(VerifyArg
             const ncnn_moe_sample_result target = v.row_results[accepted];
             if (target.status != NCNN_MOE_ROW_OK)
             {
-                if (lane == 0)
+                if (tid == 0)
                     write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ROW_ERROR, target.status, 0, 0, 0);
                 return;
             }
             if (target.token_id != v.proposed[accepted])
                 break;
-            if (lane == 0)
+            if (tid == 0)
                 v.accepted_probabilities[accepted] = 1.0f;
         }
     }
@@ -93,24 +93,49 @@ __global__ __launch_bounds__(kWaveSize) void speculative_verify_kernel(VerifyArg
             if (target.status != NCNN_MOE_ROW_OK || draft.status != NCNN_MOE_ROW_OK)
             {
                 const uint32_t row_status = target.status != NCNN_MOE_ROW_OK ? target.status : draft.status;
-                if (lane == 0)
+                if (tid == 0)
                     write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ROW_ERROR, row_status, accept_draws, 0, 0);
                 return;
             }
+            const uint32_t target_count = v.distribution_count[target_row];
+            const uint32_t draft_count = v.distribution_count[draft_row];
+            if (target_count > static_cast<uint32_t>(kVerifyCap) || draft_count > static_cast<uint32_t>(kVerifyCap))
+            {
+                // a filtered distribution longer than the step holds: reported, never approximated
+                if (tid == 0)
+                    write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW, 0, accept_draws, 0, 0);
+                return;
+            }
             const int32_t token = v.proposed[accepted];
-            const uint32_t target_count = min(v.distribution_count[target_row], v.distribution_cap);
-            const uint32_t draft_count = min(v.distribution_count[draft_row], v.distribution_cap);
-            const bool target_valid = static_cast<uint32_t>(lane) < target_count;
-            const bool draft_valid = static_cast<uint32_t>(lane) < draft_count;
-            const int32_t target_id = target_valid ? v.distribution_ids[target_row * v.distribution_cap + lane] : -1;
-            const float target_p = target_valid ? v.distribution_probabilities[target_row * v.distribution_cap + lane] : 0.0f;
-            const int32_t draft_id = draft_valid ? v.distribution_ids[draft_row * v.distribution_cap + lane] : -1;
-            const float draft_p = draft_valid ? v.distribution_probabilities[draft_row * v.distribution_cap + lane] : 0.0f;
-            const float target_probability = candidate_probability_wave(target_id, target_p, target_valid, token);
-            const float draft_probability = candidate_probability_wave(draft_id, draft_p, draft_valid, token);
+            // ---- candidate_probability (session.cpp:138-148) of the proposed token in both lists; the
+            // lists go to LDS on the way, for the residual that a rejection needs
+            if (tid < 2)
+                shared.found[tid] = 0.0f;
+            __syncthreads();
+            for (uint32_t j = tid; j < target_count; j += kVerifyThreads)
+            {
+                const int32_t id = v.distribution_ids[static_cast<size_t>(target_row) * kVerifyCap + j];
+                const float probability = v.distribution_probabilities[static_cast<size_t>(target_row) * kVerifyCap + j];
+                shared.target_ids[j] = id;
+                shared.target_probabilities[j] = probability;
+                if (id == token)
+                    shared.found[0] = probability; // ids are distinct: at most one writer
+            }
+            for (uint32_t j = tid; j < draft_count; j += kVerifyThreads)
+            {
+                const int32_t id = v.distribution_ids[static_cast<size_t>(draft_row) * kVerifyCap + j];
+                const float probability = v.distribution_probabilities[static_cast<size_t>(draft_row) * kVerifyCap + j];
+                shared.draft_ids[j] = id;
+                shared.draft_probabilities[j] = probability;
+                if (id == token)
+                    shared.found[1] = probability;
+            }
+            __syncthreads();
+            const float target_probability = shared.found[0];
+            const float draft_probability = shared.found[1];
             if (draft_probability <= 0.0f)
             {
-                if (lane == 0)
+                if (tid == 0)
                     write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ZERO_DRAFT_PROBABILITY, 0, accept_draws, 0, 0);
                 return;
             }
@@ -122,31 +147,46 @@ __global__ __launch_bounds__(kWaveSize) void speculative_verify_kernel(VerifyArg
             {
                 // ---- rejected: sample_residual_distribution (session.cpp:150-202) over
                 // max(0, target - draft), summed and walked in token-id order
-                float residual = target_p;
-                for (uint32_t j = 0; j < draft_count; ++j)
+                for (uint32_t j = tid; j < target_count; j += kVerifyThreads)
                 {
-                    const int32_t other_id = read_lane(draft_id, static_cast<int>(j));
-                    const float other_p = read_lane(draft_p, static_cast<int>(j));
-                    if (target_valid && other_id == target_id)
+                    const int32_t id = shared.target_ids[j];
+                    float residual = shared.target_probabilities[j];
+                    int rank = 0;
+                    for (uint32_t q = 0; q < draft_count; ++q)
                     {
-                        const float difference = residual - other_p;
-                        residual = 0.0f < difference ? difference : 0.0f; // std::max(0.0f, difference)
+                        if (shared.draft_ids[q] == id)
+                        {
+                            const float difference = residual - shared.draft_probabilities[q];
+                            residual = 0.0f < difference ? difference : 0.0f; // std::max(0.0f, difference)
+                        }
                     }
-                }
-                int rank = 0;
-                for (uint32_t j = 0; j < target_count; ++j)
-                    rank += read_lane(target_id, static_cast<int>(j)) < target_id ? 1 : 0;
-                if (target_valid)
-                {
-                    shared.residual[rank] = residual;
-                    shared.token[rank] = target_id;
+                    for (uint32_t q = 0; q < target_count; ++q)
+                        rank += shared.target_ids[q] < id ? 1 : 0;
+                    shared.ordered_residual[rank] = residual;
+                    shared.ordered_token[rank] = id;
                 }
                 __syncthreads();
-                const float ordered_residual = target_valid ? shared.residual[lane] : 0.0f;
-                const int32_t ordered_token = target_valid ? shared.token[lane] : -1;
-                float normalizer = 0.0f; // std::accumulate over the dense vector: zeros leave the sum as it is
-                for (uint32_t j = 0; j < target_count; ++j)
-                    normalizer += read_lane(ordered_residual, static_cast<int>(j));
+                if (wave != 0)
+                    return;
+                // one wave walks the ordered residual: entry i in slot i / 64 of lane i % 64, one fp32
+                // addition per entry in order, as std::accumulate over the dense vector does (zeros
+                // leave an fp32 sum as it is)
+                const int n = static_cast<int>(target_count);
+                float residual[kVerifySlots];
+#pragma unroll
+                for (int s = 0; s < kVerifySlots; ++s)
+                {
+                    const int i = s * kWaveSize + lane;
+                    residual[s] = i < n ? shared.ordered_residual[i] : 0.0f;
+                }
+                float normalizer = 0.0f;
+#pragma unroll
+                for (int s = 0; s < kVerifySlots; ++s)
+                {
+                    const int slot_count = min(kWaveSize, n - s * kWaveSize);
+                    for (int l = 0; l < slot_count; ++l)
+                        normalizer += read_lane(residual[s], l);
+                }
                 if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
                 {
                     if (lane == 0)
@@ -157,44 +197,48 @@ __global__ __launch_bounds__(kWaveSize) void speculative_verify_kernel(VerifyArg
                 const float sample_value = v.uniforms[accept_draws] * normalizer;
                 float cumulative = 0.0f;
                 int selected = -1;
-                for (uint32_t j = 0; j < target_count; ++j)
+                int last_positive = -1;
+#pragma unroll
+                for (int s = 0; s < kVerifySlots; ++s)
                 {
-                    cumulative += read_lane(ordered_residual, static_cast<int>(j));
-                    if (sample_value < cumulative)
+                    const int slot_count = selected >= 0 ? 0 : min(kWaveSize, n - s * kWaveSize);
+                    for (int l = 0; l < slot_count; ++l)
                     {
-                        selected = static_cast<int>(j);
-                        break;
+                        const float value = read_lane(residual[s], l);
+                        cumulative += value;
+                        if (value > 0.0f)
+                            last_positive = s * kWaveSize + l;
+                        if (sample_value < cumulative)
+                        {
+                            selected = s * kWaveSize + l;
+                            break;
+                        }
                     }
                 }
                 if (selected < 0)
-                {
-                    // session.cpp:189-198: the last token that has any residual mass
-                    const uint64_t positive = __ballot(target_valid && ordered_residual > 0.0f);
-                    if (positive != 0)
-                        selected = 63 - __builtin_clzll(positive);
-                }
+                    selected = last_positive; // session.cpp:189-198: the last token that has any residual mass
                 if (selected < 0)
                 {
                     if (lane == 0)
                         write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_RESIDUAL_FAILED, 0, accept_draws, 1, 1);
                     return;
                 }
-                const float chosen_residual = read_lane(ordered_residual, selected);
-                const int32_t chosen_token = read_lane(ordered_token, selected);
                 if (lane == 0)
-                    write_verify_result(v, accepted, chosen_token, chosen_residual / normalizer, NCNN_MOE_VERIFY_OK, 0,
+                    write_verify_result(v, accepted, shared.ordered_token[selected],
+                                        shared.ordered_residual[selected] / normalizer, NCNN_MOE_VERIFY_OK, 0,
                                         accept_draws, 1, 1);
                 return;
             }
-            if (lane == 0)
+            if (tid == 0)
                 v.accepted_probabilities[accepted] = target_probability;
+            __syncthreads(); // found[] is reset by the next position
         }
     }
 
     // ---- session.cpp:871-873: the target's own sample at the first position that was not accepted
     // (greedy mismatch) or after the last drafted token (everything accepted)
     const ncnn_moe_sample_result next = v.row_results[accepted];
-    if (lane == 0)
+    if (tid == 0)
     {
         if (next.status != NCNN_MOE_ROW_OK)
             write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ROW_ERROR, next.status, accept_draws, 0, 0);

@@ -396,12 +396,12 @@ static void test_speculative_verification(const HipSamplerPtr& sampler)
         auto outside = session.verify_speculative(target, draft, std::vector<int32_t>{0}, options);
         check(!outside && outside.error().code == ErrorCode::InternalError);
         check(outside.error().message == "sampled draft token has zero probability");
-        // no Top-K window over a vocabulary longer than 64: not served by this entry
-        std::vector<LogitsOutput> long_target = {logits_of(std::vector<float>(100, 0.5f)), logits_of(std::vector<float>(100, 0.5f))};
-        std::vector<LogitsOutput> long_draft = {logits_of(std::vector<float>(100, 0.5f))};
+        // a flat vocabulary of 3000 tokens with no filter: distributions longer than the entry holds
+        std::vector<LogitsOutput> long_target = {logits_of(std::vector<float>(3000, 0.5f)), logits_of(std::vector<float>(3000, 0.5f))};
+        std::vector<LogitsOutput> long_draft = {logits_of(std::vector<float>(3000, 0.5f))};
         auto window = session.verify_speculative(long_target, long_draft, std::vector<int32_t>{3}, SamplingOptions{});
         check(!window && window.error().code == ErrorCode::InvalidArgument);
-        // the same options over a short vocabulary are a window of its whole length
+        // the same options over a short vocabulary are served
         auto whole = session.verify_speculative(target, draft, std::vector<int32_t>{3}, SamplingOptions{});
         check(static_cast<bool>(whole));
         std::vector<LogitsOutput> broken = {logits_of(std::vector<float>(6, -std::numeric_limits<float>::infinity())), logits_of(ramp)};

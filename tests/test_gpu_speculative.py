@@ -62,6 +62,10 @@ def _propose(rng, draft, options):
     (32000, 8, dict(temperature=0.7, top_k=64, top_p=0.95, min_p=0.01)),
     (151936, 5, dict(temperature=1.2, top_k=40)),
     (151936, 16, dict(temperature=0.6, top_k=20, top_p=0.8)),
+    (32000, 3, dict(temperature=0.9, top_k=300, top_p=0.98)),        # the wide select kernel
+    (50000, 4, dict(temperature=1.0, top_k=1024)),
+    (20000, 2, dict(temperature=0.5, top_p=0.9)),                    # no Top-K window: sort + replay, short nucleus
+    (3000, 3, dict(temperature=0.8, top_k=2000, top_p=0.7, min_p=0.001)),
 ])
 def test_random_steps_match_oracle(sampler, vocab, drafts, options):
     rng = np.random.default_rng(vocab + drafts)
@@ -144,9 +148,15 @@ def test_residual_edge_cases(sampler):
 
 
 def test_unsupported_window_and_argument_errors(sampler):
-    sampler.upload_logits(np.zeros((3, 100), dtype=np.float32))
-    for options in (dict(temperature=1.0, top_k=0), dict(temperature=1.0, top_k=65)):
+    """A filtered distribution of more than 1024 candidates is reported, not approximated."""
+    flat = np.zeros((3, 5000), dtype=np.float32)
+    sampler.upload_logits(flat)
+    for options in (dict(temperature=1.0, top_k=0), dict(temperature=1.0, top_k=1025)):
         result, _ = sampler.speculative_verify([1], [0.5, 0.5], **options)
         assert result["status"] == hip_sampler.VERIFY_UNSUPPORTED_WINDOW and result["next_token_id"] == -1
+    # the same flat rows with a nucleus that keeps 1000 of them are served
+    cpu, _ = oracle_lib.oracle_speculative_verify(flat[:2], flat[2:], [1], [0.5, 0.5], temperature=1.0, top_p=0.2)
+    gpu, _ = sampler.speculative_verify([1], [0.5, 0.5], temperature=1.0, top_p=0.2)
+    assert gpu["status"] == cpu["status"] == 0 and gpu["next_token_id"] == cpu["next_token_id"]
     with pytest.raises(hip_sampler.SamplerError):
         sampler.speculative_verify([1, 2], [0.5, 0.5, 0.5], temperature=1.0, top_k=8)  # 3 rows hold one drafted token
