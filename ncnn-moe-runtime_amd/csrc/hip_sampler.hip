@@ -266,7 +266,7 @@ int launch_sampler(
             if (want_distribution)
                 hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kSortThreads), 0, stream, a);
             else
-                hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_BF16, false>), dim3(rows), dim3(kSortThreads), 0, stream, a);
+                hipLaunchKernelGGL(bf16_counting_sort_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
             hipLaunchKernelGGL(general_replay_kernel<NCNN_MOE_LOGITS_BF16>, dim3(rows), dim3(kReplayThreads), 0, stream, a);
         }
     }

@@ -1,6 +1,7 @@
 // Full-order path: rows with no Top-K window (or one too wide for the select path) need the complete
 // stable order, because the CPU sampler's sums run over it sequentially.
 //   general_sort_kernel    stable LSD radix sort of one row by descending key, one workgroup per row
+//   bf16_counting_sort_kernel  the same order for bf16 rows without indices, by counting the 65536 keys
 //   general_replay_kernel  the sampler's walk over the sorted row
 #ifndef NCNN_MOE_HIP_SAMPLER_FULL_ORDER_H
 #define NCNN_MOE_HIP_SAMPLER_FULL_ORDER_H
@@ -61,12 +62,27 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
     __syncthreads();
     // Digit histograms of every pass (plain LDS atomics: matching equal digits with ballots first, to
     // spare the same-address conflicts of the upper digits, was measured and costs more than it saves).
-    for (uint32_t i = tid; i < n; i += kSortThreads)
+    for (uint32_t first = 0; first < n; first += 8u * kSortThreads)
     {
-        const uint32_t key = descending_key(load_logit<DTYPE>(row_pointer, i));
+        float batch[8]; // eight independent loads in flight per thread
 #pragma unroll
-        for (int pass = 0; pass < kPasses; ++pass)
-            atomicAdd(&histogram[pass][(key >> (8 * (pass + kFirstDigit))) & 255u], 1u);
+        for (int k = 0; k < 8; ++k)
+        {
+            const uint32_t i = first + static_cast<uint32_t>(k * kSortThreads + tid);
+            batch[k] = load_logit<DTYPE>(row_pointer, i < n ? i : n - 1u);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+        {
+            const uint32_t i = first + static_cast<uint32_t>(k * kSortThreads + tid);
+            const uint32_t key = descending_key(batch[k]);
+            if (i < n)
+            {
+#pragma unroll
+                for (int pass = 0; pass < kPasses; ++pass)
+                    atomicAdd(&histogram[pass][(key >> (8 * (pass + kFirstDigit))) & 255u], 1u);
+            }
+        }
     }
     __syncthreads();
     // exclusive scan of each histogram by one wave (4 bins per lane)
@@ -238,6 +254,136 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
             }
         }
         __threadfence_block();
+        __syncthreads();
+    }
+}
+
+// bf16 rows without token indices: the 65536 possible keys are counted instead of sorted.  The keys of
+// a bf16 row differ only in their upper 16 bits, and sampling needs the sorted keys alone, so the
+// sorted row is the histogram written out.  Two rounds of 32768 LDS counters (non-negative logits
+// first: they sort first): count with LDS atomics, scan the counters, then every output position finds
+// its key by a binary search over the scanned counters, so the stores are coalesced.  One workgroup
+// per row; the sorted keys end in sort_keys[1], as after the radix sort.
+constexpr int kCountBins = 32768;
+
+__global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(SamplerArgs a)
+{
+    const uint32_t row = blockIdx.x;
+    if (a.row_state[row] != kRowNeedsGeneral)
+        return;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const uint32_t n = a.vocab;
+    constexpr int kBinsPerThread = kCountBins / kSortThreads;
+
+    __shared__ uint32_t bins[kCountBins];
+    __shared__ uint32_t wave_totals[kSortWaves];
+
+    const uint16_t* logits = reinterpret_cast<const uint16_t*>(
+        static_cast<const char*>(a.logits) + static_cast<size_t>(row) * a.row_stride * 2u);
+    uint32_t* sorted = a.sort_keys[1] + row * a.sort_stride;
+    const uint32_t misalignment = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(logits) & 15u) / 2u;
+    const uint16_t* aligned_logits = logits - misalignment;
+    const uint32_t aligned_end = misalignment + n; // positions [misalignment, aligned_end) hold the row
+
+    uint32_t written = 0; // keys of the earlier round
+    for (uint32_t round = 0; round < 2; ++round)
+    {
+#pragma unroll
+        for (int j = 0; j < kBinsPerThread; ++j)
+            bins[j * kSortThreads + tid] = 0;
+        __syncthreads();
+        // 16-byte loads of eight logits, four per thread in flight (single dependent 2-byte loads make
+        // the loop latency-bound); the row is read from the 16-byte boundary below its first element
+        for (uint32_t first = 0; first < aligned_end; first += 4u * 8u * kSortThreads)
+        {
+            uint4 raw[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                const uint32_t position = first + static_cast<uint32_t>(k * kSortThreads + tid) * 8u;
+                raw[k] = *reinterpret_cast<const uint4*>(aligned_logits + (position < aligned_end ? position : 0u));
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                const uint32_t position = first + static_cast<uint32_t>(k * kSortThreads + tid) * 8u;
+                const uint32_t words[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
+#pragma unroll
+                for (int c = 0; c < 8; ++c)
+                {
+                    const uint32_t bits = (c & 1) ? (words[c >> 1] >> 16) : (words[c >> 1] & 0xffffu);
+                    const uint32_t element = position + c;
+                    const uint32_t key16 = descending_key(__uint_as_float(bits << 16)) >> 16;
+                    if (element >= misalignment && element < aligned_end && (key16 >> 15) == round)
+                        atomicAdd(&bins[key16 & (kCountBins - 1)], 1u);
+                }
+            }
+        }
+        __syncthreads();
+        // exclusive scan of the counters: a thread owns kBinsPerThread consecutive bins
+        uint32_t counts[kBinsPerThread];
+        uint32_t thread_total = 0;
+#pragma unroll
+        for (int j = 0; j < kBinsPerThread; ++j)
+        {
+            counts[j] = bins[tid * kBinsPerThread + j];
+            thread_total += counts[j];
+        }
+        uint32_t inclusive = thread_total;
+#pragma unroll
+        for (int step = 1; step < kWaveSize; step <<= 1)
+        {
+            const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
+            if (lane >= step)
+                inclusive += up;
+        }
+        if (lane == kWaveSize - 1)
+            wave_totals[wave] = inclusive;
+        __syncthreads();
+        uint32_t before = inclusive - thread_total;
+        uint32_t round_total = 0;
+        for (int w = 0; w < kSortWaves; ++w)
+        {
+            const uint32_t c = wave_totals[w];
+            if (w < wave)
+                before += c;
+            round_total += c;
+        }
+#pragma unroll
+        for (int j = 0; j < kBinsPerThread; ++j)
+        {
+            bins[tid * kBinsPerThread + j] = before;
+            before += counts[j];
+        }
+        __syncthreads();
+        // write the runs: the waves take groups of 64 counters in turn (the keys of a row crowd into a
+        // narrow band of counters, so consecutive groups go to different waves), and for every counter
+        // that holds keys the wave's lanes write that many copies of the key to consecutive positions
+        {
+            for (uint32_t group = static_cast<uint32_t>(wave) * kWaveSize; group < static_cast<uint32_t>(kCountBins);
+                 group += kSortWaves * kWaveSize)
+            {
+                const uint32_t bin = group + static_cast<uint32_t>(lane);
+                const uint32_t start = bins[bin];
+                const uint32_t end = bin + 1u < static_cast<uint32_t>(kCountBins) ? bins[bin + 1u] : round_total;
+                uint64_t populated = __ballot(end > start);
+                while (populated != 0)
+                {
+                    const int source = __builtin_ctzll(populated);
+                    populated &= populated - 1;
+                    const uint32_t run_start = static_cast<uint32_t>(read_lane(static_cast<int>(start), source));
+                    const uint32_t run_end = static_cast<uint32_t>(read_lane(static_cast<int>(end), source));
+                    const uint32_t key16 = (round << 15) | (group + static_cast<uint32_t>(source));
+                    // the lower half of a key is all ones for a non-negative logit and for NaN, else zero
+                    const uint32_t key = key16 == 0xffffu ? 0xffffffffu : (key16 << 16) | (round == 0 ? 0xffffu : 0u);
+                    for (uint32_t position = run_start + static_cast<uint32_t>(lane); position < run_end; position += kWaveSize)
+                        sorted[written + position] = key;
+                }
+            }
+        }
+        written += round_total;
         __syncthreads();
     }
 }
