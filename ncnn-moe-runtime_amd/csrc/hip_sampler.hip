@@ -259,7 +259,7 @@ int launch_sampler(
                 hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_F32, true>), dim3(rows), dim3(kSortThreads), 0, stream, a);
             else
                 hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_F32, false>), dim3(rows), dim3(kSortThreads), 0, stream, a);
-            hipLaunchKernelGGL(general_replay_kernel<NCNN_MOE_LOGITS_F32>, dim3(rows), dim3(kReplayThreads), 0, stream, a);
+            hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_F32, false>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
         }
         else
         {
@@ -267,7 +267,10 @@ int launch_sampler(
                 hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kSortThreads), 0, stream, a);
             else
                 hipLaunchKernelGGL(bf16_counting_sort_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
-            hipLaunchKernelGGL(general_replay_kernel<NCNN_MOE_LOGITS_BF16>, dim3(rows), dim3(kReplayThreads), 0, stream, a);
+            if (want_distribution)
+                hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, false>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
+            else
+                hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
         }
     }
     SAMPLER_HIP_CHECK(s, hipGetLastError());

@@ -260,11 +260,13 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
 
 // bf16 rows without token indices: the 65536 possible keys are counted instead of sorted.  The keys of
 // a bf16 row differ only in their upper 16 bits, and sampling needs the sorted keys alone, so the
-// sorted row is the histogram written out.  Two rounds of 32768 LDS counters (non-negative logits
-// first: they sort first): count with LDS atomics, scan the counters, then every output position finds
-// its key by a binary search over the scanned counters, so the stores are coalesced.  One workgroup
-// per row; the sorted keys end in sort_keys[1], as after the radix sort.
+// sorted row is its histogram: it is written as RUNS, one (key, end position) pair per key that occurs,
+// in descending order of the logits, and the replay adds a run of equal terms in one step.  Two
+// rounds of 32768 LDS counters (non-negative logits first: they sort first): count with LDS atomics,
+// scan the counters and the flags "occurs", write the runs.  One workgroup per row.  Run keys go to
+// sort_keys[1], run ends to sort_keys[0], the number of runs to the row's first word of sort_indices[0].
 constexpr int kCountBins = 32768;
+constexpr int kCachedRuns = 6144; // runs of a row the replay keeps in LDS (48 KB)
 
 __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(SamplerArgs a)
 {
@@ -279,14 +281,17 @@ __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(Sample
 
     __shared__ uint32_t bins[kCountBins];
     __shared__ uint32_t wave_totals[kSortWaves];
+    __shared__ uint32_t wave_runs[kSortWaves];
 
     const uint16_t* logits = reinterpret_cast<const uint16_t*>(
         static_cast<const char*>(a.logits) + static_cast<size_t>(row) * a.row_stride * 2u);
-    uint32_t* sorted = a.sort_keys[1] + row * a.sort_stride;
+    uint32_t* run_keys = a.sort_keys[1] + row * a.sort_stride;
+    uint32_t* run_ends = a.sort_keys[0] + row * a.sort_stride;
     const uint32_t misalignment = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(logits) & 15u) / 2u;
     const uint16_t* aligned_logits = logits - misalignment;
     const uint32_t aligned_end = misalignment + n; // positions [misalignment, aligned_end) hold the row
 
+    uint32_t runs_written = 0; // runs of the earlier round
     uint32_t written = 0; // keys of the earlier round
     for (uint32_t round = 0; round < 2; ++round)
     {
@@ -322,70 +327,69 @@ __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(Sample
             }
         }
         __syncthreads();
-        // exclusive scan of the counters: a thread owns kBinsPerThread consecutive bins
+        // scan of the counts and of the number of keys that occur: a thread owns kBinsPerThread consecutive bins
         uint32_t counts[kBinsPerThread];
         uint32_t thread_total = 0;
+        uint32_t thread_runs = 0;
 #pragma unroll
         for (int j = 0; j < kBinsPerThread; ++j)
         {
             counts[j] = bins[tid * kBinsPerThread + j];
             thread_total += counts[j];
+            thread_runs += counts[j] != 0u ? 1u : 0u;
         }
         uint32_t inclusive = thread_total;
+        uint32_t inclusive_runs = thread_runs;
 #pragma unroll
         for (int step = 1; step < kWaveSize; step <<= 1)
         {
             const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
+            const uint32_t up_runs = __shfl_up(inclusive_runs, step, kWaveSize);
             if (lane >= step)
+            {
                 inclusive += up;
+                inclusive_runs += up_runs;
+            }
         }
         if (lane == kWaveSize - 1)
+        {
             wave_totals[wave] = inclusive;
+            wave_runs[wave] = inclusive_runs;
+        }
         __syncthreads();
         uint32_t before = inclusive - thread_total;
+        uint32_t runs_before = inclusive_runs - thread_runs;
         uint32_t round_total = 0;
+        uint32_t round_runs = 0;
         for (int w = 0; w < kSortWaves; ++w)
         {
-            const uint32_t c = wave_totals[w];
             if (w < wave)
-                before += c;
-            round_total += c;
+            {
+                before += wave_totals[w];
+                runs_before += wave_runs[w];
+            }
+            round_total += wave_totals[w];
+            round_runs += wave_runs[w];
         }
 #pragma unroll
         for (int j = 0; j < kBinsPerThread; ++j)
         {
-            bins[tid * kBinsPerThread + j] = before;
-            before += counts[j];
-        }
-        __syncthreads();
-        // write the runs: the waves take groups of 64 counters in turn (the keys of a row crowd into a
-        // narrow band of counters, so consecutive groups go to different waves), and for every counter
-        // that holds keys the wave's lanes write that many copies of the key to consecutive positions
-        {
-            for (uint32_t group = static_cast<uint32_t>(wave) * kWaveSize; group < static_cast<uint32_t>(kCountBins);
-                 group += kSortWaves * kWaveSize)
+            if (counts[j] != 0u)
             {
-                const uint32_t bin = group + static_cast<uint32_t>(lane);
-                const uint32_t start = bins[bin];
-                const uint32_t end = bin + 1u < static_cast<uint32_t>(kCountBins) ? bins[bin + 1u] : round_total;
-                uint64_t populated = __ballot(end > start);
-                while (populated != 0)
-                {
-                    const int source = __builtin_ctzll(populated);
-                    populated &= populated - 1;
-                    const uint32_t run_start = static_cast<uint32_t>(read_lane(static_cast<int>(start), source));
-                    const uint32_t run_end = static_cast<uint32_t>(read_lane(static_cast<int>(end), source));
-                    const uint32_t key16 = (round << 15) | (group + static_cast<uint32_t>(source));
-                    // the lower half of a key is all ones for a non-negative logit and for NaN, else zero
-                    const uint32_t key = key16 == 0xffffu ? 0xffffffffu : (key16 << 16) | (round == 0 ? 0xffffu : 0u);
-                    for (uint32_t position = run_start + static_cast<uint32_t>(lane); position < run_end; position += kWaveSize)
-                        sorted[written + position] = key;
-                }
+                const uint32_t key16 = (round << 15) | static_cast<uint32_t>(tid * kBinsPerThread + j);
+                before += counts[j];
+                // the lower half of a key is all ones for a non-negative logit and for NaN, else zero
+                run_keys[runs_written + runs_before] = key16 == 0xffffu ? 0xffffffffu : (key16 << 16) | (round == 0 ? 0xffffu : 0u);
+                run_ends[runs_written + runs_before] = written + before;
+                ++runs_before;
             }
         }
         written += round_total;
+        runs_written += round_runs;
         __syncthreads();
     }
+    if (tid == 0)
+        a.sort_indices[0][row * a.sort_stride] = runs_written;
 }
 
 struct RecoverScratch
@@ -398,11 +402,13 @@ struct RecoverScratch
 // the (rank - first position of that key)-th element, in index order, whose key equals keys[rank].
 // Every thread of the workgroup must call it.
 template <int DTYPE>
+__device__ __forceinline__ int32_t recover_token_of_key(
+    const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, RecoverScratch& scratch, int tid);
+
+template <int DTYPE>
 __device__ __forceinline__ int32_t recover_token_index(
     const void* row_pointer, uint32_t vocab, const uint32_t* keys, uint32_t rank, RecoverScratch& scratch, int tid)
 {
-    const int lane = tid & (kWaveSize - 1);
-    const int wave = tid >> 6;
     const uint32_t key = keys[rank];
     uint32_t low = 0, high = rank; // first position holding this key
     while (low < high)
@@ -413,74 +419,131 @@ __device__ __forceinline__ int32_t recover_token_index(
         else
             high = middle;
     }
-    const uint32_t ordinal = rank - low;
-    uint32_t passed = 0; // matches before the current chunk
+    return recover_token_of_key<DTYPE>(row_pointer, vocab, key, rank - low, scratch, tid);
+}
+
+// The ordinal-th element of the row, in index order, whose key equals `key`.  Every wave counts the
+// matches of its own contiguous eighth of the row (16-byte loads, four per lane in flight, no
+// barrier); the wave whose part holds the wanted match walks it again and locates the element with a
+// scan of the lanes' match counts.  Every thread of the workgroup must call it.
+template <int DTYPE>
+__device__ __forceinline__ int32_t recover_token_of_key(
+    const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, RecoverScratch& scratch, int tid)
+{
+    using Vector = LogitsVector<DTYPE>;
+    constexpr uint32_t kWidth = Vector::kWidth;
+    constexpr int kLoads = 8;
+    constexpr uint32_t kTrip = kLoads * kWaveSize * kWidth; // positions a wave looks at per trip
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    // positions count from the 16-byte boundary below the row: [misalignment, end) hold the row
+    const uint32_t misalignment =
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row_pointer) & 15u) / Vector::kElementBytes;
+    const char* aligned_base = static_cast<const char*>(row_pointer) - static_cast<size_t>(misalignment) * Vector::kElementBytes;
+    const uint32_t end = misalignment + vocab;
+    const uint32_t part = ((end + kReplayWaves - 1u) / kReplayWaves + kWidth - 1u) / kWidth * kWidth;
+    const uint32_t part_begin = min(end, static_cast<uint32_t>(wave) * part);
+    const uint32_t part_end = min(end, part_begin + part);
+
+    // per load k of a trip: the lane's matches among the kWidth positions from first + (k * 64 + lane) * kWidth
+    auto match_masks = [&](uint32_t first, uint32_t (&masks)[kLoads]) {
+        uint4 raw[kLoads];
+#pragma unroll
+        for (int k = 0; k < kLoads; ++k)
+        {
+            const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth;
+            raw[k] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(position < part_end ? position : part_begin) * Vector::kElementBytes);
+        }
+#pragma unroll
+        for (int k = 0; k < kLoads; ++k)
+        {
+            const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth;
+            float values[kWidth];
+            Vector::unpack(raw[k], values);
+            uint32_t mask = 0;
+#pragma unroll
+            for (uint32_t c = 0; c < kWidth; ++c)
+            {
+                const uint32_t element = position + c;
+                if (element >= misalignment && element < part_end && descending_key(values[c]) == key)
+                    mask |= 1u << c;
+            }
+            masks[k] = mask;
+        }
+    };
+
+    uint32_t lane_matches = 0;
+    for (uint32_t first = part_begin; first < part_end; first += kTrip)
+    {
+        uint32_t masks[kLoads];
+        match_masks(first, masks);
+#pragma unroll
+        for (int k = 0; k < kLoads; ++k)
+            lane_matches += static_cast<uint32_t>(__popc(masks[k]));
+    }
+    uint32_t matches = lane_matches;
+#pragma unroll
+    for (int step = 1; step < kWaveSize; step <<= 1)
+        matches += __shfl_xor(matches, step, kWaveSize);
+    if (lane == 0)
+        scratch.wave_counts[wave] = matches;
     if (tid == 0)
         scratch.found = -1;
     __syncthreads();
-    for (uint32_t base = 0; base < vocab; base += kReplayChunk)
+    uint32_t before = 0;
+    for (int w = 0; w < wave; ++w)
+        before += scratch.wave_counts[w];
+    if (ordinal >= before && ordinal < before + matches)
     {
-        const uint32_t first = base + static_cast<uint32_t>(tid) * kReplayPerThread;
-        uint32_t matches = 0;
-        uint32_t count = 0;
-#pragma unroll
-        for (int j = 0; j < kReplayPerThread; ++j)
+        uint32_t remaining = ordinal - before; // matches of this part still to skip
+        bool done = false;
+        for (uint32_t first = part_begin; first < part_end && !done; first += kTrip)
         {
-            const uint32_t i = first + j;
-            if (i < vocab && descending_key(load_logit<DTYPE>(row_pointer, i)) == key)
+            uint32_t masks[kLoads];
+            match_masks(first, masks);
+#pragma unroll
+            for (int k = 0; k < kLoads; ++k)
             {
-                matches |= 1u << j;
-                ++count;
-            }
-        }
-        uint32_t inclusive = count;
+                if (done)
+                    continue;
+                const uint32_t count = static_cast<uint32_t>(__popc(masks[k]));
+                uint32_t inclusive = count; // matches in lanes 0..lane of this load
 #pragma unroll
-        for (int step = 1; step < kWaveSize; step <<= 1)
-        {
-            const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
-            if (lane >= step)
-                inclusive += up;
-        }
-        if (lane == kWaveSize - 1)
-            scratch.wave_counts[wave] = inclusive;
-        __syncthreads();
-        uint32_t before = passed;
-        uint32_t chunk_total = 0;
-        for (int w = 0; w < kReplayWaves; ++w)
-        {
-            const uint32_t c = scratch.wave_counts[w];
-            if (w < wave)
-                before += c;
-            chunk_total += c;
-        }
-        before += inclusive - count;
-        if (ordinal >= before && ordinal < before + count)
-        {
-            uint32_t skip = ordinal - before;
-#pragma unroll
-            for (int j = 0; j < kReplayPerThread; ++j)
-            {
-                if (matches & (1u << j))
+                for (int step = 1; step < kWaveSize; step <<= 1)
                 {
-                    if (skip == 0)
-                        scratch.found = static_cast<int32_t>(first + j);
-                    --skip;
+                    const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
+                    if (lane >= step)
+                        inclusive += up;
                 }
+                const uint32_t total = static_cast<uint32_t>(read_lane(static_cast<int>(inclusive), kWaveSize - 1));
+                if (remaining < total)
+                {
+                    if (remaining >= inclusive - count && remaining < inclusive)
+                    {
+                        uint32_t mask = masks[k];
+                        for (uint32_t skipped = inclusive - count; skipped < remaining; ++skipped)
+                            mask &= mask - 1u;
+                        const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth +
+                            static_cast<uint32_t>(__builtin_ctz(mask));
+                        scratch.found = static_cast<int32_t>(position - misalignment);
+                    }
+                    done = true;
+                }
+                else
+                    remaining -= total;
             }
         }
-        __syncthreads();
-        if (scratch.found >= 0)
-            break;
-        passed += chunk_total;
     }
+    __syncthreads();
     const int32_t found = scratch.found;
     __syncthreads();
     return found;
 }
 
 // Full-order rows: walks the sorted row as the CPU sampler does (src/engine/session.cpp:84-134,
-// :429-442).  One workgroup per row.
-template <int DTYPE>
+// :429-442).  One workgroup per row.  With RUNS the row comes from bf16_counting_sort_kernel as runs
+// of equal keys; otherwise sort_keys[1] holds one key per element.
+template <int DTYPE, bool RUNS>
 __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerArgs a)
 {
     const uint32_t row = blockIdx.x;
@@ -489,9 +552,30 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     const int tid = threadIdx.x;
     const ncnn_moe_sample_params p = a.params[row];
     const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
-    const bool have_indices = a.distribution_count != nullptr; // the pair sort ran: indices are valid
+    const uint32_t* run_ends = RUNS ? a.sort_keys[0] + row * a.sort_stride : nullptr;
+    if constexpr (RUNS)
+    {
+        // a row of few runs is walked from LDS: its many binary searches are chains of dependent loads
+        __shared__ uint32_t cached_keys[kCachedRuns];
+        __shared__ uint32_t cached_ends[kCachedRuns];
+        const uint32_t run_total = a.sort_indices[0][row * a.sort_stride];
+        if (run_total <= static_cast<uint32_t>(kCachedRuns))
+        {
+            for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
+            {
+                cached_keys[i] = keys[i];
+                cached_ends[i] = run_ends[i];
+            }
+            __syncthreads();
+            keys = cached_keys;
+            run_ends = cached_ends;
+        }
+    }
+    const bool have_indices = !RUNS && a.distribution_count != nullptr; // the pair sort ran: indices are valid
     const uint32_t* indices = have_indices ? a.sort_indices[1] + row * a.sort_stride : nullptr;
     const uint32_t vocab = a.vocab;
+    // items: what `keys` holds one entry of (an element, or a run of equal keys)
+    const uint32_t items = RUNS ? a.sort_indices[0][row * a.sort_stride] : vocab;
     const char* row_pointer = static_cast<const char*>(a.logits) +
         static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
 
@@ -505,22 +589,39 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
         if (resolve_row_mode(p, vocab, a.max_select_top_k, 0, effective_k, status) != kModeGeneral)
             flags |= NCNN_MOE_ROW_FLAG_FALLBACK;
     }
-    if (keys[vocab - 1] == 0xffffffffu)
+    if (keys[items - 1] == 0xffffffffu)
         flags |= NCNN_MOE_ROW_FLAG_HAS_NAN;
     if (tid == 0)
         a.row_state[row] = kRowDone;
 
+    SortedRow layout; // only the run fields are used here
+    layout.keys = keys;
+    layout.run_ends = run_ends;
+    layout.run_count = items;
+    // first element of an item
+    auto first_element = [&](uint32_t item) -> uint32_t {
+        if constexpr (RUNS)
+            return item < items ? run_first_element(layout, item) : vocab;
+        else
+            return item;
+    };
     auto token_at = [&](uint32_t rank) -> int32_t {
         if (have_indices)
             return static_cast<int32_t>(indices[rank]);
-        return recover_token_index<DTYPE>(row_pointer, vocab, keys, rank, recover_scratch, tid);
+        if constexpr (RUNS)
+        {
+            const uint32_t run = run_of_element(layout, rank);
+            return recover_token_of_key<DTYPE>(row_pointer, vocab, keys[run], rank - run_first_element(layout, run), recover_scratch, tid);
+        }
+        else
+            return recover_token_index<DTYPE>(row_pointer, vocab, keys, rank, recover_scratch, tid);
     };
 
     if (p.temperature == 0.0f)
     {
         // a greedy row whose select overflowed (every logit tied): first finite logit in sorted order,
         // non-finite logits skipped (src/engine/session.cpp:404-424)
-        uint32_t low = 0, high = vocab;
+        uint32_t low = 0, high = items;
         while (low < high)
         {
             const uint32_t middle = (low + high) >> 1;
@@ -529,10 +630,10 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
             else
                 high = middle;
         }
-        const bool any_finite = low < vocab && keys[low] <= kLastFiniteKey;
+        const bool any_finite = low < items && keys[low] <= kLastFiniteKey;
         int32_t token = -1;
         if (any_finite)
-            token = token_at(low);
+            token = token_at(first_element(low));
         if (tid == 0)
         {
             if (any_finite)
@@ -562,7 +663,7 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
             write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, flags);
         return;
     }
-    uint32_t low = 0, high = vocab; // first position whose key is not finite
+    uint32_t low = 0, high = items; // first item whose key is not finite
     while (low < high)
     {
         const uint32_t middle = (low + high) >> 1;
@@ -571,10 +672,10 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
         else
             high = middle;
     }
-    uint32_t n = low;
+    uint32_t n = first_element(low);
     if (p.top_k > 0 && p.top_k < vocab && n > p.top_k)
         n = p.top_k;
-    replay_sorted_window(a, row, p, keys, n, indices, flags, scratch, tid, token_at);
+    replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at);
 }
 
 } // namespace ncnn_moe_hip
