@@ -379,3 +379,30 @@ def test_wide_windows_small_batch(small_sampler):
     plain[13:22] = False
     wide = plain & (params["top_k"] >= 1) & (params["top_k"] <= 1024)
     assert served_by_select[wide].all(), "rows with Top-K <= 1024 must not need the sort"
+
+
+def test_bf16_rows_of_few_distinct_values(batch_sampler):
+    """bf16 rows reach the full-order path as runs of equal keys; here the runs are enormous (one value
+    for the whole row, two or three values, a few hundred), so binade crossings and the Top-P / draw
+    stops fall deep inside a run, and Top-K windows end inside one."""
+    rng = np.random.default_rng(91)
+    rows, vocab = 48, 109000
+    logits = np.empty((rows, vocab), dtype=np.float32)
+    for row in range(rows):
+        distinct = int((1, 2, 3, 7, 40, 300)[row % 6])
+        values = (rng.standard_normal(distinct) * 3).astype(np.float32)
+        weights = rng.random(distinct) ** 3 + 1e-3
+        logits[row] = values[rng.choice(distinct, size=vocab, p=weights / weights.sum())]
+    logits[5, ::1000] = -np.inf
+    logits[11, 7] = np.nan
+    params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+    params["temperature"] = rng.choice(np.array([0.3, 1.0, 2.5], dtype=np.float32), size=rows)
+    params["top_k"] = rng.choice(np.array([0, 0, 1025, 5000, 60000], dtype=np.uint32), size=rows)
+    params["top_p"] = rng.choice(np.array([1.0, 0.999, 0.9, 0.5, 0.05], dtype=np.float32), size=rows)
+    params["min_p"] = rng.choice(np.array([0.0, 0.0, 0.5, 1.0], dtype=np.float32), size=rows)
+    uniforms = rng.random(rows).astype(np.float32)
+    uniforms[::5] = np.float32(1.0) - np.float32(2.0 ** -24)
+    bits = workloads.float32_to_bf16_bits(logits)
+    gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", context="bf16 rows of few distinct values")
+    assert ((gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH) != 0).all()
+    _check_rows(batch_sampler, logits, params, uniforms, context="the same rows as fp32 (radix sort)")
