@@ -2,8 +2,8 @@
 """Benchmark of the MI355X generation sampler: sampled rows/s and HBM GB/s on the logits read.
 
 A step is one pass of the sampler (ncnn_moe_hip_sampler_sample_device, every kernel of the path) over
-one batch of synthetic logits that is already resident in HBM.  The workload is configuration 2 of
-BASELINE.json: B=64, V=151,936 fp32 logits N(0, 3^2) with 8 spikes at +12 per row, temperature 0.7,
+one batch of synthetic logits that is already resident in HBM.  The workload is the headline
+configuration: B=64, V=151,936 fp32 logits N(0, 3^2) with 8 spikes at +12 per row, temperature 0.7,
 Top-K 20, Top-P 0.8.  Steps rotate over several distinct logits buffers whose total size exceeds the
 256 MB Infinity Cache, so the logits come from HBM and not from a cache warmed by the previous step.
 
