@@ -15,6 +15,7 @@
 
 #include "fixture_model_adapter.h"
 #include "kernels/cpu_ops.h"
+#include "ncnn/moe/expert_dispatcher.h"
 #include "ncnn/moe/runtime.h"
 
 #include <cstdio>
@@ -300,6 +301,74 @@ int ref_sample_residual_distribution(
     *token_id = sampled.value().token_id;
     *probability = sampled.value().probability;
     return 0;
+}
+
+/*
+ * ExpertDispatcher::dispatch (src/graph/expert_dispatcher.cpp:76-157) or, with use_dispatch_into != 0,
+ * dispatch_into (:159-301), through the reference's public class.  The plan comes back flat: routes
+ * grouped by expert in the order of plan.batches, expert_offsets[e] .. expert_offsets[e + 1] for every
+ * expert id (expert_count + 1 entries).  Returns 0, or 1 + ErrorCode with the message.
+ */
+int ref_router_dispatch(
+    const float* router_logits, uint32_t token_count,
+    uint32_t expert_count, uint32_t top_k, uint32_t score_function, uint32_t normalization, uint32_t flags,
+    float routed_scaling_factor, const float* selection_bias, const uint32_t* explicit_expert_ids,
+    int use_dispatch_into, uint32_t* expert_offsets, uint32_t* route_tokens, uint32_t* route_ranks, float* route_weights,
+    uint64_t* assignment_count, char* message, size_t message_cap)
+{
+    ExpertDispatchOptions options;
+    options.expert_count = expert_count;
+    options.top_k = top_k;
+    options.score_function = static_cast<RouterScoreFunction>(score_function);
+    options.normalization = static_cast<RouterNormalization>(normalization);
+    options.routed_scaling_factor = routed_scaling_factor;
+    options.flags = flags;
+    if (selection_bias != nullptr)
+        options.selection_bias = std::span<const float>(selection_bias, expert_count);
+    if (explicit_expert_ids != nullptr)
+        options.explicit_expert_ids = std::span<const uint32_t>(explicit_expert_ids, static_cast<size_t>(token_count) * top_k);
+    const std::span<const float> logits(router_logits, static_cast<size_t>(token_count) * expert_count);
+    ExpertDispatcher dispatcher;
+    ExpertDispatchPlan plan;
+    if (use_dispatch_into)
+    {
+        auto status = dispatcher.dispatch_into(logits, token_count, options, plan);
+        if (!status)
+        {
+            copy_message(status.error().message, message, message_cap);
+            return 1 + static_cast<int>(status.error().code);
+        }
+    }
+    else
+    {
+        auto dispatched = dispatcher.dispatch(logits, token_count, options);
+        if (!dispatched)
+        {
+            copy_message(dispatched.error().message, message, message_cap);
+            return 1 + static_cast<int>(dispatched.error().code);
+        }
+        plan = std::move(dispatched).value();
+    }
+    *assignment_count = plan.assignment_count;
+    uint32_t written = 0;
+    size_t batch = 0;
+    for (uint32_t expert_id = 0; expert_id < expert_count; ++expert_id)
+    {
+        expert_offsets[expert_id] = written;
+        if (batch < plan.batches.size() && plan.batches[batch].expert_id == expert_id)
+        {
+            for (const ExpertRoute& route : plan.batches[batch].routes)
+            {
+                route_tokens[written] = route.token_index;
+                route_ranks[written] = route.rank;
+                route_weights[written] = route.weight;
+                ++written;
+            }
+            ++batch;
+        }
+    }
+    expert_offsets[expert_count] = written;
+    return batch == plan.batches.size() ? 0 : -1; /* -1: batches were not in ascending expert order */
 }
 
 float ref_bfloat16_to_float(uint16_t value)

@@ -85,6 +85,11 @@ def oracle():
     lib.oracle_speculative_verify.argtypes = [
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32, ctypes.POINTER(SamplingOptions),
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    lib.oracle_router_status_message.restype = ctypes.c_char_p
+    lib.oracle_router_status_message.argtypes = [ctypes.c_int]
+    lib.oracle_router_scores.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p]
+    lib.oracle_router_dispatch.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p,
+                                           ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.oracle_bfloat16_to_float.restype = ctypes.c_float
     lib.oracle_bfloat16_to_float.argtypes = [ctypes.c_uint16]
     lib.oracle_float_to_bfloat16.restype = ctypes.c_uint16
@@ -253,6 +258,10 @@ def reference():
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
         ctypes.c_size_t, ctypes.c_uint64, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int32),
         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_uint64), ctypes.c_char_p, ctypes.c_size_t]
+    lib.ref_router_dispatch.argtypes = [
+        ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
+        ctypes.c_uint32, ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), ctypes.c_char_p, ctypes.c_size_t]
     lib.ref_bfloat16_to_float.restype = ctypes.c_float
     lib.ref_bfloat16_to_float.argtypes = [ctypes.c_uint16]
     lib.ref_float_to_bfloat16.restype = ctypes.c_uint16
@@ -327,3 +336,76 @@ def reference_candidate_probability(ids, probabilities, token_id):
     ids = np.ascontiguousarray(ids, dtype=np.int32)
     probabilities = np.ascontiguousarray(probabilities, dtype=np.float32)
     return reference().ref_candidate_probability(ids.ctypes.data, probabilities.ctypes.data, ids.size, int(token_id))
+
+
+# ---- expert router (MoE token dispatch)
+
+ROUTER_SOFTMAX, ROUTER_SIGMOID, ROUTER_SQRT_SOFTPLUS = 0, 1, 2
+ROUTER_OPTIONS_DTYPE = np.dtype([("expert_count", "<u4"), ("top_k", "<u4"), ("score_function", "<u4"),
+                                 ("renormalize", "<u4"), ("routed_scaling_factor", "<f4")])
+ROUTE_DTYPE = np.dtype([("token_index", "<u4"), ("rank", "<u4"), ("weight", "<f4")])
+ROUTER_MESSAGES = {
+    1: "expert dispatch requires at least one token",
+    2: "expert dispatch requires 0 < top_k <= expert_count",
+    3: "routed scaling factor must be finite and positive",
+    4: "router logits must be finite",
+    5: "explicit expert id is out of range",
+    6: "selected router weights have a non-positive sum",
+}
+
+
+def router_options(expert_count, top_k, score_function=ROUTER_SOFTMAX, renormalize=True, routed_scaling_factor=1.0):
+    options = np.zeros(1, dtype=ROUTER_OPTIONS_DTYPE)
+    options[0] = (expert_count, top_k, score_function, 1 if renormalize else 0, routed_scaling_factor)
+    return options
+
+
+def oracle_router_scores(logits, score_function):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    scores = np.empty_like(logits)
+    oracle().oracle_router_scores(logits.ctypes.data, logits.size, score_function, scores.ctypes.data)
+    return scores
+
+
+def oracle_router_dispatch(router_logits, top_k, score_function=ROUTER_SOFTMAX, renormalize=True,
+                           routed_scaling_factor=1.0, selection_bias=None, explicit_expert_ids=None):
+    """router_logits [tokens, experts] fp32.  Returns (status, expert_offsets[experts + 1], routes ROUTE_DTYPE)."""
+    router_logits = np.ascontiguousarray(router_logits, dtype=np.float32)
+    tokens, experts = router_logits.shape
+    options = router_options(experts, top_k, score_function, renormalize, routed_scaling_factor)
+    bias = None if selection_bias is None else np.ascontiguousarray(selection_bias, dtype=np.float32)
+    explicit = None if explicit_expert_ids is None else np.ascontiguousarray(explicit_expert_ids, dtype=np.uint32)
+    offsets = np.zeros(experts + 1, dtype=np.uint32)
+    routes = np.zeros(max(1, tokens * max(top_k, 1)), dtype=ROUTE_DTYPE)
+    status = oracle().oracle_router_dispatch(
+        router_logits.ctypes.data, tokens, options.ctypes.data, None if bias is None else bias.ctypes.data,
+        None if explicit is None else explicit.ctypes.data, offsets.ctypes.data, routes.ctypes.data)
+    count = int(offsets[-1]) if status == 0 else 0
+    return status, offsets, routes[:count].copy()
+
+
+def reference_router_dispatch(router_logits, top_k, score_function=ROUTER_SOFTMAX, normalization=1, flags=1,
+                              routed_scaling_factor=1.0, selection_bias=None, explicit_expert_ids=None,
+                              use_dispatch_into=False):
+    """The reference's own ExpertDispatcher.  Returns (rc, expert_offsets, routes ROUTE_DTYPE, message)."""
+    router_logits = np.ascontiguousarray(router_logits, dtype=np.float32)
+    tokens, experts = router_logits.shape
+    bias = None if selection_bias is None else np.ascontiguousarray(selection_bias, dtype=np.float32)
+    explicit = None if explicit_expert_ids is None else np.ascontiguousarray(explicit_expert_ids, dtype=np.uint32)
+    cap = max(1, tokens * max(top_k, 1))
+    offsets = np.zeros(experts + 1, dtype=np.uint32)
+    route_tokens = np.zeros(cap, dtype=np.uint32)
+    route_ranks = np.zeros(cap, dtype=np.uint32)
+    route_weights = np.zeros(cap, dtype=np.float32)
+    assignments = ctypes.c_uint64(0)
+    message = ctypes.create_string_buffer(256)
+    rc = reference().ref_router_dispatch(
+        router_logits.ctypes.data, tokens, experts, top_k, score_function, normalization, flags,
+        ctypes.c_float(routed_scaling_factor), None if bias is None else bias.ctypes.data,
+        None if explicit is None else explicit.ctypes.data, 1 if use_dispatch_into else 0,
+        offsets.ctypes.data, route_tokens.ctypes.data, route_ranks.ctypes.data, route_weights.ctypes.data,
+        ctypes.byref(assignments), message, 256)
+    count = int(offsets[-1]) if rc == 0 else 0
+    routes = np.zeros(count, dtype=ROUTE_DTYPE)
+    routes["token_index"], routes["rank"], routes["weight"] = route_tokens[:count], route_ranks[:count], route_weights[:count]
+    return rc, offsets, routes, message.value.decode()
