@@ -175,4 +175,10 @@ int oracle_router_dispatch(
     return ORACLE_ROUTER_OK;
 }
 
+void oracle_log1pf_libm_array(const float* in, float* out, size_t n)
+{
+    for (size_t i = 0; i < n; ++i)
+        out[i] = std::log1p(in[i]);
+}
+
 } // extern "C"

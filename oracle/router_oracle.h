@@ -72,6 +72,9 @@ int oracle_router_dispatch(
     const float* selection_bias, const uint32_t* explicit_expert_ids,
     uint32_t* expert_offsets, oracle_expert_route* routes);
 
+/* libm's log1pf over an array: what the device restatement of it is compared with. */
+void oracle_log1pf_libm_array(const float* in, float* out, size_t n);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,6 +88,8 @@ def oracle():
     lib.oracle_router_status_message.restype = ctypes.c_char_p
     lib.oracle_router_status_message.argtypes = [ctypes.c_int]
     lib.oracle_router_scores.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p]
+    lib.oracle_log1pf_libm_array.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+    lib.oracle_log1pf_libm_array.restype = None
     lib.oracle_router_dispatch.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p,
                                            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.oracle_bfloat16_to_float.restype = ctypes.c_float
@@ -358,6 +360,13 @@ def router_options(expert_count, top_k, score_function=ROUTER_SOFTMAX, renormali
     options = np.zeros(1, dtype=ROUTER_OPTIONS_DTYPE)
     options[0] = (expert_count, top_k, score_function, 1 if renormalize else 0, routed_scaling_factor)
     return options
+
+
+def log1pf_libm(values):
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty_like(values)
+    oracle().oracle_log1pf_libm_array(values.ctypes.data, out.ctypes.data, values.size)
+    return out
 
 
 def oracle_router_scores(logits, score_function):

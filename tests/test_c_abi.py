@@ -7,17 +7,21 @@ import subprocess
 
 import pytest
 
-from ncnn_moe_runtime_amd import hip_sampler
+from ncnn_moe_runtime_amd import hip_router, hip_sampler
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PACKAGE_DIR = os.path.join(ROOT, "ncnn-moe-runtime_amd")
 TEST_PROGRAM = os.path.join(PACKAGE_DIR, "test_session_sampler")
 
 
-def declared_functions():
-    text = open(os.path.join(ROOT, "include", "ncnn_moe_hip_sampler.h")).read()
+def declared_functions(header="ncnn_moe_hip_sampler.h", prefix="ncnn_moe_hip_sampler_"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(ncnn_moe_hip_sampler_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(" + prefix + r"[a-z0-9_]+)\s*\(", text)))
+
+
+def router_functions():
+    return declared_functions("ncnn_moe_hip_router.h", "ncnn_moe_hip_router_")
 
 
 def test_header_and_binding_agree():
@@ -28,6 +32,36 @@ def test_library_exports_every_declared_function():
     library = hip_sampler.load_library()
     for name in declared_functions():
         assert getattr(library, name) is not None
+
+
+def test_router_header_and_binding_agree():
+    assert router_functions() == sorted(hip_router.EXPORTED_SYMBOLS)
+    library = hip_router.load_library()
+    for name in router_functions():
+        assert getattr(library, name) is not None
+
+
+def test_router_status_messages_are_the_dispatcher_messages():
+    """src/graph/expert_dispatcher.cpp:80-103, :122, :133"""
+    expected = {
+        1: "expert dispatch requires at least one token",
+        2: "expert dispatch requires 0 < top_k <= expert_count",
+        3: "routed scaling factor must be finite and positive",
+        4: "router logits must be finite",
+        5: "explicit expert id is out of range",
+        6: "selected router weights have a non-positive sum",
+    }
+    for status, message in expected.items():
+        assert hip_router.status_message(status) == message
+    assert hip_router.status_message(0) == ""
+    assert hip_router.OPTIONS_DTYPE.itemsize == 20 and hip_router.ROUTE_DTYPE.itemsize == 12
+
+
+def test_router_create_without_gpu_fails_loudly():
+    if hip_sampler.device_count() > 0:
+        pytest.skip("a GPU is visible")
+    with pytest.raises(hip_router.RouterError):
+        hip_router.HipRouter(16)
 
 
 def test_status_messages_are_the_cpu_sampler_messages():
