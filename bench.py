@@ -176,6 +176,91 @@ def bench_speculative_verify(args, hip_sampler):
     print(json.dumps(line))
 
 
+def bench_router_dispatch(args):
+    """One expert dispatch of a MoE layer per step (ExpertDispatcher::dispatch): --rows tokens (4096 by
+    default, a prefill chunk) x 256 experts, Top-8, sqrt-softplus scores with a selection bias, scaling
+    1.5, every array resident in HBM (ncnn_moe_hip_router_dispatch_device).  Not the headline metric;
+    printed in the same JSON shape."""
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+    from ncnn_moe_runtime_amd import hip_router
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU: no HIP device is visible")
+    tokens = args.rows if args.rows > 0 else 4096
+    experts, top_k, score, scaling = 256, 8, hip_router.SQRT_SOFTPLUS, 1.5
+    rng = np.random.Generator(np.random.PCG64(88))
+    buffers = 16
+    host_logits = [(rng.standard_normal((tokens, experts), dtype=np.float32) * np.float32(2.0)) for _ in range(buffers)]
+    bias = (rng.standard_normal(experts, dtype=np.float32) * np.float32(0.1))
+    device = torch.device("cuda:0")
+    logits = [torch.from_numpy(values).to(device) for values in host_logits]
+    device_bias = torch.from_numpy(bias).to(device)
+    offsets = torch.zeros(experts + 1, dtype=torch.int32, device=device)
+    routes = torch.zeros(tokens * top_k * 3, dtype=torch.int32, device=device)
+    status = torch.zeros(1, dtype=torch.int32, device=device)
+    options = hip_router.make_options(experts, top_k, score, True, scaling)
+    router = hip_router.HipRouter(tokens, experts, top_k)
+    stream = torch.cuda.current_stream()
+
+    def step(index):
+        host_status = router.dispatch_device(
+            logits[index % buffers].data_ptr(), tokens, options, offsets.data_ptr(), routes.data_ptr(), status.data_ptr(),
+            bias_pointer=device_bias.data_ptr(), stream=stream.cuda_stream)
+        if host_status != 0:
+            sys.exit("router dispatch rejected its arguments: status %d" % host_status)
+
+    # parity of what is timed: every buffer against the oracle, bit for bit
+    mismatches = 0
+    cpu_seconds = []
+    for index in range(buffers):
+        step(index)
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        cpu_status, cpu_offsets, cpu_routes = oracle_lib.oracle_router_dispatch(
+            host_logits[index], top_k, score_function=score, routed_scaling_factor=scaling, selection_bias=bias)
+        cpu_seconds.append(time.perf_counter() - start)
+        got = routes.cpu().numpy().view(np.uint32).reshape(-1, 3)
+        same = int(status.item()) == cpu_status == 0 and np.array_equal(offsets.cpu().numpy().view(np.uint32), cpu_offsets)
+        same = same and np.array_equal(got[:, 0], cpu_routes["token_index"]) and np.array_equal(got[:, 1], cpu_routes["rank"])
+        same = same and np.array_equal(got[:, 2], cpu_routes["weight"].view(np.uint32))
+        mismatches += 0 if same else 1
+    for index in range(args.warmup):
+        step(index)
+    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start = time.perf_counter()
+    begin.record(stream)
+    for index in range(args.steps):
+        step(index)
+    end.record(stream)
+    torch.cuda.synchronize()
+    seconds_per_step = (time.perf_counter() - start) / args.steps
+    device_seconds_per_step = begin.elapsed_time(end) * 1e-3 / args.steps
+    bytes_per_step = tokens * experts * 4 + experts * 4 + tokens * top_k * 12 + (experts + 1) * 4 + 4
+    cpu_best = min(cpu_seconds)
+    line = {
+        "metric": "expert dispatch tokens/sec, %d experts Top-%d sqrt-softplus + bias, fp32 router logits" % (experts, top_k),
+        "value": tokens / seconds_per_step, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": seconds_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "expert dispatch of one MoE layer: %d tokens x %d experts, Top-%d, sqrt-softplus scores, "
+                               "selection bias, scaling %.1f; logits resident in HBM" % (tokens, experts, top_k, scaling),
+                   "entry_point": "ncnn_moe_hip_router_dispatch_device (no host synchronisation inside the timed region)"},
+        "roofline": {"bound": "hbm", "achieved": bytes_per_step / device_seconds_per_step / 1e9, "peak": HBM_PEAK_BYTES_PER_S / 1e9,
+                     "unit": "GB/s", "frac": bytes_per_step / device_seconds_per_step / HBM_PEAK_BYTES_PER_S, "traffic": None,
+                     "kernel": "router_clear_kernel + router_select_kernel + router_group_kernel, device time per dispatch "
+                               "between two events on the launch stream",
+                     "algorithmic_bytes_per_launch": bytes_per_step, "device_us_per_step": device_seconds_per_step * 1e6},
+        "parity": {"dispatches_checked": buffers, "dispatch_mismatches": mismatches},
+        "cpu_baseline": {"value": tokens / cpu_best, "unit": "tokens/s", "cores": 1, "kind": "port",
+                         "sample": "best of %d dispatches of the same %d tokens by the CPU oracle" % (buffers, tokens)},
+    }
+    router.close()
+    print(json.dumps(line))
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -196,6 +281,9 @@ def main():
 
     load_package()
     from ncnn_moe_runtime_amd import hip_sampler, workloads
+    if args.workload == "router_dispatch":
+        bench_router_dispatch(args)
+        return
     if args.workload == "speculative_verify":
         return bench_speculative_verify(args, hip_sampler)
     import torch

@@ -26,8 +26,8 @@ struct ncnn_moe_hip_router
     uint32_t* explicit_ids = nullptr;
     uint32_t* selected_experts = nullptr;
     float* selected_weights = nullptr;
-    uint32_t* expert_counts = nullptr;
-    uint32_t* error_words = nullptr;
+    uint32_t* chunk_counts = nullptr;
+    uint32_t* scratch_words = nullptr; // error words [2], finished workgroups [1]
     uint32_t* expert_offsets = nullptr;
     ncnn_moe_expert_route* routes = nullptr;
     uint32_t* status = nullptr;
@@ -74,8 +74,6 @@ void launch_select(const RouterArgs& args, hipStream_t stream)
 
 int enqueue(ncnn_moe_hip_router* r, const RouterArgs& args, hipStream_t stream)
 {
-    hipLaunchKernelGGL(router_clear_kernel, dim3((args.experts + 255) / 256), dim3(256), 0, stream,
-                       args.expert_counts, args.experts, args.error_words);
     const uint32_t slots = (args.experts + kWaveSize - 1) / kWaveSize;
     if (slots <= 1)
         launch_select<1>(args, stream);
@@ -87,8 +85,8 @@ int enqueue(ncnn_moe_hip_router* r, const RouterArgs& args, hipStream_t stream)
         launch_select<8>(args, stream);
     else
         launch_select<16>(args, stream);
-    const unsigned group_blocks = (args.experts + 1 + kRouterWavesPerBlock - 1) / kRouterWavesPerBlock;
-    hipLaunchKernelGGL(router_group_kernel, dim3(group_blocks), dim3(kRouterThreads), 0, stream, args);
+    const unsigned chunks = (args.tokens + kRouterChunkTokens - 1) / kRouterChunkTokens;
+    hipLaunchKernelGGL(router_group_kernel, dim3(chunks), dim3(kRouterThreads), 0, stream, args);
     ROUTER_HIP_CHECK(r, hipGetLastError());
     return NCNN_MOE_ROUTER_SUCCESS;
 }
@@ -139,8 +137,13 @@ int ncnn_moe_hip_router_create(int device, uint32_t max_tokens, uint32_t max_exp
     ok = ok && hipMalloc(&r->explicit_ids, assignments * sizeof(uint32_t)) == hipSuccess;
     ok = ok && hipMalloc(&r->selected_experts, assignments * sizeof(uint32_t)) == hipSuccess;
     ok = ok && hipMalloc(&r->selected_weights, assignments * sizeof(float)) == hipSuccess;
-    ok = ok && hipMalloc(&r->expert_counts, max_experts * sizeof(uint32_t)) == hipSuccess;
-    ok = ok && hipMalloc(&r->error_words, 2 * sizeof(uint32_t)) == hipSuccess;
+    const size_t chunk_counters = ((tokens + kRouterChunkTokens - 1) / kRouterChunkTokens) * max_experts;
+    ok = ok && hipMalloc(&r->chunk_counts, chunk_counters * sizeof(uint32_t)) == hipSuccess;
+    ok = ok && hipMalloc(&r->scratch_words, 3 * sizeof(uint32_t)) == hipSuccess;
+    // the kernels find these zeroed (no failing token: all ones) and leave them so
+    const uint32_t words[3] = {0u, 0xffffffffu, 0u};
+    ok = ok && hipMemset(r->chunk_counts, 0, chunk_counters * sizeof(uint32_t)) == hipSuccess;
+    ok = ok && hipMemcpy(r->scratch_words, words, sizeof(words), hipMemcpyHostToDevice) == hipSuccess;
     ok = ok && hipMalloc(&r->expert_offsets, (static_cast<size_t>(max_experts) + 1) * sizeof(uint32_t)) == hipSuccess;
     ok = ok && hipMalloc(&r->routes, assignments * sizeof(ncnn_moe_expert_route)) == hipSuccess;
     ok = ok && hipMalloc(&r->status, sizeof(uint32_t)) == hipSuccess;
@@ -165,8 +168,8 @@ void ncnn_moe_hip_router_destroy(ncnn_moe_hip_router* r)
         (void)hipStreamSynchronize(r->stream);
         (void)hipStreamDestroy(r->stream);
     }
-    void* buffers[] = {r->logits, r->bias, r->explicit_ids, r->selected_experts, r->selected_weights, r->expert_counts,
-                       r->error_words, r->expert_offsets, r->routes, r->status};
+    void* buffers[] = {r->logits, r->bias, r->explicit_ids, r->selected_experts, r->selected_weights, r->chunk_counts,
+                       r->scratch_words, r->expert_offsets, r->routes, r->status};
     for (void* buffer : buffers)
     {
         if (buffer != nullptr)
@@ -207,8 +210,9 @@ int ncnn_moe_hip_router_dispatch_device(
     args.scaling = options->routed_scaling_factor;
     args.selected_experts = r->selected_experts;
     args.selected_weights = r->selected_weights;
-    args.expert_counts = r->expert_counts;
-    args.error_words = r->error_words;
+    args.chunk_counts = r->chunk_counts;
+    args.error_words = r->scratch_words;
+    args.finished_chunks = r->scratch_words + 2;
     args.expert_offsets = device_expert_offsets;
     args.routes = device_routes;
     args.status = device_status;

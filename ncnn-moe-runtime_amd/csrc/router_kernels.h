@@ -1,6 +1,6 @@
 // Expert router kernels (src/graph/expert_dispatcher.cpp:12-157 of the runtime, on the device):
 //   router_select_kernel  one wave per token: scores, Top-K routes, normalised weights
-//   router_group_kernel   one wave per expert: the expert's routes, by token then rank
+//   router_group_kernel   one workgroup per 256 tokens: their routes to their places in the plan
 #ifndef NCNN_MOE_HIP_ROUTER_KERNELS_H
 #define NCNN_MOE_HIP_ROUTER_KERNELS_H
 
@@ -11,6 +11,7 @@ namespace ncnn_moe_hip {
 
 constexpr int kRouterWavesPerBlock = 4;
 constexpr int kRouterThreads = kRouterWavesPerBlock * kWaveSize;
+constexpr int kRouterChunkTokens = kRouterThreads; // tokens whose routes one workgroup of the grouping kernel places
 
 // log1pf bit-identical to glibc 2.35's (sysdeps/ieee754/flt-32/s_log1pf.c) for finite x > 0, which is
 // all stable_softplus hands it (an exponential).  Plain fp32 operations in the library's order; built
@@ -20,51 +21,34 @@ __device__ __forceinline__ float log1pf_libm_positive(float x)
     const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f;
     const float Lp1 = 6.6666668653e-01f, Lp2 = 4.0000000596e-01f, Lp3 = 2.8571429849e-01f, Lp4 = 2.2222198546e-01f,
                 Lp5 = 1.8183572590e-01f, Lp6 = 1.5313838422e-01f, Lp7 = 1.4798198640e-01f;
-    float f = 0.0f, c = 0.0f, u;
-    int32_t k = 1, hu = 0;
     const int32_t hx = static_cast<int32_t>(__float_as_uint(x));
-    if (hx < 0x3ed413d7) // x < 0.41422
+    if (hx < 0x31000000) // x < 2^-29
     {
-        if (hx < 0x31000000) // x < 2^-29
-        {
-            if (hx < 0x24800000) // x < 2^-54
-                return x;
-            return x - x * x * 0.5f;
-        }
-        k = 0;
-        f = x;
-        hu = 1;
+        if (hx < 0x24800000) // x < 2^-54
+            return x;
+        return x - x * x * 0.5f;
     }
     if (hx >= 0x7f800000)
         return x + x;
-    if (k != 0)
-    {
-        if (hx < 0x5a000000)
-        {
-            u = 1.0f + x;
-            hu = static_cast<int32_t>(__float_as_uint(u));
-            k = (hu >> 23) - 127;
-            c = (k > 0) ? 1.0f - (u - x) : x - (u - 1.0f); // correction term
-            c /= u;
-        }
-        else
-        {
-            u = x;
-            hu = static_cast<int32_t>(__float_as_uint(u));
-            k = (hu >> 23) - 127;
-            c = 0.0f;
-        }
-        hu &= 0x007fffff;
-        if (hu < 0x3504f7)
-            u = __uint_as_float(static_cast<uint32_t>(hu) | 0x3f800000u); // normalise u
-        else
-        {
-            k += 1;
-            u = __uint_as_float(static_cast<uint32_t>(hu) | 0x3f000000u); // normalise u / 2
-            hu = (0x00800000 - hu) >> 2;
-        }
-        f = u - 1.0f;
-    }
+    // The library's three range cases (x < 0.41422: no reduction; x < 2^53: reduce 1 + x and keep the
+    // rounding error of the sum as a correction; above: reduce x itself) as selects, so that lanes in
+    // different ranges share one instruction stream.
+    const bool direct = hx < 0x3ed413d7;
+    const bool huge = hx >= 0x5a000000;
+    float u = huge ? x : 1.0f + x;
+    int32_t hu = static_cast<int32_t>(__float_as_uint(u));
+    int32_t k = (hu >> 23) - 127;
+    float c = (k > 0) ? 1.0f - (u - x) : x - (u - 1.0f); // correction term
+    c = huge ? 0.0f : c / u;
+    hu &= 0x007fffff;
+    const bool low_half = hu < 0x3504f7;
+    u = __uint_as_float(static_cast<uint32_t>(hu) | (low_half ? 0x3f800000u : 0x3f000000u)); // u, or u / 2
+    k = low_half ? k : k + 1;
+    hu = low_half ? hu : (0x00800000 - hu) >> 2;
+    float f = u - 1.0f;
+    k = direct ? 0 : k;
+    f = direct ? x : f;
+    hu = direct ? 1 : hu;
     const float hfsq = 0.5f * f * f;
     const float kf = static_cast<float>(k);
     if (hu == 0) // |f| < 2^-20
@@ -84,9 +68,40 @@ __device__ __forceinline__ float log1pf_libm_positive(float x)
     const float s = f / (2.0f + f);
     const float z = s * s;
     const float R = z * (Lp1 + z * (Lp2 + z * (Lp3 + z * (Lp4 + z * (Lp5 + z * (Lp6 + z * Lp7))))));
-    if (k == 0)
-        return f - (hfsq - s * (hfsq + R));
-    return kf * ln2_hi - ((hfsq - (s * (hfsq + R) + (kf * ln2_lo + c))) - f);
+    const float near = f - (hfsq - s * (hfsq + R));
+    const float far = kf * ln2_hi - ((hfsq - (s * (hfsq + R) + (kf * ln2_lo + c))) - f);
+    return k == 0 ? near : far;
+}
+
+// Wave-wide reductions through the data-parallel primitives: four exchanges inside each row of 16
+// lanes (lane pairs at distance 1 and 2, then the two mirrors), then the four rows through scalar reads.
+template <int CONTROL>
+__device__ __forceinline__ int dpp_move(int value)
+{
+    return __builtin_amdgcn_mov_dpp(value, CONTROL, 0xf, 0xf, true);
+}
+
+constexpr int kDppSwapPairs = 0xB1;   // quad_perm:[1,0,3,2]
+constexpr int kDppSwapHalves = 0x4E;  // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // row_half_mirror
+constexpr int kDppMirror = 0x140;     // row_mirror
+
+__device__ __forceinline__ float wave_max(float value)
+{
+    value = fmaxf(value, __int_as_float(dpp_move<kDppSwapPairs>(__float_as_int(value))));
+    value = fmaxf(value, __int_as_float(dpp_move<kDppSwapHalves>(__float_as_int(value))));
+    value = fmaxf(value, __int_as_float(dpp_move<kDppHalfMirror>(__float_as_int(value))));
+    value = fmaxf(value, __int_as_float(dpp_move<kDppMirror>(__float_as_int(value))));
+    return fmaxf(fmaxf(read_lane(value, 0), read_lane(value, 16)), fmaxf(read_lane(value, 32), read_lane(value, 48)));
+}
+
+__device__ __forceinline__ int wave_min(int value)
+{
+    value = min(value, dpp_move<kDppSwapPairs>(value));
+    value = min(value, dpp_move<kDppSwapHalves>(value));
+    value = min(value, dpp_move<kDppHalfMirror>(value));
+    value = min(value, dpp_move<kDppMirror>(value));
+    return min(min(read_lane(value, 0), read_lane(value, 16)), min(read_lane(value, 32), read_lane(value, 48)));
 }
 
 // score_router_logit (src/graph/expert_dispatcher.cpp:24-38)
@@ -117,8 +132,9 @@ struct RouterArgs
     float scaling;
     uint32_t* selected_experts;   // [tokens][top_k], rank order
     float* selected_weights;      // [tokens][top_k]
-    uint32_t* expert_counts;      // [experts], zero at launch
+    uint32_t* chunk_counts;       // [chunks][experts] assignments per chunk of 256 tokens and expert, zero at launch
     uint32_t* error_words;        // [0]: non-finite logit seen, [1]: min over failing tokens of (token << 3 | status), ~0 if none
+    uint32_t* finished_chunks;    // workgroups of the grouping kernel that are done, zero at launch
     uint32_t* expert_offsets;     // [experts + 1]
     ncnn_moe_expert_route* routes; // [tokens * top_k]
     uint32_t* status;             // the call's ncnn_moe_router_status
@@ -126,13 +142,12 @@ struct RouterArgs
 
 struct RouterShared
 {
-    float scores[kRouterWavesPerBlock][NCNN_MOE_ROUTER_MAX_EXPERTS];
-    uint32_t chosen[kRouterWavesPerBlock][NCNN_MOE_ROUTER_MAX_TOP_K];
+    float scores[kRouterWavesPerBlock][NCNN_MOE_ROUTER_MAX_EXPERTS]; // a token's scores, for the caller-named experts
 };
 
 // One wave per token.  Expert e lives in slot e / 64 of lane e % 64, so a loop over slots, then lanes,
-// visits the experts in index order: the softmax sum and the sum of the selected scores are the CPU
-// loops themselves, one fp32 addition at a time.
+// visits the experts in index order: the softmax sum is the CPU loop itself, one fp32 addition at a
+// time.  The routes are chosen one per round and stay in registers: lane r keeps the route of rank r.
 template <int SLOTS>
 __global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArgs r)
 {
@@ -143,16 +158,28 @@ __global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArg
     if (token >= r.tokens)
         return;
     const int experts = static_cast<int>(r.experts);
+    const int top_k = static_cast<int>(r.top_k);
     const float* logits = r.logits + static_cast<size_t>(token) * r.experts;
+    const bool explicit_routes = r.explicit_ids != nullptr;
 
+    // every load of the token up front
     float logit[SLOTS];
+    float bias[SLOTS];
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+    {
+        const int e = s * kWaveSize + lane;
+        logit[s] = e < experts ? logits[e] : 0.0f;
+        bias[s] = (e < experts && r.selection_bias != nullptr && !explicit_routes) ? r.selection_bias[e] : 0.0f;
+    }
+    uint32_t my_expert = (explicit_routes && lane < top_k) ? r.explicit_ids[static_cast<size_t>(token) * r.top_k + lane] : 0u;
+
     bool finite = true;
     float maximum = -__builtin_inff();
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s)
     {
         const int e = s * kWaveSize + lane;
-        logit[s] = e < experts ? logits[e] : 0.0f;
         if (e < experts)
         {
             finite = finite && is_finite_f32(logit[s]);
@@ -171,9 +198,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArg
     float score[SLOTS];
     if (r.score_function == NCNN_MOE_ROUTER_SOFTMAX)
     {
-#pragma unroll
-        for (int step = 1; step < kWaveSize; step <<= 1)
-            maximum = fmaxf(maximum, __shfl_xor(maximum, step, kWaveSize));
+        maximum = wave_max(maximum);
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
             score[s] = (s * kWaveSize + lane) < experts ? expf_libm(logit[s] - maximum) : 0.0f;
@@ -195,85 +220,79 @@ __global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArg
         for (int s = 0; s < SLOTS; ++s)
             score[s] = (s * kWaveSize + lane) < experts ? router_score_of_logit(logit[s], r.score_function) : 0.0f;
     }
-#pragma unroll
-    for (int s = 0; s < SLOTS; ++s)
-    {
-        const int e = s * kWaveSize + lane;
-        if (e < experts)
-            shared.scores[wave][e] = score[s];
-    }
 
-    const int top_k = static_cast<int>(r.top_k);
-    if (r.explicit_ids != nullptr)
+    float my_score = 0.0f;
+    float selected_sum = 0.0f;
+    if (explicit_routes)
     {
         // src/graph/expert_dispatcher.cpp:124-135: the caller names the experts; rank = position
-        bool in_range = true;
-        if (lane < top_k)
-        {
-            const uint32_t expert = r.explicit_ids[static_cast<size_t>(token) * r.top_k + lane];
-            in_range = expert < r.experts;
-            shared.chosen[wave][lane] = expert;
-        }
+        const bool in_range = lane >= top_k || my_expert < r.experts;
         if (__ballot(!in_range) != 0)
         {
             if (lane == 0)
                 atomicMin(&r.error_words[1], (token << 3) | NCNN_MOE_ROUTER_EXPERT_OUT_OF_RANGE);
             return;
         }
-    }
-    else
-    {
-        // ---- select_topk_routes (src/graph/expert_dispatcher.cpp:61-77): the best top_k by
-        // (score + bias descending, expert id ascending), found one per round
-        float keyed[SLOTS];
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
         {
             const int e = s * kWaveSize + lane;
-            keyed[s] = score[s] + ((r.selection_bias == nullptr || e >= experts) ? 0.0f : r.selection_bias[e]);
+            if (e < experts)
+                shared.scores[wave][e] = score[s];
         }
+        __builtin_amdgcn_s_waitcnt(0xc07f); // this wave's LDS writes, before its lanes read them back
+        __builtin_amdgcn_wave_barrier();
+        if (lane < top_k)
+            my_score = shared.scores[wave][my_expert];
+        for (int rank = 0; rank < top_k; ++rank)
+            selected_sum += read_lane(my_score, rank);
+    }
+    else
+    {
+        // ---- select_topk_routes (src/graph/expert_dispatcher.cpp:61-77): the best top_k by
+        // (score + bias descending, expert id ascending), one per round; the selected scores are
+        // summed in rank order (src/graph/expert_dispatcher.cpp:137-143)
+        float keyed[SLOTS];
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s)
+            keyed[s] = score[s] + bias[s];
         uint32_t taken = 0; // this lane's slots already selected
         for (int round = 0; round < top_k; ++round)
         {
-            float best = 0.0f;
-            int best_expert = 0x7fffffff; // none
+            // this lane's best remaining expert: the lowest slot (lowest id) among equals
+            float lane_best = -__builtin_inff();
+            float lane_score = 0.0f;
+            int lane_expert = 0x7fffffff; // none
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s)
             {
                 const int e = s * kWaveSize + lane;
                 const bool available = e < experts && ((taken >> s) & 1u) == 0u;
-                if (available && (best_expert == 0x7fffffff || keyed[s] > best))
+                if (available && (lane_expert == 0x7fffffff || keyed[s] > lane_best))
                 {
-                    best = keyed[s];
-                    best_expert = e;
+                    lane_best = keyed[s];
+                    lane_score = score[s];
+                    lane_expert = e;
                 }
             }
-#pragma unroll
-            for (int step = 1; step < kWaveSize; step <<= 1)
+            const float best = wave_max(lane_best);
+            int winner = wave_min((lane_expert != 0x7fffffff && lane_best == best) ? lane_expert : 0x7fffffff);
+            if (winner == 0x7fffffff) // selection scores that compare unordered: any remaining expert
+                winner = wave_min(lane_expert);
+            const int winner_lane = winner & (kWaveSize - 1);
+            const float winner_score = read_lane(lane_score, winner_lane);
+            if (lane == winner_lane)
+                taken |= 1u << (winner >> 6);
+            selected_sum += winner_score;
+            if (lane == round)
             {
-                const float other = __shfl_xor(best, step, kWaveSize);
-                const int other_expert = __shfl_xor(best_expert, step, kWaveSize);
-                const bool other_wins = other_expert != 0x7fffffff &&
-                    (best_expert == 0x7fffffff || other > best || (other == best && other_expert < best_expert));
-                if (other_wins)
-                {
-                    best = other;
-                    best_expert = other_expert;
-                }
+                my_expert = static_cast<uint32_t>(winner);
+                my_score = winner_score;
             }
-            if ((best_expert & (kWaveSize - 1)) == lane)
-                taken |= 1u << (best_expert >> 6);
-            if (lane == 0)
-                shared.chosen[wave][round] = static_cast<uint32_t>(best_expert);
         }
     }
-    __builtin_amdgcn_s_waitcnt(0xc07f); // this wave's LDS writes, before its lanes read them back
-    __builtin_amdgcn_wave_barrier();
 
-    // ---- src/graph/expert_dispatcher.cpp:137-150: the selected scores are summed in rank order
-    float selected_sum = 0.0f;
-    for (int rank = 0; rank < top_k; ++rank)
-        selected_sum += shared.scores[wave][shared.chosen[wave][rank]];
+    // ---- src/graph/expert_dispatcher.cpp:144-150
     if (r.renormalize != 0u && selected_sum <= 0.0f)
     {
         if (lane == 0)
@@ -282,24 +301,53 @@ __global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArg
     }
     if (lane < top_k)
     {
-        const uint32_t expert = shared.chosen[wave][lane];
-        const float expert_score = shared.scores[wave][expert];
-        const float weight = (r.renormalize != 0u ? expert_score / selected_sum : expert_score) * r.scaling;
-        r.selected_experts[static_cast<size_t>(token) * r.top_k + lane] = expert;
+        const float weight = (r.renormalize != 0u ? my_score / selected_sum : my_score) * r.scaling;
+        r.selected_experts[static_cast<size_t>(token) * r.top_k + lane] = my_expert;
         r.selected_weights[static_cast<size_t>(token) * r.top_k + lane] = weight;
-        atomicAdd(&r.expert_counts[expert], 1u);
+        atomicAdd(&r.chunk_counts[static_cast<size_t>(token / kRouterChunkTokens) * r.experts + my_expert], 1u);
     }
 }
 
-// One wave per expert: its offset is the sum of the counts of the experts before it; its routes are
-// the assignments that name it, in (token, rank) order, which is the order of the flat array.
-// Wave 0 of the grid also settles the call's status.
+// Grouping is a stable counting sort of the flat assignment array (token-major, so already in
+// (token, rank) order) by expert id.  The select kernel counts assignments per (chunk of 256 tokens,
+// expert); one workgroup per chunk then places its chunk's routes:
+//   position = routes of lower experts (all chunks) + this expert's routes in earlier chunks
+//              + this expert's routes earlier in the chunk.
+// The last workgroup to finish returns the scratch counters to zero for the next call.
+struct GroupShared
+{
+    uint32_t wave_base[kRouterWavesPerBlock][NCNN_MOE_ROUTER_MAX_EXPERTS];
+    uint32_t wave_totals[kRouterWavesPerBlock];
+    uint32_t is_last;
+};
+
+constexpr int kGroupExpertsPerThread = NCNN_MOE_ROUTER_MAX_EXPERTS / kRouterThreads; // experts one thread owns, at most
+constexpr int kGroupBatch = 8;                                                       // loads in flight per lane
+
 __global__ __launch_bounds__(kRouterThreads) void router_group_kernel(RouterArgs r)
 {
-    const int lane = threadIdx.x & (kWaveSize - 1);
-    const uint32_t expert = blockIdx.x * kRouterWavesPerBlock + (threadIdx.x >> 6);
-    if (expert > r.experts)
-        return;
+    __shared__ GroupShared shared;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const uint32_t chunk = blockIdx.x;
+    const uint32_t chunks = gridDim.x;
+    const uint32_t experts = r.experts;
+
+    // this wave's 64 tokens of the chunk; the first loads go out before anything waits
+    const uint32_t first_token = chunk * kRouterChunkTokens + static_cast<uint32_t>(wave) * kWaveSize;
+    const uint32_t wave_tokens = first_token < r.tokens ? min(static_cast<uint32_t>(kWaveSize), r.tokens - first_token) : 0u;
+    const uint32_t first_assignment = first_token * r.top_k;
+    const uint32_t count = wave_tokens * r.top_k;
+    uint32_t first_named[kGroupBatch];
+    float first_weight[kGroupBatch];
+#pragma unroll
+    for (int k = 0; k < kGroupBatch; ++k)
+    {
+        const uint32_t i = static_cast<uint32_t>(k * kWaveSize + lane);
+        first_named[k] = i < count ? r.selected_experts[first_assignment + i] : 0xffffffffu;
+        first_weight[k] = i < count ? r.selected_weights[first_assignment + i] : 0.0f;
+    }
     const uint32_t non_finite = r.error_words[0];
     const uint32_t first_bad = r.error_words[1];
     uint32_t status = NCNN_MOE_ROUTER_OK;
@@ -307,65 +355,175 @@ __global__ __launch_bounds__(kRouterThreads) void router_group_kernel(RouterArgs
         status = NCNN_MOE_ROUTER_NON_FINITE_LOGIT;
     else if (first_bad != 0xffffffffu)
         status = first_bad & 7u;
-    uint32_t before = 0;
-    for (uint32_t e = lane; e < expert; e += kWaveSize)
-        before += r.expert_counts[e];
-#pragma unroll
-    for (int step = 1; step < kWaveSize; step <<= 1)
-        before += __shfl_xor(before, step, kWaveSize);
-    if (expert == r.experts)
-    {
-        // the extra wave writes the end of the last group and the status
-        if (lane == 0)
-        {
-            r.expert_offsets[r.experts] = status == NCNN_MOE_ROUTER_OK ? before : 0u;
-            *r.status = status;
-        }
-        return;
-    }
-    if (lane == 0)
-        r.expert_offsets[expert] = status == NCNN_MOE_ROUTER_OK ? before : 0u;
-    if (status != NCNN_MOE_ROUTER_OK)
-        return;
-    const uint32_t assignments = r.tokens * r.top_k;
-    uint32_t written = before;
-    for (uint32_t first = 0; first < assignments; first += 4u * kWaveSize)
-    {
-        uint32_t named[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-        {
-            const uint32_t i = first + static_cast<uint32_t>(k * kWaveSize + lane);
-            named[k] = i < assignments ? r.selected_experts[i] : 0xffffffffu;
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-        {
-            const uint32_t i = first + static_cast<uint32_t>(k * kWaveSize + lane);
-            const bool mine = named[k] == expert;
-            const uint64_t matches = __ballot(mine);
-            if (mine)
-            {
-                ncnn_moe_expert_route route;
-                route.token_index = i / r.top_k;
-                route.rank = i - route.token_index * r.top_k;
-                route.weight = r.selected_weights[i];
-                r.routes[written + static_cast<uint32_t>(lanes_below(matches))] = route;
-            }
-            written += static_cast<uint32_t>(__popcll(matches));
-        }
-    }
-}
+    if (chunk == 0 && tid == 0)
+        *r.status = status;
 
-__global__ void router_clear_kernel(uint32_t* expert_counts, uint32_t experts, uint32_t* error_words)
-{
-    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < experts)
-        expert_counts[i] = 0u;
-    if (i == 0)
+    if (status != NCNN_MOE_ROUTER_OK)
     {
-        error_words[0] = 0u;
-        error_words[1] = 0xffffffffu;
+        if (chunk == 0)
+        {
+            for (uint32_t e = tid; e <= experts; e += kRouterThreads)
+                r.expert_offsets[e] = 0u;
+        }
+    }
+    else
+    {
+        // ---- this thread's experts: their routes in all chunks, and in the chunks before this one
+        const uint32_t per_thread = (experts + kRouterThreads - 1) / kRouterThreads;
+        uint32_t total[kGroupExpertsPerThread];
+        uint32_t before[kGroupExpertsPerThread];
+#pragma unroll
+        for (int j = 0; j < kGroupExpertsPerThread; ++j)
+        {
+            total[j] = 0u;
+            before[j] = 0u;
+        }
+#pragma unroll 8
+        for (uint32_t c = 0; c < chunks; ++c)
+        {
+#pragma unroll
+            for (int j = 0; j < kGroupExpertsPerThread; ++j)
+            {
+                const uint32_t e = tid * per_thread + j;
+                const uint32_t routed = (static_cast<uint32_t>(j) < per_thread && e < experts) ? r.chunk_counts[c * experts + e] : 0u;
+                total[j] += routed;
+                before[j] += c < chunk ? routed : 0u;
+            }
+        }
+        uint32_t thread_sum = 0u;
+#pragma unroll
+        for (int j = 0; j < kGroupExpertsPerThread; ++j)
+            thread_sum += total[j];
+        uint32_t inclusive = thread_sum;
+#pragma unroll
+        for (int step = 1; step < kWaveSize; step <<= 1)
+        {
+            const uint32_t other = __shfl_up(inclusive, step, kWaveSize);
+            inclusive += lane >= step ? other : 0u;
+        }
+        if (lane == kWaveSize - 1)
+            shared.wave_totals[wave] = inclusive;
+
+        // ---- a histogram of the experts of this wave's tokens
+        for (uint32_t e = lane; e < experts; e += kWaveSize)
+            shared.wave_base[wave][e] = 0u;
+        lds_barrier();
+        for (uint32_t first = 0; first < count; first += kGroupBatch * kWaveSize)
+        {
+            uint32_t named[kGroupBatch];
+#pragma unroll
+            for (int k = 0; k < kGroupBatch; ++k)
+            {
+                const uint32_t i = first + static_cast<uint32_t>(k * kWaveSize + lane);
+                named[k] = first_named[k];
+                if (first != 0u)
+                    named[k] = i < count ? r.selected_experts[first_assignment + i] : 0xffffffffu;
+            }
+#pragma unroll
+            for (int k = 0; k < kGroupBatch; ++k)
+            {
+                if (named[k] != 0xffffffffu)
+                    atomicAdd(&shared.wave_base[wave][named[k]], 1u);
+            }
+        }
+        __syncthreads();
+        uint32_t exclusive = inclusive - thread_sum;
+        for (int w = 0; w < wave; ++w)
+            exclusive += shared.wave_totals[w];
+        // ---- first position of each of this thread's experts for each wave of this chunk
+#pragma unroll
+        for (int j = 0; j < kGroupExpertsPerThread; ++j)
+        {
+            const uint32_t e = tid * per_thread + j;
+            if (static_cast<uint32_t>(j) < per_thread && e < experts)
+            {
+                if (chunk == 0)
+                    r.expert_offsets[e] = exclusive;
+                uint32_t running = exclusive + before[j];
+#pragma unroll
+                for (int w = 0; w < kRouterWavesPerBlock; ++w)
+                {
+                    const uint32_t here = shared.wave_base[w][e];
+                    shared.wave_base[w][e] = running;
+                    running += here;
+                }
+            }
+            exclusive += total[j];
+        }
+        if (chunk == 0 && tid == 0)
+            r.expert_offsets[experts] = r.tokens * r.top_k;
+        __syncthreads();
+
+        // ---- place the wave's routes, 64 at a time in assignment order
+        const int bits = 32 - __clz(static_cast<int>(experts - 1u) | 1);
+        for (uint32_t first = 0; first < count; first += kGroupBatch * kWaveSize)
+        {
+            uint32_t named[kGroupBatch];
+            float weight[kGroupBatch];
+#pragma unroll
+            for (int k = 0; k < kGroupBatch; ++k)
+            {
+                const uint32_t i = first + static_cast<uint32_t>(k * kWaveSize + lane);
+                named[k] = first_named[k];
+                weight[k] = first_weight[k];
+                if (first != 0u)
+                {
+                    named[k] = i < count ? r.selected_experts[first_assignment + i] : 0xffffffffu;
+                    weight[k] = i < count ? r.selected_weights[first_assignment + i] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < kGroupBatch; ++k)
+            {
+                if (first + static_cast<uint32_t>(k * kWaveSize) >= count)
+                    break;
+                const bool valid = named[k] != 0xffffffffu;
+                uint64_t same = __ballot(valid);
+                for (int b = 0; b < bits; ++b)
+                {
+                    const bool set = ((named[k] >> b) & 1u) != 0u;
+                    const uint64_t vote = __ballot(set);
+                    same &= set ? vote : ~vote;
+                }
+                if (valid)
+                {
+                    const uint32_t earlier = static_cast<uint32_t>(lanes_below(same));
+                    const uint32_t position = shared.wave_base[wave][named[k]] + earlier;
+                    if (earlier == 0u)
+                        shared.wave_base[wave][named[k]] = position + static_cast<uint32_t>(__popcll(same));
+                    const uint32_t i = first_assignment + first + static_cast<uint32_t>(k * kWaveSize + lane);
+                    ncnn_moe_expert_route route;
+                    route.token_index = i / r.top_k;
+                    route.rank = i - route.token_index * r.top_k;
+                    route.weight = weight[k];
+                    r.routes[position] = route;
+                }
+                // the group leaders' updates, before this wave's next 64 read them (waves run different
+                // numbers of rounds: nothing here may wait for another wave)
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    }
+
+    // ---- the last workgroup to get here clears the counters for the next call
+    __syncthreads();
+    if (tid == 0)
+    {
+        const uint32_t finished = __hip_atomic_fetch_add(r.finished_chunks, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        shared.is_last = finished == chunks - 1u ? 1u : 0u;
+    }
+    __syncthreads();
+    if (shared.is_last != 0u)
+    {
+        for (uint32_t i = tid; i < chunks * experts; i += kRouterThreads)
+            r.chunk_counts[i] = 0u;
+        if (tid == 0)
+        {
+            r.error_words[0] = 0u;
+            r.error_words[1] = 0xffffffffu;
+            *r.finished_chunks = 0u;
+        }
     }
 }
 
