@@ -12,6 +12,10 @@ against the 8 TB/s HBM peak using the algorithmic bytes of a launch and the aver
 measured with HIP events on the launch stream.  `cpu_baseline` times the reference's own
 Session::sample loop (oracle/_ref, kind "reference") or, where that library is absent, the CPU
 oracle (kind "port") on the host cores, on the same rows.
+
+--workload speculative_verify and --workload router_dispatch time the two other entry points (one
+verification step of speculative generation; one expert dispatch of a MoE layer) in the same JSON
+shape; they are not the headline metric.
 """
 import argparse
 import ctypes

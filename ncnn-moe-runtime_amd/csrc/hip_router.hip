@@ -27,7 +27,7 @@ struct ncnn_moe_hip_router
     uint32_t* selected_experts = nullptr;
     float* selected_weights = nullptr;
     uint32_t* chunk_counts = nullptr;
-    uint32_t* scratch_words = nullptr; // error words [2], finished workgroups [1]
+    uint32_t* scratch_words = nullptr; // error words [2], finished workgroups of the two kernels [2]
     uint32_t* expert_offsets = nullptr;
     ncnn_moe_expert_route* routes = nullptr;
     uint32_t* status = nullptr;
@@ -69,7 +69,15 @@ template <int SLOTS>
 void launch_select(const RouterArgs& args, hipStream_t stream)
 {
     const unsigned blocks = (args.tokens + kRouterWavesPerBlock - 1) / kRouterWavesPerBlock;
-    hipLaunchKernelGGL(router_select_kernel<SLOTS>, dim3(blocks), dim3(kRouterThreads), 0, stream, args);
+    if (args.tokens <= static_cast<uint32_t>(kRouterChunkTokens))
+    {
+        // one chunk of tokens: the select kernel's last workgroup places the routes itself
+        hipLaunchKernelGGL((router_select_kernel<SLOTS, true>), dim3(blocks), dim3(kRouterThreads), 0, stream, args);
+        return;
+    }
+    hipLaunchKernelGGL((router_select_kernel<SLOTS, false>), dim3(blocks), dim3(kRouterThreads), 0, stream, args);
+    const unsigned chunks = (args.tokens + kRouterChunkTokens - 1) / kRouterChunkTokens;
+    hipLaunchKernelGGL(router_group_kernel, dim3(chunks), dim3(kRouterThreads), 0, stream, args);
 }
 
 int enqueue(ncnn_moe_hip_router* r, const RouterArgs& args, hipStream_t stream)
@@ -85,8 +93,6 @@ int enqueue(ncnn_moe_hip_router* r, const RouterArgs& args, hipStream_t stream)
         launch_select<8>(args, stream);
     else
         launch_select<16>(args, stream);
-    const unsigned chunks = (args.tokens + kRouterChunkTokens - 1) / kRouterChunkTokens;
-    hipLaunchKernelGGL(router_group_kernel, dim3(chunks), dim3(kRouterThreads), 0, stream, args);
     ROUTER_HIP_CHECK(r, hipGetLastError());
     return NCNN_MOE_ROUTER_SUCCESS;
 }
@@ -139,9 +145,9 @@ int ncnn_moe_hip_router_create(int device, uint32_t max_tokens, uint32_t max_exp
     ok = ok && hipMalloc(&r->selected_weights, assignments * sizeof(float)) == hipSuccess;
     const size_t chunk_counters = ((tokens + kRouterChunkTokens - 1) / kRouterChunkTokens) * max_experts;
     ok = ok && hipMalloc(&r->chunk_counts, chunk_counters * sizeof(uint32_t)) == hipSuccess;
-    ok = ok && hipMalloc(&r->scratch_words, 3 * sizeof(uint32_t)) == hipSuccess;
+    ok = ok && hipMalloc(&r->scratch_words, 4 * sizeof(uint32_t)) == hipSuccess;
     // the kernels find these zeroed (no failing token: all ones) and leave them so
-    const uint32_t words[3] = {0u, 0xffffffffu, 0u};
+    const uint32_t words[4] = {0u, 0xffffffffu, 0u, 0u};
     ok = ok && hipMemset(r->chunk_counts, 0, chunk_counters * sizeof(uint32_t)) == hipSuccess;
     ok = ok && hipMemcpy(r->scratch_words, words, sizeof(words), hipMemcpyHostToDevice) == hipSuccess;
     ok = ok && hipMalloc(&r->expert_offsets, (static_cast<size_t>(max_experts) + 1) * sizeof(uint32_t)) == hipSuccess;
@@ -213,6 +219,7 @@ int ncnn_moe_hip_router_dispatch_device(
     args.chunk_counts = r->chunk_counts;
     args.error_words = r->scratch_words;
     args.finished_chunks = r->scratch_words + 2;
+    args.finished_selects = r->scratch_words + 3;
     args.expert_offsets = device_expert_offsets;
     args.routes = device_routes;
     args.status = device_status;

@@ -135,6 +135,7 @@ struct RouterArgs
     uint32_t* chunk_counts;       // [chunks][experts] assignments per chunk of 256 tokens and expert, zero at launch
     uint32_t* error_words;        // [0]: non-finite logit seen, [1]: min over failing tokens of (token << 3 | status), ~0 if none
     uint32_t* finished_chunks;    // workgroups of the grouping kernel that are done, zero at launch
+    uint32_t* finished_selects;   // workgroups of the fused select kernel that are done, zero at launch
     uint32_t* expert_offsets;     // [experts + 1]
     ncnn_moe_expert_route* routes; // [tokens * top_k]
     uint32_t* status;             // the call's ncnn_moe_router_status
@@ -149,14 +150,8 @@ struct RouterShared
 // visits the experts in index order: the softmax sum is the CPU loop itself, one fp32 addition at a
 // time.  The routes are chosen one per round and stay in registers: lane r keeps the route of rank r.
 template <int SLOTS>
-__global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArgs r)
+__device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterShared& shared, uint32_t token, int lane, int wave)
 {
-    __shared__ RouterShared shared;
-    const int lane = threadIdx.x & (kWaveSize - 1);
-    const int wave = threadIdx.x >> 6;
-    const uint32_t token = blockIdx.x * kRouterWavesPerBlock + wave;
-    if (token >= r.tokens)
-        return;
     const int experts = static_cast<int>(r.experts);
     const int top_k = static_cast<int>(r.top_k);
     const float* logits = r.logits + static_cast<size_t>(token) * r.experts;
@@ -324,14 +319,11 @@ struct GroupShared
 constexpr int kGroupExpertsPerThread = NCNN_MOE_ROUTER_MAX_EXPERTS / kRouterThreads; // experts one thread owns, at most
 constexpr int kGroupBatch = 8;                                                       // loads in flight per lane
 
-__global__ __launch_bounds__(kRouterThreads) void router_group_kernel(RouterArgs r)
+__device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupShared& shared, uint32_t chunk, uint32_t chunks)
 {
-    __shared__ GroupShared shared;
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
-    const uint32_t chunk = blockIdx.x;
-    const uint32_t chunks = gridDim.x;
     const uint32_t experts = r.experts;
 
     // this wave's 64 tokens of the chunk; the first loads go out before anything waits
@@ -510,7 +502,8 @@ __global__ __launch_bounds__(kRouterThreads) void router_group_kernel(RouterArgs
     __syncthreads();
     if (tid == 0)
     {
-        const uint32_t finished = __hip_atomic_fetch_add(r.finished_chunks, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t finished =
+            chunks == 1u ? 0u : __hip_atomic_fetch_add(r.finished_chunks, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         shared.is_last = finished == chunks - 1u ? 1u : 0u;
     }
     __syncthreads();
@@ -524,6 +517,46 @@ __global__ __launch_bounds__(kRouterThreads) void router_group_kernel(RouterArgs
             r.error_words[1] = 0xffffffffu;
             *r.finished_chunks = 0u;
         }
+    }
+}
+
+__global__ __launch_bounds__(kRouterThreads) void router_group_kernel(RouterArgs r)
+{
+    __shared__ GroupShared shared;
+    place_chunk_routes(r, shared, blockIdx.x, gridDim.x);
+}
+
+// FUSED (calls of at most one chunk of tokens): the workgroup that finishes last also places the
+// routes, so the whole dispatch is one launch.
+template <int SLOTS, bool FUSED>
+__global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArgs r)
+{
+    __shared__ RouterShared shared;
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int wave = threadIdx.x >> 6;
+    const uint32_t token = blockIdx.x * kRouterWavesPerBlock + wave;
+    if (token < r.tokens)
+        select_token_routes<SLOTS>(r, shared, token, lane, wave);
+    if constexpr (FUSED)
+    {
+        __shared__ GroupShared group_shared;
+        // this workgroup's routes, counts and error words are made visible to the device, then the
+        // workgroup is counted; whoever counts last sees every other workgroup's
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __syncthreads();
+        if (threadIdx.x == 0)
+        {
+            const uint32_t finished = __hip_atomic_fetch_add(r.finished_selects, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            group_shared.is_last = finished == gridDim.x - 1u ? 1u : 0u;
+        }
+        __syncthreads();
+        if (group_shared.is_last == 0u)
+            return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (threadIdx.x == 0)
+            *r.finished_selects = 0u;
+        __syncthreads(); // is_last is read by all before place_chunk_routes writes it again
+        place_chunk_routes(r, group_shared, 0u, 1u);
     }
 }
 
