@@ -265,6 +265,63 @@ def bench_router_dispatch(args):
     print(json.dumps(line))
 
 
+def bench_generation_loop(args):
+    """The batched generation loop of the C++ host mirror (BatchGenerationLoop::generate): --rows Sessions
+    (64 by default) generate --steps tokens each from device-resident V = 151,936 fp32 logits, one device
+    call per token index; the model's decode step is outside this path and costs nothing here (the rows
+    stay resident).  Runs the C++ program and wraps its figures in the JSON shape of the other modes."""
+    import subprocess
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+    from ncnn_moe_runtime_amd.workloads import synthetic_model_logits as synthetic_logits
+
+    program = os.path.join(PACKAGE_DIR, "test_session_sampler")
+    if not os.path.exists(program):
+        sys.exit("%s is missing: build it with make -C %s" % (program, PACKAGE_DIR))
+    sessions = args.rows if args.rows > 0 else 64
+    vocab, steps = 151936, args.steps
+    done = subprocess.run([program, "--generation-bench", str(sessions), str(vocab), str(steps)],
+                          capture_output=True, text=True, timeout=1200)
+    if done.returncode != 0:
+        sys.exit("generation bench failed: " + done.stdout[-1000:] + done.stderr[-1000:])
+    fields = done.stdout.split()
+    figures = {fields[i]: fields[i + 1] for i in range(1, len(fields) - 1, 2)}
+    seconds = float(figures["seconds"]) - float(figures["prefill_seconds"])
+    tokens = int(figures["tokens"])
+    sample_seconds = int(figures["sample_time_microseconds"]) * 1e-6
+    # parity of the run that was timed: Session 0's first token, recomputed with the CPU oracle
+    first = oracle_lib.oracle_sample(synthetic_logits(vocab, 0, 0, -1), oracle_lib.OracleRng(1000).uniform(), 0.7, 20, 0.8, 0.0)
+    same = int(first["token_id"]) == int(figures["first_token"]) and \
+        int(np.float32(first["probability"]).view(np.uint32)) == int(figures["first_probability_bits"])
+    # CPU baseline: the oracle over the same rows, one thread
+    rows = np.stack([synthetic_logits(vocab, i, 0, -1) for i in range(min(sessions, 32))])
+    params = np.zeros(rows.shape[0], dtype=oracle_lib.ROW_PARAMS_DTYPE)
+    params["temperature"], params["top_k"], params["top_p"] = 0.7, 20, 0.8
+    uniforms = np.full(rows.shape[0], 0.5, dtype=np.float32)
+    start = time.perf_counter()
+    oracle_lib.oracle_sample_batch(rows, params, uniforms, threads=1)
+    cpu_seconds = time.perf_counter() - start
+    bytes_per_step = sessions * vocab * 4
+    line = {
+        "metric": "generated tokens/sec, %d Sessions, V=151936 fp32 temp+topk+topp, device-resident logits" % sessions,
+        "value": tokens / seconds, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": 20,
+        "ms_per_step": seconds / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "batched generation loop: %d Sessions x %d tokens, one device call per token index over "
+                               "%d x %d fp32 logits resident in HBM; T 0.7, Top-K 20, Top-P 0.8; decode step not included" % (
+                                   sessions, steps, sessions, vocab),
+                   "entry_point": "BatchGenerationLoop::generate (C++ host mirror) over ncnn_moe_hip_sampler_logits_buffer + _sample"},
+        "roofline": {"bound": "hbm", "achieved": bytes_per_step * steps / sample_seconds / 1e9, "peak": HBM_PEAK_BYTES_PER_S / 1e9,
+                     "unit": "GB/s", "frac": bytes_per_step * steps / sample_seconds / HBM_PEAK_BYTES_PER_S, "traffic": None,
+                     "kernel": "scan_select_kernel, wall clock of the synchronous sampling calls (SamplingStatistics::sample_time_microseconds)",
+                     "algorithmic_bytes_per_launch": bytes_per_step, "sample_us_per_step": sample_seconds / steps * 1e6},
+        "parity": {"first_token_matches_oracle": bool(same)},
+        "cpu_baseline": {"value": rows.shape[0] / cpu_seconds, "unit": "tokens/s", "cores": 1, "kind": "port",
+                         "sample": "%d rows of the same logits through the CPU oracle" % rows.shape[0]},
+    }
+    print(json.dumps(line))
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -287,6 +344,9 @@ def main():
     from ncnn_moe_runtime_amd import hip_sampler, workloads
     if args.workload == "router_dispatch":
         bench_router_dispatch(args)
+        return
+    if args.workload == "generation_loop":
+        bench_generation_loop(args)
         return
     if args.workload == "speculative_verify":
         return bench_speculative_verify(args, hip_sampler)

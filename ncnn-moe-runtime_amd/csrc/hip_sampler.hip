@@ -37,6 +37,15 @@ struct ncnn_moe_hip_sampler
     ncnn_moe_sample_result* results = nullptr;
     int32_t* stop_ids = nullptr;
     uint32_t stop_capacity = 0;
+    // the host entry's small operands travel as one block: params | uniforms | stop ids, staged in
+    // pinned memory and copied once; its results are written by the kernels straight into pinned memory
+    uint8_t* input_block = nullptr;      // device
+    uint8_t* input_block_host = nullptr; // pinned
+    size_t input_uniforms_offset = 0;
+    size_t input_stops_offset = 0;
+    uint32_t input_stop_capacity = 0;
+    ncnn_moe_sample_result* results_host = nullptr;   // pinned
+    ncnn_moe_sample_result* results_host_device = nullptr; // the same memory as the device addresses it
 
     float* segment_values = nullptr;
     int32_t* segment_indices = nullptr;
@@ -355,6 +364,14 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->results, rows * sizeof(ncnn_moe_sample_result)));
     s->stop_capacity = static_cast<uint32_t>(rows * 16);
     CREATE_CHECK(hipMalloc(&s->stop_ids, static_cast<size_t>(s->stop_capacity) * sizeof(int32_t)));
+    s->input_uniforms_offset = rows * sizeof(ncnn_moe_sample_params);
+    s->input_stops_offset = s->input_uniforms_offset + rows * sizeof(float);
+    s->input_stop_capacity = static_cast<uint32_t>(rows * 16);
+    const size_t input_bytes = s->input_stops_offset + static_cast<size_t>(s->input_stop_capacity) * sizeof(int32_t);
+    CREATE_CHECK(hipMalloc(&s->input_block, input_bytes));
+    CREATE_CHECK(hipHostMalloc(&s->input_block_host, input_bytes, hipHostMallocDefault));
+    CREATE_CHECK(hipHostMalloc(&s->results_host, rows * sizeof(ncnn_moe_sample_result), hipHostMallocDefault));
+    CREATE_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&s->results_host_device), s->results_host, 0));
     CREATE_CHECK(hipMalloc(&s->segment_values, slots * kSegmentRecordSlots * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->segment_indices, slots * kSegmentRecordSlots * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->segment_counts, slots * sizeof(uint32_t)));
@@ -404,12 +421,16 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->sort_keys[0], s->sort_keys[1],
         s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
-        s->verify_probabilities, s->verify_counts, s->verify_input, s->verify_output};
+        s->verify_probabilities, s->verify_counts, s->verify_input, s->verify_output, s->input_block};
     for (void* buffer : buffers)
     {
         if (buffer != nullptr)
             (void)hipFree(buffer);
     }
+    if (s->input_block_host != nullptr)
+        (void)hipHostFree(s->input_block_host);
+    if (s->results_host != nullptr)
+        (void)hipHostFree(s->results_host);
     if (s->verify_input_host != nullptr)
         (void)hipHostFree(s->verify_input_host);
     if (s->verify_output_host != nullptr)
@@ -486,19 +507,35 @@ int ncnn_moe_hip_sampler_sample(
         return NCNN_MOE_SAMPLER_SUCCESS;
     }
     SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
-    if (stop_id_count > s->stop_capacity)
+    // one copy brings params, uniforms and stop ids; stop-id lists beyond the block's room take the
+    // handle's growable buffer
+    const ncnn_moe_sample_params* device_params = reinterpret_cast<const ncnn_moe_sample_params*>(s->input_block);
+    const float* device_uniforms = reinterpret_cast<const float*>(s->input_block + s->input_uniforms_offset);
+    const int32_t* device_stops = nullptr;
+    std::memcpy(s->input_block_host, params, rows * sizeof(ncnn_moe_sample_params));
+    std::memcpy(s->input_block_host + s->input_uniforms_offset, uniforms, rows * sizeof(float));
+    size_t input_bytes = s->input_uniforms_offset + rows * sizeof(float);
+    if (stop_id_count > 0 && stop_id_count <= s->input_stop_capacity)
     {
-        SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
-        SAMPLER_HIP_CHECK(s, hipFree(s->stop_ids));
-        s->stop_ids = nullptr;
-        s->stop_capacity = 0;
-        SAMPLER_HIP_CHECK(s, hipMalloc(&s->stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t)));
-        s->stop_capacity = stop_id_count;
+        std::memcpy(s->input_block_host + s->input_stops_offset, stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t));
+        input_bytes = s->input_stops_offset + static_cast<size_t>(stop_id_count) * sizeof(int32_t);
+        device_stops = reinterpret_cast<const int32_t*>(s->input_block + s->input_stops_offset);
     }
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->params, params, rows * sizeof(ncnn_moe_sample_params), hipMemcpyHostToDevice, s->stream));
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->uniforms, uniforms, rows * sizeof(float), hipMemcpyHostToDevice, s->stream));
-    if (stop_id_count > 0)
+    else if (stop_id_count > 0)
+    {
+        if (stop_id_count > s->stop_capacity)
+        {
+            SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+            SAMPLER_HIP_CHECK(s, hipFree(s->stop_ids));
+            s->stop_ids = nullptr;
+            s->stop_capacity = 0;
+            SAMPLER_HIP_CHECK(s, hipMalloc(&s->stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t)));
+            s->stop_capacity = stop_id_count;
+        }
         SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->stop_ids, stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t), hipMemcpyHostToDevice, s->stream));
+        device_stops = s->stop_ids;
+    }
+    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->input_block, s->input_block_host, input_bytes, hipMemcpyHostToDevice, s->stream));
     // the host sees the options: the later passes are enqueued only if some row needs them
     SamplerPasses passes;
     passes.full_order = s->force_general != 0;
@@ -508,20 +545,18 @@ int ncnn_moe_hip_sampler_sample(
         passes.full_order = passes.full_order || row_left_pending(params[row], s->logits_vocab, kSelectTopK);
     }
     const bool full_order = passes.full_order;
-    const int32_t* device_stops = stop_id_count > 0 ? s->stop_ids : nullptr;
     int rc = launch_sampler(
         s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-        s->params, s->uniforms, device_stops, s->results, DistributionExport{}, passes, s->stream);
+        device_params, device_uniforms, device_stops, s->results_host_device, DistributionExport{}, passes, s->stream);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return rc;
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
     SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
     if (!full_order)
     {
         // a row whose ties overflowed the select buffers is finished by the full-order kernels
         bool pending = false;
         for (uint32_t row = 0; row < rows && !pending; ++row)
-            pending = results[row].status == NCNN_MOE_ROW_NEEDS_FULL_ORDER;
+            pending = s->results_host[row].status == NCNN_MOE_ROW_NEEDS_FULL_ORDER;
         if (pending)
         {
             SamplerPasses retry;
@@ -529,13 +564,13 @@ int ncnn_moe_hip_sampler_sample(
             retry.full_order = true;
             rc = launch_sampler(
                 s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-                s->params, s->uniforms, device_stops, s->results, DistributionExport{}, retry, s->stream);
+                device_params, device_uniforms, device_stops, s->results_host_device, DistributionExport{}, retry, s->stream);
             if (rc != NCNN_MOE_SAMPLER_SUCCESS)
                 return rc;
-            SAMPLER_HIP_CHECK(s, hipMemcpyAsync(results, s->results, rows * sizeof(ncnn_moe_sample_result), hipMemcpyDeviceToHost, s->stream));
             SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
         }
     }
+    std::memcpy(results, s->results_host, rows * sizeof(ncnn_moe_sample_result));
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

@@ -4,6 +4,7 @@
 #include "ncnn_moe_hip_sampler.h"
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 
 namespace ncnn {
@@ -28,6 +29,37 @@ Error error_of_call(int rc, const ncnn_moe_hip_sampler* handle)
     if (rc == NCNN_MOE_SAMPLER_INVALID_ARGUMENT)
         return Error{ErrorCode::InvalidArgument, std::string("hip sampler: ") + text};
     return Error{ErrorCode::InternalError, std::string("hip sampler: ") + text};
+}
+
+// Wall time of one device call, added to the statistics of the Sessions that took part in it.
+struct SampleTimer
+{
+    std::chrono::steady_clock::time_point started = std::chrono::steady_clock::now();
+
+    void charge(SamplingStatistics& statistics, uint64_t tokens) const
+    {
+        const auto elapsed = std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - started);
+        statistics.sample_calls += 1;
+        statistics.sampled_tokens += tokens;
+        statistics.sample_time_microseconds += static_cast<uint64_t>(elapsed.count());
+    }
+};
+
+// Locks the Sessions in ascending pointer order (src/engine/session.cpp:1249-1265); empty when the
+// list holds a null or a duplicate.
+template <typename Mutex>
+bool lock_in_pointer_order(std::vector<std::pair<const void*, Mutex*>> order, std::vector<std::unique_lock<Mutex>>& locks)
+{
+    std::sort(order.begin(), order.end());
+    for (size_t i = 0; i < order.size(); ++i)
+    {
+        if (order[i].first == nullptr || (i > 0 && order[i].first == order[i - 1].first))
+            return false;
+    }
+    locks.reserve(order.size());
+    for (const auto& entry : order)
+        locks.emplace_back(*entry.second);
+    return true;
 }
 
 template <typename T>
@@ -69,6 +101,13 @@ struct HipSampler::Impl
     std::vector<ncnn_moe_sample_params> params;
     std::vector<int32_t> stop_ids;
     std::vector<ncnn_moe_sample_result> results;
+    uint32_t resident_rows = 0; // rows x vocab the logits buffer was last laid out for
+    uint32_t resident_vocab = 0;
+
+    // Samples the rows the logits buffer holds.  The caller holds the sampler's mutex.
+    std::vector<Result<BatchSampledToken>> sample_rows(
+        size_t rows, std::span<const SamplingOptions> options, std::span<const float> uniforms,
+        std::span<const std::vector<int32_t>> stop_tokens, std::vector<uint8_t>& draw_consumed);
 
     ~Impl()
     {
@@ -128,42 +167,48 @@ std::vector<Result<BatchSampledToken>> HipSampler::sample(
     impl.staging.resize(rows * vocab);
     for (size_t row = 0; row < rows; ++row)
         std::copy(logits[row].begin(), logits[row].end(), impl.staging.begin() + row * vocab);
-    impl.params.resize(rows);
-    impl.stop_ids.clear();
+    const int rc = ncnn_moe_hip_sampler_upload_logits(
+        impl.handle, impl.staging.data(), NCNN_MOE_LOGITS_F32, static_cast<uint32_t>(rows), static_cast<uint32_t>(vocab), vocab);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return every_row<BatchSampledToken>(rows, error_of_call(rc, impl.handle));
+    impl.resident_rows = static_cast<uint32_t>(rows);
+    impl.resident_vocab = static_cast<uint32_t>(vocab);
+    return impl.sample_rows(rows, options, uniforms, stop_tokens, draw_consumed);
+}
+
+std::vector<Result<BatchSampledToken>> HipSampler::Impl::sample_rows(
+    size_t rows, std::span<const SamplingOptions> options, std::span<const float> uniforms,
+    std::span<const std::vector<int32_t>> stop_tokens, std::vector<uint8_t>& draw_consumed)
+{
+    params.resize(rows);
+    stop_ids.clear();
     for (size_t row = 0; row < rows; ++row)
     {
-        ncnn_moe_sample_params& p = impl.params[row];
+        ncnn_moe_sample_params& p = params[row];
         p.temperature = options[row].temperature;
         p.top_k = options[row].top_k;
         p.top_p = options[row].top_p;
         p.min_p = options[row].min_p;
-        p.stop_begin = static_cast<uint32_t>(impl.stop_ids.size());
+        p.stop_begin = static_cast<uint32_t>(stop_ids.size());
         p.stop_count = 0;
         if (!stop_tokens.empty())
         {
             p.stop_count = static_cast<uint32_t>(stop_tokens[row].size());
-            impl.stop_ids.insert(impl.stop_ids.end(), stop_tokens[row].begin(), stop_tokens[row].end());
+            stop_ids.insert(stop_ids.end(), stop_tokens[row].begin(), stop_tokens[row].end());
         }
     }
-    impl.results.resize(rows);
-
-    int rc = ncnn_moe_hip_sampler_upload_logits(
-        impl.handle, impl.staging.data(), NCNN_MOE_LOGITS_F32, static_cast<uint32_t>(rows), static_cast<uint32_t>(vocab), vocab);
-    if (rc == NCNN_MOE_SAMPLER_SUCCESS)
-    {
-        rc = ncnn_moe_hip_sampler_sample(
-            impl.handle, static_cast<uint32_t>(rows), impl.params.data(), uniforms.data(),
-            impl.stop_ids.empty() ? nullptr : impl.stop_ids.data(), static_cast<uint32_t>(impl.stop_ids.size()),
-            impl.results.data());
-    }
+    results.resize(rows);
+    const int rc = ncnn_moe_hip_sampler_sample(
+        handle, static_cast<uint32_t>(rows), params.data(), uniforms.data(),
+        stop_ids.empty() ? nullptr : stop_ids.data(), static_cast<uint32_t>(stop_ids.size()), results.data());
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
-        return every_row<BatchSampledToken>(rows, error_of_call(rc, impl.handle));
+        return every_row<BatchSampledToken>(rows, error_of_call(rc, handle));
 
     std::vector<Result<BatchSampledToken>> out;
     out.reserve(rows);
     for (size_t row = 0; row < rows; ++row)
     {
-        const ncnn_moe_sample_result& r = impl.results[row];
+        const ncnn_moe_sample_result& r = results[row];
         if (r.status != NCNN_MOE_ROW_OK)
         {
             out.emplace_back(error_of_row_status(r.status));
@@ -178,6 +223,42 @@ std::vector<Result<BatchSampledToken>> HipSampler::sample(
         out.emplace_back(token);
     }
     return out;
+}
+
+Result<DeviceLogitsRows> HipSampler::device_logits(uint32_t rows, uint32_t vocab, bool bf16)
+{
+    if (rows == 0 || vocab == 0)
+        return invalid_argument("cannot sample empty logits");
+    if (rows > impl_->max_rows)
+        return invalid_argument("sample batch exceeds the sampler's max_rows");
+    if (vocab > impl_->max_vocab)
+        return invalid_argument("logits exceed the sampler's max_vocab");
+    const std::lock_guard<std::mutex> lock(mutex_);
+    DeviceLogitsRows out;
+    const int rc = ncnn_moe_hip_sampler_logits_buffer(
+        impl_->handle, bf16 ? NCNN_MOE_LOGITS_BF16 : NCNN_MOE_LOGITS_F32, rows, vocab, &out.data, &out.row_stride);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return error_of_call(rc, impl_->handle);
+    out.rows = rows;
+    out.vocab = vocab;
+    out.bf16 = bf16;
+    impl_->resident_rows = rows;
+    impl_->resident_vocab = vocab;
+    return out;
+}
+
+std::vector<Result<BatchSampledToken>> HipSampler::sample_resident(
+    std::span<const SamplingOptions> options, std::span<const float> uniforms,
+    std::span<const std::vector<int32_t>> stop_tokens, std::vector<uint8_t>& draw_consumed)
+{
+    const size_t rows = options.size();
+    draw_consumed.assign(rows, 0);
+    if (rows == 0 || uniforms.size() != rows || (!stop_tokens.empty() && stop_tokens.size() != rows))
+        return every_row<BatchSampledToken>(rows, invalid_argument("sample batch operands differ in length"));
+    const std::lock_guard<std::mutex> lock(mutex_);
+    if (rows != impl_->resident_rows)
+        return every_row<BatchSampledToken>(rows, invalid_argument("sample batch differs from the rows laid out by device_logits"));
+    return impl_->sample_rows(rows, options, uniforms, stop_tokens, draw_consumed);
 }
 
 Result<std::vector<TokenProbability>> HipSampler::distribution(std::span<const float> logits, const SamplingOptions& options)
@@ -298,14 +379,22 @@ Result<SampledToken> SamplingSession::sample(const LogitsOutput& logits, const S
     const float uniform = peek_uniform(random_generator_, advanced);
     const std::span<const float> row(logits.values);
     std::vector<uint8_t> draw_consumed;
+    const SampleTimer timer;
     auto results = sampler_->sample(
         std::span<const std::span<const float>>(&row, 1), std::span<const SamplingOptions>(&options, 1),
         std::span<const float>(&uniform, 1), {}, draw_consumed);
+    timer.charge(statistics_, results[0] ? 1 : 0);
     if (!results[0])
         return results[0].error();
     if (draw_consumed[0])
         random_generator_ = advanced;
     return results[0].value().token;
+}
+
+SamplingStatistics SamplingSession::statistics() const
+{
+    const std::lock_guard<std::mutex> lock(mutex_);
+    return statistics_;
 }
 
 Result<SpeculativeVerification> SamplingSession::verify_speculative(
@@ -381,15 +470,131 @@ std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample(
     if (active.empty())
         return out;
     std::vector<uint8_t> draw_consumed;
+    const SampleTimer timer;
     auto sampled = sampler->sample(logits, options, uniforms, stop_tokens, draw_consumed);
     for (size_t j = 0; j < active.size(); ++j)
     {
         const size_t i = active[j];
         out[i] = sampled[j];
+        timer.charge(requests[i].session->statistics_, sampled[j] ? 1 : 0);
         if (sampled[j] && draw_consumed[j])
             requests[i].session->random_generator_ = advanced[j];
     }
     return out;
+}
+
+Result<std::vector<GenerationResult>> BatchGenerationLoop::generate(
+    const HipSamplerPtr& sampler, std::span<SamplingSession* const> sessions, IDeviceLogitsSource& source,
+    std::span<const GenerationOptions> options, const BatchTokenCallback& on_token)
+{
+    const size_t count = sessions.size();
+    if (count == 0)
+        return invalid_argument("generation batch is empty");
+    if (!sampler)
+        return Error{ErrorCode::InternalError, "hip sampler is unavailable (no GPU, or create() failed)"};
+    if (options.size() != 1 && options.size() != count)
+        return invalid_argument("generation options must hold one entry, or one per session");
+    if (count > sampler->max_rows())
+        return invalid_argument("generation batch exceeds the sampler's max_rows");
+    const uint32_t vocab = source.vocabulary_size();
+    const bool bf16 = source.bf16_logits();
+    std::vector<std::pair<const void*, std::mutex*>> order;
+    for (SamplingSession* session : sessions)
+        order.emplace_back(session, session != nullptr ? &session->mutex_ : nullptr);
+    std::vector<std::unique_lock<std::mutex>> locks;
+    if (!lock_in_pointer_order(std::move(order), locks))
+        return invalid_argument("generation batch contains a null or duplicate session");
+    const auto options_of = [&](size_t session_index) -> const GenerationOptions& {
+        return options[options.size() == 1 ? 0 : session_index];
+    };
+    for (size_t i = 0; i < count; ++i)
+    {
+        // Session::generate checks these before it decodes anything (src/engine/session.cpp:461-473)
+        if (options_of(i).max_new_tokens == 0)
+            return invalid_argument("max_new_tokens must be non-zero");
+        auto valid = validate_sampling_options(options_of(i).sampling);
+        if (!valid)
+            return valid.error();
+    }
+
+    std::vector<GenerationResult> results(count);
+    // the Sessions that sample at this token index, in Session order; row i of the device buffer is theirs
+    std::vector<uint32_t> active(count);
+    for (size_t i = 0; i < count; ++i)
+        active[i] = static_cast<uint32_t>(i);
+    auto rows = sampler->device_logits(static_cast<uint32_t>(count), vocab, bf16);
+    if (!rows)
+        return rows.error();
+    auto prefilled = source.prefill(active, rows.value());
+    if (!prefilled)
+        return prefilled.error();
+
+    std::vector<SamplingOptions> row_options;
+    std::vector<float> uniforms;
+    std::vector<std::mt19937_64> advanced;
+    std::vector<std::vector<int32_t>> stop_tokens;
+    std::vector<uint8_t> draw_consumed;
+    std::vector<DecodeSlot> slots;
+    std::vector<uint32_t> next_active;
+    for (uint32_t index = 0; !active.empty(); ++index)
+    {
+        row_options.clear();
+        uniforms.clear();
+        stop_tokens.clear();
+        advanced.resize(active.size());
+        for (size_t row = 0; row < active.size(); ++row)
+        {
+            const uint32_t i = active[row];
+            row_options.push_back(options_of(i).sampling);
+            uniforms.push_back(peek_uniform(sessions[i]->random_generator_, advanced[row]));
+            stop_tokens.push_back(options_of(i).stop_tokens);
+        }
+        const SampleTimer timer;
+        auto sampled = sampler->sample_resident(row_options, uniforms, stop_tokens, draw_consumed);
+        slots.clear();
+        next_active.clear();
+        for (size_t row = 0; row < active.size(); ++row)
+        {
+            const uint32_t i = active[row];
+            timer.charge(sessions[i]->statistics_, sampled[row] ? 1 : 0);
+            if (!sampled[row])
+                return sampled[row].error();
+            if (draw_consumed[row])
+                sessions[i]->random_generator_ = advanced[row];
+            StreamToken token;
+            token.index = index;
+            token.token_id = sampled[row].value().token.token_id;
+            token.probability = sampled[row].value().token.probability;
+            token.is_stop_token = sampled[row].value().is_stop_token;
+            const bool continue_generation = !on_token || on_token(i, token);
+            results[i].tokens.push_back(std::move(token));
+            // the order of src/engine/session.cpp:1000-1013: callback, stop token, token budget
+            if (!continue_generation)
+            {
+                results[i].stopped_by_callback = true;
+                continue;
+            }
+            if (results[i].tokens.back().is_stop_token)
+            {
+                results[i].stopped_by_stop_token = true;
+                continue;
+            }
+            if (index + 1 == options_of(i).max_new_tokens)
+                continue;
+            slots.push_back(DecodeSlot{i, results[i].tokens.back().token_id});
+            next_active.push_back(i);
+        }
+        active.swap(next_active);
+        if (active.empty())
+            break;
+        rows = sampler->device_logits(static_cast<uint32_t>(active.size()), vocab, bf16);
+        if (!rows)
+            return rows.error();
+        auto decoded = source.decode(slots, rows.value());
+        if (!decoded)
+            return decoded.error();
+    }
+    return results;
 }
 
 } // namespace moe

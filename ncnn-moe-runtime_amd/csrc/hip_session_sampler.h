@@ -14,6 +14,9 @@
 //       rejects duplicates (src/engine/session.cpp:1249-1265), draws one uniform per row from a COPY
 //       of each Session's generator, samples every row in one device call, and commits the copy back
 //       only for rows whose draw was consumed (session.cpp:429-433).
+//   BatchGenerationLoop  the scheduler-driven generation loop of examples/internal/run_model.cpp:726-847
+//       over device-resident logits: an IDeviceLogitsSource (the model's prefill / decode) writes
+//       each step's logits into the sampler's buffer and one device call samples every active Session.
 //
 // Everything here runs on the device through the C ABI of include/ncnn_moe_hip_sampler.h.  There is
 // no CPU fallback: without a usable GPU create() returns null and sample() reports InternalError.
@@ -21,6 +24,7 @@
 #define NCNN_MOE_HIP_SESSION_SAMPLER_H
 
 #include <cstdint>
+#include <functional>
 #include <memory>
 #include <mutex>
 #include <random>
@@ -86,6 +90,31 @@ struct SampledToken
     float probability = 0.0f;
 };
 
+// StreamToken, GenerationOptions and GenerationResult of include/ncnn/moe/session.h:63-91 (without the
+// speculative switches, which belong to Session::generate's draft model).
+struct StreamToken
+{
+    uint32_t index = 0;
+    int32_t token_id = -1;
+    float probability = 0.0f;
+    std::string text; // left empty: callers decode token ids themselves
+    bool is_stop_token = false;
+};
+
+struct GenerationOptions
+{
+    uint32_t max_new_tokens = 1;
+    SamplingOptions sampling;
+    std::vector<int32_t> stop_tokens;
+};
+
+struct GenerationResult
+{
+    std::vector<StreamToken> tokens;
+    bool stopped_by_stop_token = false;
+    bool stopped_by_callback = false;
+};
+
 } // namespace moe
 } // namespace ncnn
 
@@ -118,6 +147,16 @@ struct SpeculativeVerification
     bool next_from_residual = false;
 };
 
+// Rows of logits in device memory: row i starts at data + i * row_stride elements.
+struct DeviceLogitsRows
+{
+    void* data = nullptr;
+    uint64_t row_stride = 0; // in elements
+    uint32_t rows = 0;
+    uint32_t vocab = 0;
+    bool bf16 = false;       // bfloat16 elements instead of float
+};
+
 class HipSampler
 {
 public:
@@ -135,6 +174,20 @@ public:
     // a bad row does not fail the others.  A call-level failure yields that Error for every row.
     std::vector<Result<BatchSampledToken>> sample(
         std::span<const std::span<const float>> logits,
+        std::span<const SamplingOptions> options,
+        std::span<const float> uniforms,
+        std::span<const std::vector<int32_t>> stop_tokens,
+        std::vector<uint8_t>& draw_consumed);
+
+    // The device-resident hand-off (ncnn_moe_hip_sampler_logits_buffer): the sampler's own logits
+    // buffer laid out for rows x vocab.  A decode step writes its LM-head output there, and
+    // sample_resident() reads it: the logits never become a std::vector<float>
+    // (src/engine/cpu_executor.cpp:2988-2994, src/kernels/cpu_ops.cpp:1166-1172 are the copies this removes).
+    Result<DeviceLogitsRows> device_logits(uint32_t rows, uint32_t vocab, bool bf16 = false);
+
+    // sample() over the rows last laid out by device_logits(); the rows must be complete in device
+    // memory when this is called.
+    std::vector<Result<BatchSampledToken>> sample_resident(
         std::span<const SamplingOptions> options,
         std::span<const float> uniforms,
         std::span<const std::vector<int32_t>> stop_tokens,
@@ -164,6 +217,15 @@ private:
 
 using HipSamplerPtr = std::shared_ptr<HipSampler>;
 
+// The sampling share of SessionStatistics (include/ncnn/moe/session.h:98-160 keeps prefill/decode
+// counters and times per Session; sampling had none because it was not measurable on the CPU path).
+struct SamplingStatistics
+{
+    uint64_t sampled_tokens = 0;           // tokens this Session's sampler returned
+    uint64_t sample_calls = 0;             // device calls the Session took part in
+    uint64_t sample_time_microseconds = 0; // wall time of those calls (a batched call counts in full for each of its Sessions)
+};
+
 struct SamplingSessionOptions
 {
     uint64_t sampling_seed = 0; // SessionOptions::sampling_seed, include/ncnn/moe/session.h:280-286
@@ -183,10 +245,15 @@ public:
         std::span<const LogitsOutput> target_logits, std::span<const LogitsOutput> draft_logits,
         std::span<const int32_t> proposed_token_ids, const SamplingOptions& options = {});
 
+    // Session::statistics(), the sampling share.
+    [[nodiscard]] SamplingStatistics statistics() const;
+
 private:
     friend class SessionBatchSampler;
+    friend class BatchGenerationLoop;
     HipSamplerPtr sampler_;
     std::mt19937_64 random_generator_;
+    SamplingStatistics statistics_;
     mutable std::mutex mutex_;
 };
 
@@ -205,6 +272,44 @@ public:
     // examples/internal/run_model.cpp:776-809.  Rejects empty batches, null or duplicate Sessions and
     // rows of different lengths with InvalidArgument for every row.
     static std::vector<Result<BatchSampledToken>> sample(const HipSamplerPtr& sampler, std::span<const SampleBatchRequest> requests);
+};
+
+// One row of a decode step: DecodeBatchRequest of the batch scheduler ({session, token}).
+struct DecodeSlot
+{
+    uint32_t session_index = 0;
+    int32_t token_id = -1;
+};
+
+// The model side of the loop: what BatchScheduler::submit_prefill / submit_decode do, writing the
+// logits into device rows instead of returning LogitsOutput vectors.  Row i belongs to the i-th
+// listed Session.  The rows must be complete in device memory when a call returns.
+class IDeviceLogitsSource
+{
+public:
+    virtual ~IDeviceLogitsSource() = default;
+    virtual uint32_t vocabulary_size() const = 0;
+    virtual bool bf16_logits() const { return false; }
+    virtual Result<bool> prefill(std::span<const uint32_t> session_indices, const DeviceLogitsRows& rows) = 0;
+    virtual Result<bool> decode(std::span<const DecodeSlot> slots, const DeviceLogitsRows& rows) = 0;
+};
+
+// Called for every token as it is sampled; returning false stops that Session (GenerationResult::stopped_by_callback).
+using BatchTokenCallback = std::function<bool(uint32_t session_index, const StreamToken& token)>;
+
+class BatchGenerationLoop
+{
+public:
+    // The scheduler-driven generation of examples/internal/run_model.cpp:726-847 with the sampling
+    // of every step as ONE device call over device-resident logits: prefill all Sessions, then per
+    // token index sample the active Sessions in Session order (each with its own generator, options
+    // and stop tokens), stop those that emitted a stop token, reached max_new_tokens or whose callback
+    // declined, and decode the others' tokens for the next step.  `options` holds one entry for all
+    // Sessions or one per Session.  Token ids, probabilities, stop flags and generator states end up
+    // as Session::generate (src/engine/session.cpp:978-1020) leaves them for each Session alone.
+    static Result<std::vector<GenerationResult>> generate(
+        const HipSamplerPtr& sampler, std::span<SamplingSession* const> sessions, IDeviceLogitsSource& source,
+        std::span<const GenerationOptions> options, const BatchTokenCallback& on_token = {});
 };
 
 // validate_sampling_options (src/engine/session.cpp:65-74) on the host, with the same messages.

@@ -100,3 +100,20 @@ def make_workload(name, rows=None, seed=2024, vocab=None):
         "name": name, "rows": rows, "vocab": vocab, "dtype": dtype, "logits": logits, "params": params,
         "uniforms": _uniforms(rows, seed), "stop_ids": stop_ids, "description": description,
     }
+
+
+def synthetic_model_logits(vocab, session, position, fed_token):
+    """Logits of the stand-in model that the generation-loop test program uses (synthetic_logits in
+    tests/cpp/test_session_sampler.cpp): an integer hash of (session, position, token fed), every value
+    a multiple of 2^-20 in [-8, 14), so that C++ and numpy produce the same fp32 rows."""
+    mask = 0xFFFFFFFF
+    seed = ((session * 0x9E3779B1) ^ (position * 0x85EBCA77) ^ ((fed_token & mask) * 0xC2B2AE3D) ^ 0x27D4EB2F) & mask
+    h = (np.arange(vocab, dtype=np.uint64) * 2654435761 + seed) & mask
+    h ^= h >> np.uint64(15)
+    h = (h * 2246822519) & mask
+    h ^= h >> np.uint64(13)
+    h = (h * 3266489917) & mask
+    h ^= h >> np.uint64(16)
+    values = (h >> np.uint64(8)).astype(np.float32) * np.float32(1.0 / 1048576.0) - np.float32(8.0)
+    values[(h & np.uint64(1023)) == 0] += np.float32(6.0)
+    return values.astype(np.float32)

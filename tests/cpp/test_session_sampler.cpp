@@ -3,13 +3,24 @@
 // The first group mirrors the runtime's sampler test (tests/test_runtime.cpp:4320-4362); the rest
 // cover what that test leaves out: draws, RNG bookkeeping, batches, stop tokens, error text.
 //
-//   test_session_sampler            all tests (needs a GPU)
-//   test_session_sampler --host     only the tests that need no GPU
+//   test_session_sampler                      all tests (needs a GPU)
+//   test_session_sampler --host               only the tests that need no GPU
+//   test_session_sampler --generation-bench SESSIONS VOCAB STEPS   times the batched generation loop
+//   test_session_sampler --generation-trace   runs the batched generation loop on the synthetic
+//                                             model below and prints every emitted token, for a
+//                                             checker that recomputes the run with the CPU sampler
 #include "hip_session_sampler.h"
 
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <bit>
+#include <chrono>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <deque>
 #include <limits>
 #include <random>
 #include <stdexcept>
@@ -412,9 +423,383 @@ static void test_speculative_verification(const HipSamplerPtr& sampler)
     }
 }
 
+// ---- batched generation loop ----------------------------------------------------------------
+
+// A stand-in for the model: the logits after a Session's position p depend on (session, p, token fed)
+// through an integer hash, every value a multiple of 2^-20 in [-8, 14), so a checker in another
+// language reproduces them exactly.  It writes device rows, as a decode step on the GPU would.
+static std::vector<float> synthetic_logits(uint32_t vocab, uint32_t session, uint32_t position, int32_t fed_token)
+{
+    const uint32_t seed = (session * 0x9E3779B1u) ^ (position * 0x85EBCA77u) ^ (static_cast<uint32_t>(fed_token) * 0xC2B2AE3Du) ^ 0x27D4EB2Fu;
+    std::vector<float> row(vocab);
+    for (uint32_t v = 0; v < vocab; ++v)
+    {
+        uint32_t h = v * 2654435761u + seed;
+        h ^= h >> 15;
+        h *= 2246822519u;
+        h ^= h >> 13;
+        h *= 3266489917u;
+        h ^= h >> 16;
+        float value = static_cast<float>(h >> 8) * (1.0f / 1048576.0f) - 8.0f;
+        if ((h & 1023u) == 0u)
+            value += 6.0f;
+        row[v] = value;
+    }
+    return row;
+}
+
+class SyntheticSource : public IDeviceLogitsSource
+{
+public:
+    SyntheticSource(uint32_t vocab, uint32_t sessions) : vocab_(vocab), positions_(sessions, 0) {}
+
+    uint32_t vocabulary_size() const override { return vocab_; }
+
+    Result<bool> prefill(std::span<const uint32_t> session_indices, const DeviceLogitsRows& rows) override
+    {
+        for (size_t row = 0; row < session_indices.size(); ++row)
+        {
+            positions_[session_indices[row]] = 0;
+            auto written = write_row(rows, row, synthetic_logits(vocab_, session_indices[row], 0, -1));
+            if (!written)
+                return written;
+        }
+        ++prefill_calls;
+        return true;
+    }
+
+    Result<bool> decode(std::span<const DecodeSlot> slots, const DeviceLogitsRows& rows) override
+    {
+        if (fail_decode_at != 0 && decode_calls + 1 == fail_decode_at)
+            return Error{ErrorCode::InternalError, "synthetic decode failure"};
+        for (size_t row = 0; row < slots.size(); ++row)
+        {
+            const uint32_t position = ++positions_[slots[row].session_index];
+            auto written = write_row(rows, row, synthetic_logits(vocab_, slots[row].session_index, position, slots[row].token_id));
+            if (!written)
+                return written;
+        }
+        ++decode_calls;
+        decoded_rows += static_cast<uint32_t>(slots.size());
+        return true;
+    }
+
+    uint32_t prefill_calls = 0;
+    uint32_t decode_calls = 0;
+    uint32_t decoded_rows = 0;
+    uint32_t fail_decode_at = 0;
+
+private:
+    Result<bool> write_row(const DeviceLogitsRows& rows, size_t row, const std::vector<float>& values)
+    {
+        if (rows.bf16 || rows.vocab != vocab_ || row >= rows.rows || rows.row_stride < vocab_)
+            return Error{ErrorCode::InternalError, "synthetic source: unexpected device rows"};
+        float* target = static_cast<float*>(rows.data) + row * rows.row_stride;
+        if (hipMemcpy(target, values.data(), values.size() * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
+            return Error{ErrorCode::InternalError, "synthetic source: hipMemcpy failed"};
+        return true;
+    }
+
+    uint32_t vocab_;
+    std::vector<uint32_t> positions_;
+};
+
+struct LoopCase
+{
+    uint64_t seed;
+    GenerationOptions options;
+};
+
+static std::vector<LoopCase> loop_cases()
+{
+    std::vector<LoopCase> cases;
+    const auto add = [&](uint64_t seed, uint32_t max_new_tokens, float temperature, uint32_t top_k, float top_p, float min_p,
+                         std::vector<int32_t> stop_tokens) {
+        LoopCase entry;
+        entry.seed = seed;
+        entry.options.max_new_tokens = max_new_tokens;
+        entry.options.sampling = SamplingOptions{temperature, top_k, top_p, min_p};
+        entry.options.stop_tokens = std::move(stop_tokens);
+        cases.push_back(std::move(entry));
+    };
+    std::vector<int32_t> many_stops;
+    for (int32_t id = 0; id < 3000; id += 7)
+        many_stops.push_back(id); // a seventh of the vocabulary stops this Session early
+    add(11, 24, 0.0f, 0, 1.0f, 0.0f, {});           // greedy
+    add(12, 24, 0.7f, 20, 0.8f, 0.0f, {});          // the headline options
+    add(13, 17, 1.0f, 0, 0.9f, 0.0f, {});           // no Top-K window: the full-order kernels
+    add(14, 24, 1.3f, 300, 1.0f, 0.001f, {});       // the wide select kernel
+    add(15, 24, 0.9f, 40, 0.95f, 0.0f, many_stops); // stops early
+    add(16, 1, 0.8f, 8, 1.0f, 0.0f, {});            // one token only
+    add(17, 24, 0.5f, 1, 1.0f, 0.0f, {});           // single survivor: the generator is never advanced
+    add(18, 9, 1.0f, 64, 0.5f, 0.05f, {5, 6, 7});
+    return cases;
+}
+
+constexpr uint32_t kLoopVocab = 3000;
+
+static std::vector<GenerationResult> run_loop(const HipSamplerPtr& sampler, const std::vector<LoopCase>& cases,
+                                              std::deque<SamplingSession>& sessions, SyntheticSource& source,
+                                              const BatchTokenCallback& on_token = {})
+{
+    std::vector<SamplingSession*> pointers;
+    std::vector<GenerationOptions> options;
+    for (size_t i = 0; i < cases.size(); ++i)
+    {
+        pointers.push_back(&sessions[i]);
+        options.push_back(cases[i].options);
+    }
+    auto generated = BatchGenerationLoop::generate(sampler, pointers, source, options, on_token);
+    if (!generated)
+        throw std::runtime_error("generation loop failed: " + generated.error().message);
+    return std::move(generated).value();
+}
+
+// a deque: Sessions hold a mutex and do not move
+static void make_sessions(const HipSamplerPtr& sampler, const std::vector<LoopCase>& cases, std::deque<SamplingSession>& sessions)
+{
+    for (const LoopCase& entry : cases)
+        sessions.emplace_back(sampler, SamplingSessionOptions{entry.seed});
+}
+
+// The loop against each Session generating alone through SamplingSession::sample on host logits:
+// the order of Session::generate (src/engine/session.cpp:978-1020).
+static void test_generation_loop_equals_serial(const HipSamplerPtr& sampler)
+{
+    const std::vector<LoopCase> cases = loop_cases();
+    std::deque<SamplingSession> sessions;
+    make_sessions(sampler, cases, sessions);
+    SyntheticSource source(kLoopVocab, static_cast<uint32_t>(cases.size()));
+    const std::vector<GenerationResult> batched = run_loop(sampler, cases, sessions, source);
+    check(batched.size() == cases.size());
+    check(source.prefill_calls == 1);
+    uint32_t expected_decoded_rows = 0;
+    uint32_t longest = 0;
+    for (size_t i = 0; i < cases.size(); ++i)
+    {
+        SamplingSession alone(sampler, SamplingSessionOptions{cases[i].seed});
+        const GenerationOptions& options = cases[i].options;
+        GenerationResult serial;
+        int32_t fed = -1;
+        for (uint32_t index = 0; index < options.max_new_tokens; ++index)
+        {
+            auto sampled = alone.sample(logits_of(synthetic_logits(kLoopVocab, static_cast<uint32_t>(i), index, fed)), options.sampling);
+            check(static_cast<bool>(sampled));
+            StreamToken token;
+            token.index = index;
+            token.token_id = sampled.value().token_id;
+            token.probability = sampled.value().probability;
+            token.is_stop_token = std::find(options.stop_tokens.begin(), options.stop_tokens.end(), token.token_id) != options.stop_tokens.end();
+            serial.tokens.push_back(token);
+            if (token.is_stop_token)
+            {
+                serial.stopped_by_stop_token = true;
+                break;
+            }
+            fed = token.token_id;
+        }
+        check(batched[i].tokens.size() == serial.tokens.size());
+        check(batched[i].stopped_by_stop_token == serial.stopped_by_stop_token);
+        check(!batched[i].stopped_by_callback);
+        for (size_t t = 0; t < serial.tokens.size(); ++t)
+        {
+            check(batched[i].tokens[t].index == serial.tokens[t].index);
+            check(batched[i].tokens[t].token_id == serial.tokens[t].token_id);
+            check(std::memcmp(&batched[i].tokens[t].probability, &serial.tokens[t].probability, sizeof(float)) == 0);
+            check(batched[i].tokens[t].is_stop_token == serial.tokens[t].is_stop_token);
+        }
+        // both generators stand at the same draw afterwards
+        const LogitsOutput probe = logits_of(synthetic_logits(kLoopVocab, 99, 0, -1));
+        auto next_batched = sessions[i].sample(probe, SamplingOptions{1.0f, 50, 1.0f, 0.0f});
+        auto next_serial = alone.sample(probe, SamplingOptions{1.0f, 50, 1.0f, 0.0f});
+        check(next_batched && next_serial && next_batched.value().token_id == next_serial.value().token_id);
+        const SamplingStatistics statistics = sessions[i].statistics();
+        check(statistics.sampled_tokens == serial.tokens.size() + 1);
+        check(statistics.sample_calls == serial.tokens.size() + 1);
+        check(statistics.sample_time_microseconds > 0);
+        const uint32_t emitted = static_cast<uint32_t>(serial.tokens.size());
+        expected_decoded_rows += serial.stopped_by_stop_token ? emitted - 1 : emitted - 1;
+        longest = std::max(longest, emitted);
+    }
+    check(source.decoded_rows == expected_decoded_rows); // a stopped Session is never decoded again
+    check(source.decode_calls == longest - 1);
+    check(batched[4].stopped_by_stop_token);                // the Session with many stop tokens
+    check(batched[4].tokens.size() < 24);
+    check(batched[5].tokens.size() == 1);
+}
+
+static void test_generation_loop_callback_and_errors(const HipSamplerPtr& sampler)
+{
+    const std::vector<LoopCase> cases = loop_cases();
+    {
+        // the callback declines Session 2's fourth token: it stops there, the others run on
+        std::deque<SamplingSession> sessions;
+    make_sessions(sampler, cases, sessions);
+        SyntheticSource source(kLoopVocab, static_cast<uint32_t>(cases.size()));
+        uint32_t seen = 0;
+        const auto results = run_loop(sampler, cases, sessions, source, [&](uint32_t session_index, const StreamToken& token) {
+            ++seen;
+            return !(session_index == 2 && token.index == 3);
+        });
+        check(results[2].stopped_by_callback && results[2].tokens.size() == 4);
+        check(!results[1].stopped_by_callback && results[1].tokens.size() == 24);
+        uint32_t total = 0;
+        for (const GenerationResult& result : results)
+            total += static_cast<uint32_t>(result.tokens.size());
+        check(seen == total);
+    }
+    {
+        std::deque<SamplingSession> sessions;
+    make_sessions(sampler, cases, sessions);
+        SyntheticSource source(kLoopVocab, static_cast<uint32_t>(cases.size()));
+        std::vector<SamplingSession*> pointers = {&sessions[0], &sessions[1]};
+        std::vector<GenerationOptions> options = {cases[0].options};
+        // one shared options entry
+        auto shared = BatchGenerationLoop::generate(sampler, pointers, source, options);
+        check(shared && shared.value().size() == 2 && shared.value()[1].tokens.size() == 24);
+        // errors before anything is decoded
+        const uint32_t prefills = source.prefill_calls;
+        GenerationOptions bad = cases[1].options;
+        bad.sampling.top_p = 0.0f;
+        auto invalid = BatchGenerationLoop::generate(sampler, pointers, source, std::vector<GenerationOptions>{bad});
+        check(!invalid && invalid.error().message == "top_p must be in the range (0, 1]");
+        bad = cases[1].options;
+        bad.max_new_tokens = 0;
+        invalid = BatchGenerationLoop::generate(sampler, pointers, source, std::vector<GenerationOptions>{bad});
+        check(!invalid && invalid.error().message == "max_new_tokens must be non-zero");
+        std::vector<SamplingSession*> twice = {&sessions[0], &sessions[0]};
+        invalid = BatchGenerationLoop::generate(sampler, twice, source, options);
+        check(!invalid && invalid.error().code == ErrorCode::InvalidArgument);
+        std::vector<SamplingSession*> with_null = {&sessions[0], nullptr};
+        invalid = BatchGenerationLoop::generate(sampler, with_null, source, options);
+        check(!invalid && invalid.error().code == ErrorCode::InvalidArgument);
+        invalid = BatchGenerationLoop::generate(sampler, pointers, source, std::vector<GenerationOptions>(3, cases[0].options));
+        check(!invalid && invalid.error().code == ErrorCode::InvalidArgument);
+        invalid = BatchGenerationLoop::generate(nullptr, pointers, source, options);
+        check(!invalid && invalid.error().code == ErrorCode::InternalError);
+        check(source.prefill_calls == prefills);
+        // a decode failure ends the run with the model's error
+        source.fail_decode_at = source.decode_calls + 3;
+        auto failed = BatchGenerationLoop::generate(sampler, pointers, source, options);
+        check(!failed && failed.error().message == "synthetic decode failure");
+    }
+}
+
+// Prints "session index token_id probability_bits is_stop" per emitted token and a summary line per
+// Session; tests/test_gpu_generation_loop.py recomputes the run with the CPU sampler.
+static int print_generation_trace(const HipSamplerPtr& sampler)
+{
+    const std::vector<LoopCase> cases = loop_cases();
+    std::deque<SamplingSession> sessions;
+    make_sessions(sampler, cases, sessions);
+    SyntheticSource source(kLoopVocab, static_cast<uint32_t>(cases.size()));
+    const std::vector<GenerationResult> results = run_loop(sampler, cases, sessions, source);
+    for (size_t i = 0; i < results.size(); ++i)
+    {
+        const GenerationOptions& options = cases[i].options;
+        std::printf("session %zu seed %llu max_new_tokens %u temperature_bits %u top_k %u top_p_bits %u min_p_bits %u stops",
+                    i, static_cast<unsigned long long>(cases[i].seed), options.max_new_tokens,
+                    std::bit_cast<uint32_t>(options.sampling.temperature), options.sampling.top_k,
+                    std::bit_cast<uint32_t>(options.sampling.top_p), std::bit_cast<uint32_t>(options.sampling.min_p));
+        for (int32_t id : options.stop_tokens)
+            std::printf(" %d", id);
+        std::printf("\n");
+        for (const StreamToken& token : results[i].tokens)
+            std::printf("token %zu %u %d %u %d\n", i, token.index, token.token_id, std::bit_cast<uint32_t>(token.probability),
+                        token.is_stop_token ? 1 : 0);
+        std::printf("result %zu tokens %zu stopped_by_stop_token %d stopped_by_callback %d\n", i, results[i].tokens.size(),
+                    results[i].stopped_by_stop_token ? 1 : 0, results[i].stopped_by_callback ? 1 : 0);
+    }
+    std::printf("vocab %u\n", kLoopVocab);
+    return 0;
+}
+
+// A model whose decode step costs nothing: the rows written at prefill stay in the buffer, as if a
+// decode step on the GPU had just produced them.  What remains is the loop itself: one device call per
+// token index over device-resident logits, and the host bookkeeping around it.
+class ResidentSource : public IDeviceLogitsSource
+{
+public:
+    explicit ResidentSource(uint32_t vocab) : vocab_(vocab) {}
+    uint32_t vocabulary_size() const override { return vocab_; }
+
+    Result<bool> prefill(std::span<const uint32_t> session_indices, const DeviceLogitsRows& rows) override
+    {
+        const auto started = std::chrono::steady_clock::now();
+        for (size_t row = 0; row < session_indices.size(); ++row)
+        {
+            const std::vector<float> values = synthetic_logits(vocab_, session_indices[row], 0, -1);
+            float* target = static_cast<float*>(rows.data) + row * rows.row_stride;
+            if (hipMemcpy(target, values.data(), values.size() * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
+                return Error{ErrorCode::InternalError, "resident source: hipMemcpy failed"};
+        }
+        prefill_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - started).count();
+        return true;
+    }
+
+    Result<bool> decode(std::span<const DecodeSlot>, const DeviceLogitsRows&) override { return true; }
+
+    double prefill_seconds = 0.0;
+
+private:
+    uint32_t vocab_;
+};
+
+// --generation-bench SESSIONS VOCAB STEPS: times BatchGenerationLoop::generate and prints one line.
+static int generation_bench(uint32_t session_count, uint32_t vocab, uint32_t steps)
+{
+    HipSamplerPtr sampler = HipSampler::create(0, session_count, vocab);
+    if (!sampler)
+    {
+        std::fprintf(stderr, "HipSampler::create failed: no usable GPU\n");
+        return 2;
+    }
+    GenerationOptions options;
+    options.sampling = SamplingOptions{0.7f, 20, 0.8f, 0.0f};
+    double seconds = 0.0;
+    double prefill_seconds = 0.0;
+    uint64_t tokens = 0;
+    uint64_t sample_time_microseconds = 0;
+    int32_t first_token = -1;
+    uint32_t first_probability_bits = 0;
+    for (int pass = 0; pass < 2; ++pass) // the first pass warms up
+    {
+        std::deque<SamplingSession> sessions;
+        std::vector<SamplingSession*> pointers;
+        for (uint32_t i = 0; i < session_count; ++i)
+            pointers.push_back(&sessions.emplace_back(sampler, SamplingSessionOptions{1000 + i}));
+        options.max_new_tokens = pass == 0 ? 20 : steps;
+        ResidentSource source(vocab);
+        const auto started = std::chrono::steady_clock::now();
+        auto generated = BatchGenerationLoop::generate(sampler, pointers, source, std::vector<GenerationOptions>{options});
+        seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - started).count();
+        if (!generated)
+        {
+            std::fprintf(stderr, "generation failed: %s\n", generated.error().message.c_str());
+            return 1;
+        }
+        prefill_seconds = source.prefill_seconds;
+        tokens = 0;
+        for (const GenerationResult& result : generated.value())
+            tokens += result.tokens.size();
+        sample_time_microseconds = sessions.front().statistics().sample_time_microseconds;
+        first_token = generated.value()[0].tokens[0].token_id;
+        first_probability_bits = std::bit_cast<uint32_t>(generated.value()[0].tokens[0].probability);
+    }
+    std::printf("generation_bench sessions %u vocab %u steps %u tokens %llu seconds %.6f prefill_seconds %.6f "
+                "sample_time_microseconds %llu first_token %d first_probability_bits %u\n",
+                session_count, vocab, steps, static_cast<unsigned long long>(tokens), seconds, prefill_seconds,
+                static_cast<unsigned long long>(sample_time_microseconds), first_token, first_probability_bits);
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
+    if (argc == 5 && std::strcmp(argv[1], "--generation-bench") == 0)
+        return generation_bench(static_cast<uint32_t>(std::atoi(argv[2])), static_cast<uint32_t>(std::atoi(argv[3])),
+                                static_cast<uint32_t>(std::atoi(argv[4])));
     const bool host_only = argc > 1 && std::strcmp(argv[1], "--host") == 0;
+    const bool trace_only = argc > 1 && std::strcmp(argv[1], "--generation-trace") == 0;
     try
     {
         test_option_validation_messages();
@@ -432,12 +817,16 @@ int main(int argc, char** argv)
             std::fprintf(stderr, "HipSampler::create failed: no usable GPU\n");
             return 2;
         }
+        if (trace_only)
+            return print_generation_trace(sampler);
         test_sampling_like_the_runtime_test(sampler);
         test_rng_bookkeeping(sampler);
         test_distribution_known_answers(sampler);
         test_batch_equals_serial(sampler);
         test_batch_rejects_bad_requests(sampler);
         test_speculative_verification(sampler);
+        test_generation_loop_equals_serial(sampler);
+        test_generation_loop_callback_and_errors(sampler);
     }
     catch (const std::exception& error)
     {
