@@ -10,6 +10,8 @@
 //                                             model below and prints every emitted token, for a
 //                                             checker that recomputes the run with the CPU sampler
 #include "hip_session_sampler.h"
+#include "synthetic_model.h"
+#include "worker_wire.h"
 
 #include <hip/hip_runtime_api.h>
 
@@ -423,30 +425,118 @@ static void test_speculative_verification(const HipSamplerPtr& sampler)
     }
 }
 
-// ---- batched generation loop ----------------------------------------------------------------
+// ---- worker wire format (host only) -----------------------------------------------------------
 
-// A stand-in for the model: the logits after a Session's position p depend on (session, p, token fed)
-// through an integer hash, every value a multiple of 2^-20 in [-8, 14), so a checker in another
-// language reproduces them exactly.  It writes device rows, as a decode step on the GPU would.
-static std::vector<float> synthetic_logits(uint32_t vocab, uint32_t session, uint32_t position, int32_t fed_token)
+static void test_wire_generate_request_defaults_and_fields()
 {
-    const uint32_t seed = (session * 0x9E3779B1u) ^ (position * 0x85EBCA77u) ^ (static_cast<uint32_t>(fed_token) * 0xC2B2AE3Du) ^ 0x27D4EB2Fu;
-    std::vector<float> row(vocab);
-    for (uint32_t v = 0; v < vocab; ++v)
-    {
-        uint32_t h = v * 2654435761u + seed;
-        h ^= h >> 15;
-        h *= 2246822519u;
-        h ^= h >> 13;
-        h *= 3266489917u;
-        h ^= h >> 16;
-        float value = static_cast<float>(h >> 8) * (1.0f / 1048576.0f) - 8.0f;
-        if ((h & 1023u) == 0u)
-            value += 6.0f;
-        row[v] = value;
-    }
-    return row;
+    // the request tools/ncnn_moe_protocol.py sends
+    const std::string line =
+        "{\"op\": \"generate\", \"request_id\": \"r1\", \"session_id\": \"s\", \"prompt_tokens\": [1, 2, 3], "
+        "\"max_new_tokens\": 16, \"temperature\": 0.7, \"top_k\": 20, \"top_p\": 0.8, \"min_p\": 0.0, "
+        "\"stop_tokens\": [5, 151645], \"enable_speculative\": true, \"speculative_confidence\": 0.5, "
+        "\"speculative_max_draft\": 0, \"metrics_enabled\": true, \"metrics_interval_ms\": 1000}";
+    const wire::GenerateRequest parsed = wire::parse_generate_request(line);
+    check(parsed.request_id == "r1" && parsed.session_id == "s");
+    check(parsed.prompt_tokens == std::vector<int32_t>({1, 2, 3}));
+    check(parsed.options.max_new_tokens == 16);
+    check(parsed.options.sampling.temperature == 0.7f && parsed.options.sampling.top_k == 20);
+    check(parsed.options.sampling.top_p == 0.8f && parsed.options.sampling.min_p == 0.0f);
+    check(parsed.options.stop_tokens == std::vector<int32_t>({5, 151645}));
+
+    // what the worker assumes for absent fields: greedy, one token, the default ids
+    const wire::GenerateRequest bare = wire::parse_generate_request("{\"op\":\"generate\",\"prompt_tokens\":[7]}");
+    check(bare.request_id == "generate" && bare.session_id == "main");
+    check(bare.options.max_new_tokens == 1 && bare.options.sampling.temperature == 0.0f);
+    check(bare.options.sampling.top_k == 0 && bare.options.sampling.top_p == 1.0f && bare.options.sampling.min_p == 0.0f);
+    check(bare.options.stop_tokens.empty());
+
+    // top_k is read from an integer literal only; a temperature may be written as an integer
+    const wire::GenerateRequest odd = wire::parse_generate_request("{\"prompt_tokens\":[7],\"top_k\":20.0,\"temperature\":1}");
+    check(odd.options.sampling.top_k == 0 && odd.options.sampling.temperature == 1.0f);
+
+    const auto message_of = [](const char* text) {
+        try
+        {
+            (void)wire::parse_generate_request(text);
+        }
+        catch (const std::invalid_argument& error)
+        {
+            return std::string(error.what());
+        }
+        return std::string();
+    };
+    check(message_of("{\"op\":\"generate\"}") == "prompt_tokens must be an integer array");
+    check(message_of("{\"prompt_tokens\":[]}") == "prompt_tokens must not be empty");
+    check(message_of("{\"prompt_tokens\":[1, \"a\"]}") == "prompt_tokens must be an integer array");
+    check(message_of("{\"prompt_tokens\":[1],\"stop_tokens\":[4294967296]}") == "stop_tokens contains an out-of-range token ID");
+    check(message_of("{\"prompt_tokens\":[1],\"top_k\":-1}") == "top_k is outside the uint32 range");
+    check(message_of("{\"prompt_tokens\":[1],\"max_new_tokens\":4294967296}") == "max_new_tokens is outside the uint32 range");
+    check(!message_of("[1, 2]").empty());
 }
+
+static void test_wire_events()
+{
+    StreamToken token;
+    token.index = 3;
+    token.token_id = 151645;
+    token.probability = 0.33816584944725037f;
+    token.is_stop_token = true;
+    check(wire::token_event("r\"1", "main", token, 0.125) ==
+          "{\"event\":\"token\",\"request_id\":\"r\\\"1\",\"session_id\":\"main\",\"index\":3,\"token_id\":151645,"
+          "\"probability\":0.3381658494,\"is_stop_token\":true,\"elapsed_seconds\":0.125}");
+    token.probability = 1.0f;
+    token.token_id = -1;
+    token.is_stop_token = false;
+    check(wire::token_event("g", "s", token, 2.0).find("\"token_id\":-1,\"probability\":1,\"is_stop_token\":false,\"elapsed_seconds\":2}") != std::string::npos);
+    token.probability = 1.0e-7f;
+    check(wire::token_event("g", "s", token, 0.0).find("\"probability\":1.000000012e-07,") != std::string::npos);
+    token.probability = std::numeric_limits<float>::quiet_NaN();
+    check(wire::token_event("g", "s", token, 0.0).find("\"probability\":null,") != std::string::npos);
+
+    check(wire::error_event("r1", "top_p must be in the range (0, 1]", wire::error_code_name(ErrorCode::InvalidArgument)) ==
+          "{\"event\":\"error\",\"request_id\":\"r1\",\"code\":\"invalid_argument\",\"message\":\"top_p must be in the range (0, 1]\"}");
+    check(wire::error_event("", "line\nbreak") == "{\"event\":\"error\",\"code\":\"invalid_request\",\"message\":\"line\\nbreak\"}");
+    check(std::string(wire::error_code_name(ErrorCode::InternalError)) == "internal_error");
+    check(std::string(wire::error_code_name(ErrorCode::InvalidModel)) == "invalid_model");
+
+    GenerationResult generation;
+    generation.tokens.resize(4);
+    generation.stopped_by_stop_token = true;
+    SamplingStatistics statistics{4, 4, 180};
+    check(wire::done_event("r1", "main", generation, false, 0.5, 9, statistics) ==
+          "{\"event\":\"done\",\"request_id\":\"r1\",\"session_id\":\"main\",\"ok\":true,\"metrics_enabled\":false,"
+          "\"generated_tokens\":4,\"stopped_by_stop_token\":true,\"stopped_by_callback\":false,\"cancelled\":false,"
+          "\"elapsed_seconds\":0.5,\"tokens_per_second\":8,\"sequence_length\":9,"
+          "\"sampling\":{\"sampled_tokens\":4,\"sample_calls\":4,\"sample_time_microseconds\":180}}");
+}
+
+static void test_wire_request_fields()
+{
+    const wire::RequestFields fields(
+        " { \"a\" : \"x\\ty\\u0041\" , \"n\":-12, \"f\": 2.5e-1, \"t\":true, \"z\":null, \"arr\":[ 1 ,2,\n3 ], "
+        "\"nested\":{\"a\":\"inner\",\"arr\":[9]}, \"empty\":[] } ");
+    check(fields.string("a").value() == "x\tyA");
+    check(fields.integer("n").value() == -12 && fields.number("n").value() == -12.0);
+    check(!fields.integer("f") && fields.number("f").value() == 0.25);
+    check(fields.boolean("t").value() && !fields.boolean("n"));
+    check(!fields.string("z") && !fields.number("z") && !fields.string("missing"));
+    check(fields.integer_array("arr").value() == std::vector<int64_t>({1, 2, 3}));
+    check(fields.integer_array("empty").value().empty());
+    check(!fields.integer_array("a") && !fields.integer_array("nested"));
+    check(!fields.string("inner")); // members of nested objects are not members of the request
+    bool thrown = false;
+    try
+    {
+        wire::RequestFields broken("{\"a\": [1, 2");
+    }
+    catch (const std::invalid_argument&)
+    {
+        thrown = true;
+    }
+    check(thrown);
+}
+
+// ---- batched generation loop ----------------------------------------------------------------
 
 class SyntheticSource : public IDeviceLogitsSource
 {
@@ -806,6 +896,9 @@ int main(int argc, char** argv)
         test_defaults_match_the_runtime();
         test_peek_uniform_does_not_advance();
         test_missing_sampler_fails_loudly();
+        test_wire_generate_request_defaults_and_fields();
+        test_wire_events();
+        test_wire_request_fields();
         if (host_only)
         {
             std::printf("all host-side session sampler tests passed\n");
