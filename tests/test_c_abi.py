@@ -115,3 +115,21 @@ def test_host_mirror_on_gpu():
     done = subprocess.run([TEST_PROGRAM], capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stdout + done.stderr
     assert "all session sampler tests passed" in done.stdout
+
+
+DISPATCHER_TEST_PROGRAM = os.path.join(PACKAGE_DIR, "test_expert_dispatcher")
+
+
+def test_dispatcher_mirror_host_only_tests():
+    assert os.path.exists(DISPATCHER_TEST_PROGRAM), "build it with make -C ncnn-moe-runtime_amd"
+    done = subprocess.run([DISPATCHER_TEST_PROGRAM, "--host"], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "all host-side expert dispatcher tests passed" in done.stdout
+
+
+@pytest.mark.gpu
+def test_dispatcher_mirror_on_gpu():
+    print("[case] C++ expert dispatcher mirror test program", flush=True)
+    done = subprocess.run([DISPATCHER_TEST_PROGRAM], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "all expert dispatcher tests passed" in done.stdout
