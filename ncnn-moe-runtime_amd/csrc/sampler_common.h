@@ -108,6 +108,7 @@ __device__ __forceinline__ void finish_row_wave(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
     float value, int32_t index, int n, int lane, uint8_t flags)
 {
+    n = __builtin_amdgcn_readfirstlane(n); // the same in every lane: the loops over it stay scalar
     const float temperature = p.temperature;
     const float top_value = read_lane(value, 0);
     const float maximum = top_value / temperature;
@@ -115,9 +116,19 @@ __device__ __forceinline__ void finish_row_wave(
     if (lane < n)
         term = expf_libm(value / temperature - maximum);
 
+    // The three walks below are the CPU's sequential fp32 sums.  They run in trips of four candidates
+    // without a data-dependent exit: a lane past the end (or a filtered candidate) adds +0.0, which
+    // leaves a non-negative sum as it is, and every lane keeps the running sum at its own position, so
+    // that where the CPU loop would have stopped is read off afterwards with one ballot.  (A loop
+    // trip costs about as much as ten of these instructions.)
+    const int trips = (n + 3) >> 2;
     float normalizer = 0.0f;
-    for (int i = 0; i < n; ++i)
-        normalizer += read_lane(term, i);
+    for (int trip = 0; trip < trips; ++trip)
+    {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            normalizer += read_lane(term, trip * 4 + k);
+    }
     if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
     {
         if (lane == 0)
@@ -132,23 +143,29 @@ __device__ __forceinline__ void finish_row_wave(
         const float threshold = read_lane(probability, 0) * p.min_p;
         keep = keep && (probability >= threshold);
     }
-    uint64_t pending = __ballot(keep);
+    const uint64_t keep_mask = __ballot(keep);
 
+    // Top-P: the cumulative sum over the kept candidates in order, up to the first that reaches top_p
+    const float contribution = keep ? probability : 0.0f;
     float cumulative = 0.0f;
-    uint64_t kept_mask = 0;
-    int kept = 0;
-    while (pending != 0)
+    float cumulative_here = 0.0f;
+    for (int trip = 0; trip < trips; ++trip)
     {
-        const int i = __builtin_ctzll(pending);
-        pending &= pending - 1;
-        cumulative += read_lane(probability, i);
-        kept_mask |= 1ull << i;
-        ++kept;
-        if (cumulative >= p.top_p)
-            break;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+            cumulative += read_lane(contribution, trip * 4 + k);
+            cumulative_here = lane == trip * 4 + k ? cumulative : cumulative_here;
+        }
+        if (__ballot(keep && cumulative_here >= p.top_p) != 0)
+            break; // the nucleus is complete: the sums behind it are not needed
     }
+    const uint64_t reached = __ballot(keep && cumulative_here >= p.top_p);
+    const int last = reached != 0 ? __builtin_ctzll(reached) : 63 - __builtin_clzll(keep_mask);
+    const uint64_t kept_mask = keep_mask & ((2ull << last) - 1ull);
+    const int kept = __popcll(kept_mask);
     // The renormaliser of session.cpp:130-132 adds the same values in the same order as the Top-P scan.
-    const float renormalizer = cumulative;
+    const float renormalizer = read_lane(cumulative_here, last);
     const float final_probability = probability / renormalizer;
 
     if (a.distribution_count != nullptr)
@@ -178,20 +195,22 @@ __device__ __forceinline__ void finish_row_wave(
     {
         draw_consumed = 1;
         const float uniform = a.uniforms[row];
+        const bool is_kept = ((kept_mask >> lane) & 1ull) != 0ull;
+        const float share = is_kept ? final_probability : 0.0f;
         float running = 0.0f;
-        uint64_t walk = kept_mask;
-        selected = 63 - __builtin_clzll(kept_mask);
-        while (walk != 0)
+        float running_here = 0.0f;
+        const int draw_trips = (last + 4) >> 2; // positions 0 .. last
+        for (int trip = 0; trip < draw_trips; ++trip)
         {
-            const int i = __builtin_ctzll(walk);
-            walk &= walk - 1;
-            running += read_lane(final_probability, i);
-            if (uniform < running)
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
             {
-                selected = i;
-                break;
+                running += read_lane(share, trip * 4 + k);
+                running_here = lane == trip * 4 + k ? running : running_here;
             }
         }
+        const uint64_t passed = __ballot(is_kept && uniform < running_here);
+        selected = passed != 0 ? __builtin_ctzll(passed) : last; // past the last sum: the last kept candidate
         selected_probability = read_lane(final_probability, selected);
     }
     const int32_t token = read_lane(index, selected);
@@ -208,6 +227,7 @@ __device__ __forceinline__ void finish_row_wave_wide(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
     const float (&value)[SLOTS], const int32_t (&index)[SLOTS], int n, int lane, uint8_t flags)
 {
+    n = __builtin_amdgcn_readfirstlane(n); // the same in every lane: the loops over it stay scalar
     const float temperature = p.temperature;
     const float maximum = read_lane(value[0], 0) / temperature;
     float term[SLOTS];
@@ -461,13 +481,51 @@ __device__ __forceinline__ uint32_t select_kth_key_dispatch(const uint32_t* keys
     return select_kth_key<16>(keys_in_lds, m, top_k, lane);
 }
 
+constexpr int kRowMaxima = kScanThreads / 16; // one per row of 16 lanes
+constexpr int kRowMaximaTopK = 24;            // windows up to here take the bound from the row maxima
+
 struct BoundScratch
 {
+    uint32_t row_maxima[kRowMaxima];
     uint32_t wave_bounds[kScanWaves];
     uint32_t hot_keys[2 * kScanThreads];
     uint32_t hot_total;
     uint32_t result;
 };
+
+// A cheap lower bound of the top_k-th largest of the workgroup's keys (one per thread, each standing
+// for a distinct logit; 0 = no key) that at least top_k keys reach: the top_k-th largest of the 32
+// maxima of the rows of 16 lanes, every maximum being one of the keys.  top_k <= 32 (callers stop at
+// kRowMaximaTopK: beyond it the bound lets too many keys through).  0 when fewer
+// than top_k rows hold a key: the caller then takes the exact routine below.  Looser than the exact
+// top_k-th largest (for top_k = 20 of 10,240 values about 30 reach it instead of 20), at a third of
+// the cost: four exchanges inside the rows, one LDS round trip, a 32-step search.  All threads of the
+// workgroup must call it.
+__device__ __forceinline__ uint32_t workgroup_kth_of_row_maxima(uint32_t key, int top_k, int tid, BoundScratch& scratch)
+{
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    uint32_t row_max = key;
+    row_max = max(row_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(row_max), 0xB1, 0xf, 0xf, true)));  // lanes 1 apart
+    row_max = max(row_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(row_max), 0x4E, 0xf, 0xf, true)));  // lanes 2 apart
+    row_max = max(row_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(row_max), 0x141, 0xf, 0xf, true))); // half-row mirror
+    row_max = max(row_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(row_max), 0x140, 0xf, 0xf, true))); // row mirror
+    if ((lane & 15) == 0)
+        scratch.row_maxima[wave * 4 + (lane >> 4)] = row_max;
+    lds_barrier();
+    // every wave searches the 32 maxima itself, bit by bit (one compare per bit, the counting is
+    // scalar): no second barrier
+    const uint32_t mine = lane < kRowMaxima ? scratch.row_maxima[lane] : 0u;
+    uint32_t prefix = 0;
+#pragma unroll
+    for (int bit = 31; bit >= 0; --bit)
+    {
+        const uint32_t trial = prefix | (1u << bit);
+        if (__popcll(__ballot(mine >= trial)) >= top_k)
+            prefix = trial;
+    }
+    return prefix;
+}
 
 // The top_k-th largest of the workgroup's keys (KEYS per thread, each standing for a distinct
 // logit; 0 = no key), or with exact == false a lower bound of it that at least top_k keys still
@@ -574,6 +632,8 @@ __device__ __forceinline__ int select_best_wave(
     const uint32_t* staged_keys, const int32_t* staged_indices, int m, int top_k, int lane,
     float* final_values, int32_t* final_indices)
 {
+    m = __builtin_amdgcn_readfirstlane(m);
+    top_k = __builtin_amdgcn_readfirstlane(top_k);
     uint32_t keys[R];
 #pragma unroll
     for (int r = 0; r < R; ++r)

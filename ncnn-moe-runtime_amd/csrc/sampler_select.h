@@ -132,7 +132,9 @@ __device__ __forceinline__ void finish_from_list(
 {
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
-    int n_list = static_cast<int>(shared.list_count);
+    // the count comes from LDS: telling the compiler that it is the same in every lane keeps the loops
+    // over it scalar (a loop it takes for divergent costs several times as much per trip)
+    int n_list = __builtin_amdgcn_readfirstlane(static_cast<int>(shared.list_count));
     if (top_k <= kFastTopK)
     {
         if constexpr (WIDE)
@@ -140,7 +142,7 @@ __device__ __forceinline__ void finish_from_list(
             if (n_list > 8 * kWaveSize)
             {
                 tighten_list(shared, 0u, top_k, tid);
-                n_list = static_cast<int>(shared.list_count);
+                n_list = __builtin_amdgcn_readfirstlane(static_cast<int>(shared.list_count));
             }
         }
         if (n_list > 8 * kWaveSize)
@@ -153,21 +155,33 @@ __device__ __forceinline__ void finish_from_list(
             }
             return;
         }
-        if (wave != 0)
-            return;
         int n = 0;
         if (n_list <= kWaveSize)
         {
-            // one candidate per lane: its rank among all of them is its place in the window
+            // one candidate per lane: its rank among all of them is its place in the window.  Every
+            // wave counts the candidates of its eighth of the list that go before the lane's own;
+            // wave 0 adds the eight counts up and goes on alone.
             const uint32_t key = lane < n_list ? shared.list_keys[lane] : 0u;
             const int32_t candidate_index = lane < n_list ? shared.list_indices[lane] : 0;
-            int before = 0;
-            for (int j = 0; j < n_list; ++j)
+            constexpr int kShare = kWaveSize / kScanWaves;
+            int partial = 0;
+#pragma unroll
+            for (int k = 0; k < kShare; ++k)
             {
-                const uint32_t other_key = static_cast<uint32_t>(read_lane(static_cast<int>(key), j));
-                const int32_t other_index = read_lane(candidate_index, j);
-                before += (other_key > key || (other_key == key && other_index < candidate_index)) ? 1 : 0;
+                const int j = wave * kShare + k;
+                const uint32_t other_key = shared.list_keys[j];
+                const int32_t other_index = shared.list_indices[j];
+                partial += (j < n_list && (other_key > key || (other_key == key && other_index < candidate_index))) ? 1 : 0;
             }
+            uint32_t* const partial_counts = shared.bound.hot_keys; // kScanWaves x 64 counts
+            partial_counts[wave * kWaveSize + lane] = static_cast<uint32_t>(partial);
+            __syncthreads();
+            if (wave != 0)
+                return;
+            int before = 0;
+#pragma unroll
+            for (int w = 0; w < kScanWaves; ++w)
+                before += static_cast<int>(partial_counts[w * kWaveSize + lane]);
             if (lane < n_list && before < top_k)
             {
                 shared.final_values[before] = value_from_ascending_key(key);
@@ -187,6 +201,8 @@ __device__ __forceinline__ void finish_from_list(
             finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags);
             return;
         }
+        if (wave != 0)
+            return;
         if (n_list <= 2 * kWaveSize)
             n = select_best_wave<2>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
         else if (n_list <= 4 * kWaveSize)
@@ -204,8 +220,15 @@ __device__ __forceinline__ void finish_from_list(
         float value = lane < n ? shared.final_values[lane] : 0.0f;
         int32_t index = lane < n ? shared.final_indices[lane] : -1;
         int rank = 0;
-        for (int j = 0; j < n; ++j)
-            rank += candidate_before(read_lane(value, j), read_lane(index, j), value, index) ? 1 : 0;
+        for (int trip = 0; trip < (n + 3) >> 2; ++trip)
+        {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                const int j = trip * 4 + k;
+                rank += (j < n && candidate_before(read_lane(value, j), read_lane(index, j), value, index)) ? 1 : 0;
+            }
+        }
         if (lane < n)
         {
             shared.final_values[rank] = value;
@@ -223,7 +246,7 @@ __device__ __forceinline__ void finish_from_list(
         constexpr int kPerThread = SelectShared<WIDE>::kListCap / kScanThreads;
         if (n_list > top_k + 64)
             tighten_list(shared, 0u, top_k, tid); // fewer candidates to rank
-        const int n_ranked = static_cast<int>(shared.list_count);
+        const int n_ranked = __builtin_amdgcn_readfirstlane(static_cast<int>(shared.list_count));
         uint32_t keys[kPerThread];
         int32_t indices[kPerThread];
 #pragma unroll
@@ -478,7 +501,10 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
             else
             {
                 const uint32_t lane_keys[1] = {lane_max == __uint_as_float(kNegativeInfinity) ? 0u : ascending_key(lane_max)};
-                bound_key = max(bound_key, workgroup_kth_largest_key(lane_keys, top_k, tid, shared.bound, true));
+                uint32_t chunk_bound = top_k <= kRowMaximaTopK ? workgroup_kth_of_row_maxima(lane_keys[0], top_k, tid, shared.bound) : 0u;
+                if (chunk_bound == 0u) // a wider window, or a chunk with few values: the exact K-th largest lane maximum
+                    chunk_bound = workgroup_kth_largest_key(lane_keys, top_k, tid, shared.bound, true);
+                bound_key = max(bound_key, chunk_bound);
             }
         }
         // no bound yet (fewer than K lanes hold a finite logit): every finite logit is a candidate
@@ -594,7 +620,8 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     uint32_t* const out_indices = reinterpret_cast<uint32_t*>(a.segment_indices);
     const size_t segment_slot = static_cast<size_t>(row) * a.segments + segment;
     const uint32_t record_entries = segment_record_entries(effective_k);
-    if (LOOPED && !overflow && shared.list_count > record_entries)
+    // the record holds 2K + 16 candidates: a longer list (a loose bound, ties) is cut to the exact window first
+    if (!overflow && shared.list_count > record_entries)
         bound_key = tighten_list(shared, bound_key, top_k, tid);
     const uint32_t handed = shared.list_count;
     overflow = overflow || handed > record_entries;
@@ -670,7 +697,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         loaded_keys[j] = (q < row_entries && r < loaded_counts[j]) ? loaded_keys[j] : 0u;
         thread_key[0] = max(thread_key[0], loaded_keys[j]);
     }
-    if (__syncthreads_or(too_many ? 1 : 0))
+    if (too_many) // the same in every thread: the row's flags and the segment count
     {
         // ties (or a very long row) left more candidates than the merge holds: the full-order kernels take the row
         if (tid == 0)
@@ -690,7 +717,9 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         return;
     }
     // prune: at least K candidates reach this lower bound of the K-th largest per-thread best
-    const uint32_t prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, shared.bound, true);
+    uint32_t prune_key = top_k <= kRowMaximaTopK ? workgroup_kth_of_row_maxima(thread_key[0], top_k, tid, shared.bound) : 0u;
+    if (prune_key == 0u)
+        prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, shared.bound, true);
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
         append_candidate(shared, loaded_keys[j] != 0u && loaded_keys[j] >= prune_key, loaded_keys[j],

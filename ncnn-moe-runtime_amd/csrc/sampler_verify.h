@@ -97,8 +97,8 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
                     write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ROW_ERROR, row_status, accept_draws, 0, 0);
                 return;
             }
-            const uint32_t target_count = v.distribution_count[target_row];
-            const uint32_t draft_count = v.distribution_count[draft_row];
+            const uint32_t target_count = __builtin_amdgcn_readfirstlane(v.distribution_count[target_row]);
+            const uint32_t draft_count = __builtin_amdgcn_readfirstlane(v.distribution_count[draft_row]);
             if (target_count > static_cast<uint32_t>(kVerifyCap) || draft_count > static_cast<uint32_t>(kVerifyCap))
             {
                 // a filtered distribution longer than the step holds: reported, never approximated
