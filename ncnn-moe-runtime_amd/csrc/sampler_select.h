@@ -656,28 +656,32 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         return;
 
     // ---- last workgroup of the row: every load of the merge is issued before any is used (one trip)
+    // Thread slot q stands for entry q / 16 of segment q % 16: no division by the record length, and
+    // every row of 16 lanes sees one entry of each segment, so the candidates are spread evenly over
+    // the lanes (which is what the prune's bound from row maxima needs).
+    static_assert(kMaxSegments == 16, "the merge maps a thread slot to (entry, segment) with a shift by 4");
     const size_t row_slot = static_cast<size_t>(row) * a.segments;
-    const uint32_t row_entries = a.segments * record_entries;
+    const uint32_t row_entries = record_entries * static_cast<uint32_t>(kMaxSegments);
     constexpr int kPerThread = kMergeStageSlots / kScanThreads;
     uint32_t loaded_keys[kPerThread];
     uint32_t loaded_indices[kPerThread];
-    uint32_t loaded_counts[kPerThread];
     const uint32_t row_flags = load_agent(&a.row_flags[row]);
-    const bool stageable = row_entries <= static_cast<uint32_t>(kMergeStageSlots);
+    const bool stageable = row_entries <= static_cast<uint32_t>(kMergeStageSlots) && a.segments <= static_cast<uint32_t>(kMaxSegments);
+    // all of a thread's slots belong to one segment (the workgroup's size is a multiple of 16)
+    const uint32_t s = static_cast<uint32_t>(tid) & static_cast<uint32_t>(kMaxSegments - 1);
+    const bool segment_exists = stageable && s < a.segments;
+    const uint32_t segment_count = segment_exists ? load_agent(&a.segment_counts[row_slot + s]) : 0u;
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
     {
         const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
+        const uint32_t r = q >> 4;
         loaded_keys[j] = 0;
         loaded_indices[j] = 0;
-        loaded_counts[j] = 0;
-        if (stageable && q < row_entries)
+        if (segment_exists && q < row_entries)
         {
-            const uint32_t s = q / record_entries;
-            const uint32_t r = q - s * record_entries;
             loaded_keys[j] = load_agent(&out_values[(row_slot + s) * kSegmentRecordSlots + r]);
             loaded_indices[j] = load_agent(&out_indices[(row_slot + s) * kSegmentRecordSlots + r]);
-            loaded_counts[j] = load_agent(&a.segment_counts[row_slot + s]);
         }
     }
     const uint8_t result_flags = (row_flags & kScanSawNan) ? NCNN_MOE_ROW_FLAG_HAS_NAN : 0;
@@ -692,9 +696,8 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
     {
-        const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
-        const uint32_t r = q % record_entries;
-        loaded_keys[j] = (q < row_entries && r < loaded_counts[j]) ? loaded_keys[j] : 0u;
+        const uint32_t r = static_cast<uint32_t>(j * kScanThreads + tid) >> 4;
+        loaded_keys[j] = r < segment_count ? loaded_keys[j] : 0u; // a segment that does not exist has count 0
         thread_key[0] = max(thread_key[0], loaded_keys[j]);
     }
     if (too_many) // the same in every thread: the row's flags and the segment count
