@@ -193,7 +193,9 @@ def bench_router_dispatch(args):
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU: no HIP device is visible")
     tokens = args.rows if args.rows > 0 else 4096
-    experts, top_k, score, scaling = 256, 8, hip_router.SQRT_SOFTPLUS, 1.5
+    score_name = args.router_score
+    experts, top_k, scaling = 256, 8, 1.5
+    score = {"softmax": hip_router.SOFTMAX, "sigmoid": hip_router.SIGMOID, "sqrt_softplus": hip_router.SQRT_SOFTPLUS}[score_name]
     rng = np.random.Generator(np.random.PCG64(88))
     buffers = 16
     host_logits = [(rng.standard_normal((tokens, experts), dtype=np.float32) * np.float32(2.0)) for _ in range(buffers)]
@@ -245,12 +247,12 @@ def bench_router_dispatch(args):
     bytes_per_step = tokens * experts * 4 + experts * 4 + tokens * top_k * 12 + (experts + 1) * 4 + 4
     cpu_best = min(cpu_seconds)
     line = {
-        "metric": "expert dispatch tokens/sec, %d experts Top-%d sqrt-softplus + bias, fp32 router logits" % (experts, top_k),
+        "metric": "expert dispatch tokens/sec, %d experts Top-%d %s + bias, fp32 router logits" % (experts, top_k, score_name),
         "value": tokens / seconds_per_step, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": seconds_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "expert dispatch of one MoE layer: %d tokens x %d experts, Top-%d, sqrt-softplus scores, "
-                               "selection bias, scaling %.1f; logits resident in HBM" % (tokens, experts, top_k, scaling),
+        "config": {"workload": "expert dispatch of one MoE layer: %d tokens x %d experts, Top-%d, %s scores, "
+                               "selection bias, scaling %.1f; logits resident in HBM" % (tokens, experts, top_k, score_name, scaling),
                    "entry_point": "ncnn_moe_hip_router_dispatch_device (no host synchronisation inside the timed region)"},
         "roofline": {"bound": "hbm", "achieved": bytes_per_step / device_seconds_per_step / 1e9, "peak": HBM_PEAK_BYTES_PER_S / 1e9,
                      "unit": "GB/s", "frac": bytes_per_step / device_seconds_per_step / HBM_PEAK_BYTES_PER_S, "traffic": None,
@@ -329,6 +331,8 @@ def main():
     parser.add_argument("--warmup", type=int, default=200)
     parser.add_argument("--workload", default="cfg2_topk_topp")
     parser.add_argument("--rows", type=int, default=0, help="batch rows (0: the configuration's own)")
+    parser.add_argument("--router-score", default="sqrt_softplus", choices=["softmax", "sigmoid", "sqrt_softplus"],
+                        help="score function of --workload router_dispatch")
     parser.add_argument("--drafts", type=int, default=5, help="drafted tokens per step of --workload speculative_verify")
     parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
     parser.add_argument("--cpu-rows", type=int, default=64)

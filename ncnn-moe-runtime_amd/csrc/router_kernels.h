@@ -201,9 +201,15 @@ __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterS
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
         {
+            // in trips of eight (a loop trip of a lone wave costs as much as a dozen additions); the
+            // lanes past the last expert hold 0, which leaves the sum as it is
             const int slot_count = min(kWaveSize, experts - s * kWaveSize);
-            for (int l = 0; l < slot_count; ++l)
-                sum += read_lane(score[s], l);
+            for (int trip = 0; trip * 8 < slot_count; ++trip)
+            {
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    sum += read_lane(score[s], trip * 8 + k);
+            }
         }
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)

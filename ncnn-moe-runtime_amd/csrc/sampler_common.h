@@ -239,9 +239,14 @@ __device__ __forceinline__ void finish_row_wave_wide(
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s)
     {
+        // in trips of eight: a lane past the end holds +0.0, which leaves the sum as it is
         const int slot_count = min(kWaveSize, n - s * kWaveSize);
-        for (int l = 0; l < slot_count; ++l)
-            normalizer += read_lane(term[s], l);
+        for (int trip = 0; trip * 8 < slot_count; ++trip)
+        {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                normalizer += read_lane(term[s], trip * 8 + k);
+        }
     }
     if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
     {
@@ -263,34 +268,57 @@ __device__ __forceinline__ void finish_row_wave_wide(
         keep[s] = __ballot(kept);
     }
 
-    // Top-P (session.cpp:119-128); the renormaliser of :130-132 adds the same values in the same order
+    // Top-P (session.cpp:119-128); the renormaliser of :130-132 adds the same values in the same order.
+    // The walk runs in trips of eight candidates: a filtered candidate adds +0.0, every lane keeps the
+    // running sum at its own position, and one ballot per trip tells whether a kept candidate has
+    // reached top_p (a loop trip of a lone wave costs as much as a dozen of these instructions).
     float cumulative = 0.0f;
-    int kept_count = 0;
+    float cumulative_here[SLOTS];
     int last_slot = 0, last_lane = 0;
     bool reached = false;
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s)
     {
-        uint64_t pending = reached ? 0ull : keep[s];
-        uint64_t taken = 0;
-        while (pending != 0)
+        cumulative_here[s] = 0.0f;
+        const float contribution = ((keep[s] >> lane) & 1ull) ? probability[s] : 0.0f;
+        const int slot_count = reached ? 0 : min(kWaveSize, n - s * kWaveSize);
+        for (int trip = 0; trip * 8 < slot_count; ++trip)
         {
-            const int l = __builtin_ctzll(pending);
-            pending &= pending - 1;
-            cumulative += read_lane(probability[s], l);
-            taken |= 1ull << l;
-            ++kept_count;
-            last_slot = s;
-            last_lane = l;
-            if (cumulative >= p.top_p)
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+            {
+                cumulative += read_lane(contribution, trip * 8 + k);
+                cumulative_here[s] = lane == trip * 8 + k ? cumulative : cumulative_here[s];
+            }
+            const uint64_t crossing = __ballot(((keep[s] >> lane) & 1ull) != 0ull && cumulative_here[s] >= p.top_p);
+            if (crossing != 0)
             {
                 reached = true;
+                last_slot = s;
+                last_lane = __builtin_ctzll(crossing);
                 break;
             }
         }
-        keep[s] = taken;
+        if (!reached && keep[s] != 0)
+        {
+            last_slot = s; // so far the walk ends at the last kept candidate
+            last_lane = 63 - __builtin_clzll(keep[s]);
+        }
     }
-    const float renormalizer = cumulative;
+    int kept_count = 0;
+    float renormalizer = 0.0f;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+    {
+        if (s == last_slot)
+        {
+            keep[s] &= (2ull << last_lane) - 1ull;
+            renormalizer = read_lane(cumulative_here[s], last_lane);
+        }
+        else if (s > last_slot)
+            keep[s] = 0;
+        kept_count += __popcll(keep[s]);
+    }
     float final_probability[SLOTS];
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s)
@@ -329,16 +357,23 @@ __device__ __forceinline__ void finish_row_wave_wide(
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
         {
-            uint64_t walk = found ? 0ull : keep[s];
-            while (walk != 0)
+            float running_here = 0.0f;
+            const bool is_kept = ((keep[s] >> lane) & 1ull) != 0ull;
+            const float share = is_kept ? final_probability[s] : 0.0f;
+            const int slot_count = (found || keep[s] == 0) ? 0 : 64 - __builtin_clzll(keep[s]); // up to the last kept candidate
+            for (int trip = 0; trip * 8 < slot_count; ++trip)
             {
-                const int l = __builtin_ctzll(walk);
-                walk &= walk - 1;
-                running += read_lane(final_probability[s], l);
-                if (uniform < running)
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                {
+                    running += read_lane(share, trip * 8 + k);
+                    running_here = lane == trip * 8 + k ? running : running_here;
+                }
+                const uint64_t passed = __ballot(is_kept && uniform < running_here);
+                if (passed != 0)
                 {
                     selected_slot = s;
-                    selected_lane = l;
+                    selected_lane = __builtin_ctzll(passed);
                     found = true;
                     break;
                 }

@@ -179,13 +179,19 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
                     const int i = s * kWaveSize + lane;
                     residual[s] = i < n ? shared.ordered_residual[i] : 0.0f;
                 }
+                // the sums run in trips of eight entries (a loop trip of a lone wave costs as much as a
+                // dozen additions); an entry past the end holds +0.0, which leaves a sum as it is
                 float normalizer = 0.0f;
 #pragma unroll
                 for (int s = 0; s < kVerifySlots; ++s)
                 {
                     const int slot_count = min(kWaveSize, n - s * kWaveSize);
-                    for (int l = 0; l < slot_count; ++l)
-                        normalizer += read_lane(residual[s], l);
+                    for (int trip = 0; trip * 8 < slot_count; ++trip)
+                    {
+#pragma unroll
+                        for (int k = 0; k < 8; ++k)
+                            normalizer += read_lane(residual[s], trip * 8 + k);
+                    }
                 }
                 if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
                 {
@@ -201,19 +207,28 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
 #pragma unroll
                 for (int s = 0; s < kVerifySlots; ++s)
                 {
+                    // every lane keeps the running sum at its own entry; one ballot per trip tells
+                    // whether the draw has been passed (the first entry that passes it holds mass)
+                    float cumulative_here = 0.0f;
                     const int slot_count = selected >= 0 ? 0 : min(kWaveSize, n - s * kWaveSize);
-                    for (int l = 0; l < slot_count; ++l)
+                    for (int trip = 0; trip * 8 < slot_count; ++trip)
                     {
-                        const float value = read_lane(residual[s], l);
-                        cumulative += value;
-                        if (value > 0.0f)
-                            last_positive = s * kWaveSize + l;
-                        if (sample_value < cumulative)
+#pragma unroll
+                        for (int k = 0; k < 8; ++k)
                         {
-                            selected = s * kWaveSize + l;
+                            cumulative += read_lane(residual[s], trip * 8 + k);
+                            cumulative_here = lane == trip * 8 + k ? cumulative : cumulative_here;
+                        }
+                        const uint64_t passed = __ballot(lane < (trip + 1) * 8 && sample_value < cumulative_here);
+                        if (passed != 0)
+                        {
+                            selected = s * kWaveSize + __builtin_ctzll(passed);
                             break;
                         }
                     }
+                    const uint64_t positive = __ballot(residual[s] > 0.0f);
+                    if (selected < 0 && slot_count > 0 && positive != 0)
+                        last_positive = s * kWaveSize + 63 - __builtin_clzll(positive);
                 }
                 if (selected < 0)
                     selected = last_positive; // session.cpp:189-198: the last token that has any residual mass
