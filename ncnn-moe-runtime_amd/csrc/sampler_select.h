@@ -510,27 +510,45 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         // no bound yet (fewer than K lanes hold a finite logit): every finite logit is a candidate
         const float threshold = bound_key == 0u ? -3.402823466e+38f : fmaxf(value_from_ascending_key(bound_key), -3.402823466e+38f);
 
-        // ---- collect the values at or above the bound; only vectors whose maximum reaches it are looked at
+        // ---- collect the values at or above the bound.  Nearly every lane that holds a candidate holds
+        // exactly one, its maximum: each lane counts its candidates and locates its maximum without a
+        // branch, and one append per wave takes the maxima.  The lanes that hold more hand the others
+        // over one per round (a round per extra candidate of the fullest lane; usually none).
+        int lane_hits = 0;
+        int best_at = 0;
 #pragma unroll
-        for (int v = 0; v < kVectors; ++v)
+        for (int i = 0; i < kLaneValues; ++i)
         {
-            // the vector's maximum is recomputed here rather than kept across the bound computation
-            float vector_max = values[v * kWidth];
+            lane_hits += values[i] >= threshold ? 1 : 0;
+            best_at = values[i] == lane_max ? i : best_at;
+        }
+        const auto element_of = [&](int i) {
+            return static_cast<int32_t>(chunk_base + static_cast<uint32_t>((i / kWidth) * kScanThreads + tid) * kWidth +
+                                        static_cast<uint32_t>(i % kWidth) - misalignment);
+        };
+        append_candidate(shared, lane_hits >= 1, ascending_key(lane_max), element_of(best_at), lane);
+        if (__ballot(lane_hits > 1) != 0)
+        {
+            uint32_t rest = 0; // bit i: value i is a candidate that has not been appended
 #pragma unroll
-            for (int c = 1; c < kWidth; ++c)
-                vector_max = fmaxf(vector_max, values[v * kWidth + c]);
-            const bool vector_hit = (LOOPED ? group_max[v] : vector_max) >= threshold;
-            if (__ballot(vector_hit) != 0)
+            for (int i = 0; i < kLaneValues; ++i)
+                rest |= (lane_hits > 1 && values[i] >= threshold && i != best_at) ? (1u << i) : 0u;
+            while (__ballot(rest != 0u) != 0)
             {
-#pragma unroll
-                for (int c = 0; c < kWidth; ++c)
+                // the value is read back from the row (it sits in a register whose number is not known
+                // until run time; this path is rare and the line is in the cache)
+                const int i = rest != 0u ? __builtin_ctz(rest) : 0;
+                const int32_t element = element_of(i);
+                float x = 0.0f;
+                if (rest != 0u)
                 {
-                    const float x = values[v * kWidth + c];
-                    const uint32_t element = chunk_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth + c - misalignment;
-                    const bool hit = vector_hit && x >= threshold;
-                    if (__ballot(hit) != 0)
-                        append_candidate(shared, hit, ascending_key(x), static_cast<int32_t>(element), lane);
+                    if constexpr (DTYPE == NCNN_MOE_LOGITS_F32)
+                        x = reinterpret_cast<const float*>(row_pointer)[element];
+                    else
+                        x = __uint_as_float(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(row_pointer)[element]) << 16);
                 }
+                append_candidate(shared, rest != 0u, ascending_key(x), element, lane);
+                rest &= rest - 1u;
             }
         }
         if constexpr (!LOOPED)
