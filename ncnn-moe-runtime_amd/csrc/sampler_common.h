@@ -534,7 +534,7 @@ struct BoundScratch
 // kRowMaximaTopK: beyond it the bound lets too many keys through).  0 when fewer
 // than top_k rows hold a key: the caller then takes the exact routine below.  Looser than the exact
 // top_k-th largest (for top_k = 20 of 10,240 values about 30 reach it instead of 20), at a third of
-// the cost: four exchanges inside the rows, one LDS round trip, a 20-step search.  All threads of the
+// the cost: four exchanges inside the rows, one LDS round trip, a 16-step search.  All threads of the
 // workgroup must call it.
 __device__ __forceinline__ uint32_t workgroup_kth_of_row_maxima(uint32_t key, int top_k, int tid, BoundScratch& scratch)
 {
@@ -550,12 +550,12 @@ __device__ __forceinline__ uint32_t workgroup_kth_of_row_maxima(uint32_t key, in
     lds_barrier();
     // every wave searches the 32 maxima itself, bit by bit (one compare per bit, the counting is
     // scalar): no second barrier
-    // The lowest 12 bits are left at zero: a step costs a VALU-to-scalar round trip, and a bound that is
-    // a few thousandths lower lets hardly any more keys through.
+    // The lowest 16 bits are left at zero: a step costs a VALU-to-scalar round trip, and a bound that is
+    // half a percent lower lets hardly any more keys through.
     const uint32_t mine = lane < kRowMaxima ? scratch.row_maxima[lane] : 0u;
     uint32_t prefix = 0;
 #pragma unroll
-    for (int bit = 31; bit >= 12; --bit)
+    for (int bit = 31; bit >= 16; --bit)
     {
         const uint32_t trial = prefix | (1u << bit);
         if (__popcll(__ballot(mine >= trial)) >= top_k)

@@ -743,8 +743,12 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, shared.bound, true);
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
+    {
+        if (static_cast<uint32_t>(j * kScanThreads) >= row_entries)
+            break; // no slot of this or a later round exists (a scalar test: nothing waits for a ballot)
         append_candidate(shared, loaded_keys[j] != 0u && loaded_keys[j] >= prune_key, loaded_keys[j],
                          static_cast<int32_t>(loaded_indices[j]), lane);
+    }
     __syncthreads();
     if (shared.list_count > static_cast<uint32_t>(Shared::kListCap))
     {
