@@ -531,8 +531,8 @@ struct BoundScratch
 // A cheap lower bound of the top_k-th largest of the workgroup's keys (one per thread, each standing
 // for a distinct logit; 0 = no key) that at least top_k keys reach: the top_k-th largest of the 32
 // maxima of the rows of 16 lanes, every maximum being one of the keys.  top_k <= 32 (callers stop at
-// kRowMaximaTopK: beyond it the bound lets too many keys through).  0 when fewer
-// than top_k rows hold a key: the caller then takes the exact routine below.  Looser than the exact
+// kRowMaximaTopK: beyond it the bound lets too many keys through).  0 when top_k exceeds three
+// quarters of the rows that hold a key: the caller then takes the exact routine below.  Looser than the exact
 // top_k-th largest (for top_k = 20 of 10,240 values about 30 reach it instead of 20), at a third of
 // the cost: four exchanges inside the rows, one LDS round trip, a 16-step search.  All threads of the
 // workgroup must call it.
@@ -553,6 +553,11 @@ __device__ __forceinline__ uint32_t workgroup_kth_of_row_maxima(uint32_t key, in
     // The lowest 16 bits are left at zero: a step costs a VALU-to-scalar round trip, and a bound that is
     // half a percent lower lets hardly any more keys through.
     const uint32_t mine = lane < kRowMaxima ? scratch.row_maxima[lane] : 0u;
+    // The bound is only as tight as top_k is small beside the number of rows that hold a key (a short
+    // row fills few of them): beyond three quarters the smallest maxima decide and the exact routine is due.
+    const int rows_with_keys = __popcll(__ballot(mine != 0u));
+    if (top_k * 4 > rows_with_keys * 3)
+        return 0u;
     uint32_t prefix = 0;
 #pragma unroll
     for (int bit = 31; bit >= 16; --bit)

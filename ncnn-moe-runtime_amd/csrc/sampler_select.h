@@ -514,20 +514,27 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         // exactly one, its maximum: each lane counts its candidates and locates its maximum without a
         // branch, and one append per wave takes the maxima.  The lanes that hold more hand the others
         // over one per round (a round per extra candidate of the fullest lane; usually none).
+        // A looped workgroup's bound is tight after its first chunks: most waves then hold no candidate
+        // at all and skip the counting.  (A single-chunk workgroup's waves nearly always hold some.)
+        const bool wave_has_candidates = !LOOPED || __ballot(lane_max >= threshold) != 0;
         int lane_hits = 0;
         int best_at = 0;
-#pragma unroll
-        for (int i = 0; i < kLaneValues; ++i)
+        if (wave_has_candidates)
         {
-            lane_hits += values[i] >= threshold ? 1 : 0;
-            best_at = values[i] == lane_max ? i : best_at;
+#pragma unroll
+            for (int i = 0; i < kLaneValues; ++i)
+            {
+                lane_hits += values[i] >= threshold ? 1 : 0;
+                best_at = values[i] == lane_max ? i : best_at;
+            }
         }
         const auto element_of = [&](int i) {
             return static_cast<int32_t>(chunk_base + static_cast<uint32_t>((i / kWidth) * kScanThreads + tid) * kWidth +
                                         static_cast<uint32_t>(i % kWidth) - misalignment);
         };
-        append_candidate(shared, lane_hits >= 1, ascending_key(lane_max), element_of(best_at), lane);
-        if (__ballot(lane_hits > 1) != 0)
+        if (wave_has_candidates)
+            append_candidate(shared, lane_hits >= 1, ascending_key(lane_max), element_of(best_at), lane);
+        if (wave_has_candidates && __ballot(lane_hits > 1) != 0)
         {
             uint32_t rest = 0; // bit i: value i is a candidate that has not been appended
 #pragma unroll

@@ -406,3 +406,29 @@ def test_bf16_rows_of_few_distinct_values(batch_sampler):
     gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", context="bf16 rows of few distinct values")
     assert ((gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH) != 0).all()
     _check_rows(batch_sampler, logits, params, uniforms, context="the same rows as fp32 (radix sort)")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_windows_around_the_row_maxima_bound(batch_sampler, dtype):
+    """Windows up to 24 take their first bound from the 32 row maxima of a chunk, wider ones from the exact
+    selection over the lane maxima; a chunk with values in fewer than K rows of 16 lanes (a short row, a
+    short last segment) falls back to the exact one.  Every window size on both sides of the switch, on row
+    lengths that fill one lane row, a few, one chunk, and several segments; the select path must serve all."""
+    rng = np.random.default_rng(88)
+    windows = np.array([1, 2, 15, 16, 17, 23, 24, 25, 31, 32, 33, 63, 64], dtype=np.uint32)
+    for vocab in (40, 64, 700, 2049, 10240, 10300, 40000, 100003):
+        rows = len(windows) * 3
+        logits = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+        logits[1::3] = np.round(logits[1::3] * 8) / 8          # ties inside the window
+        logits[2::3, vocab // 2:] = -np.inf                      # half of the row carries nothing
+        params = hip_sampler.make_params(rows, 0.8, 0, 0.9, 0.0)
+        params["top_k"] = np.repeat(windows, 3)
+        params["top_p"][::2] = 1.0
+        uniforms = rng.random(rows).astype(np.float32)
+        data = workloads.float32_to_bf16_bits(logits) if dtype == "bf16" else logits
+        select_rows = np.ones(rows, dtype=bool)
+        select_rows[1::3] = vocab < 5000  # heavy ties on long rows may overflow the lists: allowed to take the sort
+        if dtype == "bf16":
+            select_rows[:] = vocab < 5000   # bf16 rounding makes every row tie-heavy
+        _check_rows(batch_sampler, data, params, uniforms, dtype=dtype,
+                    context="bound switch, V=%d %s" % (vocab, dtype), select_rows=select_rows)
