@@ -82,6 +82,8 @@ struct ncnn_moe_hip_sampler
     VerifyOutput* verify_output = nullptr;      // device
     VerifyInput* verify_input_host = nullptr;   // pinned
     VerifyOutput* verify_output_host = nullptr; // pinned
+    VerifyInput* verify_input_mapped = nullptr;   // the pinned blocks as the device addresses them: the kernels
+    VerifyOutput* verify_output_mapped = nullptr; // read the operands and write the outcome in place
 
     ncnn_moe_sample_params* single_params = nullptr;
     float* single_uniform = nullptr;
@@ -397,6 +399,8 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->verify_output, sizeof(ncnn_moe_hip_sampler::VerifyOutput)));
     CREATE_CHECK(hipHostMalloc(&s->verify_input_host, sizeof(ncnn_moe_hip_sampler::VerifyInput), hipHostMallocDefault));
     CREATE_CHECK(hipHostMalloc(&s->verify_output_host, sizeof(ncnn_moe_hip_sampler::VerifyOutput), hipHostMallocDefault));
+    CREATE_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&s->verify_input_mapped), s->verify_input_host, 0));
+    CREATE_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&s->verify_output_mapped), s->verify_output_host, 0));
     CREATE_CHECK(hipMalloc(&s->single_params, sizeof(ncnn_moe_sample_params)));
     CREATE_CHECK(hipMalloc(&s->single_uniform, sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->single_result, sizeof(ncnn_moe_sample_result)));
@@ -686,21 +690,13 @@ int ncnn_moe_hip_sampler_speculative_verify(
     in.row_uniforms[draft_count] = uniforms[draft_count]; // the draw of the row after the last drafted token
     std::memcpy(in.proposed, proposed_token_ids, draft_count * sizeof(int32_t));
     std::memcpy(in.uniforms, uniforms, (draft_count + 1) * sizeof(float));
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_input, s->verify_input_host, sizeof(in), hipMemcpyHostToDevice, s->stream));
-
+    // The small operands are read by the kernels from the pinned block itself and the outcome is written
+    // into the other one: no copy is enqueued on either side of the two launches.
     DistributionExport export_to;
     export_to.ids = s->verify_ids;
     export_to.probabilities = s->verify_probabilities;
     export_to.count = s->verify_counts;
     export_to.cap = kVerifyCap;
-    SamplerPasses passes;
-    passes.wide_select = row_left_pending(row_options, s->logits_vocab, kFastTopK);
-    passes.full_order = true; // also serves rows whose ties overflow the select lists
-    const int rc = launch_sampler(
-        s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
-        s->verify_input->params, s->verify_input->row_uniforms, nullptr, s->results, export_to, passes, s->stream);
-    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
-        return rc;
     VerifyArgs v;
     v.draft_count = draft_count;
     v.temperature = row_options.temperature;
@@ -708,14 +704,33 @@ int ncnn_moe_hip_sampler_speculative_verify(
     v.distribution_ids = s->verify_ids;
     v.distribution_probabilities = s->verify_probabilities;
     v.distribution_count = s->verify_counts;
-    v.proposed = s->verify_input->proposed;
-    v.uniforms = s->verify_input->uniforms;
-    v.accepted_probabilities = s->verify_output->accepted;
-    v.result = &s->verify_output->result;
-    hipLaunchKernelGGL(speculative_verify_kernel, dim3(1), dim3(kVerifyThreads), 0, s->stream, v);
-    SAMPLER_HIP_CHECK(s, hipGetLastError());
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->verify_output_host, s->verify_output, sizeof(ncnn_moe_hip_sampler::VerifyOutput), hipMemcpyDeviceToHost, s->stream));
-    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    v.proposed = s->verify_input_mapped->proposed;
+    v.uniforms = s->verify_input_mapped->uniforms;
+    v.accepted_probabilities = s->verify_output_mapped->accepted;
+    v.result = &s->verify_output_mapped->result;
+    // the host sees the options: the later passes are enqueued only if the rows can need them; a row whose
+    // ties overflow the select lists reports that, and the step is run again with the full-order kernels
+    SamplerPasses passes;
+    passes.wide_select = row_left_pending(row_options, s->logits_vocab, kFastTopK);
+    passes.full_order = s->force_general != 0 || row_left_pending(row_options, s->logits_vocab, kSelectTopK);
+    for (int attempt = 0; attempt < 2; ++attempt)
+    {
+        const int rc = launch_sampler(
+            s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
+            s->verify_input_mapped->params, s->verify_input_mapped->row_uniforms, nullptr, s->results, export_to, passes, s->stream);
+        if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+            return rc;
+        hipLaunchKernelGGL(speculative_verify_kernel, dim3(1), dim3(kVerifyThreads), 0, s->stream, v);
+        SAMPLER_HIP_CHECK(s, hipGetLastError());
+        SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+        const ncnn_moe_verify_result& outcome = s->verify_output_host->result;
+        const bool row_pending = outcome.status == NCNN_MOE_VERIFY_ROW_ERROR && outcome.row_status == NCNN_MOE_ROW_NEEDS_FULL_ORDER;
+        if (!row_pending || passes.full_order)
+            break;
+        passes = SamplerPasses{};
+        passes.select = false;
+        passes.full_order = true;
+    }
     *result = s->verify_output_host->result;
     std::memcpy(accepted_probabilities, s->verify_output_host->accepted, draft_count * sizeof(float));
     return NCNN_MOE_SAMPLER_SUCCESS;
