@@ -37,10 +37,10 @@ struct ncnn_moe_hip_sampler
     ncnn_moe_sample_result* results = nullptr;
     int32_t* stop_ids = nullptr;
     uint32_t stop_capacity = 0;
-    // the host entry's small operands travel as one block: params | uniforms | stop ids, staged in
-    // pinned memory and copied once; its results are written by the kernels straight into pinned memory
-    uint8_t* input_block = nullptr;      // device
+    // the host entry's small operands are staged as one block of pinned memory, params | uniforms | stop ids,
+    // that the kernels read in place; its results are written by the kernels straight into pinned memory
     uint8_t* input_block_host = nullptr; // pinned
+    uint8_t* input_block_mapped = nullptr; // the pinned block as the device addresses it
     size_t input_uniforms_offset = 0;
     size_t input_stops_offset = 0;
     uint32_t input_stop_capacity = 0;
@@ -78,8 +78,6 @@ struct ncnn_moe_hip_sampler
         ncnn_moe_verify_result result;
         float accepted[NCNN_MOE_MAX_DRAFT_TOKENS];
     };
-    VerifyInput* verify_input = nullptr;        // device
-    VerifyOutput* verify_output = nullptr;      // device
     VerifyInput* verify_input_host = nullptr;   // pinned
     VerifyOutput* verify_output_host = nullptr; // pinned
     VerifyInput* verify_input_mapped = nullptr;   // the pinned blocks as the device addresses them: the kernels
@@ -370,8 +368,8 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     s->input_stops_offset = s->input_uniforms_offset + rows * sizeof(float);
     s->input_stop_capacity = static_cast<uint32_t>(rows * 16);
     const size_t input_bytes = s->input_stops_offset + static_cast<size_t>(s->input_stop_capacity) * sizeof(int32_t);
-    CREATE_CHECK(hipMalloc(&s->input_block, input_bytes));
     CREATE_CHECK(hipHostMalloc(&s->input_block_host, input_bytes, hipHostMallocDefault));
+    CREATE_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&s->input_block_mapped), s->input_block_host, 0));
     CREATE_CHECK(hipHostMalloc(&s->results_host, rows * sizeof(ncnn_moe_sample_result), hipHostMallocDefault));
     CREATE_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&s->results_host_device), s->results_host, 0));
     CREATE_CHECK(hipMalloc(&s->segment_values, slots * kSegmentRecordSlots * sizeof(float)));
@@ -395,8 +393,6 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->verify_ids, kVerifyRows * kVerifyCap * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->verify_probabilities, kVerifyRows * kVerifyCap * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->verify_counts, kVerifyRows * sizeof(uint32_t)));
-    CREATE_CHECK(hipMalloc(&s->verify_input, sizeof(ncnn_moe_hip_sampler::VerifyInput)));
-    CREATE_CHECK(hipMalloc(&s->verify_output, sizeof(ncnn_moe_hip_sampler::VerifyOutput)));
     CREATE_CHECK(hipHostMalloc(&s->verify_input_host, sizeof(ncnn_moe_hip_sampler::VerifyInput), hipHostMallocDefault));
     CREATE_CHECK(hipHostMalloc(&s->verify_output_host, sizeof(ncnn_moe_hip_sampler::VerifyOutput), hipHostMallocDefault));
     CREATE_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&s->verify_input_mapped), s->verify_input_host, 0));
@@ -425,7 +421,7 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->sort_keys[0], s->sort_keys[1],
         s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
-        s->verify_probabilities, s->verify_counts, s->verify_input, s->verify_output, s->input_block};
+        s->verify_probabilities, s->verify_counts};
     for (void* buffer : buffers)
     {
         if (buffer != nullptr)
@@ -511,19 +507,18 @@ int ncnn_moe_hip_sampler_sample(
         return NCNN_MOE_SAMPLER_SUCCESS;
     }
     SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
-    // one copy brings params, uniforms and stop ids; stop-id lists beyond the block's room take the
-    // handle's growable buffer
-    const ncnn_moe_sample_params* device_params = reinterpret_cast<const ncnn_moe_sample_params*>(s->input_block);
-    const float* device_uniforms = reinterpret_cast<const float*>(s->input_block + s->input_uniforms_offset);
+    // params, uniforms and stop ids are staged in one pinned block that the kernels read in place (a few
+    // dozen bytes per workgroup over the host link, behind the first logits loads); stop-id lists beyond
+    // the block's room take the handle's growable device buffer
+    const ncnn_moe_sample_params* device_params = reinterpret_cast<const ncnn_moe_sample_params*>(s->input_block_mapped);
+    const float* device_uniforms = reinterpret_cast<const float*>(s->input_block_mapped + s->input_uniforms_offset);
     const int32_t* device_stops = nullptr;
     std::memcpy(s->input_block_host, params, rows * sizeof(ncnn_moe_sample_params));
     std::memcpy(s->input_block_host + s->input_uniforms_offset, uniforms, rows * sizeof(float));
-    size_t input_bytes = s->input_uniforms_offset + rows * sizeof(float);
     if (stop_id_count > 0 && stop_id_count <= s->input_stop_capacity)
     {
         std::memcpy(s->input_block_host + s->input_stops_offset, stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t));
-        input_bytes = s->input_stops_offset + static_cast<size_t>(stop_id_count) * sizeof(int32_t);
-        device_stops = reinterpret_cast<const int32_t*>(s->input_block + s->input_stops_offset);
+        device_stops = reinterpret_cast<const int32_t*>(s->input_block_mapped + s->input_stops_offset);
     }
     else if (stop_id_count > 0)
     {
@@ -539,7 +534,6 @@ int ncnn_moe_hip_sampler_sample(
         SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->stop_ids, stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t), hipMemcpyHostToDevice, s->stream));
         device_stops = s->stop_ids;
     }
-    SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->input_block, s->input_block_host, input_bytes, hipMemcpyHostToDevice, s->stream));
     // the host sees the options: the later passes are enqueued only if some row needs them
     SamplerPasses passes;
     passes.full_order = s->force_general != 0;
