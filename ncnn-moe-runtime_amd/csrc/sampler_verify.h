@@ -35,6 +35,11 @@ struct VerifyShared
     float ordered_residual[kVerifyCap]; // the residual in token-id order
     int32_t ordered_token[kVerifyCap];
     float found[2];                     // candidate_probability of the proposed token: target, draft
+    // the step's small operands, fetched once (proposed tokens and uniforms may lie in host memory)
+    ncnn_moe_sample_result row_results[2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1];
+    uint32_t counts[2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1];
+    int32_t proposed[NCNN_MOE_MAX_DRAFT_TOKENS];
+    float uniforms[NCNN_MOE_MAX_DRAFT_TOKENS + 1];
 };
 
 __device__ __forceinline__ void write_verify_result(
@@ -62,20 +67,30 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
     const uint32_t drafts = v.draft_count;
     uint32_t accepted = 0;
     uint32_t accept_draws = 0;
+    if (static_cast<uint32_t>(tid) < 2u * drafts + 1u)
+    {
+        shared.row_results[tid] = v.row_results[tid];
+        shared.counts[tid] = v.distribution_count[tid];
+    }
+    if (static_cast<uint32_t>(tid) < drafts)
+        shared.proposed[tid] = v.proposed[tid];
+    if (static_cast<uint32_t>(tid) <= drafts)
+        shared.uniforms[tid] = v.uniforms[tid];
+    __syncthreads();
 
     if (v.temperature == 0.0f)
     {
         // ---- greedy (session.cpp:778-796): a drafted token stands while it is the target's own choice
         for (; accepted < drafts; ++accepted)
         {
-            const ncnn_moe_sample_result target = v.row_results[accepted];
+            const ncnn_moe_sample_result target = shared.row_results[accepted];
             if (target.status != NCNN_MOE_ROW_OK)
             {
                 if (tid == 0)
                     write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ROW_ERROR, target.status, 0, 0, 0);
                 return;
             }
-            if (target.token_id != v.proposed[accepted])
+            if (target.token_id != shared.proposed[accepted])
                 break;
             if (tid == 0)
                 v.accepted_probabilities[accepted] = 1.0f;
@@ -88,8 +103,8 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
         {
             const uint32_t target_row = accepted;
             const uint32_t draft_row = drafts + 1u + accepted;
-            const ncnn_moe_sample_result target = v.row_results[target_row];
-            const ncnn_moe_sample_result draft = v.row_results[draft_row];
+            const ncnn_moe_sample_result target = shared.row_results[target_row];
+            const ncnn_moe_sample_result draft = shared.row_results[draft_row];
             if (target.status != NCNN_MOE_ROW_OK || draft.status != NCNN_MOE_ROW_OK)
             {
                 const uint32_t row_status = target.status != NCNN_MOE_ROW_OK ? target.status : draft.status;
@@ -97,8 +112,8 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
                     write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ROW_ERROR, row_status, accept_draws, 0, 0);
                 return;
             }
-            const uint32_t target_count = __builtin_amdgcn_readfirstlane(v.distribution_count[target_row]);
-            const uint32_t draft_count = __builtin_amdgcn_readfirstlane(v.distribution_count[draft_row]);
+            const uint32_t target_count = __builtin_amdgcn_readfirstlane(shared.counts[target_row]);
+            const uint32_t draft_count = __builtin_amdgcn_readfirstlane(shared.counts[draft_row]);
             if (target_count > static_cast<uint32_t>(kVerifyCap) || draft_count > static_cast<uint32_t>(kVerifyCap))
             {
                 // a filtered distribution longer than the step holds: reported, never approximated
@@ -106,7 +121,7 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
                     write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW, 0, accept_draws, 0, 0);
                 return;
             }
-            const int32_t token = v.proposed[accepted];
+            const int32_t token = shared.proposed[accepted];
             // ---- candidate_probability (session.cpp:138-148) of the proposed token in both lists; the
             // lists go to LDS on the way, for the residual that a rejection needs
             if (tid < 2)
@@ -141,7 +156,7 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
             }
             const float ratio = target_probability / draft_probability;
             const float acceptance = ratio < 1.0f ? ratio : 1.0f; // std::min(1.0f, ratio)
-            const float uniform = v.uniforms[accept_draws];
+            const float uniform = shared.uniforms[accept_draws];
             ++accept_draws;
             if (uniform >= acceptance)
             {
@@ -200,7 +215,7 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
                     return;
                 }
                 // uniform_real_distribution<float>(0, normalizer): canonical draw times the range
-                const float sample_value = v.uniforms[accept_draws] * normalizer;
+                const float sample_value = shared.uniforms[accept_draws] * normalizer;
                 float cumulative = 0.0f;
                 int selected = -1;
                 int last_positive = -1;
@@ -252,7 +267,7 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
 
     // ---- session.cpp:871-873: the target's own sample at the first position that was not accepted
     // (greedy mismatch) or after the last drafted token (everything accepted)
-    const ncnn_moe_sample_result next = v.row_results[accepted];
+    const ncnn_moe_sample_result next = shared.row_results[accepted];
     if (tid == 0)
     {
         if (next.status != NCNN_MOE_ROW_OK)
