@@ -331,6 +331,9 @@ def main():
     parser.add_argument("--warmup", type=int, default=200)
     parser.add_argument("--workload", default="cfg2_topk_topp")
     parser.add_argument("--rows", type=int, default=0, help="batch rows (0: the configuration's own)")
+    parser.add_argument("--batches-in-flight", action="store_true",
+                        help="also time 2 and 4 independent batches in flight (detail only; their launches overlap, "
+                             "so leave it off under a kernel trace)")
     parser.add_argument("--router-score", default="sqrt_softplus", choices=["softmax", "sigmoid", "sqrt_softplus"],
                         help="score function of --workload router_dispatch")
     parser.add_argument("--drafts", type=int, default=5, help="drafted tokens per step of --workload speculative_verify")
@@ -452,7 +455,7 @@ def main():
     # Several independent batches in flight (one handle and one stream each, steps dealt round robin): what
     # a server that keeps several micro-batches going sees.  A decode loop of ONE batch cannot do this (step
     # n + 1 needs step n's tokens), so these are reported beside the value, never as it.
-    if rows <= 256:
+    if args.batches_in_flight and rows <= 256:
         lanes = [(sampler, stream, results)]
         in_flight = {}
         for lane_count in (2, 4):

@@ -29,7 +29,7 @@ constexpr int kWideListCap = 4096;       // candidate list for Top-K windows up 
 constexpr int kSegmentRecordSlots = 256; // candidate slots of a segment's record in HBM
 constexpr int kMaxSegments = 16;
 constexpr int kWholeRowBatch = 256;          // from this many rows on, one workgroup streams a whole row
-constexpr int kSingleChunkWorkgroups = 1024;  // workgroups a smaller batch is split into when each streams one chunk (4 per CU)
+constexpr int kSingleChunkWorkgroups = 4096;  // a smaller batch is split into one-chunk workgroups up to this many (several rounds of 4 per CU beat fewer, looped ones)
 constexpr int kLoopedWorkgroups = 512;        // ... and when each streams several chunks (2 per CU)
          // segments per row the row merge can stage in one trip
 constexpr int kMergeStageSlots = 4096;   // record slots of a row loaded in one trip (8 per thread)
