@@ -201,11 +201,54 @@ __device__ __forceinline__ void finish_from_list(
             finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags);
             return;
         }
+        if (n_list <= 2 * kWaveSize)
+        {
+            // two candidates per lane of wave 0: thread t counts, for candidate t % 128, the candidates of
+            // its quarter of the list that go before it; wave 0 adds the four counts of its two up
+            const int c = tid & (2 * kWaveSize - 1);
+            const int part = tid >> 7;
+            const uint32_t key = c < n_list ? shared.list_keys[c] : 0u;
+            const int32_t candidate_index = c < n_list ? shared.list_indices[c] : 0;
+            constexpr int kShare = 2 * kWaveSize / (kScanThreads / (2 * kWaveSize));
+            int partial = 0;
+#pragma unroll 8
+            for (int k = 0; k < kShare; ++k)
+            {
+                const int j = part * kShare + k;
+                const uint32_t other_key = shared.list_keys[j];
+                const int32_t other_index = shared.list_indices[j];
+                partial += (j < n_list && (other_key > key || (other_key == key && other_index < candidate_index))) ? 1 : 0;
+            }
+            uint32_t* const partial_counts = shared.bound.hot_keys; // 4 x 128 counts
+            partial_counts[part * 2 * kWaveSize + c] = static_cast<uint32_t>(partial);
+            __syncthreads();
+            if (wave != 0)
+                return;
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+            {
+                const int mine = half * kWaveSize + lane;
+                int before = 0;
+#pragma unroll
+                for (int q = 0; q < kScanThreads / (2 * kWaveSize); ++q)
+                    before += static_cast<int>(partial_counts[q * 2 * kWaveSize + mine]);
+                if (mine < n_list && before < top_k)
+                {
+                    shared.final_values[before] = value_from_ascending_key(shared.list_keys[mine]);
+                    shared.final_indices[before] = shared.list_indices[mine];
+                }
+            }
+            n = n_list < top_k ? n_list : top_k;
+            if (lane == 0)
+                a.row_state[row] = kRowDone;
+            const float value = lane < n ? shared.final_values[lane] : 0.0f;
+            const int32_t index = lane < n ? shared.final_indices[lane] : -1;
+            finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags);
+            return;
+        }
         if (wave != 0)
             return;
-        if (n_list <= 2 * kWaveSize)
-            n = select_best_wave<2>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
-        else if (n_list <= 4 * kWaveSize)
+        if (n_list <= 4 * kWaveSize)
             n = select_best_wave<4>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
         else
             n = select_best_wave<8>(shared.list_keys, shared.list_indices, n_list, top_k, lane, shared.final_values, shared.final_indices);
@@ -477,8 +520,9 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         if (lane_max == __uint_as_float(kPositiveInfinity))
             local_flags |= kScanSawPositiveInfinity;
 
-        // ---- bound of the first chunk: the exact K-th largest lane maximum.  The lanes at or above it
-        // each hold a distinct logit at least that large, so the K-th best logit of the row is no smaller.
+        // ---- bound of the first chunk: the K-th largest lane maximum, or a cheaper bound below it.  The
+        // lanes at or above it each hold a distinct logit at least that large, so the K-th best logit of
+        // the row is no smaller.
         if (first_of_segment)
         {
             if (WIDE && top_k > kTwoKeyBoundTopK)
@@ -501,8 +545,8 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
             else
             {
                 const uint32_t lane_keys[1] = {lane_max == __uint_as_float(kNegativeInfinity) ? 0u : ascending_key(lane_max)};
-                uint32_t chunk_bound = top_k <= kRowMaximaTopK ? workgroup_kth_of_row_maxima(lane_keys[0], top_k, tid, shared.bound) : 0u;
-                if (chunk_bound == 0u) // a wider window, or a chunk with few values: the exact K-th largest lane maximum
+                uint32_t chunk_bound = workgroup_kth_of_quad_maxima(lane_keys[0], top_k, tid, shared.bound);
+                if (chunk_bound == 0u) // a chunk with few values: the exact K-th largest lane maximum
                     chunk_bound = workgroup_kth_largest_key(lane_keys, top_k, tid, shared.bound, true);
                 bound_key = max(bound_key, chunk_bound);
             }
@@ -683,7 +727,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     // ---- last workgroup of the row: every load of the merge is issued before any is used (one trip)
     // Thread slot q stands for entry q / 16 of segment q % 16: no division by the record length, and
     // every row of 16 lanes sees one entry of each segment, so the candidates are spread evenly over
-    // the lanes (which is what the prune's bound from row maxima needs).
+    // the lanes (which is what the prune's bound from the quad maxima needs).
     static_assert(kMaxSegments == 16, "the merge maps a thread slot to (entry, segment) with a shift by 4");
     const size_t row_slot = static_cast<size_t>(row) * a.segments;
     const uint32_t row_entries = record_entries * static_cast<uint32_t>(kMaxSegments);
@@ -745,7 +789,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         return;
     }
     // prune: at least K candidates reach this lower bound of the K-th largest per-thread best
-    uint32_t prune_key = top_k <= kRowMaximaTopK ? workgroup_kth_of_row_maxima(thread_key[0], top_k, tid, shared.bound) : 0u;
+    uint32_t prune_key = workgroup_kth_of_quad_maxima(thread_key[0], top_k, tid, shared.bound);
     if (prune_key == 0u)
         prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, shared.bound, true);
 #pragma unroll
