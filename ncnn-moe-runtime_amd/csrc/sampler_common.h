@@ -516,12 +516,12 @@ __device__ __forceinline__ uint32_t select_kth_key_dispatch(const uint32_t* keys
     return select_kth_key<16>(keys_in_lds, m, top_k, lane);
 }
 
-constexpr int kGroupMaxima = kScanThreads / 4; // one per quad of lanes (the smallest group the cheap bound uses)
-static_assert(kGroupMaxima == 2 * kWaveSize, "a wave searches the quad maxima two per lane");
+constexpr int kQuadMaxima = kScanThreads / 4; // one per quad of lanes
+static_assert(kQuadMaxima == 2 * kWaveSize, "a wave searches the quad maxima two per lane");
 
 struct BoundScratch
 {
-    uint32_t group_maxima[kGroupMaxima];
+    uint32_t quad_maxima[kQuadMaxima];
     uint32_t wave_bounds[kScanWaves];
     uint32_t hot_keys[2 * kScanThreads];
     uint32_t hot_total;
@@ -529,60 +529,49 @@ struct BoundScratch
 };
 
 // A cheap lower bound of the top_k-th largest of the workgroup's keys (one per thread, each standing
-// for a distinct logit; 0 = no key) that at least top_k keys reach: the top_k-th largest of the
-// maxima of the groups of GROUP neighbouring lanes (32 rows of 16, or 128 quads), every maximum being
-// one of the keys.  0 when top_k exceeds three quarters of the groups that hold a key (a short row
-// fills few of them; beyond that the smallest maxima decide): the caller then takes the exact
-// routine below.  Looser than the exact top_k-th largest (of 10,240 values, top_k = 20: about 30 reach
-// the bound of the rows and 22 that of the quads; top_k = 50, quads: about 63), at a third of the
-// cost: four or two exchanges inside the groups, one LDS round trip, a 16-step search whose steps
-// count one ballot (rows) or two (quads; a quarter of a microsecond more per call).  All threads of
-// the workgroup must call it.
-constexpr int kRowMaximaTopK = 24; // windows up to here take the bound from the 32 row maxima, wider ones from the quads
-constexpr int kMergeQuadsTopK = 4; // the merge of a window this small: few rows of lanes hold a record entry, so quads again
-
-template <int GROUP>
-__device__ __forceinline__ uint32_t workgroup_kth_of_group_maxima(uint32_t key, int top_k, int tid, BoundScratch& scratch)
+// for a distinct logit; 0 = no key) that at least top_k keys reach: the top_k-th largest of the 128
+// maxima of the quads of lanes, every maximum being one of the keys.  0 when top_k exceeds three
+// quarters of the quads that hold a key (a short row fills few of them; beyond that the smallest
+// maxima decide): the caller then takes the exact routine below.  Slightly looser than the exact
+// top_k-th largest (for top_k = 20 of 10,240 values about 22 reach it, for top_k = 50 about 63), at a
+// third of the cost: two exchanges inside the quads, an LDS round trip, a 16-step search by one wave,
+// a second LDS round trip.  All threads of the workgroup must call it.
+__device__ __forceinline__ uint32_t workgroup_kth_of_quad_maxima(uint32_t key, int top_k, int tid, BoundScratch& scratch)
 {
-    static_assert(GROUP == 4 || GROUP == 16, "quads or rows of lanes");
-    constexpr int kGroupsPerWave = kWaveSize / GROUP;
-    constexpr int kGroups = kScanThreads / GROUP;
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
-    uint32_t group_max = key;
-    group_max = max(group_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(group_max), 0xB1, 0xf, 0xf, true))); // lanes 1 apart
-    group_max = max(group_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(group_max), 0x4E, 0xf, 0xf, true))); // lanes 2 apart
-    if constexpr (GROUP == 16)
-    {
-        group_max = max(group_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(group_max), 0x141, 0xf, 0xf, true))); // half-row mirror
-        group_max = max(group_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(group_max), 0x140, 0xf, 0xf, true))); // row mirror
-    }
-    if ((lane & (GROUP - 1)) == 0)
-        scratch.group_maxima[wave * kGroupsPerWave + lane / GROUP] = group_max;
+    uint32_t quad_max = key;
+    quad_max = max(quad_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(quad_max), 0xB1, 0xf, 0xf, true))); // lanes 1 apart
+    quad_max = max(quad_max, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(quad_max), 0x4E, 0xf, 0xf, true))); // lanes 2 apart
+    if ((lane & 3) == 0)
+        scratch.quad_maxima[wave * (kWaveSize / 4) + (lane >> 2)] = quad_max;
     lds_barrier();
-    // every wave searches the maxima itself (up to two per lane), bit by bit: the counting is scalar
-    // and there is no second barrier.  The lowest 16 bits are left at zero: a step costs a
-    // VALU-to-scalar round trip, and a bound that is half a percent lower lets hardly any more keys through.
-    const uint32_t first = lane < kGroups ? scratch.group_maxima[lane] : 0u;
-    const uint32_t second = kGroups > kWaveSize ? scratch.group_maxima[(kWaveSize + lane) & (kGroupMaxima - 1)] : 0u;
-    const auto reaching = [&](uint32_t trial) {
-        int count = __popcll(__ballot(first >= trial));
-        if constexpr (kGroups > kWaveSize)
-            count += __popcll(__ballot(second >= trial));
-        return count;
-    };
-    const int groups_with_keys = reaching(1u);
-    if (top_k * 4 > groups_with_keys * 3)
-        return 0u;
-    uint32_t prefix = 0;
-#pragma unroll
-    for (int bit = 31; bit >= 16; --bit)
+    // One wave searches the 128 maxima (two per lane) bit by bit, counting with ballots, while the others
+    // wait: the steps are scalar, and eight waves searching side by side (which would save the second
+    // barrier) queue for the one scalar unit of their SIMDs and take 0.2 to 0.7 us longer per batch.
+    // The lowest 16 bits are left at zero: a step costs a VALU-to-scalar round trip, and a bound that
+    // is half a percent lower lets hardly any more keys through.
+    if (wave == 0)
     {
-        const uint32_t trial = prefix | (1u << bit);
-        if (reaching(trial) >= top_k)
-            prefix = trial;
+        const uint32_t first = scratch.quad_maxima[lane];
+        const uint32_t second = scratch.quad_maxima[kWaveSize + lane];
+        const auto reaching = [&](uint32_t trial) { return __popcll(__ballot(first >= trial)) + __popcll(__ballot(second >= trial)); };
+        uint32_t prefix = 0;
+        if (top_k * 4 <= reaching(1u) * 3)
+        {
+#pragma unroll
+            for (int bit = 31; bit >= 16; --bit)
+            {
+                const uint32_t trial = prefix | (1u << bit);
+                if (reaching(trial) >= top_k)
+                    prefix = trial;
+            }
+        }
+        if (lane == 0)
+            scratch.result = prefix;
     }
-    return prefix;
+    lds_barrier();
+    return scratch.result;
 }
 
 // The top_k-th largest of the workgroup's keys (KEYS per thread, each standing for a distinct

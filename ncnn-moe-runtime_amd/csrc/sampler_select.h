@@ -545,10 +545,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
             else
             {
                 const uint32_t lane_keys[1] = {lane_max == __uint_as_float(kNegativeInfinity) ? 0u : ascending_key(lane_max)};
-                // a looped workgroup computes one bound for many chunks: the tighter one, whatever the window
-                uint32_t chunk_bound = (!LOOPED && top_k <= kRowMaximaTopK)
-                                           ? workgroup_kth_of_group_maxima<16>(lane_keys[0], top_k, tid, shared.bound)
-                                           : workgroup_kth_of_group_maxima<4>(lane_keys[0], top_k, tid, shared.bound);
+                uint32_t chunk_bound = workgroup_kth_of_quad_maxima(lane_keys[0], top_k, tid, shared.bound);
                 if (chunk_bound == 0u) // a chunk with few values: the exact K-th largest lane maximum
                     chunk_bound = workgroup_kth_largest_key(lane_keys, top_k, tid, shared.bound, true);
                 bound_key = max(bound_key, chunk_bound);
@@ -792,11 +789,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         return;
     }
     // prune: at least K candidates reach this lower bound of the K-th largest per-thread best
-    // Entry r of segment s sits in thread 16 r + s: a row of 16 lanes holds one entry of every segment,
-    // so the records of a very small window fill too few rows for the rows' bound and take the quads'.
-    uint32_t prune_key = (top_k > kMergeQuadsTopK && top_k <= kRowMaximaTopK)
-                             ? workgroup_kth_of_group_maxima<16>(thread_key[0], top_k, tid, shared.bound)
-                             : workgroup_kth_of_group_maxima<4>(thread_key[0], top_k, tid, shared.bound);
+    uint32_t prune_key = workgroup_kth_of_quad_maxima(thread_key[0], top_k, tid, shared.bound);
     if (prune_key == 0u)
         prune_key = workgroup_kth_largest_key(thread_key, top_k, tid, shared.bound, true);
 #pragma unroll
