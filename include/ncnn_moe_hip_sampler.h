@@ -157,8 +157,9 @@ enum ncnn_moe_verify_status
     NCNN_MOE_VERIFY_ZERO_DRAFT_PROBABILITY = 2, /* "sampled draft token has zero probability" (:822-830) */
     NCNN_MOE_VERIFY_RESIDUAL_EMPTY = 3,         /* "speculative residual distribution is empty" (:170-175) */
     NCNN_MOE_VERIFY_RESIDUAL_FAILED = 4,        /* "speculative residual sampling failed" (:199-201) */
-    /* Not a CPU-sampler error: a filtered distribution (after Top-K, Min-P, Top-P) that the accept loop
-     * reached holds more than 1024 candidates, which is what this entry keeps per row. */
+    /* Not a CPU-sampler error, and not returned by ncnn_moe_hip_sampler_speculative_verify: its first
+     * kernel reports a filtered distribution (after Top-K, Min-P, Top-P) of more than 1024 candidates
+     * with it, and the entry then runs the step again through the kernel that holds whole rows. */
     NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW = 5
 };
 

@@ -65,6 +65,14 @@ struct ncnn_moe_hip_sampler
     int32_t* verify_ids = nullptr;
     float* verify_probabilities = nullptr;
     uint32_t* verify_counts = nullptr;
+    // speculative verification of filtered distributions longer than kVerifyCap: allocated by the first
+    // step that meets one (rows x max_vocab lists, two dense vectors over the vocabulary)
+    int32_t* verify_long_ids = nullptr;
+    float* verify_long_probabilities = nullptr;
+    float* verify_dense = nullptr;
+    // the options of the last step that needed them: the next step with the same options goes there at once
+    bool verify_dense_known = false;
+    ncnn_moe_sample_params verify_dense_options{};
     // operands and outcome of a step travel as one block each, through pinned host memory
     struct VerifyInput
     {
@@ -421,7 +429,7 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->sort_keys[0], s->sort_keys[1],
         s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
-        s->verify_probabilities, s->verify_counts};
+        s->verify_probabilities, s->verify_counts, s->verify_long_ids, s->verify_long_probabilities, s->verify_dense};
     for (void* buffer : buffers)
     {
         if (buffer != nullptr)
@@ -707,7 +715,8 @@ int ncnn_moe_hip_sampler_speculative_verify(
     SamplerPasses passes;
     passes.wide_select = row_left_pending(row_options, s->logits_vocab, kFastTopK);
     passes.full_order = s->force_general != 0 || row_left_pending(row_options, s->logits_vocab, kSelectTopK);
-    for (int attempt = 0; attempt < 2; ++attempt)
+    bool dense = s->verify_dense_known && std::memcmp(&s->verify_dense_options, &row_options, sizeof(row_options)) == 0;
+    for (int attempt = 0; attempt < 2 && !dense; ++attempt)
     {
         const int rc = launch_sampler(
             s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
@@ -725,6 +734,46 @@ int ncnn_moe_hip_sampler_speculative_verify(
         passes.select = false;
         passes.full_order = true;
     }
+    if (!dense && s->verify_output_host->result.status == NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW)
+    {
+        dense = true;
+        s->verify_dense_known = true;
+        s->verify_dense_options = row_options;
+    }
+    if (dense)
+    {
+        // A filtered distribution longer than the lists above: the step is run (again) with lists that
+        // hold a whole row each and the kernel that builds the residual as a dense vector.
+        if (s->verify_long_ids == nullptr)
+        {
+            const size_t entries = static_cast<size_t>(2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1) * s->max_vocab;
+            SAMPLER_HIP_CHECK(s, hipMalloc(&s->verify_long_ids, entries * sizeof(int32_t)));
+            SAMPLER_HIP_CHECK(s, hipMalloc(&s->verify_long_probabilities, entries * sizeof(float)));
+            SAMPLER_HIP_CHECK(s, hipMalloc(&s->verify_dense, 2 * static_cast<size_t>(s->max_vocab) * sizeof(float)));
+        }
+        export_to.ids = s->verify_long_ids;
+        export_to.probabilities = s->verify_long_probabilities;
+        export_to.cap = s->logits_vocab;
+        VerifyDenseArgs d;
+        d.step = v;
+        d.step.distribution_ids = s->verify_long_ids;
+        d.step.distribution_probabilities = s->verify_long_probabilities;
+        d.list_cap = s->logits_vocab;
+        d.vocab = s->logits_vocab;
+        d.dense_draft = s->verify_dense;
+        d.dense_residual = s->verify_dense + s->max_vocab;
+        SamplerPasses every_pass;
+        every_pass.wide_select = row_left_pending(row_options, s->logits_vocab, kFastTopK);
+        every_pass.full_order = true;
+        const int rc = launch_sampler(
+            s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
+            s->verify_input_mapped->params, s->verify_input_mapped->row_uniforms, nullptr, s->results, export_to, every_pass, s->stream);
+        if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+            return rc;
+        hipLaunchKernelGGL(speculative_verify_dense_kernel, dim3(1), dim3(kReplayThreads), 0, s->stream, d);
+        SAMPLER_HIP_CHECK(s, hipGetLastError());
+        SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    }
     *result = s->verify_output_host->result;
     std::memcpy(accepted_probabilities, s->verify_output_host->accepted, draft_count * sizeof(float));
     return NCNN_MOE_SAMPLER_SUCCESS;
@@ -739,7 +788,7 @@ const char* ncnn_moe_hip_sampler_verify_status_message(int verify_status)
     case NCNN_MOE_VERIFY_ZERO_DRAFT_PROBABILITY: return "sampled draft token has zero probability";
     case NCNN_MOE_VERIFY_RESIDUAL_EMPTY: return "speculative residual distribution is empty";
     case NCNN_MOE_VERIFY_RESIDUAL_FAILED: return "speculative residual sampling failed";
-    case NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW: return "speculative verification on the device holds filtered distributions of up to 1024 candidates";
+    case NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW: return "a filtered distribution exceeds the verification lists";
     default: return "unknown verification status";
     }
 }

@@ -224,12 +224,13 @@ __device__ __forceinline__ float row_term(const SortedRow& row, uint32_t i)
     return t;
 }
 
-// The running fp32 sum of terms [0, count) of the row, starting from 0, exactly as a sequential
-// loop produces it.  PHASE 0 also stops (without `stopped`) once the sum no longer moves, which
-// is final because the terms are non-increasing.  Every thread of the workgroup must call it.
-template <int PHASE>
-__device__ __forceinline__ RunningSum exact_running_sum(
-    const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
+// The running fp32 sum of the non-negative terms term_at(0) ... term_at(count - 1), starting from 0,
+// exactly as a sequential loop produces it.  With NON_INCREASING (the terms never grow) it also stops
+// (without `stopped`) once the sum no longer moves, which is then final.  Every thread of the
+// workgroup (kReplayThreads threads) must call it.
+template <bool NON_INCREASING, class TermAt>
+__device__ __forceinline__ RunningSum exact_running_sum_of_terms(
+    TermAt term_at, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
 {
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
@@ -244,7 +245,7 @@ __device__ __forceinline__ RunningSum exact_running_sum(
         for (int slot = 0; slot < kSequentialHead / kWaveSize; ++slot)
         {
             const uint32_t i = static_cast<uint32_t>(slot * kWaveSize + lane);
-            head_terms[slot] = i < head ? row_term<PHASE>(row, i) : 0.0f;
+            head_terms[slot] = i < head ? term_at(i) : 0.0f;
         }
 #pragma unroll
         for (int slot = 0; slot < kSequentialHead / kWaveSize; ++slot)
@@ -270,7 +271,7 @@ __device__ __forceinline__ RunningSum exact_running_sum(
         for (int j = 0; j < kReplayPerThread; ++j)
         {
             const uint32_t i = thread_first + j;
-            terms[j] = i < chunk_end ? row_term<PHASE>(row, i) : 0.0f;
+            terms[j] = i < chunk_end ? term_at(i) : 0.0f;
         }
         uint32_t start = max(base, head);
         while (start < chunk_end)
@@ -297,7 +298,7 @@ __device__ __forceinline__ RunningSum exact_running_sum(
             {
                 scratch.first_event = 0xffffffffu;
                 // the largest remaining term of the row does not move the sum: nothing later can
-                scratch.absorbed = (PHASE == 0 && start == base && base > 0 && first_step.even == 0u && first_step.odd == 0u) ? 1 : 0;
+                scratch.absorbed = (NON_INCREASING && start == base && base > 0 && first_step.even == 0u && first_step.odd == 0u) ? 1 : 0;
             }
             // inclusive scan of the per-thread totals across the wave, then across waves
             ParityStep inclusive = thread_total;
@@ -387,6 +388,16 @@ __device__ __forceinline__ RunningSum exact_running_sum(
         }
     }
     return RunningSum{sum, 0u, false};
+}
+
+// The running sum of terms [0, count) of a sorted row.  PHASE 0 (terms that never grow) also stops
+// once the sum no longer moves.  Every thread of the workgroup must call it.
+template <int PHASE>
+__device__ __forceinline__ RunningSum exact_running_sum(
+    const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
+{
+    return exact_running_sum_of_terms<PHASE == 0>(
+        [&row](uint32_t i) { return row_term<PHASE>(row, i); }, count, mode, bound, scratch, tid);
 }
 
 // The same running sum over a row stored as runs: `count` elements are added, run after run.  A run of

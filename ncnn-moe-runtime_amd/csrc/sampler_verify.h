@@ -5,6 +5,7 @@
 #define NCNN_MOE_HIP_SAMPLER_VERIFY_H
 
 #include "sampler_common.h"
+#include "sampler_exact_sum.h"
 
 namespace ncnn_moe_hip {
 
@@ -267,6 +268,172 @@ __global__ __launch_bounds__(kVerifyThreads) void speculative_verify_kernel(Veri
 
     // ---- session.cpp:871-873: the target's own sample at the first position that was not accepted
     // (greedy mismatch) or after the last drafted token (everything accepted)
+    const ncnn_moe_sample_result next = shared.row_results[accepted];
+    if (tid == 0)
+    {
+        if (next.status != NCNN_MOE_ROW_OK)
+            write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ROW_ERROR, next.status, accept_draws, 0, 0);
+        else
+            write_verify_result(v, accepted, next.token_id, next.probability, NCNN_MOE_VERIFY_OK, 0, accept_draws,
+                                next.draw_consumed, 0);
+    }
+}
+
+// The same step for filtered distributions of any length (a row without a Top-K window whose Top-P
+// keeps more than kVerifyCap tokens): the lists stay in global memory, `list_cap` entries per row, and
+// a rejection builds the residual as the CPU does, as a dense vector over the vocabulary
+// (session.cpp:150-202): the draft's probabilities are scattered into one vector, max(0, target - draft)
+// into another, and the sequential fp32 sum and the walk to the draw over that vector (zeros leave an
+// fp32 sum as it is) come from the exact parallel running sum.  One workgroup of kReplayThreads threads.
+struct VerifyDenseArgs
+{
+    VerifyArgs step;       // distribution_ids / distribution_probabilities hold list_cap entries per row
+    uint32_t list_cap;
+    uint32_t vocab;
+    float* dense_draft;    // [vocab]
+    float* dense_residual; // [vocab]
+};
+
+struct VerifyDenseShared
+{
+    ReplayScratch replay;
+    float found[2];
+    int last_positive;
+    ncnn_moe_sample_result row_results[2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1];
+    uint32_t counts[2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1];
+    int32_t proposed[NCNN_MOE_MAX_DRAFT_TOKENS];
+    float uniforms[NCNN_MOE_MAX_DRAFT_TOKENS + 1];
+};
+
+__global__ __launch_bounds__(kReplayThreads) void speculative_verify_dense_kernel(VerifyDenseArgs d)
+{
+    __shared__ VerifyDenseShared shared;
+    const VerifyArgs& v = d.step;
+    const int tid = threadIdx.x;
+    const uint32_t drafts = v.draft_count;
+    uint32_t accepted = 0;
+    uint32_t accept_draws = 0;
+    if (static_cast<uint32_t>(tid) < 2u * drafts + 1u)
+    {
+        shared.row_results[tid] = v.row_results[tid];
+        shared.counts[tid] = v.distribution_count[tid];
+    }
+    if (static_cast<uint32_t>(tid) < drafts)
+        shared.proposed[tid] = v.proposed[tid];
+    if (static_cast<uint32_t>(tid) <= drafts)
+        shared.uniforms[tid] = v.uniforms[tid];
+    __syncthreads();
+
+    // ---- session.cpp:797-842 (a greedy step never needs the lists and is served by the kernel above)
+    for (; accepted < drafts; ++accepted)
+    {
+        const uint32_t target_row = accepted;
+        const uint32_t draft_row = drafts + 1u + accepted;
+        const ncnn_moe_sample_result target = shared.row_results[target_row];
+        const ncnn_moe_sample_result draft = shared.row_results[draft_row];
+        if (target.status != NCNN_MOE_ROW_OK || draft.status != NCNN_MOE_ROW_OK)
+        {
+            const uint32_t row_status = target.status != NCNN_MOE_ROW_OK ? target.status : draft.status;
+            if (tid == 0)
+                write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ROW_ERROR, row_status, accept_draws, 0, 0);
+            return;
+        }
+        const uint32_t target_count = __builtin_amdgcn_readfirstlane(shared.counts[target_row]);
+        const uint32_t draft_count = __builtin_amdgcn_readfirstlane(shared.counts[draft_row]);
+        if (target_count > d.list_cap || draft_count > d.list_cap)
+        {
+            if (tid == 0)
+                write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_UNSUPPORTED_WINDOW, 0, accept_draws, 0, 0);
+            return;
+        }
+        const int32_t* const target_ids = v.distribution_ids + static_cast<size_t>(target_row) * d.list_cap;
+        const float* const target_probabilities = v.distribution_probabilities + static_cast<size_t>(target_row) * d.list_cap;
+        const int32_t* const draft_ids = v.distribution_ids + static_cast<size_t>(draft_row) * d.list_cap;
+        const float* const draft_probabilities = v.distribution_probabilities + static_cast<size_t>(draft_row) * d.list_cap;
+        const int32_t token = shared.proposed[accepted];
+        // ---- candidate_probability (session.cpp:138-148) of the proposed token in both lists
+        if (tid < 2)
+            shared.found[tid] = 0.0f;
+        __syncthreads();
+        for (uint32_t j = tid; j < target_count; j += kReplayThreads)
+        {
+            if (target_ids[j] == token)
+                shared.found[0] = target_probabilities[j]; // ids are distinct: at most one writer
+        }
+        for (uint32_t j = tid; j < draft_count; j += kReplayThreads)
+        {
+            if (draft_ids[j] == token)
+                shared.found[1] = draft_probabilities[j];
+        }
+        __syncthreads();
+        const float target_probability = shared.found[0];
+        const float draft_probability = shared.found[1];
+        if (draft_probability <= 0.0f)
+        {
+            if (tid == 0)
+                write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_ZERO_DRAFT_PROBABILITY, 0, accept_draws, 0, 0);
+            return;
+        }
+        const float ratio = target_probability / draft_probability;
+        const float acceptance = ratio < 1.0f ? ratio : 1.0f; // std::min(1.0f, ratio)
+        const float uniform = shared.uniforms[accept_draws];
+        ++accept_draws;
+        if (uniform >= acceptance)
+        {
+            // ---- rejected: sample_residual_distribution (session.cpp:150-202), dense over the vocabulary
+            for (uint32_t i = tid; i < d.vocab; i += kReplayThreads)
+            {
+                d.dense_draft[i] = 0.0f;
+                d.dense_residual[i] = 0.0f;
+            }
+            if (tid == 0)
+                shared.last_positive = -1;
+            __syncthreads();
+            for (uint32_t j = tid; j < draft_count; j += kReplayThreads)
+                d.dense_draft[draft_ids[j]] = draft_probabilities[j];
+            __syncthreads();
+            for (uint32_t j = tid; j < target_count; j += kReplayThreads)
+            {
+                const int32_t id = target_ids[j];
+                const float difference = target_probabilities[j] - d.dense_draft[id];
+                const float residual = 0.0f < difference ? difference : 0.0f; // std::max(0.0f, difference)
+                d.dense_residual[id] = residual;
+                if (residual > 0.0f)
+                    atomicMax(&shared.last_positive, id);
+            }
+            __syncthreads();
+            const float* const residual = d.dense_residual;
+            const auto residual_at = [residual](uint32_t i) { return residual[i]; };
+            const RunningSum total = exact_running_sum_of_terms<false>(residual_at, d.vocab, kStopNever, 0.0f, shared.replay, tid);
+            const float normalizer = total.sum;
+            if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
+            {
+                if (tid == 0)
+                    write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_RESIDUAL_EMPTY, 0, accept_draws, 0, 1);
+                return;
+            }
+            // uniform_real_distribution<float>(0, normalizer): canonical draw times the range
+            const float sample_value = shared.uniforms[accept_draws] * normalizer;
+            __syncthreads();
+            const RunningSum walk = exact_running_sum_of_terms<false>(residual_at, d.vocab, kStopAbove, sample_value, shared.replay, tid);
+            // session.cpp:189-198: past the end, the last token that has any residual mass
+            const int selected = walk.stopped ? static_cast<int>(walk.stop_index) : shared.last_positive;
+            if (selected < 0)
+            {
+                if (tid == 0)
+                    write_verify_result(v, accepted, -1, 0.0f, NCNN_MOE_VERIFY_RESIDUAL_FAILED, 0, accept_draws, 1, 1);
+                return;
+            }
+            if (tid == 0)
+                write_verify_result(v, accepted, selected, residual[selected] / normalizer, NCNN_MOE_VERIFY_OK, 0, accept_draws, 1, 1);
+            return;
+        }
+        if (tid == 0)
+            v.accepted_probabilities[accepted] = target_probability;
+        __syncthreads(); // found[] is reset by the next position
+    }
+
+    // ---- session.cpp:871-873: the target's own sample after the last drafted token
     const ncnn_moe_sample_result next = shared.row_results[accepted];
     if (tid == 0)
     {

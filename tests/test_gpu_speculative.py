@@ -147,16 +147,43 @@ def test_residual_edge_cases(sampler):
     _compare(sampler, tied, tied[:2], [3, 9], [0.4, 0.6, 0.2], "all logits tied", temperature=1.0, top_k=16)
 
 
-def test_unsupported_window_and_argument_errors(sampler):
-    """A filtered distribution of more than 1024 candidates is reported, not approximated."""
+def test_long_distributions_and_argument_errors(sampler):
+    """Filtered distributions of more than 1024 candidates take the dense residual; wrong shapes are refused."""
     flat = np.zeros((3, 5000), dtype=np.float32)
+    for options in (dict(temperature=1.0, top_k=0), dict(temperature=1.0, top_k=1025), dict(temperature=1.0, top_p=0.2)):
+        for uniforms in ([0.5, 0.5], [0.999, 0.7]):
+            _compare(sampler, flat[:2], flat[2:], [1], uniforms, "flat rows %s %s" % (options, uniforms), **options)
     sampler.upload_logits(flat)
-    for options in (dict(temperature=1.0, top_k=0), dict(temperature=1.0, top_k=1025)):
-        result, _ = sampler.speculative_verify([1], [0.5, 0.5], **options)
-        assert result["status"] == hip_sampler.VERIFY_UNSUPPORTED_WINDOW and result["next_token_id"] == -1
-    # the same flat rows with a nucleus that keeps 1000 of them are served
-    cpu, _ = oracle_lib.oracle_speculative_verify(flat[:2], flat[2:], [1], [0.5, 0.5], temperature=1.0, top_p=0.2)
-    gpu, _ = sampler.speculative_verify([1], [0.5, 0.5], temperature=1.0, top_p=0.2)
-    assert gpu["status"] == cpu["status"] == 0 and gpu["next_token_id"] == cpu["next_token_id"]
     with pytest.raises(hip_sampler.SamplerError):
         sampler.speculative_verify([1, 2], [0.5, 0.5, 0.5], temperature=1.0, top_k=8)  # 3 rows hold one drafted token
+
+
+@pytest.mark.parametrize("vocab,drafts,bf16,options", [
+    (5000, 2, False, dict(temperature=1.0)),
+    (40000, 3, False, dict(temperature=1.0, top_p=0.95)),
+    (40000, 3, True, dict(temperature=0.9, top_p=0.98, min_p=0.00001)),
+    (33333, 4, False, dict(temperature=1.3, top_k=3000)),
+    (151936, 5, False, dict(temperature=1.0, top_p=0.9)),
+    (151936, 2, False, dict(temperature=1.5)),
+])
+def test_long_distributions_match_the_oracle(sampler, vocab, drafts, bf16, options):
+    """Rows whose filtered distributions hold thousands of tokens: accepted prefixes of every length, the
+    residual draw early and late in the vocabulary, and the draw that follows a fully accepted draft."""
+    rng = np.random.default_rng(4242 + vocab + drafts)
+    for trial in range(4):
+        target = (rng.standard_normal((drafts + 1, vocab)) * 1.5).astype(np.float32)
+        draft = (target[:drafts] + rng.standard_normal((drafts, vocab)).astype(np.float32) * (0.2 + 0.4 * trial)).astype(np.float32)
+        if bf16:
+            target = workloads.bf16_bits_to_float32(workloads.float32_to_bf16_bits(target))
+            draft = workloads.bf16_bits_to_float32(workloads.float32_to_bf16_bits(draft))
+        proposed = _propose(rng, draft, options)
+        uniforms = rng.random(drafts + 1).astype(np.float32)
+        if trial == 1:
+            uniforms[0] = np.float32(0.9999)    # reject the first drafted token
+        if trial == 2:
+            uniforms[:drafts] = np.float32(0.0)  # accept everything
+        if trial == 3:
+            uniforms[drafts - 1] = np.float32(0.9999)
+            uniforms[drafts] = np.float32(0.99999)  # a residual draw near the end of the vocabulary
+        _compare(sampler, target, draft, proposed, uniforms,
+                 "long lists: vocab %d drafts %d trial %d %s" % (vocab, drafts, trial, options), bf16=bf16, **options)
