@@ -9,9 +9,9 @@
 
 namespace ncnn_moe_hip {
 
-constexpr int kRouterWavesPerBlock = 4;
+constexpr int kRouterWavesPerBlock = 8;
 constexpr int kRouterThreads = kRouterWavesPerBlock * kWaveSize;
-constexpr int kRouterChunkTokens = kRouterThreads; // tokens whose routes one workgroup of the grouping kernel places
+constexpr int kRouterChunkTokens = 256; // tokens whose routes one workgroup of the grouping kernel places
 
 // log1pf bit-identical to glibc 2.35's (sysdeps/ieee754/flt-32/s_log1pf.c) for finite x > 0, which is
 // all stable_softplus hands it (an exponential).  Plain fp32 operations in the library's order; built
@@ -303,8 +303,9 @@ __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterS
     if (lane < top_k)
     {
         const float weight = (r.renormalize != 0u ? my_score / selected_sum : my_score) * r.scaling;
-        r.selected_experts[static_cast<size_t>(token) * r.top_k + lane] = my_expert;
-        r.selected_weights[static_cast<size_t>(token) * r.top_k + lane] = weight;
+        // written through the per-XCD L2: the workgroup that groups the routes may sit on another XCD
+        store_agent(&r.selected_experts[static_cast<size_t>(token) * r.top_k + lane], my_expert);
+        store_agent(reinterpret_cast<uint32_t*>(&r.selected_weights[static_cast<size_t>(token) * r.top_k + lane]), __float_as_uint(weight));
         atomicAdd(&r.chunk_counts[static_cast<size_t>(token / kRouterChunkTokens) * r.experts + my_expert], 1u);
     }
 }
@@ -332,9 +333,14 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
     const int wave = tid >> 6;
     const uint32_t experts = r.experts;
 
-    // this wave's 64 tokens of the chunk; the first loads go out before anything waits
-    const uint32_t first_token = chunk * kRouterChunkTokens + static_cast<uint32_t>(wave) * kWaveSize;
-    const uint32_t wave_tokens = first_token < r.tokens ? min(static_cast<uint32_t>(kWaveSize), r.tokens - first_token) : 0u;
+    // this wave's tokens of the chunk: consecutive ones, an equal share of the chunk's (a short chunk is
+    // spread over all waves: placing is sequential inside a wave); the first loads go out before anything waits
+    const uint32_t chunk_first = chunk * kRouterChunkTokens;
+    const uint32_t chunk_tokens = min(static_cast<uint32_t>(kRouterChunkTokens), r.tokens - chunk_first);
+    const uint32_t share = (chunk_tokens + kRouterWavesPerBlock - 1) / kRouterWavesPerBlock;
+    const uint32_t wave_first = static_cast<uint32_t>(wave) * share;
+    const uint32_t first_token = chunk_first + wave_first;
+    const uint32_t wave_tokens = wave_first < chunk_tokens ? min(share, chunk_tokens - wave_first) : 0u;
     const uint32_t first_assignment = first_token * r.top_k;
     const uint32_t count = wave_tokens * r.top_k;
     uint32_t first_named[kGroupBatch];
@@ -343,11 +349,11 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
     for (int k = 0; k < kGroupBatch; ++k)
     {
         const uint32_t i = static_cast<uint32_t>(k * kWaveSize + lane);
-        first_named[k] = i < count ? r.selected_experts[first_assignment + i] : 0xffffffffu;
-        first_weight[k] = i < count ? r.selected_weights[first_assignment + i] : 0.0f;
+        first_named[k] = i < count ? load_agent(&r.selected_experts[first_assignment + i]) : 0xffffffffu;
+        first_weight[k] = i < count ? __uint_as_float(load_agent(reinterpret_cast<const uint32_t*>(&r.selected_weights[first_assignment + i]))) : 0.0f;
     }
-    const uint32_t non_finite = r.error_words[0];
-    const uint32_t first_bad = r.error_words[1];
+    const uint32_t non_finite = load_agent(&r.error_words[0]);
+    const uint32_t first_bad = load_agent(&r.error_words[1]);
     uint32_t status = NCNN_MOE_ROUTER_OK;
     if (non_finite != 0u)
         status = NCNN_MOE_ROUTER_NON_FINITE_LOGIT;
@@ -383,7 +389,7 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
             for (int j = 0; j < kGroupExpertsPerThread; ++j)
             {
                 const uint32_t e = tid * per_thread + j;
-                const uint32_t routed = (static_cast<uint32_t>(j) < per_thread && e < experts) ? r.chunk_counts[c * experts + e] : 0u;
+                const uint32_t routed = (static_cast<uint32_t>(j) < per_thread && e < experts) ? load_agent(&r.chunk_counts[c * experts + e]) : 0u;
                 total[j] += routed;
                 before[j] += c < chunk ? routed : 0u;
             }
@@ -415,7 +421,7 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
                 const uint32_t i = first + static_cast<uint32_t>(k * kWaveSize + lane);
                 named[k] = first_named[k];
                 if (first != 0u)
-                    named[k] = i < count ? r.selected_experts[first_assignment + i] : 0xffffffffu;
+                    named[k] = i < count ? load_agent(&r.selected_experts[first_assignment + i]) : 0xffffffffu;
             }
 #pragma unroll
             for (int k = 0; k < kGroupBatch; ++k)
@@ -466,8 +472,8 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
                 weight[k] = first_weight[k];
                 if (first != 0u)
                 {
-                    named[k] = i < count ? r.selected_experts[first_assignment + i] : 0xffffffffu;
-                    weight[k] = i < count ? r.selected_weights[first_assignment + i] : 0.0f;
+                    named[k] = i < count ? load_agent(&r.selected_experts[first_assignment + i]) : 0xffffffffu;
+                    weight[k] = i < count ? __uint_as_float(load_agent(reinterpret_cast<const uint32_t*>(&r.selected_weights[first_assignment + i]))) : 0.0f;
                 }
             }
 #pragma unroll
@@ -546,9 +552,10 @@ __global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArg
     if constexpr (FUSED)
     {
         __shared__ GroupShared group_shared;
-        // this workgroup's routes, counts and error words are made visible to the device, then the
-        // workgroup is counted; whoever counts last sees every other workgroup's
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        // this workgroup's routes (written through), counts and error words (atomics) have landed once
+        // its waves have waited for them; then the workgroup is counted, and whoever counts last reads
+        // every other workgroup's around its own L2: no cache write-back or invalidate is needed
+        __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         if (threadIdx.x == 0)
         {
@@ -558,7 +565,6 @@ __global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArg
         __syncthreads();
         if (group_shared.is_last == 0u)
             return;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         if (threadIdx.x == 0)
             *r.finished_selects = 0u;
         __syncthreads(); // is_last is read by all before place_chunk_routes writes it again

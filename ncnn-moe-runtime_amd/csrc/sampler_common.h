@@ -434,18 +434,6 @@ struct LogitsVector<NCNN_MOE_LOGITS_BF16>
     }
 };
 
-// Agent-scope relaxed accesses: they write through / read around the per-XCD L2, so data handed from
-// one workgroup to another needs no L2 write-back or invalidate, only a wait for the stores to land.
-__device__ __forceinline__ void store_agent(uint32_t* address, uint32_t value)
-{
-    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-__device__ __forceinline__ uint32_t load_agent(const uint32_t* address)
-{
-    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // Ascending integer key of a float for bitwise selection (larger logit, larger key); never 0 for a
 // finite logit, so 0 can mark an empty slot.
 __device__ __forceinline__ uint32_t ascending_key(float value)

@@ -214,6 +214,18 @@ __device__ __forceinline__ void lds_barrier()
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// Agent-scope relaxed accesses: they write through / read around the per-XCD L2, so data handed from
+// one workgroup to another needs no L2 write-back or invalidate, only a wait for the stores to land.
+__device__ __forceinline__ void store_agent(uint32_t* address, uint32_t value)
+{
+    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ uint32_t load_agent(const uint32_t* address)
+{
+    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ float read_lane(float value, int lane)
 {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(value), lane));
