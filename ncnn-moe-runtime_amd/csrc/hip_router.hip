@@ -71,11 +71,13 @@ void launch_select(const RouterArgs& args, hipStream_t stream)
     const unsigned blocks = (args.tokens + kRouterWavesPerBlock - 1) / kRouterWavesPerBlock;
     if (args.tokens <= static_cast<uint32_t>(kRouterChunkTokens))
     {
-        // one chunk of tokens: the select kernel's last workgroup places the routes itself
-        hipLaunchKernelGGL((router_select_kernel<SLOTS, true>), dim3(blocks), dim3(kRouterThreads), 0, stream, args);
+        // one chunk of tokens: the select kernel's last workgroup places the routes itself, and the
+        // scores are computed by all threads of a workgroup of few tokens
+        const unsigned staged_blocks = (args.tokens + kStagedTokensPerBlock - 1) / kStagedTokensPerBlock;
+        hipLaunchKernelGGL((router_select_kernel<SLOTS, true, true>), dim3(staged_blocks), dim3(kRouterThreads), 0, stream, args);
         return;
     }
-    hipLaunchKernelGGL((router_select_kernel<SLOTS, false>), dim3(blocks), dim3(kRouterThreads), 0, stream, args);
+    hipLaunchKernelGGL((router_select_kernel<SLOTS, false, false>), dim3(blocks), dim3(kRouterThreads), 0, stream, args);
     const unsigned chunks = (args.tokens + kRouterChunkTokens - 1) / kRouterChunkTokens;
     hipLaunchKernelGGL(router_group_kernel, dim3(chunks), dim3(kRouterThreads), 0, stream, args);
 }

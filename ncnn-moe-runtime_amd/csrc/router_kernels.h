@@ -143,13 +143,72 @@ struct RouterArgs
 
 struct RouterShared
 {
-    float scores[kRouterWavesPerBlock][NCNN_MOE_ROUTER_MAX_EXPERTS]; // a token's scores, for the caller-named experts
+    float scores[kRouterWavesPerBlock][NCNN_MOE_ROUTER_MAX_EXPERTS]; // a token's scores: for the caller-named experts, or staged
+    uint32_t non_finite[kRouterWavesPerBlock];                       // staged scoring: the token holds a non-finite logit
+    float staged_maximum[kRouterWavesPerBlock];                      // staged softmax: the waves' maxima
 };
+
+// Decode-sized calls (STAGED): a workgroup takes kStagedTokensPerBlock tokens instead of one per wave
+// and all its threads compute the scores, one or a few experts each, into LDS; a wave per token then
+// selects from there.  The scores of a token (exp, log1p, sqrt per expert) are two fifths of a lone
+// wave's time for it; spread over four waves they take a quarter as long.  (The softmax sum is the CPU's
+// loop, one addition at a time in expert order, and stays with the selecting wave.)
+constexpr int kStagedTokensPerBlock = 2;
+constexpr int kStagedThreadsPerToken = kRouterThreads / kStagedTokensPerBlock;
+
+__device__ __forceinline__ float router_score_of_logit(float logit, uint32_t score_function);
+
+__device__ __forceinline__ void stage_token_scores(const RouterArgs& r, RouterShared& shared, uint32_t first_token)
+{
+    const int slot = threadIdx.x / kStagedThreadsPerToken;
+    const int member = threadIdx.x % kStagedThreadsPerToken;
+    const uint32_t token = first_token + static_cast<uint32_t>(slot);
+    if (threadIdx.x < kStagedTokensPerBlock)
+        shared.non_finite[threadIdx.x] = 0u;
+    __syncthreads();
+    constexpr int kPerThread = NCNN_MOE_ROUTER_MAX_EXPERTS / kStagedThreadsPerToken;
+    float logit[kPerThread];
+    bool finite = true;
+    float maximum = -__builtin_inff();
+    const float* logits = r.logits + static_cast<size_t>(token < r.tokens ? token : 0u) * r.experts;
+#pragma unroll
+    for (int k = 0; k < kPerThread; ++k)
+    {
+        const uint32_t e = static_cast<uint32_t>(k * kStagedThreadsPerToken + member);
+        logit[k] = (token < r.tokens && e < r.experts) ? logits[e] : -__builtin_inff();
+        finite = finite && (e >= r.experts || is_finite_f32(logit[k]));
+        maximum = fmaxf(maximum, logit[k]);
+    }
+    if (token < r.tokens && !finite)
+        shared.non_finite[slot] = 1u;
+    if (r.score_function == NCNN_MOE_ROUTER_SOFTMAX)
+    {
+        // the row maximum first (src/graph/expert_dispatcher.cpp:44-46); the sum stays with the selecting wave
+        maximum = wave_max(maximum);
+        if ((threadIdx.x & (kWaveSize - 1)) == 0)
+            shared.staged_maximum[threadIdx.x >> 6] = maximum;
+        __syncthreads();
+        constexpr int kWavesPerToken = kStagedThreadsPerToken / kWaveSize;
+        maximum = shared.staged_maximum[slot * kWavesPerToken];
+#pragma unroll
+        for (int w = 1; w < kWavesPerToken; ++w)
+            maximum = fmaxf(maximum, shared.staged_maximum[slot * kWavesPerToken + w]);
+    }
+#pragma unroll
+    for (int k = 0; k < kPerThread; ++k)
+    {
+        const uint32_t e = static_cast<uint32_t>(k * kStagedThreadsPerToken + member);
+        if (token < r.tokens && e < r.experts)
+            shared.scores[slot][e] = r.score_function == NCNN_MOE_ROUTER_SOFTMAX ? expf_libm(logit[k] - maximum)
+                                                                                : router_score_of_logit(logit[k], r.score_function);
+    }
+    __syncthreads();
+}
 
 // One wave per token.  Expert e lives in slot e / 64 of lane e % 64, so a loop over slots, then lanes,
 // visits the experts in index order: the softmax sum is the CPU loop itself, one fp32 addition at a
 // time.  The routes are chosen one per round and stay in registers: lane r keeps the route of rank r.
-template <int SLOTS>
+template <int SLOTS, bool COUNT_CHUNKS, bool STAGED>
 __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterShared& shared, uint32_t token, int lane, int wave)
 {
     const int experts = static_cast<int>(r.experts);
@@ -164,7 +223,7 @@ __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterS
     for (int s = 0; s < SLOTS; ++s)
     {
         const int e = s * kWaveSize + lane;
-        logit[s] = e < experts ? logits[e] : 0.0f;
+        logit[s] = (e < experts && !STAGED) ? logits[e] : 0.0f;
         bias[s] = (e < experts && r.selection_bias != nullptr && !explicit_routes) ? r.selection_bias[e] : 0.0f;
     }
     uint32_t my_expert = (explicit_routes && lane < top_k) ? r.explicit_ids[static_cast<size_t>(token) * r.top_k + lane] : 0u;
@@ -181,7 +240,7 @@ __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterS
             maximum = fmaxf(maximum, logit[s]);
         }
     }
-    if (__ballot(!finite) != 0)
+    if (STAGED ? shared.non_finite[wave] != 0u : __ballot(!finite) != 0)
     {
         // src/graph/expert_dispatcher.cpp:98-102: any non-finite logit of the call fails it
         if (lane == 0)
@@ -196,7 +255,12 @@ __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterS
         maximum = wave_max(maximum);
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
-            score[s] = (s * kWaveSize + lane) < experts ? expf_libm(logit[s] - maximum) : 0.0f;
+        {
+            if constexpr (STAGED)
+                score[s] = (s * kWaveSize + lane) < experts ? shared.scores[wave][s * kWaveSize + lane] : 0.0f;
+            else
+                score[s] = (s * kWaveSize + lane) < experts ? expf_libm(logit[s] - maximum) : 0.0f;
+        }
         float sum = 0.0f;
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
@@ -214,6 +278,12 @@ __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterS
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
             score[s] = score[s] / sum;
+    }
+    else if constexpr (STAGED)
+    {
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s)
+            score[s] = (s * kWaveSize + lane) < experts ? shared.scores[wave][s * kWaveSize + lane] : 0.0f;
     }
     else
     {
@@ -234,6 +304,7 @@ __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterS
                 atomicMin(&r.error_words[1], (token << 3) | NCNN_MOE_ROUTER_EXPERT_OUT_OF_RANGE);
             return;
         }
+        // (staged scores are in LDS already, but a softmax row only before its division by the sum)
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
         {
@@ -306,7 +377,8 @@ __device__ __forceinline__ void select_token_routes(const RouterArgs& r, RouterS
         // written through the per-XCD L2: the workgroup that groups the routes may sit on another XCD
         store_agent(&r.selected_experts[static_cast<size_t>(token) * r.top_k + lane], my_expert);
         store_agent(reinterpret_cast<uint32_t*>(&r.selected_weights[static_cast<size_t>(token) * r.top_k + lane]), __float_as_uint(weight));
-        atomicAdd(&r.chunk_counts[static_cast<size_t>(token / kRouterChunkTokens) * r.experts + my_expert], 1u);
+        if (COUNT_CHUNKS) // a call of one chunk is counted by the workgroup that groups it
+            atomicAdd(&r.chunk_counts[static_cast<size_t>(token / kRouterChunkTokens) * r.experts + my_expert], 1u);
     }
 }
 
@@ -372,7 +444,33 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
     }
     else
     {
-        // ---- this thread's experts: their routes in all chunks, and in the chunks before this one
+        // ---- a histogram of the experts of this wave's tokens
+        const auto build_histogram = [&]() {
+            for (uint32_t e = lane; e < experts; e += kWaveSize)
+                shared.wave_base[wave][e] = 0u;
+            lds_barrier();
+            for (uint32_t first = 0; first < count; first += kGroupBatch * kWaveSize)
+            {
+                uint32_t named[kGroupBatch];
+#pragma unroll
+                for (int k = 0; k < kGroupBatch; ++k)
+                {
+                    const uint32_t i = first + static_cast<uint32_t>(k * kWaveSize + lane);
+                    named[k] = first_named[k];
+                    if (first != 0u)
+                        named[k] = i < count ? load_agent(&r.selected_experts[first_assignment + i]) : 0xffffffffu;
+                }
+#pragma unroll
+                for (int k = 0; k < kGroupBatch; ++k)
+                {
+                    if (named[k] != 0xffffffffu)
+                        atomicAdd(&shared.wave_base[wave][named[k]], 1u);
+                }
+            }
+            __syncthreads();
+        };
+        // ---- this thread's experts: their routes in all chunks, and in the chunks before this one.
+        // A call of one chunk has no chunk counters: the totals are the sums of the waves' histograms.
         const uint32_t per_thread = (experts + kRouterThreads - 1) / kRouterThreads;
         uint32_t total[kGroupExpertsPerThread];
         uint32_t before[kGroupExpertsPerThread];
@@ -382,16 +480,34 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
             total[j] = 0u;
             before[j] = 0u;
         }
-#pragma unroll 8
-        for (uint32_t c = 0; c < chunks; ++c)
+        if (chunks == 1u)
         {
+            build_histogram();
 #pragma unroll
             for (int j = 0; j < kGroupExpertsPerThread; ++j)
             {
                 const uint32_t e = tid * per_thread + j;
-                const uint32_t routed = (static_cast<uint32_t>(j) < per_thread && e < experts) ? load_agent(&r.chunk_counts[c * experts + e]) : 0u;
-                total[j] += routed;
-                before[j] += c < chunk ? routed : 0u;
+                if (static_cast<uint32_t>(j) < per_thread && e < experts)
+                {
+#pragma unroll
+                    for (int w = 0; w < kRouterWavesPerBlock; ++w)
+                        total[j] += shared.wave_base[w][e];
+                }
+            }
+        }
+        else
+        {
+#pragma unroll 8
+            for (uint32_t c = 0; c < chunks; ++c)
+            {
+#pragma unroll
+                for (int j = 0; j < kGroupExpertsPerThread; ++j)
+                {
+                    const uint32_t e = tid * per_thread + j;
+                    const uint32_t routed = (static_cast<uint32_t>(j) < per_thread && e < experts) ? load_agent(&r.chunk_counts[c * experts + e]) : 0u;
+                    total[j] += routed;
+                    before[j] += c < chunk ? routed : 0u;
+                }
             }
         }
         uint32_t thread_sum = 0u;
@@ -407,30 +523,10 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
         }
         if (lane == kWaveSize - 1)
             shared.wave_totals[wave] = inclusive;
-
-        // ---- a histogram of the experts of this wave's tokens
-        for (uint32_t e = lane; e < experts; e += kWaveSize)
-            shared.wave_base[wave][e] = 0u;
-        lds_barrier();
-        for (uint32_t first = 0; first < count; first += kGroupBatch * kWaveSize)
-        {
-            uint32_t named[kGroupBatch];
-#pragma unroll
-            for (int k = 0; k < kGroupBatch; ++k)
-            {
-                const uint32_t i = first + static_cast<uint32_t>(k * kWaveSize + lane);
-                named[k] = first_named[k];
-                if (first != 0u)
-                    named[k] = i < count ? load_agent(&r.selected_experts[first_assignment + i]) : 0xffffffffu;
-            }
-#pragma unroll
-            for (int k = 0; k < kGroupBatch; ++k)
-            {
-                if (named[k] != 0xffffffffu)
-                    atomicAdd(&shared.wave_base[wave][named[k]], 1u);
-            }
-        }
-        __syncthreads();
+        if (chunks == 1u)
+            __syncthreads();
+        else
+            build_histogram();
         uint32_t exclusive = inclusive - thread_sum;
         for (int w = 0; w < wave; ++w)
             exclusive += shared.wave_totals[w];
@@ -521,7 +617,7 @@ __device__ __forceinline__ void place_chunk_routes(const RouterArgs& r, GroupSha
     __syncthreads();
     if (shared.is_last != 0u)
     {
-        for (uint32_t i = tid; i < chunks * experts; i += kRouterThreads)
+        for (uint32_t i = tid; chunks > 1u && i < chunks * experts; i += kRouterThreads)
             r.chunk_counts[i] = 0u;
         if (tid == 0)
         {
@@ -540,15 +636,19 @@ __global__ __launch_bounds__(kRouterThreads) void router_group_kernel(RouterArgs
 
 // FUSED (calls of at most one chunk of tokens): the workgroup that finishes last also places the
 // routes, so the whole dispatch is one launch.
-template <int SLOTS, bool FUSED>
+template <int SLOTS, bool FUSED, bool STAGED>
 __global__ __launch_bounds__(kRouterThreads) void router_select_kernel(RouterArgs r)
 {
+    static_assert(FUSED || !STAGED, "staged scoring serves the single-launch calls");
     __shared__ RouterShared shared;
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int wave = threadIdx.x >> 6;
-    const uint32_t token = blockIdx.x * kRouterWavesPerBlock + wave;
-    if (token < r.tokens)
-        select_token_routes<SLOTS>(r, shared, token, lane, wave);
+    constexpr int kTokensPerBlock = STAGED ? kStagedTokensPerBlock : kRouterWavesPerBlock;
+    const uint32_t token = blockIdx.x * kTokensPerBlock + wave;
+    if constexpr (STAGED)
+        stage_token_scores(r, shared, blockIdx.x * kTokensPerBlock);
+    if (wave < kTokensPerBlock && token < r.tokens)
+        select_token_routes<SLOTS, !FUSED, STAGED>(r, shared, token, lane, wave);
     if constexpr (FUSED)
     {
         __shared__ GroupShared group_shared;
