@@ -50,7 +50,7 @@ struct ncnn_moe_hip_sampler
     float* segment_values = nullptr;
     int32_t* segment_indices = nullptr;
     uint32_t* segment_counts = nullptr;
-    uint32_t* row_counter = nullptr;
+    unsigned long long* row_counter = nullptr;
     uint32_t* row_flags = nullptr;
     uint32_t* row_state = nullptr;
 
@@ -185,7 +185,15 @@ void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, S
     a.chunks_per_segment = g.chunks_per_segment;
     a.max_select_top_k = g.wide ? kSelectTopK : kFastTopK;
     a.only_pending = only_pending ? 1 : 0;
-    const dim3 grid(g.segments, rows, 1);
+    dim3 grid(g.segments, rows, 1);
+    a.xcd_grouped = 0;
+    if (g.segments > 1)
+    {
+        // one-dimensional, rows padded to a multiple of eight: workgroup 8 t + x is segment t % segments of
+        // row 8 (t / segments) + x, so that the XCDs' turns put the segments of a row on one XCD
+        a.xcd_grouped = 1;
+        grid = dim3(((rows + 7u) / 8u) * 8u * g.segments, 1, 1);
+    }
     if (g.wide)
         hipLaunchKernelGGL((scan_select_kernel<DTYPE, true, true>), grid, dim3(kScanThreads), 0, stream, a);
     else if (g.looped)
@@ -383,10 +391,10 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->segment_values, slots * kSegmentRecordSlots * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->segment_indices, slots * kSegmentRecordSlots * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->segment_counts, slots * sizeof(uint32_t)));
-    CREATE_CHECK(hipMalloc(&s->row_counter, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMalloc(&s->row_counter, rows * sizeof(unsigned long long)));
     CREATE_CHECK(hipMalloc(&s->row_flags, rows * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->row_state, rows * sizeof(uint32_t)));
-    CREATE_CHECK(hipMemset(s->row_counter, 0, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMemset(s->row_counter, 0, rows * sizeof(unsigned long long)));
     CREATE_CHECK(hipMemset(s->row_flags, 0, rows * sizeof(uint32_t)));
     CREATE_CHECK(hipMemset(s->row_state, 0, rows * sizeof(uint32_t)));
     for (int i = 0; i < 2; ++i)

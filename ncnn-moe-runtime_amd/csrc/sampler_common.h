@@ -28,7 +28,10 @@ struct SamplerArgs
     float* segment_values;     // [rows][segments][kSegmentRecordSlots]
     int32_t* segment_indices;  // [rows][segments][kSegmentRecordSlots]
     uint32_t* segment_counts;  // [rows][segments]
-    uint32_t* row_counter;     // [rows], zero between launches
+    // [rows], zero between launches: bits 0-7 count the row's finished segments, bits 8 + 6 x count
+    // those that ran on XCD x
+    unsigned long long* row_counter;
+    uint32_t xcd_grouped;      // the grid is one-dimensional and puts the segments of a row on one XCD
     uint32_t* row_flags;       // [rows], zero between launches
     uint32_t* row_state;       // [rows], written by every launch
 

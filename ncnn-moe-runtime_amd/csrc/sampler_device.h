@@ -24,6 +24,8 @@ constexpr int kSegmentValuesBF16 = kScanThreads * kVectorsPerLaneBF16 * 8; // 12
 constexpr int kFastTopK = 64;            // widest Top-K window finished by one wave
 constexpr int kSelectTopK = 1024;
 constexpr int kTwoKeyBoundTopK = 512; // wider windows bound their first chunk by a select over all its values         // widest Top-K window of the select path (rows of one segment)
+// s_getreg operand of the XCC_ID hardware register (id 20, offset 0, 4 bits): the XCD a wave runs on
+constexpr int kXccIdRegister = ((4 - 1) << 11) | (0 << 6) | 20;
 constexpr int kNarrowListCap = 512;      // candidate list for Top-K windows up to kFastTopK
 constexpr int kWideListCap = 4096;       // candidate list for Top-K windows up to kSelectTopK
 constexpr int kSegmentRecordSlots = 256; // candidate slots of a segment's record in HBM

@@ -29,6 +29,7 @@ struct SelectShared
     uint32_t list_count;
     uint32_t block_flags;
     int block_is_last;
+    int block_all_local;
     float final_values[kFastTopK];
     int32_t final_indices[kFastTopK];
     uint32_t sorted_keys[kSortedCap];    // descending keys of the ordered window when K > 64
@@ -382,8 +383,19 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     constexpr uint32_t kNegativeInfinity = 0xff800000u;
     constexpr uint32_t kPositiveInfinity = 0x7f800000u;
 
-    const uint32_t row = blockIdx.y;
-    const uint32_t segment = blockIdx.x;
+    // Workgroups are handed to the eight XCDs in turn.  A grouped grid numbers them so that the segments
+    // of a row all land on one XCD: the row's merge can then read their records from that XCD's L2.
+    // (Nothing relies on it: the counter below records where the segments really ran.)
+    uint32_t row = blockIdx.y;
+    uint32_t segment = blockIdx.x;
+    if (a.xcd_grouped != 0u)
+    {
+        const uint32_t turn = blockIdx.x >> 3;
+        row = (turn / a.segments) * 8u + (blockIdx.x & 7u);
+        segment = turn % a.segments;
+        if (row >= a.rows)
+            return;
+    }
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
 
@@ -716,8 +728,13 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     __syncthreads();
     if (tid == 0)
     {
-        const uint32_t previous = __hip_atomic_fetch_add(&a.row_counter[row], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        shared.block_is_last = previous == a.segments - 1 ? 1 : 0;
+        const uint32_t xcd = __builtin_amdgcn_s_getreg(kXccIdRegister) & 7u;
+        const int field = 8 + 6 * static_cast<int>(xcd);
+        const unsigned long long previous =
+            __hip_atomic_fetch_add(&a.row_counter[row], 1ull + (1ull << field), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        shared.block_is_last = (previous & 0xffull) == a.segments - 1 ? 1 : 0;
+        // every other segment of the row ran on this XCD: their records are in this XCD's L2
+        shared.block_all_local = ((previous >> field) & 63ull) == a.segments - 1 ? 1 : 0;
         shared.list_count = 0;
     }
     __syncthreads();
@@ -734,12 +751,15 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     constexpr int kPerThread = kMergeStageSlots / kScanThreads;
     uint32_t loaded_keys[kPerThread];
     uint32_t loaded_indices[kPerThread];
+    const bool all_local = shared.block_all_local != 0;
+    // agent-scope loads go around the L2 to the memory side; records written on this XCD are read from its L2
+    const auto load_record = [all_local](const uint32_t* address) { return all_local ? *address : load_agent(address); };
     const uint32_t row_flags = load_agent(&a.row_flags[row]);
     const bool stageable = row_entries <= static_cast<uint32_t>(kMergeStageSlots) && a.segments <= static_cast<uint32_t>(kMaxSegments);
     // all of a thread's slots belong to one segment (the workgroup's size is a multiple of 16)
     const uint32_t s = static_cast<uint32_t>(tid) & static_cast<uint32_t>(kMaxSegments - 1);
     const bool segment_exists = stageable && s < a.segments;
-    const uint32_t segment_count = segment_exists ? load_agent(&a.segment_counts[row_slot + s]) : 0u;
+    const uint32_t segment_count = segment_exists ? load_record(&a.segment_counts[row_slot + s]) : 0u;
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
     {
@@ -749,8 +769,8 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         loaded_indices[j] = 0;
         if (segment_exists && q < row_entries)
         {
-            loaded_keys[j] = load_agent(&out_values[(row_slot + s) * kSegmentRecordSlots + r]);
-            loaded_indices[j] = load_agent(&out_indices[(row_slot + s) * kSegmentRecordSlots + r]);
+            loaded_keys[j] = load_record(&out_values[(row_slot + s) * kSegmentRecordSlots + r]);
+            loaded_indices[j] = load_record(&out_indices[(row_slot + s) * kSegmentRecordSlots + r]);
         }
     }
     const uint8_t result_flags = (row_flags & kScanSawNan) ? NCNN_MOE_ROW_FLAG_HAS_NAN : 0;
