@@ -24,6 +24,7 @@ struct ncnn_moe_hip_sampler
     uint32_t max_segments = 0;
     uint64_t logits_stride_f32 = 0; // elements per row of the handle's logits buffer, fp32 view
     int force_general = 0;
+    int scatter_segments = 0;
     hipStream_t stream = nullptr;
 
     void* logits = nullptr;
@@ -179,7 +180,7 @@ SelectGeometry select_geometry(int dtype, uint64_t span, uint32_t rows, bool wid
 }
 
 template <int DTYPE>
-void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, SamplerArgs a, bool only_pending)
+void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, SamplerArgs a, bool only_pending, bool scatter_segments)
 {
     a.segments = g.segments;
     a.chunks_per_segment = g.chunks_per_segment;
@@ -187,7 +188,7 @@ void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, S
     a.only_pending = only_pending ? 1 : 0;
     dim3 grid(g.segments, rows, 1);
     a.xcd_grouped = 0;
-    if (g.segments > 1)
+    if (g.segments > 1 && !scatter_segments)
     {
         // one-dimensional, rows padded to a multiple of eight: workgroup 8 t + x is segment t % segments of
         // row 8 (t / segments) + x, so that the XCDs' turns put the segments of a row on one XCD
@@ -263,17 +264,17 @@ int launch_sampler(
     if (passes.select)
     {
         if (dtype == NCNN_MOE_LOGITS_F32)
-            launch_select<NCNN_MOE_LOGITS_F32>(batch_geometry, rows, stream, a, false);
+            launch_select<NCNN_MOE_LOGITS_F32>(batch_geometry, rows, stream, a, false, s->scatter_segments != 0);
         else
-            launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, a, false);
+            launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, a, false, s->scatter_segments != 0);
     }
     if (passes.wide_select)
     {
         const SelectGeometry row_geometry = select_geometry(dtype, span, rows, true);
         if (dtype == NCNN_MOE_LOGITS_F32)
-            launch_select<NCNN_MOE_LOGITS_F32>(row_geometry, rows, stream, a, true);
+            launch_select<NCNN_MOE_LOGITS_F32>(row_geometry, rows, stream, a, true, s->scatter_segments != 0);
         else
-            launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, stream, a, true);
+            launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, stream, a, true, s->scatter_segments != 0);
     }
     if (passes.full_order)
     {
@@ -826,6 +827,14 @@ int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* s, int enable
     if (s == nullptr)
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     s->force_general = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_debug_scatter_segments(ncnn_moe_hip_sampler* s, int enabled)
+{
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    s->scatter_segments = enabled ? 1 : 0;
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

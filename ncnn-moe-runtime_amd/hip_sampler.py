@@ -61,6 +61,7 @@ EXPORTED_SYMBOLS = [
     "ncnn_moe_hip_sampler_status_message",
     "ncnn_moe_hip_sampler_device_count",
     "ncnn_moe_hip_sampler_debug_force_general",
+    "ncnn_moe_hip_sampler_debug_scatter_segments",
     "ncnn_moe_hip_sampler_debug_expf",
     "ncnn_moe_hip_sampler_debug_exp2_table",
 ]
@@ -103,6 +104,7 @@ def load_library():
     lib.ncnn_moe_hip_sampler_status_message.restype = ctypes.c_char_p
     lib.ncnn_moe_hip_sampler_device_count.argtypes = []
     lib.ncnn_moe_hip_sampler_debug_force_general.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_scatter_segments.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_expf.argtypes = [vp, vp, vp, ctypes.c_size_t]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.argtypes = [vp]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.restype = None
@@ -238,6 +240,10 @@ class HipSampler:
 
     def force_general(self, enabled):
         self._check(self._lib.ncnn_moe_hip_sampler_debug_force_general(self._handle, 1 if enabled else 0))
+
+    def scatter_segments(self, enabled):
+        """Test hook: split rows are launched without the XCD-aware numbering of the workgroups."""
+        self._check(self._lib.ncnn_moe_hip_sampler_debug_scatter_segments(self._handle, 1 if enabled else 0))
 
     def expf(self, values):
         values = np.ascontiguousarray(values, dtype=np.float32)

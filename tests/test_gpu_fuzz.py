@@ -60,6 +60,12 @@ def test_random_batches(sampler, seed):
     if bf16:
         logits = workloads.float32_to_bf16_bits(logits)
     sampler.upload_logits(logits)
-    gpu = sampler.sample(params, uniforms, stop_ids)
+    # every other seed without the XCD-aware numbering of the workgroups: the segments of a row then run
+    # on several XCDs and the merge reads their records around the L2
+    sampler.scatter_segments(seed % 2 == 1)
+    try:
+        gpu = sampler.sample(params, uniforms, stop_ids)
+    finally:
+        sampler.scatter_segments(False)
     cpu = parity_util.run_oracle(logits, params, uniforms, stop_ids)
     parity_util.assert_results_match(gpu, cpu, "bf16" if bf16 else "f32", "fuzz seed %d" % seed)

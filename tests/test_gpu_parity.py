@@ -259,6 +259,21 @@ def test_cfg2_full():
     assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH == 0).all()
 
 
+def test_cfg2_with_scattered_segments():
+    """The same batch launched without the XCD-aware numbering of the workgroups (the merge then takes the
+    records of segments that ran on other XCDs around the L2): identical results."""
+    w = workloads.make_workload("cfg2_topk_topp")
+    _announce("cfg2 with scattered segments")
+    with hip_sampler.HipSampler(w["rows"], w["vocab"]) as sampler:
+        grouped = parity_util.run_workload_on_gpu(w, sampler)
+        sampler.scatter_segments(True)
+        scattered = parity_util.run_workload_on_gpu(w, sampler)
+        sampler.scatter_segments(False)
+    assert grouped.tobytes() == scattered.tobytes()
+    cpu = parity_util.run_oracle(w["logits"], w["params"], w["uniforms"], w["stop_ids"])
+    parity_util.assert_results_match(scattered, cpu, "f32", "cfg2 scattered")
+
+
 def test_cfg3_full():
     _full_config("cfg3_full_nucleus", "bf16")
 
