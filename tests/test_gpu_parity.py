@@ -424,11 +424,11 @@ def test_bf16_rows_of_few_distinct_values(batch_sampler):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-def test_windows_around_the_row_maxima_bound(batch_sampler, dtype):
-    """Windows up to 24 take their first bound from the 32 row maxima of a chunk, wider ones from the exact
-    selection over the lane maxima; a chunk with values in fewer than K rows of 16 lanes (a short row, a
-    short last segment) falls back to the exact one.  Every window size on both sides of the switch, on row
-    lengths that fill one lane row, a few, one chunk, and several segments; the select path must serve all."""
+def test_windows_around_the_quad_maxima_bound(batch_sampler, dtype):
+    """Windows up to 64 take their first bound from the 128 quad maxima of a chunk; a chunk with values in
+    fewer than 4 K / 3 quads of lanes (a short row, a short last segment) falls back to the exact selection
+    over the lane maxima.  Window sizes across the range, on row lengths that fill a few lanes, one chunk,
+    and several segments; the select path must serve all."""
     rng = np.random.default_rng(88)
     windows = np.array([1, 2, 15, 16, 17, 23, 24, 25, 31, 32, 33, 63, 64], dtype=np.uint32)
     for vocab in (40, 64, 700, 2049, 10240, 10300, 40000, 100003):
