@@ -393,7 +393,10 @@ def main():
     # need the full-order kernels (no Top-K window, or one wider than 64)
     effective_k = np.where((workload["params"]["top_k"] == 0) | (workload["params"]["top_k"] >= vocab),
                            vocab, workload["params"]["top_k"])
-    may_need_full_order = bool(np.any((workload["params"]["temperature"] != 0) & (effective_k > 64)))
+    sampled = workload["params"]["temperature"] != 0
+    may_need_full_order = int(np.any(sampled & (effective_k > 64)))
+    if np.count_nonzero(sampled & (effective_k > 64) & (effective_k <= 1024)) >= 32 and np.count_nonzero(sampled & (effective_k > 1024)) >= 32:
+        may_need_full_order |= hip_sampler.PASSES_SIDE_BY_SIDE  # as a scheduler that knows its Sessions' options would
 
     def step(index):
         sampler.sample_device(

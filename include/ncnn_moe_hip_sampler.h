@@ -131,7 +131,14 @@ int ncnn_moe_hip_sampler_sample(
  * may_need_full_order: pass 0 when the caller knows from its host-side SamplingOptions that every
  * row is greedy or has 1 <= top_k <= 64 (then one kernel is enqueued); pass 1 otherwise (a select
  * kernel for Top-K windows up to 1024 and the full-order kernels are enqueued as well and pick up
- * the rows that need them).  Calls on one handle share its scratch memory and must not overlap. */
+ * the rows that need them); pass 3 (1 | NCNN_MOE_PASSES_SIDE_BY_SIDE) when the caller knows that the
+ * batch holds both rows with 64 < top_k <= 1024 and rows with a wider or no window: the two later
+ * passes, each of which keeps one workgroup per row busy, then run side by side, one of them on a
+ * second stream of the handle that forks from and joins `stream` (worth its two stream hand-overs,
+ * some 30 us, from about a hundred rows of each kind).  Calls on one handle share its scratch memory
+ * and must not overlap. */
+#define NCNN_MOE_PASSES_FULL_ORDER 1
+#define NCNN_MOE_PASSES_SIDE_BY_SIDE 2
 int ncnn_moe_hip_sampler_sample_device(
     ncnn_moe_hip_sampler* sampler,
     const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,

@@ -25,6 +25,10 @@ struct ncnn_moe_hip_sampler
     uint64_t logits_stride_f32 = 0; // elements per row of the handle's logits buffer, fp32 view
     int force_general = 0;
     int scatter_segments = 0;
+    // a call with rows for the wide select and rows for the full-order kernels runs the two side by side
+    hipStream_t side_stream = nullptr;
+    hipEvent_t side_fork = nullptr;
+    hipEvent_t side_join = nullptr;
     hipStream_t stream = nullptr;
 
     void* logits = nullptr;
@@ -212,12 +216,15 @@ struct DistributionExport
     uint32_t cap = 0;
 };
 
+constexpr uint32_t kSideBySideRows = 32; // rows of each kind from which sample() runs the two later passes side by side
+
 // Which kernels a call enqueues.  Rows a pass cannot serve are marked pending and taken by the next.
 struct SamplerPasses
 {
     bool select = true;      // the batch-shaped select kernel
     bool wide_select = false; // one workgroup per row still pending: Top-K windows up to kSelectTopK
     bool full_order = false; // sort + replay for every row still pending
+    bool side_by_side = false; // the wide select on the handle's second stream, beside the full-order kernels
 };
 
 // Enqueues the sampling path for `rows` rows.
@@ -268,16 +275,14 @@ int launch_sampler(
         else
             launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, a, false, s->scatter_segments != 0);
     }
-    if (passes.wide_select)
-    {
+    const auto launch_wide = [&](hipStream_t on) {
         const SelectGeometry row_geometry = select_geometry(dtype, span, rows, true);
         if (dtype == NCNN_MOE_LOGITS_F32)
-            launch_select<NCNN_MOE_LOGITS_F32>(row_geometry, rows, stream, a, true, s->scatter_segments != 0);
+            launch_select<NCNN_MOE_LOGITS_F32>(row_geometry, rows, on, a, true, s->scatter_segments != 0);
         else
-            launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, stream, a, true, s->scatter_segments != 0);
-    }
-    if (passes.full_order)
-    {
+            launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, on, a, true, s->scatter_segments != 0);
+    };
+    const auto launch_full_order = [&](const SamplerArgs& a) {
         // the token indices ride along with the keys only when the whole distribution is exported
         if (dtype == NCNN_MOE_LOGITS_F32)
         {
@@ -298,6 +303,30 @@ int launch_sampler(
             else
                 hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
         }
+    };
+    // Rows for the wide select and rows for the full-order kernels are disjoint and each pass keeps few
+    // compute units busy (one workgroup per row): with both kinds in the call the two passes run side by
+    // side, the wide select on the handle's second stream.  The full-order kernels then leave the wide
+    // select's rows alone, and are enqueued once more behind the join for the rows that the wide select
+    // could not finish (ties beyond its lists); without such rows that launch exits at once.
+    if (passes.side_by_side && passes.wide_select && passes.full_order && s->side_stream != nullptr)
+    {
+        if (hipEventRecord(s->side_fork, stream) != hipSuccess || hipStreamWaitEvent(s->side_stream, s->side_fork, 0) != hipSuccess)
+            return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
+        launch_wide(s->side_stream);
+        SamplerArgs own_rows = a;
+        own_rows.leave_wide_rows = 1;
+        launch_full_order(own_rows);
+        if (hipEventRecord(s->side_join, s->side_stream) != hipSuccess || hipStreamWaitEvent(stream, s->side_join, 0) != hipSuccess)
+            return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "join of the second stream failed");
+        launch_full_order(a);
+    }
+    else
+    {
+        if (passes.wide_select)
+            launch_wide(stream);
+        if (passes.full_order)
+            launch_full_order(a);
     }
     SAMPLER_HIP_CHECK(s, hipGetLastError());
     return NCNN_MOE_SAMPLER_SUCCESS;
@@ -373,6 +402,9 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
 
     CREATE_CHECK(hipSetDevice(device));
     CREATE_CHECK(hipStreamCreate(&s->stream));
+    CREATE_CHECK(hipStreamCreateWithFlags(&s->side_stream, hipStreamNonBlocking));
+    CREATE_CHECK(hipEventCreateWithFlags(&s->side_fork, hipEventDisableTiming));
+    CREATE_CHECK(hipEventCreateWithFlags(&s->side_join, hipEventDisableTiming));
     const size_t rows = max_rows;
     const size_t slots = rows * s->max_segments;
     CREATE_CHECK(hipMalloc(&s->logits, rows * s->logits_stride_f32 * sizeof(float)));
@@ -433,6 +465,15 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
         (void)hipStreamSynchronize(s->stream);
         (void)hipStreamDestroy(s->stream);
     }
+    if (s->side_stream != nullptr)
+    {
+        (void)hipStreamSynchronize(s->side_stream);
+        (void)hipStreamDestroy(s->side_stream);
+    }
+    if (s->side_fork != nullptr)
+        (void)hipEventDestroy(s->side_fork);
+    if (s->side_join != nullptr)
+        (void)hipEventDestroy(s->side_join);
     void* buffers[] = {
         s->logits, s->params, s->uniforms, s->results, s->stop_ids, s->segment_values, s->segment_indices,
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->sort_keys[0], s->sort_keys[1],
@@ -554,11 +595,19 @@ int ncnn_moe_hip_sampler_sample(
     // the host sees the options: the later passes are enqueued only if some row needs them
     SamplerPasses passes;
     passes.full_order = s->force_general != 0;
+    uint32_t wide_rows = 0;
+    uint32_t full_order_rows = 0;
     for (uint32_t row = 0; row < rows; ++row)
     {
-        passes.wide_select = passes.wide_select || row_left_pending(params[row], s->logits_vocab, kFastTopK);
-        passes.full_order = passes.full_order || row_left_pending(params[row], s->logits_vocab, kSelectTopK);
+        const bool beyond_select = row_left_pending(params[row], s->logits_vocab, kSelectTopK);
+        const bool beyond_fast = !beyond_select && row_left_pending(params[row], s->logits_vocab, kFastTopK);
+        passes.wide_select = passes.wide_select || beyond_fast;
+        passes.full_order = passes.full_order || beyond_select;
+        wide_rows += beyond_fast ? 1u : 0u;
+        full_order_rows += beyond_select ? 1u : 0u;
     }
+    // enough rows of each kind for the two passes to be worth the hand-over between two streams
+    passes.side_by_side = wide_rows >= kSideBySideRows && full_order_rows >= kSideBySideRows;
     const bool full_order = passes.full_order;
     int rc = launch_sampler(
         s, s->logits, s->logits_dtype, rows, s->logits_vocab, s->logits_stride,
@@ -609,6 +658,7 @@ int ncnn_moe_hip_sampler_sample_device(
     SamplerPasses passes;
     passes.wide_select = may_need_full_order != 0;
     passes.full_order = may_need_full_order != 0 || s->force_general != 0;
+    passes.side_by_side = (may_need_full_order & NCNN_MOE_PASSES_SIDE_BY_SIDE) != 0;
     return launch_sampler(
         s, device_logits, dtype, rows, vocab, row_stride, device_params, device_uniforms, device_stop_ids,
         device_results, DistributionExport{}, passes, static_cast<hipStream_t>(stream));
@@ -722,8 +772,8 @@ int ncnn_moe_hip_sampler_speculative_verify(
     // the host sees the options: the later passes are enqueued only if the rows can need them; a row whose
     // ties overflow the select lists reports that, and the step is run again with the full-order kernels
     SamplerPasses passes;
-    passes.wide_select = row_left_pending(row_options, s->logits_vocab, kFastTopK);
     passes.full_order = s->force_general != 0 || row_left_pending(row_options, s->logits_vocab, kSelectTopK);
+    passes.wide_select = !passes.full_order && row_left_pending(row_options, s->logits_vocab, kFastTopK);
     bool dense = s->verify_dense_known && std::memcmp(&s->verify_dense_options, &row_options, sizeof(row_options)) == 0;
     for (int attempt = 0; attempt < 2 && !dense; ++attempt)
     {

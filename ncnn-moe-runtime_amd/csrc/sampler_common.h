@@ -18,6 +18,7 @@ struct SamplerArgs
     uint32_t max_select_top_k;   // widest Top-K window the select kernel of this launch serves
     int force_general;
     int only_pending;            // serve only rows an earlier launch of the call left pending
+    int leave_wide_rows;         // full-order kernels: rows that the wide select serves are another stream's
 
     const ncnn_moe_sample_params* params;
     const float* uniforms;

@@ -10,6 +10,18 @@
 
 namespace ncnn_moe_hip {
 
+// A call that holds rows for the wide select and rows for these kernels runs the two passes side by
+// side on two streams: the rows of the wide select are pending as well and are skipped here (a later
+// launch without the flag takes those that the wide select could not finish).
+__device__ __forceinline__ bool left_to_the_wide_select(const SamplerArgs& a, uint32_t row)
+{
+    if (a.leave_wide_rows == 0)
+        return false;
+    uint32_t effective_k = 0;
+    int status = NCNN_MOE_ROW_OK;
+    return resolve_row_mode(a.params[row], a.vocab, static_cast<uint32_t>(kSelectTopK), a.force_general, effective_k, status) != kModeGeneral;
+}
+
 template <int DTYPE>
 __device__ __forceinline__ float load_logit(const void* row_pointer, uint32_t i);
 
@@ -36,7 +48,7 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
     constexpr int kPasses = DTYPE == NCNN_MOE_LOGITS_F32 ? 4 : 2;
     constexpr int kFirstDigit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0 : 2;
     const uint32_t row = blockIdx.x;
-    if (a.row_state[row] != kRowNeedsGeneral)
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
         return;
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
@@ -271,7 +283,7 @@ constexpr int kCachedRuns = 6144; // runs of a row the replay keeps in LDS (48 K
 __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(SamplerArgs a)
 {
     const uint32_t row = blockIdx.x;
-    if (a.row_state[row] != kRowNeedsGeneral)
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
         return;
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
@@ -547,7 +559,7 @@ template <int DTYPE, bool RUNS>
 __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerArgs a)
 {
     const uint32_t row = blockIdx.x;
-    if (a.row_state[row] != kRowNeedsGeneral)
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
         return;
     const int tid = threadIdx.x;
     const ncnn_moe_sample_params p = a.params[row];

@@ -33,6 +33,8 @@ VERIFY_ZERO_DRAFT_PROBABILITY = 2
 VERIFY_RESIDUAL_EMPTY = 3
 VERIFY_RESIDUAL_FAILED = 4
 VERIFY_UNSUPPORTED_WINDOW = 5
+PASSES_FULL_ORDER = 1     # sample_device: the later passes are enqueued as well
+PASSES_SIDE_BY_SIDE = 2   # ... and run side by side (rows with wide windows and rows without a window are both present)
 MAX_DRAFT_TOKENS = 16
 
 FLAG_HAS_NAN = 1
@@ -207,7 +209,7 @@ class HipSampler:
         """All pointers are device addresses (ints); enqueues and returns."""
         self._check(self._lib.ncnn_moe_hip_sampler_sample_device(
             self._handle, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr,
-            stop_ids_ptr, results_ptr, 1 if may_need_full_order else 0, stream))
+            stop_ids_ptr, results_ptr, int(may_need_full_order), stream))
 
     def distribution(self, row, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, cap=None):
         """Returns (row_status, ids, probabilities) for one row of the uploaded logits."""

@@ -57,6 +57,38 @@ def test_three_passes_on_a_caller_stream(rows):
         parity_util.assert_results_match(again, cpu, "f32", "sample_device, repeated")
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_later_passes_side_by_side(dtype):
+    """Rows with wide windows and rows without a window in one batch: the wide select on the handle's
+    second stream beside the full-order kernels (flag NCNN_MOE_PASSES_SIDE_BY_SIDE, and sample() by
+    itself from 32 rows of each kind), with tie-heavy wide rows that the wide select hands on to the
+    full-order kernels behind the join.  Same results as one pass after the other, and as the oracle."""
+    print("[case] later passes side by side, %s" % dtype, flush=True)
+    from ncnn_moe_runtime_amd import workloads
+    rng = np.random.default_rng(77)
+    rows, vocab = 120, 30011
+    logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    logits[5::12] = np.round(logits[5::12])  # a few thousand equal logits around every cut
+    params = hip_sampler.make_params(rows, 0.9, 0, 0.9, 0.0)
+    params["top_k"] = np.array([(700, 0, 20, 300, 2000, 1024)[i % 6] for i in range(rows)], dtype=np.uint32)
+    params["temperature"][::17] = 0.0
+    uniforms = rng.random(rows).astype(np.float32)
+    data = workloads.float32_to_bf16_bits(logits) if dtype == "bf16" else logits
+    cpu = parity_util.run_oracle(data, params, uniforms)
+    stream = torch.cuda.Stream(device="cuda:0")
+    with hip_sampler.HipSampler(rows, vocab) as sampler:
+        in_turn = _run(sampler, data, params, uniforms, hip_sampler.PASSES_FULL_ORDER, stream)
+        beside = _run(sampler, data, params, uniforms, hip_sampler.PASSES_FULL_ORDER | hip_sampler.PASSES_SIDE_BY_SIDE, stream)
+        assert in_turn.tobytes() == beside.tobytes()
+        parity_util.assert_results_match(beside, cpu, dtype, "side by side, device entry")
+        for _ in range(3):  # the second stream forks and joins again on every call
+            again = _run(sampler, data, params, uniforms, hip_sampler.PASSES_FULL_ORDER | hip_sampler.PASSES_SIDE_BY_SIDE, stream)
+            assert again.tobytes() == beside.tobytes()
+        sampler.upload_logits(data)
+        host = sampler.sample(params, uniforms)
+        parity_util.assert_results_match(host, cpu, dtype, "side by side, host entry")
+
+
 def test_bf16_strided_rows_on_the_default_stream():
     print("[case] sample_device, bf16, stride wider than the vocabulary", flush=True)
     from ncnn_moe_runtime_amd import workloads

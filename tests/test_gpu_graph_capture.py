@@ -18,8 +18,11 @@ def _bytes(array):
     return torch.from_numpy(np.ascontiguousarray(array).view(np.uint8).reshape(-1))
 
 
-def test_sampler_step_in_a_graph():
-    print("[case] sample_device captured in a HIP graph, 4 replays", flush=True)
+@pytest.mark.parametrize("passes", [hip_sampler.PASSES_FULL_ORDER, hip_sampler.PASSES_FULL_ORDER | hip_sampler.PASSES_SIDE_BY_SIDE])
+def test_sampler_step_in_a_graph(passes):
+    """Every pass in one captured call; with the side-by-side flag the handle's second stream forks from
+    and joins the captured stream, so the graph holds two branches."""
+    print("[case] sample_device captured in a HIP graph (passes %d), 4 replays" % passes, flush=True)
     rng = np.random.default_rng(31)
     rows, vocab = 48, 40013
     params = hip_sampler.make_params(rows, 0.8, 0, 0.9, 0.0)
@@ -34,7 +37,7 @@ def test_sampler_step_in_a_graph():
     with hip_sampler.HipSampler(rows, vocab) as sampler:
         def enqueue():
             sampler.sample_device(d_logits.data_ptr(), hip_sampler.LOGITS_F32, rows, vocab, vocab, d_params.data_ptr(),
-                                  d_uniforms.data_ptr(), None, d_results.data_ptr(), True, stream.cuda_stream)
+                                  d_uniforms.data_ptr(), None, d_results.data_ptr(), passes, stream.cuda_stream)
 
         with torch.cuda.stream(stream):
             enqueue()  # eager once: everything the entry sets up lazily exists before the capture
