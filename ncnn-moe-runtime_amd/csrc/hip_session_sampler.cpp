@@ -368,6 +368,21 @@ SamplingSession::SamplingSession(HipSamplerPtr sampler, const SamplingSessionOpt
 {
 }
 
+float SamplingSession::uniform_ahead(size_t position)
+{
+    while (drawn_ahead_.size() <= position)
+    {
+        std::uniform_real_distribution<float> distribution(0.0f, 1.0f);
+        drawn_ahead_.push_back(distribution(random_generator_));
+    }
+    return drawn_ahead_[position];
+}
+
+void SamplingSession::consume_uniforms(size_t count)
+{
+    drawn_ahead_.erase(drawn_ahead_.begin(), drawn_ahead_.begin() + static_cast<std::ptrdiff_t>(std::min(count, drawn_ahead_.size())));
+}
+
 Result<SampledToken> SamplingSession::sample(const LogitsOutput& logits, const SamplingOptions& options)
 {
     const std::lock_guard<std::mutex> lock(mutex_);
@@ -375,8 +390,7 @@ Result<SampledToken> SamplingSession::sample(const LogitsOutput& logits, const S
         return invalid_argument("cannot sample empty logits");
     if (!sampler_)
         return Error{ErrorCode::InternalError, "hip sampler is unavailable (no GPU, or create() failed)"};
-    std::mt19937_64 advanced;
-    const float uniform = peek_uniform(random_generator_, advanced);
+    const float uniform = uniform_ahead(0);
     const std::span<const float> row(logits.values);
     std::vector<uint8_t> draw_consumed;
     const SampleTimer timer;
@@ -387,7 +401,7 @@ Result<SampledToken> SamplingSession::sample(const LogitsOutput& logits, const S
     if (!results[0])
         return results[0].error();
     if (draw_consumed[0])
-        random_generator_ = advanced;
+        consume_uniforms(1);
     return results[0].value().token;
 }
 
@@ -410,17 +424,12 @@ Result<SpeculativeVerification> SamplingSession::verify_speculative(
     for (const LogitsOutput& row : draft_logits)
         draft_rows.emplace_back(row.values);
     // the draws the loop could consume, in the generator's order; only the consumed ones are committed
-    std::mt19937_64 shadow = random_generator_;
     std::vector<float> uniforms(proposed_token_ids.size() + 1);
-    for (float& uniform : uniforms)
-    {
-        std::mt19937_64 advanced;
-        uniform = peek_uniform(shadow, advanced);
-        shadow = advanced;
-    }
+    for (size_t i = 0; i < uniforms.size(); ++i)
+        uniforms[i] = uniform_ahead(i);
     uint32_t draws_consumed = 0;
     auto verified = sampler_->verify_speculative(target_rows, draft_rows, proposed_token_ids, options, uniforms, draws_consumed);
-    random_generator_.discard(draws_consumed); // one 64-bit output per uniform_real_distribution<float> draw
+    consume_uniforms(draws_consumed);
     return verified;
 }
 
@@ -453,7 +462,6 @@ std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample(
     std::vector<std::span<const float>> logits;
     std::vector<SamplingOptions> options;
     std::vector<float> uniforms;
-    std::vector<std::mt19937_64> advanced;
     std::vector<std::vector<int32_t>> stop_tokens;
     for (size_t i = 0; i < rows; ++i)
     {
@@ -462,8 +470,7 @@ std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample(
         active.push_back(i);
         logits.emplace_back(requests[i].logits->values);
         options.push_back(requests[i].sampling);
-        advanced.emplace_back();
-        uniforms.push_back(peek_uniform(requests[i].session->random_generator_, advanced.back()));
+        uniforms.push_back(requests[i].session->uniform_ahead(0));
         stop_tokens.push_back(requests[i].stop_tokens);
     }
     std::vector<Result<BatchSampledToken>> out = every_row<BatchSampledToken>(rows, invalid_argument("cannot sample empty logits"));
@@ -478,7 +485,7 @@ std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample(
         out[i] = sampled[j];
         timer.charge(requests[i].session->statistics_, sampled[j] ? 1 : 0);
         if (sampled[j] && draw_consumed[j])
-            requests[i].session->random_generator_ = advanced[j];
+            requests[i].session->consume_uniforms(1);
     }
     return out;
 }
@@ -531,7 +538,6 @@ Result<std::vector<GenerationResult>> BatchGenerationLoop::generate(
 
     std::vector<SamplingOptions> row_options;
     std::vector<float> uniforms;
-    std::vector<std::mt19937_64> advanced;
     std::vector<std::vector<int32_t>> stop_tokens;
     std::vector<uint8_t> draw_consumed;
     std::vector<DecodeSlot> slots;
@@ -540,14 +546,13 @@ Result<std::vector<GenerationResult>> BatchGenerationLoop::generate(
     {
         row_options.clear();
         uniforms.clear();
-        stop_tokens.clear();
-        advanced.resize(active.size());
+        stop_tokens.resize(active.size());
         for (size_t row = 0; row < active.size(); ++row)
         {
             const uint32_t i = active[row];
             row_options.push_back(options_of(i).sampling);
-            uniforms.push_back(peek_uniform(sessions[i]->random_generator_, advanced[row]));
-            stop_tokens.push_back(options_of(i).stop_tokens);
+            uniforms.push_back(sessions[i]->uniform_ahead(0));
+            stop_tokens[row] = options_of(i).stop_tokens; // assignment reuses the row's storage from the last step
         }
         const SampleTimer timer;
         auto sampled = sampler->sample_resident(row_options, uniforms, stop_tokens, draw_consumed);
@@ -560,7 +565,7 @@ Result<std::vector<GenerationResult>> BatchGenerationLoop::generate(
             if (!sampled[row])
                 return sampled[row].error();
             if (draw_consumed[row])
-                sessions[i]->random_generator_ = advanced[row];
+                sessions[i]->consume_uniforms(1);
             StreamToken token;
             token.index = index;
             token.token_id = sampled[row].value().token.token_id;
