@@ -27,6 +27,7 @@
 #include <random>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <vector>
 
 using namespace ncnn::moe;
@@ -290,6 +291,92 @@ static void test_batch_equals_serial(const HipSamplerPtr& sampler)
                 check(got[i].value().token.probability == expected[i].value().probability);
                 check(got[i].value().is_stop_token == (i % 2 == 0));
             }
+        }
+    }
+}
+
+// Worker threads that share one sampler, each with Sessions of its own (the runtime's scheduler
+// workers and std::async callers, src/engine/scheduler.cpp:87-104): every thread must see exactly
+// what it would have seen alone, single calls and batched calls interleaved.
+static void test_threads_share_a_sampler(const HipSamplerPtr& sampler)
+{
+    const int threads = 8;
+    const int steps = 30;
+    const int vocab = 3000;
+    std::vector<std::vector<LogitsOutput>> logits(threads, std::vector<LogitsOutput>(steps));
+    std::vector<SamplingOptions> options(threads);
+    for (int t = 0; t < threads; ++t)
+    {
+        std::mt19937_64 data(500 + t);
+        std::normal_distribution<float> normal(0.0f, 2.5f);
+        for (LogitsOutput& row : logits[t])
+        {
+            row.values.resize(vocab);
+            for (float& value : row.values)
+                value = normal(data);
+        }
+        options[t].temperature = 0.4f + 0.15f * static_cast<float>(t);
+        options[t].top_k = (t % 4 == 0) ? 0 : (t % 4 == 1) ? 40 : (t % 4 == 2) ? 200 : 8;
+        options[t].top_p = 0.7f + 0.03f * static_cast<float>(t);
+        options[t].min_p = (t % 2 == 0) ? 0.01f : 0.0f;
+    }
+    // thread t: step s is a single call on Session A when s is even, a batch over Sessions A and B when odd
+    const auto run = [&](int t, std::vector<SampledToken>& out) {
+        SamplingSessionOptions so;
+        so.sampling_seed = 7000 + t;
+        SamplingSession a(sampler, so);
+        so.sampling_seed = 8000 + t;
+        SamplingSession b(sampler, so);
+        for (int step = 0; step < steps; ++step)
+        {
+            if (step % 2 == 0)
+            {
+                auto sampled = a.sample(logits[t][step], options[t]);
+                check(static_cast<bool>(sampled));
+                out.push_back(sampled.value());
+                continue;
+            }
+            std::vector<SampleBatchRequest> requests(2);
+            requests[0].session = &a;
+            requests[0].logits = &logits[t][step];
+            requests[0].sampling = options[t];
+            requests[1].session = &b;
+            requests[1].logits = &logits[t][step - 1];
+            requests[1].sampling = options[(t + 1) % threads];
+            auto sampled = SessionBatchSampler::sample(sampler, requests);
+            check(sampled.size() == 2 && sampled[0] && sampled[1]);
+            out.push_back(sampled[0].value().token);
+            out.push_back(sampled[1].value().token);
+        }
+    };
+    std::vector<std::vector<SampledToken>> expected(threads);
+    for (int t = 0; t < threads; ++t)
+        run(t, expected[t]);
+    std::vector<std::vector<SampledToken>> got(threads);
+    std::vector<std::string> failures(threads);
+    std::vector<std::thread> workers;
+    for (int t = 0; t < threads; ++t)
+        workers.emplace_back([&, t] {
+            try
+            {
+                run(t, got[t]);
+            }
+            catch (const std::exception& error)
+            {
+                failures[t] = error.what();
+            }
+        });
+    for (std::thread& worker : workers)
+        worker.join();
+    for (int t = 0; t < threads; ++t)
+    {
+        if (!failures[t].empty())
+            throw std::runtime_error("thread " + std::to_string(t) + ": " + failures[t]);
+        check(got[t].size() == expected[t].size());
+        for (size_t i = 0; i < got[t].size(); ++i)
+        {
+            check(got[t][i].token_id == expected[t][i].token_id);
+            check(std::bit_cast<uint32_t>(got[t][i].probability) == std::bit_cast<uint32_t>(expected[t][i].probability));
         }
     }
 }
@@ -919,6 +1006,7 @@ int main(int argc, char** argv)
         test_rng_bookkeeping(sampler);
         test_distribution_known_answers(sampler);
         test_batch_equals_serial(sampler);
+        test_threads_share_a_sampler(sampler);
         test_batch_rejects_bad_requests(sampler);
         test_speculative_verification(sampler);
         test_generation_loop_equals_serial(sampler);
