@@ -58,9 +58,11 @@ __device__ __forceinline__ void append_candidate(SelectShared<WIDE>& shared, boo
 }
 
 // Raises the bound to (a lower bound of) the K-th best candidate of the list and drops the
-// candidates below it.  All threads call it; returns the new bound key.
+// candidates below it.  All threads call it; returns the new bound key.  exact == false (lists of one
+// entry per thread): the cheaper bound of the eight waves' own searches, which at least K entries
+// reach and usually two to three times as many.
 template <bool WIDE>
-__device__ __forceinline__ uint32_t tighten_list(SelectShared<WIDE>& shared, uint32_t bound_key, int top_k, int tid)
+__device__ __forceinline__ uint32_t tighten_list(SelectShared<WIDE>& shared, uint32_t bound_key, int top_k, int tid, bool exact = true)
 {
     constexpr int kPerThread = SelectShared<WIDE>::kListCap / kScanThreads;
     const int lane = tid & (kWaveSize - 1);
@@ -71,7 +73,10 @@ __device__ __forceinline__ uint32_t tighten_list(SelectShared<WIDE>& shared, uin
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
     {
-        const uint32_t q = static_cast<uint32_t>(j * kScanThreads + tid);
+        // one entry per thread: entry q goes to wave q % 8, so that every wave holds its share of a short
+        // list (the waves' own searches bound loosely where some waves hold nothing)
+        const uint32_t q = kPerThread == 1 ? static_cast<uint32_t>(lane * kScanWaves + (tid >> 6))
+                                           : static_cast<uint32_t>(j * kScanThreads + tid);
         keys[j] = q < count ? shared.list_keys[q] : 0u;
         indices[j] = q < count ? shared.list_indices[q] : 0;
         best = max(best, keys[j]);
@@ -86,7 +91,7 @@ __device__ __forceinline__ uint32_t tighten_list(SelectShared<WIDE>& shared, uin
     else
     {
         const uint32_t thread_keys[1] = {best};
-        kth = workgroup_kth_largest_key(thread_keys, top_k, tid, shared.bound, true);
+        kth = workgroup_kth_largest_key(thread_keys, top_k, tid, shared.bound, exact);
     }
     bound_key = max(bound_key, kth);
     if (tid == 0)
@@ -143,6 +148,19 @@ __device__ __forceinline__ void finish_from_list(
             if (n_list > 8 * kWaveSize)
             {
                 tighten_list(shared, 0u, top_k, tid);
+                n_list = __builtin_amdgcn_readfirstlane(static_cast<int>(shared.list_count));
+            }
+        }
+        else if (n_list > 2 * kWaveSize)
+        {
+            // A workgroup that streamed many chunks under its first chunk's bound ends with a few hundred
+            // candidates.  All eight waves cut the list down to what the rankings below take (128); one
+            // wave selecting among them bit by bit takes several times as long.
+            tighten_list(shared, 0u, top_k, tid, false);
+            n_list = __builtin_amdgcn_readfirstlane(static_cast<int>(shared.list_count));
+            if (n_list > 2 * kWaveSize)
+            {
+                tighten_list(shared, 0u, top_k, tid, true);
                 n_list = __builtin_amdgcn_readfirstlane(static_cast<int>(shared.list_count));
             }
         }
