@@ -651,7 +651,13 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
                 const uint32_t chunks = chunk - chunk_at_check + 1u;
                 const uint32_t rate = (count - count_at_check + chunks - 1u) / chunks; // candidates per chunk
                 if (count > tighten_limit)
-                    bound_key = tighten_list(shared, bound_key, top_k, tid);
+                {
+                    // the waves' own searches first (a third of the exact selection's time); what they
+                    // leave is nearly always short enough
+                    bound_key = tighten_list(shared, bound_key, top_k, tid, WIDE);
+                    if (!WIDE && shared.list_count > tighten_limit / 4u * 3u)
+                        bound_key = tighten_list(shared, bound_key, top_k, tid, true);
+                }
                 count_at_check = shared.list_count;
                 chunk_at_check = chunk + 1u;
                 const uint32_t slack = static_cast<uint32_t>(Shared::kListCap) - count_at_check;
