@@ -362,6 +362,28 @@ def test_whole_row_long_rows(batch_sampler):
     _check_rows(batch_sampler, logits, params, uniforms, context="whole-row workgroups, long sorted rows")
 
 
+def test_whole_row_long_final_lists(batch_sampler):
+    """Eleven chunks under the first chunk's bound leave a few hundred candidates for windows up to 64:
+    the workgroup cuts the final list with all its waves (loosely, then exactly where ties or a wide
+    window leave more than 128) before it ranks it."""
+    rng = np.random.default_rng(73)
+    rows, vocab = 256, 109999
+    logits = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    logits[64:128] = np.round(logits[64:128] * 8) / 8    # ties at every level, the cut included
+    logits[128:160] = np.round(logits[128:160])          # hundreds of candidates tie with the cut
+    params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+    params["top_k"] = np.array([(2, 20, 33, 48, 63, 64)[i % 6] for i in range(rows)], dtype=np.uint32)
+    params["temperature"] = rng.uniform(0.4, 1.3, size=rows).astype(np.float32)
+    params["top_p"] = rng.uniform(0.5, 1.0, size=rows).astype(np.float32)
+    uniforms = rng.random(rows).astype(np.float32)
+    select_rows = np.ones(rows, dtype=bool)
+    select_rows[128:160] = False                         # these may go on to the full-order kernels
+    _check_rows(batch_sampler, logits, params, uniforms, context="whole-row workgroups, long final lists",
+                select_rows=select_rows)
+    _check_rows(batch_sampler, workloads.float32_to_bf16_bits(logits), params, uniforms, dtype="bf16",
+                context="whole-row workgroups, long final lists, bf16", select_rows=None)
+
+
 @pytest.mark.parametrize("rows", [200, 130, 90])
 def test_multi_chunk_segments(batch_sampler, rows):
     """Between 65 and 255 rows of a long vocabulary a segment streams several chunks before the hand-over."""
