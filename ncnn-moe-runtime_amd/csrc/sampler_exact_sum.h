@@ -520,7 +520,10 @@ __device__ __forceinline__ RunningSum exact_running_sum_runs(
                 const ParityStep single = step_of_term(terms[j], exponent);
                 const bool odd = (current & 1u) != 0u;
                 const uint32_t next = current + repeated_step(odd, single, multiplicity);
-                if (multiplicity > 0u && !have_event && next >= limit)
+                // A thread that starts at or beyond the limit comes after the round's first event (the
+                // mantissa never decreases and began below the limit), so its own cannot be the first:
+                // it skips the search.  (A round that begins at the limit keeps every thread's event.)
+                if (multiplicity > 0u && !have_event && next >= limit && (current < limit || mantissa >= limit))
                 {
                     // the first addition of the run after which the mantissa reaches the limit
                     uint32_t none = 0u, some = multiplicity; // repeated additions: `none` stay below, `some` reach it
