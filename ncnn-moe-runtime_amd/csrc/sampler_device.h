@@ -41,8 +41,8 @@ constexpr int kSortThreads = 1024;
 constexpr int kSortWaves = kSortThreads / kWaveSize;
 constexpr int kSortPerThread = 8;
 constexpr int kSortTile = kSortThreads * kSortPerThread;
-constexpr int kReplayThreads = 512;
-constexpr int kReplayPerThread = 8;
+constexpr int kReplayThreads = 1024;
+constexpr int kReplayPerThread = 4;
 constexpr int kReplayChunk = kReplayThreads * kReplayPerThread;
 
 enum RowMode : int

@@ -14,8 +14,6 @@
 
 namespace ncnn_moe_hip {
 
-static_assert(kReplayThreads == kScanThreads, "the select kernel runs the window walk with its own workgroup");
-
 // Evaluates expf_libm on n values (test hook).
 __global__ void expf_probe_kernel(const float* in, float* out, size_t n)
 {

@@ -34,7 +34,6 @@ struct SelectShared
     int32_t final_indices[kFastTopK];
     uint32_t sorted_keys[kSortedCap];    // descending keys of the ordered window when K > 64
     uint32_t sorted_indices[kSortedCap];
-    ReplayScratch replay;
 };
 
 // Appends the caller's candidate (if `hit`) to the workgroup's list.  Positions are reserved per
