@@ -321,9 +321,18 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_terms(
             __syncthreads();
             if (scratch.absorbed)
                 return RunningSum{sum, 0u, false};
+            // every wave's total is read at once (independent LDS loads); the composition stays in registers
+            ParityStep totals[kReplayWaves];
+#pragma unroll
+            for (int w = 0; w < kReplayWaves; ++w)
+                totals[w] = scratch.wave_totals[w];
             ParityStep before{0u, 0u};
-            for (int w = 0; w < wave; ++w)
-                before = compose_steps(before, scratch.wave_totals[w]);
+#pragma unroll
+            for (int w = 0; w < kReplayWaves - 1; ++w)
+            {
+                if (w < wave)
+                    before = compose_steps(before, totals[w]);
+            }
             before = compose_steps(before, exclusive);
             uint32_t current = mantissa + ((mantissa & 1u) ? before.odd : before.even);
 
@@ -502,9 +511,18 @@ __device__ __forceinline__ RunningSum exact_running_sum_runs(
             __syncthreads();
             if (scratch.absorbed)
                 return RunningSum{sum, 0u, false};
+            // every wave's total is read at once (independent LDS loads); the composition stays in registers
+            ParityStep totals[kReplayWaves];
+#pragma unroll
+            for (int w = 0; w < kReplayWaves; ++w)
+                totals[w] = scratch.wave_totals[w];
             ParityStep before{0u, 0u};
-            for (int w = 0; w < wave; ++w)
-                before = compose_steps(before, scratch.wave_totals[w]);
+#pragma unroll
+            for (int w = 0; w < kReplayWaves - 1; ++w)
+            {
+                if (w < wave)
+                    before = compose_steps(before, totals[w]);
+            }
             before = compose_steps(before, exclusive);
             uint32_t current = mantissa + ((mantissa & 1u) ? before.odd : before.even);
 
