@@ -197,12 +197,15 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
             uint32_t inclusive = 0;
             if (tid < 256)
             {
+                uint32_t counts[kSortWaves]; // read at once: sixteen dependent LDS round trips otherwise
+#pragma unroll
+                for (int w = 0; w < kSortWaves; ++w)
+                    counts[w] = wave_counts[w][tid];
 #pragma unroll
                 for (int w = 0; w < kSortWaves; ++w)
                 {
-                    const uint32_t c = wave_counts[w][tid];
                     wave_counts[w][tid] = digit_total;
-                    digit_total += c;
+                    digit_total += counts[w];
                 }
                 inclusive = digit_total;
 #pragma unroll
@@ -219,8 +222,9 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
             if (tid < 256)
             {
                 uint32_t start = inclusive - digit_total;
-                for (int w = 0; w < wave; ++w)
-                    start += scan_partial[w];
+#pragma unroll
+                for (int w = 0; w < 3; ++w) // tid < 256: waves 0 to 3
+                    start += w < wave ? scan_partial[w] : 0u;
                 tile_start[tid] = start;
                 global_offset[tid] = digit_base[tid] - start;
                 digit_base[tid] += digit_total;
