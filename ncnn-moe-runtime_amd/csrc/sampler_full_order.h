@@ -520,8 +520,8 @@ __device__ __forceinline__ int32_t recover_token_of_key(
 #pragma unroll
             for (int k = 0; k < kLoads; ++k)
             {
-                if (done)
-                    continue;
+                if (done || __ballot(masks[k] != 0u) == 0)
+                    continue; // most loads hold no match at all: no scan for them
                 const uint32_t count = static_cast<uint32_t>(__popc(masks[k]));
                 uint32_t inclusive = count; // matches in lanes 0..lane of this load
 #pragma unroll
