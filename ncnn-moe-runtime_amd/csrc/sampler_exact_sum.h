@@ -30,7 +30,9 @@ struct ParityStep
 };
 
 constexpr uint32_t kBinadeFull = 1u << 24;
-constexpr int kSequentialHead = 256; // terms a running sum adds one by one before it scans
+constexpr int kSequentialHead = 64; // terms a running sum adds one by one before it scans
+constexpr int kHeadSlots = (kSequentialHead + kWaveSize - 1) / kWaveSize;
+constexpr int kSequentialHeadOfRuns = 16; // ... of a row stored as runs
 constexpr uint32_t kStepCap = 1u << 28; // sums past the binade are only compared against 2^24
 
 __device__ __forceinline__ ParityStep compose_steps(const ParityStep& first, const ParityStep& second)
@@ -240,15 +242,15 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_terms(
     // would cost the scan below a round, and a stop condition usually holds this early.
     const uint32_t head = min(count, static_cast<uint32_t>(kSequentialHead));
     {
-        float head_terms[kSequentialHead / kWaveSize];
+        float head_terms[kHeadSlots];
 #pragma unroll
-        for (int slot = 0; slot < kSequentialHead / kWaveSize; ++slot)
+        for (int slot = 0; slot < kHeadSlots; ++slot)
         {
             const uint32_t i = static_cast<uint32_t>(slot * kWaveSize + lane);
             head_terms[slot] = i < head ? term_at(i) : 0.0f;
         }
 #pragma unroll
-        for (int slot = 0; slot < kSequentialHead / kWaveSize; ++slot)
+        for (int slot = 0; slot < kHeadSlots; ++slot)
         {
             const uint32_t slot_first = static_cast<uint32_t>(slot * kWaveSize);
             const uint32_t slot_count = head > slot_first ? min(head - slot_first, static_cast<uint32_t>(kWaveSize)) : 0u;
@@ -432,7 +434,7 @@ __device__ __forceinline__ RunningSum exact_running_sum_runs(
         const uint32_t head_runs = min(runs, static_cast<uint32_t>(kWaveSize));
         const float head_term = static_cast<uint32_t>(lane) < head_runs ? row_term<PHASE>(row, static_cast<uint32_t>(lane)) : 0.0f;
         const uint32_t head_end = static_cast<uint32_t>(lane) < head_runs ? min(row.run_ends[lane], count) : 0u;
-        const uint32_t head_limit = min(count, static_cast<uint32_t>(kSequentialHead));
+        const uint32_t head_limit = min(count, static_cast<uint32_t>(kSequentialHeadOfRuns));
         for (uint32_t run = 0; run < head_runs && start < head_limit; ++run)
         {
             const float term = read_lane(head_term, static_cast<int>(run));
