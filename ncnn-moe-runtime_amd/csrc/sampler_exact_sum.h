@@ -427,7 +427,7 @@ __device__ __forceinline__ RunningSum exact_running_sum_runs(
     const uint32_t runs = run_of_element(row, count - 1u) + 1u;
     uint32_t start = 0; // elements before this one have been added
 
-    // The first kSequentialHead elements are added one by one, as the CPU does (every thread runs the
+    // The first kSequentialHeadOfRuns elements are added one by one, as the CPU does (every thread runs the
     // same loop on wave-uniform values): the sum climbs through most of its binades here, each of
     // which would cost the scan below a round, and a stop condition usually holds this early.
     {
