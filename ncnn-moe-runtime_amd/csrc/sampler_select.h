@@ -782,7 +782,10 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     // all of a thread's slots belong to one segment (the workgroup's size is a multiple of 16)
     const uint32_t s = static_cast<uint32_t>(tid) & static_cast<uint32_t>(kMaxSegments - 1);
     const bool segment_exists = stageable && s < a.segments;
-    const uint32_t segment_count = segment_exists ? load_record(&a.segment_counts[row_slot + s]) : 0u;
+    // The counts of several rows share a 128-byte line, which this compute unit's vector cache may hold
+    // from the merge of another row, taken before this row's segments stored theirs: always read around it.
+    // (A record is 1 KB, aligned, and read by this workgroup only: a plain load cannot find it stale.)
+    const uint32_t segment_count = segment_exists ? load_agent(&a.segment_counts[row_slot + s]) : 0u;
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j)
     {
