@@ -1,7 +1,8 @@
-// Tests of the C++ host face of the HIP expert router, written in the manner of the runtime's own
-// dispatcher tests (tests/test_runtime.cpp:3366-3540: grouping, weights, storage reuse of
-// dispatch_into, tied scores, wide Top-K, caller-named experts, the sqrt-softplus router with a
-// selection bias), plus the error texts and their order.
+// Tests of the C++ host face of the HIP expert router: a table of known plans (the vectors of the
+// runtime's own dispatcher tests, tests/test_runtime.cpp:3366-3540: grouping, weights, tied scores, wide
+// Top-K, caller-named experts, the sqrt-softplus router with a selection bias) run by one loop that also
+// checks the plan's invariants and dispatch_into against dispatch; the error texts and their order; a
+// large random call.
 //
 //   test_expert_dispatcher            all tests (needs a GPU)
 //   test_expert_dispatcher --host     only the tests that need no GPU
@@ -47,157 +48,169 @@ static void test_defaults_match_the_runtime()
     check(HipExpertDispatcher::create(0, 0, 64, 8) == nullptr);
 }
 
-static void test_groups_routes(HipExpertDispatcher& dispatcher)
+// ---- known plans.  The inputs and the facts checked are those of the runtime's dispatcher tests
+// (tests/test_runtime.cpp:3366-3540), kept here as data: one record per call, the expected plan as the
+// flat list of routes in plan order (expert ascending, then token, then rank).  A weight below zero is
+// not compared; token_weight_sum below zero likewise.
+struct ExpectedRoute
 {
-    ExpertDispatchOptions options;
-    options.expert_count = 6;
-    options.top_k = 1;
-    const std::vector<float> logits = {
-        0.0f, 5.0f, 0.0f, 0.0f, 0.0f, 1.0f,
-        0.0f, 1.0f, 0.0f, 0.0f, 0.0f, 5.0f,
-        0.0f, 4.0f, 0.0f, 0.0f, 0.0f, 1.0f,
-        0.0f, 1.0f, 0.0f, 0.0f, 0.0f, 4.0f,
+    uint32_t expert;
+    uint32_t token;
+    uint32_t rank;
+    double weight;
+};
+
+struct PlanCase
+{
+    const char* name;
+    uint32_t tokens;
+    uint32_t experts;
+    uint32_t top_k;
+    RouterScoreFunction score;
+    RouterNormalization normalization;
+    float scaling;
+    uint32_t flags;
+    std::vector<float> bias;
+    std::vector<uint32_t> named_experts;
+    std::vector<float> logits;
+    std::vector<ExpectedRoute> routes; // empty: only the invariants and dispatch == dispatch_into are checked
+    double token_weight_sum;
+};
+
+static std::vector<float> cyclic_logits(size_t count)
+{
+    std::vector<float> logits(count);
+    for (size_t i = 0; i < count; ++i)
+        logits[i] = static_cast<float>(static_cast<int>(i % 7) - 3);
+    return logits;
+}
+
+static std::vector<PlanCase> known_plans()
+{
+    const auto softmax = RouterScoreFunction::Softmax;
+    const auto selected = RouterNormalization::SelectedExperts;
+    const uint32_t renormalize = ExpertDispatchNormalizeTopKWeights;
+    const double e = std::exp(1.0);
+    const double high = std::sqrt(std::log1p(std::exp(4.0)));  // sqrt(softplus(4))
+    const double low = std::sqrt(std::log1p(std::exp(-4.0)));  // sqrt(softplus(-4))
+    return {
+        {"four tokens, two experts in use (:3366-3391)", 4, 6, 1, softmax, selected, 1.0f, renormalize, {}, {},
+         {0, 5, 0, 0, 0, 1, 0, 1, 0, 0, 0, 5, 0, 4, 0, 0, 0, 1, 0, 1, 0, 0, 0, 4},
+         {{1, 0, 0, 1.0}, {1, 2, 0, 1.0}, {5, 1, 0, 1.0}, {5, 3, 0, 1.0}}, 1.0},
+        {"Top-2 of three, renormalised (:3393-3404)", 1, 3, 2, softmax, selected, 1.0f, renormalize, {}, {},
+         {2, 1, 0}, {{0, 0, 0, e / (1.0 + e)}, {1, 0, 1, 1.0 / (1.0 + e)}}, 1.0},
+        {"the next step's logits (:3425-3435)", 1, 3, 2, softmax, selected, 1.0f, renormalize, {}, {},
+         {0, 1, 2}, {{1, 0, 1, 1.0 / (1.0 + e)}, {2, 0, 0, e / (1.0 + e)}}, 1.0},
+        {"tied sigmoid scores keep the lower ids, no renormalisation, scale 2 (:3437-3446)", 1, 4, 2,
+         RouterScoreFunction::Sigmoid, RouterNormalization::None, 2.0f, 0, {}, {},
+         {0, 0, -1, -1}, {{0, 0, 0, 1.0}, {1, 0, 1, 1.0}}, -1.0},
+        {"Top-16 of twenty (:3448-3456)", 1, 20, 16, softmax, selected, 1.0f, renormalize, {}, {}, cyclic_logits(20), {}, 1.0},
+        {"Top-17 of twenty (:3457-3458)", 1, 20, 17, softmax, selected, 1.0f, renormalize, {}, {}, cyclic_logits(20), {}, 1.0},
+        {"one expert named twice (:3460-3468)", 1, 4, 2, softmax, selected, 1.0f, renormalize, {}, {1, 1},
+         {0, 1, 2, 3}, {{1, 0, 0, 0.5}, {1, 0, 1, 0.5}}, 1.0},
+        {"sqrt-softplus with a selection bias: the bias picks, the unbiased scores weigh (:3499-3518)", 1, 4, 2,
+         RouterScoreFunction::SqrtSoftplus, selected, 1.5f, renormalize, {0, 100, 0, 0}, {},
+         {4, -4, 3, 2}, {{0, 0, 1, high / (low + high) * 1.5}, {1, 0, 0, low / (low + high) * 1.5}}, 1.5},
+        {"sqrt-softplus, experts named by the caller (:3520-3533)", 1, 4, 2,
+         RouterScoreFunction::SqrtSoftplus, selected, 1.5f, renormalize, {}, {3, 2},
+         {4, -4, 3, 2}, {{2, 0, 1, -1.0}, {3, 0, 0, -1.0}}, 1.5},
     };
-    auto dispatch = dispatcher.dispatch(logits, 4, options);
-    check(static_cast<bool>(dispatch));
-    check(dispatch.value().assignment_count == 4);
-    check(dispatch.value().batches.size() == 2);
-    check(dispatch.value().batches[0].expert_id == 1);
-    check(dispatch.value().batches[0].routes.size() == 2);
-    check(dispatch.value().batches[0].routes[0].token_index == 0);
-    check(dispatch.value().batches[0].routes[1].token_index == 2);
-    check_near(dispatch.value().batches[0].routes[0].weight, 1.0f, 1e-6f);
-    check(dispatch.value().batches[1].expert_id == 5);
-    check(dispatch.value().batches[1].routes.size() == 2);
-    check(dispatch.value().batches[1].routes[0].token_index == 1);
-    check(dispatch.value().batches[1].routes[1].token_index == 3);
-
-    options.expert_count = 3;
-    options.top_k = 2;
-    const std::vector<float> weighted_logits = {2.0f, 1.0f, 0.0f};
-    auto weighted = dispatcher.dispatch(weighted_logits, 1, options);
-    check(static_cast<bool>(weighted));
-    check(weighted.value().assignment_count == 2);
-    check(weighted.value().batches.size() == 2);
-    check(weighted.value().batches[0].routes[0].rank == 0);
-    check(weighted.value().batches[1].routes[0].rank == 1);
-    check_near(weighted.value().batches[0].routes[0].weight + weighted.value().batches[1].routes[0].weight, 1.0f, 1e-6f);
-
-    // dispatch_into gives the same plan and keeps the caller's storage across steps
-    ExpertDispatchPlan reusable;
-    auto dispatched_into = dispatcher.dispatch_into(weighted_logits, 1, options, reusable);
-    check(static_cast<bool>(dispatched_into));
-    check(reusable.assignment_count == weighted.value().assignment_count);
-    check(reusable.batches.size() == weighted.value().batches.size());
-    for (size_t index = 0; index < reusable.batches.size(); ++index)
-    {
-        check(reusable.batches[index].expert_id == weighted.value().batches[index].expert_id);
-        check(reusable.batches[index].routes.front().rank == weighted.value().batches[index].routes.front().rank);
-        check(reusable.batches[index].routes.front().weight == weighted.value().batches[index].routes.front().weight);
-    }
-    const ExpertBatch* reused_batches = reusable.batches.data();
-    const ExpertRoute* reused_first_route = reusable.batches.front().routes.data();
-    const std::vector<float> next_logits = {0.0f, 1.0f, 2.0f};
-    dispatched_into = dispatcher.dispatch_into(next_logits, 1, options, reusable);
-    check(static_cast<bool>(dispatched_into));
-    check(reusable.batches.data() == reused_batches);
-    check(reusable.batches.front().routes.data() == reused_first_route);
-    check(reusable.batches[0].expert_id == 1 && reusable.batches[1].expert_id == 2);
-    check(reusable.batches[1].routes[0].rank == 0);
 }
 
-static void check_dispatch_into_matches(HipExpertDispatcher& dispatcher, std::span<const float> logits, const ExpertDispatchOptions& options)
-{
-    auto expected = dispatcher.dispatch(logits, 1, options);
-    check(static_cast<bool>(expected));
-    ExpertDispatchPlan actual;
-    auto status = dispatcher.dispatch_into(logits, 1, options, actual);
-    check(static_cast<bool>(status));
-    check(actual.assignment_count == expected.value().assignment_count);
-    check(actual.batches.size() == expected.value().batches.size());
-    size_t routes = 0;
-    for (size_t b = 0; b < actual.batches.size(); ++b)
-    {
-        check(actual.batches[b].expert_id == expected.value().batches[b].expert_id);
-        check(actual.batches[b].routes.size() == expected.value().batches[b].routes.size());
-        for (size_t r = 0; r < actual.batches[b].routes.size(); ++r)
-        {
-            check(actual.batches[b].routes[r].token_index == expected.value().batches[b].routes[r].token_index);
-            check(actual.batches[b].routes[r].rank == expected.value().batches[b].routes[r].rank);
-            check(actual.batches[b].routes[r].weight == expected.value().batches[b].routes[r].weight);
-        }
-        routes += actual.batches[b].routes.size();
-    }
-    check(routes == options.top_k);
-}
-
-static void test_ties_wide_windows_and_named_experts(HipExpertDispatcher& dispatcher)
-{
-    ExpertDispatchOptions sigmoid_options;
-    sigmoid_options.expert_count = 4;
-    sigmoid_options.top_k = 2;
-    sigmoid_options.score_function = RouterScoreFunction::Sigmoid;
-    sigmoid_options.normalization = RouterNormalization::None;
-    sigmoid_options.routed_scaling_factor = 2.0f;
-    sigmoid_options.flags = 0;
-    const std::array<float, 4> tied_sigmoid_logits = {0.0f, 0.0f, -1.0f, -1.0f};
-    check_dispatch_into_matches(dispatcher, tied_sigmoid_logits, sigmoid_options);
-    auto tied = dispatcher.dispatch(tied_sigmoid_logits, 1, sigmoid_options);
-    check(tied.value().batches[0].expert_id == 0 && tied.value().batches[1].expert_id == 1); // the lower ids of the tie
-    check(tied.value().batches[0].routes[0].weight == 1.0f);                                  // sigmoid(0) * 2, not renormalised
-
-    ExpertDispatchOptions wide_options;
-    wide_options.expert_count = 20;
-    std::array<float, 20> wide_logits;
-    for (size_t index = 0; index < wide_logits.size(); ++index)
-        wide_logits[index] = static_cast<float>(static_cast<int>(index % 7) - 3);
-    wide_options.top_k = 16;
-    check_dispatch_into_matches(dispatcher, wide_logits, wide_options);
-    wide_options.top_k = 17;
-    check_dispatch_into_matches(dispatcher, wide_logits, wide_options);
-
-    ExpertDispatchOptions duplicate_options;
-    duplicate_options.expert_count = 4;
-    duplicate_options.top_k = 2;
-    const std::array<uint32_t, 2> duplicate_experts = {1, 1};
-    duplicate_options.explicit_expert_ids = duplicate_experts;
-    const std::array<float, 4> duplicate_logits = {0.0f, 1.0f, 2.0f, 3.0f};
-    check_dispatch_into_matches(dispatcher, duplicate_logits, duplicate_options);
-    auto duplicated = dispatcher.dispatch(duplicate_logits, 1, duplicate_options);
-    check(duplicated.value().batches.size() == 1 && duplicated.value().batches[0].routes.size() == 2);
-    check(duplicated.value().batches[0].routes[0].rank == 0 && duplicated.value().batches[0].routes[1].rank == 1);
-}
-
-static void test_sqrt_softplus_router(HipExpertDispatcher& dispatcher)
+static ExpertDispatchOptions options_of(const PlanCase& c)
 {
     ExpertDispatchOptions options;
-    options.expert_count = 4;
-    options.top_k = 2;
-    options.score_function = RouterScoreFunction::SqrtSoftplus;
-    options.routed_scaling_factor = 1.5f;
-    const std::array<float, 4> selection_bias = {0.0f, 100.0f, 0.0f, 0.0f};
-    options.selection_bias = selection_bias;
-    const std::array<float, 4> logits = {4.0f, -4.0f, 3.0f, 2.0f};
-    auto routed = dispatcher.dispatch(logits, 1, options);
-    check(static_cast<bool>(routed));
-    check(routed.value().batches.size() == 2);
-    check(routed.value().batches[0].expert_id == 0);
-    check(routed.value().batches[1].expert_id == 1);
-    check_near(routed.value().batches[0].routes[0].weight + routed.value().batches[1].routes[0].weight, 1.5f, 1e-5f);
-    // the weights come from the unbiased scores: sqrt(softplus(4)) and sqrt(softplus(-4))
-    const float high = std::sqrt(std::log1p(std::exp(4.0f)));
-    const float low = std::sqrt(std::log1p(std::exp(-4.0f)));
-    check(routed.value().batches[0].routes[0].weight == high / (low + high) * 1.5f); // rank order: expert 1 (biased) first
-    check(routed.value().batches[1].routes[0].rank == 0 && routed.value().batches[0].routes[0].rank == 1);
+    options.expert_count = c.experts;
+    options.top_k = c.top_k;
+    options.score_function = c.score;
+    options.normalization = c.normalization;
+    options.routed_scaling_factor = c.scaling;
+    options.flags = c.flags;
+    options.selection_bias = c.bias;
+    options.explicit_expert_ids = c.named_experts;
+    return options;
+}
 
-    const std::array<uint32_t, 2> explicit_experts = {3, 2};
-    options.selection_bias = {};
-    options.explicit_expert_ids = explicit_experts;
-    routed = dispatcher.dispatch(logits, 1, options);
-    check(static_cast<bool>(routed));
-    check(routed.value().batches[0].expert_id == 2);
-    check(routed.value().batches[1].expert_id == 3);
-    check(routed.value().batches[0].routes[0].rank == 1 && routed.value().batches[1].routes[0].rank == 0);
+static std::vector<ExpectedRoute> flatten(const ExpertDispatchPlan& plan)
+{
+    std::vector<ExpectedRoute> flat;
+    for (const ExpertBatch& batch : plan.batches)
+    {
+        check(!batch.routes.empty());
+        for (const ExpertRoute& route : batch.routes)
+            flat.push_back({batch.expert_id, route.token_index, route.rank, static_cast<double>(route.weight)});
+    }
+    return flat;
+}
+
+static void test_known_plans(HipExpertDispatcher& dispatcher)
+{
+    ExpertDispatchPlan reused; // one plan object through every case: dispatch_into keeps the caller's storage
+    for (const PlanCase& c : known_plans())
+    {
+        try
+        {
+            const ExpertDispatchOptions options = options_of(c);
+            auto result = dispatcher.dispatch(c.logits, c.tokens, options);
+            check(static_cast<bool>(result));
+            const ExpertDispatchPlan& plan = result.value();
+            const std::vector<ExpectedRoute> flat = flatten(plan);
+            check(plan.assignment_count == static_cast<size_t>(c.tokens) * c.top_k);
+            check(flat.size() == plan.assignment_count);
+            std::vector<double> sums(c.tokens, 0.0);
+            for (size_t i = 0; i < flat.size(); ++i)
+            {
+                check(flat[i].expert < c.experts && flat[i].token < c.tokens && flat[i].rank < c.top_k);
+                if (i > 0) // plan order
+                    check(flat[i - 1].expert < flat[i].expert ||
+                          (flat[i - 1].expert == flat[i].expert &&
+                           (flat[i - 1].token < flat[i].token || (flat[i - 1].token == flat[i].token && flat[i - 1].rank < flat[i].rank))));
+                sums[flat[i].token] += flat[i].weight;
+            }
+            if (c.token_weight_sum >= 0.0)
+            {
+                for (double sum : sums)
+                    check_near(static_cast<float>(sum), static_cast<float>(c.token_weight_sum), 1e-5f);
+            }
+            if (!c.routes.empty())
+            {
+                check(flat.size() == c.routes.size());
+                for (size_t i = 0; i < flat.size(); ++i)
+                {
+                    check(flat[i].expert == c.routes[i].expert && flat[i].token == c.routes[i].token && flat[i].rank == c.routes[i].rank);
+                    if (c.routes[i].weight >= 0.0)
+                        check_near(static_cast<float>(flat[i].weight), static_cast<float>(c.routes[i].weight), 1e-6f);
+                }
+            }
+            // dispatch_into: the same plan, bit for bit, in storage that it does not reallocate when it fits
+            const ExpertBatch* batches_before = reused.batches.data();
+            const size_t capacity_before = reused.batches.capacity();
+            auto status = dispatcher.dispatch_into(c.logits, c.tokens, options, reused);
+            check(static_cast<bool>(status));
+            if (plan.batches.size() <= capacity_before)
+                check(reused.batches.data() == batches_before);
+            const std::vector<ExpectedRoute> again = flatten(reused);
+            check(reused.assignment_count == plan.assignment_count && again.size() == flat.size());
+            for (size_t i = 0; i < flat.size(); ++i)
+            {
+                check(again[i].expert == flat[i].expert && again[i].token == flat[i].token && again[i].rank == flat[i].rank);
+                const float a = static_cast<float>(again[i].weight), b = static_cast<float>(flat[i].weight);
+                check(std::memcmp(&a, &b, sizeof(a)) == 0);
+            }
+        }
+        catch (const std::exception& error)
+        {
+            throw std::runtime_error(std::string("known plan \"") + c.name + "\": " + error.what());
+        }
+    }
+    // a route's storage is kept as well: the same call twice leaves every vector where it was
+    const PlanCase c = known_plans()[1];
+    const ExpertDispatchOptions options = options_of(c);
+    check(static_cast<bool>(dispatcher.dispatch_into(c.logits, c.tokens, options, reused)));
+    const ExpertBatch* batches = reused.batches.data();
+    const ExpertRoute* first_routes = reused.batches.front().routes.data();
+    check(static_cast<bool>(dispatcher.dispatch_into(c.logits, c.tokens, options, reused)));
+    check(reused.batches.data() == batches && reused.batches.front().routes.data() == first_routes);
 }
 
 static void test_errors(HipExpertDispatcher& dispatcher)
@@ -329,9 +342,7 @@ int main(int argc, char** argv)
             std::fprintf(stderr, "HipExpertDispatcher::create failed: no usable GPU\n");
             return 2;
         }
-        test_groups_routes(*dispatcher);
-        test_ties_wide_windows_and_named_experts(*dispatcher);
-        test_sqrt_softplus_router(*dispatcher);
+        test_known_plans(*dispatcher);
         test_errors(*dispatcher);
         test_many_tokens(*dispatcher);
     }
