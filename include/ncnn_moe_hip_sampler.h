@@ -146,6 +146,26 @@ int ncnn_moe_hip_sampler_sample_device(
     const int32_t* device_stop_ids,
     ncnn_moe_sample_result* device_results, int may_need_full_order, void* stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  The select pass of
+ * ncnn_moe_hip_sampler_sample_device (may_need_full_order = 0) without a handle: the call allocates
+ * nothing, on the device or through any library; its scratch (the segments' candidate records and the
+ * per-row hand-over words, 8.4 MB) is a static device array that every GPU the library runs on holds
+ * from its first call until the process ends.  Greedy rows and rows with 1 <= top_k <= 64 are final;
+ * any other row comes back NCNN_MOE_ROW_NEEDS_FULL_ORDER.  Limits: rows <= NCNN_MOE_STATIC_MAX_ROWS,
+ * any vocab; a larger batch is rejected with NCNN_MOE_SAMPLER_INVALID_ARGUMENT and the reason is
+ * ncnn_moe_hip_sampler_last_error(NULL) on the calling thread.  `device` is made current.  All calls on
+ * one GPU share the one array: calls that overlap on a GPU (two streams, two threads) race; calls in
+ * one stream, or otherwise ordered, do not.  The first call on a device looks the array up and
+ * clears it on `stream`: make that call outside stream capture. */
+#define NCNN_MOE_STATIC_MAX_ROWS 1024
+int ncnn_moe_hip_sampler_sample_device_static(
+    int device,
+    const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
+    const ncnn_moe_sample_params* device_params, const float* device_uniforms,
+    const int32_t* device_stop_ids,
+    ncnn_moe_sample_result* device_results, void* stream);
+
 /* sampling_distribution (src/engine/session.cpp:76-136) for one row of the handle's logits buffer:
  * the filtered, renormalised (token id, probability) list in the CPU order.  Writes min(*count, cap)
  * entries.  Used by parity tests and by speculative verification (src/engine/session.cpp:799-804).
@@ -202,7 +222,8 @@ int ncnn_moe_hip_sampler_speculative_verify(
 /* The fixed message of a verification status (src/engine/session.cpp:174, :201, :829). */
 const char* ncnn_moe_hip_sampler_verify_status_message(int verify_status);
 
-/* Error text of the last failed call on this handle (Error::message, include/ncnn/moe/result.h:21-25). */
+/* Error text of the last failed call on this handle (Error::message, include/ncnn/moe/result.h:21-25);
+ * with a null handle, of the calling thread's last failed ncnn_moe_hip_sampler_sample_device_static. */
 const char* ncnn_moe_hip_sampler_last_error(const ncnn_moe_hip_sampler* sampler);
 
 /* The CPU sampler's fixed message for a row status (src/engine/session.cpp:68,70,72,85,103,399). */

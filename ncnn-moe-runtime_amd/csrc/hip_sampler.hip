@@ -10,6 +10,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -183,6 +184,29 @@ SelectGeometry select_geometry(int dtype, uint64_t span, uint32_t rows, bool wid
     return g;
 }
 
+// Device memory that the select kernels use beyond their operands: the segments' candidate records
+// and per-row hand-over words.  A handle allocates them in create(); the entry that allocates nothing
+// points them into its static array.
+struct SelectScratch
+{
+    float* segment_values;
+    int32_t* segment_indices;
+    uint32_t* segment_counts;
+    unsigned long long* row_counter;
+    uint32_t* row_flags;
+    uint32_t* row_state;
+};
+
+void use_select_scratch(SamplerArgs& a, const SelectScratch& scratch)
+{
+    a.segment_values = scratch.segment_values;
+    a.segment_indices = scratch.segment_indices;
+    a.segment_counts = scratch.segment_counts;
+    a.row_counter = scratch.row_counter;
+    a.row_flags = scratch.row_flags;
+    a.row_state = scratch.row_state;
+}
+
 template <int DTYPE>
 void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, SamplerArgs a, bool only_pending, bool scatter_segments)
 {
@@ -246,12 +270,7 @@ int launch_sampler(
     a.uniforms = uniforms;
     a.stop_ids = stop_ids;
     a.results = results;
-    a.segment_values = s->segment_values;
-    a.segment_indices = s->segment_indices;
-    a.segment_counts = s->segment_counts;
-    a.row_counter = s->row_counter;
-    a.row_flags = s->row_flags;
-    a.row_state = s->row_state;
+    use_select_scratch(a, SelectScratch{s->segment_values, s->segment_indices, s->segment_counts, s->row_counter, s->row_flags, s->row_state});
     a.sort_keys[0] = s->sort_keys[0];
     a.sort_keys[1] = s->sort_keys[1];
     a.sort_indices[0] = s->sort_indices[0];
@@ -351,6 +370,51 @@ int check_shape(ncnn_moe_hip_sampler* s, int dtype, uint32_t rows, uint32_t voca
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 
+// ---- ncnn_moe_hip_sampler_sample_device_static: the select pass with no handle and no allocation.
+// Its scratch is this file-scope device array; every GPU the library runs on holds its own copy, at its
+// own address, until the process ends.  The name `scratch` is only a host-side stand-in for it: host code
+// takes the device address once per device with hipGetSymbolAddress and uses that pointer everywhere.
+constexpr uint32_t kStaticMaxRows = NCNN_MOE_STATIC_MAX_ROWS;
+constexpr uint32_t kStaticSplitRows = kWholeRowBatch - 1; // larger batches stream whole rows and keep no records
+constexpr int kStaticMaxDevices = 64;
+
+struct StaticScratchLayout
+{
+    float segment_values[static_cast<size_t>(kStaticSplitRows) * kMaxSegments * kSegmentRecordSlots];
+    int32_t segment_indices[static_cast<size_t>(kStaticSplitRows) * kMaxSegments * kSegmentRecordSlots];
+    uint32_t segment_counts[static_cast<size_t>(kStaticSplitRows) * kMaxSegments];
+    unsigned long long row_counter[kStaticMaxRows];
+    uint32_t row_flags[kStaticMaxRows];
+    uint32_t row_state[kStaticMaxRows];
+};
+static_assert(kStaticMaxRows >= kStaticSplitRows, "a split batch must fit the per-row words");
+
+static __device__ __align__(256) unsigned char scratch[sizeof(StaticScratchLayout)];
+
+std::mutex g_static_mutex;
+StaticScratchLayout* g_static_scratch[kStaticMaxDevices] = {}; // device address of `scratch`, per device
+thread_local char g_static_error[256] = "";
+
+int static_fail(int rc, const char* message, const char* detail = "")
+{
+    std::snprintf(g_static_error, sizeof(g_static_error), "%s%s%s", message, detail[0] != 0 ? ": " : "", detail);
+    return rc;
+}
+
+// The words that a launch expects to find at zero (the kernels return them to zero themselves).
+__global__ void static_scratch_clear_kernel(StaticScratchLayout* layout)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < kStaticMaxRows)
+    {
+        layout->row_counter[i] = 0ull;
+        layout->row_flags[i] = 0u;
+        layout->row_state[i] = 0u;
+    }
+    if (i < kStaticSplitRows * kMaxSegments)
+        layout->segment_counts[i] = 0u;
+}
+
 } // namespace
 
 extern "C" {
@@ -427,6 +491,7 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->row_counter, rows * sizeof(unsigned long long)));
     CREATE_CHECK(hipMalloc(&s->row_flags, rows * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->row_state, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMemset(s->segment_counts, 0, slots * sizeof(uint32_t)));
     CREATE_CHECK(hipMemset(s->row_counter, 0, rows * sizeof(unsigned long long)));
     CREATE_CHECK(hipMemset(s->row_flags, 0, rows * sizeof(uint32_t)));
     CREATE_CHECK(hipMemset(s->row_state, 0, rows * sizeof(uint32_t)));
@@ -664,6 +729,76 @@ int ncnn_moe_hip_sampler_sample_device(
         device_results, DistributionExport{}, passes, static_cast<hipStream_t>(stream));
 }
 
+int ncnn_moe_hip_sampler_sample_device_static(
+    int device,
+    const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride,
+    const ncnn_moe_sample_params* device_params, const float* device_uniforms,
+    const int32_t* device_stop_ids,
+    ncnn_moe_sample_result* device_results, void* stream)
+{
+    g_static_error[0] = 0;
+    if (device_logits == nullptr || device_params == nullptr || device_uniforms == nullptr || device_results == nullptr)
+        return static_fail(NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "a device pointer is null");
+    if (dtype != NCNN_MOE_LOGITS_F32 && dtype != NCNN_MOE_LOGITS_BF16)
+        return static_fail(NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "unknown logits dtype");
+    if (rows == 0 || rows > kStaticMaxRows)
+        return static_fail(NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "rows must be in [1, NCNN_MOE_STATIC_MAX_ROWS]");
+    if (vocab == 0)
+        return static_fail(NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab must be positive");
+    if (row_stride < vocab)
+        return static_fail(NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "row_stride is smaller than vocab");
+    if (device < 0 || device >= kStaticMaxDevices)
+        return static_fail(NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "device index out of range");
+    hipError_t error = hipSetDevice(device);
+    if (error != hipSuccess)
+        return static_fail(NCNN_MOE_SAMPLER_HIP_ERROR, "hipSetDevice", hipGetErrorString(error));
+    const hipStream_t on = static_cast<hipStream_t>(stream);
+    StaticScratchLayout* layout = nullptr;
+    {
+        // Set-up, once per device, with that device current: this GPU's address of the array.
+        std::lock_guard<std::mutex> lock(g_static_mutex);
+        if (g_static_scratch[device] == nullptr)
+        {
+            void* address = nullptr;
+            error = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+            if (error != hipSuccess || address == nullptr)
+                return static_fail(NCNN_MOE_SAMPLER_HIP_ERROR, "hipGetSymbolAddress(scratch)", hipGetErrorString(error));
+            constexpr uint32_t kClearThreads = 256;
+            constexpr uint32_t kClearWords = kStaticSplitRows * kMaxSegments > kStaticMaxRows ? kStaticSplitRows * kMaxSegments : kStaticMaxRows;
+            hipLaunchKernelGGL(static_scratch_clear_kernel, dim3((kClearWords + kClearThreads - 1) / kClearThreads), dim3(kClearThreads), 0, on,
+                               static_cast<StaticScratchLayout*>(address));
+            error = hipGetLastError();
+            if (error != hipSuccess)
+                return static_fail(NCNN_MOE_SAMPLER_HIP_ERROR, "clearing the static scratch", hipGetErrorString(error));
+            g_static_scratch[device] = static_cast<StaticScratchLayout*>(address);
+        }
+        layout = g_static_scratch[device];
+    }
+    SamplerArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.logits = device_logits;
+    a.row_stride = row_stride;
+    a.rows = rows;
+    a.vocab = vocab;
+    a.params = device_params;
+    a.uniforms = device_uniforms;
+    a.stop_ids = device_stop_ids;
+    a.results = device_results;
+    use_select_scratch(a, SelectScratch{layout->segment_values, layout->segment_indices, layout->segment_counts,
+                                        layout->row_counter, layout->row_flags, layout->row_state});
+    const SelectGeometry geometry = select_geometry(dtype, logits_span(vocab, dtype, device_logits, row_stride), rows, false);
+    if (geometry.segments > 1 && rows > kStaticSplitRows)
+        return static_fail(NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "the batch shape needs more segment records than the static scratch holds");
+    if (dtype == NCNN_MOE_LOGITS_F32)
+        launch_select<NCNN_MOE_LOGITS_F32>(geometry, rows, on, a, false, false);
+    else
+        launch_select<NCNN_MOE_LOGITS_BF16>(geometry, rows, on, a, false, false);
+    error = hipGetLastError();
+    if (error != hipSuccess)
+        return static_fail(NCNN_MOE_SAMPLER_HIP_ERROR, "select kernel launch", hipGetErrorString(error));
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
 int ncnn_moe_hip_sampler_distribution(
     ncnn_moe_hip_sampler* s, uint32_t row, const ncnn_moe_sample_params* params,
     uint32_t cap, int32_t* ids, float* probabilities, uint32_t* count, uint32_t* status)
@@ -854,7 +989,7 @@ const char* ncnn_moe_hip_sampler_verify_status_message(int verify_status)
 
 const char* ncnn_moe_hip_sampler_last_error(const ncnn_moe_hip_sampler* s)
 {
-    return s == nullptr ? "" : s->last_error.c_str();
+    return s == nullptr ? g_static_error : s->last_error.c_str();
 }
 
 const char* ncnn_moe_hip_sampler_status_message(int row_status)

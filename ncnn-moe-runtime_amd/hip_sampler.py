@@ -56,6 +56,7 @@ EXPORTED_SYMBOLS = [
     "ncnn_moe_hip_sampler_upload_logits",
     "ncnn_moe_hip_sampler_sample",
     "ncnn_moe_hip_sampler_sample_device",
+    "ncnn_moe_hip_sampler_sample_device_static",
     "ncnn_moe_hip_sampler_distribution",
     "ncnn_moe_hip_sampler_speculative_verify",
     "ncnn_moe_hip_sampler_verify_status_message",
@@ -95,6 +96,8 @@ def load_library():
     lib.ncnn_moe_hip_sampler_sample.argtypes = [vp, ctypes.c_uint32, vp, vp, vp, ctypes.c_uint32, vp]
     lib.ncnn_moe_hip_sampler_sample_device.argtypes = [
         vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp, vp, vp, vp, ctypes.c_int, vp]
+    lib.ncnn_moe_hip_sampler_sample_device_static.argtypes = [
+        ctypes.c_int, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp, vp, vp, vp, vp]
     lib.ncnn_moe_hip_sampler_distribution.argtypes = [
         vp, ctypes.c_uint32, vp, ctypes.c_uint32, vp, vp, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32)]
     lib.ncnn_moe_hip_sampler_speculative_verify.argtypes = [vp, ctypes.c_uint32, vp, vp, vp, vp, vp]
@@ -252,6 +255,21 @@ class HipSampler:
         out = np.empty_like(values)
         self._check(self._lib.ncnn_moe_hip_sampler_debug_expf(self._handle, values.ctypes.data, out.ctypes.data, values.size))
         return out
+
+
+STATIC_MAX_ROWS = 1024
+
+
+def sample_device_static(device, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr,
+                         stop_ids_ptr, results_ptr, stream=None):
+    """The select pass without a handle and without any allocation (static device scratch); all pointers
+    are device addresses.  Returns the call's return code; last_static_error() has the reason."""
+    return load_library().ncnn_moe_hip_sampler_sample_device_static(
+        device, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr, stop_ids_ptr, results_ptr, stream)
+
+
+def last_static_error():
+    return load_library().ncnn_moe_hip_sampler_last_error(None).decode()
 
 
 def device_count():
