@@ -232,15 +232,6 @@ const char* ncnn_moe_hip_sampler_status_message(int row_status);
 /* Number of HIP devices visible, 0 if none (no counterpart: the CPU sampler needs no device). */
 int ncnn_moe_hip_sampler_device_count(void);
 
-/* Test hooks (no counterpart in the runtime).  force_general routes every non-greedy row through
- * the full-order path; scatter_segments launches split rows without the XCD-aware numbering of the
- * workgroups, so that the segments of a row run on several XCDs and the merge takes its records
- * around the L2; expf evaluates the device exponential on n host values. */
-int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* sampler, int enabled);
-int ncnn_moe_hip_sampler_debug_scatter_segments(ncnn_moe_hip_sampler* sampler, int enabled);
-int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* sampler, const float* in, float* out, size_t n);
-void ncnn_moe_hip_sampler_debug_exp2_table(uint64_t out[32]);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,35 @@
+/*
+ * Test hooks of the MI355X generation sampler library: exported by the same shared library, used by this
+ * repository's tests only, and not part of the boundary that the runtime binds (no counterpart in the
+ * runtime).
+ */
+#ifndef NCNN_MOE_HIP_SAMPLER_TESTING_H
+#define NCNN_MOE_HIP_SAMPLER_TESTING_H
+
+#include "ncnn_moe_hip_sampler.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* force_general routes every non-greedy row through the full-order path; scatter_segments launches
+ * split rows without the XCD-aware numbering of the workgroups, so that the segments of a row run on
+ * several XCDs and the merge finds their records outside its L2; expf evaluates the device exponential
+ * on n host values. */
+int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* sampler, int enabled);
+int ncnn_moe_hip_sampler_debug_scatter_segments(ncnn_moe_hip_sampler* sampler, int enabled);
+int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* sampler, const float* in, float* out, size_t n);
+void ncnn_moe_hip_sampler_debug_exp2_table(uint64_t out[32]);
+
+/* How the first select kernel covers a batch of this shape (rows aligned to 16 bytes): workgroups per
+ * row, chunks each of them streams, and the kernel variant (0: one workgroup streams and finishes a whole
+ * row; 1: a row is split into one-chunk workgroups; 2: into workgroups that stream several chunks).  No
+ * GPU needed. */
+int ncnn_moe_hip_sampler_debug_select_geometry(
+    int dtype, uint32_t rows, uint32_t vocab, uint32_t* segments, uint32_t* chunks_per_segment, uint32_t* variant);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NCNN_MOE_HIP_SAMPLER_TESTING_H */

@@ -1,5 +1,6 @@
 // C ABI of the gfx950 generation sampler: handle, device buffers and kernel launches.
 #include "ncnn_moe_hip_sampler.h"
+#include "ncnn_moe_hip_sampler_testing.h"
 
 #include "sampler_kernels.h"
 #include "sampler_verify.h"
@@ -59,6 +60,8 @@ struct ncnn_moe_hip_sampler
     unsigned long long* row_counter = nullptr;
     uint32_t* row_flags = nullptr;
     uint32_t* row_state = nullptr;
+    unsigned long long* split_records = nullptr;
+    uint32_t* row_epoch = nullptr;
 
     uint32_t* sort_keys[2] = {nullptr, nullptr};
     uint32_t* sort_indices[2] = {nullptr, nullptr};
@@ -195,6 +198,8 @@ struct SelectScratch
     unsigned long long* row_counter;
     uint32_t* row_flags;
     uint32_t* row_state;
+    unsigned long long* split_records;
+    uint32_t* row_epoch;
 };
 
 void use_select_scratch(SamplerArgs& a, const SelectScratch& scratch)
@@ -205,6 +210,8 @@ void use_select_scratch(SamplerArgs& a, const SelectScratch& scratch)
     a.row_counter = scratch.row_counter;
     a.row_flags = scratch.row_flags;
     a.row_state = scratch.row_state;
+    a.split_records = scratch.split_records;
+    a.row_epoch = scratch.row_epoch;
 }
 
 template <int DTYPE>
@@ -227,6 +234,8 @@ void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, S
         hipLaunchKernelGGL((scan_select_kernel<DTYPE, true, true>), grid, dim3(kScanThreads), 0, stream, a);
     else if (g.looped)
         hipLaunchKernelGGL((scan_select_kernel<DTYPE, true, false>), grid, dim3(kScanThreads), 0, stream, a);
+    else if (g.segments > 1)
+        hipLaunchKernelGGL((split_select_kernel<DTYPE>), grid, dim3(kScanThreads), 0, stream, a);
     else
         hipLaunchKernelGGL((scan_select_kernel<DTYPE, false, false>), grid, dim3(kScanThreads), 0, stream, a);
 }
@@ -270,7 +279,8 @@ int launch_sampler(
     a.uniforms = uniforms;
     a.stop_ids = stop_ids;
     a.results = results;
-    use_select_scratch(a, SelectScratch{s->segment_values, s->segment_indices, s->segment_counts, s->row_counter, s->row_flags, s->row_state});
+    use_select_scratch(a, SelectScratch{s->segment_values, s->segment_indices, s->segment_counts, s->row_counter, s->row_flags, s->row_state,
+                                        s->split_records, s->row_epoch});
     a.sort_keys[0] = s->sort_keys[0];
     a.sort_keys[1] = s->sort_keys[1];
     a.sort_indices[0] = s->sort_indices[0];
@@ -386,6 +396,8 @@ struct StaticScratchLayout
     unsigned long long row_counter[kStaticMaxRows];
     uint32_t row_flags[kStaticMaxRows];
     uint32_t row_state[kStaticMaxRows];
+    unsigned long long split_records[static_cast<size_t>(kStaticSplitRows) * kMaxSegments * kSplitRecordSlots];
+    uint32_t row_epoch[kStaticMaxRows];
 };
 static_assert(kStaticMaxRows >= kStaticSplitRows, "a split batch must fit the per-row words");
 
@@ -410,9 +422,14 @@ __global__ void static_scratch_clear_kernel(StaticScratchLayout* layout)
         layout->row_counter[i] = 0ull;
         layout->row_flags[i] = 0u;
         layout->row_state[i] = 0u;
+        layout->row_epoch[i] = 1u;
     }
     if (i < kStaticSplitRows * kMaxSegments)
+    {
         layout->segment_counts[i] = 0u;
+        for (uint32_t entry = 0; entry < static_cast<uint32_t>(kSplitRecordSlots); ++entry)
+            layout->split_records[static_cast<size_t>(i) * kSplitRecordSlots + entry] = 0ull; // epoch 0 tags nothing
+    }
 }
 
 } // namespace
@@ -491,6 +508,12 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->row_counter, rows * sizeof(unsigned long long)));
     CREATE_CHECK(hipMalloc(&s->row_flags, rows * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->row_state, rows * sizeof(uint32_t)));
+    // split path: records start untagged (epoch 0 tags nothing), every row at epoch 1
+    const size_t split_rows = std::min<size_t>(rows, static_cast<size_t>(kWholeRowBatch) - 1);
+    CREATE_CHECK(hipMalloc(&s->split_records, split_rows * kMaxSegments * kSplitRecordSlots * sizeof(unsigned long long)));
+    CREATE_CHECK(hipMemset(s->split_records, 0, split_rows * kMaxSegments * kSplitRecordSlots * sizeof(unsigned long long)));
+    CREATE_CHECK(hipMalloc(&s->row_epoch, rows * sizeof(uint32_t)));
+    CREATE_CHECK(hipMemsetD32(reinterpret_cast<hipDeviceptr_t>(s->row_epoch), 1, rows));
     CREATE_CHECK(hipMemset(s->segment_counts, 0, slots * sizeof(uint32_t)));
     CREATE_CHECK(hipMemset(s->row_counter, 0, rows * sizeof(unsigned long long)));
     CREATE_CHECK(hipMemset(s->row_flags, 0, rows * sizeof(uint32_t)));
@@ -541,7 +564,7 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
         (void)hipEventDestroy(s->side_join);
     void* buffers[] = {
         s->logits, s->params, s->uniforms, s->results, s->stop_ids, s->segment_values, s->segment_indices,
-        s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->sort_keys[0], s->sort_keys[1],
+        s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->split_records, s->row_epoch, s->sort_keys[0], s->sort_keys[1],
         s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
         s->verify_probabilities, s->verify_counts, s->verify_long_ids, s->verify_long_probabilities, s->verify_dense};
@@ -764,7 +787,7 @@ int ncnn_moe_hip_sampler_sample_device_static(
             if (error != hipSuccess || address == nullptr)
                 return static_fail(NCNN_MOE_SAMPLER_HIP_ERROR, "hipGetSymbolAddress(scratch)", hipGetErrorString(error));
             constexpr uint32_t kClearThreads = 256;
-            constexpr uint32_t kClearWords = kStaticSplitRows * kMaxSegments > kStaticMaxRows ? kStaticSplitRows * kMaxSegments : kStaticMaxRows;
+            constexpr uint32_t kClearWords = std::max<uint32_t>(kStaticSplitRows * kMaxSegments, kStaticMaxRows);
             hipLaunchKernelGGL(static_scratch_clear_kernel, dim3((kClearWords + kClearThreads - 1) / kClearThreads), dim3(kClearThreads), 0, on,
                                static_cast<StaticScratchLayout*>(address));
             error = hipGetLastError();
@@ -785,7 +808,8 @@ int ncnn_moe_hip_sampler_sample_device_static(
     a.stop_ids = device_stop_ids;
     a.results = device_results;
     use_select_scratch(a, SelectScratch{layout->segment_values, layout->segment_indices, layout->segment_counts,
-                                        layout->row_counter, layout->row_flags, layout->row_state});
+                                        layout->row_counter, layout->row_flags, layout->row_state,
+                                        layout->split_records, layout->row_epoch});
     const SelectGeometry geometry = select_geometry(dtype, logits_span(vocab, dtype, device_logits, row_stride), rows, false);
     if (geometry.segments > 1 && rows > kStaticSplitRows)
         return static_fail(NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "the batch shape needs more segment records than the static scratch holds");
@@ -1023,6 +1047,19 @@ int ncnn_moe_hip_sampler_debug_scatter_segments(ncnn_moe_hip_sampler* s, int ena
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 
+int ncnn_moe_hip_sampler_debug_select_geometry(
+    int dtype, uint32_t rows, uint32_t vocab, uint32_t* segments, uint32_t* chunks_per_segment, uint32_t* variant)
+{
+    if (segments == nullptr || chunks_per_segment == nullptr || variant == nullptr || rows == 0 || vocab == 0 ||
+        (dtype != NCNN_MOE_LOGITS_F32 && dtype != NCNN_MOE_LOGITS_BF16))
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    const SelectGeometry g = select_geometry(dtype, vocab, rows, false);
+    *segments = g.segments;
+    *chunks_per_segment = g.chunks_per_segment;
+    *variant = g.segments == 1 ? 0u : (g.looped ? 2u : 1u);
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
 int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* s, const float* in, float* out, size_t n)
 {
     if (s == nullptr || in == nullptr || out == nullptr)
@@ -1053,6 +1090,23 @@ int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* s, const float* in, fl
         return hip_fail(s, error, "debug_expf");
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
+
+#ifdef NCNN_MOE_TIMELINE
+// Only in the library built with -DNCNN_MOE_TIMELINE: the wall-clock stamps (100 MHz ticks) that the split
+// kernel's workgroups left, [64 rows][16 segments][16 slots].
+int ncnn_moe_hip_sampler_debug_timeline(unsigned long long* out, size_t count)
+{
+    const size_t bytes = std::min(count * sizeof(unsigned long long), sizeof(unsigned long long) * kTimelineRows * kMaxSegments * kTimelineSlots);
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(ncnn_moe_hip::g_timeline), bytes) == hipSuccess ? NCNN_MOE_SAMPLER_SUCCESS : NCNN_MOE_SAMPLER_HIP_ERROR;
+}
+
+// ... and the stamps of the rows' last waves inside the epilogue, [64 rows][16 slots].
+int ncnn_moe_hip_sampler_debug_timeline_rows(unsigned long long* out, size_t count)
+{
+    const size_t bytes = std::min(count * sizeof(unsigned long long), sizeof(unsigned long long) * kTimelineRows * kTimelineSlots);
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(ncnn_moe_hip::g_timeline_rows), bytes) == hipSuccess ? NCNN_MOE_SAMPLER_SUCCESS : NCNN_MOE_SAMPLER_HIP_ERROR;
+}
+#endif
 
 void ncnn_moe_hip_sampler_debug_exp2_table(uint64_t out[32])
 {

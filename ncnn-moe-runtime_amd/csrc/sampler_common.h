@@ -35,6 +35,10 @@ struct SamplerArgs
     uint32_t xcd_grouped;      // the grid is one-dimensional and puts the segments of a row on one XCD
     uint32_t* row_flags;       // [rows], zero between launches
     uint32_t* row_state;       // [rows], written by every launch
+    // split path: [rows][kMaxSegments][kSplitRecordSlots] entries of (key, epoch | token index), and the
+    // row's epoch (1 .. 16383; the row's last workgroup moves it on in every launch)
+    unsigned long long* split_records;
+    uint32_t* row_epoch;
 
     // general-path scratch, [rows][sort_stride] each
     uint32_t* sort_keys[2];
@@ -107,24 +111,27 @@ __device__ __forceinline__ void write_token(
 
 // The CPU sampler from the sorted Top-K window onwards (src/engine/session.cpp:89-134, :429-442),
 // executed by one wave: lane i holds candidate i of n <= 64 candidates in (logit descending, index
-// ascending) order.  Sums run in candidate order on every lane redundantly.
+// ascending) order.  Sums run in candidate order on every lane redundantly.  uniform is the row's draw
+// (a.uniforms[row], loaded by the caller long before: a load here would sit on the row's critical path).
 __device__ __forceinline__ void finish_row_wave(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
-    float value, int32_t index, int n, int lane, uint8_t flags)
+    float value, int32_t index, int n, int lane, uint8_t flags, float uniform, const uint64_t* exp2_table)
 {
+    NCNN_MOE_STAMP_ROW(row, 0);
     n = __builtin_amdgcn_readfirstlane(n); // the same in every lane: the loops over it stay scalar
     const float temperature = p.temperature;
     const float top_value = read_lane(value, 0);
     const float maximum = top_value / temperature;
     float term = 0.0f;
     if (lane < n)
-        term = expf_libm(value / temperature - maximum);
+        term = expf_libm(value / temperature - maximum, exp2_table);
 
     // The three walks below are the CPU's sequential fp32 sums.  They run in trips of four candidates
     // without a data-dependent exit: a lane past the end (or a filtered candidate) adds +0.0, which
     // leaves a non-negative sum as it is, and every lane keeps the running sum at its own position, so
     // that where the CPU loop would have stopped is read off afterwards with one ballot.  (A loop
     // trip costs about as much as ten of these instructions.)
+    NCNN_MOE_STAMP_ROW(row, 1);
     const int trips = (n + 3) >> 2;
     float normalizer = 0.0f;
     for (int trip = 0; trip < trips; ++trip)
@@ -139,6 +146,7 @@ __device__ __forceinline__ void finish_row_wave(
             write_error(a, row, NCNN_MOE_ROW_INVALID_DISTRIBUTION, flags);
         return;
     }
+    NCNN_MOE_STAMP_ROW(row, 2);
     const float probability = term / normalizer;
 
     bool keep = lane < n;
@@ -164,6 +172,7 @@ __device__ __forceinline__ void finish_row_wave(
         if (__ballot(keep && cumulative_here >= p.top_p) != 0)
             break; // the nucleus is complete: the sums behind it are not needed
     }
+    NCNN_MOE_STAMP_ROW(row, 3);
     const uint64_t reached = __ballot(keep && cumulative_here >= p.top_p);
     const int last = reached != 0 ? __builtin_ctzll(reached) : 63 - __builtin_clzll(keep_mask);
     const uint64_t kept_mask = keep_mask & ((2ull << last) - 1ull);
@@ -188,6 +197,7 @@ __device__ __forceinline__ void finish_row_wave(
             a.distribution_count[row] = static_cast<uint32_t>(kept);
     }
 
+    NCNN_MOE_STAMP_ROW(row, 4);
     int selected = 0;
     uint8_t draw_consumed = 0;
     float selected_probability = 1.0f;
@@ -198,7 +208,6 @@ __device__ __forceinline__ void finish_row_wave(
     else
     {
         draw_consumed = 1;
-        const float uniform = a.uniforms[row];
         const bool is_kept = ((kept_mask >> lane) & 1ull) != 0ull;
         const float share = is_kept ? final_probability : 0.0f;
         float running = 0.0f;
@@ -217,9 +226,11 @@ __device__ __forceinline__ void finish_row_wave(
         selected = passed != 0 ? __builtin_ctzll(passed) : last; // past the last sum: the last kept candidate
         selected_probability = read_lane(final_probability, selected);
     }
+    NCNN_MOE_STAMP_ROW(row, 5);
     const int32_t token = read_lane(index, selected);
     if (lane == 0)
         write_token(a, row, p, token, selected_probability, static_cast<uint32_t>(kept), draw_consumed, flags);
+    NCNN_MOE_STAMP_ROW(row, 6);
 }
 
 // The same walk for an ordered window of up to 64 * SLOTS candidates held by one wave: candidate i
@@ -528,7 +539,8 @@ struct BoundScratch
 // top_k-th largest (for top_k = 20 of 10,240 values about 22 reach it, for top_k = 50 about 63), at a
 // third of the cost: two exchanges inside the quads, an LDS round trip, a 16-step search by one wave,
 // a second LDS round trip.  All threads of the workgroup must call it.
-__device__ __forceinline__ uint32_t workgroup_kth_of_quad_maxima(uint32_t key, int top_k, int tid, BoundScratch& scratch)
+__device__ __forceinline__ uint32_t workgroup_kth_of_quad_maxima(
+    uint32_t key, int top_k, int tid, BoundScratch& scratch, uint32_t* maximum_out = nullptr)
 {
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
@@ -548,6 +560,13 @@ __device__ __forceinline__ uint32_t workgroup_kth_of_quad_maxima(uint32_t key, i
         const uint32_t first = scratch.quad_maxima[lane];
         const uint32_t second = scratch.quad_maxima[kWaveSize + lane];
         const auto reaching = [&](uint32_t trial) { return __popcll(__ballot(first >= trial)) + __popcll(__ballot(second >= trial)); };
+        if (maximum_out != nullptr)
+        {
+            // the largest key of the workgroup (an address in LDS), for callers that want the range of the keys
+            const uint32_t largest = wave_max_u32(max(first, second));
+            if (lane == 0)
+                *maximum_out = largest;
+        }
         uint32_t prefix = 0;
         if (top_k * 4 <= reaching(1u) * 3)
         {

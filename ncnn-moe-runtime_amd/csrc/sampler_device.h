@@ -30,6 +30,7 @@ constexpr int kNarrowListCap = 512;      // candidate list for Top-K windows up 
 constexpr int kWideListCap = 4096;       // candidate list for Top-K windows up to kSelectTopK
 constexpr int kSegmentRecordSlots = 256; // candidate slots of a segment's record in HBM
 constexpr int kMaxSegments = 16;
+constexpr int kSplitRecordSlots = 160;   // 8-byte entries of a segment's record on the split path: 2 header entries + up to 2 * 64 + 16 candidates
 constexpr int kWholeRowBatch = 256;          // from this many rows on, one workgroup streams a whole row
 constexpr int kSingleChunkWorkgroups = 4096;  // a smaller batch is split into one-chunk workgroups up to this many (several rounds of 4 per CU beat fewer, looped ones)
 constexpr int kLoopedWorkgroups = 512;        // ... and when each streams several chunks (2 per CU)
@@ -44,6 +45,45 @@ constexpr int kSortTile = kSortThreads * kSortPerThread;
 constexpr int kReplayThreads = 1024;
 constexpr int kReplayPerThread = 4;
 constexpr int kReplayChunk = kReplayThreads * kReplayPerThread;
+
+// Wall-clock stamps for a timeline of the split path, compiled in only with -DNCNN_MOE_TIMELINE (a
+// separate library, built by `make timeline`; the shipped one carries none).
+#ifdef NCNN_MOE_TIMELINE
+constexpr int kTimelineRows = 64;
+constexpr int kTimelineSlots = 16;
+__device__ unsigned long long g_timeline[kTimelineRows * kMaxSegments * kTimelineSlots];
+#define NCNN_MOE_STAMP(row, segment, slot)                                                                   \
+    do                                                                                                       \
+    {                                                                                                        \
+        if (threadIdx.x == 0 && (row) < static_cast<uint32_t>(kTimelineRows))                                \
+            g_timeline[((row) * kMaxSegments + (segment)) * kTimelineSlots + (slot)] = wall_clock64();       \
+    } while (0)
+#define NCNN_MOE_STAMP_VALUE(row, segment, slot, value)                                                     \
+    do                                                                                                       \
+    {                                                                                                        \
+        if (threadIdx.x == 0 && (row) < static_cast<uint32_t>(kTimelineRows))                                \
+            g_timeline[((row) * kMaxSegments + (segment)) * kTimelineSlots + (slot)] = (value);              \
+    } while (0)
+// stamps of the row's last workgroup, from code that does not know its segment; the calling lane is that wave's first
+__device__ unsigned long long g_timeline_rows[kTimelineRows * kTimelineSlots];
+#define NCNN_MOE_STAMP_ROW(row, slot)                                                                        \
+    do                                                                                                       \
+    {                                                                                                        \
+        if ((threadIdx.x & 63) == 0 && (row) < static_cast<uint32_t>(kTimelineRows))                         \
+            g_timeline_rows[(row) * kTimelineSlots + (slot)] = wall_clock64();                               \
+    } while (0)
+#define NCNN_MOE_STAMP_VALUE_FROM(leader, row, segment, slot, value)                                        \
+    do                                                                                                       \
+    {                                                                                                        \
+        if ((leader) && (row) < static_cast<uint32_t>(kTimelineRows))                                        \
+            g_timeline[((row) * kMaxSegments + (segment)) * kTimelineSlots + (slot)] = (value);              \
+    } while (0)
+#else
+#define NCNN_MOE_STAMP_VALUE_FROM(leader, row, segment, slot, value) ((void)0)
+#define NCNN_MOE_STAMP_ROW(row, slot) ((void)0)
+#define NCNN_MOE_STAMP(row, segment, slot) ((void)0)
+#define NCNN_MOE_STAMP_VALUE(row, segment, slot, value) ((void)0)
+#endif
 
 enum RowMode : int
 {
@@ -137,7 +177,9 @@ __device__ __constant__ const uint64_t kExp2Table[32] = {NCNN_MOE_EXP2_TABLE_VAL
 // src/engine/session.cpp:98): x * 32/ln2 = k + r, exp(x) = 2^(k/32) * (1 + c2 r + c1 r^2 + c0 r^3),
 // all in double, one rounding to float at the end.  The reduction uses fma(32/ln2, x, -k), as the
 // FMA build of that routine does; the polynomial rounds identically with or without fused steps.
-__device__ __forceinline__ float expf_libm(float x)
+// table: the 32 entries of kExp2Table, in constant memory or a copy of them in LDS (a caller on a
+// latency-critical path stages it there while it waits for something else).
+__device__ __forceinline__ float expf_libm(float x, const uint64_t* table = kExp2Table)
 {
     const uint32_t bits = __float_as_uint(x);
     const uint32_t abstop = (bits >> 20) & 0x7ffu;
@@ -163,7 +205,7 @@ __device__ __forceinline__ float expf_libm(float x)
     const uint64_t ki = static_cast<uint64_t>(__double_as_longlong(kd));
     kd -= shift;
     const double r = fma(inverse_ln2_scaled, xd, -kd);
-    const uint64_t scale_bits = kExp2Table[ki & 31u] + (ki << 47);
+    const uint64_t scale_bits = table[ki & 31u] + (ki << 47);
     const double scale = __longlong_as_double(static_cast<long long>(scale_bits));
     const double p = fma(c0, r, c1);
     const double r2 = r * r;
@@ -236,6 +278,48 @@ __device__ __forceinline__ float read_lane(float value, int lane)
 __device__ __forceinline__ int read_lane(int value, int lane)
 {
     return __builtin_amdgcn_readlane(value, lane);
+}
+
+template <int CONTROL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_source(uint32_t value)
+{
+    // a lane whose source the control or the row mask leaves out reads 0
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(value), CONTROL, ROW_MASK, 0xf, false));
+}
+
+// Reduction over each row of 16 lanes (every lane receives its row's result), by four DPP exchanges:
+// inside pairs, quads, half rows, rows.
+template <typename Op>
+__device__ __forceinline__ uint32_t row16_reduce_u32(uint32_t value, Op op)
+{
+    value = op(value, dpp_source<0xB1, 0xf>(value));  // quad_perm [1,0,3,2]
+    value = op(value, dpp_source<0x4E, 0xf>(value));  // quad_perm [2,3,0,1]
+    value = op(value, dpp_source<0x141, 0xf>(value)); // row_half_mirror
+    value = op(value, dpp_source<0x140, 0xf>(value)); // row_mirror
+    return value;
+}
+
+// Maximum over the wave, returned to every lane.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t value)
+{
+    const auto larger = [](uint32_t x, uint32_t y) { return max(x, y); };
+    value = row16_reduce_u32(value, larger);
+    value = max(value, dpp_source<0x142, 0xa>(value)); // row_bcast15 into rows 1 and 3
+    value = max(value, dpp_source<0x143, 0xc>(value)); // row_bcast31 into rows 2 and 3
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(value), 63));
+}
+
+// Inclusive prefix sum over the wave's lanes (lane i: sum of lanes 0 .. i), by DPP shifts inside rows of
+// 16 lanes and two broadcasts across rows.  A lane that a shift leaves without a source adds zero.
+__device__ __forceinline__ uint32_t wave_prefix_sum_u32(uint32_t value)
+{
+    value += dpp_source<0x111, 0xf>(value); // row_shr:1
+    value += dpp_source<0x112, 0xf>(value); // row_shr:2
+    value += dpp_source<0x114, 0xf>(value); // row_shr:4
+    value += dpp_source<0x118, 0xf>(value); // row_shr:8
+    value += dpp_source<0x142, 0xa>(value); // row_bcast15: rows 1 and 3 add the row before
+    value += dpp_source<0x143, 0xc>(value); // row_bcast31: rows 2 and 3 add rows 0 + 1
+    return value;
 }
 
 // One compare-exchange stage across lanes at distance j; keep_max selects which partner value stays.

@@ -11,6 +11,7 @@
 
 #include "sampler_full_order.h"
 #include "sampler_select.h"
+#include "sampler_split.h"
 
 namespace ncnn_moe_hip {
 

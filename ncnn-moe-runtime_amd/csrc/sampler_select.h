@@ -106,7 +106,7 @@ __device__ __forceinline__ uint32_t tighten_list(SelectShared<WIDE>& shared, uin
 // The ordered window (lane i holds candidate i of n <= 64) to the row's result; one wave.
 __device__ __forceinline__ void finish_ordered_wave(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p, bool greedy,
-    float value, int32_t index, int n, int lane, uint8_t result_flags)
+    float value, int32_t index, int n, int lane, uint8_t result_flags, float uniform, const uint64_t* exp2_table)
 {
     if (greedy)
     {
@@ -125,7 +125,7 @@ __device__ __forceinline__ void finish_ordered_wave(
         }
         return;
     }
-    finish_row_wave(a, row, p, value, index, n, lane, result_flags);
+    finish_row_wave(a, row, p, value, index, n, lane, result_flags, uniform, exp2_table);
 }
 
 // From the candidate list to the sampled token: exact best K, their order, the epilogue.
@@ -133,7 +133,7 @@ __device__ __forceinline__ void finish_ordered_wave(
 template <bool WIDE>
 __device__ __forceinline__ void finish_from_list(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p, bool greedy, int top_k,
-    SelectShared<WIDE>& shared, uint8_t result_flags, int tid)
+    SelectShared<WIDE>& shared, uint8_t result_flags, int tid, float uniform, const uint64_t* exp2_table = kExp2Table)
 {
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
@@ -216,7 +216,7 @@ __device__ __forceinline__ void finish_from_list(
             }
             const float value = lane < n ? shared.final_values[lane] : 0.0f;
             const int32_t index = lane < n ? shared.final_indices[lane] : -1;
-            finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags);
+            finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags, uniform, exp2_table);
             return;
         }
         if (n_list <= 2 * kWaveSize)
@@ -261,7 +261,7 @@ __device__ __forceinline__ void finish_from_list(
                 a.row_state[row] = kRowDone;
             const float value = lane < n ? shared.final_values[lane] : 0.0f;
             const int32_t index = lane < n ? shared.final_indices[lane] : -1;
-            finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags);
+            finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags, uniform, exp2_table);
             return;
         }
         if (wave != 0)
@@ -297,7 +297,7 @@ __device__ __forceinline__ void finish_from_list(
         }
         value = lane < n ? shared.final_values[lane] : 0.0f;
         index = lane < n ? shared.final_indices[lane] : -1;
-        finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags);
+        finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags, uniform, exp2_table);
         return;
     }
     if constexpr (WIDE)
@@ -441,6 +441,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     uint4 raw[2][kVectors];
     load_chunk<DTYPE, kVectors>(raw[0], aligned_base, first_chunk * kChunk, valid_begin, segment_end, valid_end, tid);
     const ncnn_moe_sample_params p = a.params[row];
+    const float uniform = a.uniforms[row];
     uint32_t effective_k = 0;
     int status = NCNN_MOE_ROW_OK;
     const int mode = resolve_row_mode(p, a.vocab, a.max_select_top_k, a.force_general, effective_k, status);
@@ -552,7 +553,9 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         // ---- bound of the first chunk: the K-th largest lane maximum, or a cheaper bound below it.  The
         // lanes at or above it each hold a distinct logit at least that large, so the K-th best logit of
         // the row is no smaller.
-        if (first_of_segment)
+        // (also a later chunk while there is no bound yet: a row that begins with a stretch of -inf, a masked
+        // part of the vocabulary, must not pour its first chunk of finite logits into the list unfiltered)
+        if (first_of_segment || (LOOPED && bound_key == 0u))
         {
             if (WIDE && top_k > kTwoKeyBoundTopK)
             {
@@ -715,7 +718,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
             }
             return;
         }
-        finish_from_list(a, row, p, greedy, top_k, shared, result_flags, tid);
+        finish_from_list(a, row, p, greedy, top_k, shared, result_flags, tid, uniform);
         return;
     }
 
@@ -856,7 +859,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         }
         return;
     }
-    finish_from_list(a, row, p, greedy, top_k, shared, result_flags, tid);
+    finish_from_list(a, row, p, greedy, top_k, shared, result_flags, tid, uniform);
 }
 
 } // namespace ncnn_moe_hip

@@ -1,0 +1,547 @@
+// Split rows: the HBM pass for small batches, where a row is covered by several workgroups of one chunk
+// each so that every compute unit streams (greedy rows and Top-K windows up to kFastTopK).
+//
+// Every workgroup of a row keeps the logits of its chunk that can belong to the row's Top-K window (the
+// values at or above a bound that at least K values of the chunk reach) and hands them over through a
+// record in device memory; the workgroup of the row that arrives last merges the records and finishes
+// the row.  Between the last logit and the row's result lies a chain of dependent steps, and at these
+// batch sizes that chain, not the streaming, sets the time of the launch.  The hand-over is therefore
+// built so that nothing on it waits for a store to be acknowledged:
+//   * a record entry is 8 bytes, (key, epoch | token index), written with one store; the epoch is a
+//     per-row launch number kept in device memory, so a reader tells an entry of this launch from what an
+//     earlier launch left behind without any clearing;
+//   * a workgroup issues its entries and, without waiting for them, counts itself on the row's counter;
+//   * the last workgroup reads every record (first through this XCD's L2, which holds what the row's
+//     other workgroups wrote if they ran on this XCD) and checks the epochs: an entry that has not landed
+//     yet, or a stale line, fails the check and the records are read again around the L2.  Such a retry
+//     waits only for stores that were issued before their workgroup counted itself, never for another
+//     workgroup to run;
+//   * the merge cuts the row's candidates with one histogram over the key range [largest segment bound,
+//     row maximum] in LDS, scanned by every wave for itself, and ranks what is left.
+#ifndef NCNN_MOE_HIP_SAMPLER_SPLIT_H
+#define NCNN_MOE_HIP_SAMPLER_SPLIT_H
+
+#include "sampler_select.h"
+
+namespace ncnn_moe_hip {
+
+constexpr int kSplitHeaderEntries = 2;  // (segment bound, count | flags) and (segment maximum, 0)
+constexpr int kSplitLanesPerSegment = kScanThreads / kMaxSegments; // 32 lanes read one segment's record
+constexpr int kSplitSlotsPerLane = (kSplitRecordSlots + kSplitLanesPerSegment - 1) / kSplitLanesPerSegment;
+constexpr uint32_t kSplitIndexBits = 18; // a split row holds at most 16 chunks of 12,288 logits
+constexpr uint32_t kSplitIndexMask = (1u << kSplitIndexBits) - 1u;
+constexpr uint32_t kSplitLastEpoch = (1u << (32 - kSplitIndexBits)) - 1u; // epochs run 1 .. 16383; 0 never tags an entry
+constexpr int kSplitBins = kWaveSize;    // one histogram bin per lane of the scanning wave
+constexpr uint32_t kSplitRetryLimit = 1u << 16;
+static_assert(kMaxSegments * kSegmentValuesBF16 + 8 <= (1 << kSplitIndexBits), "token indices of a split row fit the entry");
+static_assert(kSplitHeaderEntries + 2 * kFastTopK + 16 <= kSplitRecordSlots, "a record holds the widest hand-over");
+static_assert(kSplitLanesPerSegment * 2 == kWaveSize, "a wave reads the records of two segments");
+
+struct SplitSegmentInfo
+{
+    uint32_t bound;
+    uint32_t maximum;
+    uint32_t count_and_flags; // bits 0-7 entries handed over, bits 8-10 ScanFlags, bit 31 the header was valid
+};
+
+struct SplitShared
+{
+    SelectShared<false> select;
+    SplitSegmentInfo segments[kMaxSegments];
+    uint32_t histogram[kSplitBins];
+    uint32_t segment_maximum;
+    uint64_t exp2_table[32];
+    int is_last;
+};
+
+// A scalar load through the scalar cache, for a word that nobody writes before the caller's last use
+// of it in this launch (the cache starts a launch empty).  Every wave of a workgroup, and every workgroup
+// of a row, asks for the same word: through the cache that costs next to nothing, around it (glc) seven
+// thousand loads of 64 words took 100 us.
+__device__ __forceinline__ uint32_t scalar_load_u32(const uint32_t* address)
+{
+    uint32_t value;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(value) : "s"(address) : "memory");
+    return value;
+}
+
+// One record entry.  Stores go through to device memory (any workgroup of the row may merge); the first
+// read of the merge stops at this XCD's L2 (and goes around the compute unit's vector cache), a repeated
+// one goes around the L2 as well.
+__device__ __forceinline__ void store_entry(unsigned long long* address, uint32_t key, uint32_t tagged)
+{
+    __hip_atomic_store(address, static_cast<unsigned long long>(key) | (static_cast<unsigned long long>(tagged) << 32),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ unsigned long long load_entry(const unsigned long long* address, bool around_l2)
+{
+    return around_l2 ? __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                     : __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+template <int DTYPE>
+__global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4) void split_select_kernel(SamplerArgs a)
+{
+    using Vector = LogitsVector<DTYPE>;
+    constexpr int kWidth = Vector::kWidth;
+    constexpr int kVectors = Vector::kVectorsPerLane;
+    constexpr int kLaneValues = kVectors * kWidth;
+    constexpr uint32_t kChunk = static_cast<uint32_t>(kScanThreads) * kLaneValues;
+    constexpr uint32_t kNegativeInfinity = 0xff800000u;
+    constexpr uint32_t kPositiveInfinity = 0x7f800000u;
+
+    // Workgroups are handed to the eight XCDs in turn: a grouped grid numbers them so that the segments
+    // of a row land on one XCD and the merge finds their records in that XCD's L2.  (Nothing relies on
+    // it: a record that is not there fails the epoch check and is read again from device memory.)
+    uint32_t row = blockIdx.y;
+    uint32_t segment = blockIdx.x;
+    if (a.xcd_grouped != 0u)
+    {
+        const uint32_t turn = blockIdx.x >> 3;
+        row = (turn / a.segments) * 8u + (blockIdx.x & 7u);
+        segment = turn % a.segments;
+        if (row >= a.rows)
+            return;
+    }
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+
+    __shared__ SplitShared shared;
+    SelectShared<false>& select = shared.select;
+
+    NCNN_MOE_STAMP(row, segment, 0);
+    // The chunk's loads go out before anything that waits for the row's options.
+    const char* row_pointer = static_cast<const char*>(a.logits) +
+        static_cast<size_t>(row) * a.row_stride * Vector::kElementBytes;
+    const uint32_t misalignment =
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row_pointer) & 15u) / Vector::kElementBytes;
+    const char* aligned_base = row_pointer - static_cast<size_t>(misalignment) * Vector::kElementBytes;
+    const uint32_t valid_begin = misalignment;
+    const uint32_t valid_end = misalignment + a.vocab;
+    const uint32_t chunk_base = segment * kChunk;
+    const uint32_t segment_end = min(valid_end, chunk_base + kChunk);
+
+    // The first workgroup on every XCD touches the small operands of that XCD's rows (options, draw,
+    // epoch) before the memory system fills up with the logits: a first access to them
+    // by a workgroup that starts a microsecond later queues behind tens of megabytes and takes several
+    // microseconds; once they sit in the XCD's L2 it takes a few hundred nanoseconds.
+    uint32_t touched = 0;
+    if (a.xcd_grouped != 0u && blockIdx.x < 8u)
+    {
+        const uint32_t other_row = blockIdx.x + 8u * static_cast<uint32_t>(tid);
+        if (other_row < a.rows)
+        {
+            touched = reinterpret_cast<const uint32_t*>(a.params + other_row)[0] ^ reinterpret_cast<const uint32_t*>(a.params + other_row)[5] ^
+                __float_as_uint(a.uniforms[other_row]) ^ a.row_epoch[other_row];
+        }
+    }
+    uint4 raw[kVectors];
+    load_chunk<DTYPE, kVectors>(raw, aligned_base, chunk_base, valid_begin, segment_end, valid_end, tid);
+    const ncnn_moe_sample_params p = a.params[row];
+    const float uniform = a.uniforms[row];
+    const uint64_t exp2_entry = kExp2Table[tid & 31]; // staged in LDS below: the merge's exponentials find it there
+    const uint32_t epoch = scalar_load_u32(&a.row_epoch[row]);
+    uint32_t effective_k = 0;
+    int status = NCNN_MOE_ROW_OK;
+    const int mode = resolve_row_mode(p, a.vocab, kFastTopK, a.force_general, effective_k, status);
+    if (mode == kModeInvalid || mode == kModeGeneral)
+    {
+        if (segment == 0 && tid == 0)
+        {
+            if (mode == kModeInvalid)
+            {
+                write_error(a, row, status, 0);
+                a.row_state[row] = kRowDone;
+            }
+            else
+            {
+                write_pending(a, row);
+                a.row_state[row] = kRowNeedsGeneral;
+            }
+        }
+        return;
+    }
+    const bool greedy = mode == kModeGreedy;
+    const int top_k = static_cast<int>(effective_k);
+    const uint32_t record_entries = segment_record_entries(effective_k);
+    if (tid == 0)
+    {
+        select.block_flags = 0;
+        select.list_count = 0;
+        shared.segment_maximum = 0xffffffffu; // unknown unless the bound routine below reports it
+    }
+    if (tid < 32)
+        shared.exp2_table[tid] = exp2_entry;
+    if (touched == 0x9e3779b9u)
+        select.block_flags = 0; // keeps the touching loads alive; the value is never that
+    __syncthreads(); // also waits for the chunk
+    NCNN_MOE_STAMP(row, segment, 1);
+
+    // ---- the chunk: maxima, flags.  Nearly every chunk lies inside the row (only a row's last chunk, or
+    // the first one of a row that does not start on a 16-byte boundary, holds foreign elements): those skip
+    // the masking, a few hundred instructions per wave that four workgroups per compute unit would
+    // otherwise all issue at the moment their logits arrive.
+    float values[kLaneValues];
+    float lane_max = __uint_as_float(kNegativeInfinity);
+    bool saw_nan = false;
+    const bool interior = chunk_base >= valid_begin && chunk_base + kChunk <= segment_end; // the same in every thread
+    if (interior)
+    {
+#pragma unroll
+        for (int v = 0; v < kVectors; ++v)
+            Vector::unpack(raw[v], &values[v * kWidth]);
+#pragma unroll
+        for (int i = 0; i < kLaneValues; i += 2)
+        {
+            saw_nan = saw_nan || __builtin_isunordered(values[i], values[i + 1]);
+            lane_max = fmaxf(lane_max, fmaxf(values[i], values[i + 1]));
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int v = 0; v < kVectors; ++v)
+        {
+            const uint32_t first = chunk_base + static_cast<uint32_t>(v * kScanThreads + tid) * kWidth;
+            const bool any_valid = first < segment_end && first + kWidth > valid_begin;
+            if (any_valid)
+                Vector::unpack(raw[v], &values[v * kWidth]);
+            else
+            {
+#pragma unroll
+                for (int c = 0; c < kWidth; ++c)
+                    values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
+            }
+            if (any_valid && (first < valid_begin || first + kWidth > segment_end))
+            {
+#pragma unroll
+                for (int c = 0; c < kWidth; ++c)
+                {
+                    const uint32_t position = first + c;
+                    if (position < valid_begin || position >= segment_end)
+                        values[v * kWidth + c] = __uint_as_float(kNegativeInfinity);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < kWidth; ++c)
+            {
+                const float x = values[v * kWidth + c];
+                saw_nan = saw_nan || (x != x);
+                lane_max = fmaxf(lane_max, x);
+            }
+        }
+    }
+    uint32_t local_flags = saw_nan ? kScanSawNan : 0u;
+    if (__ballot(lane_max == __uint_as_float(kPositiveInfinity)) != 0)
+    {
+        local_flags |= lane_max == __uint_as_float(kPositiveInfinity) ? kScanSawPositiveInfinity : 0u;
+        if (greedy)
+        {
+            // greedy skips every non-finite logit (session.cpp:411-412): rare, so redone out of line
+            lane_max = __uint_as_float(kNegativeInfinity);
+#pragma unroll
+            for (int i = 0; i < kLaneValues; ++i)
+            {
+                if (values[i] == __uint_as_float(kPositiveInfinity))
+                    values[i] = __uint_as_float(kNegativeInfinity);
+                lane_max = fmaxf(lane_max, values[i]);
+            }
+        }
+    }
+
+    // ---- bound: at least K logits of the chunk reach it, so the row's K-th best is no smaller
+    const uint32_t lane_keys[1] = {lane_max == __uint_as_float(kNegativeInfinity) ? 0u : ascending_key(lane_max)};
+    uint32_t bound_key = workgroup_kth_of_quad_maxima(lane_keys[0], top_k, tid, select.bound, &shared.segment_maximum);
+    if (bound_key == 0u) // a chunk with few values: the exact K-th largest lane maximum
+        bound_key = workgroup_kth_largest_key(lane_keys, top_k, tid, select.bound, true);
+    NCNN_MOE_STAMP(row, segment, 2);
+    // no bound (fewer than K lanes hold a finite logit): every finite logit is a candidate
+    const float threshold = bound_key == 0u ? -3.402823466e+38f : fmaxf(value_from_ascending_key(bound_key), -3.402823466e+38f);
+
+    // ---- collect the values at or above the bound.  Nearly every lane that holds a candidate holds
+    // exactly one, its maximum: each lane counts its candidates and locates its maximum without a branch,
+    // one append per wave takes the maxima, and the lanes that hold more hand the others over one per
+    // round.  (A compare, a ballot and a branch per slot costs a wave twice as much: each is a trip from
+    // the vector to the scalar unit.)
+    int lane_hits = 0;
+    int best_at = 0;
+#pragma unroll
+    for (int i = 0; i < kLaneValues; ++i)
+    {
+        lane_hits += values[i] >= threshold ? 1 : 0;
+        best_at = values[i] == lane_max ? i : best_at;
+    }
+    const auto element_of = [&](int i) {
+        return static_cast<int32_t>(chunk_base + static_cast<uint32_t>((i / kWidth) * kScanThreads + tid) * kWidth +
+                                    static_cast<uint32_t>(i % kWidth) - misalignment);
+    };
+    append_candidate(select, lane_hits >= 1, ascending_key(lane_max), element_of(best_at), lane);
+    if (__ballot(lane_hits > 1) != 0)
+    {
+        uint32_t rest = 0; // bit i: value i is a candidate that has not been appended
+#pragma unroll
+        for (int i = 0; i < kLaneValues; ++i)
+            rest |= (lane_hits > 1 && values[i] >= threshold && i != best_at) ? (1u << i) : 0u;
+        while (__ballot(rest != 0u) != 0)
+        {
+            // the value is read back from the row (its register is not known until run time)
+            const int i = rest != 0u ? __builtin_ctz(rest) : 0;
+            const int32_t element = element_of(i);
+            float x = 0.0f;
+            if (rest != 0u)
+            {
+                if constexpr (DTYPE == NCNN_MOE_LOGITS_F32)
+                    x = reinterpret_cast<const float*>(row_pointer)[element];
+                else
+                    x = __uint_as_float(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(row_pointer)[element]) << 16);
+            }
+            append_candidate(select, rest != 0u, ascending_key(x), element, lane);
+            rest &= rest - 1u;
+        }
+    }
+    if (local_flags != 0)
+        atomicOr(&select.block_flags, local_flags);
+    __syncthreads();
+    NCNN_MOE_STAMP(row, segment, 3);
+    bool overflow = select.list_count > static_cast<uint32_t>(kNarrowListCap);
+    // the record holds 2K + 16 candidates: a longer list (a loose bound, ties) is cut to the exact window first
+    if (!overflow && select.list_count > record_entries)
+        bound_key = tighten_list(select, bound_key, top_k, tid);
+    const uint32_t handed = select.list_count;
+    overflow = overflow || handed > record_entries;
+    const uint32_t segment_flags = select.block_flags | (overflow ? static_cast<uint32_t>(kScanOverflow) : 0u);
+    const uint32_t own_count = overflow ? 0u : handed;
+
+    // ---- hand-over: the entries go out, nothing waits for them
+    unsigned long long* const row_records = a.split_records + static_cast<size_t>(row) * kMaxSegments * kSplitRecordSlots;
+    unsigned long long* const own_record = row_records + static_cast<size_t>(segment) * kSplitRecordSlots;
+    const uint32_t tag = epoch << kSplitIndexBits;
+    for (uint32_t j = tid; j < own_count; j += kScanThreads)
+        store_entry(&own_record[kSplitHeaderEntries + j], select.list_keys[j], tag | static_cast<uint32_t>(select.list_indices[j]));
+    if (tid == 0)
+    {
+        store_entry(&own_record[0], bound_key, tag | own_count | (segment_flags << 8));
+        store_entry(&own_record[1], shared.segment_maximum, tag);
+    }
+    // How the row's last workgroup reads the records: lanes 32 h .. 32 h + 31 of wave w read the record of
+    // segment 2 w + h, entry by entry (consecutive lanes, consecutive entries); the workgroup's own list
+    // stays in LDS.  (Issuing these loads before the counter's atomic, so that they travel beside it, does
+    // not pay: two times out of three an entry of a workgroup that counted itself a moment earlier has
+    // not landed yet, and the second trip costs more than the first saved.)
+    const uint32_t read_segment = static_cast<uint32_t>(2 * wave + (lane >> 5));
+    const int read_lane = lane & (kSplitLanesPerSegment - 1);
+    const uint32_t entries_to_read = static_cast<uint32_t>(kSplitHeaderEntries) + record_entries;
+    const unsigned long long* const read_record = row_records + static_cast<size_t>(read_segment) * kSplitRecordSlots;
+    const bool reads_own = read_segment == segment;
+    const bool reads_any = read_segment < a.segments && !reads_own;
+    unsigned long long loaded[kSplitSlotsPerLane];
+    const auto load_records = [&](bool around_l2) {
+#pragma unroll
+        for (int j = 0; j < kSplitSlotsPerLane; ++j)
+        {
+            const uint32_t entry = static_cast<uint32_t>(j * kSplitLanesPerSegment + read_lane);
+            if (!reads_own) // the lanes that stand for this workgroup's own segment keep what they took from its list
+                loaded[j] = 0ull;
+            if (reads_any && entry < entries_to_read)
+                loaded[j] = load_entry(&read_record[entry], around_l2);
+        }
+    };
+    // The last wave counts the workgroup in (its lanes stored nothing unless the list is very long, so
+    // the atomic's return does not queue behind a store's acknowledgement).
+    if (tid == kScanThreads - kWaveSize)
+    {
+        const unsigned long long previous = __hip_atomic_fetch_add(&a.row_counter[row], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        shared.is_last = previous == a.segments - 1 ? 1 : 0;
+    }
+    lds_barrier();
+    NCNN_MOE_STAMP(row, segment, 4);
+    if (!shared.is_last)
+        return;
+
+    // ---- last workgroup of the row.  The row's next launch gets a new epoch whatever happens below.
+    if (tid == 0)
+    {
+        a.row_counter[row] = 0;
+        store_agent(&a.row_epoch[row], epoch == kSplitLastEpoch ? 1u : epoch + 1u);
+    }
+    // this workgroup's own candidates, from its list (entry numbering as in a record)
+    if (reads_own)
+    {
+#pragma unroll
+        for (int j = 0; j < kSplitSlotsPerLane; ++j)
+        {
+            const uint32_t entry = static_cast<uint32_t>(j * kSplitLanesPerSegment + read_lane);
+            loaded[j] = 0ull;
+            if (entry >= static_cast<uint32_t>(kSplitHeaderEntries) && entry - kSplitHeaderEntries < own_count)
+            {
+                const uint32_t q = entry - kSplitHeaderEntries;
+                loaded[j] = static_cast<unsigned long long>(select.list_keys[q]) |
+                    (static_cast<unsigned long long>(tag | static_cast<uint32_t>(select.list_indices[q])) << 32);
+            }
+        }
+    }
+    load_records(false);
+    uint32_t lower = 0, upper = 0, row_flags = 0;
+    uint32_t my_count = 0;
+    uint32_t attempts = 0;
+    for (uint32_t attempt = 0;; ++attempt)
+    {
+        attempts = attempt + 1u;
+        // headers: entries 0 and 1 sit in lanes 0 and 1 of the 32 lanes that read the segment
+        const int low_word = static_cast<int>(static_cast<uint32_t>(loaded[0]));
+        const int high_word = static_cast<int>(static_cast<uint32_t>(loaded[0] >> 32));
+        const bool upper_half = lane >= kSplitLanesPerSegment;
+        const uint32_t bound_word = static_cast<uint32_t>(upper_half ? __builtin_amdgcn_readlane(low_word, 32) : __builtin_amdgcn_readlane(low_word, 0));
+        const uint32_t bound_tag = static_cast<uint32_t>(upper_half ? __builtin_amdgcn_readlane(high_word, 32) : __builtin_amdgcn_readlane(high_word, 0));
+        const uint32_t maximum_word = static_cast<uint32_t>(upper_half ? __builtin_amdgcn_readlane(low_word, 33) : __builtin_amdgcn_readlane(low_word, 1));
+        const uint32_t maximum_tag = static_cast<uint32_t>(upper_half ? __builtin_amdgcn_readlane(high_word, 33) : __builtin_amdgcn_readlane(high_word, 1));
+        SplitSegmentInfo info;
+        bool valid = true;
+        if (reads_own)
+        {
+            info.bound = bound_key;
+            info.maximum = shared.segment_maximum;
+            info.count_and_flags = own_count | (segment_flags << 8);
+        }
+        else if (reads_any)
+        {
+            valid = (bound_tag >> kSplitIndexBits) == epoch && (maximum_tag >> kSplitIndexBits) == epoch;
+            info.bound = bound_word;
+            info.maximum = maximum_word;
+            info.count_and_flags = bound_tag & 0x7ffu;
+        }
+        else
+        {
+            info.bound = 0u;
+            info.maximum = 0u;
+            info.count_and_flags = 0u;
+        }
+        my_count = valid ? (info.count_and_flags & 0xffu) : 0u;
+        if (reads_any && valid)
+        {
+#pragma unroll
+            for (int j = 0; j < kSplitSlotsPerLane; ++j)
+            {
+                const uint32_t entry = static_cast<uint32_t>(j * kSplitLanesPerSegment + read_lane);
+                if (entry >= static_cast<uint32_t>(kSplitHeaderEntries) && entry - kSplitHeaderEntries < my_count)
+                    valid = valid && (static_cast<uint32_t>(loaded[j] >> 32) >> kSplitIndexBits) == epoch;
+            }
+        }
+        // bit 31: something of this segment's record is not of this launch (each half of the wave for its own)
+        const uint64_t invalid_lanes = __ballot(!valid);
+        const uint32_t half_invalid = upper_half ? static_cast<uint32_t>(invalid_lanes >> 32) : static_cast<uint32_t>(invalid_lanes);
+        info.count_and_flags |= half_invalid != 0u ? 0x80000000u : 0u;
+        if (tid < kSplitBins)
+            shared.histogram[tid] = 0;
+        if (read_lane == 0)
+            shared.segments[read_segment] = info;
+        lds_barrier();
+        // every wave reduces the sixteen segments for itself
+        const SplitSegmentInfo other = shared.segments[lane & (kMaxSegments - 1)];
+        const auto larger = [](uint32_t x, uint32_t y) { return max(x, y); };
+        lower = row16_reduce_u32(other.bound, larger);
+        upper = row16_reduce_u32(other.maximum, larger);
+        row_flags = row16_reduce_u32(other.count_and_flags >> 8, [](uint32_t x, uint32_t y) { return x | y; });
+        if ((row_flags & 0x800000u) == 0u)
+            break;
+        lds_barrier(); // every wave has read the segments before the next round rewrites them
+        // An entry of this launch has not landed yet (or the L2 held a stale line): read the records
+        // again from device memory.  The stores in question were issued before their workgroup counted
+        // itself, so they land without anyone else having to run.
+        if (attempt >= kSplitRetryLimit)
+        {
+            if (tid == 0)
+            {
+                write_pending(a, row);
+                a.row_state[row] = kRowNeedsGeneral;
+            }
+            return;
+        }
+        load_records(true);
+    }
+    if (epoch == kSplitLastEpoch)
+    {
+        // the epochs start over: nothing that the old ones tagged may be left (the records are read)
+        for (uint32_t j = tid; j < static_cast<uint32_t>(kMaxSegments * kSplitRecordSlots); j += kScanThreads)
+            store_entry(&row_records[j], 0u, 0u);
+    }
+    NCNN_MOE_STAMP(row, segment, 5);
+    NCNN_MOE_STAMP_VALUE(row, segment, 8, attempts);
+    const uint8_t result_flags = (row_flags & kScanSawNan) ? NCNN_MOE_ROW_FLAG_HAS_NAN : 0;
+    if (row_flags & kScanOverflow)
+    {
+        // ties (or values that defeat the bound) left more candidates than a record holds: the full-order kernels take the row
+        if (tid == 0)
+        {
+            write_pending(a, row);
+            a.row_state[row] = kRowNeedsGeneral;
+        }
+        return;
+    }
+    if (!greedy && (row_flags & kScanSawPositiveInfinity))
+    {
+        // the stable order puts +inf first and the CPU sampler rejects the row (session.cpp:84-85)
+        if (tid == 0)
+        {
+            write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
+            a.row_state[row] = kRowDone;
+        }
+        return;
+    }
+
+    // ---- cut: a histogram of the candidates at or above the largest segment bound (at least K logits of
+    // that segment reach it, so nothing below it is in the window) over [that bound, row maximum], bin 0
+    // at the top.  The first bin at which the count from the top reaches K ends the selection.
+    const uint32_t span = upper >= lower ? upper - lower : 0u;
+    const float scale = static_cast<float>(kSplitBins) / (static_cast<float>(span) + 1.0f);
+    int bins[kSplitSlotsPerLane];
+#pragma unroll
+    for (int j = 0; j < kSplitSlotsPerLane; ++j)
+    {
+        const uint32_t entry = static_cast<uint32_t>(j * kSplitLanesPerSegment + read_lane);
+        const uint32_t key = static_cast<uint32_t>(loaded[j]);
+        const bool candidate = entry >= static_cast<uint32_t>(kSplitHeaderEntries) && entry - kSplitHeaderEntries < my_count && key >= lower;
+        bins[j] = -1;
+        if (candidate)
+        {
+            const uint32_t distance = min(key, upper) - lower;
+            const int from_bottom = min(kSplitBins - 1, static_cast<int>(static_cast<float>(distance) * scale));
+            bins[j] = kSplitBins - 1 - from_bottom;
+            atomicAdd(&shared.histogram[bins[j]], 1u);
+        }
+    }
+    if (tid == 0)
+        select.list_count = 0;
+    lds_barrier();
+    const uint32_t from_top = wave_prefix_sum_u32(shared.histogram[lane]);
+    const uint64_t reached = __ballot(from_top >= static_cast<uint32_t>(top_k));
+    const int cut = reached != 0 ? __builtin_ctzll(reached) : kSplitBins - 1;
+    const uint32_t selected = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(from_top), cut));
+    if (selected > static_cast<uint32_t>(kNarrowListCap))
+    {
+        if (tid == 0)
+        {
+            write_pending(a, row);
+            a.row_state[row] = kRowNeedsGeneral;
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < kSplitSlotsPerLane; ++j)
+    {
+        if (static_cast<uint32_t>(j * kSplitLanesPerSegment) >= entries_to_read)
+            break; // no entry of this or a later round exists (a scalar test)
+        append_candidate(select, bins[j] >= 0 && bins[j] <= cut, static_cast<uint32_t>(loaded[j]),
+                         static_cast<int32_t>(static_cast<uint32_t>(loaded[j] >> 32) & kSplitIndexMask), lane);
+    }
+    __syncthreads();
+    NCNN_MOE_STAMP(row, segment, 6);
+    finish_from_list(a, row, p, greedy, top_k, select, result_flags, tid, uniform, shared.exp2_table);
+    NCNN_MOE_STAMP(row, segment, 7);
+}
+
+} // namespace ncnn_moe_hip
+
+#endif // NCNN_MOE_HIP_SAMPLER_SPLIT_H

@@ -63,10 +63,15 @@ EXPORTED_SYMBOLS = [
     "ncnn_moe_hip_sampler_last_error",
     "ncnn_moe_hip_sampler_status_message",
     "ncnn_moe_hip_sampler_device_count",
+]
+
+# include/ncnn_moe_hip_sampler_testing.h: hooks for this repository's tests
+TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_force_general",
     "ncnn_moe_hip_sampler_debug_scatter_segments",
     "ncnn_moe_hip_sampler_debug_expf",
     "ncnn_moe_hip_sampler_debug_exp2_table",
+    "ncnn_moe_hip_sampler_debug_select_geometry",
 ]
 
 
@@ -113,6 +118,9 @@ def load_library():
     lib.ncnn_moe_hip_sampler_debug_expf.argtypes = [vp, vp, vp, ctypes.c_size_t]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.argtypes = [vp]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.restype = None
+    lib.ncnn_moe_hip_sampler_debug_select_geometry.argtypes = [
+        ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
+        ctypes.POINTER(ctypes.c_uint32)]
     _library = lib
     return lib
 
@@ -123,6 +131,21 @@ def status_message(row_status):
 
 def verify_status_message(verify_status):
     return load_library().ncnn_moe_hip_sampler_verify_status_message(int(verify_status)).decode()
+
+
+GEOMETRY_WHOLE_ROW = 0
+GEOMETRY_SPLIT_ONE_CHUNK = 1
+GEOMETRY_SPLIT_LOOPED = 2
+
+
+def select_geometry(dtype, rows, vocab):
+    """(workgroups per row, chunks per workgroup, kernel variant) of the first select kernel for this shape."""
+    segments, chunks, variant = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
+    rc = load_library().ncnn_moe_hip_sampler_debug_select_geometry(
+        dtype, rows, vocab, ctypes.byref(segments), ctypes.byref(chunks), ctypes.byref(variant))
+    if rc != RC_SUCCESS:
+        raise SamplerError("select_geometry: rc=%d" % rc)
+    return segments.value, chunks.value, variant.value
 
 
 def exp2_table():

@@ -26,12 +26,27 @@ def router_functions():
 
 def test_header_and_binding_agree():
     assert declared_functions() == sorted(hip_sampler.EXPORTED_SYMBOLS)
+    assert declared_functions("ncnn_moe_hip_sampler_testing.h") == sorted(hip_sampler.TESTING_SYMBOLS)
+    assert not [name for name in declared_functions() if "_debug_" in name], "test hooks belong in the testing header"
 
 
 def test_library_exports_every_declared_function():
     library = hip_sampler.load_library()
-    for name in declared_functions():
+    for name in declared_functions() + declared_functions("ncnn_moe_hip_sampler_testing.h"):
         assert getattr(library, name) is not None
+
+
+def test_select_geometry_of_the_benchmark_shapes():
+    """The kernel variant behind each benchmark configuration, and the shapes that the GPU tests name."""
+    f32, bf16 = hip_sampler.LOGITS_F32, hip_sampler.LOGITS_BF16
+    assert hip_sampler.select_geometry(f32, 64, 151936) == (15, 1, hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK)
+    assert hip_sampler.select_geometry(f32, 1, 32000) == (4, 1, hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK)
+    assert hip_sampler.select_geometry(f32, 512, 129280)[2] == hip_sampler.GEOMETRY_WHOLE_ROW
+    assert hip_sampler.select_geometry(bf16, 1024, 262144)[2] == hip_sampler.GEOMETRY_WHOLE_ROW
+    for rows in (8, 64, 130, 200, 255):
+        for vocab in (163841, 262144):
+            segments, chunks, variant = hip_sampler.select_geometry(f32, rows, vocab)
+            assert variant == hip_sampler.GEOMETRY_SPLIT_LOOPED and chunks > 1 and segments > 1
 
 
 def test_router_header_and_binding_agree():

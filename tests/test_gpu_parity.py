@@ -385,10 +385,14 @@ def test_whole_row_long_final_lists(batch_sampler):
 
 
 @pytest.mark.parametrize("rows", [200, 130, 90])
-def test_multi_chunk_segments(batch_sampler, rows):
-    """Between 65 and 255 rows of a long vocabulary a segment streams several chunks before the hand-over."""
+def test_many_segments_per_row(batch_sampler, rows):
+    """Between 65 and 255 rows of a long vocabulary: eleven (fp32) or nine (bf16) one-chunk workgroups per
+    row, with sorted rows whose chunks defeat each other's bounds.  (Workgroups that stream several chunks
+    before the hand-over: tests/test_gpu_split_rows.py.)"""
     rng = np.random.default_rng(73 + rows)
     vocab = 109000
+    assert hip_sampler.select_geometry(hip_sampler.LOGITS_F32, rows, vocab) == (11, 1, hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK)
+    assert hip_sampler.select_geometry(hip_sampler.LOGITS_BF16, rows, vocab) == (9, 1, hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK)
     logits = (rng.standard_normal((rows, vocab)) * 2).astype(np.float32)
     logits[::4] = np.sort(logits[::4], axis=1)
     _plant_edge_rows(logits, 20)
@@ -396,10 +400,10 @@ def test_multi_chunk_segments(batch_sampler, rows):
     uniforms = rng.random(rows).astype(np.float32)
     select_rows = _select_rows(params, [20])
     select_rows[::4] = False   # ascending rows may overflow the candidate list: every chunk beats the bound
-    _check_rows(batch_sampler, logits, params, uniforms, context="multi-chunk segments, %d rows" % rows,
+    _check_rows(batch_sampler, logits, params, uniforms, context="many segments per row, %d rows" % rows,
                 select_rows=select_rows)
     bf16 = workloads.float32_to_bf16_bits(logits)
-    _check_rows(batch_sampler, bf16, params, uniforms, dtype="bf16", context="multi-chunk segments bf16, %d rows" % rows)
+    _check_rows(batch_sampler, bf16, params, uniforms, dtype="bf16", context="many segments per row, bf16, %d rows" % rows)
 
 
 def test_wide_windows_small_batch(small_sampler):
