@@ -51,12 +51,48 @@ def algorithmic_bytes(rows, vocab, element_bytes):
 
 def measured_traffic(workload_name):
     """HBM bytes per launch of the dominant kernel as measured with rocprofv3 --pmc FETCH_SIZE and
-    WRITE_SIZE (each scaled by the reading of a 256 MiB copy), recorded beside the profile summaries."""
-    path = os.path.join(ROOT, "profiles", "scan_select_%s_traffic.json" % workload_name)
+    WRITE_SIZE (each scaled by the reading of a 256 MiB copy), recorded beside the profile summaries:
+    a stored figure from those counter runs, not something this run measures.  Returns (bytes, file)."""
+    name = "scan_select_%s_traffic.json" % workload_name
+    path = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(path):
-        return None
+        return None, None
     with open(path) as handle:
-        return json.load(handle).get("hbm_bytes_per_launch")
+        return json.load(handle).get("hbm_bytes_per_launch"), "profiles/" + name
+
+
+def host_description():
+    """CPU model, physical cores and hardware threads of this host (from /proc/cpuinfo)."""
+    model, cores, threads = "unknown", set(), 0
+    try:
+        physical = core = None
+        with open("/proc/cpuinfo") as handle:
+            for line in handle:
+                key, _, value = line.partition(":")
+                key, value = key.strip(), value.strip()
+                if key == "model name":
+                    model = value
+                elif key == "processor":
+                    threads += 1
+                elif key == "physical id":
+                    physical = value
+                elif key == "core id":
+                    core = value
+                elif not key and physical is not None and core is not None:
+                    cores.add((physical, core))
+                    physical = core = None
+    except OSError:
+        pass
+    return {"cpu_model": model, "physical_cores": len(cores) if cores else None, "hardware_threads": threads or os.cpu_count()}
+
+
+METRICS = {
+    "cfg1_plumbing": "sampled rows/sec + HBM GB/s (% peak), B=1 V=32000 fp32 temp+topk+topp",
+    "cfg2_topk_topp": "sampled rows/sec + HBM GB/s (% peak), B=64 V=151936 fp32 temp+topk+topp",
+    "cfg3_full_nucleus": "sampled rows/sec + HBM GB/s (% peak), B=256 V=201088 bf16 full-vocabulary nucleus top_p 0.95",
+    "cfg4_service_mix": "sampled rows/sec + HBM GB/s (% peak), B=512 V=129280 fp32 per-row mixed options + stop ids",
+    "cfg5_tie_stress": "sampled rows/sec + HBM GB/s (% peak), B=1024 V=262144 bf16 temp+topk+topp+minp, tie-heavy",
+}
 
 
 def cpu_baseline(workload, host_threads, sample_rows):
@@ -109,10 +145,14 @@ def cpu_baseline(workload, host_threads, sample_rows):
 
     single = best_of(1, 2)
     multi = best_of(host_threads, 3) if host_threads > 1 else single
+    host = host_description()
     return {
         "value": rows / multi,
         "unit": "rows/s",
         "cores": host_threads,
+        "cpu_model": host["cpu_model"],
+        "host_physical_cores": host["physical_cores"],
+        "host_hardware_threads": host["hardware_threads"],
         "kind": kind,
         "sample": "%d rows of the benchmark batch, best of 3 passes on %d threads (one Session per row); "
                   "1 thread: %.1f rows/s" % (rows, host_threads, rows / single),
@@ -324,6 +364,82 @@ def bench_generation_loop(args):
     print(json.dumps(line))
 
 
+def bench_timeline(args):
+    """Where the time of a split-row launch goes: the library built with wall-clock stamps in the split
+    kernel (make -C ncnn-moe-runtime_amd timeline) runs bursts of 12 launches over rotated logits buffers;
+    the stamps of every burst's last launch are read back.  Prints a table (text, not the JSON line): times
+    are microseconds after the launch's first workgroup entered the kernel."""
+    import torch
+    from ncnn_moe_runtime_amd import hip_sampler, workloads
+
+    library = os.path.join(PACKAGE_DIR, "libncnn_moe_hip_sampler_timeline.so")
+    if not os.path.exists(library):
+        sys.exit("%s is missing: build it with make -C %s timeline" % (library, PACKAGE_DIR))
+    hip_sampler.LIBRARY_PATH = library
+    lib = hip_sampler.load_library()
+    lib.ncnn_moe_hip_sampler_debug_timeline.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    lib.ncnn_moe_hip_sampler_debug_timeline_rows.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    names = ["entered", "logits arrived", "bound", "collected", "counted itself"]
+    merge_names = ["counted itself", "records read and checked", "cut and list", "result written"]
+    device = torch.device("cuda:0")
+    for rows in sorted({1, args.rows if args.rows > 0 else 64}):
+        workload = workloads.make_workload(args.workload, rows=rows)
+        vocab = workload["vocab"]
+        dtype_code = hip_sampler.LOGITS_F32 if workload["dtype"] == "f32" else hip_sampler.LOGITS_BF16
+        segments, chunks, variant = hip_sampler.select_geometry(dtype_code, rows, vocab)
+        if variant != hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK or rows > 64:
+            sys.exit("--timeline covers the split kernel (one-chunk workgroups) at up to 64 rows")
+        host = torch.from_numpy(workload["logits"].view(np.int16) if workload["dtype"] != "f32" else workload["logits"])
+        buffers = [host.to(device)]
+        for _ in range(8):
+            buffers.append(buffers[0][:, torch.randperm(vocab, device=device)].contiguous())
+        params = torch.from_numpy(workload["params"].view(np.uint8).reshape(rows, -1)).to(device)
+        uniforms = torch.from_numpy(workload["uniforms"]).to(device)
+        results = torch.zeros(rows * 16, dtype=torch.uint8, device=device)
+        stream = torch.cuda.current_stream()
+        segment_times, merge_times, fine_times, retries = [], [], [], []
+        with hip_sampler.HipSampler(rows, vocab) as sampler:
+            for burst in range(40):
+                for launch in range(12):
+                    sampler.sample_device(buffers[(burst * 12 + launch) % 9].data_ptr(), dtype_code, rows, vocab, vocab,
+                                          params.data_ptr(), uniforms.data_ptr(), None, results.data_ptr(), 0, stream.cuda_stream)
+                torch.cuda.synchronize()
+                if burst < 10:
+                    continue
+                stamps = np.zeros(64 * 16 * 16, dtype=np.uint64)
+                fine = np.zeros(64 * 16, dtype=np.uint64)
+                assert lib.ncnn_moe_hip_sampler_debug_timeline(stamps.ctypes.data, stamps.size) == 0
+                assert lib.ncnn_moe_hip_sampler_debug_timeline_rows(fine.ctypes.data, fine.size) == 0
+                t = stamps.reshape(64, 16, 16)[:rows, :segments].astype(np.int64)
+                start = t[:, :, 0].min()
+                relative = (t[:, :, :8] - start) / 100.0  # the clock ticks at 100 MHz
+                merger = relative[:, :, 7].argmax(axis=1)  # the stamps of an earlier launch's merge are older
+                merge = relative[np.arange(rows), merger]
+                segment_times.append(relative[:, :, :5])
+                merge_times.append(merge[:, 4:8])
+                epilogue = (fine.reshape(64, 16)[:rows, :7].astype(np.int64) - start) / 100.0
+                fine_times.append(np.concatenate([merge[:, 6:7], epilogue, merge[:, 7:8]], axis=1))
+                retries.append(t[np.arange(rows), merger, 8] - 1)
+        seg, mer, fin = np.stack(segment_times), np.stack(merge_times), np.stack(fine_times)
+        print("%s, %d rows x %d (%d workgroups per row), %d launches sampled: microseconds after the first workgroup entered" % (
+            args.workload, rows, vocab, segments, len(segment_times)))
+        for slot, name in enumerate(names):
+            v = seg[..., slot]
+            print("  every workgroup: %-26s min %6.2f  median %6.2f  p90 %6.2f  max %6.2f" % (name, v.min(), np.median(v), np.percentile(v, 90), v.max()))
+        for slot, name in enumerate(merge_names):
+            v = mer[..., slot]
+            print("  row's last workgroup: %-21s min %6.2f  median %6.2f  p90 %6.2f  max %6.2f" % (name, v.min(), np.median(v), np.percentile(v, 90), v.max()))
+        d, dm, df = np.diff(seg, axis=-1), np.diff(mer, axis=-1), np.diff(fin, axis=-1)
+        print("  phases of a workgroup (medians): wait for the logits %.2f | maxima + bound %.2f | collect %.2f | entries out + counter atomic %.2f" % tuple(
+            np.median(d[..., k]) for k in range(4)))
+        print("  phases of the merge (medians): read + check records %.2f | histogram cut + list %.2f | rank + epilogue %.2f" % tuple(
+            np.median(dm[..., k]) for k in range(3)))
+        print("  inside rank + epilogue (medians): rank %.2f | divide + expf %.2f | normaliser %.2f | divide + Min-P + Top-P %.2f | export %.2f | draw %.2f | "
+              "result store %.2f | exit %.2f" % tuple(np.median(df[..., k]) for k in range(8)))
+        print("  last result of a launch (median over launches) %.2f us; last logits of a launch %.2f us; re-reads of records per merge: mean %.2f" % (
+            np.median(mer[..., 3].max(axis=1)), np.median(seg[..., 1].reshape(len(segment_times), -1).max(axis=1)), np.concatenate(retries).mean()))
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -340,6 +456,9 @@ def main():
     parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
     parser.add_argument("--cpu-rows", type=int, default=64)
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--timeline", action="store_true",
+                        help="print where the time of a split-row launch goes (needs the stamped library: make timeline); "
+                             "a table, not the JSON line")
     parser.add_argument("--copy-calibration", type=int, default=0,
                         help="after the timed steps, copy a 256 MiB buffer this many times (a kernel of known "
                              "traffic for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -349,6 +468,9 @@ def main():
 
     load_package()
     from ncnn_moe_runtime_amd import hip_sampler, workloads
+    if args.timeline:
+        bench_timeline(args)
+        return
     if args.workload == "router_dispatch":
         bench_router_dispatch(args)
         return
@@ -406,10 +528,14 @@ def main():
 
     torch.cuda.synchronize()
     with torch.cuda.stream(stream):
-        # parity of the measured path on buffer 0 against the CPU oracle
-        step(0)
-        stream.synchronize()
-        gpu = results.cpu().numpy().view(hip_sampler.RESULT_DTYPE).reshape(rows)
+        # parity of the measured path against the CPU oracle on EVERY buffer that the timed steps rotate
+        # over (the oracle runs after the timed region, on host copies of the buffers)
+        gpu_per_buffer = []
+        for index in range(buffers):
+            step(index)
+            stream.synchronize()
+            gpu_per_buffer.append(results.cpu().numpy().view(hip_sampler.RESULT_DTYPE).reshape(rows).copy())
+        gpu = gpu_per_buffer[0]
         for index in range(args.warmup):
             step(index)
         stream.synchronize()
@@ -429,7 +555,7 @@ def main():
 
     # Beside the headline: the spread of single launches (one event pair per launch, which adds the
     # event's own cost to each) and the same loop on ONE buffer, which the 256 MB Infinity Cache holds.
-    detail_steps = min(args.steps, 200)
+    detail_steps = 200
     with torch.cuda.stream(stream):
         pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(detail_steps)]
         for index, (first, last) in enumerate(pairs):
@@ -450,6 +576,7 @@ def main():
     torch.cuda.synchronize()
     detail = {
         "single_launch_us_p10_median_p90": [float(np.percentile(single_launch_us, q)) for q in (10, 50, 90)],
+        "single_launches": detail_steps,
         "single_launch_note": "one HIP event pair per launch, %d launches; includes the events' own cost" % detail_steps,
         "cache_resident_ms_per_step": resident_start.elapsed_time(resident_stop) / detail_steps,
         "cache_resident_note": "same loop on one logits buffer (%.1f MB), held by the Infinity Cache where it fits; "
@@ -498,16 +625,35 @@ def main():
     import oracle_lib
     import parity_util
     host_threads = min(16, os.cpu_count() or 1)
-    cpu = oracle_lib.oracle_sample_batch(workload["logits"], workload["params"], workload["uniforms"],
-                                         workload["stop_ids"], threads=host_threads)
-    parity = parity_util.parity_counters(gpu, cpu)
-    parity["status_mismatches"] = int(np.count_nonzero(gpu["status"] != cpu["status"]))
-    parity["kept_count_mismatches"] = int(np.count_nonzero(gpu["kept_count"] != cpu["kept_count"]))
+    parity = None
+    for index in range(buffers):
+        host_buffer = workload["logits"] if index == 0 else logits[index].cpu().numpy().view(workload["logits"].dtype)
+        cpu = oracle_lib.oracle_sample_batch(host_buffer, workload["params"], workload["uniforms"],
+                                             workload["stop_ids"], threads=host_threads)
+        counters = parity_util.parity_counters(gpu_per_buffer[index], cpu)
+        counters["status_mismatches"] = int(np.count_nonzero(gpu_per_buffer[index]["status"] != cpu["status"]))
+        counters["kept_count_mismatches"] = int(np.count_nonzero(gpu_per_buffer[index]["kept_count"] != cpu["kept_count"]))
+        if parity is None:
+            parity = counters
+        else:
+            for key, value in counters.items():
+                parity[key] += value
+    parity["buffers_checked"] = buffers
 
     bytes_per_launch = algorithmic_bytes(rows, vocab, element_bytes)
     achieved = bytes_per_launch / seconds_per_step
+    traffic, traffic_file = measured_traffic(workload["name"]) if args.rows == 0 else (None, None)
+    segments, chunks, variant = hip_sampler.select_geometry(dtype_code, rows, vocab)
+    kernel = {hip_sampler.GEOMETRY_WHOLE_ROW: "scan_select_kernel (one workgroup per row)",
+              hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK: "split_select_kernel (%d one-chunk workgroups per row)" % segments,
+              hip_sampler.GEOMETRY_SPLIT_LOOPED: "scan_select_kernel (%d workgroups per row, %d chunks each)" % (segments, chunks)}[variant]
+    if may_need_full_order:
+        kernel += " + the later passes for rows without a Top-K window of at most 64 (wide select, sort, replay)"
+    metric = METRICS.get(workload["name"], "sampled rows/sec + HBM GB/s (% peak), " + workload["name"])
+    if args.rows > 0:
+        metric += " [rows overridden: %d]" % rows
     line = {
-        "metric": "sampled rows/sec + HBM GB/s (% peak), B=64 V=151936 fp32 temp+topk+topp",
+        "metric": metric,
         "value": rows / seconds_per_step,
         "unit": "rows/s",
         "n_gpus": 1,
@@ -534,8 +680,10 @@ def main():
             "peak": HBM_PEAK_BYTES_PER_S / 1e9,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_BYTES_PER_S,
-            "traffic": measured_traffic(workload["name"]) if args.rows == 0 else None,
-            "kernel": "scan_select_kernel",
+            "traffic": traffic,
+            "traffic_source": None if traffic is None else "stored from %s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
+                                                           "command, scaled by a copy kernel); not measured in this run" % traffic_file,
+            "kernel": kernel,
             "algorithmic_bytes_per_launch": bytes_per_launch,
         },
         "parity": parity,
