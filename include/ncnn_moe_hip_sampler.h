@@ -98,6 +98,7 @@ typedef struct ncnn_moe_sample_result
  * create() of the runtime's backend operators (src/backends/ncnn/ncnn_linear.h:45-71).  Allocates the
  * device logits buffer and every scratch buffer up front for max_rows x max_vocab, so that sampling
  * itself allocates nothing. */
+#define NCNN_MOE_SAMPLER_MAX_ROWS 65535 /* create() refuses more rows per handle */
 int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_vocab, ncnn_moe_hip_sampler** out);
 void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* sampler);
 
@@ -117,7 +118,8 @@ int ncnn_moe_hip_sampler_upload_logits(
 /* The batched form of Session::sample (include/ncnn/moe/session.h:326, src/engine/session.cpp:452-456)
  * over the handle's logits buffer: replaces the serial per-session loop of
  * examples/internal/run_model.cpp:776-809.  All pointers are host memory; the call returns when
- * results[] is filled.  uniforms[row] is the draw the row's Session RNG would produce next. */
+ * results[] is filled.  uniforms[row] is the draw the row's Session RNG would produce next.  At most
+ * max(64 * max_rows, max_vocab) stop ids per call (they are staged in memory sized by create()). */
 int ncnn_moe_hip_sampler_sample(
     ncnn_moe_hip_sampler* sampler, uint32_t rows,
     const ncnn_moe_sample_params* params, const float* uniforms,

@@ -42,8 +42,6 @@ struct ncnn_moe_hip_sampler
     ncnn_moe_sample_params* params = nullptr;
     float* uniforms = nullptr;
     ncnn_moe_sample_result* results = nullptr;
-    int32_t* stop_ids = nullptr;
-    uint32_t stop_capacity = 0;
     // the host entry's small operands are staged as one block of pinned memory, params | uniforms | stop ids,
     // that the kernels read in place; its results are written by the kernels straight into pinned memory
     uint8_t* input_block_host = nullptr; // pinned
@@ -74,8 +72,8 @@ struct ncnn_moe_hip_sampler
     int32_t* verify_ids = nullptr;
     float* verify_probabilities = nullptr;
     uint32_t* verify_counts = nullptr;
-    // speculative verification of filtered distributions longer than kVerifyCap: allocated by the first
-    // step that meets one (rows x max_vocab lists, two dense vectors over the vocabulary)
+    // speculative verification of filtered distributions longer than kVerifyCap: rows x max_vocab lists and
+    // two dense vectors over the vocabulary
     int32_t* verify_long_ids = nullptr;
     float* verify_long_probabilities = nullptr;
     float* verify_dense = nullptr;
@@ -449,8 +447,8 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     if (out == nullptr)
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     *out = nullptr;
-    if (max_rows == 0 || max_vocab == 0)
-        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    if (max_rows == 0 || max_vocab == 0 || max_rows > NCNN_MOE_SAMPLER_MAX_ROWS)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT; // the kernels put rows on a grid dimension
     int count = 0;
     if (hipGetDeviceCount(&count) != hipSuccess || count == 0)
         return NCNN_MOE_SAMPLER_NO_DEVICE;
@@ -492,11 +490,10 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->params, rows * sizeof(ncnn_moe_sample_params)));
     CREATE_CHECK(hipMalloc(&s->uniforms, rows * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->results, rows * sizeof(ncnn_moe_sample_result)));
-    s->stop_capacity = static_cast<uint32_t>(rows * 16);
-    CREATE_CHECK(hipMalloc(&s->stop_ids, static_cast<size_t>(s->stop_capacity) * sizeof(int32_t)));
     s->input_uniforms_offset = rows * sizeof(ncnn_moe_sample_params);
     s->input_stops_offset = s->input_uniforms_offset + rows * sizeof(float);
-    s->input_stop_capacity = static_cast<uint32_t>(rows * 16);
+    // room for stop ids: 64 per row, or one list as long as the vocabulary, whichever is more
+    s->input_stop_capacity = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(rows * 64, max_vocab), 1u << 28));
     const size_t input_bytes = s->input_stops_offset + static_cast<size_t>(s->input_stop_capacity) * sizeof(int32_t);
     CREATE_CHECK(hipHostMalloc(&s->input_block_host, input_bytes, hipHostMallocDefault));
     CREATE_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&s->input_block_mapped), s->input_block_host, 0));
@@ -530,6 +527,15 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->verify_ids, kVerifyRows * kVerifyCap * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->verify_probabilities, kVerifyRows * kVerifyCap * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->verify_counts, kVerifyRows * sizeof(uint32_t)));
+    // lists that hold whole rows and two dense vectors over the vocabulary, for steps whose filtered
+    // distributions are longer than kVerifyCap (a handle for fewer rows than a step needs never gets there)
+    if (max_rows >= 3)
+    {
+        const size_t long_rows = std::min<size_t>(kVerifyRows, rows);
+        CREATE_CHECK(hipMalloc(&s->verify_long_ids, long_rows * max_vocab * sizeof(int32_t)));
+        CREATE_CHECK(hipMalloc(&s->verify_long_probabilities, long_rows * max_vocab * sizeof(float)));
+        CREATE_CHECK(hipMalloc(&s->verify_dense, 2 * static_cast<size_t>(max_vocab) * sizeof(float)));
+    }
     CREATE_CHECK(hipHostMalloc(&s->verify_input_host, sizeof(ncnn_moe_hip_sampler::VerifyInput), hipHostMallocDefault));
     CREATE_CHECK(hipHostMalloc(&s->verify_output_host, sizeof(ncnn_moe_hip_sampler::VerifyOutput), hipHostMallocDefault));
     CREATE_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&s->verify_input_mapped), s->verify_input_host, 0));
@@ -563,7 +569,7 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
     if (s->side_join != nullptr)
         (void)hipEventDestroy(s->side_join);
     void* buffers[] = {
-        s->logits, s->params, s->uniforms, s->results, s->stop_ids, s->segment_values, s->segment_indices,
+        s->logits, s->params, s->uniforms, s->results, s->segment_values, s->segment_indices,
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->split_records, s->row_epoch, s->sort_keys[0], s->sort_keys[1],
         s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
@@ -637,6 +643,8 @@ int ncnn_moe_hip_sampler_sample(
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     if (rows == 0 || rows > s->logits_rows)
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "rows exceeds the rows of the logits buffer");
+    if (stop_id_count > 0 && stop_ids == nullptr)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "stop_id_count is positive and stop_ids is null");
     for (uint32_t row = 0; row < rows; ++row)
     {
         const uint64_t end = static_cast<uint64_t>(params[row].stop_begin) + params[row].stop_count;
@@ -654,8 +662,8 @@ int ncnn_moe_hip_sampler_sample(
     }
     SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
     // params, uniforms and stop ids are staged in one pinned block that the kernels read in place (a few
-    // dozen bytes per workgroup over the host link, behind the first logits loads); stop-id lists beyond
-    // the block's room take the handle's growable device buffer
+    // dozen bytes per workgroup over the host link, behind the first logits loads); the block has room for
+    // max(64 * max_rows, max_vocab) stop ids, and a call with more is refused (nothing is allocated here)
     const ncnn_moe_sample_params* device_params = reinterpret_cast<const ncnn_moe_sample_params*>(s->input_block_mapped);
     const float* device_uniforms = reinterpret_cast<const float*>(s->input_block_mapped + s->input_uniforms_offset);
     const int32_t* device_stops = nullptr;
@@ -667,19 +675,7 @@ int ncnn_moe_hip_sampler_sample(
         device_stops = reinterpret_cast<const int32_t*>(s->input_block_mapped + s->input_stops_offset);
     }
     else if (stop_id_count > 0)
-    {
-        if (stop_id_count > s->stop_capacity)
-        {
-            SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
-            SAMPLER_HIP_CHECK(s, hipFree(s->stop_ids));
-            s->stop_ids = nullptr;
-            s->stop_capacity = 0;
-            SAMPLER_HIP_CHECK(s, hipMalloc(&s->stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t)));
-            s->stop_capacity = stop_id_count;
-        }
-        SAMPLER_HIP_CHECK(s, hipMemcpyAsync(s->stop_ids, stop_ids, static_cast<size_t>(stop_id_count) * sizeof(int32_t), hipMemcpyHostToDevice, s->stream));
-        device_stops = s->stop_ids;
-    }
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "more stop ids than the handle holds (max(64 * max_rows, max_vocab))");
     // the host sees the options: the later passes are enqueued only if some row needs them
     SamplerPasses passes;
     passes.full_order = s->force_general != 0;
@@ -743,6 +739,7 @@ int ncnn_moe_hip_sampler_sample_device(
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab must be positive");
     if (row_stride < vocab)
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "row_stride is smaller than vocab");
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
     SamplerPasses passes;
     passes.wide_select = may_need_full_order != 0;
     passes.full_order = may_need_full_order != 0 || s->force_general != 0;
@@ -962,13 +959,6 @@ int ncnn_moe_hip_sampler_speculative_verify(
     {
         // A filtered distribution longer than the lists above: the step is run (again) with lists that
         // hold a whole row each and the kernel that builds the residual as a dense vector.
-        if (s->verify_long_ids == nullptr)
-        {
-            const size_t entries = static_cast<size_t>(2 * NCNN_MOE_MAX_DRAFT_TOKENS + 1) * s->max_vocab;
-            SAMPLER_HIP_CHECK(s, hipMalloc(&s->verify_long_ids, entries * sizeof(int32_t)));
-            SAMPLER_HIP_CHECK(s, hipMalloc(&s->verify_long_probabilities, entries * sizeof(float)));
-            SAMPLER_HIP_CHECK(s, hipMalloc(&s->verify_dense, 2 * static_cast<size_t>(s->max_vocab) * sizeof(float)));
-        }
         export_to.ids = s->verify_long_ids;
         export_to.probabilities = s->verify_long_probabilities;
         export_to.cap = s->logits_vocab;

@@ -4,8 +4,13 @@
 #include "ncnn_moe_hip_sampler.h"
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cmath>
+#include <condition_variable>
+#include <deque>
+#include <thread>
+#include <unordered_map>
 
 namespace ncnn {
 namespace moe {
@@ -83,6 +88,11 @@ Result<bool> validate_sampling_options(const SamplingOptions& options)
     if (!std::isfinite(options.min_p) || options.min_p < 0.0f || options.min_p > 1.0f)
         return invalid_argument("min_p must be in the range [0, 1]");
     return true;
+}
+
+uint32_t hip_sampler_capabilities()
+{
+    return ncnn_moe_hip_sampler_device_count() > 0 ? static_cast<uint32_t>(RuntimeCapabilityHipSampler) : 0u;
 }
 
 float peek_uniform(const std::mt19937_64& generator, std::mt19937_64& advanced)
@@ -296,9 +306,12 @@ Result<SpeculativeVerification> HipSampler::verify_speculative(
     std::span<const int32_t> proposed_token_ids,
     const SamplingOptions& options,
     std::span<const float> uniforms,
-    uint32_t& draws_consumed)
+    uint32_t& draws_consumed,
+    uint32_t* accept_draws)
 {
     draws_consumed = 0;
+    if (accept_draws != nullptr)
+        *accept_draws = 0;
     const size_t drafts = proposed_token_ids.size();
     if (drafts == 0 || drafts > NCNN_MOE_MAX_DRAFT_TOKENS)
         return invalid_argument("speculative verification takes 1 to 16 proposed tokens");
@@ -343,6 +356,8 @@ Result<SpeculativeVerification> HipSampler::verify_speculative(
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return error_of_call(rc, impl.handle);
     draws_consumed = verified.accept_draws + verified.final_draw_consumed;
+    if (accept_draws != nullptr)
+        *accept_draws = verified.accept_draws;
     switch (verified.status)
     {
     case NCNN_MOE_VERIFY_OK:
@@ -364,8 +379,18 @@ Result<SpeculativeVerification> HipSampler::verify_speculative(
 }
 
 SamplingSession::SamplingSession(HipSamplerPtr sampler, const SamplingSessionOptions& options)
-    : sampler_(std::move(sampler)), random_generator_(options.sampling_seed)
+    : sampler_(std::move(sampler)), logits_output_mode_(options.logits_output_mode), random_generator_(options.sampling_seed)
 {
+}
+
+Result<SamplingSessionPtr> create_sampling_session(const HipSamplerPtr& sampler, const SamplingSessionOptions& options)
+{
+    // src/engine/runtime.cpp:575-582 accepts FullLogits only; the device sampler adds SampledToken
+    if (options.logits_output_mode == LogitsOutputMode::SampledToken && !sampler)
+        return Error{ErrorCode::UnsupportedModel, "the current executor supports full logits output only"};
+    if (options.logits_output_mode == LogitsOutputMode::TopKCandidates)
+        return Error{ErrorCode::UnsupportedModel, "the current executor supports full logits and sampled token output only"};
+    return std::make_shared<SamplingSession>(sampler, options);
 }
 
 float SamplingSession::uniform_ahead(size_t position)
@@ -386,6 +411,8 @@ void SamplingSession::consume_uniforms(size_t count)
 Result<SampledToken> SamplingSession::sample(const LogitsOutput& logits, const SamplingOptions& options)
 {
     const std::lock_guard<std::mutex> lock(mutex_);
+    if (logits_output_mode_ != LogitsOutputMode::FullLogits)
+        return invalid_argument("session output mode is SampledToken: its logits stay in device memory");
     if (logits.values.empty())
         return invalid_argument("cannot sample empty logits");
     if (!sampler_)
@@ -415,6 +442,13 @@ Result<SpeculativeVerification> SamplingSession::verify_speculative(
     std::span<const LogitsOutput> target_logits, std::span<const LogitsOutput> draft_logits,
     std::span<const int32_t> proposed_token_ids, const SamplingOptions& options)
 {
+    return verify_speculative(target_logits, draft_logits, proposed_token_ids, options, true);
+}
+
+Result<SpeculativeVerification> SamplingSession::verify_speculative(
+    std::span<const LogitsOutput> target_logits, std::span<const LogitsOutput> draft_logits,
+    std::span<const int32_t> proposed_token_ids, const SamplingOptions& options, bool state_cache_transactions)
+{
     const std::lock_guard<std::mutex> lock(mutex_);
     if (!sampler_)
         return Error{ErrorCode::InternalError, "hip sampler is unavailable (no GPU, or create() failed)"};
@@ -428,7 +462,18 @@ Result<SpeculativeVerification> SamplingSession::verify_speculative(
     for (size_t i = 0; i < uniforms.size(); ++i)
         uniforms[i] = uniform_ahead(i);
     uint32_t draws_consumed = 0;
-    auto verified = sampler_->verify_speculative(target_rows, draft_rows, proposed_token_ids, options, uniforms, draws_consumed);
+    uint32_t accept_draws = 0;
+    auto verified = sampler_->verify_speculative(target_rows, draft_rows, proposed_token_ids, options, uniforms, draws_consumed, &accept_draws);
+    if (verified && verified.value().accepted.empty() && !state_cache_transactions)
+    {
+        // src/engine/session.cpp:843-857: nothing accepted and no cache transactions to keep part of the
+        // step: roll back and leave speculative mode before the next token is drawn.  The device computed
+        // that token as well; it is dropped and its draw stays unconsumed.
+        consume_uniforms(accept_draws);
+        SpeculativeVerification fallen_back;
+        fallen_back.fell_back = true;
+        return fallen_back;
+    }
     consume_uniforms(draws_consumed);
     return verified;
 }
@@ -452,6 +497,11 @@ std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample(
     std::sort(ordered.begin(), ordered.end());
     if (std::adjacent_find(ordered.begin(), ordered.end()) != ordered.end())
         return every_row<BatchSampledToken>(rows, invalid_argument("sample batch contains duplicate sessions"));
+    for (const SampleBatchRequest& request : requests)
+    {
+        if (request.session->logits_output_mode_ != LogitsOutputMode::FullLogits)
+            return every_row<BatchSampledToken>(rows, invalid_argument("session output mode is SampledToken: its logits stay in device memory"));
+    }
     std::vector<std::unique_lock<std::mutex>> locks;
     locks.reserve(rows);
     for (SamplingSession* session : ordered)
@@ -488,6 +538,342 @@ std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample(
             requests[i].session->consume_uniforms(1);
     }
     return out;
+}
+
+std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample_resident(
+    const HipSamplerPtr& sampler, std::span<const SampleBatchRequest> requests)
+{
+    const size_t rows = requests.size();
+    if (rows == 0)
+        return {};
+    if (!sampler)
+        return every_row<BatchSampledToken>(rows, Error{ErrorCode::InternalError, "hip sampler is unavailable (no GPU, or create() failed)"});
+    std::vector<std::pair<const void*, std::mutex*>> order;
+    for (const SampleBatchRequest& request : requests)
+    {
+        if (request.session == nullptr)
+            return every_row<BatchSampledToken>(rows, invalid_argument("sample batch contains a null session or logits"));
+        if (request.logits != nullptr || request.session->logits_output_mode_ != LogitsOutputMode::SampledToken)
+            return every_row<BatchSampledToken>(rows, invalid_argument("session output mode is FullLogits: pass its logits to sample()"));
+        order.emplace_back(request.session, &request.session->mutex_);
+    }
+    std::vector<std::unique_lock<std::mutex>> locks;
+    if (!lock_in_pointer_order(std::move(order), locks))
+        return every_row<BatchSampledToken>(rows, invalid_argument("sample batch contains duplicate sessions"));
+    std::vector<SamplingOptions> options;
+    std::vector<float> uniforms;
+    std::vector<std::vector<int32_t>> stop_tokens;
+    for (const SampleBatchRequest& request : requests)
+    {
+        options.push_back(request.sampling);
+        uniforms.push_back(request.session->uniform_ahead(0));
+        stop_tokens.push_back(request.stop_tokens);
+    }
+    std::vector<uint8_t> draw_consumed;
+    const SampleTimer timer;
+    auto sampled = sampler->sample_resident(options, uniforms, stop_tokens, draw_consumed);
+    for (size_t i = 0; i < rows; ++i)
+    {
+        timer.charge(requests[i].session->statistics_, sampled[i] ? 1 : 0);
+        if (sampled[i] && draw_consumed[i])
+            requests[i].session->consume_uniforms(1);
+    }
+    return sampled;
+}
+
+// ---- BatchSampleScheduler -----------------------------------------------------------------------------------
+
+class BatchSampleScheduler::Implementation
+{
+public:
+    using Results = std::vector<Result<BatchSampledToken>>;
+
+    Implementation(HipSamplerPtr sampler, const SampleSchedulerOptions& options)
+        : sampler_(std::move(sampler)), window_(options.cross_call_window_microseconds)
+    {
+        const uint32_t hardware_threads = std::max(1u, std::thread::hardware_concurrency());
+        worker_count_ = options.worker_count == 0 ? std::min(4u, hardware_threads) : std::min(options.worker_count, 1024u);
+        max_collected_ = options.cross_call_max_batch_size != 0 ? options.cross_call_max_batch_size
+                                                                : (sampler_ ? sampler_->max_rows() : 1u);
+        for (uint32_t i = 0; i < worker_count_; ++i)
+            workers_.emplace_back([this] { worker_loop(); });
+        if (window_ != 0)
+            collector_ = std::thread([this] { collector_loop(); });
+    }
+
+    ~Implementation()
+    {
+        {
+            const std::lock_guard<std::mutex> lock(mutex_);
+            stopping_ = true;
+        }
+        work_ready_.notify_all();
+        single_ready_.notify_all();
+        if (collector_.joinable())
+            collector_.join();
+        for (std::thread& worker : workers_)
+            worker.join();
+    }
+
+    std::future<Results> submit(std::vector<SampleBatchRequest> requests)
+    {
+        submitted_batches_.fetch_add(1, std::memory_order_relaxed);
+        submitted_requests_.fetch_add(requests.size(), std::memory_order_relaxed);
+        update_max(max_batch_size_, requests.size());
+        std::promise<Results> promise;
+        std::future<Results> future = promise.get_future();
+        const auto reject = [&](const char* message) {
+            rejected_requests_.fetch_add(requests.size(), std::memory_order_relaxed);
+            promise.set_value(every_row<BatchSampledToken>(requests.size(), invalid_argument(message)));
+            return std::move(future);
+        };
+        if (requests.empty())
+        {
+            promise.set_value({});
+            return future;
+        }
+        std::vector<const SamplingSession*> named;
+        for (const SampleBatchRequest& request : requests)
+        {
+            if (request.session == nullptr)
+                return reject("sample batch contains a null session or logits");
+            named.push_back(request.session);
+        }
+        std::sort(named.begin(), named.end());
+        if (std::adjacent_find(named.begin(), named.end()) != named.end())
+            return reject("sample batch contains duplicate sessions");
+        {
+            const std::lock_guard<std::mutex> lock(mutex_);
+            // the place of every request in its Session's order is fixed here, whichever way it travels
+            std::vector<uint64_t> tickets;
+            for (const SampleBatchRequest& request : requests)
+            {
+                std::deque<uint64_t>& order = session_order_[request.session];
+                if (!order.empty())
+                    serialized_session_requests_.fetch_add(1, std::memory_order_relaxed);
+                order.push_back(next_ticket_);
+                tickets.push_back(next_ticket_++);
+            }
+            if (requests.size() == 1 && collector_.joinable())
+            {
+                singles_.push_back(Single{std::move(requests.front()), tickets.front(), std::move(promise), std::chrono::steady_clock::now()});
+                single_ready_.notify_one();
+                return future;
+            }
+            queue_.push_back(Batch{std::move(requests), std::move(tickets), {}, std::move(promise)});
+        }
+        work_ready_.notify_one();
+        return future;
+    }
+
+    SampleSchedulerStatistics statistics() const noexcept
+    {
+        SampleSchedulerStatistics out;
+        out.submitted_batches = submitted_batches_.load(std::memory_order_relaxed);
+        out.submitted_requests = submitted_requests_.load(std::memory_order_relaxed);
+        out.completed_requests = completed_requests_.load(std::memory_order_relaxed);
+        out.rejected_requests = rejected_requests_.load(std::memory_order_relaxed);
+        out.max_batch_size = max_batch_size_.load(std::memory_order_relaxed);
+        out.serialized_session_requests = serialized_session_requests_.load(std::memory_order_relaxed);
+        out.cross_call_collected_batches = collected_batches_.load(std::memory_order_relaxed);
+        out.cross_call_collected_requests = collected_requests_.load(std::memory_order_relaxed);
+        out.cross_call_collection_timeouts = collection_timeouts_.load(std::memory_order_relaxed);
+        out.device_calls = device_calls_.load(std::memory_order_relaxed);
+        out.worker_count = worker_count_;
+        return out;
+    }
+
+private:
+    struct Single
+    {
+        SampleBatchRequest request;
+        uint64_t ticket = 0;
+        std::promise<Results> promise;
+        std::chrono::steady_clock::time_point submitted_at;
+    };
+
+    // One device call's worth of requests.  A collected batch answers one promise per request.
+    struct Batch
+    {
+        std::vector<SampleBatchRequest> requests;
+        std::vector<uint64_t> tickets; // one per request: its place in its Session's order
+        std::vector<std::promise<Results>> single_promises;
+        std::promise<Results> promise;
+    };
+
+    static void update_max(std::atomic<uint64_t>& slot, uint64_t value)
+    {
+        uint64_t seen = slot.load(std::memory_order_relaxed);
+        while (seen < value && !slot.compare_exchange_weak(seen, value, std::memory_order_relaxed))
+        {
+        }
+    }
+
+    // mutex_ held.  The first batch every request of which is the oldest unfinished one of its Session:
+    // requests of a Session run in the order of their submission and never two at a time.  (A batch waits
+    // only for requests with smaller tickets, so some batch can always run.)
+    bool take_runnable_locked(Batch& out)
+    {
+        for (auto batch = queue_.begin(); batch != queue_.end(); ++batch)
+        {
+            bool runnable = true;
+            for (size_t i = 0; i < batch->requests.size() && runnable; ++i)
+                runnable = session_order_[batch->requests[i].session].front() == batch->tickets[i];
+            if (runnable)
+            {
+                out = std::move(*batch);
+                queue_.erase(batch);
+                return true;
+            }
+        }
+        return false;
+    }
+
+    void worker_loop()
+    {
+        for (;;)
+        {
+            Batch batch;
+            {
+                std::unique_lock<std::mutex> lock(mutex_);
+                work_ready_.wait(lock, [&] { return take_runnable_locked(batch) || (stopping_ && queue_.empty() && singles_.empty() && !collecting_); });
+                if (batch.requests.empty())
+                    return;
+            }
+            Results results;
+            try
+            {
+                const bool resident = batch.requests.front().logits == nullptr;
+                results = resident ? SessionBatchSampler::sample_resident(sampler_, batch.requests)
+                                   : SessionBatchSampler::sample(sampler_, batch.requests);
+                device_calls_.fetch_add(1, std::memory_order_relaxed);
+            }
+            catch (const std::exception& error)
+            {
+                results = every_row<BatchSampledToken>(batch.requests.size(), Error{ErrorCode::InternalError, std::string("sample batch failed: ") + error.what()});
+            }
+            completed_requests_.fetch_add(batch.requests.size(), std::memory_order_relaxed);
+            {
+                const std::lock_guard<std::mutex> lock(mutex_);
+                for (const SampleBatchRequest& request : batch.requests)
+                {
+                    auto order = session_order_.find(request.session);
+                    order->second.pop_front(); // this request was the Session's oldest
+                    if (order->second.empty())
+                        session_order_.erase(order);
+                }
+            }
+            work_ready_.notify_all(); // a batch that waited for one of these Sessions may run now
+            if (batch.single_promises.empty())
+                batch.promise.set_value(std::move(results));
+            else
+            {
+                for (size_t i = 0; i < batch.single_promises.size(); ++i)
+                {
+                    Results one;
+                    one.push_back(std::move(results[i]));
+                    batch.single_promises[i].set_value(std::move(one));
+                }
+            }
+        }
+    }
+
+    // Gathers single-request submissions: waits, from the oldest one's submission, up to the window for a
+    // request of another Session to come in, then takes one request per Session, oldest first, into a batch.
+    void collector_loop()
+    {
+        for (;;)
+        {
+            Batch batch;
+            {
+                std::unique_lock<std::mutex> lock(mutex_);
+                single_ready_.wait(lock, [&] { return stopping_ || !singles_.empty(); });
+                if (singles_.empty())
+                    return;
+                collecting_ = true;
+                const auto distinct_sessions = [&] {
+                    std::vector<const SamplingSession*> seen;
+                    for (const Single& single : singles_)
+                    {
+                        if (std::find(seen.begin(), seen.end(), single.request.session) == seen.end())
+                            seen.push_back(single.request.session);
+                    }
+                    return seen.size();
+                };
+                const auto deadline = singles_.front().submitted_at + std::chrono::microseconds(window_);
+                size_t seen_before = distinct_sessions();
+                // every new Session extends nothing: the window runs from the oldest submission
+                while (!stopping_ && seen_before < max_collected_ && std::chrono::steady_clock::now() < deadline)
+                {
+                    single_ready_.wait_until(lock, deadline);
+                    seen_before = distinct_sessions();
+                }
+                std::vector<const SamplingSession*> taken;
+                for (auto single = singles_.begin(); single != singles_.end() && batch.requests.size() < max_collected_;)
+                {
+                    const bool resident = single->request.logits == nullptr;
+                    const bool same_kind = batch.requests.empty() || resident == (batch.requests.front().logits == nullptr);
+                    if (!same_kind || std::find(taken.begin(), taken.end(), single->request.session) != taken.end())
+                    {
+                        ++single;
+                        continue;
+                    }
+                    taken.push_back(single->request.session);
+                    batch.tickets.push_back(single->ticket);
+                    batch.requests.push_back(std::move(single->request));
+                    batch.single_promises.push_back(std::move(single->promise));
+                    single = singles_.erase(single);
+                }
+                if (batch.requests.size() > 1)
+                {
+                    collected_batches_.fetch_add(1, std::memory_order_relaxed);
+                    collected_requests_.fetch_add(batch.requests.size(), std::memory_order_relaxed);
+                    update_max(max_batch_size_, batch.requests.size());
+                }
+                else
+                    collection_timeouts_.fetch_add(1, std::memory_order_relaxed);
+                queue_.push_back(std::move(batch));
+                collecting_ = !singles_.empty();
+            }
+            work_ready_.notify_one();
+        }
+    }
+
+    HipSamplerPtr sampler_;
+    uint32_t window_ = 0;
+    uint32_t worker_count_ = 1;
+    size_t max_collected_ = 1;
+    std::vector<std::thread> workers_;
+    std::thread collector_;
+    mutable std::mutex mutex_;
+    std::condition_variable work_ready_;
+    std::condition_variable single_ready_;
+    std::deque<Batch> queue_;
+    std::deque<Single> singles_;
+    std::unordered_map<const SamplingSession*, std::deque<uint64_t>> session_order_; // unfinished requests, oldest first
+    uint64_t next_ticket_ = 1;
+    bool stopping_ = false;
+    bool collecting_ = false;
+    std::atomic<uint64_t> submitted_batches_{0}, submitted_requests_{0}, completed_requests_{0}, rejected_requests_{0};
+    std::atomic<uint64_t> max_batch_size_{0}, serialized_session_requests_{0}, collected_batches_{0}, collected_requests_{0};
+    std::atomic<uint64_t> collection_timeouts_{0}, device_calls_{0};
+};
+
+BatchSampleScheduler::BatchSampleScheduler(HipSamplerPtr sampler, const SampleSchedulerOptions& options)
+    : implementation_(std::make_unique<Implementation>(std::move(sampler), options))
+{
+}
+
+BatchSampleScheduler::~BatchSampleScheduler() = default;
+
+std::future<std::vector<Result<BatchSampledToken>>> BatchSampleScheduler::submit_sample(std::vector<SampleBatchRequest> requests)
+{
+    return implementation_->submit(std::move(requests));
+}
+
+SampleSchedulerStatistics BatchSampleScheduler::statistics() const noexcept
+{
+    return implementation_->statistics();
 }
 
 Result<std::vector<GenerationResult>> BatchGenerationLoop::generate(
@@ -558,12 +944,17 @@ Result<std::vector<GenerationResult>> BatchGenerationLoop::generate(
         auto sampled = sampler->sample_resident(row_options, uniforms, stop_tokens, draw_consumed);
         slots.clear();
         next_active.clear();
+        // a row that failed fails the call before anything of this step is committed: no draw is taken
+        // from a generator, no callback runs and no token is appended for the Sessions in front of it
+        for (size_t row = 0; row < active.size(); ++row)
+        {
+            if (!sampled[row])
+                return sampled[row].error();
+        }
         for (size_t row = 0; row < active.size(); ++row)
         {
             const uint32_t i = active[row];
-            timer.charge(sessions[i]->statistics_, sampled[row] ? 1 : 0);
-            if (!sampled[row])
-                return sampled[row].error();
+            timer.charge(sessions[i]->statistics_, 1);
             if (draw_consumed[row])
                 sessions[i]->consume_uniforms(1);
             StreamToken token;

@@ -14,6 +14,10 @@
 //       rejects duplicates (src/engine/session.cpp:1249-1265), draws one uniform per row from a COPY
 //       of each Session's generator, samples every row in one device call, and commits the copy back
 //       only for rows whose draw was consumed (session.cpp:429-433).
+//   BatchSampleScheduler the batched-sample hand-off of the batch scheduler: submit_sample() beside
+//       BatchScheduler::submit_decode (include/ncnn/moe/scheduler.h:122-123), with the scheduler's worker
+//       threads, per-Session order and cross-call collection (src/engine/scheduler.cpp:87-104, :416-437,
+//       :975-1096, :1104-1138), so that callers that each sample one row share one device call.
 //   BatchGenerationLoop  the scheduler-driven generation loop of examples/internal/run_model.cpp:726-847
 //       over device-resident logits: an IDeviceLogitsSource (the model's prefill / decode) writes
 //       each step's logits into the sampler's buffer and one device call samples every active Session.
@@ -25,6 +29,7 @@
 
 #include <cstdint>
 #include <functional>
+#include <future>
 #include <memory>
 #include <mutex>
 #include <random>
@@ -74,6 +79,14 @@ private:
 struct LogitsOutput
 {
     std::vector<float> values;
+};
+
+// include/ncnn/moe/types.h:304-309
+enum class LogitsOutputMode
+{
+    FullLogits,
+    TopKCandidates,
+    SampledToken
 };
 
 struct SamplingOptions
@@ -145,7 +158,21 @@ struct SpeculativeVerification
     std::vector<SampledToken> accepted; // the proposed tokens that stand, each with its reported probability
     SampledToken next;                  // the token emitted after them (residual draw, or the target's own sample)
     bool next_from_residual = false;
+    // Nothing was accepted and the caller's state keeps no cache transactions: the step is rolled back and
+    // speculative mode left before `next` is drawn (src/engine/session.cpp:843-857); `next` is not set and
+    // only the accept test's draw was consumed.
+    bool fell_back = false;
 };
+
+// The capability bit a runtime with this backend reports beside RuntimeCapabilityFlag
+// (include/ncnn/moe/runtime.h:40-59; bits 0-17 are taken there).
+#define NCNN_MOE_RUNTIME_CAP_HIP_SAMPLER_BIT 18
+enum : uint32_t
+{
+    RuntimeCapabilityHipSampler = UINT32_C(1) << NCNN_MOE_RUNTIME_CAP_HIP_SAMPLER_BIT
+};
+// RuntimeCapabilityHipSampler if a HIP device is usable, else 0 (what Runtime::capabilities() would OR in).
+uint32_t hip_sampler_capabilities();
 
 // Rows of logits in device memory: row i starts at data + i * row_stride elements.
 struct DeviceLogitsRows
@@ -206,7 +233,8 @@ public:
         std::span<const int32_t> proposed_token_ids,
         const SamplingOptions& options,
         std::span<const float> uniforms,
-        uint32_t& draws_consumed);
+        uint32_t& draws_consumed,
+        uint32_t* accept_draws = nullptr); // of draws_consumed, those of the accept tests (the rest is the last token's draw)
 
 private:
     HipSampler();
@@ -229,6 +257,10 @@ struct SamplingStatistics
 struct SamplingSessionOptions
 {
     uint64_t sampling_seed = 0; // SessionOptions::sampling_seed, include/ncnn/moe/session.h:280-286
+    // SessionOptions::logits_output_mode.  FullLogits: the Session's logits are host vectors (LogitsOutput).
+    // SampledToken: they stay in the sampler's device buffer and only tokens come back; such a Session
+    // is sampled through SessionBatchSampler::sample_resident, BatchSampleScheduler or BatchGenerationLoop.
+    LogitsOutputMode logits_output_mode = LogitsOutputMode::FullLogits;
 };
 
 class SamplingSession
@@ -245,13 +277,21 @@ public:
         std::span<const LogitsOutput> target_logits, std::span<const LogitsOutput> draft_logits,
         std::span<const int32_t> proposed_token_ids, const SamplingOptions& options = {});
 
+    // state_cache_transactions = false: the model state cannot roll back part of a step, so a step in which
+    // nothing is accepted falls back (SpeculativeVerification::fell_back) before the next token is drawn.
+    [[nodiscard]] Result<SpeculativeVerification> verify_speculative(
+        std::span<const LogitsOutput> target_logits, std::span<const LogitsOutput> draft_logits,
+        std::span<const int32_t> proposed_token_ids, const SamplingOptions& options, bool state_cache_transactions);
+
     // Session::statistics(), the sampling share.
     [[nodiscard]] SamplingStatistics statistics() const;
+    [[nodiscard]] LogitsOutputMode logits_output_mode() const noexcept { return logits_output_mode_; }
 
 private:
     friend class SessionBatchSampler;
     friend class BatchGenerationLoop;
     HipSamplerPtr sampler_;
+    LogitsOutputMode logits_output_mode_ = LogitsOutputMode::FullLogits;
     // The uniform the sampler would draw `position` draws from now, without consuming it, and the
     // consumption of the next `count` of them.  A draw that was looked at but not consumed (a greedy
     // call, Top-K 1, an error: src/engine/session.cpp:404, :425-433) stays at the head of
@@ -268,10 +308,17 @@ private:
     mutable std::mutex mutex_;
 };
 
+using SamplingSessionPtr = std::shared_ptr<SamplingSession>;
+
+// Runtime::create_session for the sampling slice (src/engine/runtime.cpp:575-582): with a HIP sampler the
+// Session may be created in SampledToken mode, which the CPU executor refuses; TopKCandidates stays
+// unsupported, and without a sampler only FullLogits is accepted, with the runtime's own message.
+Result<SamplingSessionPtr> create_sampling_session(const HipSamplerPtr& sampler, const SamplingSessionOptions& options = {});
+
 struct SampleBatchRequest
 {
     SamplingSession* session = nullptr;
-    const LogitsOutput* logits = nullptr;
+    const LogitsOutput* logits = nullptr; // null for a Session in SampledToken mode: its row is in the device buffer
     SamplingOptions sampling;
     std::vector<int32_t> stop_tokens; // GenerationOptions::stop_tokens
 };
@@ -283,6 +330,56 @@ public:
     // examples/internal/run_model.cpp:776-809.  Rejects empty batches, null or duplicate Sessions and
     // rows of different lengths with InvalidArgument for every row.
     static std::vector<Result<BatchSampledToken>> sample(const HipSamplerPtr& sampler, std::span<const SampleBatchRequest> requests);
+
+    // The same for Sessions in SampledToken mode: request i samples row i of the rows last laid out by
+    // HipSampler::device_logits (the decode step wrote them there); every request's logits must be null.
+    static std::vector<Result<BatchSampledToken>> sample_resident(const HipSamplerPtr& sampler, std::span<const SampleBatchRequest> requests);
+};
+
+// BatchScheduler's options and counters, as far as sampling uses them (include/ncnn/moe/scheduler.h:41-109).
+struct SampleSchedulerOptions
+{
+    uint32_t worker_count = 0;                     // 0: min(4, hardware threads), src/engine/scheduler.cpp:87
+    uint32_t cross_call_window_microseconds = 200; // zero disables cross-call collection
+    uint32_t cross_call_max_batch_size = 0;        // 0: the sampler's max_rows
+};
+
+struct SampleSchedulerStatistics
+{
+    uint64_t submitted_batches = 0;
+    uint64_t submitted_requests = 0;
+    uint64_t completed_requests = 0;
+    uint64_t rejected_requests = 0;
+    uint64_t max_batch_size = 0;
+    uint64_t serialized_session_requests = 0; // requests that waited for an earlier one of their Session
+    uint64_t cross_call_collected_batches = 0;
+    uint64_t cross_call_collected_requests = 0;
+    uint64_t cross_call_collection_timeouts = 0;
+    uint64_t device_calls = 0;
+    uint32_t worker_count = 0;
+};
+
+// The batched-sample entry of the batch scheduler.  submit_sample() returns at once; worker threads run
+// the batches, each as ONE device call (SessionBatchSampler::sample).  Requests of one Session run in
+// the order they were submitted and never two at a time; a batch that names a Session twice is rejected
+// (src/engine/session.cpp:1257-1265).  Submissions of a single request, the shape of a serving loop with one
+// thread per Session, are collected across calls for up to cross_call_window_microseconds and sampled
+// together, one request per Session and batch.  The Sessions and logits a request points to must stay
+// alive until its future is ready.
+class BatchSampleScheduler
+{
+public:
+    explicit BatchSampleScheduler(HipSamplerPtr sampler, const SampleSchedulerOptions& options = {});
+    ~BatchSampleScheduler();
+    BatchSampleScheduler(const BatchSampleScheduler&) = delete;
+    BatchSampleScheduler& operator=(const BatchSampleScheduler&) = delete;
+
+    [[nodiscard]] std::future<std::vector<Result<BatchSampledToken>>> submit_sample(std::vector<SampleBatchRequest> requests);
+    [[nodiscard]] SampleSchedulerStatistics statistics() const noexcept;
+
+private:
+    class Implementation;
+    std::unique_ptr<Implementation> implementation_;
 };
 
 // One row of a decode step: DecodeBatchRequest of the batch scheduler ({session, token}).

@@ -23,6 +23,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <deque>
+#include <future>
 #include <limits>
 #include <random>
 #include <stdexcept>
@@ -515,6 +516,250 @@ static void test_speculative_verification(const HipSamplerPtr& sampler)
     }
 }
 
+// ---- the scheduler's batched-sample entry, output modes, capability bit ---------------------------
+
+static void test_scheduler_and_modes_without_a_sampler()
+{
+    // Runtime::create_session (src/engine/runtime.cpp:575-582): without the device sampler only full logits
+    auto full = create_sampling_session(nullptr, SamplingSessionOptions{3, LogitsOutputMode::FullLogits});
+    check(static_cast<bool>(full) && full.value()->logits_output_mode() == LogitsOutputMode::FullLogits);
+    auto sampled_only = create_sampling_session(nullptr, SamplingSessionOptions{3, LogitsOutputMode::SampledToken});
+    check(!sampled_only && sampled_only.error().code == ErrorCode::UnsupportedModel);
+    check(sampled_only.error().message == "the current executor supports full logits output only");
+    auto candidates = create_sampling_session(nullptr, SamplingSessionOptions{3, LogitsOutputMode::TopKCandidates});
+    check(!candidates && candidates.error().code == ErrorCode::UnsupportedModel);
+    check(RuntimeCapabilityHipSampler == (UINT32_C(1) << 18)); // the runtime's own flags end at bit 17
+    check((hip_sampler_capabilities() & ~static_cast<uint32_t>(RuntimeCapabilityHipSampler)) == 0);
+
+    // the scheduler without a sampler: every row of every submission reports the missing device
+    BatchSampleScheduler scheduler(nullptr, SampleSchedulerOptions{2, 100, 0});
+    SamplingSession a(nullptr), b(nullptr);
+    const LogitsOutput logits = logits_of({1.0f, 2.0f, 3.0f});
+    std::vector<SampleBatchRequest> pair = {SampleBatchRequest{&a, &logits, {}, {}}, SampleBatchRequest{&b, &logits, {}, {}}};
+    auto results = scheduler.submit_sample(pair).get();
+    check(results.size() == 2 && !results[0] && !results[1]);
+    check(results[0].error().code == ErrorCode::InternalError);
+    auto single = scheduler.submit_sample({SampleBatchRequest{&a, &logits, {}, {}}}).get();
+    check(single.size() == 1 && !single[0] && single[0].error().code == ErrorCode::InternalError);
+    // rejected at submission: a Session named twice (src/engine/session.cpp:1257-1265), a null Session
+    auto duplicate = scheduler.submit_sample({SampleBatchRequest{&a, &logits, {}, {}}, SampleBatchRequest{&a, &logits, {}, {}}}).get();
+    check(duplicate.size() == 2 && !duplicate[0] && duplicate[0].error().code == ErrorCode::InvalidArgument);
+    check(duplicate[0].error().message == "sample batch contains duplicate sessions");
+    auto missing = scheduler.submit_sample({SampleBatchRequest{nullptr, &logits, {}, {}}}).get();
+    check(missing.size() == 1 && !missing[0] && missing[0].error().code == ErrorCode::InvalidArgument);
+    check(scheduler.submit_sample({}).get().empty());
+    const SampleSchedulerStatistics statistics = scheduler.statistics();
+    check(statistics.worker_count == 2);
+    check(statistics.submitted_batches == 5 && statistics.submitted_requests == 6);
+    check(statistics.rejected_requests == 3 && statistics.completed_requests == 3);
+}
+
+// One Session per thread, each sampling its own row again and again through the scheduler: the rows of
+// different threads share device calls, and every Session sees the tokens it would have drawn alone.
+static void test_scheduler_collects_across_calls(const HipSamplerPtr& sampler)
+{
+    constexpr int kSessions = 12, kSteps = 10;
+    const uint32_t vocab = 5000;
+    SamplingOptions options;
+    options.temperature = 0.9f;
+    options.top_k = 40;
+    options.top_p = 0.95f;
+    std::vector<std::vector<SampledToken>> alone(kSessions), together(kSessions);
+    for (int s = 0; s < kSessions; ++s)
+    {
+        SamplingSession session(sampler, SamplingSessionOptions{static_cast<uint64_t>(100 + s)});
+        for (int step = 0; step < kSteps; ++step)
+        {
+            auto token = session.sample(logits_of(synthetic_logits(vocab, s, step, 17)), options);
+            check(static_cast<bool>(token));
+            alone[s].push_back(token.value());
+        }
+    }
+    std::deque<SamplingSession> sessions;
+    for (int s = 0; s < kSessions; ++s)
+        sessions.emplace_back(sampler, SamplingSessionOptions{static_cast<uint64_t>(100 + s)});
+    BatchSampleScheduler scheduler(sampler, SampleSchedulerOptions{3, 2000, 0});
+    std::vector<std::thread> threads;
+    std::vector<std::string> failures(kSessions);
+    for (int s = 0; s < kSessions; ++s)
+    {
+        threads.emplace_back([&, s] {
+            for (int step = 0; step < kSteps; ++step)
+            {
+                const LogitsOutput logits = logits_of(synthetic_logits(vocab, s, step, 17));
+                auto results = scheduler.submit_sample({SampleBatchRequest{&sessions[s], &logits, options, {}}}).get();
+                if (results.size() != 1 || !results[0])
+                {
+                    failures[s] = results.empty() ? "no result" : results[0].error().message;
+                    return;
+                }
+                together[s].push_back(results[0].value().token);
+            }
+        });
+    }
+    for (std::thread& thread : threads)
+        thread.join();
+    for (int s = 0; s < kSessions; ++s)
+    {
+        check(failures[s].empty());
+        check(together[s].size() == alone[s].size());
+        for (int step = 0; step < kSteps; ++step)
+        {
+            check(together[s][step].token_id == alone[s][step].token_id);
+            check(std::bit_cast<uint32_t>(together[s][step].probability) == std::bit_cast<uint32_t>(alone[s][step].probability));
+        }
+    }
+    const SampleSchedulerStatistics statistics = scheduler.statistics();
+    check(statistics.completed_requests == kSessions * kSteps && statistics.rejected_requests == 0);
+    check(statistics.device_calls <= static_cast<uint64_t>(kSessions * kSteps));
+    check(statistics.cross_call_collected_requests + statistics.cross_call_collection_timeouts >= statistics.device_calls);
+    std::printf("scheduler: %d requests in %llu device calls (largest batch %llu, %llu requests collected across calls)\n", kSessions * kSteps,
+                static_cast<unsigned long long>(statistics.device_calls), static_cast<unsigned long long>(statistics.max_batch_size),
+                static_cast<unsigned long long>(statistics.cross_call_collected_requests));
+}
+
+// Requests of one Session keep their order (its generator's draws go to them in that order), alone
+// or mixed into batches with other Sessions; a multi-request submission is one device call.
+static void test_scheduler_keeps_a_sessions_order(const HipSamplerPtr& sampler)
+{
+    const uint32_t vocab = 3000;
+    SamplingOptions options;
+    options.top_k = 30;
+    constexpr int kRequests = 9;
+    std::vector<LogitsOutput> rows;
+    for (int i = 0; i < kRequests; ++i)
+        rows.push_back(logits_of(synthetic_logits(vocab, 5, i, 3)));
+    SamplingSession serial(sampler, SamplingSessionOptions{77});
+    std::vector<SampledToken> expected;
+    for (int i = 0; i < kRequests; ++i)
+        expected.push_back(serial.sample(rows[i], options).value());
+    SamplingSession session(sampler, SamplingSessionOptions{77});
+    SamplingSession other(sampler, SamplingSessionOptions{78});
+    BatchSampleScheduler scheduler(sampler, SampleSchedulerOptions{4, 300, 0}); // after the Sessions: its workers stop first
+    std::vector<std::future<std::vector<Result<BatchSampledToken>>>> futures;
+    for (int i = 0; i < kRequests; ++i)
+    {
+        if (i % 3 == 1) // in a batch with another Session
+            futures.push_back(scheduler.submit_sample({SampleBatchRequest{&other, &rows[0], options, {}}, SampleBatchRequest{&session, &rows[i], options, {}}}));
+        else
+            futures.push_back(scheduler.submit_sample({SampleBatchRequest{&session, &rows[i], options, {}}}));
+    }
+    for (int i = 0; i < kRequests; ++i)
+    {
+        auto results = futures[i].get();
+        const Result<BatchSampledToken>& mine = results.back();
+        check(static_cast<bool>(mine));
+        check(mine.value().token.token_id == expected[i].token_id);
+        check(std::bit_cast<uint32_t>(mine.value().token.probability) == std::bit_cast<uint32_t>(expected[i].probability));
+    }
+    check(scheduler.statistics().serialized_session_requests >= 1);
+}
+
+// Sessions in SampledToken mode: the rows are written into the sampler's device buffer (here with a copy,
+// by a decode step in the runtime) and only tokens come back; same tokens as the full-logits Sessions.
+static void test_sampled_token_mode(const HipSamplerPtr& sampler)
+{
+    const uint32_t vocab = 4001, count = 6;
+    check(hip_sampler_capabilities() == RuntimeCapabilityHipSampler);
+    SamplingOptions options;
+    options.temperature = 0.8f;
+    options.top_k = 25;
+    std::vector<SamplingSessionPtr> resident, full;
+    for (uint32_t i = 0; i < count; ++i)
+    {
+        auto a = create_sampling_session(sampler, SamplingSessionOptions{500 + i, LogitsOutputMode::SampledToken});
+        auto b = create_sampling_session(sampler, SamplingSessionOptions{500 + i, LogitsOutputMode::FullLogits});
+        check(static_cast<bool>(a) && static_cast<bool>(b));
+        resident.push_back(a.value());
+        full.push_back(b.value());
+    }
+    auto host_entry = resident[0]->sample(logits_of({1.0f, 2.0f}), options);
+    check(!host_entry && host_entry.error().code == ErrorCode::InvalidArgument);
+    for (uint32_t step = 0; step < 3; ++step)
+    {
+        auto rows = sampler->device_logits(count, vocab);
+        check(static_cast<bool>(rows));
+        std::vector<LogitsOutput> host_rows;
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            host_rows.push_back(logits_of(synthetic_logits(vocab, i, step, 9)));
+            check(hipMemcpy(static_cast<float*>(rows.value().data) + static_cast<size_t>(i) * rows.value().row_stride, host_rows[i].values.data(),
+                            vocab * sizeof(float), hipMemcpyHostToDevice) == hipSuccess);
+        }
+        std::vector<SampleBatchRequest> requests, full_requests;
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            requests.push_back(SampleBatchRequest{resident[i].get(), nullptr, options, {}});
+            full_requests.push_back(SampleBatchRequest{full[i].get(), &host_rows[i], options, {}});
+        }
+        auto expected = SessionBatchSampler::sample(sampler, full_requests);
+        // the upload of the full-logits batch replaced the buffer's rows with the same values
+        auto got = SessionBatchSampler::sample_resident(sampler, requests);
+        check(got.size() == count && expected.size() == count);
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            check(static_cast<bool>(got[i]) && static_cast<bool>(expected[i]));
+            check(got[i].value().token.token_id == expected[i].value().token.token_id);
+            check(std::bit_cast<uint32_t>(got[i].value().token.probability) == std::bit_cast<uint32_t>(expected[i].value().token.probability));
+        }
+    }
+    // the two kinds do not mix
+    const LogitsOutput row = logits_of({1.0f, 2.0f, 3.0f});
+    auto mixed = SessionBatchSampler::sample(sampler, std::vector<SampleBatchRequest>{SampleBatchRequest{resident[0].get(), &row, options, {}}});
+    check(mixed.size() == 1 && !mixed[0] && mixed[0].error().code == ErrorCode::InvalidArgument);
+    auto wrong = SessionBatchSampler::sample_resident(sampler, std::vector<SampleBatchRequest>{SampleBatchRequest{full[0].get(), nullptr, options, {}}});
+    check(wrong.size() == 1 && !wrong[0] && wrong[0].error().code == ErrorCode::InvalidArgument);
+}
+
+// A state without cache transactions: a step in which nothing is accepted falls back before the next token
+// is drawn (src/engine/session.cpp:843-857); only the accept test's draw is consumed.
+static void test_speculative_fallback(const HipSamplerPtr& sampler)
+{
+    const std::vector<float> ramp = {0.0f, 1.0f, 2.0f, 3.0f, 2.5f, -1.0f};
+    SamplingOptions two;
+    two.top_k = 2;
+    // sampled: the target's window (Top-2: tokens 3 and 4) does not hold the proposed token, so the
+    // accept test fails whatever the draw is
+    {
+        std::vector<float> draft_row = ramp;
+        draft_row[0] = 9.0f;
+        SamplingSession session(sampler, SamplingSessionOptions{21});
+        std::vector<LogitsOutput> target = {logits_of(ramp), logits_of(ramp)};
+        std::vector<LogitsOutput> draft = {logits_of(draft_row)};
+        auto verified = session.verify_speculative(target, draft, std::vector<int32_t>{0}, two, false);
+        check(static_cast<bool>(verified));
+        check(verified.value().fell_back && verified.value().accepted.empty() && verified.value().next.token_id == -1);
+        std::mt19937_64 shadow(21);
+        std::uniform_real_distribution<float> canonical(0.0f, 1.0f);
+        canonical(shadow); // the accept test's draw; the residual's draw was not taken
+        const float u = canonical(shadow);
+        auto sampled = session.sample(logits_of({0, 5, 5, -1}), two);
+        check(sampled.value().token_id == (u < 0.5f ? 1 : 2));
+        // with cache transactions the same step draws the next token from the residual
+        SamplingSession transactional(sampler, SamplingSessionOptions{21});
+        auto kept = transactional.verify_speculative(target, draft, std::vector<int32_t>{0}, two, true);
+        check(static_cast<bool>(kept) && !kept.value().fell_back && kept.value().next_from_residual && kept.value().next.token_id >= 0);
+        canonical(shadow);
+    }
+    // greedy: the proposal differs from the target's choice; no draw at all
+    {
+        SamplingSession session(sampler, SamplingSessionOptions{22});
+        SamplingOptions greedy;
+        greedy.temperature = 0.0f;
+        std::vector<LogitsOutput> target = {logits_of(ramp), logits_of(ramp)};
+        std::vector<LogitsOutput> draft = {logits_of(ramp)};
+        auto verified = session.verify_speculative(target, draft, std::vector<int32_t>{1}, greedy, false);
+        check(static_cast<bool>(verified) && verified.value().fell_back);
+        std::mt19937_64 shadow(22);
+        const float u = std::uniform_real_distribution<float>(0.0f, 1.0f)(shadow);
+        auto sampled = session.sample(logits_of({0, 5, 5, -1}), two);
+        check(sampled.value().token_id == (u < 0.5f ? 1 : 2));
+        // something accepted: no fall-back even without cache transactions
+        auto accepted = session.verify_speculative(target, draft, std::vector<int32_t>{3}, greedy, false);
+        check(static_cast<bool>(accepted) && !accepted.value().fell_back && accepted.value().accepted.size() == 1);
+    }
+}
+
 // ---- worker wire format (host only) -----------------------------------------------------------
 
 static void test_wire_generate_request_defaults_and_fields()
@@ -986,6 +1231,7 @@ int main(int argc, char** argv)
         test_defaults_match_the_runtime();
         test_peek_uniform_does_not_advance();
         test_missing_sampler_fails_loudly();
+        test_scheduler_and_modes_without_a_sampler();
         test_wire_generate_request_defaults_and_fields();
         test_wire_events();
         test_wire_request_fields();
@@ -1009,6 +1255,10 @@ int main(int argc, char** argv)
         test_threads_share_a_sampler(sampler);
         test_batch_rejects_bad_requests(sampler);
         test_speculative_verification(sampler);
+        test_speculative_fallback(sampler);
+        test_scheduler_collects_across_calls(sampler);
+        test_scheduler_keeps_a_sessions_order(sampler);
+        test_sampled_token_mode(sampler);
         test_generation_loop_equals_serial(sampler);
         test_generation_loop_callback_and_errors(sampler);
     }

@@ -148,3 +148,27 @@ def test_dispatcher_mirror_on_gpu():
     done = subprocess.run([DISPATCHER_TEST_PROGRAM], capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stdout + done.stderr
     assert "all expert dispatcher tests passed" in done.stdout
+
+
+REFERENCE_INCLUDE = "/root/reference/include"
+
+
+@pytest.mark.reference
+@pytest.mark.parametrize("source, forced_includes", [
+    ("hip_session_sampler.cpp", ["ncnn/moe/session.h"]),
+    ("worker_wire.cpp", ["ncnn/moe/session.h"]),
+    ("hip_expert_dispatcher.cpp", ["ncnn/moe/session.h", "ncnn/moe/expert_dispatcher.h"]),
+])
+def test_host_mirrors_compile_inside_the_runtime(source, forced_includes):
+    """The host mirrors are meant to be compiled inside the runtime, where its own headers come first and
+    the mirrors must use the runtime's types instead of their stand-alone equivalents: syntax-check each
+    source with the runtime's public headers force-included (nothing is linked or run)."""
+    if not os.path.exists(os.path.join(REFERENCE_INCLUDE, "ncnn", "moe", "session.h")):
+        pytest.skip("the runtime's headers are not present on this machine")
+    command = ["g++", "-std=c++20", "-fsyntax-only", "-I" + REFERENCE_INCLUDE, "-I" + os.path.join(ROOT, "include"),
+               "-I" + os.path.join(PACKAGE_DIR, "csrc")]
+    for header in forced_includes:
+        command += ["-include", header]
+    command.append(os.path.join(PACKAGE_DIR, "csrc", source))
+    done = subprocess.run(command, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-3000:]
