@@ -18,6 +18,9 @@ extern "C" {
  * on n host values. */
 int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* sampler, int enabled);
 int ncnn_moe_hip_sampler_debug_scatter_segments(ncnn_moe_hip_sampler* sampler, int enabled);
+/* spread_sort (on by default): the radix sort of a long full-order row runs on several workgroups; off,
+ * every row is sorted by one workgroup. */
+int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* sampler, int enabled);
 int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* sampler, const float* in, float* out, size_t n);
 void ncnn_moe_hip_sampler_debug_exp2_table(uint64_t out[32]);
 

@@ -27,6 +27,7 @@ struct ncnn_moe_hip_sampler
     uint64_t logits_stride_f32 = 0; // elements per row of the handle's logits buffer, fp32 view
     int force_general = 0;
     int scatter_segments = 0;
+    int spread_sort = 1; // a long row's radix sort runs on several workgroups
     // a call with rows for the wide select and rows for the full-order kernels runs the two side by side
     hipStream_t side_stream = nullptr;
     hipEvent_t side_fork = nullptr;
@@ -64,6 +65,7 @@ struct ncnn_moe_hip_sampler
     uint32_t* sort_keys[2] = {nullptr, nullptr};
     uint32_t* sort_indices[2] = {nullptr, nullptr};
     uint64_t sort_stride = 0;
+    uint32_t* sort_part_counts = nullptr; // [rows][kMaxSortParts][256]
 
     int32_t* distribution_ids = nullptr;
     float* distribution_probabilities = nullptr;
@@ -284,6 +286,7 @@ int launch_sampler(
     a.sort_indices[0] = s->sort_indices[0];
     a.sort_indices[1] = s->sort_indices[1];
     a.sort_stride = s->sort_stride;
+    a.sort_part_counts = s->sort_part_counts;
     if (want_distribution)
     {
         a.distribution_ids = export_to.ids;
@@ -309,27 +312,60 @@ int launch_sampler(
         else
             launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, on, a, true, s->scatter_segments != 0);
     };
-    const auto launch_full_order = [&](const SamplerArgs& a) {
+    // A long row's radix sort is spread over several workgroups (two tiles each, at most kMaxSortParts):
+    // two launches per pass over a (parts, rows) grid.  Short rows keep the one-workgroup kernel.
+    const uint32_t sort_tiles = static_cast<uint32_t>((static_cast<uint64_t>(vocab) + kSortTile - 1) / kSortTile);
+    const uint32_t sort_tiles_per_part = std::max<uint32_t>(2, (sort_tiles + kMaxSortParts - 1) / kMaxSortParts);
+    const uint32_t sort_parts = std::max<uint32_t>(1, (sort_tiles + sort_tiles_per_part - 1) / sort_tiles_per_part);
+    const auto launch_spread_sort = [&](SamplerArgs spread, auto dtype_tag, auto pairs_tag) {
+        constexpr int kType = decltype(dtype_tag)::value;
+        constexpr bool kPairs = decltype(pairs_tag)::value;
+        spread.sort_parts = sort_parts;
+        spread.sort_tiles_per_part = sort_tiles_per_part;
+        const int passes = kType == NCNN_MOE_LOGITS_F32 ? 4 : 2;
+        for (int pass = 0; pass < passes; ++pass)
+        {
+            spread.sort_pass = static_cast<uint32_t>(pass);
+            hipLaunchKernelGGL((sort_part_histogram_kernel<kType>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
+            hipLaunchKernelGGL((sort_part_scatter_kernel<kType, kPairs>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
+        }
+    };
+    // `leftovers`: the launch behind the wide select, for the few rows (usually none) that it could not
+    // finish; it is kept to two kernels, because every launch costs its few microseconds even with no row to serve.
+    const auto launch_full_order = [&](SamplerArgs a, bool leftovers) {
+        const bool spread_sort = sort_parts > 1 && s->spread_sort != 0 && !leftovers;
+        const bool runs = dtype == NCNN_MOE_LOGITS_BF16 && !want_distribution;
         // the token indices ride along with the keys only when the whole distribution is exported
-        if (dtype == NCNN_MOE_LOGITS_F32)
-        {
-            if (want_distribution)
-                hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_F32, true>), dim3(rows), dim3(kSortThreads), 0, stream, a);
+        const auto sort_rows = [&](auto dtype_tag, auto pairs_tag) {
+            constexpr int kType = decltype(dtype_tag)::value;
+            constexpr bool kPairs = decltype(pairs_tag)::value;
+            if (spread_sort)
+                launch_spread_sort(a, dtype_tag, pairs_tag);
             else
-                hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_F32, false>), dim3(rows), dim3(kSortThreads), 0, stream, a);
-            hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_F32, false>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
-        }
+                hipLaunchKernelGGL((general_sort_kernel<kType, kPairs>), dim3(rows), dim3(kSortThreads), 0, stream, a);
+        };
+        using F32 = std::integral_constant<int, NCNN_MOE_LOGITS_F32>;
+        using BF16 = std::integral_constant<int, NCNN_MOE_LOGITS_BF16>;
+        if (runs)
+            hipLaunchKernelGGL(bf16_counting_sort_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
+        else if (dtype == NCNN_MOE_LOGITS_F32 && want_distribution)
+            sort_rows(F32{}, std::true_type{});
+        else if (dtype == NCNN_MOE_LOGITS_F32)
+            sort_rows(F32{}, std::false_type{});
         else
+            sort_rows(BF16{}, std::true_type{});
+        if (!runs && !leftovers)
         {
-            if (want_distribution)
-                hipLaunchKernelGGL((general_sort_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kSortThreads), 0, stream, a);
-            else
-                hipLaunchKernelGGL(bf16_counting_sort_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
-            if (want_distribution)
-                hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, false>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
-            else
-                hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
+            const uint32_t parts = (vocab + kTermsThreads * kTermsPerThread - 1) / (kTermsThreads * kTermsPerThread);
+            hipLaunchKernelGGL(full_order_terms_kernel, dim3(parts, rows), dim3(kTermsThreads), 0, stream, a);
+            a.terms_precomputed = 1;
         }
+        if (runs)
+            hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
+        else if (dtype == NCNN_MOE_LOGITS_F32)
+            hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_F32, false>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
+        else
+            hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, false>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
     };
     // Rows for the wide select and rows for the full-order kernels are disjoint and each pass keeps few
     // compute units busy (one workgroup per row): with both kinds in the call the two passes run side by
@@ -343,17 +379,17 @@ int launch_sampler(
         launch_wide(s->side_stream);
         SamplerArgs own_rows = a;
         own_rows.leave_wide_rows = 1;
-        launch_full_order(own_rows);
+        launch_full_order(own_rows, false);
         if (hipEventRecord(s->side_join, s->side_stream) != hipSuccess || hipStreamWaitEvent(stream, s->side_join, 0) != hipSuccess)
             return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "join of the second stream failed");
-        launch_full_order(a);
+        launch_full_order(a, true);
     }
     else
     {
         if (passes.wide_select)
             launch_wide(stream);
         if (passes.full_order)
-            launch_full_order(a);
+            launch_full_order(a, false);
     }
     SAMPLER_HIP_CHECK(s, hipGetLastError());
     return NCNN_MOE_SAMPLER_SUCCESS;
@@ -520,6 +556,7 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
         CREATE_CHECK(hipMalloc(&s->sort_keys[i], rows * s->sort_stride * sizeof(uint32_t)));
         CREATE_CHECK(hipMalloc(&s->sort_indices[i], rows * s->sort_stride * sizeof(uint32_t)));
     }
+    CREATE_CHECK(hipMalloc(&s->sort_part_counts, rows * kMaxSortParts * 256 * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->distribution_ids, static_cast<size_t>(max_vocab) * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->distribution_probabilities, static_cast<size_t>(max_vocab) * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->distribution_count, sizeof(uint32_t)));
@@ -571,7 +608,7 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
     void* buffers[] = {
         s->logits, s->params, s->uniforms, s->results, s->segment_values, s->segment_indices,
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->split_records, s->row_epoch, s->sort_keys[0], s->sort_keys[1],
-        s->sort_indices[0], s->sort_indices[1], s->distribution_ids, s->distribution_probabilities,
+        s->sort_indices[0], s->sort_indices[1], s->sort_part_counts, s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
         s->verify_probabilities, s->verify_counts, s->verify_long_ids, s->verify_long_probabilities, s->verify_dense};
     for (void* buffer : buffers)
@@ -1026,6 +1063,14 @@ int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* s, int enable
     if (s == nullptr)
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     s->force_general = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* s, int enabled)
+{
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    s->spread_sort = enabled ? 1 : 0;
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

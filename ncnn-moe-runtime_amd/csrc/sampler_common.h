@@ -44,6 +44,14 @@ struct SamplerArgs
     uint32_t* sort_keys[2];
     uint32_t* sort_indices[2];
     uint64_t sort_stride;
+    // full-order path with a row's sort spread over several workgroups: [rows][sort_parts][256] digit counts
+    // of the pass in flight, the number of parts, tiles (kSortTile keys) per part, and the pass
+    uint32_t* sort_part_counts;
+    uint32_t sort_parts;
+    uint32_t sort_tiles_per_part;
+    uint32_t sort_pass;
+    // full_order_terms_kernel has run: sort_keys[0] holds exp(logit/T - maximum) of the sorted rows' elements
+    uint32_t terms_precomputed;
 
     // optional filtered-distribution output: row r writes at most distribution_cap (id, probability)
     // entries from r * distribution_cap on, and its full kept length to distribution_count[r]

@@ -42,9 +42,19 @@ constexpr int kSortThreads = 1024;
 constexpr int kSortWaves = kSortThreads / kWaveSize;
 constexpr int kSortPerThread = 8;
 constexpr int kSortTile = kSortThreads * kSortPerThread;
+constexpr int kMaxSortParts = 8;              // workgroups one row's radix sort is spread over
 constexpr int kReplayThreads = 1024;
-constexpr int kReplayPerThread = 4;
-constexpr int kReplayChunk = kReplayThreads * kReplayPerThread;
+// The exact running sums are the work of the workgroup's first kSumWaves waves (two per SIMD), each thread
+// composing a few consecutive terms: every wave that takes part pays the scan across its lanes and the
+// composition of the waves' totals again, and a thread's terms are a chain of dependent instructions.
+// Measured on full-order batches (sixteen waves x 4 terms, eight x 8, eight x 4, four x 16, sixteen x 8):
+// rows of single elements do best with eight waves x 8 terms, rows of runs with eight waves x 4.
+constexpr int kSumWaves = 8;
+constexpr int kSumThreads = kSumWaves * 64;
+constexpr int kReplayPerThread = 8;
+constexpr int kRunsPerThread = 4;
+constexpr int kRunsChunk = kSumThreads * kRunsPerThread;
+constexpr int kReplayChunk = kSumThreads * kReplayPerThread;
 
 // Wall-clock stamps for a timeline of the split path, compiled in only with -DNCNN_MOE_TIMELINE (a
 // separate library, built by `make timeline`; the shipped one carries none).
@@ -72,6 +82,29 @@ __device__ unsigned long long g_timeline_rows[kTimelineRows * kTimelineSlots];
         if ((threadIdx.x & 63) == 0 && (row) < static_cast<uint32_t>(kTimelineRows))                         \
             g_timeline_rows[(row) * kTimelineSlots + (slot)] = wall_clock64();                               \
     } while (0)
+// successive stamps of one code path: slot numbers from a counter kept in g_timeline[..][15]
+#define NCNN_MOE_STAMP_NEXT(row, segment)                                                                    \
+    do                                                                                                       \
+    {                                                                                                        \
+        if (threadIdx.x == 0 && (row) < static_cast<uint32_t>(kTimelineRows))                                \
+        {                                                                                                    \
+            unsigned long long* base_ = g_timeline + ((row) * kMaxSegments + (segment)) * kTimelineSlots;    \
+            const unsigned long long slot_ = base_[15];                                                      \
+            if (slot_ < 15)                                                                                  \
+            {                                                                                                \
+                base_[slot_] = wall_clock64();                                                               \
+                base_[15] = slot_ + 1;                                                                       \
+            }                                                                                                \
+        }                                                                                                    \
+    } while (0)
+#define NCNN_MOE_STAMP_RESET(row, segment) NCNN_MOE_STAMP_VALUE(row, segment, 15, 0ull)
+// events counted rather than timed (the reader takes differences between launches)
+#define NCNN_MOE_COUNT(row, segment, slot)                                                                   \
+    do                                                                                                       \
+    {                                                                                                        \
+        if (threadIdx.x == 0 && (row) < static_cast<uint32_t>(kTimelineRows))                                \
+            g_timeline[((row) * kMaxSegments + (segment)) * kTimelineSlots + (slot)] += 1;                   \
+    } while (0)
 #define NCNN_MOE_STAMP_VALUE_FROM(leader, row, segment, slot, value)                                        \
     do                                                                                                       \
     {                                                                                                        \
@@ -81,6 +114,9 @@ __device__ unsigned long long g_timeline_rows[kTimelineRows * kTimelineSlots];
 #else
 #define NCNN_MOE_STAMP_VALUE_FROM(leader, row, segment, slot, value) ((void)0)
 #define NCNN_MOE_STAMP_ROW(row, slot) ((void)0)
+#define NCNN_MOE_COUNT(row, segment, slot) ((void)0)
+#define NCNN_MOE_STAMP_NEXT(row, segment) ((void)0)
+#define NCNN_MOE_STAMP_RESET(row, segment) ((void)0)
 #define NCNN_MOE_STAMP(row, segment, slot) ((void)0)
 #define NCNN_MOE_STAMP_VALUE(row, segment, slot, value) ((void)0)
 #endif

@@ -69,7 +69,62 @@ __device__ __forceinline__ uint32_t repeated_step(bool odd, const ParityStep& s,
 
 __device__ __forceinline__ ParityStep repeat_steps(const ParityStep& s, uint32_t count)
 {
+    // The two steps differ only for a term that ends exactly half an ulp above a multiple of it; when no lane
+    // of the wave holds such a term, every addition moves the mantissa by the same step.
+    if (__builtin_amdgcn_ballot_w64(s.even != s.odd) == 0ull)
+    {
+        const uint64_t total = static_cast<uint64_t>(s.even) * count;
+        const uint32_t capped = total > kStepCap ? kStepCap : static_cast<uint32_t>(total);
+        return ParityStep{capped, capped};
+    }
     return ParityStep{repeated_step(false, s, count), repeated_step(true, s, count)};
+}
+
+// Inclusive scan of the lanes' steps in lane order (lane i: the composition of lanes 0 .. i), by DPP shifts
+// inside rows of 16 lanes and two broadcasts across rows; a lane without a source composes with the
+// identity (a step of zero).
+__device__ __forceinline__ ParityStep wave_scan_steps(ParityStep v)
+{
+#define NCNN_MOE_SCAN_STAGE(CONTROL, ROW_MASK)                                                              \
+    {                                                                                                        \
+        const ParityStep earlier{dpp_source<CONTROL, ROW_MASK>(v.even), dpp_source<CONTROL, ROW_MASK>(v.odd)}; \
+        v = compose_steps(earlier, v);                                                                       \
+    }
+    NCNN_MOE_SCAN_STAGE(0x111, 0xf) // row_shr:1
+    NCNN_MOE_SCAN_STAGE(0x112, 0xf) // row_shr:2
+    NCNN_MOE_SCAN_STAGE(0x114, 0xf) // row_shr:4
+    NCNN_MOE_SCAN_STAGE(0x118, 0xf) // row_shr:8
+    NCNN_MOE_SCAN_STAGE(0x142, 0xa) // row_bcast15: rows 1 and 3 compose with the row before
+    NCNN_MOE_SCAN_STAGE(0x143, 0xc) // row_bcast31: rows 2 and 3 compose with rows 0 + 1
+#undef NCNN_MOE_SCAN_STAGE
+    return v;
+}
+
+__device__ __forceinline__ uint32_t apply_step(uint32_t mantissa, const ParityStep& step)
+{
+    return mantissa + ((mantissa & 1u) ? step.odd : step.even);
+}
+
+// First index in [0, count) at which a predicate that holds on a prefix stops holding; the wave probes
+// 64 places per step (three dependent loads for 2^18 items where a bisection takes eighteen).  The
+// arguments must be the same in every lane of the wave; every lane receives the result.
+template <class Holds>
+__device__ __forceinline__ uint32_t wave_partition_point(uint32_t count, Holds holds)
+{
+    const uint32_t lane = static_cast<uint32_t>(lane_id());
+    uint32_t low = 0, high = count;
+    while (low < high)
+    {
+        const uint32_t step = (high - low + kWaveSize - 1u) / kWaveSize;
+        const uint32_t probe = low + lane * step;
+        const bool ok = probe < high && holds(probe);
+        const uint32_t passed = static_cast<uint32_t>(__popcll(__builtin_amdgcn_ballot_w64(ok)));
+        if (passed == 0u)
+            break;
+        high = min(high, low + passed * step);
+        low = low + (passed - 1u) * step + 1u;
+    }
+    return low;
 }
 
 // Biased exponent (denormals and zero share exponent 1) and integer mantissa of a non-negative float:
@@ -90,46 +145,27 @@ __device__ __forceinline__ float encode_sum(int exponent, uint32_t mantissa)
     return __uint_as_float((static_cast<uint32_t>(exponent - 1) << 23) + mantissa);
 }
 
-// The step a term causes on a sum with biased exponent `exponent`.
+// The step a term causes on a sum with biased exponent `exponent`: with the term's mantissa split at
+// the sum's ulp into `whole` ulps and a rest, the sum moves by whole ulps, one more when the rest is
+// above half an ulp, and on a rest of exactly half to the even neighbour: up when the mantissa and
+// `whole` differ in parity.  Adding (half - 1 + [whole odd]) before the shift rounds that way for an
+// even mantissa, (half - [whole odd]) for an odd one.
 __device__ __forceinline__ ParityStep step_of_term(float term, int exponent)
 {
-    int term_exponent;
-    uint32_t term_mantissa;
-    decode_sum(term, term_exponent, term_mantissa);
-    ParityStep step;
-    const int shift = exponent - term_exponent;
-    if (term_mantissa == 0u || shift >= 25)
-    {
-        step.even = 0u;
-        step.odd = 0u;
-    }
-    else if (shift <= 0)
-    {
-        step.even = kBinadeFull; // at least half the sum: the addition leaves the binade
-        step.odd = kBinadeFull;
-    }
-    else
-    {
-        const uint32_t whole = term_mantissa >> shift;
-        const uint32_t rest = term_mantissa & ((1u << shift) - 1u);
-        const uint32_t half = 1u << (shift - 1);
-        if (rest > half)
-        {
-            step.even = whole + 1u;
-            step.odd = whole + 1u;
-        }
-        else if (rest < half)
-        {
-            step.even = whole;
-            step.odd = whole;
-        }
-        else
-        {
-            step.even = whole + (whole & 1u);
-            step.odd = whole + 1u - (whole & 1u);
-        }
-    }
-    return step;
+    // Without branches (a workgroup runs this for every term of every round).  A shift of 25 or more, or a
+    // term of zero, gives zero by the arithmetic itself: mantissa + half stays below 2^shift.
+    const uint32_t bits = __float_as_uint(term);
+    const int stored_exponent = static_cast<int>(bits >> 23);
+    const int term_exponent = max(stored_exponent, 1);
+    const uint32_t term_mantissa = (bits & 0x7fffffu) | (stored_exponent != 0 ? 0x800000u : 0u);
+    const int difference = exponent - term_exponent;
+    const uint32_t shift = static_cast<uint32_t>(min(max(difference, 1), 25));
+    const uint32_t half = 1u << (shift - 1u);
+    const uint32_t whole_odd = (term_mantissa >> shift) & 1u;
+    const uint32_t even = (term_mantissa + half - 1u + whole_odd) >> shift;
+    const uint32_t odd = (term_mantissa + half - whole_odd) >> shift;
+    const bool leaves = difference <= 0 && term_mantissa != 0u; // at least half the sum: the addition leaves the binade
+    return ParityStep{leaves ? kBinadeFull : even, leaves ? kBinadeFull : odd};
 }
 
 enum StopMode : int
@@ -163,13 +199,16 @@ __device__ __forceinline__ uint32_t stop_mantissa(int mode, float bound, int exp
 
 constexpr int kReplayWaves = kReplayThreads / kWaveSize;
 
+// Two copies of everything, used by alternate rounds: a round's values are read after one of its barriers
+// and written again two rounds later, with barriers in between, so that a round needs two barriers (three
+// with an event) and none at its end.
 struct ReplayScratch
 {
-    ParityStep wave_totals[kReplayWaves];
-    uint32_t first_event; // (index << 1 | kind) of the earliest event of the round, kind 0 = leaves the binade, 1 = stop
-    uint32_t final_mantissa;
-    float event_sum;
-    int absorbed;
+    ParityStep wave_totals[2][kSumWaves];
+    uint32_t first_event[2]; // (index << 1 | kind) of the earliest event of the round, kind 0 = leaves the binade, 1 = stop
+    uint32_t final_mantissa[2];
+    float event_sum[2];
+    int absorbed[2];
 };
 
 struct RunningSum
@@ -188,6 +227,7 @@ struct SortedRow
     const uint32_t* keys;     // one key per element, or one per run of equal keys
     const uint32_t* run_ends; // runs only: position behind the last element of each run (null otherwise)
     uint32_t run_count;
+    const float* terms0;      // exp(logit/T - maximum) of every item (element or run), computed beforehand
     float temperature;
     float maximum;
     float normalizer;
@@ -215,10 +255,18 @@ __device__ __forceinline__ uint32_t run_of_element(const SortedRow& row, uint32_
     return low;
 }
 
+// ... the same for an element that every lane of the wave asks for
+__device__ __forceinline__ uint32_t run_of_element_uniform(const SortedRow& row, uint32_t element)
+{
+    const uint32_t* run_ends = row.run_ends;
+    return wave_partition_point(row.run_count, [run_ends, element](uint32_t run) { return run_ends[run] <= element; });
+}
+
+// The term of item i that the CPU loop of `PHASE` adds.
 template <int PHASE>
 __device__ __forceinline__ float row_term(const SortedRow& row, uint32_t i)
 {
-    float t = expf_libm(value_from_descending_key(row.keys[i]) / row.temperature - row.maximum);
+    float t = row.terms0[i];
     if (PHASE >= 1)
         t = t / row.normalizer;
     if (PHASE >= 2)
@@ -226,16 +274,124 @@ __device__ __forceinline__ float row_term(const SortedRow& row, uint32_t i)
     return t;
 }
 
-// The running fp32 sum of the non-negative terms term_at(0) ... term_at(count - 1), starting from 0,
-// exactly as a sequential loop produces it.  With NON_INCREASING (the terms never grow) it also stops
-// (without `stopped`) once the sum no longer moves, which is then final.  Every thread of the
-// workgroup (kReplayThreads threads) must call it.
-template <bool NON_INCREASING, class TermAt>
-__device__ __forceinline__ RunningSum exact_running_sum_of_terms(
-    TermAt term_at, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
+// What the rounds of the two running sums below share.  A round has every thread compose the steps of its
+// own terms; this turns the threads' totals into the mantissa in front of each thread, finds the first
+// event (the sum leaves its binade, or the stop condition first holds) and hands it to every thread.
+//   thread_total   composition of the calling thread's steps
+//   find_event     called in a thread whose range holds an event, with the mantissa in front of the thread:
+//                  fills the event's key (index << 1 | kind), mantissa and term
+// Returns kRoundPlain when the round ended without an event: `sum` is then the sum behind the round's last
+// term.  With an event (kRoundEvent), `sum` is the sum behind the event's term and event_key names it.
+// With CHECK_ABSORBED, thread 0 has written scratch.absorbed[slot] before the call: when set, the round
+// is abandoned (kRoundAbsorbed, `sum` unchanged).
+enum RoundOutcome : int
+{
+    kRoundPlain = 0,
+    kRoundEvent = 1,
+    kRoundAbsorbed = 2
+};
+
+struct RoundEvent
+{
+    uint32_t key;
+    uint32_t mantissa; // kind 0: before the term is added; kind 1: behind it
+    float term;
+};
+
+template <bool CHECK_ABSORBED, class FindEvent>
+__device__ __forceinline__ RoundOutcome finish_round(
+    const ParityStep& thread_total, int exponent, uint32_t mantissa, uint32_t limit, FindEvent find_event,
+    ReplayScratch& scratch, uint32_t slot, int tid, float& sum, uint32_t& event_key)
 {
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
+    const bool summing = wave < kSumWaves; // the other waves only follow the round's barriers and its outcome
+    ParityStep exclusive{0u, 0u};
+    if (summing)
+    {
+        const ParityStep inclusive = wave_scan_steps(thread_total);
+        exclusive.even = __shfl_up(inclusive.even, 1, kWaveSize);
+        exclusive.odd = __shfl_up(inclusive.odd, 1, kWaveSize);
+        if (lane == 0)
+            exclusive = ParityStep{0u, 0u};
+        if (lane == kWaveSize - 1)
+            scratch.wave_totals[slot][wave] = inclusive;
+    }
+    NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
+    lds_barrier();
+    NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
+    if (tid == 0)
+        scratch.first_event[slot ^ 1u] = 0xffffffffu; // for the next round: its readers are behind the barrier
+    if (CHECK_ABSORBED)
+    {
+        if (scratch.absorbed[slot])
+        {
+            lds_barrier(); // every thread has read the flag before a later call writes it
+            return kRoundAbsorbed;
+        }
+    }
+    RoundEvent found{0u, 0u, 0.0f};
+    bool reported = false;
+    if (summing)
+    {
+        // every wave's total is read at once (independent LDS loads); the composition stays in registers
+        ParityStep totals[kSumWaves];
+#pragma unroll
+        for (int w = 0; w < kSumWaves; ++w)
+            totals[w] = scratch.wave_totals[slot][w];
+        ParityStep before{0u, 0u};
+#pragma unroll
+        for (int w = 0; w < kSumWaves - 1; ++w)
+        {
+            const ParityStep with = compose_steps(before, totals[w]);
+            before = ParityStep{w < wave ? with.even : before.even, w < wave ? with.odd : before.odd};
+        }
+        before = compose_steps(before, exclusive);
+        const uint32_t current = apply_step(mantissa, before);
+        const uint32_t behind = apply_step(current, thread_total);
+        // The mantissa never decreases: the first event lies in the thread whose range takes it to the limit.
+        // (A round that begins at the limit - a stop bound of zero - has its event at its first term.)
+        const bool have_event = behind >= limit && (current < limit || mantissa >= limit);
+        if (have_event)
+            reported = find_event(current, found);
+        if (reported)
+            atomicMin(&scratch.first_event[slot], found.key);
+        if (tid == kSumThreads - 1)
+            scratch.final_mantissa[slot] = behind;
+    }
+    NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
+    lds_barrier();
+    NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
+    const uint32_t event = scratch.first_event[slot];
+    if (event == 0xffffffffu)
+    {
+        sum = encode_sum(exponent, scratch.final_mantissa[slot]);
+        return kRoundPlain;
+    }
+    if (reported && found.key == event)
+    {
+        const float at_event = encode_sum(exponent, found.mantissa);
+        scratch.event_sum[slot] = (event & 1u) ? at_event : at_event + found.term;
+    }
+    lds_barrier();
+    sum = scratch.event_sum[slot];
+    event_key = event;
+    return kRoundEvent;
+}
+
+// The running fp32 sum of the non-negative terms term(0) ... term(count - 1), starting from 0, exactly as
+// a sequential loop produces it; term(i) = terms[i], divided by `divisor` and then by `second_divisor` with
+// DIVIDED (a divisor of one leaves a term as it is).  With NON_INCREASING (the terms never grow) it also
+// stops (without `stopped`) once the sum no longer moves, which is then final.  Every thread of the
+// workgroup (kReplayThreads threads) must call it.
+template <bool NON_INCREASING, bool DIVIDED>
+__device__ __noinline__ RunningSum exact_running_sum_of_array(
+    const float* terms_array, float divisor, float second_divisor, uint32_t count, int mode, float bound,
+    ReplayScratch& scratch, int tid)
+{
+    const auto scaled = [divisor, second_divisor](float t) { return DIVIDED ? (t / divisor) / second_divisor : t; };
+    const auto term_at = [&](uint32_t i) { return scaled(terms_array[i]); };
+    const int lane = tid & (kWaveSize - 1);
     float sum = 0.0f;
     // The first kSequentialHead terms are added one by one, as the CPU does (every thread runs the same
     // loop on wave-uniform values): the sum climbs through most of its binades here, each of which
@@ -264,6 +420,37 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_terms(
         if (head >= count)
             return RunningSum{sum, 0u, false};
     }
+    if (tid == 0)
+        scratch.first_event[0] = 0xffffffffu;
+    uint32_t round = 0;
+    // the terms of the next chunk are asked for while this one is summed
+    float upcoming[kReplayPerThread];
+    const bool summing = tid < kSumThreads;
+    const bool aligned = (reinterpret_cast<uintptr_t>(terms_array) & 15u) == 0u;
+    const auto fetch = [&](uint32_t base) {
+        const uint32_t chunk_end = min(count, base + static_cast<uint32_t>(kReplayChunk));
+        const uint32_t first = base + static_cast<uint32_t>(tid) * kReplayPerThread;
+        if (aligned && first + kReplayPerThread <= chunk_end)
+        {
+            // (only whole groups: nothing is read behind `count`)
+#pragma unroll
+            for (int j = 0; j < kReplayPerThread; j += 4)
+            {
+                const float4 four = *reinterpret_cast<const float4*>(terms_array + first + j);
+                upcoming[j + 0] = four.x;
+                upcoming[j + 1] = four.y;
+                upcoming[j + 2] = four.z;
+                upcoming[j + 3] = four.w;
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int j = 0; j < kReplayPerThread; ++j)
+                upcoming[j] = (summing && first + j < chunk_end) ? terms_array[first + j] : 0.0f;
+        }
+    };
+    fetch(0);
     for (uint32_t base = 0; base < count; base += kReplayChunk)
     {
         const uint32_t chunk_end = min(count, base + static_cast<uint32_t>(kReplayChunk));
@@ -271,10 +458,9 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_terms(
         float terms[kReplayPerThread];
 #pragma unroll
         for (int j = 0; j < kReplayPerThread; ++j)
-        {
-            const uint32_t i = thread_first + j;
-            terms[j] = i < chunk_end ? term_at(i) : 0.0f;
-        }
+            terms[j] = scaled(upcoming[j]);
+        if (base + kReplayChunk < count)
+            fetch(base + kReplayChunk);
         uint32_t start = max(base, head);
         while (start < chunk_end)
         {
@@ -282,115 +468,67 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_terms(
             uint32_t mantissa;
             decode_sum(sum, exponent, mantissa);
             const uint32_t stop_at = stop_mantissa(mode, bound, exponent);
+            const uint32_t limit = min(stop_at, kBinadeFull);
+            const uint32_t slot = round & 1u;
+            ++round;
+            NCNN_MOE_COUNT(blockIdx.x, 15, 12);
+            NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
 
-            ParityStep thread_total{0u, 0u};
-            ParityStep first_step{0u, 0u};
-#pragma unroll
-            for (int j = 0; j < kReplayPerThread; ++j)
-            {
+            const auto step_at = [&](int j) {
                 const uint32_t i = thread_first + j;
-                ParityStep step{0u, 0u};
-                if (i >= start && i < chunk_end)
-                    step = step_of_term(terms[j], exponent);
-                if (j == 0)
-                    first_step = step;
-                thread_total = compose_steps(thread_total, step);
-            }
-            if (tid == 0)
-            {
-                scratch.first_event = 0xffffffffu;
-                // the largest remaining term of the row does not move the sum: nothing later can
-                scratch.absorbed = (NON_INCREASING && start == base && base > 0 && first_step.even == 0u && first_step.odd == 0u) ? 1 : 0;
-            }
-            // inclusive scan of the per-thread totals across the wave, then across waves
-            ParityStep inclusive = thread_total;
-#pragma unroll
-            for (int step = 1; step < kWaveSize; step <<= 1)
-            {
-                ParityStep earlier;
-                earlier.even = __shfl_up(inclusive.even, step, kWaveSize);
-                earlier.odd = __shfl_up(inclusive.odd, step, kWaveSize);
-                if (lane >= step)
-                    inclusive = compose_steps(earlier, inclusive);
-            }
-            ParityStep exclusive;
-            exclusive.even = __shfl_up(inclusive.even, 1, kWaveSize);
-            exclusive.odd = __shfl_up(inclusive.odd, 1, kWaveSize);
-            if (lane == 0)
-                exclusive = ParityStep{0u, 0u};
-            if (lane == kWaveSize - 1)
-                scratch.wave_totals[wave] = inclusive;
-            __syncthreads();
-            if (scratch.absorbed)
-                return RunningSum{sum, 0u, false};
-            // every wave's total is read at once (independent LDS loads); the composition stays in registers
-            ParityStep totals[kReplayWaves];
-#pragma unroll
-            for (int w = 0; w < kReplayWaves; ++w)
-                totals[w] = scratch.wave_totals[w];
-            ParityStep before{0u, 0u};
-#pragma unroll
-            for (int w = 0; w < kReplayWaves - 1; ++w)
-            {
-                if (w < wave)
-                    before = compose_steps(before, totals[w]);
-            }
-            before = compose_steps(before, exclusive);
-            uint32_t current = mantissa + ((mantissa & 1u) ? before.odd : before.even);
-
-            // walk this thread's terms with the true mantissa; remember the first event
-            bool have_event = false;
-            uint32_t event_key = 0;
-            uint32_t event_mantissa = 0;
-            float event_term = 0.0f;
-#pragma unroll
-            for (int j = 0; j < kReplayPerThread; ++j)
-            {
-                const uint32_t i = thread_first + j;
+                const ParityStep step = step_of_term(terms[j], exponent);
                 const bool active = i >= start && i < chunk_end;
-                ParityStep step{0u, 0u};
-                if (active)
-                    step = step_of_term(terms[j], exponent);
-                const uint32_t next = current + ((current & 1u) ? step.odd : step.even);
-                if (active && !have_event)
+                return ParityStep{active ? step.even : 0u, active ? step.odd : 0u};
+            };
+            ParityStep thread_total{0u, 0u};
+            if (summing)
+            {
+#pragma unroll
+                for (int j = 0; j < kReplayPerThread; ++j)
+                    thread_total = compose_steps(thread_total, step_at(j));
+            }
+            if (NON_INCREASING)
+            {
+                // the largest remaining term of the row does not move the sum: nothing later can
+                if (tid == 0)
                 {
+                    const ParityStep first_step = step_at(0);
+                    scratch.absorbed[slot] = (start == base && base > 0 && first_step.even == 0u && first_step.odd == 0u) ? 1 : 0;
+                }
+            }
+            const auto find_event = [&](uint32_t current, RoundEvent& found) -> bool {
+                // Walk this thread's terms from the mantissa in front of them.  One thread of a round does this,
+                // in few rounds: a short loop that reads the terms again, rather than sixteen unrolled copies
+                // over the registers.
+                const uint32_t first = max(thread_first, start);
+                const uint32_t last = min(thread_first + static_cast<uint32_t>(kReplayPerThread), chunk_end);
+#pragma unroll 1
+                for (uint32_t i = first; i < last; ++i)
+                {
+                    const float term = term_at(i);
+                    const uint32_t next = apply_step(current, step_of_term(term, exponent));
                     if (next >= kBinadeFull)
                     {
-                        have_event = true;
-                        event_key = i << 1;
-                        event_mantissa = current;
-                        event_term = terms[j];
+                        found = RoundEvent{i << 1, current, term};
+                        return true;
                     }
-                    else if (next >= stop_at)
+                    if (next >= stop_at)
                     {
-                        have_event = true;
-                        event_key = (i << 1) | 1u;
-                        event_mantissa = next;
+                        found = RoundEvent{(i << 1) | 1u, next, 0.0f};
+                        return true;
                     }
+                    current = next;
                 }
-                current = next;
-            }
-            if (have_event)
-                atomicMin(&scratch.first_event, event_key);
-            if (tid == kReplayThreads - 1)
-                scratch.final_mantissa = current;
-            __syncthreads();
-            const uint32_t event = scratch.first_event;
-            if (event == 0xffffffffu)
-            {
-                sum = encode_sum(exponent, scratch.final_mantissa);
-                __syncthreads();
+                return false;
+            };
+            uint32_t event = 0;
+            const RoundOutcome outcome =
+                finish_round<NON_INCREASING>(thread_total, exponent, mantissa, limit, find_event, scratch, slot, tid, sum, event);
+            if (outcome == kRoundAbsorbed)
+                return RunningSum{sum, 0u, false};
+            if (outcome == kRoundPlain)
                 break;
-            }
-            if (have_event && event_key == event)
-            {
-                const float at_event = encode_sum(exponent, event_mantissa);
-                scratch.event_sum = (event & 1u) ? at_event : at_event + event_term;
-            }
-            __syncthreads();
-            sum = scratch.event_sum;
             const uint32_t event_index = event >> 1;
-            __syncthreads();
             if (event & 1u)
                 return RunningSum{sum, event_index, true};
             if ((mode == kStopAtOrAbove && sum >= bound) || (mode == kStopAbove && sum > bound))
@@ -407,24 +545,30 @@ template <int PHASE>
 __device__ __forceinline__ RunningSum exact_running_sum(
     const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
 {
-    return exact_running_sum_of_terms<PHASE == 0>(
-        [&row](uint32_t i) { return row_term<PHASE>(row, i); }, count, mode, bound, scratch, tid);
+    return exact_running_sum_of_array<PHASE == 0, PHASE != 0>(
+        row.terms0, row.normalizer, PHASE == 2 ? row.renormalizer : 1.0f, count, mode, bound, scratch, tid);
 }
 
 // The same running sum over a row stored as runs: `count` elements are added, run after run.  A run of
 // m equal terms is one step (repeat_steps); when an event (the sum leaves its binade, or the stop
 // condition first holds) falls inside a run, the thread that owns the run finds the addition it
 // falls on by bisection over repeated_step, which is monotone in the number of additions.
-template <int PHASE>
-__device__ __forceinline__ RunningSum exact_running_sum_runs(
-    const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
+template <bool FIRST>
+__device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
+    const SortedRow& row, float divisor, float second_divisor, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
 {
+    // FIRST: the terms as they are (they never grow: the sum also stops once it no longer moves); else
+    // divided by the two divisors, one after the other (a divisor of one leaves a term as it is)
+    const float* const terms0 = row.terms0;
+    const auto term_of_run = [terms0, divisor, second_divisor](uint32_t run) {
+        const float t = terms0[run];
+        return FIRST ? t : (t / divisor) / second_divisor;
+    };
     const int lane = tid & (kWaveSize - 1);
-    const int wave = tid >> 6;
     float sum = 0.0f;
     if (count == 0u)
         return RunningSum{sum, 0u, false};
-    const uint32_t runs = run_of_element(row, count - 1u) + 1u;
+    const uint32_t runs = run_of_element_uniform(row, count - 1u) + 1u;
     uint32_t start = 0; // elements before this one have been added
 
     // The first kSequentialHeadOfRuns elements are added one by one, as the CPU does (every thread runs the
@@ -432,7 +576,7 @@ __device__ __forceinline__ RunningSum exact_running_sum_runs(
     // which would cost the scan below a round, and a stop condition usually holds this early.
     {
         const uint32_t head_runs = min(runs, static_cast<uint32_t>(kWaveSize));
-        const float head_term = static_cast<uint32_t>(lane) < head_runs ? row_term<PHASE>(row, static_cast<uint32_t>(lane)) : 0.0f;
+        const float head_term = static_cast<uint32_t>(lane) < head_runs ? term_of_run(static_cast<uint32_t>(lane)) : 0.0f;
         const uint32_t head_end = static_cast<uint32_t>(lane) < head_runs ? min(row.run_ends[lane], count) : 0u;
         const uint32_t head_limit = min(count, static_cast<uint32_t>(kSequentialHeadOfRuns));
         for (uint32_t run = 0; run < head_runs && start < head_limit; ++run)
@@ -449,20 +593,24 @@ __device__ __forceinline__ RunningSum exact_running_sum_runs(
         if (start >= count)
             return RunningSum{sum, 0u, false};
     }
-    const uint32_t first_run = run_of_element(row, start);
-    for (uint32_t base = first_run; base < runs; base += kReplayChunk)
+    const uint32_t first_run = run_of_element_uniform(row, start);
+    if (tid == 0)
+        scratch.first_event[0] = 0xffffffffu;
+    uint32_t round = 0;
+    for (uint32_t base = first_run; base < runs; base += kRunsChunk)
     {
-        const uint32_t chunk_end = min(runs, base + static_cast<uint32_t>(kReplayChunk));
-        const uint32_t thread_first = base + static_cast<uint32_t>(tid) * kReplayPerThread;
-        float terms[kReplayPerThread];
-        uint32_t firsts[kReplayPerThread]; // first and one-past-last element of each run, clipped to count
-        uint32_t lasts[kReplayPerThread];
+        const uint32_t chunk_end = min(runs, base + static_cast<uint32_t>(kRunsChunk));
+        const uint32_t thread_first = base + static_cast<uint32_t>(tid) * kRunsPerThread;
+        float terms[kRunsPerThread];
+        uint32_t firsts[kRunsPerThread]; // first and one-past-last element of each run, clipped to count
+        uint32_t lasts[kRunsPerThread];
+        const bool summing = tid < kSumThreads;
 #pragma unroll
-        for (int j = 0; j < kReplayPerThread; ++j)
+        for (int j = 0; j < kRunsPerThread; ++j)
         {
             const uint32_t i = thread_first + j;
-            const bool valid = i < chunk_end;
-            terms[j] = valid ? row_term<PHASE>(row, i) : 0.0f;
+            const bool valid = summing && i < chunk_end;
+            terms[j] = valid ? term_of_run(i) : 0.0f;
             firsts[j] = valid ? run_first_element(row, i) : 0u;
             lasts[j] = valid ? min(row.run_ends[i], count) : 0u;
         }
@@ -474,126 +622,104 @@ __device__ __forceinline__ RunningSum exact_running_sum_runs(
             decode_sum(sum, exponent, mantissa);
             const uint32_t stop_at = stop_mantissa(mode, bound, exponent);
             const uint32_t limit = min(stop_at, kBinadeFull);
+            const uint32_t slot = round & 1u;
+            ++round;
+            NCNN_MOE_COUNT(blockIdx.x, 15, 13);
 
+            // A run of m equal terms moves the mantissa m times by the term's step - unless the term ends exactly
+            // half an ulp above a multiple of the ulp (its two steps differ): a wave that holds such a term
+            // composes its totals again the long way.
             ParityStep thread_total{0u, 0u};
-            ParityStep first_step{0u, 0u};
-#pragma unroll
-            for (int j = 0; j < kReplayPerThread; ++j)
+            bool tie = false;
+            ParityStep first_single{0u, 0u};
+            uint32_t first_multiplicity = 0;
+            if (summing)
             {
-                const uint32_t low = max(firsts[j], start);
-                const uint32_t multiplicity = lasts[j] > low ? lasts[j] - low : 0u;
-                const ParityStep single = step_of_term(terms[j], exponent);
-                if (j == 0)
-                    first_step = multiplicity > 0u ? single : ParityStep{0u, 0u};
-                thread_total = compose_steps(thread_total, repeat_steps(single, multiplicity));
-            }
-            if (tid == 0)
-            {
-                scratch.first_event = 0xffffffffu;
-                // the largest remaining term of the row does not move the sum: nothing later can
-                scratch.absorbed = (PHASE == 0 && fresh && base > first_run && first_step.even == 0u && first_step.odd == 0u) ? 1 : 0;
-            }
-            ParityStep inclusive = thread_total;
 #pragma unroll
-            for (int step = 1; step < kWaveSize; step <<= 1)
-            {
-                ParityStep earlier;
-                earlier.even = __shfl_up(inclusive.even, step, kWaveSize);
-                earlier.odd = __shfl_up(inclusive.odd, step, kWaveSize);
-                if (lane >= step)
-                    inclusive = compose_steps(earlier, inclusive);
-            }
-            ParityStep exclusive;
-            exclusive.even = __shfl_up(inclusive.even, 1, kWaveSize);
-            exclusive.odd = __shfl_up(inclusive.odd, 1, kWaveSize);
-            if (lane == 0)
-                exclusive = ParityStep{0u, 0u};
-            if (lane == kWaveSize - 1)
-                scratch.wave_totals[wave] = inclusive;
-            __syncthreads();
-            if (scratch.absorbed)
-                return RunningSum{sum, 0u, false};
-            // every wave's total is read at once (independent LDS loads); the composition stays in registers
-            ParityStep totals[kReplayWaves];
-#pragma unroll
-            for (int w = 0; w < kReplayWaves; ++w)
-                totals[w] = scratch.wave_totals[w];
-            ParityStep before{0u, 0u};
-#pragma unroll
-            for (int w = 0; w < kReplayWaves - 1; ++w)
-            {
-                if (w < wave)
-                    before = compose_steps(before, totals[w]);
-            }
-            before = compose_steps(before, exclusive);
-            uint32_t current = mantissa + ((mantissa & 1u) ? before.odd : before.even);
-
-            bool have_event = false;
-            uint32_t event_key = 0;
-            uint32_t event_mantissa = 0;
-            float event_term = 0.0f;
-#pragma unroll
-            for (int j = 0; j < kReplayPerThread; ++j)
-            {
-                const uint32_t low = max(firsts[j], start);
-                const uint32_t multiplicity = lasts[j] > low ? lasts[j] - low : 0u;
-                const ParityStep single = step_of_term(terms[j], exponent);
-                const bool odd = (current & 1u) != 0u;
-                const uint32_t next = current + repeated_step(odd, single, multiplicity);
-                // A thread that starts at or beyond the limit comes after the round's first event (the
-                // mantissa never decreases and began below the limit), so its own cannot be the first:
-                // it skips the search.  (A round that begins at the limit keeps every thread's event.)
-                if (multiplicity > 0u && !have_event && next >= limit && (current < limit || mantissa >= limit))
+                for (int j = 0; j < kRunsPerThread; ++j)
                 {
-                    // the first addition of the run after which the mantissa reaches the limit
-                    uint32_t none = 0u, some = multiplicity; // repeated additions: `none` stay below, `some` reach it
-                    while (some - none > 1u)
+                    const uint32_t low = max(firsts[j], start);
+                    const uint32_t multiplicity = lasts[j] > low ? lasts[j] - low : 0u;
+                    const ParityStep single = step_of_term(terms[j], exponent);
+                    if (j == 0)
                     {
-                        const uint32_t middle = none + ((some - none) >> 1);
-                        if (current + repeated_step(odd, single, middle) >= limit)
-                            some = middle;
-                        else
-                            none = middle;
+                        first_single = single;
+                        first_multiplicity = multiplicity;
                     }
-                    const uint32_t before_event = current + repeated_step(odd, single, none);
-                    const uint32_t after_event = before_event + ((before_event & 1u) ? single.odd : single.even);
-                    const uint32_t element = low + none;
-                    have_event = true;
-                    if (after_event >= kBinadeFull)
+                    tie = tie || (single.even != single.odd && multiplicity != 0u);
+                    const uint64_t product = static_cast<uint64_t>(single.even) * multiplicity;
+                    const uint32_t repeated = product > kStepCap ? kStepCap : static_cast<uint32_t>(product);
+                    thread_total = compose_steps(thread_total, ParityStep{repeated, repeated});
+                }
+                if (__builtin_amdgcn_ballot_w64(tie) != 0ull)
+                {
+                    thread_total = ParityStep{0u, 0u};
+                    const uint32_t last_run = min(thread_first + static_cast<uint32_t>(kRunsPerThread), chunk_end);
+#pragma unroll 1
+                    for (uint32_t run = thread_first; run < last_run; ++run)
                     {
-                        event_key = element << 1;
-                        event_mantissa = before_event;
-                        event_term = terms[j];
-                    }
-                    else
-                    {
-                        event_key = (element << 1) | 1u;
-                        event_mantissa = after_event;
+                        const uint32_t low = max(run_first_element(row, run), start);
+                        const uint32_t high = min(row.run_ends[run], count);
+                        const uint32_t multiplicity = high > low ? high - low : 0u;
+                        const ParityStep single = step_of_term(term_of_run(run), exponent);
+                        thread_total = compose_steps(
+                            thread_total, ParityStep{repeated_step(false, single, multiplicity), repeated_step(true, single, multiplicity)});
                     }
                 }
-                current = next;
             }
-            if (have_event)
-                atomicMin(&scratch.first_event, event_key);
-            if (tid == kReplayThreads - 1)
-                scratch.final_mantissa = current;
-            __syncthreads();
-            const uint32_t event = scratch.first_event;
-            if (event == 0xffffffffu)
+            if (FIRST)
             {
-                sum = encode_sum(exponent, scratch.final_mantissa);
-                __syncthreads();
+                // the largest remaining term of the row does not move the sum: nothing later can
+                if (tid == 0)
+                    scratch.absorbed[slot] =
+                        (fresh && base > first_run && (first_multiplicity == 0u || (first_single.even == 0u && first_single.odd == 0u))) ? 1 : 0;
+            }
+            const auto find_event = [&](uint32_t current, RoundEvent& found) -> bool {
+                // (one thread of a round, in few rounds: a short loop that reads the runs again)
+                const uint32_t last_run = min(thread_first + static_cast<uint32_t>(kRunsPerThread), chunk_end);
+#pragma unroll 1
+                for (uint32_t run = thread_first; run < last_run; ++run)
+                {
+                    const uint32_t low = max(run_first_element(row, run), start);
+                    const uint32_t high = min(row.run_ends[run], count);
+                    const uint32_t multiplicity = high > low ? high - low : 0u;
+                    const float term = term_of_run(run);
+                    const ParityStep single = step_of_term(term, exponent);
+                    const bool odd = (current & 1u) != 0u;
+                    const uint32_t next = current + repeated_step(odd, single, multiplicity);
+                    if (multiplicity > 0u && next >= limit)
+                    {
+                        // the first addition of the run after which the mantissa reaches the limit
+                        uint32_t none = 0u, some = multiplicity; // repeated additions: `none` stay below, `some` reach it
+                        while (some - none > 1u)
+                        {
+                            const uint32_t middle = none + ((some - none) >> 1);
+                            if (current + repeated_step(odd, single, middle) >= limit)
+                                some = middle;
+                            else
+                                none = middle;
+                        }
+                        const uint32_t before_event = current + repeated_step(odd, single, none);
+                        const uint32_t after_event = apply_step(before_event, single);
+                        const uint32_t element = low + none;
+                        if (after_event >= kBinadeFull)
+                            found = RoundEvent{element << 1, before_event, term};
+                        else
+                            found = RoundEvent{(element << 1) | 1u, after_event, 0.0f};
+                        return true;
+                    }
+                    current = next;
+                }
+                return false;
+            };
+            uint32_t event = 0;
+            const RoundOutcome outcome =
+                finish_round<FIRST>(thread_total, exponent, mantissa, limit, find_event, scratch, slot, tid, sum, event);
+            if (outcome == kRoundAbsorbed)
+                return RunningSum{sum, 0u, false};
+            if (outcome == kRoundPlain)
                 break;
-            }
-            if (have_event && event_key == event)
-            {
-                const float at_event = encode_sum(exponent, event_mantissa);
-                scratch.event_sum = (event & 1u) ? at_event : at_event + event_term;
-            }
-            __syncthreads();
-            sum = scratch.event_sum;
             const uint32_t event_element = event >> 1;
-            __syncthreads();
             if (event & 1u)
                 return RunningSum{sum, event_element, true};
             if ((mode == kStopAtOrAbove && sum >= bound) || (mode == kStopAbove && sum > bound))
@@ -603,6 +729,14 @@ __device__ __forceinline__ RunningSum exact_running_sum_runs(
         }
     }
     return RunningSum{sum, 0u, false};
+}
+
+template <int PHASE>
+__device__ __forceinline__ RunningSum exact_running_sum_runs(
+    const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
+{
+    return exact_running_sum_runs_scaled<PHASE == 0>(
+        row, row.normalizer, PHASE == 2 ? row.renormalizer : 1.0f, count, mode, bound, scratch, tid);
 }
 
 // The CPU sampler from the sorted Top-K window onwards (src/engine/session.cpp:89-134, :429-442) for a
@@ -617,12 +751,14 @@ template <bool RUNS, typename TokenAt>
 __device__ __forceinline__ void replay_sorted_window(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
     const uint32_t* keys, const uint32_t* run_ends, uint32_t run_count, uint32_t n,
-    const uint32_t* sorted_indices, uint8_t flags, ReplayScratch& scratch, int tid, TokenAt token_at)
+    const uint32_t* sorted_indices, uint8_t flags, ReplayScratch& scratch, int tid, TokenAt token_at,
+    const float* terms0 = nullptr)
 {
     SortedRow sorted;
     sorted.keys = keys;
     sorted.run_ends = run_ends;
     sorted.run_count = run_count;
+    sorted.terms0 = terms0;
     sorted.temperature = p.temperature;
     sorted.maximum = value_from_descending_key(keys[0]) / p.temperature;
     sorted.normalizer = 1.0f;
@@ -635,14 +771,15 @@ __device__ __forceinline__ void replay_sorted_window(
             return exact_running_sum<kPhase>(sorted, count, mode, bound, scratch, tid);
     };
     // the item (element, or run) that holds an element
-    auto item_of = [&](uint32_t element) -> uint32_t {
+    auto item_of = [&](uint32_t element) -> uint32_t { // for an element that the whole wave asks for
         if constexpr (RUNS)
-            return run_of_element(sorted, element);
+            return run_of_element_uniform(sorted, element);
         else
             return element;
     };
 
     // ---- normaliser (session.cpp:92-103).  A first term that is not finite poisons the sum.
+    NCNN_MOE_STAMP_RESET(blockIdx.x, 13);
     const float first_term = row_term<0>(sorted, 0);
     float normalizer = first_term;
     if (is_finite_f32(first_term))
@@ -654,31 +791,28 @@ __device__ __forceinline__ void replay_sorted_window(
         return;
     }
     sorted.normalizer = normalizer;
+    NCNN_MOE_STAMP(blockIdx.x, 15, 3);
 
     // ---- Min-P (session.cpp:107-117): probabilities are non-increasing, so the survivors are a prefix
     uint32_t candidates = n;
     if (p.min_p > 0.0f)
     {
         const float threshold = row_term<1>(sorted, 0) * p.min_p;
-        uint32_t first = 0, last = RUNS ? item_of(n - 1u) + 1u : n; // first item whose probability is below the threshold
-        while (first < last)
-        {
-            const uint32_t middle = (first + last) >> 1;
-            if (row_term<1>(sorted, middle) >= threshold)
-                first = middle + 1;
-            else
-                last = middle;
-        }
+        // first item whose probability is below the threshold
+        const uint32_t first = wave_partition_point(
+            RUNS ? item_of(n - 1u) + 1u : n, [&sorted, threshold](uint32_t item) { return row_term<1>(sorted, item) >= threshold; });
         if constexpr (RUNS)
             candidates = min(n, run_first_element(sorted, first));
         else
             candidates = first;
     }
 
+    NCNN_MOE_STAMP(blockIdx.x, 15, 4);
     // ---- Top-P (session.cpp:119-128) and the renormaliser (:130-132), which adds the same values
     const RunningSum nucleus = running_sum(std::integral_constant<int, 1>{}, candidates, kStopAtOrAbove, p.top_p);
     const uint32_t kept = nucleus.stopped ? nucleus.stop_index + 1u : candidates;
     sorted.renormalizer = nucleus.sum;
+    NCNN_MOE_STAMP(blockIdx.x, 15, 5);
 
     if (a.distribution_count != nullptr && sorted_indices != nullptr)
     {
@@ -687,7 +821,7 @@ __device__ __forceinline__ void replay_sorted_window(
         for (uint32_t i = tid; i < limit; i += kReplayThreads)
         {
             a.distribution_ids[first + i] = static_cast<int32_t>(sorted_indices[i]);
-            a.distribution_probabilities[first + i] = row_term<2>(sorted, item_of(i));
+            a.distribution_probabilities[first + i] = row_term<2>(sorted, RUNS ? run_of_element(sorted, i) : i);
         }
         if (tid == 0)
             a.distribution_count[row] = kept;
@@ -704,9 +838,12 @@ __device__ __forceinline__ void replay_sorted_window(
     // ---- inverse-CDF draw over the kept prefix (session.cpp:432-442)
     const RunningSum draw = running_sum(std::integral_constant<int, 2>{}, kept, kStopAbove, a.uniforms[row]);
     const uint32_t selected = draw.stopped ? draw.stop_index : kept - 1u;
+    NCNN_MOE_STAMP(blockIdx.x, 15, 6);
     const int32_t token = token_at(selected);
+    NCNN_MOE_STAMP(blockIdx.x, 15, 7);
+    const float probability = row_term<2>(sorted, item_of(selected)); // (item_of: every lane takes part)
     if (tid == 0)
-        write_token(a, row, p, token, row_term<2>(sorted, item_of(selected)), kept, 1, flags);
+        write_token(a, row, p, token, probability, kept, 1, flags);
 }
 
 } // namespace ncnn_moe_hip

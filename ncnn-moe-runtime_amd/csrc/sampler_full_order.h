@@ -274,15 +274,423 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
     }
 }
 
+// ---- the same sort with a row spread over several workgroups.  A batch rarely holds more full-order
+// rows than the GPU has compute units (a service batch of 512 rows: about a hundred), and one workgroup
+// per row leaves the rest idle while each row takes the whole latency of four passes.  Here part g of a
+// row owns a fixed range of tiles; every pass is two launches over a (parts, rows) grid:
+//   sort_part_histogram_kernel  counts the pass's digits in each part, in the order the keys have NOW
+//   sort_part_scatter_kernel    gives part g, for digit d, the positions behind all smaller digits of
+//       the row and behind digit d's keys of the parts before it, and moves its tiles as the one-workgroup
+//       kernel does (stable inside the part, parts in order: stable over the row).
+// Pass p reads the logits (p = 0) or keys[(p + 1) & 1] and writes keys[p & 1]; four passes for fp32,
+// two for bf16 rows that carry indices.
+template <int DTYPE, bool PAIRS>
+__device__ __forceinline__ void load_sort_keys(
+    const SamplerArgs& a, uint32_t row, int pass, uint32_t first, uint32_t n, int tid_in_group, int group_stride,
+    uint32_t (&out_keys)[kSortPerThread], uint32_t (&out_indices)[kSortPerThread])
+{
+    const char* row_pointer = static_cast<const char*>(a.logits) +
+        static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
+    const uint32_t* source_keys = a.sort_keys[(pass + 1) & 1] + row * a.sort_stride;
+    const uint32_t* source_indices = a.sort_indices[(pass + 1) & 1] + row * a.sort_stride;
+#pragma unroll
+    for (int e = 0; e < kSortPerThread; ++e)
+    {
+        const uint32_t i = first + static_cast<uint32_t>(e * group_stride + tid_in_group);
+        const uint32_t source = i < n ? i : n - 1u; // always a valid address; masked below
+        uint32_t key;
+        uint32_t index = i;
+        if (pass == 0)
+            key = descending_key(load_logit<DTYPE>(row_pointer, source));
+        else
+        {
+            key = source_keys[source];
+            if (PAIRS)
+                index = source_indices[source];
+        }
+        out_keys[e] = i < n ? key : 0xffffffffu;
+        out_indices[e] = i < n ? index : i;
+    }
+}
+
+template <int DTYPE>
+__global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(SamplerArgs a)
+{
+    constexpr int kFirstDigit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0 : 2;
+    const uint32_t part = blockIdx.x;
+    const uint32_t row = blockIdx.y;
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+        return;
+    const int tid = threadIdx.x;
+    const uint32_t n = a.vocab;
+    const int pass = static_cast<int>(a.sort_pass);
+    const int shift = 8 * (pass + kFirstDigit);
+    __shared__ uint32_t counts[256];
+    if (tid < 256)
+        counts[tid] = 0;
+    __syncthreads();
+    const uint32_t first_tile = part * a.sort_tiles_per_part * kSortTile;
+    const uint32_t end = min(n, first_tile + a.sort_tiles_per_part * kSortTile);
+    for (uint32_t tile = first_tile; tile < end; tile += kSortTile)
+    {
+        uint32_t keys[kSortPerThread];
+        uint32_t unused[kSortPerThread];
+        load_sort_keys<DTYPE, false>(a, row, pass, tile, n, tid, kSortThreads, keys, unused);
+#pragma unroll
+        for (int e = 0; e < kSortPerThread; ++e)
+        {
+            if (tile + static_cast<uint32_t>(e * kSortThreads + tid) < n)
+                atomicAdd(&counts[(keys[e] >> shift) & 255u], 1u);
+        }
+    }
+    __syncthreads();
+    if (tid < 256)
+        a.sort_part_counts[(static_cast<size_t>(row) * a.sort_parts + part) * 256 + tid] = counts[tid];
+}
+
+template <int DTYPE, bool PAIRS>
+__global__ __launch_bounds__(kSortThreads) void sort_part_scatter_kernel(SamplerArgs a)
+{
+    constexpr int kFirstDigit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0 : 2;
+    const uint32_t part = blockIdx.x;
+    const uint32_t row = blockIdx.y;
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+        return;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const uint32_t n = a.vocab;
+    const int pass = static_cast<int>(a.sort_pass);
+    const int shift = 8 * (pass + kFirstDigit);
+
+    __shared__ uint32_t digit_base[256];          // output position of the next key of each digit
+    __shared__ uint32_t wave_counts[kSortWaves][256];
+    __shared__ uint32_t tile_start[256];          // first slot of each digit in the staged tile
+    __shared__ uint32_t global_offset[256];       // output position minus staged slot, per digit
+    __shared__ uint32_t scan_partial[4];
+    __shared__ uint32_t staged_keys[kSortTile];   // the tile ordered by digit, written out in runs
+    __shared__ uint32_t staged_indices[PAIRS ? kSortTile : 1];
+
+    uint32_t* target_keys = a.sort_keys[pass & 1] + row * a.sort_stride;
+    uint32_t* target_indices = a.sort_indices[pass & 1] + row * a.sort_stride;
+
+    // where this part's keys of every digit go: behind the row's smaller digits and behind the same
+    // digit's keys of the parts before this one
+    {
+        uint32_t row_total = 0, before = 0, inclusive = 0;
+        if (tid < 256)
+        {
+            const uint32_t* counts = a.sort_part_counts + static_cast<size_t>(row) * a.sort_parts * 256 + tid;
+            for (uint32_t g = 0; g < a.sort_parts; ++g)
+            {
+                const uint32_t c = counts[static_cast<size_t>(g) * 256];
+                row_total += c;
+                before += g < part ? c : 0u;
+            }
+            inclusive = row_total;
+#pragma unroll
+            for (int step = 1; step < kWaveSize; step <<= 1)
+            {
+                const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
+                if (lane >= step)
+                    inclusive += up;
+            }
+            if (lane == kWaveSize - 1)
+                scan_partial[wave] = inclusive;
+        }
+        __syncthreads();
+        if (tid < 256)
+        {
+            uint32_t start = inclusive - row_total;
+#pragma unroll
+            for (int w = 0; w < 3; ++w) // tid < 256: waves 0 to 3
+                start += w < wave ? scan_partial[w] : 0u;
+            digit_base[tid] = start + before;
+        }
+        __syncthreads();
+    }
+
+    const uint32_t first_tile = part * a.sort_tiles_per_part * kSortTile;
+    const uint32_t end = min(n, first_tile + a.sort_tiles_per_part * kSortTile);
+    if (first_tile >= end)
+        return;
+    // A wave owns 512 consecutive keys of a tile and ranks them in 8 rounds of 64, so that the order
+    // inside the wave is the input order (see general_sort_kernel).
+    uint32_t tile_keys[kSortPerThread];
+    uint32_t tile_indices[kSortPerThread];
+    load_sort_keys<DTYPE, PAIRS>(a, row, pass, first_tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread), n, lane, kWaveSize,
+                                 tile_keys, tile_indices);
+    for (uint32_t tile = first_tile; tile < end; tile += kSortTile)
+    {
+        uint32_t next_keys[kSortPerThread];
+        uint32_t next_indices[kSortPerThread];
+        const uint32_t next_tile = tile + kSortTile < end ? tile + kSortTile : tile;
+        load_sort_keys<DTYPE, PAIRS>(a, row, pass, next_tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread), n, lane, kWaveSize,
+                                     next_keys, next_indices);
+        for (int i = tid; i < kSortWaves * 256; i += kSortThreads)
+            (&wave_counts[0][0])[i] = 0;
+        uint32_t tile_ranks[kSortPerThread];
+        const uint32_t wave_first = tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread);
+        lds_barrier();
+#pragma unroll
+        for (int e = 0; e < kSortPerThread; ++e)
+        {
+            const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+            const bool valid = i < n;
+            const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+            uint64_t peers = __ballot(valid);
+#pragma unroll
+            for (int b = 0; b < 8; ++b)
+            {
+                const bool bit = (digit >> b) & 1u;
+                const uint64_t set = __ballot(valid && bit);
+                peers &= bit ? set : ~set;
+            }
+            const int rank_in_round = lanes_below(peers);
+            uint32_t seen = 0;
+            if (valid)
+                seen = wave_counts[wave][digit];
+            tile_ranks[e] = seen + static_cast<uint32_t>(rank_in_round);
+            if (valid && rank_in_round == 0)
+                wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popcll(peers));
+        }
+        lds_barrier();
+        uint32_t digit_total = 0;
+        uint32_t inclusive = 0;
+        if (tid < 256)
+        {
+            uint32_t counts[kSortWaves];
+#pragma unroll
+            for (int w = 0; w < kSortWaves; ++w)
+                counts[w] = wave_counts[w][tid];
+#pragma unroll
+            for (int w = 0; w < kSortWaves; ++w)
+            {
+                wave_counts[w][tid] = digit_total;
+                digit_total += counts[w];
+            }
+            inclusive = digit_total;
+#pragma unroll
+            for (int step = 1; step < kWaveSize; step <<= 1)
+            {
+                const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
+                if (lane >= step)
+                    inclusive += up;
+            }
+            if (lane == kWaveSize - 1)
+                scan_partial[wave] = inclusive;
+        }
+        lds_barrier();
+        if (tid < 256)
+        {
+            uint32_t start = inclusive - digit_total;
+#pragma unroll
+            for (int w = 0; w < 3; ++w)
+                start += w < wave ? scan_partial[w] : 0u;
+            tile_start[tid] = start;
+            global_offset[tid] = digit_base[tid] - start;
+            digit_base[tid] += digit_total;
+        }
+        lds_barrier();
+#pragma unroll
+        for (int e = 0; e < kSortPerThread; ++e)
+        {
+            const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+            if (i < n)
+            {
+                const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+                const uint32_t slot = tile_start[digit] + wave_counts[wave][digit] + tile_ranks[e];
+                staged_keys[slot] = tile_keys[e];
+                if (PAIRS)
+                    staged_indices[slot] = tile_indices[e];
+            }
+        }
+        lds_barrier();
+        const uint32_t tile_count = min(static_cast<uint32_t>(kSortTile), n - tile);
+#pragma unroll
+        for (int e = 0; e < kSortPerThread; ++e)
+        {
+            const uint32_t slot = static_cast<uint32_t>(e * kSortThreads + tid);
+            if (slot < tile_count)
+            {
+                const uint32_t key = staged_keys[slot];
+                const uint32_t position = global_offset[(key >> shift) & 255u] + slot;
+                target_keys[position] = key;
+                if (PAIRS)
+                    target_indices[position] = staged_indices[slot];
+            }
+        }
+        lds_barrier();
+#pragma unroll
+        for (int e = 0; e < kSortPerThread; ++e)
+        {
+            tile_keys[e] = next_keys[e];
+            tile_indices[e] = next_indices[e];
+        }
+    }
+}
+
 // bf16 rows without token indices: the 65536 possible keys are counted instead of sorted.  The keys of
 // a bf16 row differ only in their upper 16 bits, and sampling needs the sorted keys alone, so the
 // sorted row is its histogram: it is written as RUNS, one (key, end position) pair per key that occurs,
-// in descending order of the logits, and the replay adds a run of equal terms in one step.  Two
-// rounds of 32768 LDS counters (non-negative logits first: they sort first): count with LDS atomics,
-// scan the counters and the flags "occurs", write the runs.  One workgroup per row.  Run keys go to
-// sort_keys[1], run ends to sort_keys[0], the number of runs to the row's first word of sort_indices[0].
-constexpr int kCountBins = 32768;
+// in descending order of the logits, and the replay adds a run of equal terms in one step.  One
+// workgroup per row.  Run keys go to sort_keys[1], run ends to sort_keys[0], the number of runs to the
+// row's first word of sort_indices[0].
+//
+// The row is read once: 65536 counters of 16 bits, two to an LDS word (key16 2w in the lower half, 2w + 1
+// in the upper), counted with one LDS atomic per logit.  A counter that passes 65535 carries into its
+// neighbour or out of the word; every such carry makes the sum of the decoded counters smaller than the
+// number of logits (by 65535 or 65536 per carry, never larger), so the sum is the test: a row that fails it
+// (some value occurs 65536 times or more) is counted again in two rounds of 32768 counters of 32 bits.
+constexpr int kCountWords = 32768;
 constexpr int kCachedRuns = 6144; // runs of a row the replay keeps in LDS (48 KB)
+
+// Counts the row's keys into `bins`.  PACKED: every key, 16-bit counters; else the keys whose top bit is
+// `round`, 32-bit counters indexed by the lower 15 bits.  16-byte loads of eight logits, four per thread
+// and batch, the next batch in flight while this one is counted; the row is read from the 16-byte
+// boundary below its first element.
+template <bool PACKED>
+__device__ __forceinline__ void count_bf16_keys(
+    const uint16_t* aligned_logits, uint32_t misalignment, uint32_t aligned_end, uint32_t round, uint32_t* bins, int tid)
+{
+    constexpr uint32_t kBatch = 4u * 8u * kSortThreads;
+    const auto load_batch = [&](uint32_t first, uint4 (&raw)[4]) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+            const uint32_t position = first + static_cast<uint32_t>(k * kSortThreads + tid) * 8u;
+            raw[k] = *reinterpret_cast<const uint4*>(aligned_logits + (position < aligned_end ? position : 0u));
+        }
+    };
+    uint4 raw[4];
+    load_batch(0, raw);
+    for (uint32_t first = 0; first < aligned_end; first += kBatch)
+    {
+        uint4 next[4];
+        load_batch(first + kBatch < aligned_end ? first + kBatch : first, next);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+            const uint32_t position = first + static_cast<uint32_t>(k * kSortThreads + tid) * 8u;
+            const uint32_t words[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+            {
+                const uint32_t bits = (c & 1) ? (words[c >> 1] >> 16) : (words[c >> 1] & 0xffffu);
+                const uint32_t element = position + c;
+                const uint32_t key16 = descending_key(__uint_as_float(bits << 16)) >> 16;
+                const bool inside = element >= misalignment && element < aligned_end;
+                if (PACKED)
+                {
+                    if (inside)
+                        atomicAdd(&bins[key16 >> 1], (key16 & 1u) ? 0x10000u : 1u);
+                }
+                else if (inside && (key16 >> 15) == round)
+                    atomicAdd(&bins[key16 & 0x7fffu], 1u);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            raw[k] = next[k];
+    }
+}
+
+struct CountScratch
+{
+    uint32_t wave_totals[kSortWaves];
+    uint32_t wave_runs[kSortWaves];
+};
+
+// Turns the counters into runs.  Wave w owns words [2048 w, 2048 (w + 1)) and reads them 64 consecutive
+// words at a time (lane l of trip j: word 2048 w + 64 j + l: no bank conflicts), so the order of the keys
+// inside the wave is (trip, lane, half).  Returns false (and writes nothing) when PACKED counters have
+// overflowed.  key_base: key16 of word 0's first counter; written / runs_written: totals of an earlier round.
+template <bool PACKED>
+__device__ __forceinline__ bool write_runs_of_counts(
+    const uint32_t* bins, uint32_t expected, uint32_t key_base, uint32_t& written, uint32_t& runs_written,
+    uint32_t* run_keys, uint32_t* run_ends, CountScratch& scratch, int tid)
+{
+    constexpr int kTrips = kCountWords / kSortWaves / kWaveSize; // 32
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const uint32_t wave_first_word = static_cast<uint32_t>(wave) * (kTrips * kWaveSize);
+    uint32_t words[kTrips];
+    uint32_t lane_total = 0, lane_runs = 0;
+#pragma unroll
+    for (int j = 0; j < kTrips; ++j)
+    {
+        words[j] = bins[wave_first_word + static_cast<uint32_t>(j * kWaveSize + lane)];
+        if (PACKED)
+        {
+            lane_total += (words[j] & 0xffffu) + (words[j] >> 16);
+            lane_runs += ((words[j] & 0xffffu) != 0u ? 1u : 0u) + ((words[j] >> 16) != 0u ? 1u : 0u);
+        }
+        else
+        {
+            lane_total += words[j];
+            lane_runs += words[j] != 0u ? 1u : 0u;
+        }
+    }
+    const uint32_t wave_total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(lane_total)), 63));
+    const uint32_t wave_run_total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(lane_runs)), 63));
+    if (lane == 0)
+    {
+        scratch.wave_totals[wave] = wave_total;
+        scratch.wave_runs[wave] = wave_run_total;
+    }
+    __syncthreads();
+    uint32_t position = written;      // elements before the keys this wave looks at next
+    uint32_t run = runs_written;      // runs before them
+    uint32_t all = 0, all_runs = 0;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w)
+    {
+        const uint32_t t = scratch.wave_totals[w];
+        const uint32_t r = scratch.wave_runs[w];
+        position += w < wave ? t : 0u;
+        run += w < wave ? r : 0u;
+        all += t;
+        all_runs += r;
+    }
+    __syncthreads(); // the scratch is written again by a later call
+    if (PACKED && all != expected)
+        return false;
+#pragma unroll
+    for (int j = 0; j < kTrips; ++j)
+    {
+        const uint32_t low = PACKED ? (words[j] & 0xffffu) : words[j];
+        const uint32_t high = PACKED ? (words[j] >> 16) : 0u;
+        const uint64_t has_low = __ballot(low != 0u);
+        const uint64_t has_high = PACKED ? __ballot(high != 0u) : 0ull;
+        if ((has_low | has_high) == 0ull)
+            continue;
+        const uint32_t inclusive = wave_prefix_sum_u32(low + high);
+        const uint32_t before = position + inclusive - (low + high);
+        uint32_t slot = run + static_cast<uint32_t>(lanes_below(has_low) + lanes_below(has_high));
+        const uint32_t word = wave_first_word + static_cast<uint32_t>(j * kWaveSize + lane);
+        const uint32_t first_key16 = key_base + (PACKED ? 2u * word : word);
+        // the lower half of a key is all ones for a non-negative logit and for NaN, else zero
+        const auto full_key = [](uint32_t key16) {
+            return key16 == 0xffffu ? 0xffffffffu : (key16 << 16) | ((key16 >> 15) == 0u ? 0xffffu : 0u);
+        };
+        if (low != 0u)
+        {
+            run_keys[slot] = full_key(first_key16);
+            run_ends[slot] = before + low;
+            ++slot;
+        }
+        if (PACKED && high != 0u)
+        {
+            run_keys[slot] = full_key(first_key16 + 1u);
+            run_ends[slot] = before + low + high;
+        }
+        position += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive), 63));
+        run += static_cast<uint32_t>(__popcll(has_low) + __popcll(has_high));
+    }
+    written += all;
+    runs_written += all_runs;
+    return true;
+}
 
 __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(SamplerArgs a)
 {
@@ -290,14 +698,10 @@ __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(Sample
     if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
         return;
     const int tid = threadIdx.x;
-    const int lane = tid & (kWaveSize - 1);
-    const int wave = tid >> 6;
     const uint32_t n = a.vocab;
-    constexpr int kBinsPerThread = kCountBins / kSortThreads;
 
-    __shared__ uint32_t bins[kCountBins];
-    __shared__ uint32_t wave_totals[kSortWaves];
-    __shared__ uint32_t wave_runs[kSortWaves];
+    __shared__ uint32_t bins[kCountWords];
+    __shared__ CountScratch scratch;
 
     const uint16_t* logits = reinterpret_cast<const uint16_t*>(
         static_cast<const char*>(a.logits) + static_cast<size_t>(row) * a.row_stride * 2u);
@@ -307,102 +711,33 @@ __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(Sample
     const uint16_t* aligned_logits = logits - misalignment;
     const uint32_t aligned_end = misalignment + n; // positions [misalignment, aligned_end) hold the row
 
-    uint32_t runs_written = 0; // runs of the earlier round
-    uint32_t written = 0; // keys of the earlier round
-    for (uint32_t round = 0; round < 2; ++round)
+    const auto clear_bins = [&]() {
+        uint4* wide = reinterpret_cast<uint4*>(bins);
+#pragma unroll
+        for (int j = 0; j < kCountWords / 4 / kSortThreads; ++j)
+            wide[j * kSortThreads + tid] = uint4{0u, 0u, 0u, 0u};
+        __syncthreads();
+    };
+    uint32_t runs_written = 0;
+    uint32_t written = 0;
+    NCNN_MOE_STAMP(blockIdx.x, 14, 0);
+    clear_bins();
+    count_bf16_keys<true>(aligned_logits, misalignment, aligned_end, 0u, bins, tid);
+    __syncthreads();
+    NCNN_MOE_STAMP(blockIdx.x, 14, 1);
+    const bool packed_sound =
+        write_runs_of_counts<true>(bins, n, 0u, written, runs_written, run_keys, run_ends, scratch, tid);
+    NCNN_MOE_STAMP(blockIdx.x, 14, 2);
+    if (!packed_sound)
     {
-#pragma unroll
-        for (int j = 0; j < kBinsPerThread; ++j)
-            bins[j * kSortThreads + tid] = 0;
-        __syncthreads();
-        // 16-byte loads of eight logits, four per thread in flight (single dependent 2-byte loads make
-        // the loop latency-bound); the row is read from the 16-byte boundary below its first element
-        for (uint32_t first = 0; first < aligned_end; first += 4u * 8u * kSortThreads)
+        for (uint32_t round = 0; round < 2; ++round)
         {
-            uint4 raw[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-            {
-                const uint32_t position = first + static_cast<uint32_t>(k * kSortThreads + tid) * 8u;
-                raw[k] = *reinterpret_cast<const uint4*>(aligned_logits + (position < aligned_end ? position : 0u));
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-            {
-                const uint32_t position = first + static_cast<uint32_t>(k * kSortThreads + tid) * 8u;
-                const uint32_t words[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
-#pragma unroll
-                for (int c = 0; c < 8; ++c)
-                {
-                    const uint32_t bits = (c & 1) ? (words[c >> 1] >> 16) : (words[c >> 1] & 0xffffu);
-                    const uint32_t element = position + c;
-                    const uint32_t key16 = descending_key(__uint_as_float(bits << 16)) >> 16;
-                    if (element >= misalignment && element < aligned_end && (key16 >> 15) == round)
-                        atomicAdd(&bins[key16 & (kCountBins - 1)], 1u);
-                }
-            }
+            __syncthreads();
+            clear_bins();
+            count_bf16_keys<false>(aligned_logits, misalignment, aligned_end, round, bins, tid);
+            __syncthreads();
+            write_runs_of_counts<false>(bins, 0u, round << 15, written, runs_written, run_keys, run_ends, scratch, tid);
         }
-        __syncthreads();
-        // scan of the counts and of the number of keys that occur: a thread owns kBinsPerThread consecutive bins
-        uint32_t counts[kBinsPerThread];
-        uint32_t thread_total = 0;
-        uint32_t thread_runs = 0;
-#pragma unroll
-        for (int j = 0; j < kBinsPerThread; ++j)
-        {
-            counts[j] = bins[tid * kBinsPerThread + j];
-            thread_total += counts[j];
-            thread_runs += counts[j] != 0u ? 1u : 0u;
-        }
-        uint32_t inclusive = thread_total;
-        uint32_t inclusive_runs = thread_runs;
-#pragma unroll
-        for (int step = 1; step < kWaveSize; step <<= 1)
-        {
-            const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
-            const uint32_t up_runs = __shfl_up(inclusive_runs, step, kWaveSize);
-            if (lane >= step)
-            {
-                inclusive += up;
-                inclusive_runs += up_runs;
-            }
-        }
-        if (lane == kWaveSize - 1)
-        {
-            wave_totals[wave] = inclusive;
-            wave_runs[wave] = inclusive_runs;
-        }
-        __syncthreads();
-        uint32_t before = inclusive - thread_total;
-        uint32_t runs_before = inclusive_runs - thread_runs;
-        uint32_t round_total = 0;
-        uint32_t round_runs = 0;
-        for (int w = 0; w < kSortWaves; ++w)
-        {
-            if (w < wave)
-            {
-                before += wave_totals[w];
-                runs_before += wave_runs[w];
-            }
-            round_total += wave_totals[w];
-            round_runs += wave_runs[w];
-        }
-#pragma unroll
-        for (int j = 0; j < kBinsPerThread; ++j)
-        {
-            if (counts[j] != 0u)
-            {
-                const uint32_t key16 = (round << 15) | static_cast<uint32_t>(tid * kBinsPerThread + j);
-                before += counts[j];
-                // the lower half of a key is all ones for a non-negative logit and for NaN, else zero
-                run_keys[runs_written + runs_before] = key16 == 0xffffu ? 0xffffffffu : (key16 << 16) | (round == 0 ? 0xffffu : 0u);
-                run_ends[runs_written + runs_before] = written + before;
-                ++runs_before;
-            }
-        }
-        written += round_total;
-        runs_written += round_runs;
-        __syncthreads();
     }
     if (tid == 0)
         a.sort_indices[0][row * a.sort_stride] = runs_written;
@@ -418,7 +753,7 @@ struct RecoverScratch
 // the (rank - first position of that key)-th element, in index order, whose key equals keys[rank].
 // Every thread of the workgroup must call it.
 template <int DTYPE>
-__device__ __forceinline__ int32_t recover_token_of_key(
+__device__ __noinline__ int32_t recover_token_of_key(
     const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, RecoverScratch& scratch, int tid);
 
 template <int DTYPE>
@@ -443,7 +778,7 @@ __device__ __forceinline__ int32_t recover_token_index(
 // barrier); the wave whose part holds the wanted match walks it again and locates the element with a
 // scan of the lanes' match counts.  Every thread of the workgroup must call it.
 template <int DTYPE>
-__device__ __forceinline__ int32_t recover_token_of_key(
+__device__ __noinline__ int32_t recover_token_of_key(
     const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, RecoverScratch& scratch, int tid)
 {
     using Vector = LogitsVector<DTYPE>;
@@ -566,27 +901,62 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
         return;
     const int tid = threadIdx.x;
+    NCNN_MOE_STAMP(blockIdx.x, 15, 0);
     const ncnn_moe_sample_params p = a.params[row];
     const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
     const uint32_t* run_ends = RUNS ? a.sort_keys[0] + row * a.sort_stride : nullptr;
+    // exp(logit/T - maximum) of every item, computed once for the three sums that use it (greedy rows add nothing)
+    const float* terms0 = nullptr;
+    const auto term_of_key = [&p](uint32_t key, float maximum) {
+        return expf_libm(value_from_descending_key(key) / p.temperature - maximum);
+    };
     if constexpr (RUNS)
     {
-        // a row of few runs is walked from LDS: its many binary searches are chains of dependent loads
+        // a row of few runs is walked from LDS; the terms of a longer one go to the sort's spare index buffer
         __shared__ uint32_t cached_keys[kCachedRuns];
         __shared__ uint32_t cached_ends[kCachedRuns];
+        __shared__ __align__(16) float cached_terms[kCachedRuns];
         const uint32_t run_total = a.sort_indices[0][row * a.sort_stride];
+        const float maximum = value_from_descending_key(keys[0]) / p.temperature;
         if (run_total <= static_cast<uint32_t>(kCachedRuns))
         {
             for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
             {
-                cached_keys[i] = keys[i];
+                const uint32_t key = keys[i];
+                cached_keys[i] = key;
                 cached_ends[i] = run_ends[i];
+                cached_terms[i] = term_of_key(key, maximum);
             }
             __syncthreads();
             keys = cached_keys;
             run_ends = cached_ends;
+            terms0 = cached_terms;
+        }
+        else
+        {
+            float* terms = reinterpret_cast<float*>(a.sort_indices[1] + row * a.sort_stride);
+            if (p.temperature != 0.0f)
+            {
+                for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
+                    terms[i] = term_of_key(keys[i], maximum);
+            }
+            __syncthreads();
+            terms0 = terms;
         }
     }
+    else
+    {
+        float* terms = reinterpret_cast<float*>(a.sort_keys[0] + row * a.sort_stride);
+        if (a.terms_precomputed == 0 && p.temperature != 0.0f)
+        {
+            const float maximum = value_from_descending_key(keys[0]) / p.temperature;
+            for (uint32_t i = threadIdx.x; i < a.vocab; i += kReplayThreads)
+                terms[i] = term_of_key(keys[i], maximum);
+            __syncthreads();
+        }
+        terms0 = terms;
+    }
+    NCNN_MOE_STAMP(blockIdx.x, 15, 1);
     const bool have_indices = !RUNS && a.distribution_count != nullptr; // the pair sort ran: indices are valid
     const uint32_t* indices = have_indices ? a.sort_indices[1] + row * a.sort_stride : nullptr;
     const uint32_t vocab = a.vocab;
@@ -637,15 +1007,7 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     {
         // a greedy row whose select overflowed (every logit tied): first finite logit in sorted order,
         // non-finite logits skipped (src/engine/session.cpp:404-424)
-        uint32_t low = 0, high = items;
-        while (low < high)
-        {
-            const uint32_t middle = (low + high) >> 1;
-            if (keys[middle] <= kPositiveInfinityKey)
-                low = middle + 1;
-            else
-                high = middle;
-        }
+        const uint32_t low = wave_partition_point(items, [keys](uint32_t item) { return keys[item] <= kPositiveInfinityKey; });
         const bool any_finite = low < items && keys[low] <= kLastFiniteKey;
         int32_t token = -1;
         if (any_finite)
@@ -679,19 +1041,46 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
             write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, flags);
         return;
     }
-    uint32_t low = 0, high = items; // first item whose key is not finite
-    while (low < high)
-    {
-        const uint32_t middle = (low + high) >> 1;
-        if (keys[middle] <= kLastFiniteKey)
-            low = middle + 1;
-        else
-            high = middle;
-    }
+    // first item whose key is not finite
+    const uint32_t low = wave_partition_point(items, [keys](uint32_t item) { return keys[item] <= kLastFiniteKey; });
     uint32_t n = first_element(low);
     if (p.top_k > 0 && p.top_k < vocab && n > p.top_k)
         n = p.top_k;
-    replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at);
+    NCNN_MOE_STAMP(blockIdx.x, 15, 2);
+    replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0);
+}
+
+// exp(logit/T - maximum) of every element of the sorted full-order rows, written over the sort's other key
+// buffer: the replay that follows adds these terms one workgroup per row, and computing them there would
+// put a few dozen instructions per element on that workgroup's path; here the whole GPU shares them.
+// grid (parts, rows).
+constexpr int kTermsThreads = 256;
+constexpr int kTermsPerThread = 8;
+
+__global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(SamplerArgs a)
+{
+    const uint32_t row = blockIdx.y;
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+        return;
+    const float temperature = a.params[row].temperature;
+    const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
+    float* terms = reinterpret_cast<float*>(a.sort_keys[0] + row * a.sort_stride);
+    const float maximum = value_from_descending_key(keys[0]) / temperature;
+    const uint32_t first = blockIdx.x * (kTermsThreads * kTermsPerThread) + threadIdx.x;
+    uint32_t loaded[kTermsPerThread];
+#pragma unroll
+    for (int j = 0; j < kTermsPerThread; ++j)
+    {
+        const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
+        loaded[j] = i < a.vocab ? keys[i] : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < kTermsPerThread; ++j)
+    {
+        const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
+        if (i < a.vocab)
+            terms[i] = expf_libm(value_from_descending_key(loaded[j]) / temperature - maximum);
+    }
 }
 
 } // namespace ncnn_moe_hip

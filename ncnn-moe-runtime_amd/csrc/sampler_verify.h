@@ -403,8 +403,7 @@ __global__ __launch_bounds__(kReplayThreads) void speculative_verify_dense_kerne
             }
             __syncthreads();
             const float* const residual = d.dense_residual;
-            const auto residual_at = [residual](uint32_t i) { return residual[i]; };
-            const RunningSum total = exact_running_sum_of_terms<false>(residual_at, d.vocab, kStopNever, 0.0f, shared.replay, tid);
+            const RunningSum total = exact_running_sum_of_array<false, false>(residual, 1.0f, 1.0f, d.vocab, kStopNever, 0.0f, shared.replay, tid);
             const float normalizer = total.sum;
             if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
             {
@@ -415,7 +414,7 @@ __global__ __launch_bounds__(kReplayThreads) void speculative_verify_dense_kerne
             // uniform_real_distribution<float>(0, normalizer): canonical draw times the range
             const float sample_value = shared.uniforms[accept_draws] * normalizer;
             __syncthreads();
-            const RunningSum walk = exact_running_sum_of_terms<false>(residual_at, d.vocab, kStopAbove, sample_value, shared.replay, tid);
+            const RunningSum walk = exact_running_sum_of_array<false, false>(residual, 1.0f, 1.0f, d.vocab, kStopAbove, sample_value, shared.replay, tid);
             // session.cpp:189-198: past the end, the last token that has any residual mass
             const int selected = walk.stopped ? static_cast<int>(walk.stop_index) : shared.last_positive;
             if (selected < 0)

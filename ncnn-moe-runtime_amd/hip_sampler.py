@@ -69,6 +69,7 @@ EXPORTED_SYMBOLS = [
 TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_force_general",
     "ncnn_moe_hip_sampler_debug_scatter_segments",
+    "ncnn_moe_hip_sampler_debug_spread_sort",
     "ncnn_moe_hip_sampler_debug_expf",
     "ncnn_moe_hip_sampler_debug_exp2_table",
     "ncnn_moe_hip_sampler_debug_select_geometry",
@@ -115,6 +116,7 @@ def load_library():
     lib.ncnn_moe_hip_sampler_device_count.argtypes = []
     lib.ncnn_moe_hip_sampler_debug_force_general.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_scatter_segments.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_spread_sort.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_expf.argtypes = [vp, vp, vp, ctypes.c_size_t]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.argtypes = [vp]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.restype = None
@@ -272,6 +274,10 @@ class HipSampler:
     def scatter_segments(self, enabled):
         """Test hook: split rows are launched without the XCD-aware numbering of the workgroups."""
         self._check(self._lib.ncnn_moe_hip_sampler_debug_scatter_segments(self._handle, 1 if enabled else 0))
+
+    def spread_sort(self, enabled):
+        """Test hook: the radix sort of long full-order rows on several workgroups (default) or on one."""
+        self._check(self._lib.ncnn_moe_hip_sampler_debug_spread_sort(self._handle, 1 if enabled else 0))
 
     def expf(self, values):
         values = np.ascontiguousarray(values, dtype=np.float32)

@@ -473,3 +473,73 @@ def test_windows_around_the_quad_maxima_bound(batch_sampler, dtype):
             select_rows[:] = vocab < 5000   # bf16 rounding makes every row tie-heavy
         _check_rows(batch_sampler, data, params, uniforms, dtype=dtype,
                     context="bound switch, V=%d %s" % (vocab, dtype), select_rows=select_rows)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("vocab", [16384, 16385, 24577, 65536, 109999])
+def test_full_order_rows_sorted_by_several_workgroups(batch_sampler, dtype, vocab):
+    """Full-order rows (no Top-K, nucleus over the whole row) whose radix sort is spread over two to seven
+    workgroups, part boundaries on and off a tile edge, heavy ties and edge rows included: the oracle's
+    results, and byte for byte those of the one-workgroup sort.  The exported distribution takes the sort
+    that carries the token indices."""
+    rng = np.random.default_rng(9100 + vocab)
+    rows = 48
+    logits = (rng.standard_normal((rows, vocab)) * 3.0).astype(np.float32)
+    used = _plant_edge_rows(logits, 8)
+    logits[20, :] = np.round(logits[20, :])            # a few dozen distinct values
+    logits[21, :] = np.float32(0.5)
+    logits[21, vocab - 1] = 4.0                        # the winner is the row's last logit
+    if dtype == "bf16":
+        logits = workloads.float32_to_bf16_bits(logits)
+    params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+    params["temperature"] = rng.uniform(0.4, 1.5, size=rows).astype(np.float32)
+    params["top_p"] = np.where(np.arange(rows) % 3 == 0, 1.0, rng.uniform(0.5, 0.999, size=rows)).astype(np.float32)
+    params["min_p"] = np.where(np.arange(rows) % 4 == 1, rng.uniform(0.0, 0.02, size=rows), 0.0).astype(np.float32)
+    params["top_k"][5::7] = 5000                       # wider than the select kernels take
+    uniforms = rng.random(rows, dtype=np.float32)
+    assert used <= 12
+    spread, _ = _check_rows(batch_sampler, logits, params, uniforms, dtype=dtype, vocab=vocab,
+                            context="full order, %s, V=%d, spread sort" % (dtype, vocab))
+    assert (spread["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).sum() >= rows - 12
+    batch_sampler.spread_sort(False)
+    try:
+        single = batch_sampler.sample(params, uniforms, None)
+    finally:
+        batch_sampler.spread_sort(True)
+    assert spread.tobytes() == single.tobytes()
+    for row in (0, 20):
+        options = dict(temperature=float(params["temperature"][row]), top_k=0, top_p=0.9, min_p=0.0)
+        status, ids, probabilities, count = batch_sampler.distribution(row, **options)
+        oracle_status, oracle_ids, oracle_probabilities = oracle_lib.oracle_distribution(
+            oracle_lib.widen_bf16(logits[row]) if dtype == "bf16" else logits[row], **options)
+        assert status == oracle_status
+        assert count == len(oracle_ids)
+        assert np.array_equal(ids[:count], oracle_ids)
+        assert np.array_equal(probabilities[:count].view(np.uint32), np.asarray(oracle_probabilities, dtype=np.float32).view(np.uint32))
+
+
+def test_bf16_counters_that_overflow_sixteen_bits(batch_sampler):
+    """bf16 full-order rows are counted in 16-bit counters, two to a word; a row in which one value occurs
+    65536 times or more is counted again in 32-bit counters.  Rows just below and at the limit, in the lower
+    and in the upper half of a word (neighbouring bf16 values), in both, and a constant row."""
+    rng = np.random.default_rng(77)
+    vocab = 109999
+    rows = 12
+    logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    low, high = np.float32(1.5), np.float32(1.5078125)   # neighbouring bf16 values: keys 2w and 2w + 1 or the reverse
+    for row, (count_low, count_high) in enumerate([(65535, 0), (65536, 0), (0, 65535), (0, 65536), (65536, 40000),
+                                                    (30000, 65537), (65535, 44464), (109999, 0), (0, 109999)]):
+        order = rng.permutation(vocab)
+        logits[row, order[:count_low]] = low
+        logits[row, order[count_low:count_low + count_high]] = high
+    logits[9, :] = -np.inf
+    logits[9, :70000] = 0.25
+    bits = workloads.float32_to_bf16_bits(logits)
+    params = hip_sampler.make_params(rows, 1.0, 0, 0.95, 0.0)
+    params["temperature"] = rng.uniform(0.5, 1.4, size=rows).astype(np.float32)
+    params["top_p"][::2] = 1.0
+    for trial in range(3):
+        uniforms = rng.random(rows, dtype=np.float32)
+        gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", vocab=vocab,
+                             context="bf16 counters at the 16-bit limit, draw %d" % trial)
+        assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
