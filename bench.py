@@ -519,6 +519,8 @@ def main():
     may_need_full_order = int(np.any(sampled & (effective_k > 64)))
     if np.count_nonzero(sampled & (effective_k > 64) & (effective_k <= 1024)) >= 32 and np.count_nonzero(sampled & (effective_k > 1024)) >= 32:
         may_need_full_order |= hip_sampler.PASSES_SIDE_BY_SIDE  # as a scheduler that knows its Sessions' options would
+    if may_need_full_order and not np.any(sampled & (effective_k > 64) & (effective_k <= 1024)):
+        may_need_full_order |= hip_sampler.PASSES_NO_WIDE_WINDOWS
 
     def step(index):
         sampler.sample_device(

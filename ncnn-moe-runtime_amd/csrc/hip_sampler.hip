@@ -778,9 +778,9 @@ int ncnn_moe_hip_sampler_sample_device(
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "row_stride is smaller than vocab");
     SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
     SamplerPasses passes;
-    passes.wide_select = may_need_full_order != 0;
+    passes.wide_select = may_need_full_order != 0 && (may_need_full_order & NCNN_MOE_PASSES_NO_WIDE_WINDOWS) == 0;
     passes.full_order = may_need_full_order != 0 || s->force_general != 0;
-    passes.side_by_side = (may_need_full_order & NCNN_MOE_PASSES_SIDE_BY_SIDE) != 0;
+    passes.side_by_side = passes.wide_select && (may_need_full_order & NCNN_MOE_PASSES_SIDE_BY_SIDE) != 0;
     return launch_sampler(
         s, device_logits, dtype, rows, vocab, row_stride, device_params, device_uniforms, device_stop_ids,
         device_results, DistributionExport{}, passes, static_cast<hipStream_t>(stream));

@@ -745,7 +745,7 @@ __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(Sample
 
 struct RecoverScratch
 {
-    uint32_t wave_counts[kReplayWaves];
+    uint32_t wave_counts[2][kReplayWaves]; // of alternate trips
     int32_t found;
 };
 
@@ -761,22 +761,16 @@ __device__ __forceinline__ int32_t recover_token_index(
     const void* row_pointer, uint32_t vocab, const uint32_t* keys, uint32_t rank, RecoverScratch& scratch, int tid)
 {
     const uint32_t key = keys[rank];
-    uint32_t low = 0, high = rank; // first position holding this key
-    while (low < high)
-    {
-        const uint32_t middle = (low + high) >> 1;
-        if (keys[middle] < key)
-            low = middle + 1;
-        else
-            high = middle;
-    }
+    // first position holding this key
+    const uint32_t low = wave_partition_point(rank, [keys, key](uint32_t position) { return keys[position] < key; });
     return recover_token_of_key<DTYPE>(row_pointer, vocab, key, rank - low, scratch, tid);
 }
 
-// The ordinal-th element of the row, in index order, whose key equals `key`.  Every wave counts the
-// matches of its own contiguous eighth of the row (16-byte loads, four per lane in flight, no
-// barrier); the wave whose part holds the wanted match walks it again and locates the element with a
-// scan of the lanes' match counts.  Every thread of the workgroup must call it.
+// The ordinal-th element of the row, in index order, whose key equals `key`.  The workgroup reads the row
+// front to back in trips of sixteen consecutive slices, one per wave (16-byte loads, eight per lane in
+// flight); after each trip the waves' match counts tell whether the wanted match lies in it, and the wave
+// whose slice holds it locates the element from the masks it still has in registers.  The row is read
+// once, and only as far as the match.  Every thread of the workgroup must call it.
 template <int DTYPE>
 __device__ __noinline__ int32_t recover_token_of_key(
     const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, RecoverScratch& scratch, int tid)
@@ -784,7 +778,7 @@ __device__ __noinline__ int32_t recover_token_of_key(
     using Vector = LogitsVector<DTYPE>;
     constexpr uint32_t kWidth = Vector::kWidth;
     constexpr int kLoads = 8;
-    constexpr uint32_t kTrip = kLoads * kWaveSize * kWidth; // positions a wave looks at per trip
+    constexpr uint32_t kSlice = kLoads * kWaveSize * kWidth; // positions a wave looks at per trip
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
     // positions count from the 16-byte boundary below the row: [misalignment, end) hold the row
@@ -792,98 +786,105 @@ __device__ __noinline__ int32_t recover_token_of_key(
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row_pointer) & 15u) / Vector::kElementBytes;
     const char* aligned_base = static_cast<const char*>(row_pointer) - static_cast<size_t>(misalignment) * Vector::kElementBytes;
     const uint32_t end = misalignment + vocab;
-    const uint32_t part = ((end + kReplayWaves - 1u) / kReplayWaves + kWidth - 1u) / kWidth * kWidth;
-    const uint32_t part_begin = min(end, static_cast<uint32_t>(wave) * part);
-    const uint32_t part_end = min(end, part_begin + part);
 
-    // per load k of a trip: the lane's matches among the kWidth positions from first + (k * 64 + lane) * kWidth
-    auto match_masks = [&](uint32_t first, uint32_t (&masks)[kLoads]) {
+    // An element matches when its key equals `key`.  Keys are one-to-one with the logits' bit patterns except
+    // that the two zeros share a key, and all NaNs another: the raw bits are compared (with the sign masked for
+    // zero), which takes a third of the instructions of building every element's key.
+    constexpr uint32_t kAbsoluteBits = DTYPE == NCNN_MOE_LOGITS_F32 ? 0x7fffffffu : 0x7fffu;
+    constexpr uint32_t kInfinityBits = DTYPE == NCNN_MOE_LOGITS_F32 ? 0x7f800000u : 0x7f80u;
+    const bool wants_nan = key == 0xffffffffu;
+    const uint32_t value_bits = __float_as_uint(value_from_descending_key(key));
+    const uint32_t pattern = DTYPE == NCNN_MOE_LOGITS_F32 ? value_bits : value_bits >> 16;
+    const uint32_t compared = (pattern & kAbsoluteBits) == 0u ? kAbsoluteBits : 0xffffffffu;
+    const auto matches_key = [&](uint32_t bits) {
+        const bool is_nan = (bits & kAbsoluteBits) > kInfinityBits;
+        return wants_nan ? is_nan : ((bits ^ pattern) & compared) == 0u;
+    };
+
+    if (tid == 0)
+        scratch.found = -1;
+    uint32_t seen = 0; // matches in the trips before this one
+    uint32_t parity = 0;
+    for (uint32_t trip = 0; trip < end; trip += kSlice * kReplayWaves, parity ^= 1u)
+    {
+        const uint32_t first = trip + static_cast<uint32_t>(wave) * kSlice;
+        // per load k: the lane's matches among the kWidth positions from first + (k * 64 + lane) * kWidth
         uint4 raw[kLoads];
 #pragma unroll
         for (int k = 0; k < kLoads; ++k)
         {
             const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth;
-            raw[k] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(position < part_end ? position : part_begin) * Vector::kElementBytes);
+            raw[k] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(position < end ? position : 0u) * Vector::kElementBytes);
         }
+        uint32_t masks[kLoads];
+        uint32_t lane_matches = 0;
 #pragma unroll
         for (int k = 0; k < kLoads; ++k)
         {
             const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth;
-            float values[kWidth];
-            Vector::unpack(raw[k], values);
+            const uint32_t words[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
             uint32_t mask = 0;
 #pragma unroll
             for (uint32_t c = 0; c < kWidth; ++c)
             {
-                const uint32_t element = position + c;
-                if (element >= misalignment && element < part_end && descending_key(values[c]) == key)
-                    mask |= 1u << c;
+                const uint32_t bits = DTYPE == NCNN_MOE_LOGITS_F32 ? words[c]
+                                                                   : ((c & 1u) ? words[c >> 1] >> 16 : words[c >> 1] & 0xffffu);
+                mask |= matches_key(bits) ? 1u << c : 0u;
             }
-            masks[k] = mask;
-        }
-    };
-
-    uint32_t lane_matches = 0;
-    for (uint32_t first = part_begin; first < part_end; first += kTrip)
-    {
-        uint32_t masks[kLoads];
-        match_masks(first, masks);
-#pragma unroll
-        for (int k = 0; k < kLoads; ++k)
+            // positions in front of the row's first element and behind its last are no elements of it
+            const uint32_t below = position < misalignment ? min(misalignment - position, kWidth) : 0u;
+            const uint32_t inside = position < end ? min(end - position, kWidth) : 0u;
+            masks[k] = mask & ((1u << inside) - 1u) & ~((1u << below) - 1u);
             lane_matches += static_cast<uint32_t>(__popc(masks[k]));
-    }
-    uint32_t matches = lane_matches;
-#pragma unroll
-    for (int step = 1; step < kWaveSize; step <<= 1)
-        matches += __shfl_xor(matches, step, kWaveSize);
-    if (lane == 0)
-        scratch.wave_counts[wave] = matches;
-    if (tid == 0)
-        scratch.found = -1;
-    __syncthreads();
-    uint32_t before = 0;
-    for (int w = 0; w < wave; ++w)
-        before += scratch.wave_counts[w];
-    if (ordinal >= before && ordinal < before + matches)
-    {
-        uint32_t remaining = ordinal - before; // matches of this part still to skip
-        bool done = false;
-        for (uint32_t first = part_begin; first < part_end && !done; first += kTrip)
-        {
-            uint32_t masks[kLoads];
-            match_masks(first, masks);
-#pragma unroll
-            for (int k = 0; k < kLoads; ++k)
-            {
-                if (done || __ballot(masks[k] != 0u) == 0)
-                    continue; // most loads hold no match at all: no scan for them
-                const uint32_t count = static_cast<uint32_t>(__popc(masks[k]));
-                uint32_t inclusive = count; // matches in lanes 0..lane of this load
-#pragma unroll
-                for (int step = 1; step < kWaveSize; step <<= 1)
-                {
-                    const uint32_t up = __shfl_up(inclusive, step, kWaveSize);
-                    if (lane >= step)
-                        inclusive += up;
-                }
-                const uint32_t total = static_cast<uint32_t>(read_lane(static_cast<int>(inclusive), kWaveSize - 1));
-                if (remaining < total)
-                {
-                    if (remaining >= inclusive - count && remaining < inclusive)
-                    {
-                        uint32_t mask = masks[k];
-                        for (uint32_t skipped = inclusive - count; skipped < remaining; ++skipped)
-                            mask &= mask - 1u;
-                        const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth +
-                            static_cast<uint32_t>(__builtin_ctz(mask));
-                        scratch.found = static_cast<int32_t>(position - misalignment);
-                    }
-                    done = true;
-                }
-                else
-                    remaining -= total;
-            }
         }
+        const uint32_t wave_matches =
+            static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(lane_matches)), kWaveSize - 1));
+        if (lane == 0)
+            scratch.wave_counts[parity][wave] = wave_matches;
+        __syncthreads();
+        uint32_t before = seen; // matches in front of this wave's slice
+        uint32_t trip_matches = 0;
+#pragma unroll
+        for (int w = 0; w < kReplayWaves; ++w)
+        {
+            const uint32_t count = scratch.wave_counts[parity][w];
+            before += w < wave ? count : 0u;
+            trip_matches += count;
+        }
+        if (ordinal < seen + trip_matches)
+        {
+            if (ordinal >= before && ordinal < before + wave_matches)
+            {
+                uint32_t remaining = ordinal - before; // matches of this slice still to skip
+                bool done = false;
+#pragma unroll
+                for (int k = 0; k < kLoads; ++k)
+                {
+                    if (done || __ballot(masks[k] != 0u) == 0)
+                        continue; // most loads hold no match at all: no scan for them
+                    const uint32_t count = static_cast<uint32_t>(__popc(masks[k]));
+                    const uint32_t inclusive = wave_prefix_sum_u32(count); // matches in lanes 0..lane of this load
+                    const uint32_t total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive), kWaveSize - 1));
+                    if (remaining < total)
+                    {
+                        if (remaining >= inclusive - count && remaining < inclusive)
+                        {
+                            uint32_t mask = masks[k];
+                            for (uint32_t skipped = inclusive - count; skipped < remaining; ++skipped)
+                                mask &= mask - 1u;
+                            const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth +
+                                static_cast<uint32_t>(__builtin_ctz(mask));
+                            scratch.found = static_cast<int32_t>(position - misalignment);
+                        }
+                        done = true;
+                    }
+                    else
+                        remaining -= total;
+                }
+            }
+            break;
+        }
+        seen += trip_matches;
     }
     __syncthreads();
     const int32_t found = scratch.found;

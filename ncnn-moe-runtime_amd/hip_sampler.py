@@ -35,6 +35,7 @@ VERIFY_RESIDUAL_FAILED = 4
 VERIFY_UNSUPPORTED_WINDOW = 5
 PASSES_FULL_ORDER = 1     # sample_device: the later passes are enqueued as well
 PASSES_SIDE_BY_SIDE = 2   # ... and run side by side (rows with wide windows and rows without a window are both present)
+PASSES_NO_WIDE_WINDOWS = 4  # ... but no row has 64 < top_k <= 1024: the select kernel for such windows is left out
 MAX_DRAFT_TOKENS = 16
 
 FLAG_HAS_NAN = 1

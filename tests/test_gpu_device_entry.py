@@ -109,3 +109,32 @@ def test_bf16_strided_rows_on_the_default_stream():
         torch.cuda.synchronize()
     gpu = d_results.cpu().numpy().view(hip_sampler.RESULT_DTYPE).reshape(rows)
     parity_util.assert_results_match(gpu, cpu, "bf16", "sample_device, bf16 strided")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_no_wide_windows_flag(dtype):
+    """NCNN_MOE_PASSES_NO_WIDE_WINDOWS leaves out the select kernel for 64 < top_k <= 1024.  With no such row
+    the results are those of the full set of passes; a row that has such a window after all (the caller's
+    promise broken) is served by the full-order kernels, with the same result."""
+    print("[case] sample_device without the wide select, %s" % dtype, flush=True)
+    from ncnn_moe_runtime_amd import workloads
+    rng = np.random.default_rng(404)
+    rows, vocab = 96, 40013
+    logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    data = workloads.float32_to_bf16_bits(logits) if dtype == "bf16" else logits
+    params = hip_sampler.make_params(rows, 0.9, 0, 0.9, 0.0)
+    params["top_k"] = np.array([(0, 20, 5000, 1, 64, 0)[i % 6] for i in range(rows)], dtype=np.uint32)
+    uniforms = rng.random(rows).astype(np.float32)
+    stream = torch.cuda.Stream(device="cuda:0")
+    flags = hip_sampler.PASSES_FULL_ORDER | hip_sampler.PASSES_NO_WIDE_WINDOWS
+    with hip_sampler.HipSampler(rows, vocab) as sampler:
+        cpu = parity_util.run_oracle(data, params, uniforms)
+        every_pass = _run(sampler, data, params, uniforms, hip_sampler.PASSES_FULL_ORDER, stream)
+        without = _run(sampler, data, params, uniforms, flags, stream)
+        assert every_pass.tobytes() == without.tobytes()
+        parity_util.assert_results_match(without, cpu, dtype, "no wide windows")
+        params["top_k"][3::6] = 700   # wide windows after all
+        cpu = parity_util.run_oracle(data, params, uniforms)
+        broken_promise = _run(sampler, data, params, uniforms, flags | hip_sampler.PASSES_SIDE_BY_SIDE, stream)
+        parity_util.assert_results_match(broken_promise, cpu, dtype, "wide windows without the wide select")
+        assert (broken_promise["flags"][3::6] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
