@@ -369,9 +369,12 @@ int launch_sampler(
     };
     // Rows for the wide select and rows for the full-order kernels are disjoint and each pass keeps few
     // compute units busy (one workgroup per row): with both kinds in the call the two passes run side by
-    // side, the wide select on the handle's second stream.  The full-order kernels then leave the wide
-    // select's rows alone, and are enqueued once more behind the join for the rows that the wide select
-    // could not finish (ties beyond its lists); without such rows that launch exits at once.
+    // side, the wide select on the handle's second stream.  (Starting it only beside the replay, behind a
+    // sort that is spread over every compute unit, was measured and is slower: the two one-workgroup-per-row
+    // kernels then share compute units and the wide select takes 330 us instead of 210.)
+    // The full-order kernels leave the wide select's rows alone, and are enqueued once more behind the
+    // join for the rows that the wide select could not finish (ties beyond its lists); without such rows
+    // that launch exits at once.
     if (passes.side_by_side && passes.wide_select && passes.full_order && s->side_stream != nullptr)
     {
         if (hipEventRecord(s->side_fork, stream) != hipSuccess || hipStreamWaitEvent(s->side_stream, s->side_fork, 0) != hipSuccess)

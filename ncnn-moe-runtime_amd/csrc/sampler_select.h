@@ -447,7 +447,9 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     const int mode = resolve_row_mode(p, a.vocab, a.max_select_top_k, a.force_general, effective_k, status);
     if (mode == kModeInvalid || mode == kModeGeneral)
     {
-        if (segment == 0 && tid == 0)
+        // (a launch for pending rows finds a full-order row marked already, and the full-order kernels may be
+        // serving it at this moment on another stream: it is not touched)
+        if (segment == 0 && tid == 0 && !(a.only_pending && mode == kModeGeneral))
         {
             if (mode == kModeInvalid)
             {
