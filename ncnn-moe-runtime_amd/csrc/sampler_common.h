@@ -241,184 +241,6 @@ __device__ __forceinline__ void finish_row_wave(
     NCNN_MOE_STAMP_ROW(row, 6);
 }
 
-// The same walk for an ordered window of up to 64 * SLOTS candidates held by one wave: candidate i
-// sits in slot i / 64 of lane i % 64.  The sums are the CPU loops themselves, one fp32 addition per
-// candidate in order (a wave-uniform v_readlane feeds each addition), so nothing has to be proved
-// about them; a 1024-candidate window costs about 10,000 cycles per pass.
-template <int SLOTS>
-__device__ __forceinline__ void finish_row_wave_wide(
-    const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
-    const float (&value)[SLOTS], const int32_t (&index)[SLOTS], int n, int lane, uint8_t flags)
-{
-    n = __builtin_amdgcn_readfirstlane(n); // the same in every lane: the loops over it stay scalar
-    const float temperature = p.temperature;
-    const float maximum = read_lane(value[0], 0) / temperature;
-    float term[SLOTS];
-#pragma unroll
-    for (int s = 0; s < SLOTS; ++s)
-        term[s] = (s * kWaveSize + lane) < n ? expf_libm(value[s] / temperature - maximum) : 0.0f;
-
-    float normalizer = 0.0f;
-#pragma unroll
-    for (int s = 0; s < SLOTS; ++s)
-    {
-        // in trips of eight: a lane past the end holds +0.0, which leaves the sum as it is
-        const int slot_count = min(kWaveSize, n - s * kWaveSize);
-        for (int trip = 0; trip * 8 < slot_count; ++trip)
-        {
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-                normalizer += read_lane(term[s], trip * 8 + k);
-        }
-    }
-    if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
-    {
-        if (lane == 0)
-            write_error(a, row, NCNN_MOE_ROW_INVALID_DISTRIBUTION, flags);
-        return;
-    }
-    float probability[SLOTS];
-    uint64_t keep[SLOTS];
-    const float threshold = (term[0] / normalizer) * p.min_p; // lane 0 holds the first candidate
-    const float first_threshold = read_lane(threshold, 0);
-#pragma unroll
-    for (int s = 0; s < SLOTS; ++s)
-    {
-        probability[s] = term[s] / normalizer;
-        bool kept = (s * kWaveSize + lane) < n;
-        if (p.min_p > 0.0f)
-            kept = kept && probability[s] >= first_threshold;
-        keep[s] = __ballot(kept);
-    }
-
-    // Top-P (session.cpp:119-128); the renormaliser of :130-132 adds the same values in the same order.
-    // The walk runs in trips of eight candidates: a filtered candidate adds +0.0, every lane keeps the
-    // running sum at its own position, and one ballot per trip tells whether a kept candidate has
-    // reached top_p (a loop trip of a lone wave costs as much as a dozen of these instructions).
-    float cumulative = 0.0f;
-    float cumulative_here[SLOTS];
-    int last_slot = 0, last_lane = 0;
-    bool reached = false;
-#pragma unroll
-    for (int s = 0; s < SLOTS; ++s)
-    {
-        cumulative_here[s] = 0.0f;
-        const float contribution = ((keep[s] >> lane) & 1ull) ? probability[s] : 0.0f;
-        const int slot_count = reached ? 0 : min(kWaveSize, n - s * kWaveSize);
-        for (int trip = 0; trip * 8 < slot_count; ++trip)
-        {
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-            {
-                cumulative += read_lane(contribution, trip * 8 + k);
-                cumulative_here[s] = lane == trip * 8 + k ? cumulative : cumulative_here[s];
-            }
-            const uint64_t crossing = __ballot(((keep[s] >> lane) & 1ull) != 0ull && cumulative_here[s] >= p.top_p);
-            if (crossing != 0)
-            {
-                reached = true;
-                last_slot = s;
-                last_lane = __builtin_ctzll(crossing);
-                break;
-            }
-        }
-        if (!reached && keep[s] != 0)
-        {
-            last_slot = s; // so far the walk ends at the last kept candidate
-            last_lane = 63 - __builtin_clzll(keep[s]);
-        }
-    }
-    int kept_count = 0;
-    float renormalizer = 0.0f;
-#pragma unroll
-    for (int s = 0; s < SLOTS; ++s)
-    {
-        if (s == last_slot)
-        {
-            keep[s] &= (2ull << last_lane) - 1ull;
-            renormalizer = read_lane(cumulative_here[s], last_lane);
-        }
-        else if (s > last_slot)
-            keep[s] = 0;
-        kept_count += __popcll(keep[s]);
-    }
-    float final_probability[SLOTS];
-#pragma unroll
-    for (int s = 0; s < SLOTS; ++s)
-        final_probability[s] = probability[s] / renormalizer;
-
-    if (a.distribution_count != nullptr)
-    {
-        const size_t first = static_cast<size_t>(row) * a.distribution_cap;
-        uint32_t before = 0;
-#pragma unroll
-        for (int s = 0; s < SLOTS; ++s)
-        {
-            if ((keep[s] >> lane) & 1ull)
-            {
-                const uint32_t position = before + static_cast<uint32_t>(lanes_below(keep[s]));
-                if (position < a.distribution_cap)
-                {
-                    a.distribution_ids[first + position] = index[s];
-                    a.distribution_probabilities[first + position] = final_probability[s];
-                }
-            }
-            before += static_cast<uint32_t>(__popcll(keep[s]));
-        }
-        if (lane == 0)
-            a.distribution_count[row] = static_cast<uint32_t>(kept_count);
-    }
-
-    int selected_slot = last_slot, selected_lane = last_lane; // the draw falls through to the last candidate
-    uint8_t draw_consumed = 0;
-    if (kept_count > 1)
-    {
-        draw_consumed = 1;
-        const float uniform = a.uniforms[row];
-        float running = 0.0f;
-        bool found = false;
-#pragma unroll
-        for (int s = 0; s < SLOTS; ++s)
-        {
-            float running_here = 0.0f;
-            const bool is_kept = ((keep[s] >> lane) & 1ull) != 0ull;
-            const float share = is_kept ? final_probability[s] : 0.0f;
-            const int slot_count = (found || keep[s] == 0) ? 0 : 64 - __builtin_clzll(keep[s]); // up to the last kept candidate
-            for (int trip = 0; trip * 8 < slot_count; ++trip)
-            {
-#pragma unroll
-                for (int k = 0; k < 8; ++k)
-                {
-                    running += read_lane(share, trip * 8 + k);
-                    running_here = lane == trip * 8 + k ? running : running_here;
-                }
-                const uint64_t passed = __ballot(is_kept && uniform < running_here);
-                if (passed != 0)
-                {
-                    selected_slot = s;
-                    selected_lane = __builtin_ctzll(passed);
-                    found = true;
-                    break;
-                }
-            }
-        }
-    }
-    float selected_probability = 1.0f;
-    int32_t token = -1;
-#pragma unroll
-    for (int s = 0; s < SLOTS; ++s)
-    {
-        if (s == selected_slot)
-        {
-            token = read_lane(index[s], selected_lane);
-            if (kept_count > 1)
-                selected_probability = read_lane(final_probability[s], selected_lane);
-        }
-    }
-    if (lane == 0)
-        write_token(a, row, p, token, selected_probability, static_cast<uint32_t>(kept_count), draw_consumed, flags);
-}
-
 template <int DTYPE>
 struct LogitsVector;
 

@@ -383,7 +383,7 @@ __device__ __forceinline__ RoundOutcome finish_round(
 // a sequential loop produces it; term(i) = terms[i], divided by `divisor` and then by `second_divisor` with
 // DIVIDED (a divisor of one leaves a term as it is).  With NON_INCREASING (the terms never grow) it also
 // stops (without `stopped`) once the sum no longer moves, which is then final.  Every thread of the
-// workgroup (kReplayThreads threads) must call it.
+// workgroup (kSumThreads or more) must call it.
 template <bool NON_INCREASING, bool DIVIDED>
 __device__ __noinline__ RunningSum exact_running_sum_of_array(
     const float* terms_array, float divisor, float second_divisor, uint32_t count, int mode, float bound,
@@ -818,7 +818,7 @@ __device__ __forceinline__ void replay_sorted_window(
     {
         const size_t first = static_cast<size_t>(row) * a.distribution_cap;
         const uint32_t limit = kept < a.distribution_cap ? kept : a.distribution_cap;
-        for (uint32_t i = tid; i < limit; i += kReplayThreads)
+        for (uint32_t i = tid; i < limit; i += blockDim.x)
         {
             a.distribution_ids[first + i] = static_cast<int32_t>(sorted_indices[i]);
             a.distribution_probabilities[first + i] = row_term<2>(sorted, RUNS ? run_of_element(sorted, i) : i);

@@ -23,8 +23,9 @@ struct SelectShared
 {
     static constexpr int kListCap = WIDE ? kWideListCap : kNarrowListCap;
     static constexpr int kSortedCap = WIDE ? kSelectTopK : 1;
+    static_assert(kSelectTopK <= 2 * kScanThreads, "the ordered window is copied two entries per thread");
     BoundScratch bound;
-    uint32_t list_keys[kListCap];
+    alignas(16) uint32_t list_keys[kListCap]; // (the wide finish sorts the list as one array of 64-bit pairs over these two)
     int32_t list_indices[kListCap];
     uint32_t list_count;
     uint32_t block_flags;
@@ -34,6 +35,7 @@ struct SelectShared
     int32_t final_indices[kFastTopK];
     uint32_t sorted_keys[kSortedCap];    // descending keys of the ordered window when K > 64
     uint32_t sorted_indices[kSortedCap];
+    ReplayScratch replay;                // of the exact running sums over such a window
 };
 
 // Appends the caller's candidate (if `hit`) to the workgroup's list.  Positions are reserved per
@@ -317,25 +319,62 @@ __device__ __forceinline__ void finish_from_list(
             keys[j] = q < n_ranked ? shared.list_keys[q] : 0u;
             indices[j] = q < n_ranked ? shared.list_indices[q] : 0;
         }
-        // rank of every candidate among all candidates; the best top_k go, in order, to sorted_*
+        // The candidates are put in order by a bitonic sort in LDS: (key, index) pairs as one 64-bit number,
+        // larger = earlier, written over the list itself (its two arrays are one array of pairs), padded
+        // with zeros to a power of two.  (Ranking every candidate by counting those ahead of it, a million
+        // comparisons for a full window, took five times as long.)
         __syncthreads();
+        NCNN_MOE_STAMP_NEXT(row, 12);
+        uint64_t* const pairs = reinterpret_cast<uint64_t*>(shared.list_keys);
+        int padded = kScanThreads * 2;
+        while (padded < n_ranked)
+            padded <<= 1;
 #pragma unroll
         for (int j = 0; j < kPerThread; ++j)
         {
-            if (keys[j] == 0u)
-                continue;
-            int rank = 0;
-#pragma unroll 8
-            for (int q = 0; q < n_ranked; ++q)
+            const int q = j * kScanThreads + tid;
+            if (q < padded)
+                pairs[q] = (q < n_ranked && keys[j] != 0u)
+                    ? (static_cast<uint64_t>(keys[j]) << 32) | (0xffffffffu - static_cast<uint32_t>(indices[j])) : 0ull;
+        }
+        __syncthreads();
+        for (int k = 2; k <= padded; k <<= 1)
+        {
+            for (int j = k >> 1; j > 0; j >>= 1)
             {
-                const uint32_t other_key = shared.list_keys[q];
-                const int32_t other_index = shared.list_indices[q];
-                rank += (other_key > keys[j] || (other_key == keys[j] && other_index < indices[j])) ? 1 : 0;
+                for (int pair = tid; pair < padded / 2; pair += kScanThreads)
+                {
+                    const int low = ((pair & ~(j - 1)) << 1) | (pair & (j - 1));
+                    const int high = low | j;
+                    const uint64_t first = pairs[low];
+                    const uint64_t second = pairs[high];
+                    const bool descending = (low & k) == 0; // the last merge (k == padded) is descending throughout
+                    if (descending ? first < second : first > second)
+                    {
+                        pairs[low] = second;
+                        pairs[high] = first;
+                    }
+                }
+                __syncthreads();
             }
-            if (rank < top_k)
+        }
+        NCNN_MOE_STAMP_NEXT(row, 12);
+        const int ordered = n_ranked < top_k ? n_ranked : top_k;
+        uint64_t chosen[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) // top_k <= kSelectTopK = two per thread
+        {
+            const int rank = j * kScanThreads + tid;
+            chosen[j] = rank < ordered ? pairs[rank] : 0ull;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+        {
+            const int rank = j * kScanThreads + tid;
+            if (rank < ordered && chosen[j] != 0ull)
             {
-                shared.sorted_keys[rank] = descending_key(value_from_ascending_key(keys[j]));
-                shared.sorted_indices[rank] = static_cast<uint32_t>(indices[j]);
+                shared.sorted_keys[rank] = descending_key(value_from_ascending_key(static_cast<uint32_t>(chosen[j] >> 32)));
+                shared.sorted_indices[rank] = 0xffffffffu - static_cast<uint32_t>(chosen[j]);
             }
         }
         __syncthreads();
@@ -348,20 +387,17 @@ __device__ __forceinline__ void finish_from_list(
                 write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
             return;
         }
-        if (wave != 0)
-            return;
-        // wave 0 walks the ordered window: candidate i in slot i / 64 of lane i % 64
-        constexpr int kSlots = kSelectTopK / kWaveSize;
-        float values[kSlots];
-        int32_t tokens[kSlots];
-#pragma unroll
-        for (int s = 0; s < kSlots; ++s)
-        {
-            const int i = s * kWaveSize + lane;
-            values[s] = i < n ? value_from_descending_key(shared.sorted_keys[i]) : 0.0f;
-            tokens[s] = i < n ? static_cast<int32_t>(shared.sorted_indices[i]) : -1;
-        }
-        finish_row_wave_wide<kSlots>(a, row, p, values, tokens, n, lane, result_flags);
+        // the walk over the ordered window with exact running sums, as for a full-order row: the
+        // window's exp terms go where the list was
+        float* const terms = reinterpret_cast<float*>(shared.list_keys);
+        const float maximum = value_from_descending_key(shared.sorted_keys[0]) / p.temperature;
+        for (int i = tid; i < n; i += kScanThreads)
+            terms[i] = expf_libm(value_from_descending_key(shared.sorted_keys[i]) / p.temperature - maximum, exp2_table);
+        __syncthreads();
+        const uint32_t* const sorted_indices = shared.sorted_indices;
+        const auto token_at = [sorted_indices](uint32_t rank) { return static_cast<int32_t>(sorted_indices[rank]); };
+        replay_sorted_window<false>(a, row, p, shared.sorted_keys, nullptr, static_cast<uint32_t>(n), static_cast<uint32_t>(n),
+                                    shared.sorted_indices, result_flags, shared.replay, tid, token_at, terms);
     }
 }
 
@@ -420,6 +456,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
 
     if (a.only_pending && a.row_state[row] != kRowNeedsGeneral)
         return;
+    if (WIDE) { NCNN_MOE_STAMP_RESET(row, 12); NCNN_MOE_STAMP_NEXT(row, 12); }
     // The first chunk's loads go out before anything that waits for the row's options.
     const char* row_pointer = static_cast<const char*>(a.logits) +
         static_cast<size_t>(row) * a.row_stride * Vector::kElementBytes;
@@ -720,7 +757,9 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
             }
             return;
         }
+        if (WIDE) NCNN_MOE_STAMP_NEXT(row, 12);
         finish_from_list(a, row, p, greedy, top_k, shared, result_flags, tid, uniform);
+        if (WIDE) NCNN_MOE_STAMP_NEXT(row, 12);
         return;
     }
 
