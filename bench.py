@@ -440,6 +440,73 @@ def bench_timeline(args):
             np.median(mer[..., 3].max(axis=1)), np.median(seg[..., 1].reshape(len(segment_times), -1).max(axis=1)), np.concatenate(retries).mean()))
 
 
+def bench_full_order_timeline(args):
+    """Where the time of the later passes goes (rows without a Top-K window, or with one wider than 64): the
+    stamped library runs the workload's batch a few times; the stamps that the first 64 rows' workgroups left
+    in the last launch are read back.  Prints a table (text, not the JSON line), microseconds."""
+    import torch
+    from ncnn_moe_runtime_amd import hip_sampler, workloads
+
+    library = os.path.join(PACKAGE_DIR, "libncnn_moe_hip_sampler_timeline.so")
+    if not os.path.exists(library):
+        sys.exit("%s is missing: build it with make -C %s timeline" % (library, PACKAGE_DIR))
+    hip_sampler.LIBRARY_PATH = library
+    lib = hip_sampler.load_library()
+    lib.ncnn_moe_hip_sampler_debug_timeline.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    workload = workloads.make_workload(args.workload)
+    rows, vocab = workload["rows"], workload["vocab"]
+    device = torch.device("cuda:0")
+    dtype_code = hip_sampler.LOGITS_F32 if workload["dtype"] == "f32" else hip_sampler.LOGITS_BF16
+    logits = torch.from_numpy(workload["logits"].view(np.int16) if workload["dtype"] != "f32" else workload["logits"]).to(device)
+    params = torch.from_numpy(workload["params"].view(np.uint8).reshape(rows, -1)).to(device)
+    uniforms = torch.from_numpy(workload["uniforms"]).to(device)
+    stop_ids = None if workload["stop_ids"] is None else torch.from_numpy(workload["stop_ids"]).to(device)
+    results = torch.zeros(rows * 16, dtype=torch.uint8, device=device)
+    stream = torch.cuda.current_stream()
+
+    def read_stamps():
+        stamps = np.zeros(64 * 16 * 16, dtype=np.uint64)
+        assert lib.ncnn_moe_hip_sampler_debug_timeline(stamps.ctypes.data, stamps.size) == 0
+        return stamps.reshape(64, 16, 16).astype(np.int64)
+
+    with hip_sampler.HipSampler(rows, vocab) as sampler:
+        for _ in range(6):
+            before = read_stamps()
+            sampler.sample_device(logits.data_ptr(), dtype_code, rows, vocab, vocab, params.data_ptr(), uniforms.data_ptr(),
+                                  None if stop_ids is None else stop_ids.data_ptr(), results.data_ptr(),
+                                  hip_sampler.PASSES_FULL_ORDER, stream.cuda_stream)
+            torch.cuda.synchronize()
+            after = read_stamps()
+    out = results.cpu().numpy().view(hip_sampler.RESULT_DTYPE)
+    top_k = workload["params"]["top_k"][:64]
+    sampled = workload["params"]["temperature"][:64] != 0
+    full_order = np.nonzero((out["flags"][:64] & hip_sampler.FLAG_GENERAL_PATH) != 0)[0]
+    wide = np.nonzero(sampled & (top_k > 64) & (top_k <= 1024) & ((out["flags"][:64] & hip_sampler.FLAG_GENERAL_PATH) == 0))[0]
+    print("%s, %d rows x %d %s; of the first 64 rows %d took the full-order kernels and %d the wide select" % (
+        args.workload, rows, vocab, workload["dtype"], full_order.size, wide.size))
+
+    def table(title, stamps, names):
+        relative = (stamps - stamps[:, :1]) / 100.0  # the clock ticks at 100 MHz
+        phases = np.diff(stamps, axis=1) / 100.0
+        print("  " + title)
+        for slot, name in enumerate(names[1:]):
+            print("    %-46s at %7.1f (median)   phase: median %6.1f  max %6.1f" % (
+                name, np.median(relative[:, slot + 1]), np.median(phases[:, slot]), phases[:, slot].max()))
+
+    if full_order.size:
+        if workload["dtype"] != "f32":
+            table("bf16_counting_sort_kernel, one workgroup per row, after its entry:", after[full_order, 14, :3],
+                  ["entered", "row counted (one pass, 16-bit counters)", "runs written"])
+        table("general_replay_kernel, one workgroup per row, after its entry:", after[full_order, 15, :8],
+              ["entered", "exp terms of the row ready", "finite prefix found", "normaliser (exact running sum)", "Min-P cut",
+               "Top-P walk (exact running sum)", "draw (exact running sum)", "token index recovered from the logits"])
+        rounds = (after - before)[full_order, 15, 12:14].sum(axis=1)
+        print("    rounds of the exact running sums per row: median %d, max %d" % (np.median(rounds), rounds.max()))
+    if wide.size:
+        table("scan_select_kernel<wide>, one workgroup per row, after its entry:", after[wide, 12, :5],
+              ["entered", "row streamed, candidates listed", "list cut to the window", "window sorted (bitonic, LDS)", "window walked, result written"])
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -457,8 +524,8 @@ def main():
     parser.add_argument("--cpu-rows", type=int, default=64)
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--timeline", action="store_true",
-                        help="print where the time of a split-row launch goes (needs the stamped library: make timeline); "
-                             "a table, not the JSON line")
+                        help="print where the time of a launch goes: the split kernel's phases (cfg2 and the like), or the later "
+                             "passes' (cfg3, cfg4); needs the stamped library (make timeline); a table, not the JSON line")
     parser.add_argument("--copy-calibration", type=int, default=0,
                         help="after the timed steps, copy a 256 MiB buffer this many times (a kernel of known "
                              "traffic for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -469,7 +536,10 @@ def main():
     load_package()
     from ncnn_moe_runtime_amd import hip_sampler, workloads
     if args.timeline:
-        bench_timeline(args)
+        if args.workload in ("cfg3_full_nucleus", "cfg4_service_mix"):
+            bench_full_order_timeline(args)
+        else:
+            bench_timeline(args)
         return
     if args.workload == "router_dispatch":
         bench_router_dispatch(args)

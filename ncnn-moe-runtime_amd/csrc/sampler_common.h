@@ -513,6 +513,90 @@ __device__ __forceinline__ uint32_t workgroup_kth_of_keys(
     return prefix;
 }
 
+// The exact top_k-th largest of the workgroup's N keys per thread (0 = no key; 0 when fewer than top_k keys
+// exist), digit by digit: four rounds of a 256-bin histogram of the keys that share the digits found so
+// far, from which every wave reads off the digit at which the count from the top reaches the wanted rank
+// (lane l takes bins 255 - 4 l down to 252 - 4 l, so a prefix sum over the lanes counts from the largest
+// digit down).  A tenth of the barriers of the bit-by-bit search above.  The keys of a candidate list
+// share their upper digits: a wave first counts the lanes that hold its first lane's digit and adds them
+// with one atomic (twice), and only what is left goes to the histogram lane by lane.
+// All threads of the workgroup must call it.
+template <int N>
+__device__ __forceinline__ uint32_t workgroup_kth_of_keys_by_digits(
+    const uint32_t (&keys)[N], int top_k, int tid, BoundScratch& scratch)
+{
+    const int lane = tid & (kWaveSize - 1);
+    uint32_t prefix = 0;     // the digits found so far, in place
+    uint32_t determined = 0; // the bits they occupy
+    uint32_t wanted = static_cast<uint32_t>(top_k); // rank among the keys that share those digits
+    for (int level = 0; level < 4; ++level)
+    {
+        const int shift = 24 - 8 * level;
+        uint32_t* const bins = scratch.hot_keys + 256 * (level & 1); // alternate levels, alternate bins: one barrier less
+        if (tid < 256)
+            bins[tid] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+        {
+            bool pending = keys[i] != 0u && (keys[i] & determined) == prefix;
+            const uint32_t digit = (keys[i] >> shift) & 255u;
+#pragma unroll
+            for (int round = 0; round < 2; ++round)
+            {
+                const uint64_t holders = __ballot(pending);
+                if (holders == 0ull)
+                    break;
+                const int leader = __builtin_ctzll(holders);
+                const uint32_t leader_digit = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(digit), leader));
+                const uint64_t same = __ballot(pending && digit == leader_digit);
+                if (lane == leader)
+                    atomicAdd(&bins[leader_digit], static_cast<uint32_t>(__popcll(same)));
+                pending = pending && digit != leader_digit;
+            }
+            if (pending)
+                atomicAdd(&bins[digit], 1u);
+        }
+        __syncthreads();
+        const uint32_t top_bin = 255u - 4u * static_cast<uint32_t>(lane);
+        const uint32_t c0 = bins[top_bin], c1 = bins[top_bin - 1u], c2 = bins[top_bin - 2u], c3 = bins[top_bin - 3u];
+        const uint32_t inclusive = wave_prefix_sum_u32(c0 + c1 + c2 + c3);
+        const uint32_t total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive), kWaveSize - 1));
+        if (total < wanted)
+        {
+            __syncthreads();
+            return 0u; // (only at the first level: fewer keys than top_k)
+        }
+        const int crossing = __builtin_ctzll(__ballot(inclusive >= wanted));
+        const uint32_t before = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive - (c0 + c1 + c2 + c3)), crossing));
+        const uint32_t d0 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(c0), crossing));
+        const uint32_t d1 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(c1), crossing));
+        const uint32_t d2 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(c2), crossing));
+        uint32_t step = 0, above = before; // bins of the crossing lane in front of the one that holds the rank
+        if (above + d0 < wanted)
+        {
+            above += d0;
+            step = 1;
+            if (above + d1 < wanted)
+            {
+                above += d1;
+                step = 2;
+                if (above + d2 < wanted)
+                {
+                    above += d2;
+                    step = 3;
+                }
+            }
+        }
+        const uint32_t digit = 255u - 4u * static_cast<uint32_t>(crossing) - step;
+        wanted -= above;
+        prefix |= digit << shift;
+        determined |= 255u << shift;
+    }
+    __syncthreads();
+    return prefix;
+}
+
 // Exact best-K selection over m <= 64 * R candidates in LDS by one wave; keys live in registers.
 // Selected candidates (at most top_k) are written, unordered, to final_values / final_indices.
 template <int R>

@@ -317,9 +317,7 @@ __device__ __forceinline__ RoundOutcome finish_round(
         if (lane == kWaveSize - 1)
             scratch.wave_totals[slot][wave] = inclusive;
     }
-    NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
     lds_barrier();
-    NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
     if (tid == 0)
         scratch.first_event[slot ^ 1u] = 0xffffffffu; // for the next round: its readers are behind the barrier
     if (CHECK_ABSORBED)
@@ -359,9 +357,7 @@ __device__ __forceinline__ RoundOutcome finish_round(
         if (tid == kSumThreads - 1)
             scratch.final_mantissa[slot] = behind;
     }
-    NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
     lds_barrier();
-    NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
     const uint32_t event = scratch.first_event[slot];
     if (event == 0xffffffffu)
     {
@@ -472,8 +468,7 @@ __device__ __noinline__ RunningSum exact_running_sum_of_array(
             const uint32_t slot = round & 1u;
             ++round;
             NCNN_MOE_COUNT(blockIdx.x, 15, 12);
-            NCNN_MOE_STAMP_NEXT(blockIdx.x, 13);
-
+        
             const auto step_at = [&](int j) {
                 const uint32_t i = thread_first + j;
                 const ParityStep step = step_of_term(terms[j], exponent);
@@ -754,6 +749,9 @@ __device__ __forceinline__ void replay_sorted_window(
     const uint32_t* sorted_indices, uint8_t flags, ReplayScratch& scratch, int tid, TokenAt token_at,
     const float* terms0 = nullptr)
 {
+#ifdef NCNN_MOE_TIMELINE
+    const uint32_t stamp_row = a.only_pending ? 0xffffffffu : row; // the full-order rows' stamps (not the wide select's)
+#endif
     SortedRow sorted;
     sorted.keys = keys;
     sorted.run_ends = run_ends;
@@ -779,7 +777,6 @@ __device__ __forceinline__ void replay_sorted_window(
     };
 
     // ---- normaliser (session.cpp:92-103).  A first term that is not finite poisons the sum.
-    NCNN_MOE_STAMP_RESET(blockIdx.x, 13);
     const float first_term = row_term<0>(sorted, 0);
     float normalizer = first_term;
     if (is_finite_f32(first_term))
@@ -791,7 +788,7 @@ __device__ __forceinline__ void replay_sorted_window(
         return;
     }
     sorted.normalizer = normalizer;
-    NCNN_MOE_STAMP(blockIdx.x, 15, 3);
+    NCNN_MOE_STAMP(stamp_row, 15, 3);
 
     // ---- Min-P (session.cpp:107-117): probabilities are non-increasing, so the survivors are a prefix
     uint32_t candidates = n;
@@ -807,12 +804,12 @@ __device__ __forceinline__ void replay_sorted_window(
             candidates = first;
     }
 
-    NCNN_MOE_STAMP(blockIdx.x, 15, 4);
+    NCNN_MOE_STAMP(stamp_row, 15, 4);
     // ---- Top-P (session.cpp:119-128) and the renormaliser (:130-132), which adds the same values
     const RunningSum nucleus = running_sum(std::integral_constant<int, 1>{}, candidates, kStopAtOrAbove, p.top_p);
     const uint32_t kept = nucleus.stopped ? nucleus.stop_index + 1u : candidates;
     sorted.renormalizer = nucleus.sum;
-    NCNN_MOE_STAMP(blockIdx.x, 15, 5);
+    NCNN_MOE_STAMP(stamp_row, 15, 5);
 
     if (a.distribution_count != nullptr && sorted_indices != nullptr)
     {
@@ -838,9 +835,9 @@ __device__ __forceinline__ void replay_sorted_window(
     // ---- inverse-CDF draw over the kept prefix (session.cpp:432-442)
     const RunningSum draw = running_sum(std::integral_constant<int, 2>{}, kept, kStopAbove, a.uniforms[row]);
     const uint32_t selected = draw.stopped ? draw.stop_index : kept - 1u;
-    NCNN_MOE_STAMP(blockIdx.x, 15, 6);
+    NCNN_MOE_STAMP(stamp_row, 15, 6);
     const int32_t token = token_at(selected);
-    NCNN_MOE_STAMP(blockIdx.x, 15, 7);
+    NCNN_MOE_STAMP(stamp_row, 15, 7);
     const float probability = row_term<2>(sorted, item_of(selected)); // (item_of: every lane takes part)
     if (tid == 0)
         write_token(a, row, p, token, probability, kept, 1, flags);

@@ -87,7 +87,7 @@ __device__ __forceinline__ uint32_t tighten_list(SelectShared<WIDE>& shared, uin
     {
         // a long list: the exact K-th best of all its entries (a bound from per-thread maxima would keep
         // most of a list whose threads hold several members of a wide window each)
-        kth = workgroup_kth_of_keys<32>(keys, top_k, tid, shared.bound);
+        kth = workgroup_kth_of_keys_by_digits(keys, top_k, tid, shared.bound);
     }
     else
     {
@@ -603,7 +603,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
 #pragma unroll
                 for (int i = 0; i < kLaneValues; ++i)
                     value_keys[i] = values[i] > -__builtin_inff() ? ascending_key(values[i]) : 0u; // false for NaN as well
-                bound_key = max(bound_key, workgroup_kth_of_keys<32>(value_keys, top_k, tid, shared.bound));
+                bound_key = max(bound_key, workgroup_kth_of_keys_by_digits(value_keys, top_k, tid, shared.bound));
             }
             else if constexpr (WIDE)
             {
@@ -662,7 +662,15 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
                 const int i = rest != 0u ? __builtin_ctz(rest) : 0;
                 const int32_t element = element_of(i);
                 float x = 0.0f;
-                if (rest != 0u)
+                if constexpr (WIDE)
+                {
+                    // under a wide window's bound most lanes hold several candidates: the value is picked out of
+                    // the registers (a chain of selects) rather than waited for
+#pragma unroll
+                    for (int k = 0; k < kLaneValues; ++k)
+                        x = i == k ? values[k] : x;
+                }
+                else if (rest != 0u)
                 {
                     if constexpr (DTYPE == NCNN_MOE_LOGITS_F32)
                         x = reinterpret_cast<const float*>(row_pointer)[element];
