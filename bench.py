@@ -53,7 +53,7 @@ def measured_traffic(workload_name):
     """HBM bytes per launch of the dominant kernel as measured with rocprofv3 --pmc FETCH_SIZE and
     WRITE_SIZE (each scaled by the reading of a 256 MiB copy), recorded beside the profile summaries:
     a stored figure from those counter runs, not something this run measures.  Returns (bytes, file)."""
-    name = "scan_select_%s_traffic.json" % workload_name
+    name = "split_select_%s_traffic.json" % workload_name
     path = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(path):
         return None, None
