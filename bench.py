@@ -523,6 +523,8 @@ def main():
     parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
     parser.add_argument("--cpu-rows", type=int, default=64)
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--host-entry", action="store_true",
+                        help="also time the host-buffer entry (upload_logits + sample(): the logits cross PCIe); detail only")
     parser.add_argument("--timeline", action="store_true",
                         help="print where the time of a launch goes: the split kernel's phases (cfg2 and the like), or the later "
                              "passes' (cfg3, cfg4); needs the stamped library (make timeline); a table, not the JSON line")
@@ -686,6 +688,22 @@ def main():
                                             "robin, wall clock over %d steps; not the reported value" % (detail_steps * 4))
         for handle, _, _ in lanes[1:]:
             handle.close()
+    if args.host_entry:
+        # the boundary's host-buffer entry: logits cross PCIe from pageable host memory, then the synchronous call
+        upload_seconds, sample_seconds = [], []
+        for _ in range(12):
+            begin = time.perf_counter()
+            sampler.upload_logits(workload["logits"])
+            middle = time.perf_counter()
+            sampler.sample(workload["params"], workload["uniforms"], workload["stop_ids"])
+            upload_seconds.append(middle - begin)
+            sample_seconds.append(time.perf_counter() - middle)
+        upload, call = float(np.median(upload_seconds[2:])), float(np.median(sample_seconds[2:]))
+        detail["host_entry"] = {
+            "upload_logits_ms": upload * 1e3, "upload_GB_per_s": rows * vocab * element_bytes / upload / 1e9,
+            "sample_call_ms": call * 1e3, "rows_per_s_including_pcie": rows / (upload + call),
+            "note": "upload_logits from pageable host memory + the synchronous sample() through the Python binding, "
+                    "medians of 10 calls; never the reported value"}
     if args.copy_calibration > 0:
         source = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=device)
         target = torch.empty_like(source)
