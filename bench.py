@@ -656,6 +656,22 @@ def main():
         "cache_resident_note": "same loop on one logits buffer (%.1f MB), held by the Infinity Cache where it fits; "
                                "not the reported value" % (batch_bytes / 1e6),
     }
+    if hip_sampler.select_geometry(dtype_code, rows, vocab)[2] == hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK:
+        # what a launch of this grid costs for streaming the logits alone: the split kernel's loads with
+        # nothing behind them, over the same rotated buffers
+        with torch.cuda.stream(stream):
+            for index in range(20):
+                sampler.stream_only(logits[index % buffers].data_ptr(), dtype_code, rows, vocab, vocab, stream_pointer)
+            stream_start = torch.cuda.Event(enable_timing=True)
+            stream_stop = torch.cuda.Event(enable_timing=True)
+            stream_start.record(stream)
+            for index in range(detail_steps * 4):
+                sampler.stream_only(logits[index % buffers].data_ptr(), dtype_code, rows, vocab, vocab, stream_pointer)
+            stream_stop.record(stream)
+            stream.synchronize()
+        detail["stream_only_ms_per_launch"] = stream_start.elapsed_time(stream_stop) / (detail_steps * 4)
+        detail["stream_only_note"] = ("the split kernel's grid and loads with nothing behind them (%d launches over the rotated "
+                                      "buffers): the cost of streaming the logits alone; not the reported value" % (detail_steps * 4))
     # Several independent batches in flight (one handle and one stream each, steps dealt round robin): what
     # a server that keeps several micro-batches going sees.  A decode loop of ONE batch cannot do this (step
     # n + 1 needs step n's tokens), so these are reported beside the value, never as it.

@@ -18,6 +18,11 @@ extern "C" {
  * on n host values. */
 int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* sampler, int enabled);
 int ncnn_moe_hip_sampler_debug_scatter_segments(ncnn_moe_hip_sampler* sampler, int enabled);
+/* A launch with the split select kernel's grid and loads and nothing behind them (each wave stores one word that
+ * depends on its share of the chunk): what streaming the logits alone costs at that shape.  For the benchmark's
+ * detail; batches below 256 rows with rows of 2 to 16 chunks. */
+int ncnn_moe_hip_sampler_debug_stream_only(
+    ncnn_moe_hip_sampler* sampler, const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride, void* stream);
 /* spread_sort (on by default): the radix sort of a long full-order row runs on several workgroups; off,
  * every row is sorted by one workgroup. */
 int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* sampler, int enabled);

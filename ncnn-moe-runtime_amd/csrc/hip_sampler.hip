@@ -1098,6 +1098,36 @@ int ncnn_moe_hip_sampler_debug_select_geometry(
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 
+int ncnn_moe_hip_sampler_debug_stream_only(
+    ncnn_moe_hip_sampler* s, const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride, void* stream)
+{
+    if (s == nullptr || device_logits == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    const int rc = check_shape(s, dtype, rows, vocab);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return rc;
+    const SelectGeometry g = select_geometry(dtype, vocab, rows, false);
+    if (g.looped || g.segments < 2 || row_stride < vocab)
+        return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "the stream-only probe has the split kernel's geometry: rows of 2 to 16 chunks in a batch below 256 rows");
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
+    SamplerArgs a{};
+    a.logits = device_logits;
+    a.rows = rows;
+    a.vocab = vocab;
+    a.row_stride = row_stride;
+    a.segments = g.segments;
+    a.xcd_grouped = 1;
+    // the sink: one word per wave, in the (unused here) segment records of the looped variant
+    uint32_t* sink = reinterpret_cast<uint32_t*>(s->segment_values);
+    const dim3 grid(((rows + 7u) / 8u) * 8u * g.segments, 1, 1);
+    if (dtype == NCNN_MOE_LOGITS_F32)
+        hipLaunchKernelGGL((split_stream_only_kernel<NCNN_MOE_LOGITS_F32>), grid, dim3(kScanThreads), 0, static_cast<hipStream_t>(stream), a, sink);
+    else
+        hipLaunchKernelGGL((split_stream_only_kernel<NCNN_MOE_LOGITS_BF16>), grid, dim3(kScanThreads), 0, static_cast<hipStream_t>(stream), a, sink);
+    SAMPLER_HIP_CHECK(s, hipGetLastError());
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
 int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* s, const float* in, float* out, size_t n)
 {
     if (s == nullptr || in == nullptr || out == nullptr)

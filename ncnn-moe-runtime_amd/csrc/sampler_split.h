@@ -542,6 +542,44 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     NCNN_MOE_STAMP(row, segment, 7);
 }
 
+// The split kernel's grid and loads with nothing behind them: every workgroup reads its chunk and one lane
+// per wave stores a word that depends on all of it.  What a launch of this shape costs for streaming the
+// logits alone (a probe for the benchmark's detail, not part of the sampling path).
+template <int DTYPE>
+__global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4) void split_stream_only_kernel(SamplerArgs a, uint32_t* sink)
+{
+    using Vector = LogitsVector<DTYPE>;
+    constexpr int kVectors = Vector::kVectorsPerLane;
+    constexpr uint32_t kChunk = static_cast<uint32_t>(kScanThreads) * kVectors * Vector::kWidth;
+    uint32_t row = blockIdx.y;
+    uint32_t segment = blockIdx.x;
+    if (a.xcd_grouped != 0u)
+    {
+        const uint32_t turn = blockIdx.x >> 3;
+        row = (turn / a.segments) * 8u + (blockIdx.x & 7u);
+        segment = turn % a.segments;
+        if (row >= a.rows)
+            return;
+    }
+    const int tid = threadIdx.x;
+    const char* row_pointer = static_cast<const char*>(a.logits) +
+        static_cast<size_t>(row) * a.row_stride * Vector::kElementBytes;
+    const uint32_t misalignment =
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row_pointer) & 15u) / Vector::kElementBytes;
+    const char* aligned_base = row_pointer - static_cast<size_t>(misalignment) * Vector::kElementBytes;
+    const uint32_t valid_end = misalignment + a.vocab;
+    const uint32_t chunk_base = segment * kChunk;
+    uint4 raw[kVectors];
+    load_chunk<DTYPE, kVectors>(raw, aligned_base, chunk_base, misalignment, min(valid_end, chunk_base + kChunk), valid_end, tid);
+    uint32_t folded = 0;
+#pragma unroll
+    for (int v = 0; v < kVectors; ++v)
+        folded ^= raw[v].x ^ raw[v].y ^ raw[v].z ^ raw[v].w;
+    folded = wave_max_u32(folded);
+    if ((tid & (kWaveSize - 1)) == 0)
+        sink[(static_cast<size_t>(row) * a.segments + segment) * kScanWaves + (tid >> 6)] = folded;
+}
+
 } // namespace ncnn_moe_hip
 
 #endif // NCNN_MOE_HIP_SAMPLER_SPLIT_H

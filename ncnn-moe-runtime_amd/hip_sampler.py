@@ -71,6 +71,7 @@ TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_force_general",
     "ncnn_moe_hip_sampler_debug_scatter_segments",
     "ncnn_moe_hip_sampler_debug_spread_sort",
+    "ncnn_moe_hip_sampler_debug_stream_only",
     "ncnn_moe_hip_sampler_debug_expf",
     "ncnn_moe_hip_sampler_debug_exp2_table",
     "ncnn_moe_hip_sampler_debug_select_geometry",
@@ -118,6 +119,7 @@ def load_library():
     lib.ncnn_moe_hip_sampler_debug_force_general.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_scatter_segments.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_spread_sort.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_stream_only.argtypes = [vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp]
     lib.ncnn_moe_hip_sampler_debug_expf.argtypes = [vp, vp, vp, ctypes.c_size_t]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.argtypes = [vp]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.restype = None
@@ -275,6 +277,10 @@ class HipSampler:
     def scatter_segments(self, enabled):
         """Test hook: split rows are launched without the XCD-aware numbering of the workgroups."""
         self._check(self._lib.ncnn_moe_hip_sampler_debug_scatter_segments(self._handle, 1 if enabled else 0))
+
+    def stream_only(self, logits_ptr, dtype, rows, vocab, row_stride, stream=None):
+        """Test hook: a launch with the split kernel's grid and loads and nothing behind them."""
+        self._check(self._lib.ncnn_moe_hip_sampler_debug_stream_only(self._handle, logits_ptr, dtype, rows, vocab, row_stride, stream))
 
     def spread_sort(self, enabled):
         """Test hook: the radix sort of long full-order rows on several workgroups (default) or on one."""
