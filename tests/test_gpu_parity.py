@@ -543,3 +543,48 @@ def test_bf16_counters_that_overflow_sixteen_bits(batch_sampler):
         gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", vocab=vocab,
                              context="bf16 counters at the 16-bit limit, draw %d" % trial)
         assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+
+
+def test_bf16_rows_of_many_runs(batch_sampler):
+    """bf16 full-order rows with more distinct values than the replay keeps in LDS (6144 runs): the runs and
+    their exp terms are then walked from device memory.  Logits spread over sixty binades."""
+    rng = np.random.default_rng(515)
+    rows, vocab = 40, 109999
+    magnitude = np.exp2(rng.uniform(-40.0, 4.0, size=(rows, vocab)))
+    logits = (rng.standard_normal((rows, vocab)) * magnitude).astype(np.float32)
+    bits = workloads.float32_to_bf16_bits(logits)
+    distinct = [np.unique(bits[row]).size for row in range(rows)]
+    assert min(distinct) > 6144, distinct
+    params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+    params["temperature"] = rng.uniform(0.5, 3.0, size=rows).astype(np.float32)
+    params["top_p"] = np.where(np.arange(rows) % 3 == 0, 1.0, rng.uniform(0.6, 0.999, size=rows)).astype(np.float32)
+    params["min_p"][1::5] = 0.001
+    for trial in range(2):
+        uniforms = rng.random(rows, dtype=np.float32)
+        gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", vocab=vocab,
+                             context="bf16 rows of more than 6144 runs, draw %d" % trial)
+        assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+
+
+@pytest.mark.parametrize("tied", [0, 700, 1500, 2600])
+def test_wide_windows_with_ties_at_the_cut(batch_sampler, tied):
+    """Top-K windows of several hundred to a thousand whose K-th value is shared by `tied` further logits: the
+    list that the wide select orders is then K + tied entries long (its bitonic sort runs over 1024, 2048 or
+    4096 slots), and the ties resolve toward the lower token index."""
+    rng = np.random.default_rng(4242 + tied)
+    rows, vocab = 24, 60013
+    logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    params = hip_sampler.make_params(rows, 0.9, 0, 0.97, 0.0)
+    params["top_k"] = np.array([(300, 700, 1000, 1024)[i % 4] for i in range(rows)], dtype=np.uint32)
+    for row in range(rows):
+        if tied:
+            k = int(params["top_k"][row])
+            order = np.argsort(-logits[row], kind="stable")
+            cut_value = logits[row, order[k - 1 - (row % 3)]]      # the window's last value, or one just inside it
+            lower = order[k + 50:]                                  # logits below the window take its value
+            chosen = rng.choice(lower, size=tied, replace=False)
+            logits[row, chosen] = cut_value
+    uniforms = rng.random(rows, dtype=np.float32)
+    gpu, cpu = _check_rows(batch_sampler, logits, params, uniforms, context="wide windows, %d ties at the cut" % tied)
+    served = (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH) == 0
+    assert served.sum() >= (rows if tied <= 1500 else 0)
