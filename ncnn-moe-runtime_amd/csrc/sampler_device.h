@@ -44,16 +44,20 @@ constexpr int kSortPerThread = 8;
 constexpr int kSortTile = kSortThreads * kSortPerThread;
 constexpr int kMaxSortParts = 8;              // workgroups one row's radix sort is spread over
 constexpr int kReplayThreads = 1024;
-// The exact running sums are the work of the workgroup's first kSumWaves waves (two per SIMD), each thread
+// The exact running sums are the work of the workgroup's first eight waves (two per SIMD), each thread
 // composing a few consecutive terms: every wave that takes part pays the scan across its lanes and the
 // composition of the waves' totals again, and a thread's terms are a chain of dependent instructions.
-// Measured on full-order batches (sixteen waves x 4 terms, eight x 8, eight x 4, four x 16, sixteen x 8):
-// rows of single elements do best with eight waves x 8 terms, rows of runs with eight waves x 4.
+// Measured on full-order batches.  Rows of single elements (configuration 4): sixteen waves x 4 terms 964 us,
+// eight x 8 931, eight x 4 967, four x 16 976, sixteen x 8 939.  Rows of runs (configuration 3): eight waves
+// x 2 runs 120.4 us, eight x 3 120.5, eight x 1 122, four x 2 121.7, four x 4 123, eight x 4 123.9,
+// sixteen x 2 126, sixteen x 4 129, four x 8 137: short chunks lose nothing, because a sum that stops
+// early (Top-P, the draw) stops a chunk sooner.
 constexpr int kSumWaves = 8;
 constexpr int kSumThreads = kSumWaves * 64;
 constexpr int kReplayPerThread = 8;
-constexpr int kRunsPerThread = 4;
-constexpr int kRunsChunk = kSumThreads * kRunsPerThread;
+constexpr int kRunsWaves = 8;
+constexpr int kRunsPerThread = 2;
+constexpr int kRunsChunk = kRunsWaves * 64 * kRunsPerThread;
 constexpr int kReplayChunk = kSumThreads * kReplayPerThread;
 
 // Wall-clock stamps for a timeline of the split path, compiled in only with -DNCNN_MOE_TIMELINE (a

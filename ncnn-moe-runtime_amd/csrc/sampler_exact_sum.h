@@ -204,7 +204,7 @@ constexpr int kReplayWaves = kReplayThreads / kWaveSize;
 // with an event) and none at its end.
 struct ReplayScratch
 {
-    ParityStep wave_totals[2][kSumWaves];
+    ParityStep wave_totals[2][kReplayWaves];
     uint32_t first_event[2]; // (index << 1 | kind) of the earliest event of the round, kind 0 = leaves the binade, 1 = stop
     uint32_t final_mantissa[2];
     float event_sum[2];
@@ -298,14 +298,14 @@ struct RoundEvent
     float term;
 };
 
-template <bool CHECK_ABSORBED, class FindEvent>
+template <int WAVES, bool CHECK_ABSORBED, class FindEvent>
 __device__ __forceinline__ RoundOutcome finish_round(
     const ParityStep& thread_total, int exponent, uint32_t mantissa, uint32_t limit, FindEvent find_event,
     ReplayScratch& scratch, uint32_t slot, int tid, float& sum, uint32_t& event_key)
 {
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
-    const bool summing = wave < kSumWaves; // the other waves only follow the round's barriers and its outcome
+    const bool summing = wave < WAVES; // the other waves only follow the round's barriers and its outcome
     ParityStep exclusive{0u, 0u};
     if (summing)
     {
@@ -333,13 +333,13 @@ __device__ __forceinline__ RoundOutcome finish_round(
     if (summing)
     {
         // every wave's total is read at once (independent LDS loads); the composition stays in registers
-        ParityStep totals[kSumWaves];
+        ParityStep totals[WAVES];
 #pragma unroll
-        for (int w = 0; w < kSumWaves; ++w)
+        for (int w = 0; w < WAVES; ++w)
             totals[w] = scratch.wave_totals[slot][w];
         ParityStep before{0u, 0u};
 #pragma unroll
-        for (int w = 0; w < kSumWaves - 1; ++w)
+        for (int w = 0; w < WAVES - 1; ++w)
         {
             const ParityStep with = compose_steps(before, totals[w]);
             before = ParityStep{w < wave ? with.even : before.even, w < wave ? with.odd : before.odd};
@@ -354,7 +354,7 @@ __device__ __forceinline__ RoundOutcome finish_round(
             reported = find_event(current, found);
         if (reported)
             atomicMin(&scratch.first_event[slot], found.key);
-        if (tid == kSumThreads - 1)
+        if (tid == WAVES * kWaveSize - 1)
             scratch.final_mantissa[slot] = behind;
     }
     lds_barrier();
@@ -518,7 +518,7 @@ __device__ __noinline__ RunningSum exact_running_sum_of_array(
             };
             uint32_t event = 0;
             const RoundOutcome outcome =
-                finish_round<NON_INCREASING>(thread_total, exponent, mantissa, limit, find_event, scratch, slot, tid, sum, event);
+                finish_round<kSumWaves, NON_INCREASING>(thread_total, exponent, mantissa, limit, find_event, scratch, slot, tid, sum, event);
             if (outcome == kRoundAbsorbed)
                 return RunningSum{sum, 0u, false};
             if (outcome == kRoundPlain)
@@ -599,7 +599,7 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
         float terms[kRunsPerThread];
         uint32_t firsts[kRunsPerThread]; // first and one-past-last element of each run, clipped to count
         uint32_t lasts[kRunsPerThread];
-        const bool summing = tid < kSumThreads;
+        const bool summing = tid < kRunsWaves * kWaveSize;
 #pragma unroll
         for (int j = 0; j < kRunsPerThread; ++j)
         {
@@ -709,7 +709,7 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
             };
             uint32_t event = 0;
             const RoundOutcome outcome =
-                finish_round<FIRST>(thread_total, exponent, mantissa, limit, find_event, scratch, slot, tid, sum, event);
+                finish_round<kRunsWaves, FIRST>(thread_total, exponent, mantissa, limit, find_event, scratch, slot, tid, sum, event);
             if (outcome == kRoundAbsorbed)
                 return RunningSum{sum, 0u, false};
             if (outcome == kRoundPlain)
