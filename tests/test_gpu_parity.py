@@ -588,3 +588,52 @@ def test_wide_windows_with_ties_at_the_cut(batch_sampler, tied):
     gpu, cpu = _check_rows(batch_sampler, logits, params, uniforms, context="wide windows, %d ties at the cut" % tied)
     served = (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH) == 0
     assert served.sum() >= (rows if tied <= 1500 else 0)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_sampled_zeros_of_both_signs(batch_sampler, dtype):
+    """+0.0 and -0.0 tie (the reference compares logits with ==), so a row whose best logits are zeros of both
+    signs orders them by index alone; the full-order path recovers the sampled token's index by comparing
+    bit patterns and must treat the two patterns as one key.  Every draw lands on a zero."""
+    rng = np.random.default_rng(31337)
+    rows, vocab = 32, 70001
+    logits = (-20.0 - 5.0 * rng.random((rows, vocab))).astype(np.float32)
+    zeros_per_row = 40
+    for row in range(rows):
+        where = rng.choice(vocab, size=zeros_per_row, replace=False)
+        logits[row, where] = np.where(rng.random(zeros_per_row) < 0.5, np.float32(0.0), np.float32(-0.0))
+    data = workloads.float32_to_bf16_bits(logits) if dtype == "bf16" else logits
+    if dtype == "bf16":
+        assert (data == 0x8000).any() and (data == 0x0000).any()
+    params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)      # no window: full-order path
+    params["top_k"][1::2] = 5000
+    tokens = set()
+    for trial in range(4):
+        uniforms = rng.random(rows, dtype=np.float32)
+        gpu, cpu = _check_rows(batch_sampler, data, params, uniforms, dtype=dtype, vocab=vocab,
+                               context="zeros of both signs, %s, draw %d" % (dtype, trial))
+        assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+        picked = logits[np.arange(rows), gpu["token_id"]]
+        assert (picked == 0.0).all()
+        tokens.update(int(t) for t in gpu["token_id"])
+    assert len(tokens) > rows  # the draws spread over the zeros
+
+
+def test_distribution_of_a_wide_window(batch_sampler):
+    """The filtered distribution of a row with a window of several hundred tokens, exported by the wide select
+    (all of its threads write the list): ids and probabilities bit for bit those of the oracle."""
+    rng = np.random.default_rng(808)
+    vocab = 90007
+    logits = (rng.standard_normal((4, vocab)) * 2.5).astype(np.float32)
+    batch_sampler.upload_logits(logits, vocab=vocab)
+    for row, options in enumerate([dict(temperature=0.9, top_k=700, top_p=1.0, min_p=0.0),
+                                   dict(temperature=1.3, top_k=1024, top_p=0.99, min_p=0.0),
+                                   dict(temperature=0.7, top_k=300, top_p=0.95, min_p=0.001),
+                                   dict(temperature=1.0, top_k=65, top_p=1.0, min_p=0.0)]):
+        _announce("distribution of a wide window, row %d" % row)
+        status, ids, probabilities, count = batch_sampler.distribution(row, **options)
+        oracle_status, oracle_ids, oracle_probabilities = oracle_lib.oracle_distribution(logits[row], **options)
+        assert status == oracle_status
+        assert count == len(oracle_ids) and count > 64
+        assert np.array_equal(ids[:count], oracle_ids)
+        assert np.array_equal(probabilities[:count].view(np.uint32), np.asarray(oracle_probabilities, dtype=np.float32).view(np.uint32))
