@@ -325,9 +325,9 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(Sampl
     const uint32_t n = a.vocab;
     const int pass = static_cast<int>(a.sort_pass);
     const int shift = 8 * (pass + kFirstDigit);
-    __shared__ uint32_t counts[256];
-    if (tid < 256)
-        counts[tid] = 0;
+    __shared__ uint32_t counts[8][257]; // (257: the copies of a digit's counter lie in eight different banks)
+    for (int i = tid; i < 8 * 257; i += kSortThreads)
+        (&counts[0][0])[i] = 0;
     __syncthreads();
     const uint32_t first_tile = part * a.sort_tiles_per_part * kSortTile;
     const uint32_t end = min(n, first_tile + a.sort_tiles_per_part * kSortTile);
@@ -339,13 +339,21 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(Sampl
 #pragma unroll
         for (int e = 0; e < kSortPerThread; ++e)
         {
+            // (eight copies of the counters, a lane using copy lane % 8: the uppermost digit of a row's keys
+            // takes few values, and 64 atomics on one address take as many turns)
             if (tile + static_cast<uint32_t>(e * kSortThreads + tid) < n)
-                atomicAdd(&counts[(keys[e] >> shift) & 255u], 1u);
+                atomicAdd(&counts[tid & 7][(keys[e] >> shift) & 255u], 1u);
         }
     }
     __syncthreads();
     if (tid < 256)
-        a.sort_part_counts[(static_cast<size_t>(row) * a.sort_parts + part) * 256 + tid] = counts[tid];
+    {
+        uint32_t total = 0;
+#pragma unroll
+        for (int copy = 0; copy < 8; ++copy)
+            total += counts[copy][tid];
+        a.sort_part_counts[(static_cast<size_t>(row) * a.sort_parts + part) * 256 + tid] = total;
+    }
 }
 
 template <int DTYPE, bool PAIRS>
