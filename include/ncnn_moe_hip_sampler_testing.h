@@ -23,6 +23,10 @@ int ncnn_moe_hip_sampler_debug_scatter_segments(ncnn_moe_hip_sampler* sampler, i
  * detail; batches below 256 rows with rows of 2 to 16 chunks. */
 int ncnn_moe_hip_sampler_debug_stream_only(
     ncnn_moe_hip_sampler* sampler, const void* device_logits, int dtype, uint32_t rows, uint32_t vocab, uint64_t row_stride, void* stream);
+/* chunk_steps (on by default): the composed steps of the whole chunks of a sorted fp32 row's terms are worked out by
+ * a kernel of their own before the replay, which then adds such a chunk in one step; off, the replay runs every chunk's
+ * round itself.  Same results either way. */
+int ncnn_moe_hip_sampler_debug_chunk_steps(ncnn_moe_hip_sampler* sampler, int enabled);
 /* spread_sort (on by default): the radix sort of a long full-order row runs on several workgroups; off,
  * every row is sorted by one workgroup. */
 int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* sampler, int enabled);

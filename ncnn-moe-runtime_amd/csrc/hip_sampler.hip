@@ -66,6 +66,11 @@ struct ncnn_moe_hip_sampler
     uint32_t* sort_indices[2] = {nullptr, nullptr};
     uint64_t sort_stride = 0;
     uint32_t* sort_part_counts = nullptr; // [rows][kMaxSortParts][256]
+    double* term_sums = nullptr;          // [rows][term_sum_parts]: fp64 sums of the terms kernel's blocks
+    uint4* chunk_steps = nullptr;         // [rows][chunk_capacity]: composed step of every whole chunk of a sorted row's terms
+    uint32_t term_sum_parts = 0;
+    uint32_t chunk_capacity = 0;
+    int chunk_steps_enabled = 1;
 
     int32_t* distribution_ids = nullptr;
     float* distribution_probabilities = nullptr;
@@ -287,6 +292,10 @@ int launch_sampler(
     a.sort_indices[1] = s->sort_indices[1];
     a.sort_stride = s->sort_stride;
     a.sort_part_counts = s->sort_part_counts;
+    a.term_sums = s->term_sums;
+    a.chunk_steps = s->chunk_steps;
+    a.term_sum_parts = s->term_sum_parts;
+    a.chunk_capacity = s->chunk_capacity;
     if (want_distribution)
     {
         a.distribution_ids = export_to.ids;
@@ -359,6 +368,12 @@ int launch_sampler(
             const uint32_t parts = (vocab + kTermsThreads * kTermsPerThread - 1) / (kTermsThreads * kTermsPerThread);
             hipLaunchKernelGGL(full_order_terms_kernel, dim3(parts, rows), dim3(kTermsThreads), 0, stream, a);
             a.terms_precomputed = 1;
+            const uint32_t whole_chunks = vocab / kReplayChunk;
+            if (whole_chunks > 0 && s->chunk_steps_enabled != 0)
+            {
+                hipLaunchKernelGGL(full_order_chunk_steps_kernel, dim3(whole_chunks, rows), dim3(kChunkStepThreads), 0, stream, a);
+                a.chunk_steps_ready = 1;
+            }
         }
         if (runs)
             hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
@@ -560,6 +575,10 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
         CREATE_CHECK(hipMalloc(&s->sort_indices[i], rows * s->sort_stride * sizeof(uint32_t)));
     }
     CREATE_CHECK(hipMalloc(&s->sort_part_counts, rows * kMaxSortParts * 256 * sizeof(uint32_t)));
+    s->term_sum_parts = (max_vocab + kTermsThreads * kTermsPerThread - 1) / (kTermsThreads * kTermsPerThread);
+    s->chunk_capacity = max_vocab / kReplayChunk + 1;
+    CREATE_CHECK(hipMalloc(&s->term_sums, rows * s->term_sum_parts * sizeof(double)));
+    CREATE_CHECK(hipMalloc(&s->chunk_steps, rows * s->chunk_capacity * sizeof(uint4)));
     CREATE_CHECK(hipMalloc(&s->distribution_ids, static_cast<size_t>(max_vocab) * sizeof(int32_t)));
     CREATE_CHECK(hipMalloc(&s->distribution_probabilities, static_cast<size_t>(max_vocab) * sizeof(float)));
     CREATE_CHECK(hipMalloc(&s->distribution_count, sizeof(uint32_t)));
@@ -611,7 +630,7 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
     void* buffers[] = {
         s->logits, s->params, s->uniforms, s->results, s->segment_values, s->segment_indices,
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->split_records, s->row_epoch, s->sort_keys[0], s->sort_keys[1],
-        s->sort_indices[0], s->sort_indices[1], s->sort_part_counts, s->distribution_ids, s->distribution_probabilities,
+        s->sort_indices[0], s->sort_indices[1], s->sort_part_counts, s->term_sums, s->chunk_steps, s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
         s->verify_probabilities, s->verify_counts, s->verify_long_ids, s->verify_long_probabilities, s->verify_dense};
     for (void* buffer : buffers)
@@ -1074,6 +1093,14 @@ int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* s, int enabled)
     if (s == nullptr)
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     s->spread_sort = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_debug_chunk_steps(ncnn_moe_hip_sampler* s, int enabled)
+{
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    s->chunk_steps_enabled = enabled ? 1 : 0;
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

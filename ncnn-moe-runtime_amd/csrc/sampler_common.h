@@ -52,6 +52,14 @@ struct SamplerArgs
     uint32_t sort_pass;
     // full_order_terms_kernel has run: sort_keys[0] holds exp(logit/T - maximum) of the sorted rows' elements
     uint32_t terms_precomputed;
+    // ... and what every whole chunk of kReplayChunk of them does to a running sum of a guessed exponent:
+    // term_sums [rows][term_sum_parts] (fp64 sums of the terms kernel's blocks), chunk_steps [rows][chunk_capacity]
+    // (exponent, step on an even mantissa, step on an odd one, valid); chunk_steps_ready: the kernels that fill them have run
+    double* term_sums;
+    uint4* chunk_steps;
+    uint32_t term_sum_parts;
+    uint32_t chunk_capacity;
+    uint32_t chunk_steps_ready;
 
     // optional filtered-distribution output: row r writes at most distribution_cap (id, probability)
     // entries from r * distribution_cap on, and its full kept length to distribution_count[r]

@@ -228,6 +228,7 @@ struct SortedRow
     const uint32_t* run_ends; // runs only: position behind the last element of each run (null otherwise)
     uint32_t run_count;
     const float* terms0;      // exp(logit/T - maximum) of every item (element or run), computed beforehand
+    const uint4* chunk_steps; // elements only, may be null: (exponent, even step, odd step, valid) of every whole chunk of terms0
     float temperature;
     float maximum;
     float normalizer;
@@ -383,7 +384,7 @@ __device__ __forceinline__ RoundOutcome finish_round(
 template <bool NON_INCREASING, bool DIVIDED>
 __device__ __noinline__ RunningSum exact_running_sum_of_array(
     const float* terms_array, float divisor, float second_divisor, uint32_t count, int mode, float bound,
-    ReplayScratch& scratch, int tid)
+    ReplayScratch& scratch, int tid, const uint4* chunk_steps = nullptr)
 {
     const auto scaled = [divisor, second_divisor](float t) { return DIVIDED ? (t / divisor) / second_divisor : t; };
     const auto term_at = [&](uint32_t i) { return scaled(terms_array[i]); };
@@ -447,9 +448,36 @@ __device__ __noinline__ RunningSum exact_running_sum_of_array(
         }
     };
     fetch(0);
+    bool fetched = true; // `upcoming` holds the terms of the chunk at `base`
     for (uint32_t base = 0; base < count; base += kReplayChunk)
     {
         const uint32_t chunk_end = min(count, base + static_cast<uint32_t>(kReplayChunk));
+        if (NON_INCREASING && !DIVIDED && chunk_steps != nullptr && mode == kStopNever &&
+            chunk_end == base + static_cast<uint32_t>(kReplayChunk) && head == static_cast<uint32_t>(kSequentialHead))
+        {
+            // A whole chunk whose composed step was worked out beforehand for the exponent that the sum has now:
+            // if that step leaves the mantissa inside the binade, nothing inside the chunk left it either (the
+            // mantissa never decreases), and the chunk is this one addition.
+            const uint4 composed = chunk_steps[base / kReplayChunk];
+            int exponent;
+            uint32_t mantissa;
+            decode_sum(sum, exponent, mantissa);
+            if (composed.w != 0u && composed.x == static_cast<uint32_t>(exponent))
+            {
+                const uint32_t behind = apply_step(mantissa, ParityStep{composed.y, composed.z});
+                if (behind < kBinadeFull)
+                {
+                    if (composed.y == 0u && composed.z == 0u)
+                        return RunningSum{sum, 0u, false}; // no term of the chunk moves the sum: none behind it can
+                    sum = encode_sum(exponent, behind);
+                    fetched = false;
+                    continue;
+                }
+            }
+        }
+        if (!fetched)
+            fetch(base);
+        fetched = true;
         const uint32_t thread_first = base + static_cast<uint32_t>(tid) * kReplayPerThread;
         float terms[kReplayPerThread];
 #pragma unroll
@@ -541,7 +569,8 @@ __device__ __forceinline__ RunningSum exact_running_sum(
     const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
 {
     return exact_running_sum_of_array<PHASE == 0, PHASE != 0>(
-        row.terms0, row.normalizer, PHASE == 2 ? row.renormalizer : 1.0f, count, mode, bound, scratch, tid);
+        row.terms0, row.normalizer, PHASE == 2 ? row.renormalizer : 1.0f, count, mode, bound, scratch, tid,
+        PHASE == 0 ? row.chunk_steps : nullptr);
 }
 
 // The same running sum over a row stored as runs: `count` elements are added, run after run.  A run of
@@ -747,7 +776,7 @@ __device__ __forceinline__ void replay_sorted_window(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
     const uint32_t* keys, const uint32_t* run_ends, uint32_t run_count, uint32_t n,
     const uint32_t* sorted_indices, uint8_t flags, ReplayScratch& scratch, int tid, TokenAt token_at,
-    const float* terms0 = nullptr)
+    const float* terms0 = nullptr, const uint4* chunk_steps = nullptr)
 {
 #ifdef NCNN_MOE_TIMELINE
     const uint32_t stamp_row = a.only_pending ? 0xffffffffu : row; // the full-order rows' stamps (not the wide select's)
@@ -757,6 +786,7 @@ __device__ __forceinline__ void replay_sorted_window(
     sorted.run_ends = run_ends;
     sorted.run_count = run_count;
     sorted.terms0 = terms0;
+    sorted.chunk_steps = RUNS ? nullptr : chunk_steps;
     sorted.temperature = p.temperature;
     sorted.maximum = value_from_descending_key(keys[0]) / p.temperature;
     sorted.normalizer = 1.0f;

@@ -1056,7 +1056,13 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     if (p.top_k > 0 && p.top_k < vocab && n > p.top_k)
         n = p.top_k;
     NCNN_MOE_STAMP(blockIdx.x, 15, 2);
-    replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0);
+    const uint4* chunk_steps = nullptr;
+    if constexpr (!RUNS)
+    {
+        if (a.chunk_steps_ready != 0)
+            chunk_steps = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity;
+    }
+    replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0, chunk_steps);
 }
 
 // exp(logit/T - maximum) of every element of the sorted full-order rows, written over the sort's other key
@@ -1083,12 +1089,127 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
         const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
         loaded[j] = i < a.vocab ? keys[i] : 0u;
     }
+    double sum = 0.0;
 #pragma unroll
     for (int j = 0; j < kTermsPerThread; ++j)
     {
         const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
         if (i < a.vocab)
-            terms[i] = expf_libm(value_from_descending_key(loaded[j]) / temperature - maximum);
+        {
+            const float term = expf_libm(value_from_descending_key(loaded[j]) / temperature - maximum);
+            terms[i] = term;
+            sum += static_cast<double>(term);
+        }
+    }
+    // the block's sum (fp64: an estimate of where the sequential fp32 sum stands, for full_order_chunk_steps_kernel)
+    __shared__ double wave_sums[kTermsThreads / kWaveSize];
+#pragma unroll
+    for (int step = kWaveSize / 2; step > 0; step >>= 1)
+        sum += __shfl_down(sum, step, kWaveSize);
+    if ((threadIdx.x & (kWaveSize - 1)) == 0)
+        wave_sums[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        double total = 0.0;
+#pragma unroll
+        for (int w = 0; w < kTermsThreads / kWaveSize; ++w)
+            total += wave_sums[w];
+        a.term_sums[static_cast<size_t>(row) * a.term_sum_parts + blockIdx.x] = total;
+    }
+}
+
+// What every whole chunk of kReplayChunk terms does to the normaliser's running sum, computed by the whole GPU
+// before the replay walks the row one workgroup per row: the composition of the chunk's steps (see
+// sampler_exact_sum.h) for the exponent that the sum most likely has when it reaches the chunk, guessed from
+// the fp64 sum of the terms in front of it.  The replay checks the guess against its exact sum: where the
+// exponent is the one assumed here and the composed step leaves the mantissa inside its binade (the mantissa
+// never decreases, so nothing inside the chunk left it either), the chunk costs it one addition instead of a
+// round; everywhere else it runs the round as before.  A wrong guess costs time, never exactness.
+// grid (chunks, rows); thread t composes the chunk's terms 16 t .. 16 t + 15.
+constexpr int kChunkStepThreads = 256;
+constexpr int kChunkStepPerThread = kReplayChunk / kChunkStepThreads;
+
+__global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kernel(SamplerArgs a)
+{
+    static_assert(kChunkStepPerThread * kChunkStepThreads == kReplayChunk && kChunkStepPerThread % 4 == 0, "float4 loads over a whole chunk");
+    static_assert(kReplayChunk % (kTermsThreads * kTermsPerThread) == 0, "a chunk is a whole number of the terms kernel's blocks");
+    const uint32_t row = blockIdx.y;
+    const uint32_t chunk = blockIdx.x;
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+        return;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    constexpr int kWaves = kChunkStepThreads / kWaveSize;
+    __shared__ double wave_sums[kWaves];
+    __shared__ ParityStep wave_totals[kWaves];
+    const float* terms = reinterpret_cast<const float*>(a.sort_keys[0] + row * a.sort_stride);
+    uint4* const out = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity + chunk;
+    const uint32_t base = chunk * kReplayChunk;
+    if (base + kReplayChunk > a.vocab)
+    {
+        if (tid == 0)
+            *out = uint4{0u, 0u, 0u, 0u}; // not a whole chunk: the replay never asks
+        return;
+    }
+    // the sum in front of the chunk: the blocks of the terms kernel before it, or (first chunk) the 64 terms
+    // that every running sum adds one by one
+    double before = 0.0;
+    if (chunk == 0)
+        before = tid < kSequentialHead ? static_cast<double>(terms[tid]) : 0.0;
+    else
+    {
+        const uint32_t blocks = chunk * (kReplayChunk / (kTermsThreads * kTermsPerThread));
+        for (uint32_t block = tid; block < blocks; block += kChunkStepThreads)
+            before += a.term_sums[static_cast<size_t>(row) * a.term_sum_parts + block];
+    }
+#pragma unroll
+    for (int step = kWaveSize / 2; step > 0; step >>= 1)
+        before += __shfl_down(before, step, kWaveSize);
+    if (lane == 0)
+        wave_sums[wave] = before;
+    __syncthreads();
+    double estimate = 0.0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w)
+        estimate += wave_sums[w];
+    const float estimate_f32 = static_cast<float>(estimate);
+    if (!(estimate_f32 > 0.0f) || !is_finite_f32(estimate_f32))
+    {
+        if (tid == 0)
+            *out = uint4{0u, 0u, 0u, 0u};
+        return;
+    }
+    int exponent;
+    uint32_t unused_mantissa;
+    decode_sum(estimate_f32, exponent, unused_mantissa);
+    const uint32_t first = base + static_cast<uint32_t>(tid) * kChunkStepPerThread;
+    ParityStep total{0u, 0u};
+#pragma unroll
+    for (int j = 0; j < kChunkStepPerThread; j += 4)
+    {
+        const float4 four = *reinterpret_cast<const float4*>(terms + first + j);
+        const float values[4] = {four.x, four.y, four.z, four.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+        {
+            const ParityStep step = step_of_term(values[c], exponent);
+            const bool counted = first + j + c >= static_cast<uint32_t>(kSequentialHead); // the head is added before the chunks
+            total = compose_steps(total, ParityStep{counted ? step.even : 0u, counted ? step.odd : 0u});
+        }
+    }
+    const ParityStep inclusive = wave_scan_steps(total);
+    if (lane == kWaveSize - 1)
+        wave_totals[wave] = inclusive;
+    __syncthreads();
+    if (tid == 0)
+    {
+        ParityStep all{0u, 0u};
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w)
+            all = compose_steps(all, wave_totals[w]);
+        *out = uint4{static_cast<uint32_t>(exponent), all.even, all.odd, 1u};
     }
 }
 

@@ -71,6 +71,7 @@ TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_force_general",
     "ncnn_moe_hip_sampler_debug_scatter_segments",
     "ncnn_moe_hip_sampler_debug_spread_sort",
+    "ncnn_moe_hip_sampler_debug_chunk_steps",
     "ncnn_moe_hip_sampler_debug_stream_only",
     "ncnn_moe_hip_sampler_debug_expf",
     "ncnn_moe_hip_sampler_debug_exp2_table",
@@ -119,6 +120,7 @@ def load_library():
     lib.ncnn_moe_hip_sampler_debug_force_general.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_scatter_segments.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_spread_sort.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_chunk_steps.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_stream_only.argtypes = [vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp]
     lib.ncnn_moe_hip_sampler_debug_expf.argtypes = [vp, vp, vp, ctypes.c_size_t]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.argtypes = [vp]
@@ -281,6 +283,10 @@ class HipSampler:
     def stream_only(self, logits_ptr, dtype, rows, vocab, row_stride, stream=None):
         """Test hook: a launch with the split kernel's grid and loads and nothing behind them."""
         self._check(self._lib.ncnn_moe_hip_sampler_debug_stream_only(self._handle, logits_ptr, dtype, rows, vocab, row_stride, stream))
+
+    def chunk_steps(self, enabled):
+        """Test hook: whole chunks of a sorted fp32 row added in one precomputed step (default) or round by round."""
+        self._check(self._lib.ncnn_moe_hip_sampler_debug_chunk_steps(self._handle, 1 if enabled else 0))
 
     def spread_sort(self, enabled):
         """Test hook: the radix sort of long full-order rows on several workgroups (default) or on one."""

@@ -507,6 +507,13 @@ def test_full_order_rows_sorted_by_several_workgroups(batch_sampler, dtype, voca
     finally:
         batch_sampler.spread_sort(True)
     assert spread.tobytes() == single.tobytes()
+    # ... and with every chunk of the normaliser summed round by round instead of in its precomputed step
+    batch_sampler.chunk_steps(False)
+    try:
+        by_rounds = batch_sampler.sample(params, uniforms, None)
+    finally:
+        batch_sampler.chunk_steps(True)
+    assert spread.tobytes() == by_rounds.tobytes()
     for row in (0, 20):
         options = dict(temperature=float(params["temperature"][row]), top_k=0, top_p=0.9, min_p=0.0)
         status, ids, probabilities, count = batch_sampler.distribution(row, **options)
