@@ -1077,6 +1077,9 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
     const uint32_t row = blockIdx.y;
     if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
         return;
+    __shared__ uint64_t exp2_table[32]; // a copy in LDS: the lookups of a wave are 64 different addresses
+    if (threadIdx.x < 32)
+        exp2_table[threadIdx.x] = kExp2Table[threadIdx.x];
     const float temperature = a.params[row].temperature;
     const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
     float* terms = reinterpret_cast<float*>(a.sort_keys[0] + row * a.sort_stride);
@@ -1089,6 +1092,7 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
         const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
         loaded[j] = i < a.vocab ? keys[i] : 0u;
     }
+    __syncthreads();
     double sum = 0.0;
 #pragma unroll
     for (int j = 0; j < kTermsPerThread; ++j)
@@ -1096,7 +1100,7 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
         const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
         if (i < a.vocab)
         {
-            const float term = expf_libm(value_from_descending_key(loaded[j]) / temperature - maximum);
+            const float term = expf_libm(value_from_descending_key(loaded[j]) / temperature - maximum, exp2_table);
             terms[i] = term;
             sum += static_cast<double>(term);
         }
@@ -1153,6 +1157,12 @@ __global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kern
             *out = uint4{0u, 0u, 0u, 0u}; // not a whole chunk: the replay never asks
         return;
     }
+    // the chunk's terms are asked for first: the estimate below is a chain of loads, a reduction and a barrier
+    const uint32_t first = base + static_cast<uint32_t>(tid) * kChunkStepPerThread;
+    float4 loaded[kChunkStepPerThread / 4];
+#pragma unroll
+    for (int j = 0; j < kChunkStepPerThread / 4; ++j)
+        loaded[j] = *reinterpret_cast<const float4*>(terms + first + 4 * j);
     // the sum in front of the chunk: the blocks of the terms kernel before it, or (first chunk) the 64 terms
     // that every running sum adds one by one
     double before = 0.0;
@@ -1184,12 +1194,11 @@ __global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kern
     int exponent;
     uint32_t unused_mantissa;
     decode_sum(estimate_f32, exponent, unused_mantissa);
-    const uint32_t first = base + static_cast<uint32_t>(tid) * kChunkStepPerThread;
     ParityStep total{0u, 0u};
 #pragma unroll
     for (int j = 0; j < kChunkStepPerThread; j += 4)
     {
-        const float4 four = *reinterpret_cast<const float4*>(terms + first + j);
+        const float4 four = loaded[j / 4];
         const float values[4] = {four.x, four.y, four.z, four.w};
 #pragma unroll
         for (int c = 0; c < 4; ++c)
