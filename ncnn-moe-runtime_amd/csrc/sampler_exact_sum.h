@@ -381,8 +381,10 @@ __device__ __forceinline__ RoundOutcome finish_round(
 // DIVIDED (a divisor of one leaves a term as it is).  With NON_INCREASING (the terms never grow) it also
 // stops (without `stopped`) once the sum no longer moves, which is then final.  Every thread of the
 // workgroup (kSumThreads or more) must call it.
-template <bool NON_INCREASING, bool DIVIDED>
-__device__ __noinline__ RunningSum exact_running_sum_of_array(
+// CHECK_FIRST: a first term that is not finite is returned as the sum at once (it poisons the sum; the caller need
+// not load it beforehand to find out).
+template <bool NON_INCREASING, bool DIVIDED, bool CHECK_FIRST = false>
+__device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
     const float* terms_array, float divisor, float second_divisor, uint32_t count, int mode, float bound,
     ReplayScratch& scratch, int tid, const uint4* chunk_steps = nullptr)
 {
@@ -390,36 +392,7 @@ __device__ __noinline__ RunningSum exact_running_sum_of_array(
     const auto term_at = [&](uint32_t i) { return scaled(terms_array[i]); };
     const int lane = tid & (kWaveSize - 1);
     float sum = 0.0f;
-    // The first kSequentialHead terms are added one by one, as the CPU does (every thread runs the same
-    // loop on wave-uniform values): the sum climbs through most of its binades here, each of which
-    // would cost the scan below a round, and a stop condition usually holds this early.
     const uint32_t head = min(count, static_cast<uint32_t>(kSequentialHead));
-    {
-        float head_terms[kHeadSlots];
-#pragma unroll
-        for (int slot = 0; slot < kHeadSlots; ++slot)
-        {
-            const uint32_t i = static_cast<uint32_t>(slot * kWaveSize + lane);
-            head_terms[slot] = i < head ? term_at(i) : 0.0f;
-        }
-#pragma unroll
-        for (int slot = 0; slot < kHeadSlots; ++slot)
-        {
-            const uint32_t slot_first = static_cast<uint32_t>(slot * kWaveSize);
-            const uint32_t slot_count = head > slot_first ? min(head - slot_first, static_cast<uint32_t>(kWaveSize)) : 0u;
-            for (uint32_t l = 0; l < slot_count; ++l)
-            {
-                sum += read_lane(head_terms[slot], static_cast<int>(l));
-                if ((mode == kStopAtOrAbove && sum >= bound) || (mode == kStopAbove && sum > bound))
-                    return RunningSum{sum, slot_first + l, true};
-            }
-        }
-        if (head >= count)
-            return RunningSum{sum, 0u, false};
-    }
-    if (tid == 0)
-        scratch.first_event[0] = 0xffffffffu;
-    uint32_t round = 0;
     // the terms of the next chunk are asked for while this one is summed
     float upcoming[kReplayPerThread];
     const bool summing = tid < kSumThreads;
@@ -447,7 +420,51 @@ __device__ __noinline__ RunningSum exact_running_sum_of_array(
                 upcoming[j] = (summing && first + j < chunk_end) ? terms_array[first + j] : 0.0f;
         }
     };
-    fetch(0);
+    // A sum that runs over the whole row (the normaliser) asks for everything it will need first - the composed
+    // steps of the first 64 whole chunks, one per lane, and the first chunk's terms - so that the loads of the
+    // head below are not the first of three trips to memory, one behind the other.
+    uint4 own_chunk_steps{0u, 0u, 0u, 0u};
+    if (NON_INCREASING && !DIVIDED && chunk_steps != nullptr && static_cast<uint32_t>(lane) < count / kReplayChunk)
+        own_chunk_steps = chunk_steps[lane];
+    if (NON_INCREASING && count > head)
+        fetch(0);
+    // The first kSequentialHead terms are added one by one, as the CPU does (every thread runs the same
+    // loop on wave-uniform values): the sum climbs through most of its binades here, each of which
+    // would cost the scan below a round, and a stop condition usually holds this early.
+    {
+        float head_terms[kHeadSlots];
+#pragma unroll
+        for (int slot = 0; slot < kHeadSlots; ++slot)
+        {
+            const uint32_t i = static_cast<uint32_t>(slot * kWaveSize + lane);
+            head_terms[slot] = i < head ? term_at(i) : 0.0f;
+        }
+        if (CHECK_FIRST)
+        {
+            const float first_term = read_lane(head_terms[0], 0);
+            if (!is_finite_f32(first_term))
+                return RunningSum{first_term, 0u, false};
+        }
+#pragma unroll
+        for (int slot = 0; slot < kHeadSlots; ++slot)
+        {
+            const uint32_t slot_first = static_cast<uint32_t>(slot * kWaveSize);
+            const uint32_t slot_count = head > slot_first ? min(head - slot_first, static_cast<uint32_t>(kWaveSize)) : 0u;
+            for (uint32_t l = 0; l < slot_count; ++l)
+            {
+                sum += read_lane(head_terms[slot], static_cast<int>(l));
+                if ((mode == kStopAtOrAbove && sum >= bound) || (mode == kStopAbove && sum > bound))
+                    return RunningSum{sum, slot_first + l, true};
+            }
+        }
+        if (head >= count)
+            return RunningSum{sum, 0u, false};
+    }
+    if (tid == 0)
+        scratch.first_event[0] = 0xffffffffu;
+    uint32_t round = 0;
+    if (!NON_INCREASING)
+        fetch(0);
     bool fetched = true; // `upcoming` holds the terms of the chunk at `base`
     for (uint32_t base = 0; base < count; base += kReplayChunk)
     {
@@ -458,7 +475,17 @@ __device__ __noinline__ RunningSum exact_running_sum_of_array(
             // A whole chunk whose composed step was worked out beforehand for the exponent that the sum has now:
             // if that step leaves the mantissa inside the binade, nothing inside the chunk left it either (the
             // mantissa never decreases), and the chunk is this one addition.
-            const uint4 composed = chunk_steps[base / kReplayChunk];
+            const uint32_t chunk = base / kReplayChunk;
+            uint4 composed;
+            if (chunk < static_cast<uint32_t>(kWaveSize))
+            {
+                composed.x = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_chunk_steps.x), static_cast<int>(chunk)));
+                composed.y = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_chunk_steps.y), static_cast<int>(chunk)));
+                composed.z = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_chunk_steps.z), static_cast<int>(chunk)));
+                composed.w = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_chunk_steps.w), static_cast<int>(chunk)));
+            }
+            else
+                composed = chunk_steps[chunk];
             int exponent;
             uint32_t mantissa;
             decode_sum(sum, exponent, mantissa);
@@ -562,15 +589,27 @@ __device__ __noinline__ RunningSum exact_running_sum_of_array(
     return RunningSum{sum, 0u, false};
 }
 
+// ... as a function of its own: a kernel that sums several times (Top-P walk, draw, the verification's residual)
+// holds one copy of it.
+template <bool NON_INCREASING, bool DIVIDED>
+__device__ __noinline__ RunningSum exact_running_sum_of_array(
+    const float* terms_array, float divisor, float second_divisor, uint32_t count, int mode, float bound,
+    ReplayScratch& scratch, int tid, const uint4* chunk_steps = nullptr)
+{
+    return exact_running_sum_of_array_inline<NON_INCREASING, DIVIDED>(terms_array, divisor, second_divisor, count, mode, bound, scratch, tid, chunk_steps);
+}
+
 // The running sum of terms [0, count) of a sorted row.  PHASE 0 (terms that never grow) also stops
 // once the sum no longer moves.  Every thread of the workgroup must call it.
 template <int PHASE>
 __device__ __forceinline__ RunningSum exact_running_sum(
     const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
 {
-    return exact_running_sum_of_array<PHASE == 0, PHASE != 0>(
-        row.terms0, row.normalizer, PHASE == 2 ? row.renormalizer : 1.0f, count, mode, bound, scratch, tid,
-        PHASE == 0 ? row.chunk_steps : nullptr);
+    if constexpr (PHASE == 0) // the normaliser: one call per kernel, inlined (a call saves and restores its registers through memory)
+        return exact_running_sum_of_array_inline<true, false, true>(row.terms0, 1.0f, 1.0f, count, mode, bound, scratch, tid, row.chunk_steps);
+    else
+        return exact_running_sum_of_array<false, true>(
+            row.terms0, row.normalizer, PHASE == 2 ? row.renormalizer : 1.0f, count, mode, bound, scratch, tid, nullptr);
 }
 
 // The same running sum over a row stored as runs: `count` elements are added, run after run.  A run of
@@ -807,10 +846,16 @@ __device__ __forceinline__ void replay_sorted_window(
     };
 
     // ---- normaliser (session.cpp:92-103).  A first term that is not finite poisons the sum.
-    const float first_term = row_term<0>(sorted, 0);
-    float normalizer = first_term;
-    if (is_finite_f32(first_term))
-        normalizer = running_sum(std::integral_constant<int, 0>{}, n, kStopNever, 0.0f).sum;
+    float normalizer;
+    if constexpr (RUNS)
+    {
+        const float first_term = row_term<0>(sorted, 0);
+        normalizer = first_term;
+        if (is_finite_f32(first_term))
+            normalizer = running_sum(std::integral_constant<int, 0>{}, n, kStopNever, 0.0f).sum;
+    }
+    else
+        normalizer = running_sum(std::integral_constant<int, 0>{}, n, kStopNever, 0.0f).sum; // (checks the first term itself)
     if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
     {
         if (tid == 0)
