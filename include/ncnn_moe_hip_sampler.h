@@ -137,7 +137,9 @@ int ncnn_moe_hip_sampler_sample(
  * batch holds both rows with 64 < top_k <= 1024 and rows with a wider or no window: the two later
  * passes, each of which keeps one workgroup per row busy, then run side by side, one of them on a
  * second stream of the handle that forks from and joins `stream` (worth its two stream hand-overs,
- * some 30 us, from about a hundred rows of each kind); add NCNN_MOE_PASSES_NO_WIDE_WINDOWS when the
+ * some 30 us, from about a hundred rows of each kind; a row with top_k <= 64 whose ties overflow the
+ * first kernel's lists is then finished by the full-order kernels rather than by the select kernel for
+ * wider windows: same result, NCNN_MOE_ROW_FLAG_GENERAL_PATH set); add NCNN_MOE_PASSES_NO_WIDE_WINDOWS when the
  * caller knows that no row has 64 < top_k <= 1024: the select kernel for such windows is then not
  * enqueued (a row that has one after all is served by the full-order kernels: slower, same result).
  * Calls on one handle share its scratch memory and must not overlap. */

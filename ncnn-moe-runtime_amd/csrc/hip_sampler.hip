@@ -220,12 +220,12 @@ void use_select_scratch(SamplerArgs& a, const SelectScratch& scratch)
 }
 
 template <int DTYPE>
-void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, SamplerArgs a, bool only_pending, bool scatter_segments)
+void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, SamplerArgs a, int only_pending, bool scatter_segments)
 {
     a.segments = g.segments;
     a.chunks_per_segment = g.chunks_per_segment;
     a.max_select_top_k = g.wide ? kSelectTopK : kFastTopK;
-    a.only_pending = only_pending ? 1 : 0;
+    a.only_pending = only_pending;
     dim3 grid(g.segments, rows, 1);
     a.xcd_grouped = 0;
     if (g.segments > 1 && !scatter_segments)
@@ -307,20 +307,33 @@ int launch_sampler(
     if (batch_geometry.segments > s->max_segments)
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab exceeds the handle's max_vocab");
 
-    if (passes.select)
-    {
-        if (dtype == NCNN_MOE_LOGITS_F32)
-            launch_select<NCNN_MOE_LOGITS_F32>(batch_geometry, rows, stream, a, false, s->scatter_segments != 0);
-        else
-            launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, a, false, s->scatter_segments != 0);
-    }
-    const auto launch_wide = [&](hipStream_t on) {
+    // only_pending: 1 = the rows an earlier launch left pending, 2 = the rows whose options ask for a wide window
+    const auto launch_wide = [&](hipStream_t on, int only_pending) {
         const SelectGeometry row_geometry = select_geometry(dtype, span, rows, true);
         if (dtype == NCNN_MOE_LOGITS_F32)
-            launch_select<NCNN_MOE_LOGITS_F32>(row_geometry, rows, on, a, true, s->scatter_segments != 0);
+            launch_select<NCNN_MOE_LOGITS_F32>(row_geometry, rows, on, a, only_pending, s->scatter_segments != 0);
         else
-            launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, on, a, true, s->scatter_segments != 0);
+            launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, on, a, only_pending, s->scatter_segments != 0);
     };
+    // Side by side (see below) with the first select in the call: the wide select is forked off in front of it
+    // and picks its rows by their options, and the first select leaves those rows alone.
+    const bool side_by_side = passes.side_by_side && passes.wide_select && passes.full_order && s->side_stream != nullptr;
+    const bool early_wide = side_by_side && passes.select;
+    if (early_wide)
+    {
+        if (hipEventRecord(s->side_fork, stream) != hipSuccess || hipStreamWaitEvent(s->side_stream, s->side_fork, 0) != hipSuccess)
+            return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
+        launch_wide(s->side_stream, 2);
+    }
+    if (passes.select)
+    {
+        SamplerArgs first = a;
+        first.leave_wide_rows = early_wide ? 1 : 0;
+        if (dtype == NCNN_MOE_LOGITS_F32)
+            launch_select<NCNN_MOE_LOGITS_F32>(batch_geometry, rows, stream, first, 0, s->scatter_segments != 0);
+        else
+            launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, first, 0, s->scatter_segments != 0);
+    }
     // A long row's radix sort is spread over several workgroups (two tiles each, at most kMaxSortParts):
     // two launches per pass over a (parts, rows) grid.  Short rows keep the one-workgroup kernel.
     const uint32_t sort_tiles = static_cast<uint32_t>((static_cast<uint64_t>(vocab) + kSortTile - 1) / kSortTile);
@@ -388,13 +401,16 @@ int launch_sampler(
     // sort that is spread over every compute unit, was measured and is slower: the two one-workgroup-per-row
     // kernels then share compute units and the wide select takes 330 us instead of 210.)
     // The full-order kernels leave the wide select's rows alone, and are enqueued once more behind the
-    // join for the rows that the wide select could not finish (ties beyond its lists); without such rows
-    // that launch exits at once.
-    if (passes.side_by_side && passes.wide_select && passes.full_order && s->side_stream != nullptr)
+    // join for the rows that the wide select (or, when that one started beside it, the first select) could
+    // not finish: ties beyond their lists; without such rows that launch exits at once.
+    if (side_by_side)
     {
-        if (hipEventRecord(s->side_fork, stream) != hipSuccess || hipStreamWaitEvent(s->side_stream, s->side_fork, 0) != hipSuccess)
-            return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
-        launch_wide(s->side_stream);
+        if (!early_wide)
+        {
+            if (hipEventRecord(s->side_fork, stream) != hipSuccess || hipStreamWaitEvent(s->side_stream, s->side_fork, 0) != hipSuccess)
+                return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
+            launch_wide(s->side_stream, 1);
+        }
         SamplerArgs own_rows = a;
         own_rows.leave_wide_rows = 1;
         launch_full_order(own_rows, false);
@@ -405,7 +421,7 @@ int launch_sampler(
     else
     {
         if (passes.wide_select)
-            launch_wide(stream);
+            launch_wide(stream, 1);
         if (passes.full_order)
             launch_full_order(a, false);
     }

@@ -17,8 +17,9 @@ struct SamplerArgs
     uint32_t chunks_per_segment; // chunks (512 x 5 fp32 / 3 bf16 vectors) one workgroup streams
     uint32_t max_select_top_k;   // widest Top-K window the select kernel of this launch serves
     int force_general;
-    int only_pending;            // serve only rows an earlier launch of the call left pending
-    int leave_wide_rows;         // full-order kernels: rows that the wide select serves are another stream's
+    int only_pending;            // wide select: 1 = serve the rows an earlier launch of the call left pending; 2 = serve the rows
+                                 // whose options ask for a window of 65 to 1024, whatever their state (it runs beside the first select)
+    int leave_wide_rows;         // first select and full-order kernels: rows that the wide select serves are another stream's
 
     const ncnn_moe_sample_params* params;
     const float* uniforms;

@@ -454,7 +454,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
 
     __shared__ Shared shared;
 
-    if (a.only_pending && a.row_state[row] != kRowNeedsGeneral)
+    if (a.only_pending == 1 && a.row_state[row] != kRowNeedsGeneral)
         return;
     if (WIDE) { NCNN_MOE_STAMP_RESET(row, 12); NCNN_MOE_STAMP_NEXT(row, 12); }
     // The first chunk's loads go out before anything that waits for the row's options.
@@ -484,9 +484,18 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     const int mode = resolve_row_mode(p, a.vocab, a.max_select_top_k, a.force_general, effective_k, status);
     if (mode == kModeInvalid || mode == kModeGeneral)
     {
-        // (a launch for pending rows finds a full-order row marked already, and the full-order kernels may be
-        // serving it at this moment on another stream: it is not touched)
-        if (segment == 0 && tid == 0 && !(a.only_pending && mode == kModeGeneral))
+        // A row that another launch of the call serves is not touched: a launch for pending rows finds a
+        // full-order row marked already (the full-order kernels may be serving it at this moment on another
+        // stream); a wide select that runs beside the first select leaves the marking of every row to that
+        // one; and the first select leaves the wide select's rows alone when told that one runs beside it.
+        bool not_mine = a.only_pending == 2 || (a.only_pending == 1 && mode == kModeGeneral);
+        if (!WIDE && a.leave_wide_rows != 0 && mode == kModeGeneral)
+        {
+            uint32_t wide_k = 0;
+            int wide_status = NCNN_MOE_ROW_OK;
+            not_mine = resolve_row_mode(p, a.vocab, static_cast<uint32_t>(kSelectTopK), a.force_general, wide_k, wide_status) != kModeGeneral;
+        }
+        if (segment == 0 && tid == 0 && !not_mine)
         {
             if (mode == kModeInvalid)
             {
@@ -503,6 +512,8 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     }
     const bool greedy = mode == kModeGreedy;
     const int top_k = static_cast<int>(effective_k);
+    if (WIDE && a.only_pending == 2 && (greedy || effective_k <= static_cast<uint32_t>(kFastTopK)))
+        return; // the first select's row
     // the list is tightened when it grows past this; a wide list keeps room for a chunk's additions
     const uint32_t tighten_limit = WIDE ? static_cast<uint32_t>(2 * top_k + 64) : static_cast<uint32_t>(kNarrowListCap - 192);
     uint32_t next_check = 0;      // chunk at which the list is looked at next

@@ -148,7 +148,15 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     const int mode = resolve_row_mode(p, a.vocab, kFastTopK, a.force_general, effective_k, status);
     if (mode == kModeInvalid || mode == kModeGeneral)
     {
-        if (segment == 0 && tid == 0)
+        // (a row with a window of 65 to 1024 is left alone when a wide select runs beside this kernel)
+        bool not_mine = false;
+        if (a.leave_wide_rows != 0 && mode == kModeGeneral)
+        {
+            uint32_t wide_k = 0;
+            int wide_status = NCNN_MOE_ROW_OK;
+            not_mine = resolve_row_mode(p, a.vocab, static_cast<uint32_t>(kSelectTopK), a.force_general, wide_k, wide_status) != kModeGeneral;
+        }
+        if (segment == 0 && tid == 0 && !not_mine)
         {
             if (mode == kModeInvalid)
             {

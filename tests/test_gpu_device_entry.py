@@ -61,14 +61,16 @@ def test_three_passes_on_a_caller_stream(rows):
 def test_later_passes_side_by_side(dtype):
     """Rows with wide windows and rows without a window in one batch: the wide select on the handle's
     second stream beside the full-order kernels (flag NCNN_MOE_PASSES_SIDE_BY_SIDE, and sample() by
-    itself from 32 rows of each kind), with tie-heavy wide rows that the wide select hands on to the
-    full-order kernels behind the join.  Same results as one pass after the other, and as the oracle."""
+    itself from 32 rows of each kind), with tie-heavy rows that the wide select, and the first select for a
+    window of 20, hand on to the full-order kernels behind the join.  Same results as one pass after the
+    other, and as the oracle."""
     print("[case] later passes side by side, %s" % dtype, flush=True)
     from ncnn_moe_runtime_amd import workloads
     rng = np.random.default_rng(77)
     rows, vocab = 120, 30011
     logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
     logits[5::12] = np.round(logits[5::12])  # a few thousand equal logits around every cut
+    logits[2::12] = np.round(logits[2::12] / 2.0) * 2.0  # (top_k 20: hundreds of equal logits at the cut)
     params = hip_sampler.make_params(rows, 0.9, 0, 0.9, 0.0)
     params["top_k"] = np.array([(700, 0, 20, 300, 2000, 1024)[i % 6] for i in range(rows)], dtype=np.uint32)
     params["temperature"][::17] = 0.0
@@ -79,7 +81,16 @@ def test_later_passes_side_by_side(dtype):
     with hip_sampler.HipSampler(rows, vocab) as sampler:
         in_turn = _run(sampler, data, params, uniforms, hip_sampler.PASSES_FULL_ORDER, stream)
         beside = _run(sampler, data, params, uniforms, hip_sampler.PASSES_FULL_ORDER | hip_sampler.PASSES_SIDE_BY_SIDE, stream)
-        assert in_turn.tobytes() == beside.tobytes()
+        # (a row that the first select hands on is served by the wide select when the passes run in turn and by
+        # the full-order kernels behind the join when they run side by side: the same result, and the flag
+        # that names the path differs)
+        handed_on = np.zeros(rows, dtype=bool)
+        handed_on[2::12] = params["temperature"][2::12] != 0.0
+        assert in_turn[~handed_on].tobytes() == beside[~handed_on].tobytes()
+        assert ((beside["flags"] ^ in_turn["flags"])[handed_on] == hip_sampler.FLAG_GENERAL_PATH).all()
+        for field in beside.dtype.names:
+            if field != "flags":
+                assert in_turn[field].tobytes() == beside[field].tobytes(), field
         parity_util.assert_results_match(beside, cpu, dtype, "side by side, device entry")
         for _ in range(3):  # the second stream forks and joins again on every call
             again = _run(sampler, data, params, uniforms, hip_sampler.PASSES_FULL_ORDER | hip_sampler.PASSES_SIDE_BY_SIDE, stream)
