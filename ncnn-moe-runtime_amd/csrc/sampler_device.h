@@ -291,6 +291,24 @@ __device__ __forceinline__ int lanes_below(uint64_t mask)
         static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)));
 }
 
+// The valid lanes of the wave that hold the same 8-bit digit as the calling lane, as the two halves of
+// a lane mask (a lane that is not valid gets no peers and is nobody's peer).  One compare and two
+// three-operand bit operations per bit of the digit.
+__device__ __forceinline__ void wave_digit_peers(uint32_t digit, bool valid, uint32_t& low, uint32_t& high)
+{
+    const uint64_t all = __builtin_amdgcn_ballot_w64(valid);
+    low = valid ? static_cast<uint32_t>(all) : 0u;
+    high = valid ? static_cast<uint32_t>(all >> 32) : 0u;
+#pragma unroll
+    for (int b = 0; b < 8; ++b)
+    {
+        const uint32_t mine = static_cast<uint32_t>(static_cast<int32_t>(digit << (31 - b)) >> 31); // all ones if the bit is set
+        const uint64_t set = __builtin_amdgcn_ballot_w64(mine != 0u);
+        low &= ~(static_cast<uint32_t>(set) ^ mine);
+        high &= ~(static_cast<uint32_t>(set >> 32) ^ mine);
+    }
+}
+
 // Workgroup barrier that orders LDS traffic only: waits for this wave's LDS operations, not for its
 // outstanding global loads and stores (which __syncthreads() would also wait for).
 __device__ __forceinline__ void lds_barrier()

@@ -175,21 +175,15 @@ __global__ __launch_bounds__(kSortThreads) void general_sort_kernel(SamplerArgs 
                 const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
                 const bool valid = i < n;
                 const uint32_t digit = (tile_keys[e] >> shift) & 255u;
-                uint64_t peers = __ballot(valid);
-#pragma unroll
-                for (int b = 0; b < 8; ++b)
-                {
-                    const bool bit = (digit >> b) & 1u;
-                    const uint64_t set = __ballot(valid && bit);
-                    peers &= bit ? set : ~set;
-                }
-                const int rank_in_round = lanes_below(peers);
+                uint32_t peers_low, peers_high;
+                wave_digit_peers(digit, valid, peers_low, peers_high);
+                const uint32_t rank_in_round = __builtin_amdgcn_mbcnt_hi(peers_high, __builtin_amdgcn_mbcnt_lo(peers_low, 0u));
                 uint32_t seen = 0;
                 if (valid)
                     seen = wave_counts[wave][digit];
-                tile_ranks[e] = seen + static_cast<uint32_t>(rank_in_round);
+                tile_ranks[e] = seen + rank_in_round;
                 if (valid && rank_in_round == 0)
-                    wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popcll(peers));
+                    wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popc(peers_low) + __popc(peers_high));
             }
             lds_barrier();
             // per digit: slots of the waves inside the digit's run, the run's length, then the runs' starts
@@ -293,23 +287,42 @@ __device__ __forceinline__ void load_sort_keys(
         static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
     const uint32_t* source_keys = a.sort_keys[(pass + 1) & 1] + row * a.sort_stride;
     const uint32_t* source_indices = a.sort_indices[(pass + 1) & 1] + row * a.sort_stride;
+    // (one loop per source, so that a thread's loads are in flight together)
+    if (pass == 0)
+    {
+        float values[kSortPerThread];
+#pragma unroll
+        for (int e = 0; e < kSortPerThread; ++e)
+        {
+            const uint32_t i = first + static_cast<uint32_t>(e * group_stride + tid_in_group);
+            values[e] = load_logit<DTYPE>(row_pointer, i < n ? i : n - 1u); // always a valid address; masked below
+        }
+#pragma unroll
+        for (int e = 0; e < kSortPerThread; ++e)
+        {
+            const uint32_t i = first + static_cast<uint32_t>(e * group_stride + tid_in_group);
+            out_keys[e] = i < n ? descending_key(values[e]) : 0xffffffffu;
+            out_indices[e] = i;
+        }
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < kSortPerThread; ++e)
     {
         const uint32_t i = first + static_cast<uint32_t>(e * group_stride + tid_in_group);
-        const uint32_t source = i < n ? i : n - 1u; // always a valid address; masked below
-        uint32_t key;
-        uint32_t index = i;
-        if (pass == 0)
-            key = descending_key(load_logit<DTYPE>(row_pointer, source));
-        else
+        const uint32_t source = i < n ? i : n - 1u;
+        out_keys[e] = source_keys[source];
+        out_indices[e] = PAIRS ? source_indices[source] : i;
+    }
+#pragma unroll
+    for (int e = 0; e < kSortPerThread; ++e)
+    {
+        const uint32_t i = first + static_cast<uint32_t>(e * group_stride + tid_in_group);
+        if (i >= n)
         {
-            key = source_keys[source];
-            if (PAIRS)
-                index = source_indices[source];
+            out_keys[e] = 0xffffffffu;
+            out_indices[e] = i;
         }
-        out_keys[e] = i < n ? key : 0xffffffffu;
-        out_indices[e] = i < n ? index : i;
     }
 }
 
@@ -446,21 +459,15 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_scatter_kernel(Sampler
             const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
             const bool valid = i < n;
             const uint32_t digit = (tile_keys[e] >> shift) & 255u;
-            uint64_t peers = __ballot(valid);
-#pragma unroll
-            for (int b = 0; b < 8; ++b)
-            {
-                const bool bit = (digit >> b) & 1u;
-                const uint64_t set = __ballot(valid && bit);
-                peers &= bit ? set : ~set;
-            }
-            const int rank_in_round = lanes_below(peers);
+            uint32_t peers_low, peers_high;
+            wave_digit_peers(digit, valid, peers_low, peers_high);
+            const uint32_t rank_in_round = __builtin_amdgcn_mbcnt_hi(peers_high, __builtin_amdgcn_mbcnt_lo(peers_low, 0u));
             uint32_t seen = 0;
             if (valid)
                 seen = wave_counts[wave][digit];
-            tile_ranks[e] = seen + static_cast<uint32_t>(rank_in_round);
+            tile_ranks[e] = seen + rank_in_round;
             if (valid && rank_in_round == 0)
-                wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popcll(peers));
+                wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popc(peers_low) + __popc(peers_high));
         }
         lds_barrier();
         uint32_t digit_total = 0;
