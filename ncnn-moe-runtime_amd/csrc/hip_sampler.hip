@@ -337,7 +337,7 @@ int launch_sampler(
     // A long row's radix sort is spread over several workgroups (two tiles each, at most kMaxSortParts):
     // two launches per pass over a (parts, rows) grid.  Short rows keep the one-workgroup kernel.
     const uint32_t sort_tiles = static_cast<uint32_t>((static_cast<uint64_t>(vocab) + kSortTile - 1) / kSortTile);
-    const uint32_t sort_tiles_per_part = std::max<uint32_t>(2, (sort_tiles + kMaxSortParts - 1) / kMaxSortParts);
+    const uint32_t sort_tiles_per_part = std::max<uint32_t>(1, (sort_tiles + kMaxSortParts - 1) / kMaxSortParts);
     const uint32_t sort_parts = std::max<uint32_t>(1, (sort_tiles + sort_tiles_per_part - 1) / sort_tiles_per_part);
     const auto launch_spread_sort = [&](SamplerArgs spread, auto dtype_tag, auto pairs_tag) {
         constexpr int kType = decltype(dtype_tag)::value;
@@ -355,7 +355,7 @@ int launch_sampler(
     // `leftovers`: the launch behind the wide select, for the few rows (usually none) that it could not
     // finish; it is kept to two kernels, because every launch costs its few microseconds even with no row to serve.
     const auto launch_full_order = [&](SamplerArgs a, bool leftovers) {
-        const bool spread_sort = sort_parts > 1 && s->spread_sort != 0 && !leftovers;
+        const bool spread_sort = sort_tiles >= 4 && s->spread_sort != 0 && !leftovers;
         const bool runs = dtype == NCNN_MOE_LOGITS_BF16 && !want_distribution;
         // the token indices ride along with the keys only when the whole distribution is exported
         const auto sort_rows = [&](auto dtype_tag, auto pairs_tag) {

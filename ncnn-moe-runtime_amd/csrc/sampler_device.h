@@ -42,7 +42,7 @@ constexpr int kSortThreads = 1024;
 constexpr int kSortWaves = kSortThreads / kWaveSize;
 constexpr int kSortPerThread = 8;
 constexpr int kSortTile = kSortThreads * kSortPerThread;
-constexpr int kMaxSortParts = 8;              // workgroups one row's radix sort is spread over
+constexpr int kMaxSortParts = 16;             // workgroups one row's radix sort is spread over
 constexpr int kReplayThreads = 1024;
 // The exact running sums are the work of the workgroup's first eight waves (two per SIMD), each thread
 // composing a few consecutive terms: every wave that takes part pays the scan across its lanes and the

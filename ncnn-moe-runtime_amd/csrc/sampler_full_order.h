@@ -369,8 +369,9 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(Sampl
     }
 }
 
+// (at most 64 registers a thread: two workgroups of 1,024 threads share a compute unit)
 template <int DTYPE, bool PAIRS>
-__global__ __launch_bounds__(kSortThreads) void sort_part_scatter_kernel(SamplerArgs a)
+__global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void sort_part_scatter_kernel(SamplerArgs a)
 {
     constexpr int kFirstDigit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0 : 2;
     const uint32_t part = blockIdx.x;
@@ -437,17 +438,13 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_scatter_kernel(Sampler
         return;
     // A wave owns 512 consecutive keys of a tile and ranks them in 8 rounds of 64, so that the order
     // inside the wave is the input order (see general_sort_kernel).
-    uint32_t tile_keys[kSortPerThread];
-    uint32_t tile_indices[kSortPerThread];
-    load_sort_keys<DTYPE, PAIRS>(a, row, pass, first_tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread), n, lane, kWaveSize,
-                                 tile_keys, tile_indices);
+    // (no tile is fetched ahead: a workgroup has one tile or few, and two workgroups share a compute unit)
     for (uint32_t tile = first_tile; tile < end; tile += kSortTile)
     {
-        uint32_t next_keys[kSortPerThread];
-        uint32_t next_indices[kSortPerThread];
-        const uint32_t next_tile = tile + kSortTile < end ? tile + kSortTile : tile;
-        load_sort_keys<DTYPE, PAIRS>(a, row, pass, next_tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread), n, lane, kWaveSize,
-                                     next_keys, next_indices);
+        uint32_t tile_keys[kSortPerThread];
+        uint32_t tile_indices[kSortPerThread];
+        load_sort_keys<DTYPE, PAIRS>(a, row, pass, tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread), n, lane, kWaveSize,
+                                     tile_keys, tile_indices);
         for (int i = tid; i < kSortWaves * 256; i += kSortThreads)
             (&wave_counts[0][0])[i] = 0;
         uint32_t tile_ranks[kSortPerThread];
@@ -536,12 +533,6 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_scatter_kernel(Sampler
             }
         }
         lds_barrier();
-#pragma unroll
-        for (int e = 0; e < kSortPerThread; ++e)
-        {
-            tile_keys[e] = next_keys[e];
-            tile_indices[e] = next_indices[e];
-        }
     }
 }
 
