@@ -349,7 +349,10 @@ int launch_sampler(
         {
             spread.sort_pass = static_cast<uint32_t>(pass);
             hipLaunchKernelGGL((sort_part_histogram_kernel<kType>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
-            hipLaunchKernelGGL((sort_part_scatter_kernel<kType, kPairs>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
+            if (pass == 0 && !kPairs) // (keys alone: the first pass need not keep the order of equal digits)
+                hipLaunchKernelGGL((sort_part_scatter_kernel<kType, kPairs, true>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
+            else
+                hipLaunchKernelGGL((sort_part_scatter_kernel<kType, kPairs>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
         }
     };
     // `leftovers`: the launch behind the wide select, for the few rows (usually none) that it could not

@@ -370,7 +370,10 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(Sampl
 }
 
 // (at most 64 registers a thread: two workgroups of 1,024 threads share a compute unit)
-template <int DTYPE, bool PAIRS>
+// ANY_ORDER: the keys of one digit value may leave in any order.  That holds for the first pass of a sort
+// of keys alone (equal keys cannot be told apart, and there is no earlier pass whose order must survive);
+// a key's rank among its wave's keys of the same digit is then what an LDS atomic returns.
+template <int DTYPE, bool PAIRS, bool ANY_ORDER = false>
 __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void sort_part_scatter_kernel(SamplerArgs a)
 {
     constexpr int kFirstDigit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0 : 2;
@@ -456,6 +459,11 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
             const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
             const bool valid = i < n;
             const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+            if (ANY_ORDER)
+            {
+                tile_ranks[e] = valid ? atomicAdd(&wave_counts[wave][digit], 1u) : 0u;
+                continue;
+            }
             uint32_t peers_low, peers_high;
             wave_digit_peers(digit, valid, peers_low, peers_high);
             const uint32_t rank_in_round = __builtin_amdgcn_mbcnt_hi(peers_high, __builtin_amdgcn_mbcnt_lo(peers_low, 0u));
