@@ -65,6 +65,7 @@ struct ncnn_moe_hip_sampler
     uint32_t* sort_keys[2] = {nullptr, nullptr};
     uint32_t* sort_indices[2] = {nullptr, nullptr};
     uint64_t sort_stride = 0;
+    uint32_t* row_list = nullptr;         // [1 + rows], see SamplerArgs::row_list
     uint32_t* sort_part_counts = nullptr; // [rows][kMaxSortParts][256]
     double* term_sums = nullptr;          // [rows][term_sum_parts]: fp64 sums of the terms kernel's blocks
     uint4* chunk_steps = nullptr;         // [rows][chunk_capacity]: composed step of every whole chunk of a sorted row's terms
@@ -348,7 +349,7 @@ int launch_sampler(
         for (int pass = 0; pass < passes; ++pass)
         {
             spread.sort_pass = static_cast<uint32_t>(pass);
-            hipLaunchKernelGGL((sort_part_histogram_kernel<kType>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
+            hipLaunchKernelGGL((sort_part_histogram_kernel<kType>), dim3((sort_parts + kHistogramParts - 1) / kHistogramParts, rows), dim3(kSortThreads), 0, stream, spread);
             if (pass == 0 && !kPairs) // (keys alone: the first pass need not keep the order of equal digits)
                 hipLaunchKernelGGL((sort_part_scatter_kernel<kType, kPairs, true>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
             else
@@ -360,6 +361,12 @@ int launch_sampler(
     const auto launch_full_order = [&](SamplerArgs a, bool leftovers) {
         const bool spread_sort = sort_tiles >= 4 && s->spread_sort != 0 && !leftovers;
         const bool runs = dtype == NCNN_MOE_LOGITS_BF16 && !want_distribution;
+        if (!leftovers && !runs)
+        {
+            // (the kernels over a (parts, rows) grid find their rows in a list)
+            hipLaunchKernelGGL(full_order_row_list_kernel, dim3(1), dim3(kSortThreads), 0, stream, a, rows, s->row_list);
+            a.row_list = s->row_list;
+        }
         // the token indices ride along with the keys only when the whole distribution is exported
         const auto sort_rows = [&](auto dtype_tag, auto pairs_tag) {
             constexpr int kType = decltype(dtype_tag)::value;
@@ -593,6 +600,7 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
         CREATE_CHECK(hipMalloc(&s->sort_keys[i], rows * s->sort_stride * sizeof(uint32_t)));
         CREATE_CHECK(hipMalloc(&s->sort_indices[i], rows * s->sort_stride * sizeof(uint32_t)));
     }
+    CREATE_CHECK(hipMalloc(&s->row_list, (static_cast<size_t>(rows) + 1) * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->sort_part_counts, rows * kMaxSortParts * 256 * sizeof(uint32_t)));
     s->term_sum_parts = (max_vocab + kTermsThreads * kTermsPerThread - 1) / (kTermsThreads * kTermsPerThread);
     s->chunk_capacity = max_vocab / kReplayChunk + 1;
@@ -649,7 +657,7 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
     void* buffers[] = {
         s->logits, s->params, s->uniforms, s->results, s->segment_values, s->segment_indices,
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->split_records, s->row_epoch, s->sort_keys[0], s->sort_keys[1],
-        s->sort_indices[0], s->sort_indices[1], s->sort_part_counts, s->term_sums, s->chunk_steps, s->distribution_ids, s->distribution_probabilities,
+        s->sort_indices[0], s->sort_indices[1], s->sort_part_counts, s->row_list, s->term_sums, s->chunk_steps, s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
         s->verify_probabilities, s->verify_counts, s->verify_long_ids, s->verify_long_probabilities, s->verify_dense};
     for (void* buffer : buffers)

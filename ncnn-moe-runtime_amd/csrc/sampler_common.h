@@ -61,6 +61,9 @@ struct SamplerArgs
     uint32_t term_sum_parts;
     uint32_t chunk_capacity;
     uint32_t chunk_steps_ready;
+    // the rows that the full-order kernels serve, listed by full_order_row_list_kernel: [0] their number, then
+    // the rows in ascending order.  Kernels over a (parts, rows) grid look their row up here (null: in row_state).
+    const uint32_t* row_list;
 
     // optional filtered-distribution output: row r writes at most distribution_cap (id, probability)
     // entries from r * distribution_cap on, and its full kept length to distribution_count[r]

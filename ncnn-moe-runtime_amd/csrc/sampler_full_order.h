@@ -22,6 +22,57 @@ __device__ __forceinline__ bool left_to_the_wide_select(const SamplerArgs& a, ui
     return resolve_row_mode(a.params[row], a.vocab, static_cast<uint32_t>(kSelectTopK), a.force_general, effective_k, status) != kModeGeneral;
 }
 
+// The row of a workgroup of a (parts, rows) grid, and whether the full-order kernels serve it.  Most rows
+// of a mixed batch are not theirs, and a workgroup that finds that out from row_state has waited for a
+// trip to memory: with sixteen parts a row those workgroups alone would keep a kernel going for 15 us.
+// With the list, workgroup (part, j) takes the j-th listed row, and the others leave after one load of
+// the list's length, which the scalar cache holds.
+__device__ __forceinline__ bool spread_grid_row(const SamplerArgs& a, uint32_t& row)
+{
+    if (a.row_list != nullptr)
+    {
+        if (blockIdx.y >= a.row_list[0])
+            return false;
+        row = a.row_list[1u + blockIdx.y];
+        return true;
+    }
+    row = blockIdx.y;
+    return a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
+}
+
+// Lists the rows that the full-order kernels serve (see SamplerArgs::row_list).  One workgroup.
+__global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(SamplerArgs a, uint32_t rows, uint32_t* list)
+{
+    __shared__ uint32_t wave_totals[kSortWaves];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    uint32_t listed = 0;
+    for (uint32_t first = 0; first < rows; first += kSortThreads)
+    {
+        const uint32_t row = first + static_cast<uint32_t>(tid);
+        const bool mine = row < rows && a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
+        const uint64_t mask = __builtin_amdgcn_ballot_w64(mine);
+        if (lane == 0)
+            wave_totals[wave] = static_cast<uint32_t>(__popcll(mask));
+        __syncthreads();
+        uint32_t before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w)
+        {
+            const uint32_t t = wave_totals[w];
+            before += w < wave ? t : 0u;
+            total += t;
+        }
+        if (mine)
+            list[1u + listed + before + static_cast<uint32_t>(lanes_below(mask))] = row;
+        listed += total;
+        __syncthreads();
+    }
+    if (tid == 0)
+        list[0] = listed;
+}
+
 template <int DTYPE>
 __device__ __forceinline__ float load_logit(const void* row_pointer, uint32_t i);
 
@@ -326,46 +377,65 @@ __device__ __forceinline__ void load_sort_keys(
     }
 }
 
+// One workgroup counts kHistogramParts consecutive parts of a row, with the loads of all of them in flight
+// together: a workgroup's time is one trip to memory and the hand-over of its counts, whatever it counts,
+// so a part per workgroup would only add rounds of workgroups.  grid (parts / kHistogramParts rounded up, rows).
+constexpr int kHistogramParts = 4;
+
 template <int DTYPE>
 __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(SamplerArgs a)
 {
     constexpr int kFirstDigit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0 : 2;
-    const uint32_t part = blockIdx.x;
-    const uint32_t row = blockIdx.y;
-    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+    const uint32_t first_part = blockIdx.x * kHistogramParts;
+    uint32_t row;
+    if (!spread_grid_row(a, row))
         return;
     const int tid = threadIdx.x;
     const uint32_t n = a.vocab;
     const int pass = static_cast<int>(a.sort_pass);
     const int shift = 8 * (pass + kFirstDigit);
-    __shared__ uint32_t counts[8][257]; // (257: the copies of a digit's counter lie in eight different banks)
-    for (int i = tid; i < 8 * 257; i += kSortThreads)
-        (&counts[0][0])[i] = 0;
+    __shared__ uint32_t counts[kHistogramParts][8][257]; // (257: the copies of a digit's counter lie in eight different banks)
+    for (int i = tid; i < kHistogramParts * 8 * 257; i += kSortThreads)
+        (&counts[0][0][0])[i] = 0;
     __syncthreads();
-    const uint32_t first_tile = part * a.sort_tiles_per_part * kSortTile;
-    const uint32_t end = min(n, first_tile + a.sort_tiles_per_part * kSortTile);
-    for (uint32_t tile = first_tile; tile < end; tile += kSortTile)
+    const uint32_t part_span = a.sort_tiles_per_part * kSortTile;
+    for (uint32_t offset = 0; offset < part_span; offset += kSortTile)
     {
-        uint32_t keys[kSortPerThread];
-        uint32_t unused[kSortPerThread];
-        load_sort_keys<DTYPE, false>(a, row, pass, tile, n, tid, kSortThreads, keys, unused);
+        uint32_t keys[kHistogramParts][kSortPerThread];
 #pragma unroll
-        for (int e = 0; e < kSortPerThread; ++e)
+        for (int q = 0; q < kHistogramParts; ++q)
         {
-            // (eight copies of the counters, a lane using copy lane % 8: the uppermost digit of a row's keys
-            // takes few values, and 64 atomics on one address take as many turns)
-            if (tile + static_cast<uint32_t>(e * kSortThreads + tid) < n)
-                atomicAdd(&counts[tid & 7][(keys[e] >> shift) & 255u], 1u);
+            uint32_t unused[kSortPerThread];
+            const uint32_t tile = min((first_part + q) * part_span + offset, n - 1u); // (a tile behind the row: its keys are not counted)
+            load_sort_keys<DTYPE, false>(a, row, pass, tile, n, tid, kSortThreads, keys[q], unused);
+        }
+#pragma unroll
+        for (int q = 0; q < kHistogramParts; ++q)
+        {
+            const uint32_t tile = (first_part + q) * part_span + offset;
+#pragma unroll
+            for (int e = 0; e < kSortPerThread; ++e)
+            {
+                // (eight copies of the counters, a lane using copy lane % 8: the uppermost digit of a row's keys
+                // takes few values, and 64 atomics on one address take as many turns)
+                if (tile + static_cast<uint32_t>(e * kSortThreads + tid) < n)
+                    atomicAdd(&counts[q][tid & 7][(keys[q][e] >> shift) & 255u], 1u);
+            }
         }
     }
     __syncthreads();
-    if (tid < 256)
     {
-        uint32_t total = 0;
+        const int q = tid >> 8; // kSortThreads / 256 == kHistogramParts
+        const int digit = tid & 255;
+        static_assert(kSortThreads == 256 * kHistogramParts, "a thread per part and digit");
+        if (first_part + q < a.sort_parts)
+        {
+            uint32_t total = 0;
 #pragma unroll
-        for (int copy = 0; copy < 8; ++copy)
-            total += counts[copy][tid];
-        a.sort_part_counts[(static_cast<size_t>(row) * a.sort_parts + part) * 256 + tid] = total;
+            for (int copy = 0; copy < 8; ++copy)
+                total += counts[q][copy][digit];
+            a.sort_part_counts[(static_cast<size_t>(row) * a.sort_parts + first_part + q) * 256 + digit] = total;
+        }
     }
 }
 
@@ -378,8 +448,8 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
 {
     constexpr int kFirstDigit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0 : 2;
     const uint32_t part = blockIdx.x;
-    const uint32_t row = blockIdx.y;
-    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+    uint32_t row;
+    if (!spread_grid_row(a, row))
         return;
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
@@ -1080,8 +1150,8 @@ constexpr int kTermsPerThread = 8;
 
 __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(SamplerArgs a)
 {
-    const uint32_t row = blockIdx.y;
-    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+    uint32_t row;
+    if (!spread_grid_row(a, row))
         return;
     __shared__ uint64_t exp2_table[32]; // a copy in LDS: the lookups of a wave are 64 different addresses
     if (threadIdx.x < 32)
@@ -1144,9 +1214,9 @@ __global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kern
 {
     static_assert(kChunkStepPerThread * kChunkStepThreads == kReplayChunk && kChunkStepPerThread % 4 == 0, "float4 loads over a whole chunk");
     static_assert(kReplayChunk % (kTermsThreads * kTermsPerThread) == 0, "a chunk is a whole number of the terms kernel's blocks");
-    const uint32_t row = blockIdx.y;
     const uint32_t chunk = blockIdx.x;
-    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+    uint32_t row;
+    if (!spread_grid_row(a, row))
         return;
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
