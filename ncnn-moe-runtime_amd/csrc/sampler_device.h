@@ -345,6 +345,25 @@ __device__ __forceinline__ uint32_t dpp_source(uint32_t value)
     return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(value), CONTROL, ROW_MASK, 0xf, false));
 }
 
+// The fp32 sums behind each of 64 non-negative terms, one term per lane, added in lane order as a
+// sequential loop adds them: lane l returns ((t0 + t1) + ...) + tl.  Every lane adds the sum its lower
+// neighbour holds (wave_shr:1) to its own term, 63 times over; after turn k the lanes up to k hold their
+// final value, since lane l's depends on lane l - 1's alone.  63 dependent additions and no branch: a
+// loop that broadcasts one term per turn and tests a stop condition costs several times that, in every
+// wave of the workgroup at once.
+__device__ __forceinline__ float wave_sequential_sums(float term)
+{
+    float sums = term;
+#pragma unroll
+    for (int turn = 1; turn < kWaveSize; ++turn)
+    {
+        // lane 0 has no lower neighbour and reads 0: 0 + t0 = t0 (the terms are not negative zero)
+        const float below = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sums), 0x138, 0xf, 0xf, true));
+        sums = below + term;
+    }
+    return sums;
+}
+
 // Reduction over each row of 16 lanes (every lane receives its row's result), by four DPP exchanges:
 // inside pairs, quads, half rows, rows.
 template <typename Op>

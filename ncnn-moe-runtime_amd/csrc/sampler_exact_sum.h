@@ -35,11 +35,20 @@ constexpr int kHeadSlots = (kSequentialHead + kWaveSize - 1) / kWaveSize;
 constexpr int kSequentialHeadOfRuns = 16; // ... of a row stored as runs
 constexpr uint32_t kStepCap = 1u << 28; // sums past the binade are only compared against 2^24
 
-__device__ __forceinline__ ParityStep compose_steps(const ParityStep& first, const ParityStep& second)
+// `odd` where the lowest bit of `parity_of` is set, else `even`.  (Written on the values: a choice between
+// the two members of a ParityStep that the compiler sees as two loads becomes one load at a computed
+// address, which moves the struct from registers into scratch memory, a trip to memory per use.)
+__device__ __forceinline__ uint32_t pick_by_parity(uint32_t parity_of, uint32_t even, uint32_t odd)
+{
+    const uint32_t mask = 0u - (parity_of & 1u);
+    return even ^ ((even ^ odd) & mask);
+}
+
+__device__ __forceinline__ ParityStep compose_steps(const ParityStep first, const ParityStep second)
 {
     ParityStep r;
-    r.even = first.even + ((first.even & 1u) ? second.odd : second.even);
-    r.odd = first.odd + ((first.odd & 1u) ? second.even : second.odd);
+    r.even = first.even + pick_by_parity(first.even, second.even, second.odd);
+    r.odd = first.odd + pick_by_parity(first.odd, second.odd, second.even);
     r.even = min(r.even, kStepCap);
     r.odd = min(r.odd, kStepCap);
     return r;
@@ -48,17 +57,17 @@ __device__ __forceinline__ ParityStep compose_steps(const ParityStep& first, con
 // The mantissa increment of `count` successive additions of one term (step `s`) to a mantissa of the
 // given parity.  An even step keeps the parity, so the same step repeats; an odd step flips it, and
 // the flipped parity either stays (even step there) or flips back (the two steps alternate).
-__device__ __forceinline__ uint32_t repeated_step(bool odd, const ParityStep& s, uint32_t count)
+__device__ __forceinline__ uint32_t repeated_step(bool odd, const ParityStep s, uint32_t count)
 {
     if (count == 0u)
         return 0u;
-    const uint64_t first = odd ? s.odd : s.even;
+    const uint64_t first = pick_by_parity(odd ? 1u : 0u, s.even, s.odd);
     uint64_t total;
     if ((first & 1u) == 0u)
         total = first * count;
     else
     {
-        const uint64_t flipped = odd ? s.even : s.odd;
+        const uint64_t flipped = pick_by_parity(odd ? 1u : 0u, s.odd, s.even);
         if ((flipped & 1u) == 0u)
             total = first + flipped * (count - 1u);
         else
@@ -67,7 +76,7 @@ __device__ __forceinline__ uint32_t repeated_step(bool odd, const ParityStep& s,
     return total > kStepCap ? kStepCap : static_cast<uint32_t>(total);
 }
 
-__device__ __forceinline__ ParityStep repeat_steps(const ParityStep& s, uint32_t count)
+__device__ __forceinline__ ParityStep repeat_steps(const ParityStep s, uint32_t count)
 {
     // The two steps differ only for a term that ends exactly half an ulp above a multiple of it; when no lane
     // of the wave holds such a term, every addition moves the mantissa by the same step.
@@ -100,9 +109,9 @@ __device__ __forceinline__ ParityStep wave_scan_steps(ParityStep v)
     return v;
 }
 
-__device__ __forceinline__ uint32_t apply_step(uint32_t mantissa, const ParityStep& step)
+__device__ __forceinline__ uint32_t apply_step(uint32_t mantissa, const ParityStep step)
 {
-    return mantissa + ((mantissa & 1u) ? step.odd : step.even);
+    return mantissa + pick_by_parity(mantissa, step.even, step.odd);
 }
 
 // First index in [0, count) at which a predicate that holds on a prefix stops holding; the wave probes
@@ -299,10 +308,18 @@ struct RoundEvent
     float term;
 };
 
-template <int WAVES, bool CHECK_ABSORBED, class FindEvent>
-__device__ __forceinline__ RoundOutcome finish_round(
-    const ParityStep& thread_total, int exponent, uint32_t mantissa, uint32_t limit, FindEvent find_event,
-    ReplayScratch& scratch, uint32_t slot, int tid, float& sum, uint32_t& event_key)
+// The first half of a round: the mantissa in front of the calling thread's terms, and whether the round's
+// first event lies among them.
+struct RoundFront
+{
+    uint32_t current;
+    bool have_event;
+    bool absorbed; // (CHECK_ABSORBED) the round is abandoned; the caller returns at once
+};
+
+template <int WAVES, bool CHECK_ABSORBED>
+__device__ __forceinline__ RoundFront begin_round(
+    const ParityStep& thread_total, uint32_t mantissa, uint32_t limit, ReplayScratch& scratch, uint32_t slot, int tid)
 {
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
@@ -326,11 +343,10 @@ __device__ __forceinline__ RoundOutcome finish_round(
         if (scratch.absorbed[slot])
         {
             lds_barrier(); // every thread has read the flag before a later call writes it
-            return kRoundAbsorbed;
+            return RoundFront{0u, false, true};
         }
     }
-    RoundEvent found{0u, 0u, 0.0f};
-    bool reported = false;
+    RoundFront front{0u, false, false};
     if (summing)
     {
         // every wave's total is read at once (independent LDS loads); the composition stays in registers
@@ -346,18 +362,23 @@ __device__ __forceinline__ RoundOutcome finish_round(
             before = ParityStep{w < wave ? with.even : before.even, w < wave ? with.odd : before.odd};
         }
         before = compose_steps(before, exclusive);
-        const uint32_t current = apply_step(mantissa, before);
-        const uint32_t behind = apply_step(current, thread_total);
+        front.current = apply_step(mantissa, before);
+        const uint32_t behind = apply_step(front.current, thread_total);
         // The mantissa never decreases: the first event lies in the thread whose range takes it to the limit.
         // (A round that begins at the limit - a stop bound of zero - has its event at its first term.)
-        const bool have_event = behind >= limit && (current < limit || mantissa >= limit);
-        if (have_event)
-            reported = find_event(current, found);
-        if (reported)
-            atomicMin(&scratch.first_event[slot], found.key);
+        front.have_event = behind >= limit && (front.current < limit || mantissa >= limit);
         if (tid == WAVES * kWaveSize - 1)
             scratch.final_mantissa[slot] = behind;
     }
+    return front;
+}
+
+// The second half: `reported` threads have found an event in their range (`found`); the first of them wins.
+__device__ __forceinline__ RoundOutcome end_round(
+    bool reported, const RoundEvent& found, int exponent, ReplayScratch& scratch, uint32_t slot, float& sum, uint32_t& event_key)
+{
+    if (reported)
+        atomicMin(&scratch.first_event[slot], found.key);
     lds_barrier();
     const uint32_t event = scratch.first_event[slot];
     if (event == 0xffffffffu)
@@ -374,6 +395,21 @@ __device__ __forceinline__ RoundOutcome finish_round(
     sum = scratch.event_sum[slot];
     event_key = event;
     return kRoundEvent;
+}
+
+template <int WAVES, bool CHECK_ABSORBED, class FindEvent>
+__device__ __forceinline__ RoundOutcome finish_round(
+    const ParityStep& thread_total, int exponent, uint32_t mantissa, uint32_t limit, FindEvent find_event,
+    ReplayScratch& scratch, uint32_t slot, int tid, float& sum, uint32_t& event_key)
+{
+    const RoundFront front = begin_round<WAVES, CHECK_ABSORBED>(thread_total, mantissa, limit, scratch, slot, tid);
+    if (CHECK_ABSORBED && front.absorbed)
+        return kRoundAbsorbed;
+    RoundEvent found{0u, 0u, 0.0f};
+    bool reported = false;
+    if (front.have_event)
+        reported = find_event(front.current, found);
+    return end_round(reported, found, exponent, scratch, slot, sum, event_key);
 }
 
 // The running fp32 sum of the non-negative terms term(0) ... term(count - 1), starting from 0, exactly as
@@ -428,35 +464,28 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
         own_chunk_steps = chunk_steps[lane];
     if (NON_INCREASING && count > head)
         fetch(0);
-    // The first kSequentialHead terms are added one by one, as the CPU does (every thread runs the same
-    // loop on wave-uniform values): the sum climbs through most of its binades here, each of which
-    // would cost the scan below a round, and a stop condition usually holds this early.
+    // The first kSequentialHead terms are added in order, as the CPU does, a term per lane (every wave does the
+    // same): the sum climbs through most of its binades here, each of which would cost the scan below a
+    // round, and a stop condition usually holds this early.
     {
-        float head_terms[kHeadSlots];
-#pragma unroll
-        for (int slot = 0; slot < kHeadSlots; ++slot)
-        {
-            const uint32_t i = static_cast<uint32_t>(slot * kWaveSize + lane);
-            head_terms[slot] = i < head ? term_at(i) : 0.0f;
-        }
+        static_assert(kHeadSlots == 1, "the head is one term per lane");
+        const float own = static_cast<uint32_t>(lane) < head ? term_at(static_cast<uint32_t>(lane)) : 0.0f;
         if (CHECK_FIRST)
         {
-            const float first_term = read_lane(head_terms[0], 0);
+            const float first_term = read_lane(own, 0);
             if (!is_finite_f32(first_term))
                 return RunningSum{first_term, 0u, false};
         }
-#pragma unroll
-        for (int slot = 0; slot < kHeadSlots; ++slot)
+        const float sums = wave_sequential_sums(own); // (lanes behind the head add zero: they hold the head's sum)
+        const bool stops = static_cast<uint32_t>(lane) < head &&
+            ((mode == kStopAtOrAbove && sums >= bound) || (mode == kStopAbove && sums > bound));
+        const uint64_t stopping = __builtin_amdgcn_ballot_w64(stops);
+        if (stopping != 0ull)
         {
-            const uint32_t slot_first = static_cast<uint32_t>(slot * kWaveSize);
-            const uint32_t slot_count = head > slot_first ? min(head - slot_first, static_cast<uint32_t>(kWaveSize)) : 0u;
-            for (uint32_t l = 0; l < slot_count; ++l)
-            {
-                sum += read_lane(head_terms[slot], static_cast<int>(l));
-                if ((mode == kStopAtOrAbove && sum >= bound) || (mode == kStopAbove && sum > bound))
-                    return RunningSum{sum, slot_first + l, true};
-            }
+            const int first = __builtin_ctzll(stopping);
+            return RunningSum{read_lane(sums, first), static_cast<uint32_t>(first), true};
         }
+        sum = read_lane(sums, kWaveSize - 1);
         if (head >= count)
             return RunningSum{sum, 0u, false};
     }
@@ -530,50 +559,50 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
                 const bool active = i >= start && i < chunk_end;
                 return ParityStep{active ? step.even : 0u, active ? step.odd : 0u};
             };
+            ParityStep steps[kReplayPerThread];
             ParityStep thread_total{0u, 0u};
-            if (summing)
-            {
 #pragma unroll
-                for (int j = 0; j < kReplayPerThread; ++j)
-                    thread_total = compose_steps(thread_total, step_at(j));
+            for (int j = 0; j < kReplayPerThread; ++j)
+            {
+                steps[j] = summing ? step_at(j) : ParityStep{0u, 0u};
+                thread_total = compose_steps(thread_total, steps[j]);
             }
             if (NON_INCREASING)
             {
                 // the largest remaining term of the row does not move the sum: nothing later can
                 if (tid == 0)
                 {
-                    const ParityStep first_step = step_at(0);
+                    const ParityStep first_step = steps[0];
                     scratch.absorbed[slot] = (start == base && base > 0 && first_step.even == 0u && first_step.odd == 0u) ? 1 : 0;
                 }
             }
-            const auto find_event = [&](uint32_t current, RoundEvent& found) -> bool {
-                // Walk this thread's terms from the mantissa in front of them.  One thread of a round does this,
-                // in few rounds: a short loop that reads the terms again, rather than sixteen unrolled copies
-                // over the registers.
-                const uint32_t first = max(thread_first, start);
-                const uint32_t last = min(thread_first + static_cast<uint32_t>(kReplayPerThread), chunk_end);
-#pragma unroll 1
-                for (uint32_t i = first; i < last; ++i)
+            const RoundFront front = begin_round<kSumWaves, NON_INCREASING>(thread_total, mantissa, limit, scratch, slot, tid);
+            if (NON_INCREASING && front.absorbed)
+                return RunningSum{sum, 0u, false};
+            // The thread whose range holds the round's first event walks its terms from the mantissa in front of
+            // them, with the steps worked out above and without a branch (every other thread waits for it).
+            RoundEvent found{0u, 0u, 0.0f};
+            bool hit = false;
+            if (front.have_event)
+            {
+                uint32_t current = front.current;
+#pragma unroll
+                for (int j = 0; j < kReplayPerThread; ++j)
                 {
-                    const float term = term_at(i);
-                    const uint32_t next = apply_step(current, step_of_term(term, exponent));
-                    if (next >= kBinadeFull)
-                    {
-                        found = RoundEvent{i << 1, current, term};
-                        return true;
-                    }
-                    if (next >= stop_at)
-                    {
-                        found = RoundEvent{(i << 1) | 1u, next, 0.0f};
-                        return true;
-                    }
+                    const uint32_t i = thread_first + static_cast<uint32_t>(j);
+                    const bool active = i >= start && i < chunk_end;
+                    const uint32_t next = apply_step(current, steps[j]); // (a term that is not active has no step)
+                    const bool leaves = next >= kBinadeFull;
+                    const bool here = active && !hit && (leaves || next >= stop_at);
+                    found.key = here ? ((i << 1) | (leaves ? 0u : 1u)) : found.key;
+                    found.mantissa = here ? (leaves ? current : next) : found.mantissa;
+                    found.term = here ? (leaves ? terms[j] : 0.0f) : found.term;
+                    hit = hit || here;
                     current = next;
                 }
-                return false;
-            };
+            }
             uint32_t event = 0;
-            const RoundOutcome outcome =
-                finish_round<kSumWaves, NON_INCREASING>(thread_total, exponent, mantissa, limit, find_event, scratch, slot, tid, sum, event);
+            const RoundOutcome outcome = end_round(hit, found, exponent, scratch, slot, sum, event);
             if (outcome == kRoundAbsorbed)
                 return RunningSum{sum, 0u, false};
             if (outcome == kRoundPlain)
