@@ -391,10 +391,10 @@ int launch_sampler(
             const uint32_t parts = (vocab + kTermsThreads * kTermsPerThread - 1) / (kTermsThreads * kTermsPerThread);
             hipLaunchKernelGGL(full_order_terms_kernel, dim3(parts, rows), dim3(kTermsThreads), 0, stream, a);
             a.terms_precomputed = 1;
-            const uint32_t whole_chunks = vocab / kReplayChunk;
-            if (whole_chunks > 0 && s->chunk_steps_enabled != 0)
+            const uint32_t chunks = (vocab + kReplayChunk - 1) / kReplayChunk;
+            if (vocab >= static_cast<uint32_t>(kReplayChunk) && s->chunk_steps_enabled != 0)
             {
-                hipLaunchKernelGGL(full_order_chunk_steps_kernel, dim3(whole_chunks, rows), dim3(kChunkStepThreads), 0, stream, a);
+                hipLaunchKernelGGL(full_order_chunk_steps_kernel, dim3(chunks, rows), dim3(kChunkStepThreads), 0, stream, a);
                 a.chunk_steps_ready = 1;
             }
         }

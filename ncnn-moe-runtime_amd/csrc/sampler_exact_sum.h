@@ -237,7 +237,8 @@ struct SortedRow
     const uint32_t* run_ends; // runs only: position behind the last element of each run (null otherwise)
     uint32_t run_count;
     const float* terms0;      // exp(logit/T - maximum) of every item (element or run), computed beforehand
-    const uint4* chunk_steps; // elements only, may be null: (exponent, even step, odd step, valid) of every whole chunk of terms0
+    const uint4* chunk_steps; // elements only, may be null: (exponent, even step, odd step, valid) of every chunk of terms0 ...
+    uint32_t chunk_steps_cover; // ... up to this element (the last chunk may be a partial one)
     float temperature;
     float maximum;
     float normalizer;
@@ -422,7 +423,7 @@ __device__ __forceinline__ RoundOutcome finish_round(
 template <bool NON_INCREASING, bool DIVIDED, bool CHECK_FIRST = false>
 __device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
     const float* terms_array, float divisor, float second_divisor, uint32_t count, int mode, float bound,
-    ReplayScratch& scratch, int tid, const uint4* chunk_steps = nullptr)
+    ReplayScratch& scratch, int tid, const uint4* chunk_steps = nullptr, uint32_t chunk_steps_cover = 0u)
 {
     const auto scaled = [divisor, second_divisor](float t) { return DIVIDED ? (t / divisor) / second_divisor : t; };
     const auto term_at = [&](uint32_t i) { return scaled(terms_array[i]); };
@@ -460,7 +461,8 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
     // steps of the first 64 whole chunks, one per lane, and the first chunk's terms - so that the loads of the
     // head below are not the first of three trips to memory, one behind the other.
     uint4 own_chunk_steps{0u, 0u, 0u, 0u};
-    if (NON_INCREASING && !DIVIDED && chunk_steps != nullptr && static_cast<uint32_t>(lane) < count / kReplayChunk)
+    if (NON_INCREASING && !DIVIDED && chunk_steps != nullptr &&
+        static_cast<uint32_t>(lane) < (chunk_steps_cover + static_cast<uint32_t>(kReplayChunk) - 1u) / kReplayChunk)
         own_chunk_steps = chunk_steps[lane];
     if (NON_INCREASING && count > head)
         fetch(0);
@@ -498,36 +500,56 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
     for (uint32_t base = 0; base < count; base += kReplayChunk)
     {
         const uint32_t chunk_end = min(count, base + static_cast<uint32_t>(kReplayChunk));
-        if (NON_INCREASING && !DIVIDED && chunk_steps != nullptr && mode == kStopNever &&
-            chunk_end == base + static_cast<uint32_t>(kReplayChunk) && head == static_cast<uint32_t>(kSequentialHead))
+        if (NON_INCREASING && !DIVIDED && chunk_steps != nullptr && mode == kStopNever && head == static_cast<uint32_t>(kSequentialHead))
         {
-            // A whole chunk whose composed step was worked out beforehand for the exponent that the sum has now:
-            // if that step leaves the mantissa inside the binade, nothing inside the chunk left it either (the
-            // mantissa never decreases), and the chunk is this one addition.
+            // Chunks whose composed step was worked out beforehand for the exponent that the sum has now: if that
+            // step leaves the mantissa inside the binade, nothing inside the chunk left it either (the mantissa
+            // never decreases), and the chunk is this one addition.  A chunk's step is usable when the sum's
+            // terms cover the chunk as far as the step does.
             const uint32_t chunk = base / kReplayChunk;
-            uint4 composed;
-            if (chunk < static_cast<uint32_t>(kWaveSize))
-            {
-                composed.x = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_chunk_steps.x), static_cast<int>(chunk)));
-                composed.y = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_chunk_steps.y), static_cast<int>(chunk)));
-                composed.z = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_chunk_steps.z), static_cast<int>(chunk)));
-                composed.w = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_chunk_steps.w), static_cast<int>(chunk)));
-            }
-            else
-                composed = chunk_steps[chunk];
             int exponent;
             uint32_t mantissa;
             decode_sum(sum, exponent, mantissa);
-            if (composed.w != 0u && composed.x == static_cast<uint32_t>(exponent))
+            if (chunk < static_cast<uint32_t>(kWaveSize))
             {
-                const uint32_t behind = apply_step(mantissa, ParityStep{composed.y, composed.z});
-                if (behind < kBinadeFull)
+                // lane c holds the step of chunk c: all the chunks from this one on that can be added so, at once
+                // (a scan over the lanes; a row's flat tail is some dozens of such chunks, one after the other)
+                const uint32_t lane_base = static_cast<uint32_t>(lane) * kReplayChunk;
+                const bool usable = static_cast<uint32_t>(lane) >= chunk && lane_base < count &&
+                    min(count, lane_base + static_cast<uint32_t>(kReplayChunk)) == min(chunk_steps_cover, lane_base + static_cast<uint32_t>(kReplayChunk)) &&
+                    own_chunk_steps.w != 0u && own_chunk_steps.x == static_cast<uint32_t>(exponent);
+                const ParityStep through = wave_scan_steps(ParityStep{usable ? own_chunk_steps.y : 0u, usable ? own_chunk_steps.z : 0u});
+                const uint32_t behind = apply_step(mantissa, through);
+                const uint64_t not_so = __builtin_amdgcn_ballot_w64(static_cast<uint32_t>(lane) >= chunk && !(usable && behind < kBinadeFull));
+                const uint64_t still = __builtin_amdgcn_ballot_w64(usable && own_chunk_steps.y == 0u && own_chunk_steps.z == 0u);
+                const uint32_t first_not_so = not_so != 0ull ? static_cast<uint32_t>(__builtin_ctzll(not_so)) : static_cast<uint32_t>(kWaveSize);
+                const uint32_t first_still = still != 0ull ? static_cast<uint32_t>(__builtin_ctzll(still)) : static_cast<uint32_t>(kWaveSize);
+                const uint32_t stop = min(first_not_so, first_still);
+                if (stop > chunk)
+                    sum = encode_sum(exponent, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(behind), static_cast<int>(stop - 1u))));
+                if (first_still < first_not_so)
+                    return RunningSum{sum, 0u, false}; // no term of that chunk moves the sum: none behind it can
+                if (stop > chunk)
                 {
-                    if (composed.y == 0u && composed.z == 0u)
-                        return RunningSum{sum, 0u, false}; // no term of the chunk moves the sum: none behind it can
-                    sum = encode_sum(exponent, behind);
+                    base = (stop - 1u) * kReplayChunk; // (the loop moves on to chunk `stop`)
                     fetched = false;
                     continue;
+                }
+            }
+            else if (chunk_end == min(chunk_steps_cover, base + static_cast<uint32_t>(kReplayChunk)))
+            {
+                const uint4 composed = chunk_steps[chunk];
+                if (composed.w != 0u && composed.x == static_cast<uint32_t>(exponent))
+                {
+                    const uint32_t behind = apply_step(mantissa, ParityStep{composed.y, composed.z});
+                    if (behind < kBinadeFull)
+                    {
+                        if (composed.y == 0u && composed.z == 0u)
+                            return RunningSum{sum, 0u, false}; // no term of the chunk moves the sum: none behind it can
+                        sum = encode_sum(exponent, behind);
+                        fetched = false;
+                        continue;
+                    }
                 }
             }
         }
@@ -623,9 +645,9 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
 template <bool NON_INCREASING, bool DIVIDED>
 __device__ __noinline__ RunningSum exact_running_sum_of_array(
     const float* terms_array, float divisor, float second_divisor, uint32_t count, int mode, float bound,
-    ReplayScratch& scratch, int tid, const uint4* chunk_steps = nullptr)
+    ReplayScratch& scratch, int tid, const uint4* chunk_steps = nullptr, uint32_t chunk_steps_cover = 0u)
 {
-    return exact_running_sum_of_array_inline<NON_INCREASING, DIVIDED>(terms_array, divisor, second_divisor, count, mode, bound, scratch, tid, chunk_steps);
+    return exact_running_sum_of_array_inline<NON_INCREASING, DIVIDED>(terms_array, divisor, second_divisor, count, mode, bound, scratch, tid, chunk_steps, chunk_steps_cover);
 }
 
 // The running sum of terms [0, count) of a sorted row.  PHASE 0 (terms that never grow) also stops
@@ -635,7 +657,7 @@ __device__ __forceinline__ RunningSum exact_running_sum(
     const SortedRow& row, uint32_t count, int mode, float bound, ReplayScratch& scratch, int tid)
 {
     if constexpr (PHASE == 0) // the normaliser: one call per kernel, inlined (a call saves and restores its registers through memory)
-        return exact_running_sum_of_array_inline<true, false, true>(row.terms0, 1.0f, 1.0f, count, mode, bound, scratch, tid, row.chunk_steps);
+        return exact_running_sum_of_array_inline<true, false, true>(row.terms0, 1.0f, 1.0f, count, mode, bound, scratch, tid, row.chunk_steps, row.chunk_steps_cover);
     else
         return exact_running_sum_of_array<false, true>(
             row.terms0, row.normalizer, PHASE == 2 ? row.renormalizer : 1.0f, count, mode, bound, scratch, tid, nullptr);
@@ -844,7 +866,7 @@ __device__ __forceinline__ void replay_sorted_window(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
     const uint32_t* keys, const uint32_t* run_ends, uint32_t run_count, uint32_t n,
     const uint32_t* sorted_indices, uint8_t flags, ReplayScratch& scratch, int tid, TokenAt token_at,
-    const float* terms0 = nullptr, const uint4* chunk_steps = nullptr)
+    const float* terms0 = nullptr, const uint4* chunk_steps = nullptr, uint32_t chunk_steps_cover = 0u)
 {
 #ifdef NCNN_MOE_TIMELINE
     const uint32_t stamp_row = a.only_pending ? 0xffffffffu : row; // the full-order rows' stamps (not the wide select's)
@@ -855,6 +877,7 @@ __device__ __forceinline__ void replay_sorted_window(
     sorted.run_count = run_count;
     sorted.terms0 = terms0;
     sorted.chunk_steps = RUNS ? nullptr : chunk_steps;
+    sorted.chunk_steps_cover = chunk_steps_cover;
     sorted.temperature = p.temperature;
     sorted.maximum = value_from_descending_key(keys[0]) / p.temperature;
     sorted.normalizer = 1.0f;

@@ -1138,7 +1138,7 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
         if (a.chunk_steps_ready != 0)
             chunk_steps = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity;
     }
-    replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0, chunk_steps);
+    replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0, chunk_steps, a.vocab);
 }
 
 // exp(logit/T - maximum) of every element of the sorted full-order rows, written over the sort's other key
@@ -1227,18 +1227,20 @@ __global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kern
     const float* terms = reinterpret_cast<const float*>(a.sort_keys[0] + row * a.sort_stride);
     uint4* const out = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity + chunk;
     const uint32_t base = chunk * kReplayChunk;
-    if (base + kReplayChunk > a.vocab)
-    {
-        if (tid == 0)
-            *out = uint4{0u, 0u, 0u, 0u}; // not a whole chunk: the replay never asks
-        return;
-    }
     // the chunk's terms are asked for first: the estimate below is a chain of loads, a reduction and a barrier
+    // (the row's last chunk may be a partial one: the terms behind the row count as zero)
     const uint32_t first = base + static_cast<uint32_t>(tid) * kChunkStepPerThread;
     float4 loaded[kChunkStepPerThread / 4];
 #pragma unroll
     for (int j = 0; j < kChunkStepPerThread / 4; ++j)
-        loaded[j] = *reinterpret_cast<const float4*>(terms + first + 4 * j);
+    {
+        const uint32_t at = first + 4u * static_cast<uint32_t>(j);
+        if (at + 4u <= a.vocab)
+            loaded[j] = *reinterpret_cast<const float4*>(terms + at);
+        else
+            loaded[j] = float4{at < a.vocab ? terms[at] : 0.0f, at + 1u < a.vocab ? terms[at + 1u] : 0.0f,
+                               at + 2u < a.vocab ? terms[at + 2u] : 0.0f, 0.0f};
+    }
     // the sum in front of the chunk: the blocks of the terms kernel before it, or (first chunk) the 64 terms
     // that every running sum adds one by one
     double before = 0.0;
