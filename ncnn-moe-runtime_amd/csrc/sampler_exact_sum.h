@@ -30,7 +30,7 @@ struct ParityStep
 };
 
 constexpr uint32_t kBinadeFull = 1u << 24;
-constexpr int kSequentialHead = 64; // terms a running sum adds one by one before it scans
+constexpr int kSequentialHead = 256; // terms a running sum adds one by one before it scans
 constexpr int kHeadSlots = (kSequentialHead + kWaveSize - 1) / kWaveSize;
 constexpr int kSequentialHeadOfRuns = 16; // ... of a row stored as runs
 constexpr uint32_t kStepCap = 1u << 28; // sums past the binade are only compared against 2^24
@@ -466,28 +466,42 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
         own_chunk_steps = chunk_steps[lane];
     if (NON_INCREASING && count > head)
         fetch(0);
-    // The first kSequentialHead terms are added in order, as the CPU does, a term per lane (every wave does the
-    // same): the sum climbs through most of its binades here, each of which would cost the scan below a
-    // round, and a stop condition usually holds this early.
+    // The first kSequentialHead terms are added in order, as the CPU does, 64 at a time with a term per lane
+    // (every wave does the same): the sum climbs through most of its binades here, each of which would cost
+    // the scan below a round, and a stop condition usually holds this early.
     {
-        static_assert(kHeadSlots == 1, "the head is one term per lane");
-        const float own = static_cast<uint32_t>(lane) < head ? term_at(static_cast<uint32_t>(lane)) : 0.0f;
+        float head_terms[kHeadSlots];
+#pragma unroll
+        for (int slot = 0; slot < kHeadSlots; ++slot)
+        {
+            const uint32_t i = static_cast<uint32_t>(slot * kWaveSize + lane);
+            head_terms[slot] = i < head ? term_at(i) : 0.0f;
+        }
         if (CHECK_FIRST)
         {
-            const float first_term = read_lane(own, 0);
+            const float first_term = read_lane(head_terms[0], 0);
             if (!is_finite_f32(first_term))
                 return RunningSum{first_term, 0u, false};
         }
-        const float sums = wave_sequential_sums(own); // (lanes behind the head add zero: they hold the head's sum)
-        const bool stops = static_cast<uint32_t>(lane) < head &&
-            ((mode == kStopAtOrAbove && sums >= bound) || (mode == kStopAbove && sums > bound));
-        const uint64_t stopping = __builtin_amdgcn_ballot_w64(stops);
-        if (stopping != 0ull)
+#pragma unroll
+        for (int slot = 0; slot < kHeadSlots; ++slot)
         {
-            const int first = __builtin_ctzll(stopping);
-            return RunningSum{read_lane(sums, first), static_cast<uint32_t>(first), true};
+            const uint32_t slot_first = static_cast<uint32_t>(slot * kWaveSize);
+            if (slot > 0 && slot_first >= head)
+                break;
+            // (the sum so far goes in front of the slot's first term: one addition, the one the loop would make)
+            const float own = (slot > 0 && lane == 0) ? sum + head_terms[slot] : head_terms[slot];
+            const float sums = wave_sequential_sums(own); // (lanes behind the head add zero: they hold the head's sum)
+            const bool stops = slot_first + static_cast<uint32_t>(lane) < head &&
+                ((mode == kStopAtOrAbove && sums >= bound) || (mode == kStopAbove && sums > bound));
+            const uint64_t stopping = __builtin_amdgcn_ballot_w64(stops);
+            if (stopping != 0ull)
+            {
+                const int first = __builtin_ctzll(stopping);
+                return RunningSum{read_lane(sums, first), slot_first + static_cast<uint32_t>(first), true};
+            }
+            sum = read_lane(sums, kWaveSize - 1);
         }
-        sum = read_lane(sums, kWaveSize - 1);
         if (head >= count)
             return RunningSum{sum, 0u, false};
     }

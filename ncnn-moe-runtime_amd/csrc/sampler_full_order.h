@@ -1241,11 +1241,14 @@ __global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kern
             loaded[j] = float4{at < a.vocab ? terms[at] : 0.0f, at + 1u < a.vocab ? terms[at + 1u] : 0.0f,
                                at + 2u < a.vocab ? terms[at + 2u] : 0.0f, 0.0f};
     }
-    // the sum in front of the chunk: the blocks of the terms kernel before it, or (first chunk) the 64 terms
-    // that every running sum adds one by one
+    // the sum in front of the chunk: the blocks of the terms kernel before it, or (first chunk) the head of
+    // terms that every running sum adds one by one
     double before = 0.0;
     if (chunk == 0)
-        before = tid < kSequentialHead ? static_cast<double>(terms[tid]) : 0.0;
+    {
+        for (int i = tid; i < kSequentialHead; i += kChunkStepThreads)
+            before += static_cast<double>(terms[i]);
+    }
     else
     {
         const uint32_t blocks = chunk * (kReplayChunk / (kTermsThreads * kTermsPerThread));
