@@ -488,13 +488,9 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         // full-order row marked already (the full-order kernels may be serving it at this moment on another
         // stream); a wide select that runs beside the first select leaves the marking of every row to that
         // one; and the first select leaves the wide select's rows alone when told that one runs beside it.
-        bool not_mine = a.only_pending == 2 || (a.only_pending == 1 && mode == kModeGeneral);
-        if (!WIDE && a.leave_wide_rows != 0 && mode == kModeGeneral)
-        {
-            uint32_t wide_k = 0;
-            int wide_status = NCNN_MOE_ROW_OK;
-            not_mine = resolve_row_mode(p, a.vocab, static_cast<uint32_t>(kSelectTopK), a.force_general, wide_k, wide_status) != kModeGeneral;
-        }
+        const bool not_mine = a.only_pending == 2 || (a.only_pending == 1 && mode == kModeGeneral) ||
+            (!WIDE && a.leave_wide_rows != 0 && mode == kModeGeneral && a.force_general == 0 &&
+             effective_k <= static_cast<uint32_t>(kSelectTopK));
         if (segment == 0 && tid == 0 && !not_mine)
         {
             if (mode == kModeInvalid)

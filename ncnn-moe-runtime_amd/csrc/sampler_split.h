@@ -149,13 +149,8 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     if (mode == kModeInvalid || mode == kModeGeneral)
     {
         // (a row with a window of 65 to 1024 is left alone when a wide select runs beside this kernel)
-        bool not_mine = false;
-        if (a.leave_wide_rows != 0 && mode == kModeGeneral)
-        {
-            uint32_t wide_k = 0;
-            int wide_status = NCNN_MOE_ROW_OK;
-            not_mine = resolve_row_mode(p, a.vocab, static_cast<uint32_t>(kSelectTopK), a.force_general, wide_k, wide_status) != kModeGeneral;
-        }
+        const bool not_mine = a.leave_wide_rows != 0 && mode == kModeGeneral && a.force_general == 0 &&
+            effective_k <= static_cast<uint32_t>(kSelectTopK);
         if (segment == 0 && tid == 0 && !not_mine)
         {
             if (mode == kModeInvalid)
