@@ -32,7 +32,7 @@ struct ParityStep
 constexpr uint32_t kBinadeFull = 1u << 24;
 constexpr int kSequentialHead = 256; // terms a running sum adds one by one before it scans
 constexpr int kHeadSlots = (kSequentialHead + kWaveSize - 1) / kWaveSize;
-constexpr int kSequentialHeadOfRuns = 16; // ... of a row stored as runs
+constexpr int kSequentialHeadOfRuns = 64; // ... of a row stored as runs
 constexpr uint32_t kStepCap = 1u << 28; // sums past the binade are only compared against 2^24
 
 // `odd` where the lowest bit of `parity_of` is set, else `even`.  (Written on the values: a choice between
@@ -699,25 +699,37 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
     const uint32_t runs = run_of_element_uniform(row, count - 1u) + 1u;
     uint32_t start = 0; // elements before this one have been added
 
-    // The first kSequentialHeadOfRuns elements are added one by one, as the CPU does (every thread runs the
-    // same loop on wave-uniform values): the sum climbs through most of its binades here, each of
-    // which would cost the scan below a round, and a stop condition usually holds this early.
+    // The first kSequentialHeadOfRuns elements are added in order, as the CPU does, an element per lane (every
+    // wave does the same): the sum climbs through most of its binades here, each of which would cost the
+    // scan below a round, and a stop condition usually holds this early.
     {
+        static_assert(kSequentialHeadOfRuns == kWaveSize, "the head is one element per lane");
         const uint32_t head_runs = min(runs, static_cast<uint32_t>(kWaveSize));
         const float head_term = static_cast<uint32_t>(lane) < head_runs ? term_of_run(static_cast<uint32_t>(lane)) : 0.0f;
-        const uint32_t head_end = static_cast<uint32_t>(lane) < head_runs ? min(row.run_ends[lane], count) : 0u;
+        // (a lane without a run: an end that no element lies behind)
+        const uint32_t head_end = static_cast<uint32_t>(lane) < head_runs ? min(row.run_ends[lane], count) : 0xffffffffu;
         const uint32_t head_limit = min(count, static_cast<uint32_t>(kSequentialHeadOfRuns));
-        for (uint32_t run = 0; run < head_runs && start < head_limit; ++run)
+        // the run of element `lane`: the number of runs that end at or in front of it (the ends ascend with the lanes)
+        uint32_t run = 0;
+#pragma unroll
+        for (uint32_t step = kWaveSize / 2; step > 0u; step >>= 1)
         {
-            const float term = read_lane(head_term, static_cast<int>(run));
-            const uint32_t run_end = min(static_cast<uint32_t>(read_lane(static_cast<int>(head_end), static_cast<int>(run))), head_limit);
-            for (; start < run_end; ++start)
-            {
-                sum += term;
-                if ((mode == kStopAtOrAbove && sum >= bound) || (mode == kStopAbove && sum > bound))
-                    return RunningSum{sum, start, true};
-            }
+            const uint32_t end_there = static_cast<uint32_t>(__shfl(static_cast<int>(head_end), static_cast<int>(run + step - 1u), kWaveSize));
+            run += end_there <= static_cast<uint32_t>(lane) ? step : 0u;
         }
+        const float term_there = __shfl(head_term, static_cast<int>(run), kWaveSize);
+        const float own = static_cast<uint32_t>(lane) < head_limit ? term_there : 0.0f;
+        const float sums = wave_sequential_sums(own); // (lanes behind the head add zero: they hold the head's sum)
+        const bool stops = static_cast<uint32_t>(lane) < head_limit &&
+            ((mode == kStopAtOrAbove && sums >= bound) || (mode == kStopAbove && sums > bound));
+        const uint64_t stopping = __builtin_amdgcn_ballot_w64(stops);
+        if (stopping != 0ull)
+        {
+            const int first = __builtin_ctzll(stopping);
+            return RunningSum{read_lane(sums, first), static_cast<uint32_t>(first), true};
+        }
+        sum = read_lane(sums, kWaveSize - 1);
+        start = head_limit;
         if (start >= count)
             return RunningSum{sum, 0u, false};
     }
