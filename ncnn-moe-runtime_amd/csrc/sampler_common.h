@@ -61,9 +61,6 @@ struct SamplerArgs
     uint32_t term_sum_parts;
     uint32_t chunk_capacity;
     uint32_t chunk_steps_ready;
-    // the rows that the full-order kernels serve, listed by full_order_row_list_kernel: [0] their number, then
-    // the rows in ascending order.  Kernels over a (parts, rows) grid look their row up here (null: in row_state).
-    const uint32_t* row_list;
 
     // optional filtered-distribution output: row r writes at most distribution_cap (id, probability)
     // entries from r * distribution_cap on, and its full kept length to distribution_count[r]
@@ -71,6 +68,11 @@ struct SamplerArgs
     float* distribution_probabilities;
     uint32_t distribution_cap;
     uint32_t* distribution_count;
+
+    // the rows that the full-order kernels serve, listed by full_order_row_list_kernel: [0] their number, then
+    // the rows in ascending order.  Kernels over a (parts, rows) grid look their row up here (null: in row_state).
+    // (The struct's last member: what the select kernels read keeps its place among the kernel's arguments.)
+    const uint32_t* row_list;
 };
 
 __device__ __forceinline__ uint8_t stop_flag(const SamplerArgs& a, const ncnn_moe_sample_params& p, int32_t token)
