@@ -24,6 +24,7 @@ struct SelectShared
     static constexpr int kListCap = WIDE ? kWideListCap : kNarrowListCap;
     static constexpr int kSortedCap = WIDE ? kSelectTopK : 1;
     static_assert(kSelectTopK <= 2 * kScanThreads, "the ordered window is copied two entries per thread");
+    static_assert(kSumThreads <= kScanThreads, "the exact running sums need kSumThreads threads of the workgroup that calls them");
     BoundScratch bound;
     alignas(16) uint32_t list_keys[kListCap]; // (the wide finish sorts the list as one array of 64-bit pairs over these two)
     int32_t list_indices[kListCap];

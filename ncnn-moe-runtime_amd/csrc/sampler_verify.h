@@ -10,6 +10,7 @@
 namespace ncnn_moe_hip {
 
 constexpr int kVerifyThreads = 512;
+static_assert(kSumThreads <= kVerifyThreads, "the exact running sums need kSumThreads threads of the workgroup that calls them");
 constexpr int kVerifyCap = kSelectTopK; // candidates of a row's filtered distribution the step can use
 constexpr int kVerifySlots = kVerifyCap / kWaveSize;
 
