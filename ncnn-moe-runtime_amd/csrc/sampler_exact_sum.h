@@ -574,7 +574,14 @@ __device__ __forceinline__ RunningSum exact_running_sum_of_array_inline(
         float terms[kReplayPerThread];
 #pragma unroll
         for (int j = 0; j < kReplayPerThread; ++j)
-            terms[j] = scaled(upcoming[j]);
+            terms[j] = DIVIDED ? upcoming[j] / divisor : upcoming[j];
+        // (a second divisor of one, the Top-P walk's, leaves the quotients as they are: eight divisions not made)
+        if (DIVIDED && second_divisor != 1.0f)
+        {
+#pragma unroll
+            for (int j = 0; j < kReplayPerThread; ++j)
+                terms[j] = terms[j] / second_divisor;
+        }
         if (base + kReplayChunk < count)
             fetch(base + kReplayChunk);
         uint32_t start = max(base, head);
