@@ -525,6 +525,28 @@ def test_full_order_rows_sorted_by_several_workgroups(batch_sampler, dtype, voca
         assert np.array_equal(probabilities[:count].view(np.uint32), np.asarray(oracle_probabilities, dtype=np.float32).view(np.uint32))
 
 
+def test_full_order_rows_listed_in_a_batch_of_many_rows():
+    """The kernels of the spread sort find their rows in a list that one workgroup writes 1,024 rows at a time:
+    a batch of 1,300 rows, greedy but for a few dozen full-order rows at both ends of the batch, around row
+    1,024 and scattered in between (fp32 rows of four tiles each)."""
+    _announce("row list of the full-order kernels, 1300 rows")
+    rng = np.random.default_rng(1300)
+    rows, vocab = 1300, 32768
+    logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    params = hip_sampler.make_params(rows, 0.0, 0, 1.0, 0.0)
+    full_order = np.unique(np.concatenate([[0, 1, 63, 64, 1022, 1023, 1024, 1025, 1298, 1299], rng.choice(rows, size=30, replace=False)]))
+    params["temperature"][full_order] = rng.uniform(0.5, 1.3, size=full_order.size).astype(np.float32)
+    params["top_p"][full_order] = rng.uniform(0.6, 1.0, size=full_order.size).astype(np.float32)
+    uniforms = rng.random(rows, dtype=np.float32)
+    with hip_sampler.HipSampler(rows, vocab) as sampler:
+        sampler.upload_logits(logits)
+        gpu = sampler.sample(params, uniforms, None)
+    cpu = parity_util.run_oracle(logits, params, uniforms)
+    parity_util.assert_results_match(gpu, cpu, "f32", "row list, 1300 rows")
+    served_in_full_order = (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH) != 0
+    assert np.array_equal(np.nonzero(served_in_full_order)[0], full_order)
+
+
 def test_bf16_counters_that_overflow_sixteen_bits(batch_sampler):
     """bf16 full-order rows are counted in 16-bit counters, two to a word; a row in which one value occurs
     65536 times or more is counted again in 32-bit counters.  Rows just below and at the limit, in the lower
