@@ -652,6 +652,32 @@ __device__ __forceinline__ void count_bf16_keys(
     {
         uint4 next[4];
         load_batch(first + kBatch < aligned_end ? first + kBatch : first, next);
+        // A batch that lies wholly inside the row (all but the first, if the row does not start on a 16-byte
+        // boundary, and the last) is counted without a test per logit and without a branch: the kernel is bound
+        // by the instructions it issues per logit, not by HBM.
+        if (PACKED && first >= misalignment && first + kBatch <= aligned_end)
+        {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                const uint32_t words[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
+#pragma unroll
+                for (int c = 0; c < 8; ++c)
+                {
+                    // descending_key of the logit's fp32 value, upper half, but for NaN and -0: those are counted
+                    // under the keys that the plain mapping gives them (which no other value has) and moved to
+                    // their places by fold_special_bf16_counts
+                    const uint32_t bits = (c & 1) ? (words[c >> 1] & 0xffff0000u) : (words[c >> 1] << 16);
+                    const uint32_t sign = static_cast<uint32_t>(static_cast<int32_t>(bits) >> 31);
+                    const uint32_t key16 = (bits ^ (~sign & 0x7fffffffu)) >> 16;
+                    atomicAdd(&bins[key16 >> 1], 1u << ((key16 & 1u) << 4));
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                raw[k] = next[k];
+            continue;
+        }
 #pragma unroll
         for (int k = 0; k < 4; ++k)
         {
@@ -677,6 +703,50 @@ __device__ __forceinline__ void count_bf16_keys(
         for (int k = 0; k < 4; ++k)
             raw[k] = next[k];
     }
+}
+
+// count_bf16_keys<true> counts the logits of whole batches under descending_key's plain mapping (the bits of a
+// negative value; the complement of a positive value's lower 15 bits), which gives NaN and -0 keys of their
+// own: 0x0000-0x007e (positive NaN, in front of +inf at 0x007f), 0xff81-0xffff (negative NaN, behind -inf at
+// 0xff80) and 0x8000 (-0, next to +0 at 0x7fff).  The first wave moves those counts to where descending_key
+// puts the values: all NaN at 0xffff, -0 with +0.  Returns false if a sum does not fit its 16-bit counter (the
+// caller then counts the row again in 32-bit counters, with descending_key itself).  Call between barriers.
+__device__ __forceinline__ bool fold_special_bf16_counts(uint32_t* bins, int tid)
+{
+    bool fits = true;
+    if (tid < kWaveSize)
+    {
+        const uint32_t lane = static_cast<uint32_t>(tid);
+        // positive NaN: words 0 .. 63 but for the upper half of word 63 (+inf)
+        const uint32_t front = bins[lane];
+        const uint32_t front_nan = (front & 0xffffu) + (lane < 63u ? front >> 16 : 0u);
+        bins[lane] = lane < 63u ? 0u : front & 0xffff0000u;
+        // negative NaN: words 0x7fc0 .. 0x7fff but for the lower half of word 0x7fc0 (-inf); the upper half of
+        // word 0x7fff is where they all go
+        const uint32_t back = bins[0x7fc0u + lane];
+        const uint32_t back_nan = (back >> 16) + (lane > 0u ? back & 0xffffu : 0u);
+        const uint32_t all_nan = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(front_nan + back_nan)), kWaveSize - 1));
+        fits = all_nan <= 0xffffu;
+        if (fits)
+            bins[0x7fc0u + lane] = lane == 0u ? back & 0xffffu : (lane == 63u ? all_nan << 16 : 0u);
+        else
+            bins[lane] = front; // (nothing is moved: the counters are abandoned)
+        if (lane == 0u)
+        {
+            // -0 (key 0x8000: lower half of word 0x4000) joins +0 (key 0x7fff: upper half of word 0x3fff)
+            const uint32_t negative_zero = bins[0x4000u] & 0xffffu;
+            const uint32_t positive_zero = bins[0x3fffu] >> 16;
+            if (negative_zero + positive_zero <= 0xffffu)
+            {
+                bins[0x4000u] &= 0xffff0000u;
+                bins[0x3fffu] = (bins[0x3fffu] & 0xffffu) | ((negative_zero + positive_zero) << 16);
+            }
+            else
+                fits = false;
+        }
+        fits = __builtin_amdgcn_ballot_w64(!fits) == 0ull;
+    }
+    return fits;
 }
 
 struct CountScratch
@@ -808,9 +878,17 @@ __global__ __launch_bounds__(kSortThreads) void bf16_counting_sort_kernel(Sample
     clear_bins();
     count_bf16_keys<true>(aligned_logits, misalignment, aligned_end, 0u, bins, tid);
     __syncthreads();
+    __shared__ uint32_t specials_fit;
+    {
+        const bool fits = fold_special_bf16_counts(bins, tid);
+        if (tid == 0)
+            specials_fit = fits ? 1u : 0u;
+    }
+    __syncthreads();
     NCNN_MOE_STAMP(blockIdx.x, 14, 1);
+    // (counts of NaN or of zeros that do not fit 16 bits: a number of logits that no sum of counters reaches)
     const bool packed_sound =
-        write_runs_of_counts<true>(bins, n, 0u, written, runs_written, run_keys, run_ends, scratch, tid);
+        write_runs_of_counts<true>(bins, specials_fit != 0u ? n : 0xffffffffu, 0u, written, runs_written, run_keys, run_ends, scratch, tid);
     NCNN_MOE_STAMP(blockIdx.x, 14, 2);
     if (!packed_sound)
     {

@@ -550,7 +550,8 @@ def test_full_order_rows_listed_in_a_batch_of_many_rows():
 def test_bf16_counters_that_overflow_sixteen_bits(batch_sampler):
     """bf16 full-order rows are counted in 16-bit counters, two to a word; a row in which one value occurs
     65536 times or more is counted again in 32-bit counters.  Rows just below and at the limit, in the lower
-    and in the upper half of a word (neighbouring bf16 values), in both, and a constant row."""
+    and in the upper half of a word (neighbouring bf16 values), in both, a constant row, and rows whose NaN
+    or zeros add up to the limit."""
     rng = np.random.default_rng(77)
     vocab = 109999
     rows = 12
@@ -564,6 +565,14 @@ def test_bf16_counters_that_overflow_sixteen_bits(batch_sampler):
     logits[9, :] = -np.inf
     logits[9, :70000] = 0.25
     bits = workloads.float32_to_bf16_bits(logits)
+    # NaN of many payloads and both signs, and zeros of both signs, are counted under keys of their own first and
+    # then added up under one key each: sums that just fit a 16-bit counter and sums that do not
+    nan_payloads = np.concatenate([np.arange(0x7F81, 0x8000), np.arange(0xFF81, 0x10000)]).astype(np.uint16)
+    for row, (nans, positive_zeros, negative_zeros) in zip((10, 11), ((65535, 30000, 35535), (65536, 30000, 35536))):
+        order = rng.permutation(vocab)
+        bits[row, order[:nans]] = nan_payloads[rng.integers(0, nan_payloads.size, size=nans)]
+        bits[row, order[nans:nans + positive_zeros]] = 0x0000
+        bits[row, order[nans + positive_zeros:nans + positive_zeros + negative_zeros]] = 0x8000
     params = hip_sampler.make_params(rows, 1.0, 0, 0.95, 0.0)
     params["temperature"] = rng.uniform(0.5, 1.4, size=rows).astype(np.float32)
     params["top_p"][::2] = 1.0
