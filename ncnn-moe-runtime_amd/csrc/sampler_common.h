@@ -148,20 +148,12 @@ __device__ __forceinline__ void finish_row_wave(
     if (lane < n)
         term = expf_libm(value / temperature - maximum, exp2_table);
 
-    // The three walks below are the CPU's sequential fp32 sums.  They run in trips of four candidates
-    // without a data-dependent exit: a lane past the end (or a filtered candidate) adds +0.0, which
-    // leaves a non-negative sum as it is, and every lane keeps the running sum at its own position, so
-    // that where the CPU loop would have stopped is read off afterwards with one ballot.  (A loop
-    // trip costs about as much as ten of these instructions.)
+    // The three walks below are the CPU's sequential fp32 sums.  Each is a chain of DPP shifts over the lanes
+    // (wave_sequential_sums_of_first): every lane ends up with the running sum at its own position, without a
+    // data-dependent exit; a lane past the end (or a filtered candidate) adds +0.0, which leaves a
+    // non-negative sum as it is, and where the CPU loop would have stopped is read off afterwards with one ballot.
     NCNN_MOE_STAMP_ROW(row, 1);
-    const int trips = (n + 3) >> 2;
-    float normalizer = 0.0f;
-    for (int trip = 0; trip < trips; ++trip)
-    {
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-            normalizer += read_lane(term, trip * 4 + k);
-    }
+    const float normalizer = read_lane(wave_sequential_sums_of_first(term, n), n - 1);
     if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
     {
         if (lane == 0)
@@ -181,19 +173,7 @@ __device__ __forceinline__ void finish_row_wave(
 
     // Top-P: the cumulative sum over the kept candidates in order, up to the first that reaches top_p
     const float contribution = keep ? probability : 0.0f;
-    float cumulative = 0.0f;
-    float cumulative_here = 0.0f;
-    for (int trip = 0; trip < trips; ++trip)
-    {
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-        {
-            cumulative += read_lane(contribution, trip * 4 + k);
-            cumulative_here = lane == trip * 4 + k ? cumulative : cumulative_here;
-        }
-        if (__ballot(keep && cumulative_here >= p.top_p) != 0)
-            break; // the nucleus is complete: the sums behind it are not needed
-    }
+    const float cumulative_here = wave_sequential_sums_of_first(contribution, n);
     NCNN_MOE_STAMP_ROW(row, 3);
     const uint64_t reached = __ballot(keep && cumulative_here >= p.top_p);
     const int last = reached != 0 ? __builtin_ctzll(reached) : 63 - __builtin_clzll(keep_mask);
@@ -232,18 +212,7 @@ __device__ __forceinline__ void finish_row_wave(
         draw_consumed = 1;
         const bool is_kept = ((kept_mask >> lane) & 1ull) != 0ull;
         const float share = is_kept ? final_probability : 0.0f;
-        float running = 0.0f;
-        float running_here = 0.0f;
-        const int draw_trips = (last + 4) >> 2; // positions 0 .. last
-        for (int trip = 0; trip < draw_trips; ++trip)
-        {
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-            {
-                running += read_lane(share, trip * 4 + k);
-                running_here = lane == trip * 4 + k ? running : running_here;
-            }
-        }
+        const float running_here = wave_sequential_sums_of_first(share, last + 1); // positions 0 .. last
         const uint64_t passed = __ballot(is_kept && uniform < running_here);
         selected = passed != 0 ? __builtin_ctzll(passed) : last; // past the last sum: the last kept candidate
         selected_probability = read_lane(final_probability, selected);

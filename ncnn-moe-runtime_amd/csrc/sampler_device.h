@@ -364,6 +364,24 @@ __device__ __forceinline__ float wave_sequential_sums(float term)
     return sums;
 }
 
+// The same for the wave's first `count` lanes (count: the same in every lane): count - 1 turns, rounded up to
+// whole trips of four (a turn too many changes nothing: a lane whose lower neighbour is final computes its own
+// final value again).  The lanes from `count` on return no sum of anything.
+__device__ __forceinline__ float wave_sequential_sums_of_first(float term, int count)
+{
+    float sums = term;
+    for (int turn = 1; turn < count; turn += 4)
+    {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+            const float below = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sums), 0x138, 0xf, 0xf, true));
+            sums = below + term;
+        }
+    }
+    return sums;
+}
+
 // Reduction over each row of 16 lanes (every lane receives its row's result), by four DPP exchanges:
 // inside pairs, quads, half rows, rows.
 template <typename Op>
