@@ -115,7 +115,35 @@ __device__ unsigned long long g_timeline_rows[kTimelineRows * kTimelineSlots];
         if ((leader) && (row) < static_cast<uint32_t>(kTimelineRows))                                        \
             g_timeline[((row) * kMaxSegments + (segment)) * kTimelineSlots + (slot)] = (value);              \
     } while (0)
+// Stamps of the split kernel are kept in LDS while the workgroup runs and written out when it leaves: a
+// store to device memory in the middle of the kernel would be waited for by the next full barrier.
+#define NCNN_MOE_LSTAMP_DECLARE __shared__ unsigned long long timeline_staging[kTimelineSlots]
+#define NCNN_MOE_LSTAMP(slot)                                                                                \
+    do                                                                                                       \
+    {                                                                                                        \
+        if (threadIdx.x == 0)                                                                                \
+            timeline_staging[slot] = wall_clock64();                                                         \
+    } while (0)
+#define NCNN_MOE_LSTAMP_VALUE(slot, value)                                                                   \
+    do                                                                                                       \
+    {                                                                                                        \
+        if (threadIdx.x == 0)                                                                                \
+            timeline_staging[slot] = (value);                                                                \
+    } while (0)
+#define NCNN_MOE_LSTAMP_FLUSH(row, segment, first, last)                                                     \
+    do                                                                                                       \
+    {                                                                                                        \
+        if (threadIdx.x == 0 && (row) < static_cast<uint32_t>(kTimelineRows))                                \
+        {                                                                                                    \
+            for (int slot_ = (first); slot_ <= (last); ++slot_)                                              \
+                g_timeline[((row) * kMaxSegments + (segment)) * kTimelineSlots + slot_] = timeline_staging[slot_]; \
+        }                                                                                                    \
+    } while (0)
 #else
+#define NCNN_MOE_LSTAMP_DECLARE ((void)0)
+#define NCNN_MOE_LSTAMP(slot) ((void)0)
+#define NCNN_MOE_LSTAMP_VALUE(slot, value) ((void)0)
+#define NCNN_MOE_LSTAMP_FLUSH(row, segment, first, last) ((void)0)
 #define NCNN_MOE_STAMP_VALUE_FROM(leader, row, segment, slot, value) ((void)0)
 #define NCNN_MOE_STAMP_ROW(row, slot) ((void)0)
 #define NCNN_MOE_COUNT(row, segment, slot) ((void)0)
@@ -401,6 +429,16 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t value)
     value = row16_reduce_u32(value, larger);
     value = max(value, dpp_source<0x142, 0xa>(value)); // row_bcast15 into rows 1 and 3
     value = max(value, dpp_source<0x143, 0xc>(value)); // row_bcast31 into rows 2 and 3
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(value), 63));
+}
+
+// Bitwise OR over the wave, returned to every lane (the same value in all: a scalar).
+__device__ __forceinline__ uint32_t wave_or_u32(uint32_t value)
+{
+    const auto either = [](uint32_t x, uint32_t y) { return x | y; };
+    value = row16_reduce_u32(value, either);
+    value |= dpp_source<0x142, 0xa>(value); // row_bcast15 into rows 1 and 3
+    value |= dpp_source<0x143, 0xc>(value); // row_bcast31 into rows 2 and 3
     return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(value), 63));
 }
 

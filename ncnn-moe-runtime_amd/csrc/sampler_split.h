@@ -32,6 +32,7 @@ constexpr uint32_t kSplitIndexBits = 18; // a split row holds at most 16 chunks 
 constexpr uint32_t kSplitIndexMask = (1u << kSplitIndexBits) - 1u;
 constexpr uint32_t kSplitLastEpoch = (1u << (32 - kSplitIndexBits)) - 1u; // epochs run 1 .. 16383; 0 never tags an entry
 constexpr int kSplitBins = kWaveSize;    // one histogram bin per lane of the scanning wave
+constexpr int kSplitBinCapacity = 16;    // candidates of one bin that the merge orders in place (more: the list and its rankings)
 constexpr uint32_t kSplitRetryLimit = 1u << 16;
 static_assert(kMaxSegments * kSegmentValuesBF16 + 8 <= (1 << kSplitIndexBits), "token indices of a split row fit the entry");
 static_assert(kSplitHeaderEntries + 2 * kFastTopK + 16 <= kSplitRecordSlots, "a record holds the widest hand-over");
@@ -49,6 +50,9 @@ struct SplitShared
     SelectShared<false> select;
     SplitSegmentInfo segments[kMaxSegments];
     uint32_t histogram[kSplitBins];
+    alignas(16) uint32_t bin_keys[kSplitBins * kSplitBinCapacity];   // the candidates of a bin, in the order the histogram's atomics placed them
+    alignas(16) uint32_t bin_indices[kSplitBins * kSplitBinCapacity];
+    uint32_t retry;
     uint32_t segment_maximum;
     uint64_t exp2_table[32];
     int is_last;
@@ -111,7 +115,10 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     __shared__ SplitShared shared;
     SelectShared<false>& select = shared.select;
 
-    NCNN_MOE_STAMP(row, segment, 0);
+    NCNN_MOE_LSTAMP_DECLARE;
+    NCNN_MOE_LSTAMP(0);
+    NCNN_MOE_LSTAMP_VALUE(10, static_cast<unsigned long long>(__builtin_amdgcn_s_getreg((31 << 11) | 4)) |
+                         (static_cast<unsigned long long>(__builtin_amdgcn_s_getreg(kXccIdRegister)) << 32));
     // The chunk's loads go out before anything that waits for the row's options.
     const char* row_pointer = static_cast<const char*>(a.logits) +
         static_cast<size_t>(row) * a.row_stride * Vector::kElementBytes;
@@ -139,6 +146,7 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     }
     uint4 raw[kVectors];
     load_chunk<DTYPE, kVectors>(raw, aligned_base, chunk_base, valid_begin, segment_end, valid_end, tid);
+    NCNN_MOE_LSTAMP(9); // (the loads are on their way)
     const ncnn_moe_sample_params p = a.params[row];
     const float uniform = a.uniforms[row];
     const uint64_t exp2_entry = kExp2Table[tid & 31]; // staged in LDS below: the merge's exponentials find it there
@@ -174,13 +182,29 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
         select.block_flags = 0;
         select.list_count = 0;
         shared.segment_maximum = 0xffffffffu; // unknown unless the bound routine below reports it
+        shared.retry = 0;
     }
     if (tid < 32)
         shared.exp2_table[tid] = exp2_entry;
+    if (tid >= kScanThreads - kSplitBins)
+        shared.histogram[tid - (kScanThreads - kSplitBins)] = 0; // (of the merge, should this workgroup be the row's last)
     if (touched == 0x9e3779b9u)
         select.block_flags = 0; // keeps the touching loads alive; the value is never that
     __syncthreads(); // also waits for the chunk
-    NCNN_MOE_STAMP(row, segment, 1);
+    NCNN_MOE_LSTAMP(1);
+    // The launch ends with its last rows: once their logits are there, their workgroups go first where they
+    // share a compute unit's vector units with workgroups of earlier rows (the workgroups of a compute unit
+    // come from the four quarters of the grid, one each).  Not before: a wave of lower priority would also
+    // issue its loads later.
+    {
+        const uint32_t quarter = row * 4u / max(a.rows, 1u);
+        if (quarter >= 3u)
+            __builtin_amdgcn_s_setprio(3);
+        else if (quarter == 2u)
+            __builtin_amdgcn_s_setprio(2);
+        else if (quarter == 1u)
+            __builtin_amdgcn_s_setprio(1);
+    }
 
     // ---- the chunk: maxima, flags.  Nearly every chunk lies inside the row (only a row's last chunk, or
     // the first one of a row that does not start on a 16-byte boundary, holds foreign elements): those skip
@@ -259,7 +283,7 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     uint32_t bound_key = workgroup_kth_of_quad_maxima(lane_keys[0], top_k, tid, select.bound, &shared.segment_maximum);
     if (bound_key == 0u) // a chunk with few values: the exact K-th largest lane maximum
         bound_key = workgroup_kth_largest_key(lane_keys, top_k, tid, select.bound, true);
-    NCNN_MOE_STAMP(row, segment, 2);
+    NCNN_MOE_LSTAMP(2);
     // no bound (fewer than K lanes hold a finite logit): every finite logit is a candidate
     const float threshold = bound_key == 0u ? -3.402823466e+38f : fmaxf(value_from_ascending_key(bound_key), -3.402823466e+38f);
 
@@ -289,7 +313,8 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
             rest |= (lane_hits > 1 && values[i] >= threshold && i != best_at) ? (1u << i) : 0u;
         while (__ballot(rest != 0u) != 0)
         {
-            // the value is read back from the row (its register is not known until run time)
+            // the value is read back from the row (its register is not known until run time; picking it out of
+            // the registers, by selects or by handing the lane's values to the wave's other lanes, was no faster)
             const int i = rest != 0u ? __builtin_ctz(rest) : 0;
             const int32_t element = element_of(i);
             float x = 0.0f;
@@ -307,7 +332,7 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     if (local_flags != 0)
         atomicOr(&select.block_flags, local_flags);
     __syncthreads();
-    NCNN_MOE_STAMP(row, segment, 3);
+    NCNN_MOE_LSTAMP(3);
     bool overflow = select.list_count > static_cast<uint32_t>(kNarrowListCap);
     // the record holds 2K + 16 candidates: a longer list (a loose bound, ties) is cut to the exact window first
     if (!overflow && select.list_count > record_entries)
@@ -359,9 +384,13 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
         shared.is_last = previous == a.segments - 1 ? 1 : 0;
     }
     lds_barrier();
-    NCNN_MOE_STAMP(row, segment, 4);
+    NCNN_MOE_LSTAMP(4);
     if (!shared.is_last)
+    {
+        NCNN_MOE_LSTAMP_FLUSH(row, segment, 0, 4);
+        NCNN_MOE_LSTAMP_FLUSH(row, segment, 9, 14);
         return;
+    }
 
     // ---- last workgroup of the row.  The row's next launch gets a new epoch whatever happens below.
     if (tid == 0)
@@ -385,44 +414,49 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
             }
         }
     }
+    // Every wave reads the headers of all the row's segments for itself (lane s the first entry of segment s,
+    // lane 16 + s the second): the row's bound, maximum and flags then come from exchanges inside the wave,
+    // without a trip through LDS and a barrier behind the records' arrival.
+    const uint32_t header_segment = static_cast<uint32_t>(lane & (kMaxSegments - 1));
+    const bool header_lane = lane < 2 * kMaxSegments && header_segment < a.segments;
+    const bool own_header = header_segment == segment;
+    const unsigned long long* const header_address = row_records + static_cast<size_t>(header_segment) * kSplitRecordSlots + ((lane >> 4) & 1);
+    unsigned long long header = 0ull;
+    const auto load_headers = [&](bool around_l2) {
+        if (header_lane && !own_header)
+            header = load_entry(header_address, around_l2);
+    };
+    load_headers(false);
     load_records(false);
     uint32_t lower = 0, upper = 0, row_flags = 0;
     uint32_t my_count = 0;
     uint32_t attempts = 0;
+    int bins[kSplitSlotsPerLane];
+    uint32_t bin_counts = 0;
     for (uint32_t attempt = 0;; ++attempt)
     {
         attempts = attempt + 1u;
-        // headers: entries 0 and 1 sit in lanes 0 and 1 of the 32 lanes that read the segment
-        const int low_word = static_cast<int>(static_cast<uint32_t>(loaded[0]));
-        const int high_word = static_cast<int>(static_cast<uint32_t>(loaded[0] >> 32));
-        const bool upper_half = lane >= kSplitLanesPerSegment;
-        const uint32_t bound_word = static_cast<uint32_t>(upper_half ? __builtin_amdgcn_readlane(low_word, 32) : __builtin_amdgcn_readlane(low_word, 0));
-        const uint32_t bound_tag = static_cast<uint32_t>(upper_half ? __builtin_amdgcn_readlane(high_word, 32) : __builtin_amdgcn_readlane(high_word, 0));
-        const uint32_t maximum_word = static_cast<uint32_t>(upper_half ? __builtin_amdgcn_readlane(low_word, 33) : __builtin_amdgcn_readlane(low_word, 1));
-        const uint32_t maximum_tag = static_cast<uint32_t>(upper_half ? __builtin_amdgcn_readlane(high_word, 33) : __builtin_amdgcn_readlane(high_word, 1));
-        SplitSegmentInfo info;
-        bool valid = true;
-        if (reads_own)
+        uint32_t word = static_cast<uint32_t>(header);
+        uint32_t tag_word = static_cast<uint32_t>(header >> 32);
+        if (lane < 2 * kMaxSegments && own_header)
         {
-            info.bound = bound_key;
-            info.maximum = shared.segment_maximum;
-            info.count_and_flags = own_count | (segment_flags << 8);
+            word = lane < kMaxSegments ? bound_key : shared.segment_maximum;
+            tag_word = lane < kMaxSegments ? (tag | own_count | (segment_flags << 8)) : tag;
         }
-        else if (reads_any)
-        {
-            valid = (bound_tag >> kSplitIndexBits) == epoch && (maximum_tag >> kSplitIndexBits) == epoch;
-            info.bound = bound_word;
-            info.maximum = maximum_word;
-            info.count_and_flags = bound_tag & 0x7ffu;
-        }
-        else
-        {
-            info.bound = 0u;
-            info.maximum = 0u;
-            info.count_and_flags = 0u;
-        }
-        my_count = valid ? (info.count_and_flags & 0xffu) : 0u;
-        if (reads_any && valid)
+        bool valid = !header_lane || (tag_word >> kSplitIndexBits) == epoch;
+        // rows of 16 lanes: the first holds the segments' bounds, counts and flags, the second their maxima
+        const auto larger = [](uint32_t x, uint32_t y) { return max(x, y); };
+        const uint32_t extremes = row16_reduce_u32(header_lane ? word : 0u, larger);
+        lower = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(extremes), 0));
+        upper = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(extremes), kMaxSegments));
+        const uint32_t flag_bits = row16_reduce_u32((header_lane && lane < kMaxSegments) ? ((tag_word >> 8) & 7u) : 0u,
+                                                    [](uint32_t x, uint32_t y) { return x | y; });
+        row_flags = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(flag_bits), 0));
+        const uint32_t count_word = (header_lane && lane < kMaxSegments) ? (tag_word & 0xffu) : 0u;
+        const uint32_t count_low = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(count_word), 2 * wave));
+        const uint32_t count_high = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(count_word), 2 * wave + 1));
+        my_count = lane >= kSplitLanesPerSegment ? count_high : count_low;
+        if (reads_any)
         {
 #pragma unroll
             for (int j = 0; j < kSplitSlotsPerLane; ++j)
@@ -432,37 +466,56 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
                     valid = valid && (static_cast<uint32_t>(loaded[j] >> 32) >> kSplitIndexBits) == epoch;
             }
         }
-        // bit 31: something of this segment's record is not of this launch (each half of the wave for its own)
-        const uint64_t invalid_lanes = __ballot(!valid);
-        const uint32_t half_invalid = upper_half ? static_cast<uint32_t>(invalid_lanes >> 32) : static_cast<uint32_t>(invalid_lanes);
-        info.count_and_flags |= half_invalid != 0u ? 0x80000000u : 0u;
+        if (__ballot(!valid) != 0ull && lane == 0)
+            shared.retry = 1; // something of this launch has not landed yet (or the L2 held a stale line)
+
+        // ---- cut and order in one pass: a histogram of the candidates at or above the largest segment
+        // bound (at least K logits of that segment reach it, so nothing below it is in the window) over
+        // [that bound, row maximum], bin 0 at the top.  The atomic that counts a candidate also gives it a
+        // place in its bin's short list; behind the barrier a scan over the bins tells every candidate how
+        // many lie in the bins above its own, its bin's list how many of its own bin go before it: that is its
+        // place in the window.
+        const uint32_t span = upper >= lower ? upper - lower : 0u;
+        const float scale = static_cast<float>(kSplitBins) / (static_cast<float>(span) + 1.0f);
+#pragma unroll
+        for (int j = 0; j < kSplitSlotsPerLane; ++j)
+        {
+            bins[j] = -1;
+            if (static_cast<uint32_t>(j * kSplitLanesPerSegment) >= entries_to_read)
+                continue; // no entry of this or a later round exists (a scalar test)
+            const uint32_t entry = static_cast<uint32_t>(j * kSplitLanesPerSegment + read_lane);
+            const uint32_t key = static_cast<uint32_t>(loaded[j]);
+            const bool candidate = entry >= static_cast<uint32_t>(kSplitHeaderEntries) && entry - kSplitHeaderEntries < my_count && key >= lower;
+            if (candidate)
+            {
+                const uint32_t distance = min(key, upper) - lower;
+                const int from_bottom = min(kSplitBins - 1, static_cast<int>(static_cast<float>(distance) * scale));
+                bins[j] = kSplitBins - 1 - from_bottom;
+                const uint32_t place = atomicAdd(&shared.histogram[bins[j]], 1u);
+                if (place < static_cast<uint32_t>(kSplitBinCapacity))
+                {
+                    shared.bin_keys[bins[j] * kSplitBinCapacity + place] = key;
+                    shared.bin_indices[bins[j] * kSplitBinCapacity + place] = static_cast<uint32_t>(loaded[j] >> 32) & kSplitIndexMask;
+                }
+            }
+        }
+        lds_barrier();
+        bin_counts = shared.histogram[lane];
+        if (shared.retry == 0)
+            break;
+        // An entry of this launch has not landed yet: read the records again from device memory.  The
+        // stores in question were issued before their workgroup counted itself, so they land without
+        // anyone else having to run.
+        lds_barrier(); // every wave has read the flag and its bins before they are cleared
         if (tid < kSplitBins)
             shared.histogram[tid] = 0;
-        if (read_lane == 0)
-            shared.segments[read_segment] = info;
-        lds_barrier();
-        // every wave reduces the sixteen segments for itself
-        const SplitSegmentInfo other = shared.segments[lane & (kMaxSegments - 1)];
-        const auto larger = [](uint32_t x, uint32_t y) { return max(x, y); };
-        lower = row16_reduce_u32(other.bound, larger);
-        upper = row16_reduce_u32(other.maximum, larger);
-        row_flags = row16_reduce_u32(other.count_and_flags >> 8, [](uint32_t x, uint32_t y) { return x | y; });
-        if ((row_flags & 0x800000u) == 0u)
-            break;
-        lds_barrier(); // every wave has read the segments before the next round rewrites them
-        // An entry of this launch has not landed yet (or the L2 held a stale line): read the records
-        // again from device memory.  The stores in question were issued before their workgroup counted
-        // itself, so they land without anyone else having to run.
+        if (tid == 0)
+            shared.retry = 0;
         if (attempt >= kSplitRetryLimit)
-        {
-            if (tid == 0)
-            {
-                write_pending(a, row);
-                a.row_state[row] = kRowNeedsGeneral;
-            }
-            return;
-        }
+            break;
+        load_headers(true);
         load_records(true);
+        lds_barrier();
     }
     if (epoch == kSplitLastEpoch)
     {
@@ -470,12 +523,13 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
         for (uint32_t j = tid; j < static_cast<uint32_t>(kMaxSegments * kSplitRecordSlots); j += kScanThreads)
             store_entry(&row_records[j], 0u, 0u);
     }
-    NCNN_MOE_STAMP(row, segment, 5);
-    NCNN_MOE_STAMP_VALUE(row, segment, 8, attempts);
+    NCNN_MOE_LSTAMP(5);
+    NCNN_MOE_LSTAMP_VALUE(8, attempts);
     const uint8_t result_flags = (row_flags & kScanSawNan) ? NCNN_MOE_ROW_FLAG_HAS_NAN : 0;
-    if (row_flags & kScanOverflow)
+    if (attempts > kSplitRetryLimit || (row_flags & kScanOverflow))
     {
-        // ties (or values that defeat the bound) left more candidates than a record holds: the full-order kernels take the row
+        // entries that never landed, or ties (or values that defeat the bound) that left more candidates than a
+        // record holds: the full-order kernels take the row
         if (tid == 0)
         {
             write_pending(a, row);
@@ -494,34 +548,70 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
         return;
     }
 
-    // ---- cut: a histogram of the candidates at or above the largest segment bound (at least K logits of
-    // that segment reach it, so nothing below it is in the window) over [that bound, row maximum], bin 0
-    // at the top.  The first bin at which the count from the top reaches K ends the selection.
-    const uint32_t span = upper >= lower ? upper - lower : 0u;
-    const float scale = static_cast<float>(kSplitBins) / (static_cast<float>(span) + 1.0f);
-    int bins[kSplitSlotsPerLane];
-#pragma unroll
-    for (int j = 0; j < kSplitSlotsPerLane; ++j)
-    {
-        const uint32_t entry = static_cast<uint32_t>(j * kSplitLanesPerSegment + read_lane);
-        const uint32_t key = static_cast<uint32_t>(loaded[j]);
-        const bool candidate = entry >= static_cast<uint32_t>(kSplitHeaderEntries) && entry - kSplitHeaderEntries < my_count && key >= lower;
-        bins[j] = -1;
-        if (candidate)
-        {
-            const uint32_t distance = min(key, upper) - lower;
-            const int from_bottom = min(kSplitBins - 1, static_cast<int>(static_cast<float>(distance) * scale));
-            bins[j] = kSplitBins - 1 - from_bottom;
-            atomicAdd(&shared.histogram[bins[j]], 1u);
-        }
-    }
-    if (tid == 0)
-        select.list_count = 0;
-    lds_barrier();
-    const uint32_t from_top = wave_prefix_sum_u32(shared.histogram[lane]);
+    // The first bin at which the count from the top reaches K ends the selection.
+    const uint32_t from_top = wave_prefix_sum_u32(bin_counts);
     const uint64_t reached = __ballot(from_top >= static_cast<uint32_t>(top_k));
     const int cut = reached != 0 ? __builtin_ctzll(reached) : kSplitBins - 1;
     const uint32_t selected = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(from_top), cut));
+    const uint32_t fullest = wave_max_u32(lane <= cut ? bin_counts : 0u); // of the bins that hold the window
+    if (fullest <= static_cast<uint32_t>(kSplitBinCapacity))
+    {
+        // (above, bin count) of every bin in one word, fetched by the candidates of that bin
+        const uint32_t packed = ((from_top - bin_counts) << 16) | bin_counts;
+#pragma unroll
+        for (int j = 0; j < kSplitSlotsPerLane; ++j)
+        {
+            if (static_cast<uint32_t>(j * kSplitLanesPerSegment) >= entries_to_read)
+                break;
+            const int bin = bins[j] >= 0 ? bins[j] : 0;
+            const uint32_t of_bin = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(bin << 2, static_cast<int>(packed)));
+            if (bins[j] >= 0 && bins[j] <= cut)
+            {
+                const uint32_t key = static_cast<uint32_t>(loaded[j]);
+                const uint32_t index = static_cast<uint32_t>(loaded[j] >> 32) & kSplitIndexMask;
+                const uint32_t in_bin = of_bin & 0xffffu;
+                uint32_t before = of_bin >> 16;
+                for (uint32_t first = 0; first < fullest; first += 4u) // (fullest is the same in every lane)
+                {
+                    const uint4 other_keys = *reinterpret_cast<const uint4*>(&shared.bin_keys[bin * kSplitBinCapacity + first]);
+                    const uint4 other_indices = *reinterpret_cast<const uint4*>(&shared.bin_indices[bin * kSplitBinCapacity + first]);
+                    before += (first + 0u < in_bin && (other_keys.x > key || (other_keys.x == key && other_indices.x < index))) ? 1u : 0u;
+                    before += (first + 1u < in_bin && (other_keys.y > key || (other_keys.y == key && other_indices.y < index))) ? 1u : 0u;
+                    before += (first + 2u < in_bin && (other_keys.z > key || (other_keys.z == key && other_indices.z < index))) ? 1u : 0u;
+                    before += (first + 3u < in_bin && (other_keys.w > key || (other_keys.w == key && other_indices.w < index))) ? 1u : 0u;
+                }
+                if (before < static_cast<uint32_t>(top_k))
+                {
+                    select.final_values[before] = value_from_ascending_key(key);
+                    select.final_indices[before] = static_cast<int32_t>(index);
+                }
+            }
+        }
+        lds_barrier();
+        NCNN_MOE_LSTAMP(6);
+        if (wave == 0)
+        {
+            const int n = static_cast<int>(min(selected, static_cast<uint32_t>(top_k)));
+            if (lane == 0)
+                a.row_state[row] = kRowDone;
+            if (n == 0)
+            {
+                if (lane == 0)
+                    write_error(a, row, NCNN_MOE_ROW_NO_FINITE_LOGIT, result_flags);
+            }
+            else
+            {
+                const float value = lane < n ? select.final_values[lane] : 0.0f;
+                const int32_t index = lane < n ? select.final_indices[lane] : -1;
+                finish_ordered_wave(a, row, p, greedy, value, index, n, lane, result_flags, uniform, shared.exp2_table);
+            }
+        }
+        NCNN_MOE_LSTAMP(7);
+        NCNN_MOE_LSTAMP_FLUSH(row, segment, 0, 14);
+        return;
+    }
+    // A bin of the window holds more candidates than its list (ties, or a window that is most of its range's
+    // lower end): the candidates above the cut go to the list and are ranked from there.
     if (selected > static_cast<uint32_t>(kNarrowListCap))
     {
         if (tid == 0)
@@ -531,6 +621,9 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
         }
         return;
     }
+    if (tid == 0)
+        select.list_count = 0;
+    __syncthreads();
 #pragma unroll
     for (int j = 0; j < kSplitSlotsPerLane; ++j)
     {
@@ -540,9 +633,10 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
                          static_cast<int32_t>(static_cast<uint32_t>(loaded[j] >> 32) & kSplitIndexMask), lane);
     }
     __syncthreads();
-    NCNN_MOE_STAMP(row, segment, 6);
+    NCNN_MOE_LSTAMP(6);
     finish_from_list(a, row, p, greedy, top_k, select, result_flags, tid, uniform, shared.exp2_table);
-    NCNN_MOE_STAMP(row, segment, 7);
+    NCNN_MOE_LSTAMP(7);
+    NCNN_MOE_LSTAMP_FLUSH(row, segment, 0, 14);
 }
 
 // The split kernel's grid and loads with nothing behind them: every workgroup reads its chunk and one lane
