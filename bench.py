@@ -656,19 +656,22 @@ def main():
         "cache_resident_note": "same loop on one logits buffer (%.1f MB), held by the Infinity Cache where it fits; "
                                "not the reported value" % (batch_bytes / 1e6),
     }
-    if hip_sampler.select_geometry(dtype_code, rows, vocab)[2] == hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK:
+    if os.path.exists(hip_sampler.TESTING_LIBRARY_PATH) and \
+            hip_sampler.select_geometry(dtype_code, rows, vocab)[2] == hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK:
         # what a launch of this grid costs for streaming the logits alone: the split kernel's loads with
-        # nothing behind them, over the same rotated buffers
+        # nothing behind them, over the same rotated buffers (a probe kernel of the library's testing build)
+        probe = hip_sampler.HipSampler(rows, vocab, testing=True)
         with torch.cuda.stream(stream):
             for index in range(20):
-                sampler.stream_only(logits[index % buffers].data_ptr(), dtype_code, rows, vocab, vocab, stream_pointer)
+                probe.stream_only(logits[index % buffers].data_ptr(), dtype_code, rows, vocab, vocab, stream_pointer)
             stream_start = torch.cuda.Event(enable_timing=True)
             stream_stop = torch.cuda.Event(enable_timing=True)
             stream_start.record(stream)
             for index in range(detail_steps * 4):
-                sampler.stream_only(logits[index % buffers].data_ptr(), dtype_code, rows, vocab, vocab, stream_pointer)
+                probe.stream_only(logits[index % buffers].data_ptr(), dtype_code, rows, vocab, vocab, stream_pointer)
             stream_stop.record(stream)
             stream.synchronize()
+        probe.close()
         detail["stream_only_ms_per_launch"] = stream_start.elapsed_time(stream_stop) / (detail_steps * 4)
         detail["stream_only_note"] = ("the split kernel's grid and loads with nothing behind them (%d launches over the rotated "
                                       "buffers): the cost of streaming the logits alone; not the reported value" % (detail_steps * 4))

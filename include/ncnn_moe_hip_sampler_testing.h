@@ -30,6 +30,10 @@ int ncnn_moe_hip_sampler_debug_chunk_steps(ncnn_moe_hip_sampler* sampler, int en
 /* spread_sort (on by default): the radix sort of a long full-order row runs on several workgroups; off,
  * every row is sorted by one workgroup. */
 int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* sampler, int enabled);
+/* Sets the per-row launch numbers (epochs, 1 .. 16383) that tag the split kernel's hand-over records: of the
+ * handle, or with a null handle of the static scratch of `device` (after it has served a call).  Tests start a
+ * few launches in front of the point where the epochs start over. */
+int ncnn_moe_hip_sampler_debug_set_row_epochs(ncnn_moe_hip_sampler* sampler, int device, uint32_t epoch);
 int ncnn_moe_hip_sampler_debug_expf(ncnn_moe_hip_sampler* sampler, const float* in, float* out, size_t n);
 void ncnn_moe_hip_sampler_debug_exp2_table(uint64_t out[32]);
 

@@ -874,6 +874,10 @@ int ncnn_moe_hip_sampler_sample_device_static(
             hipLaunchKernelGGL(static_scratch_clear_kernel, dim3((kClearWords + kClearThreads - 1) / kClearThreads), dim3(kClearThreads), 0, on,
                                static_cast<StaticScratchLayout*>(address));
             error = hipGetLastError();
+            // The first call on a device waits for the clearing kernel: a second caller, on another stream,
+            // finds the pointer only once the array is in the state every launch expects.
+            if (error == hipSuccess)
+                error = hipStreamSynchronize(on);
             if (error != hipSuccess)
                 return static_fail(NCNN_MOE_SAMPLER_HIP_ERROR, "clearing the static scratch", hipGetErrorString(error));
             g_static_scratch[device] = static_cast<StaticScratchLayout*>(address);
@@ -1107,6 +1111,8 @@ const char* ncnn_moe_hip_sampler_status_message(int row_status)
     }
 }
 
+// ---- test hooks (include/ncnn_moe_hip_sampler_testing.h): compiled into the testing build of the library only
+#ifdef NCNN_MOE_TESTING
 int ncnn_moe_hip_sampler_debug_force_general(ncnn_moe_hip_sampler* s, int enabled)
 {
     if (s == nullptr)
@@ -1120,6 +1126,37 @@ int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* s, int enabled)
     if (s == nullptr)
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     s->spread_sort = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+// Sets the launch number (epoch) of every row, of a handle's split records or, with a null handle, of the
+// static scratch of `device` (which must have served a call before): tests start a few launches in front
+// of the point where the epochs start over.
+int ncnn_moe_hip_sampler_debug_set_row_epochs(ncnn_moe_hip_sampler* s, int device, uint32_t epoch)
+{
+    if (epoch == 0u || epoch > kSplitLastEpoch)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    uint32_t* epochs = nullptr;
+    size_t count = 0;
+    if (s != nullptr)
+    {
+        if (hipSetDevice(s->device) != hipSuccess)
+            return NCNN_MOE_SAMPLER_HIP_ERROR;
+        epochs = s->row_epoch;
+        count = s->max_rows;
+    }
+    else
+    {
+        std::lock_guard<std::mutex> lock(g_static_mutex);
+        if (device < 0 || device >= kStaticMaxDevices || g_static_scratch[device] == nullptr || hipSetDevice(device) != hipSuccess)
+            return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+        epochs = g_static_scratch[device]->row_epoch;
+        count = kStaticMaxRows;
+    }
+    if (hipDeviceSynchronize() != hipSuccess ||
+        hipMemsetD32(reinterpret_cast<hipDeviceptr_t>(epochs), static_cast<int>(epoch), count) != hipSuccess ||
+        hipDeviceSynchronize() != hipSuccess)
+        return NCNN_MOE_SAMPLER_HIP_ERROR;
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 
@@ -1235,5 +1272,7 @@ void ncnn_moe_hip_sampler_debug_exp2_table(uint64_t out[32])
     static const uint64_t table[32] = {NCNN_MOE_EXP2_TABLE_VALUES};
     std::memcpy(out, table, sizeof(table));
 }
+
+#endif // NCNN_MOE_TESTING
 
 } // extern "C"

@@ -15,13 +15,15 @@
 
 namespace ncnn_moe_hip {
 
-// Evaluates expf_libm on n values (test hook).
+#ifdef NCNN_MOE_TESTING
+// Evaluates expf_libm on n values (test hook; in the testing build of the library only).
 __global__ void expf_probe_kernel(const float* in, float* out, size_t n)
 {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < n)
         out[i] = expf_libm(in[i]);
 }
+#endif
 
 } // namespace ncnn_moe_hip
 

@@ -639,9 +639,10 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     NCNN_MOE_LSTAMP_FLUSH(row, segment, 0, 14);
 }
 
+#ifdef NCNN_MOE_TESTING
 // The split kernel's grid and loads with nothing behind them: every workgroup reads its chunk and one lane
 // per wave stores a word that depends on all of it.  What a launch of this shape costs for streaming the
-// logits alone (a probe for the benchmark's detail, not part of the sampling path).
+// logits alone (a probe for the benchmark's detail, not part of the sampling path; in the testing build only).
 template <int DTYPE>
 __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4) void split_stream_only_kernel(SamplerArgs a, uint32_t* sink)
 {
@@ -676,6 +677,7 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     if ((tid & (kWaveSize - 1)) == 0)
         sink[(static_cast<size_t>(row) * a.segments + segment) * kScanWaves + (tid >> 6)] = folded;
 }
+#endif // NCNN_MOE_TESTING
 
 } // namespace ncnn_moe_hip
 

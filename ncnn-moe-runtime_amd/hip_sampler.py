@@ -9,6 +9,7 @@ import numpy as np
 
 PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
 LIBRARY_PATH = os.path.join(PACKAGE_DIR, "libncnn_moe_hip_sampler.so")
+TESTING_LIBRARY_PATH = os.path.join(PACKAGE_DIR, "libncnn_moe_hip_sampler_testing.so")
 
 LOGITS_F32 = 0
 LOGITS_BF16 = 1
@@ -73,6 +74,7 @@ TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_spread_sort",
     "ncnn_moe_hip_sampler_debug_chunk_steps",
     "ncnn_moe_hip_sampler_debug_stream_only",
+    "ncnn_moe_hip_sampler_debug_set_row_epochs",
     "ncnn_moe_hip_sampler_debug_expf",
     "ncnn_moe_hip_sampler_debug_exp2_table",
     "ncnn_moe_hip_sampler_debug_select_geometry",
@@ -84,17 +86,10 @@ class SamplerError(RuntimeError):
 
 
 _library = None
+_testing_library = None
 
 
-def load_library():
-    """Loads the C-ABI library; raises if it has not been built."""
-    global _library
-    if _library is not None:
-        return _library
-    if not os.path.exists(LIBRARY_PATH):
-        raise SamplerError(
-            "%s is missing: build it with `make -C %s` (or __graft_entry__.build())" % (LIBRARY_PATH, PACKAGE_DIR))
-    lib = ctypes.CDLL(LIBRARY_PATH)
+def _bind(lib, testing):
     vp = ctypes.c_void_p
     lib.ncnn_moe_hip_sampler_create.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(vp)]
     lib.ncnn_moe_hip_sampler_destroy.argtypes = [vp]
@@ -117,22 +112,50 @@ def load_library():
     lib.ncnn_moe_hip_sampler_status_message.argtypes = [ctypes.c_int]
     lib.ncnn_moe_hip_sampler_status_message.restype = ctypes.c_char_p
     lib.ncnn_moe_hip_sampler_device_count.argtypes = []
+    if not testing:
+        return lib
     lib.ncnn_moe_hip_sampler_debug_force_general.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_scatter_segments.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_spread_sort.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_chunk_steps.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_stream_only.argtypes = [vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp]
+    lib.ncnn_moe_hip_sampler_debug_set_row_epochs.argtypes = [vp, ctypes.c_int, ctypes.c_uint32]
     lib.ncnn_moe_hip_sampler_debug_expf.argtypes = [vp, vp, vp, ctypes.c_size_t]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.argtypes = [vp]
     lib.ncnn_moe_hip_sampler_debug_exp2_table.restype = None
     lib.ncnn_moe_hip_sampler_debug_select_geometry.argtypes = [
         ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
         ctypes.POINTER(ctypes.c_uint32)]
-    _library = lib
     return lib
 
 
+def load_library():
+    """Loads the C-ABI library (the boundary of include/ncnn_moe_hip_sampler.h); raises if it has not been built."""
+    global _library
+    if _library is not None:
+        return _library
+    if not os.path.exists(LIBRARY_PATH):
+        raise SamplerError(
+            "%s is missing: build it with `make -C %s` (or __graft_entry__.build())" % (LIBRARY_PATH, PACKAGE_DIR))
+    _library = _bind(ctypes.CDLL(LIBRARY_PATH), False)
+    return _library
+
+
+def load_testing_library():
+    """Loads the testing build of the library: the same source with the hooks of
+    include/ncnn_moe_hip_sampler_testing.h compiled in.  For this repository's tests and the benchmark's probes."""
+    global _testing_library
+    if _testing_library is not None:
+        return _testing_library
+    if not os.path.exists(TESTING_LIBRARY_PATH):
+        raise SamplerError(
+            "%s is missing: build it with `make -C %s` (or __graft_entry__.build())" % (TESTING_LIBRARY_PATH, PACKAGE_DIR))
+    _testing_library = _bind(ctypes.CDLL(TESTING_LIBRARY_PATH), True)
+    return _testing_library
+
+
 def status_message(row_status):
+    """The CPU sampler's message for a per-row status."""
     return load_library().ncnn_moe_hip_sampler_status_message(int(row_status)).decode()
 
 
@@ -148,7 +171,7 @@ GEOMETRY_SPLIT_LOOPED = 2
 def select_geometry(dtype, rows, vocab):
     """(workgroups per row, chunks per workgroup, kernel variant) of the first select kernel for this shape."""
     segments, chunks, variant = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
-    rc = load_library().ncnn_moe_hip_sampler_debug_select_geometry(
+    rc = load_testing_library().ncnn_moe_hip_sampler_debug_select_geometry(
         dtype, rows, vocab, ctypes.byref(segments), ctypes.byref(chunks), ctypes.byref(variant))
     if rc != RC_SUCCESS:
         raise SamplerError("select_geometry: rc=%d" % rc)
@@ -157,7 +180,7 @@ def select_geometry(dtype, rows, vocab):
 
 def exp2_table():
     out = np.zeros(32, dtype=np.uint64)
-    load_library().ncnn_moe_hip_sampler_debug_exp2_table(out.ctypes.data)
+    load_testing_library().ncnn_moe_hip_sampler_debug_exp2_table(out.ctypes.data)
     return out
 
 
@@ -171,10 +194,12 @@ def make_params(rows, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
 
 
 class HipSampler:
-    """One sampler handle on one device."""
+    """One sampler handle on one device.  testing=True creates it in the testing build of the library, whose
+    handles take the test hooks (force_general, scatter_segments, ...)."""
 
-    def __init__(self, max_rows, max_vocab, device=0):
-        self._lib = load_library()
+    def __init__(self, max_rows, max_vocab, device=0, testing=False):
+        self._testing = bool(testing)
+        self._lib = load_testing_library() if testing else load_library()
         self._handle = ctypes.c_void_p()
         rc = self._lib.ncnn_moe_hip_sampler_create(device, max_rows, max_vocab, ctypes.byref(self._handle))
         if rc != RC_SUCCESS:
@@ -273,45 +298,67 @@ class HipSampler:
             accepted.ctypes.data, result.ctypes.data))
         return result[0], accepted[:drafts]
 
+    def _hooks(self, enabling=True):
+        if not self._testing and not enabling:
+            return None  # switching off what the shipped library never switches on
+        if not self._testing:
+            raise SamplerError("test hooks live in the testing build of the library: create the sampler with testing=True")
+        return self._lib
+
     def force_general(self, enabled):
-        self._check(self._lib.ncnn_moe_hip_sampler_debug_force_general(self._handle, 1 if enabled else 0))
+        hooks = self._hooks(bool(enabled))
+        if hooks is not None:
+            self._check(hooks.ncnn_moe_hip_sampler_debug_force_general(self._handle, 1 if enabled else 0))
 
     def scatter_segments(self, enabled):
         """Test hook: split rows are launched without the XCD-aware numbering of the workgroups."""
-        self._check(self._lib.ncnn_moe_hip_sampler_debug_scatter_segments(self._handle, 1 if enabled else 0))
+        hooks = self._hooks(bool(enabled))
+        if hooks is not None:
+            self._check(hooks.ncnn_moe_hip_sampler_debug_scatter_segments(self._handle, 1 if enabled else 0))
 
     def stream_only(self, logits_ptr, dtype, rows, vocab, row_stride, stream=None):
         """Test hook: a launch with the split kernel's grid and loads and nothing behind them."""
-        self._check(self._lib.ncnn_moe_hip_sampler_debug_stream_only(self._handle, logits_ptr, dtype, rows, vocab, row_stride, stream))
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_stream_only(self._handle, logits_ptr, dtype, rows, vocab, row_stride, stream))
 
     def chunk_steps(self, enabled):
         """Test hook: whole chunks of a sorted fp32 row added in one precomputed step (default) or round by round."""
-        self._check(self._lib.ncnn_moe_hip_sampler_debug_chunk_steps(self._handle, 1 if enabled else 0))
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_chunk_steps(self._handle, 1 if enabled else 0))
 
     def spread_sort(self, enabled):
         """Test hook: the radix sort of long full-order rows on several workgroups (default) or on one."""
-        self._check(self._lib.ncnn_moe_hip_sampler_debug_spread_sort(self._handle, 1 if enabled else 0))
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_spread_sort(self._handle, 1 if enabled else 0))
+
+    def set_row_epochs(self, epoch):
+        """Test hook: the launch number that tags the split kernel's hand-over records, for every row (1 .. LAST_EPOCH)."""
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_set_row_epochs(self._handle, 0, epoch))
 
     def expf(self, values):
         values = np.ascontiguousarray(values, dtype=np.float32)
         out = np.empty_like(values)
-        self._check(self._lib.ncnn_moe_hip_sampler_debug_expf(self._handle, values.ctypes.data, out.ctypes.data, values.size))
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_expf(self._handle, values.ctypes.data, out.ctypes.data, values.size))
         return out
 
 
 STATIC_MAX_ROWS = 1024
+LAST_EPOCH = 16383  # the launch numbers of the split kernel's records run 1 .. LAST_EPOCH and start over
+
+
+def set_static_row_epochs(device, epoch):
+    """Test hook: set_row_epochs for the scratch of the entry that allocates nothing (after its first call on the device)."""
+    return load_testing_library().ncnn_moe_hip_sampler_debug_set_row_epochs(None, device, epoch)
 
 
 def sample_device_static(device, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr,
-                         stop_ids_ptr, results_ptr, stream=None):
+                         stop_ids_ptr, results_ptr, stream=None, testing=False):
     """The select pass without a handle and without any allocation (static device scratch); all pointers
-    are device addresses.  Returns the call's return code; last_static_error() has the reason."""
-    return load_library().ncnn_moe_hip_sampler_sample_device_static(
+    are device addresses.  Returns the call's return code; last_static_error() has the reason.  (Each build of
+    the library has a static array of its own: testing=True calls the testing build's.)"""
+    return (load_testing_library() if testing else load_library()).ncnn_moe_hip_sampler_sample_device_static(
         device, logits_ptr, dtype, rows, vocab, row_stride, params_ptr, uniforms_ptr, stop_ids_ptr, results_ptr, stream)
 
 
-def last_static_error():
-    return load_library().ncnn_moe_hip_sampler_last_error(None).decode()
+def last_static_error(testing=False):
+    return (load_testing_library() if testing else load_library()).ncnn_moe_hip_sampler_last_error(None).decode()
 
 
 def device_count():

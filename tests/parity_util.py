@@ -51,7 +51,7 @@ def parity_counters(gpu, cpu):
 def run_workload_on_gpu(workload, sampler=None, force_general=False):
     own = sampler is None
     if own:
-        sampler = hip_sampler.HipSampler(workload["rows"], workload["vocab"])
+        sampler = hip_sampler.HipSampler(workload["rows"], workload["vocab"], testing=force_general)
     try:
         sampler.force_general(force_general)
         sampler.upload_logits(workload["logits"])

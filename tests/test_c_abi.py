@@ -31,9 +31,17 @@ def test_header_and_binding_agree():
 
 
 def test_library_exports_every_declared_function():
+    """The shipped library exports the boundary and none of the test hooks; the testing build exports both."""
     library = hip_sampler.load_library()
-    for name in declared_functions() + declared_functions("ncnn_moe_hip_sampler_testing.h"):
+    for name in declared_functions():
         assert getattr(library, name) is not None
+    for name in declared_functions("ncnn_moe_hip_sampler_testing.h"):
+        assert not hasattr(library, name), "%s is a test hook: it belongs in the testing build only" % name
+    exported = subprocess.run(["nm", "-D", "--defined-only", hip_sampler.LIBRARY_PATH], capture_output=True, text=True, check=True).stdout
+    assert "_debug_" not in exported and "stream_only" not in exported
+    testing = hip_sampler.load_testing_library()
+    for name in declared_functions() + declared_functions("ncnn_moe_hip_sampler_testing.h"):
+        assert getattr(testing, name) is not None
 
 
 def test_select_geometry_of_the_benchmark_shapes():

@@ -15,7 +15,7 @@ MAX_ROWS, MAX_VOCAB = 300, 70000
 
 @pytest.fixture(scope="module")
 def sampler():
-    handle = hip_sampler.HipSampler(MAX_ROWS, MAX_VOCAB)
+    handle = hip_sampler.HipSampler(MAX_ROWS, MAX_VOCAB, testing=True)
     yield handle
     handle.close()
 

@@ -15,7 +15,7 @@ STATUS_OF_ANY_ERROR = {hip_sampler.ROW_NO_FINITE_LOGIT, hip_sampler.ROW_INVALID_
 def test_small_rows(general):
     g = golden_util.load()
     print("[case] golden small rows general=%s" % general, flush=True)
-    with hip_sampler.HipSampler(1, 64) as sampler:
+    with hip_sampler.HipSampler(1, 64, testing=general) as sampler:
         sampler.force_general(general)
         for case in range(g["small_vocab"].size):
             vocab = int(g["small_vocab"][case])

@@ -16,7 +16,7 @@ def _announce(text):
 
 @pytest.fixture(scope="module")
 def small_sampler():
-    sampler = hip_sampler.HipSampler(64, 40000)
+    sampler = hip_sampler.HipSampler(64, 40000, testing=True)
     yield sampler
     sampler.close()
 
@@ -264,7 +264,7 @@ def test_cfg2_with_scattered_segments():
     records of segments that ran on other XCDs around the L2): identical results."""
     w = workloads.make_workload("cfg2_topk_topp")
     _announce("cfg2 with scattered segments")
-    with hip_sampler.HipSampler(w["rows"], w["vocab"]) as sampler:
+    with hip_sampler.HipSampler(w["rows"], w["vocab"], testing=True) as sampler:
         grouped = parity_util.run_workload_on_gpu(w, sampler)
         sampler.scatter_segments(True)
         scattered = parity_util.run_workload_on_gpu(w, sampler)
@@ -327,7 +327,7 @@ def _select_rows(params, edge_blocks):
 
 @pytest.fixture(scope="module")
 def batch_sampler():
-    sampler = hip_sampler.HipSampler(320, 110000)
+    sampler = hip_sampler.HipSampler(320, 110000, testing=True)
     yield sampler
     sampler.close()
 

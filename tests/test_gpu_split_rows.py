@@ -45,7 +45,7 @@ def _check(sampler, logits, params, uniforms, context, dtype="f32", scattered=Fa
 
 @pytest.fixture(scope="module")
 def long_sampler():
-    sampler = hip_sampler.HipSampler(255, 262144)
+    sampler = hip_sampler.HipSampler(255, 262144, testing=True)
     yield sampler
     sampler.close()
 
@@ -87,7 +87,7 @@ def test_many_launches_on_one_handle():
     the rows move on independently (a row that is not in a launch keeps its epoch), records are never
     cleared, and every launch must match the oracle."""
     rng = np.random.default_rng(5150)
-    with hip_sampler.HipSampler(96, 60000) as sampler:
+    with hip_sampler.HipSampler(96, 60000, testing=True) as sampler:
         for launch in range(300):
             rows = int(rng.choice([1, 3, 17, 64, 96]))
             vocab = int(rng.choice([10241, 25000, 41000, 60000]))
@@ -102,3 +102,24 @@ def test_many_launches_on_one_handle():
                 cpu = parity_util.run_oracle(data, params, uniforms)
                 parity_util.assert_results_match(gpu, cpu, dtype, "launch %d" % launch)
         sampler.scatter_segments(False)
+
+
+def test_launch_numbers_start_over():
+    """The per-row launch numbers (epochs) that tag the hand-over records run 1 .. 16383 and start over; a
+    serving loop gets there within minutes.  A handle that has records of its first launches in place is
+    set three launches in front of that point and runs eight launches of changing shape, data and window
+    across it: the launch at the last number clears the rows' records, so that what the first launches
+    tagged 1, 2, 3 cannot pass for an entry of the launches that get those numbers again."""
+    rng = np.random.default_rng(909)
+    shapes = [(64, 41000), (17, 60000), (96, 25000), (64, 41000), (3, 60000), (96, 10241), (64, 25000), (17, 41000)]
+    with hip_sampler.HipSampler(96, 60000, testing=True) as sampler:
+        for launch in range(4):  # numbers 1 .. 4: wide windows, so that the records are long
+            logits, params, uniforms = _batch(7000 + launch, 96, 60000)
+            params["top_k"] = 64
+            _check(sampler, logits, params, uniforms, "launch number %d, 96 x 60000" % (launch + 1))
+        sampler.set_row_epochs(hip_sampler.LAST_EPOCH - 2)
+        for launch, (rows, vocab) in enumerate(shapes):
+            logits, params, uniforms = _batch(7100 + launch, rows, vocab)
+            params["top_k"] = rng.choice(np.array([1, 5, 20, 64], dtype=np.uint32), size=rows)
+            _check(sampler, logits, params, uniforms, "launch %d across the restart, %d x %d" % (launch, rows, vocab),
+                   scattered=launch % 3 == 2)
