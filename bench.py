@@ -364,6 +364,65 @@ def bench_generation_loop(args):
     print(json.dumps(line))
 
 
+def bench_scheduler(args):
+    """Micro-batches through the scheduler seam of the C++ host mirror: BatchSampleScheduler over --samplers
+    samplers (2 by default), a worker each, --rows device-resident rows (64 by default) of V = 151,936 fp32 per
+    batch, as many batches in flight as there are samplers, every batch one synchronous device call of the
+    worker that runs it (ncnn_moe_hip_sampler_sample: enqueue, wait, read the results).  Runs the C++ program
+    and wraps its figures in the JSON shape of the other modes; the tokens of the first batch are checked
+    against the CPU oracle."""
+    import subprocess
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+    from ncnn_moe_runtime_amd.workloads import synthetic_model_logits as synthetic_logits
+
+    program = os.path.join(PACKAGE_DIR, "test_session_sampler")
+    if not os.path.exists(program):
+        sys.exit("%s is missing: build it with make -C %s" % (program, PACKAGE_DIR))
+    rows = args.rows if args.rows > 0 else 64
+    vocab, steps, samplers = 151936, args.steps, args.samplers
+    done = subprocess.run([program, "--scheduler-bench", str(rows), str(vocab), str(samplers), str(steps)],
+                          capture_output=True, text=True, timeout=1200)
+    if done.returncode != 0:
+        sys.exit("scheduler bench failed: " + done.stdout[-1000:] + done.stderr[-1000:])
+    fields = done.stdout.split()
+    at = fields.index("first_batch")
+    figures = {fields[i]: fields[i + 1] for i in range(1, at, 2)}
+    first_batch = [tuple(int(v) for v in entry.split(":")) for entry in fields[at + 1:]]
+    seconds = float(figures["seconds"])
+    mismatches = 0
+    checked = min(rows, 16)
+    for i in range(checked):
+        expected = oracle_lib.oracle_sample(synthetic_logits(vocab, i, 0, -1), oracle_lib.OracleRng(5000 + i).uniform(), 0.7, 20, 0.8, 0.0)
+        same = int(expected["token_id"]) == first_batch[i][0] and int(np.float32(expected["probability"]).view(np.uint32)) == first_batch[i][1]
+        mismatches += 0 if same else 1
+    sample = np.stack([synthetic_logits(vocab, i, 0, -1) for i in range(min(rows, 32))])
+    params = np.zeros(sample.shape[0], dtype=oracle_lib.ROW_PARAMS_DTYPE)
+    params["temperature"], params["top_k"], params["top_p"] = 0.7, 20, 0.8
+    start = time.perf_counter()
+    oracle_lib.oracle_sample_batch(sample, params, np.full(sample.shape[0], 0.5, dtype=np.float32), threads=1)
+    cpu_seconds = time.perf_counter() - start
+    bytes_per_step = rows * vocab * 4 + rows * 44
+    line = {
+        "metric": "sampled rows/sec through BatchSampleScheduler, %d samplers, B=%d V=151936 fp32 temp+topk+topp, device-resident logits" % (samplers, rows),
+        "value": rows * steps / seconds, "unit": "rows/s", "n_gpus": 1, "steps": steps, "warmup": 4 * samplers,
+        "ms_per_step": seconds / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "scheduler seam: batches of %d x %d fp32 rows resident in HBM, %d samplers and workers, %d batches in flight; "
+                               "T 0.7, Top-K 20, Top-P 0.8" % (rows, vocab, samplers, samplers),
+                   "entry_point": "BatchSampleScheduler::submit_sample (C++ host mirror) over ncnn_moe_hip_sampler_sample"},
+        "roofline": {"bound": "hbm", "achieved": bytes_per_step * steps / seconds / 1e9, "peak": HBM_PEAK_BYTES_PER_S / 1e9,
+                     "unit": "GB/s", "frac": bytes_per_step * steps / seconds / HBM_PEAK_BYTES_PER_S, "traffic": None,
+                     "kernel": "split_select_kernel, wall clock of the whole loop (host threads, synchronous device calls)",
+                     "algorithmic_bytes_per_launch": bytes_per_step},
+        "parity": {"rows_checked": checked, "token_or_probability_mismatches": mismatches},
+        "detail": {"device_calls": int(figures["device_calls"]), "device_calls_begun_while_another_ran": int(figures["overlapped_device_calls"])},
+        "cpu_baseline": {"value": sample.shape[0] / cpu_seconds, "unit": "rows/s", "cores": 1, "kind": "port",
+                         "sample": "%d rows of the same logits through the CPU oracle" % sample.shape[0]},
+    }
+    print(json.dumps(line))
+
+
 def bench_timeline(args):
     """Where the time of a split-row launch goes: the library built with wall-clock stamps in the split
     kernel (make -C ncnn-moe-runtime_amd timeline) runs bursts of 12 launches over rotated logits buffers;
@@ -519,6 +578,7 @@ def main():
                              "so leave it off under a kernel trace)")
     parser.add_argument("--router-score", default="sqrt_softplus", choices=["softmax", "sigmoid", "sqrt_softplus"],
                         help="score function of --workload router_dispatch")
+    parser.add_argument("--samplers", type=int, default=2, help="samplers (and workers) of --workload scheduler")
     parser.add_argument("--drafts", type=int, default=5, help="drafted tokens per step of --workload speculative_verify")
     parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
     parser.add_argument("--cpu-rows", type=int, default=64)
@@ -548,6 +608,9 @@ def main():
         return
     if args.workload == "generation_loop":
         bench_generation_loop(args)
+        return
+    if args.workload == "scheduler":
+        bench_scheduler(args)
         return
     if args.workload == "speculative_verify":
         return bench_speculative_verify(args, hip_sampler)

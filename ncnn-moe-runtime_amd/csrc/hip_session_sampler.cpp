@@ -9,6 +9,7 @@
 #include <cmath>
 #include <condition_variable>
 #include <deque>
+#include <limits>
 #include <thread>
 #include <unordered_map>
 
@@ -113,6 +114,12 @@ struct HipSampler::Impl
     std::vector<ncnn_moe_sample_result> results;
     uint32_t resident_rows = 0; // rows x vocab the logits buffer was last laid out for
     uint32_t resident_vocab = 0;
+    bool resident_overwritten = false; // a sample() of host logits has used the buffer since
+
+    // The verification step over the 2 D + 1 rows the logits buffer holds.  The caller holds the sampler's mutex.
+    Result<SpeculativeVerification> verify_rows(
+        std::span<const int32_t> proposed_token_ids, const SamplingOptions& options, std::span<const float> uniforms,
+        uint32_t& draws_consumed, uint32_t* accept_draws, bool* failed_behind_an_empty_accept_loop);
 
     // Samples the rows the logits buffer holds.  The caller holds the sampler's mutex.
     std::vector<Result<BatchSampledToken>> sample_rows(
@@ -181,8 +188,10 @@ std::vector<Result<BatchSampledToken>> HipSampler::sample(
         impl.handle, impl.staging.data(), NCNN_MOE_LOGITS_F32, static_cast<uint32_t>(rows), static_cast<uint32_t>(vocab), vocab);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return every_row<BatchSampledToken>(rows, error_of_call(rc, impl.handle));
-    impl.resident_rows = static_cast<uint32_t>(rows);
-    impl.resident_vocab = static_cast<uint32_t>(vocab);
+    // the buffer now holds this call's rows: what device_logits() laid out before is gone
+    impl.resident_rows = 0;
+    impl.resident_vocab = 0;
+    impl.resident_overwritten = true;
     return impl.sample_rows(rows, options, uniforms, stop_tokens, draw_consumed);
 }
 
@@ -190,6 +199,7 @@ std::vector<Result<BatchSampledToken>> HipSampler::Impl::sample_rows(
     size_t rows, std::span<const SamplingOptions> options, std::span<const float> uniforms,
     std::span<const std::vector<int32_t>> stop_tokens, std::vector<uint8_t>& draw_consumed)
 {
+    draw_consumed.assign(rows, 0);
     params.resize(rows);
     stop_ids.clear();
     for (size_t row = 0; row < rows; ++row)
@@ -254,21 +264,105 @@ Result<DeviceLogitsRows> HipSampler::device_logits(uint32_t rows, uint32_t vocab
     out.bf16 = bf16;
     impl_->resident_rows = rows;
     impl_->resident_vocab = vocab;
+    impl_->resident_overwritten = false;
+    return out;
+}
+
+Result<DeviceLogitsRows> HipSampler::upload_resident(std::span<const std::span<const float>> logits)
+{
+    const size_t rows = logits.size();
+    if (rows == 0 || logits[0].empty())
+        return invalid_argument("cannot sample empty logits");
+    if (rows > impl_->max_rows)
+        return invalid_argument("sample batch exceeds the sampler's max_rows");
+    const size_t vocab = logits[0].size();
+    for (const std::span<const float>& row : logits)
+    {
+        if (row.size() != vocab)
+            return invalid_argument("sample batch rows differ in length");
+    }
+    if (vocab > impl_->max_vocab)
+        return invalid_argument("logits exceed the sampler's max_vocab");
+    const std::lock_guard<std::mutex> lock(mutex_);
+    Impl& impl = *impl_;
+    impl.staging.resize(rows * vocab);
+    for (size_t row = 0; row < rows; ++row)
+        std::copy(logits[row].begin(), logits[row].end(), impl.staging.begin() + row * vocab);
+    int rc = ncnn_moe_hip_sampler_upload_logits(
+        impl.handle, impl.staging.data(), NCNN_MOE_LOGITS_F32, static_cast<uint32_t>(rows), static_cast<uint32_t>(vocab), vocab);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return error_of_call(rc, impl.handle);
+    DeviceLogitsRows out;
+    rc = ncnn_moe_hip_sampler_logits_buffer(
+        impl.handle, NCNN_MOE_LOGITS_F32, static_cast<uint32_t>(rows), static_cast<uint32_t>(vocab), &out.data, &out.row_stride);
+    if (rc != NCNN_MOE_SAMPLER_SUCCESS)
+        return error_of_call(rc, impl.handle);
+    out.rows = static_cast<uint32_t>(rows);
+    out.vocab = static_cast<uint32_t>(vocab);
+    impl.resident_rows = out.rows;
+    impl.resident_vocab = out.vocab;
+    impl.resident_overwritten = false;
     return out;
 }
 
 std::vector<Result<BatchSampledToken>> HipSampler::sample_resident(
     std::span<const SamplingOptions> options, std::span<const float> uniforms,
-    std::span<const std::vector<int32_t>> stop_tokens, std::vector<uint8_t>& draw_consumed)
+    std::span<const std::vector<int32_t>> stop_tokens, std::vector<uint8_t>& draw_consumed,
+    std::span<const uint32_t> device_rows)
 {
     const size_t rows = options.size();
     draw_consumed.assign(rows, 0);
-    if (rows == 0 || uniforms.size() != rows || (!stop_tokens.empty() && stop_tokens.size() != rows))
+    if (rows == 0 || uniforms.size() != rows || (!stop_tokens.empty() && stop_tokens.size() != rows) ||
+        (!device_rows.empty() && device_rows.size() != rows))
         return every_row<BatchSampledToken>(rows, invalid_argument("sample batch operands differ in length"));
     const std::lock_guard<std::mutex> lock(mutex_);
-    if (rows != impl_->resident_rows)
-        return every_row<BatchSampledToken>(rows, invalid_argument("sample batch differs from the rows laid out by device_logits"));
-    return impl_->sample_rows(rows, options, uniforms, stop_tokens, draw_consumed);
+    if (impl_->resident_overwritten)
+        return every_row<BatchSampledToken>(rows, invalid_argument("the rows laid out by device_logits were overwritten by a sample() of host logits"));
+    if (device_rows.empty())
+    {
+        if (rows != impl_->resident_rows)
+            return every_row<BatchSampledToken>(rows, invalid_argument("sample batch differs from the rows laid out by device_logits"));
+        return impl_->sample_rows(rows, options, uniforms, stop_tokens, draw_consumed);
+    }
+    // Named rows, in any order: the device call covers rows 0 .. the largest one named.  A row that nobody
+    // named carries options that fail validation at once (its workgroups leave before they look at a logit)
+    // and its result is dropped.
+    uint32_t covered = 0;
+    for (uint32_t row : device_rows)
+    {
+        if (row >= impl_->resident_rows)
+            return every_row<BatchSampledToken>(rows, invalid_argument("sample request names a row beyond those laid out by device_logits"));
+        covered = std::max(covered, row + 1u);
+    }
+    std::vector<uint8_t> named(covered, 0);
+    for (uint32_t row : device_rows)
+    {
+        if (named[row])
+            return every_row<BatchSampledToken>(rows, invalid_argument("sample batch names a device row twice"));
+        named[row] = 1;
+    }
+    SamplingOptions unused;
+    unused.temperature = std::numeric_limits<float>::quiet_NaN();
+    std::vector<SamplingOptions> all_options(covered, unused);
+    std::vector<float> all_uniforms(covered, 0.0f);
+    std::vector<std::vector<int32_t>> all_stop_tokens(stop_tokens.empty() ? 0 : covered);
+    for (size_t i = 0; i < rows; ++i)
+    {
+        all_options[device_rows[i]] = options[i];
+        all_uniforms[device_rows[i]] = uniforms[i];
+        if (!stop_tokens.empty())
+            all_stop_tokens[device_rows[i]] = stop_tokens[i];
+    }
+    std::vector<uint8_t> all_consumed;
+    std::vector<Result<BatchSampledToken>> all = impl_->sample_rows(covered, all_options, all_uniforms, all_stop_tokens, all_consumed);
+    std::vector<Result<BatchSampledToken>> out;
+    out.reserve(rows);
+    for (size_t i = 0; i < rows; ++i)
+    {
+        out.push_back(all[device_rows[i]]);
+        draw_consumed[i] = all_consumed.size() > device_rows[i] ? all_consumed[device_rows[i]] : 0;
+    }
+    return out;
 }
 
 Result<std::vector<TokenProbability>> HipSampler::distribution(std::span<const float> logits, const SamplingOptions& options)
@@ -307,11 +401,14 @@ Result<SpeculativeVerification> HipSampler::verify_speculative(
     const SamplingOptions& options,
     std::span<const float> uniforms,
     uint32_t& draws_consumed,
-    uint32_t* accept_draws)
+    uint32_t* accept_draws,
+    bool* failed_behind_an_empty_accept_loop)
 {
     draws_consumed = 0;
     if (accept_draws != nullptr)
         *accept_draws = 0;
+    if (failed_behind_an_empty_accept_loop != nullptr)
+        *failed_behind_an_empty_accept_loop = false;
     const size_t drafts = proposed_token_ids.size();
     if (drafts == 0 || drafts > NCNN_MOE_MAX_DRAFT_TOKENS)
         return invalid_argument("speculative verification takes 1 to 16 proposed tokens");
@@ -343,21 +440,63 @@ Result<SpeculativeVerification> HipSampler::verify_speculative(
         std::copy(target_logits[row].begin(), target_logits[row].end(), impl.staging.begin() + row * vocab);
     for (size_t row = 0; row < drafts; ++row)
         std::copy(draft_logits[row].begin(), draft_logits[row].end(), impl.staging.begin() + (drafts + 1 + row) * vocab);
-    int rc = ncnn_moe_hip_sampler_upload_logits(
+    const int rc = ncnn_moe_hip_sampler_upload_logits(
         impl.handle, impl.staging.data(), NCNN_MOE_LOGITS_F32, static_cast<uint32_t>(rows), static_cast<uint32_t>(vocab), vocab);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
         return error_of_call(rc, impl.handle);
+    impl.resident_rows = 0;
+    impl.resident_vocab = 0;
+    impl.resident_overwritten = true;
+    return impl.verify_rows(proposed_token_ids, options, uniforms, draws_consumed, accept_draws, failed_behind_an_empty_accept_loop);
+}
+
+Result<SpeculativeVerification> HipSampler::verify_speculative_resident(
+    std::span<const int32_t> proposed_token_ids, const SamplingOptions& options, std::span<const float> uniforms,
+    uint32_t& draws_consumed, uint32_t* accept_draws, bool* failed_behind_an_empty_accept_loop)
+{
+    draws_consumed = 0;
+    if (accept_draws != nullptr)
+        *accept_draws = 0;
+    if (failed_behind_an_empty_accept_loop != nullptr)
+        *failed_behind_an_empty_accept_loop = false;
+    const size_t drafts = proposed_token_ids.size();
+    if (drafts == 0 || drafts > NCNN_MOE_MAX_DRAFT_TOKENS)
+        return invalid_argument("speculative verification takes 1 to 16 proposed tokens");
+    if (uniforms.size() != drafts + 1)
+        return invalid_argument("speculative verification operands differ in length");
+    const std::lock_guard<std::mutex> lock(mutex_);
+    if (impl_->resident_overwritten)
+        return invalid_argument("the rows laid out by device_logits were overwritten by a sample() of host logits");
+    if (impl_->resident_rows != 2 * drafts + 1)
+        return invalid_argument("speculative verification needs the 2 D + 1 rows of its step laid out by device_logits");
+    return impl_->verify_rows(proposed_token_ids, options, uniforms, draws_consumed, accept_draws, failed_behind_an_empty_accept_loop);
+}
+
+Result<SpeculativeVerification> HipSampler::Impl::verify_rows(
+    std::span<const int32_t> proposed_token_ids, const SamplingOptions& options, std::span<const float> uniforms,
+    uint32_t& draws_consumed, uint32_t* accept_draws, bool* failed_behind_an_empty_accept_loop)
+{
+    const size_t drafts = proposed_token_ids.size();
     const ncnn_moe_sample_params p{options.temperature, options.top_k, options.top_p, options.min_p, 0, 0};
     std::vector<float> accepted_probabilities(drafts, 0.0f);
     ncnn_moe_verify_result verified{};
-    rc = ncnn_moe_hip_sampler_speculative_verify(
-        impl.handle, static_cast<uint32_t>(drafts), &p, proposed_token_ids.data(), uniforms.data(),
+    const int rc = ncnn_moe_hip_sampler_speculative_verify(
+        handle, static_cast<uint32_t>(drafts), &p, proposed_token_ids.data(), uniforms.data(),
         accepted_probabilities.data(), &verified);
     if (rc != NCNN_MOE_SAMPLER_SUCCESS)
-        return error_of_call(rc, impl.handle);
+        return error_of_call(rc, handle);
     draws_consumed = verified.accept_draws + verified.final_draw_consumed;
     if (accept_draws != nullptr)
         *accept_draws = verified.accept_draws;
+    if (verified.status != NCNN_MOE_VERIFY_OK && failed_behind_an_empty_accept_loop != nullptr && verified.accepted == 0)
+    {
+        // The accept loop fails at a position before that position's draw; once a draw has rejected the first
+        // proposal (sampled rows), or the first proposal differed from the target's choice (greedy rows), the
+        // loop has ended and what failed is the draw of the next token.
+        const bool sampled_row = options.temperature != 0.0f;
+        const bool residual_stage = verified.status == NCNN_MOE_VERIFY_RESIDUAL_EMPTY || verified.status == NCNN_MOE_VERIFY_RESIDUAL_FAILED;
+        *failed_behind_an_empty_accept_loop = residual_stage || (sampled_row && verified.status == NCNN_MOE_VERIFY_ROW_ERROR && verified.accept_draws > 0);
+    }
     switch (verified.status)
     {
     case NCNN_MOE_VERIFY_OK:
@@ -463,8 +602,10 @@ Result<SpeculativeVerification> SamplingSession::verify_speculative(
         uniforms[i] = uniform_ahead(i);
     uint32_t draws_consumed = 0;
     uint32_t accept_draws = 0;
-    auto verified = sampler_->verify_speculative(target_rows, draft_rows, proposed_token_ids, options, uniforms, draws_consumed, &accept_draws);
-    if (verified && verified.value().accepted.empty() && !state_cache_transactions)
+    bool failed_behind_an_empty_accept_loop = false;
+    auto verified = sampler_->verify_speculative(target_rows, draft_rows, proposed_token_ids, options, uniforms, draws_consumed, &accept_draws,
+                                                 &failed_behind_an_empty_accept_loop);
+    if (!state_cache_transactions && ((verified && verified.value().accepted.empty()) || failed_behind_an_empty_accept_loop))
     {
         // src/engine/session.cpp:843-857: nothing accepted and no cache transactions to keep part of the
         // step: roll back and leave speculative mode before the next token is drawn.  The device computed
@@ -560,18 +701,27 @@ std::vector<Result<BatchSampledToken>> SessionBatchSampler::sample_resident(
     std::vector<std::unique_lock<std::mutex>> locks;
     if (!lock_in_pointer_order(std::move(order), locks))
         return every_row<BatchSampledToken>(rows, invalid_argument("sample batch contains duplicate sessions"));
+    // either every request names its device row, or none does and request i samples row i
+    size_t named_rows = 0;
+    for (const SampleBatchRequest& request : requests)
+        named_rows += request.device_row != SampleBatchRequest::kRowByPosition ? 1 : 0;
+    if (named_rows != 0 && named_rows != rows)
+        return every_row<BatchSampledToken>(rows, invalid_argument("sample batch names the device row of some requests only"));
     std::vector<SamplingOptions> options;
     std::vector<float> uniforms;
     std::vector<std::vector<int32_t>> stop_tokens;
+    std::vector<uint32_t> device_rows;
     for (const SampleBatchRequest& request : requests)
     {
         options.push_back(request.sampling);
         uniforms.push_back(request.session->uniform_ahead(0));
         stop_tokens.push_back(request.stop_tokens);
+        if (named_rows != 0)
+            device_rows.push_back(request.device_row);
     }
     std::vector<uint8_t> draw_consumed;
     const SampleTimer timer;
-    auto sampled = sampler->sample_resident(options, uniforms, stop_tokens, draw_consumed);
+    auto sampled = sampler->sample_resident(options, uniforms, stop_tokens, draw_consumed, device_rows);
     for (size_t i = 0; i < rows; ++i)
     {
         timer.charge(requests[i].session->statistics_, sampled[i] ? 1 : 0);
@@ -588,13 +738,16 @@ class BatchSampleScheduler::Implementation
 public:
     using Results = std::vector<Result<BatchSampledToken>>;
 
-    Implementation(HipSamplerPtr sampler, const SampleSchedulerOptions& options)
-        : sampler_(std::move(sampler)), window_(options.cross_call_window_microseconds)
+    Implementation(std::vector<HipSamplerPtr> samplers, const SampleSchedulerOptions& options)
+        : samplers_(std::move(samplers)), window_(options.cross_call_window_microseconds)
     {
+        spin_microseconds_ = options.worker_spin_microseconds;
+        if (samplers_.empty())
+            samplers_.push_back(nullptr); // (a scheduler without a sampler answers every request with InternalError)
         const uint32_t hardware_threads = std::max(1u, std::thread::hardware_concurrency());
         worker_count_ = options.worker_count == 0 ? std::min(4u, hardware_threads) : std::min(options.worker_count, 1024u);
         max_collected_ = options.cross_call_max_batch_size != 0 ? options.cross_call_max_batch_size
-                                                                : (sampler_ ? sampler_->max_rows() : 1u);
+                                                                : (samplers_.front() ? samplers_.front()->max_rows() : 1u);
         for (uint32_t i = 0; i < worker_count_; ++i)
             workers_.emplace_back([this] { worker_loop(); });
         if (window_ != 0)
@@ -642,6 +795,22 @@ public:
         std::sort(named.begin(), named.end());
         if (std::adjacent_find(named.begin(), named.end()) != named.end())
             return reject("sample batch contains duplicate sessions");
+        // A batch is of one kind.  Device-resident requests sample rows of ONE sampler's buffer, which they all
+        // name; a request that names no row takes the row of its place in the batch, so such a batch runs as it
+        // was submitted and is never merged with others.
+        const bool resident = requests.front().logits == nullptr;
+        bool rows_named = true;
+        for (const SampleBatchRequest& request : requests)
+        {
+            if ((request.logits == nullptr) != resident)
+                return reject("sample batch mixes host logits and device-resident rows");
+            if (resident && request.resident_sampler != requests.front().resident_sampler)
+                return reject("sample batch names device rows of several samplers");
+            if (resident && request.resident_sampler >= samplers_.size())
+                return reject("sample request names a sampler the scheduler does not have");
+            rows_named = rows_named && request.device_row != SampleBatchRequest::kRowByPosition;
+        }
+        const bool collectable = requests.size() == 1 && collector_.joinable() && (!resident || rows_named);
         {
             const std::lock_guard<std::mutex> lock(mutex_);
             // the place of every request in its Session's order is fixed here, whichever way it travels
@@ -654,17 +823,21 @@ public:
                 order.push_back(next_ticket_);
                 tickets.push_back(next_ticket_++);
             }
-            if (requests.size() == 1 && collector_.joinable())
+            if (collectable)
             {
                 singles_.push_back(Single{std::move(requests.front()), tickets.front(), std::move(promise), std::chrono::steady_clock::now()});
                 single_ready_.notify_one();
                 return future;
             }
             queue_.push_back(Batch{std::move(requests), std::move(tickets), {}, std::move(promise)});
+            queue_changes_.fetch_add(1, std::memory_order_release);
         }
         work_ready_.notify_one();
         return future;
     }
+
+    size_t sampler_count() const noexcept { return samplers_.size(); }
+    HipSamplerPtr sampler(size_t index) const { return index < samplers_.size() ? samplers_[index] : nullptr; }
 
     SampleSchedulerStatistics statistics() const noexcept
     {
@@ -679,6 +852,7 @@ public:
         out.cross_call_collected_requests = collected_requests_.load(std::memory_order_relaxed);
         out.cross_call_collection_timeouts = collection_timeouts_.load(std::memory_order_relaxed);
         out.device_calls = device_calls_.load(std::memory_order_relaxed);
+        out.overlapped_device_calls = overlapped_calls_.load(std::memory_order_relaxed);
         out.worker_count = worker_count_;
         return out;
     }
@@ -709,6 +883,14 @@ private:
         }
     }
 
+    // Host-logits batches keep off the first sampler while there are others: its buffer is where a decode
+    // step that knows of one sampler only (resident_sampler 0) leaves its rows, and a sample() of host
+    // logits would overwrite them.
+    size_t host_lane(uint64_t turn) const
+    {
+        return samplers_.size() > 1 ? 1 + static_cast<size_t>(turn % (samplers_.size() - 1)) : 0;
+    }
+
     // mutex_ held.  The first batch every request of which is the oldest unfinished one of its Session:
     // requests of a Session run in the order of their submission and never two at a time.  (A batch waits
     // only for requests with smaller tickets, so some batch can always run.)
@@ -734,6 +916,25 @@ private:
         for (;;)
         {
             Batch batch;
+            if (spin_microseconds_ != 0)
+            {
+                // look for work without sleeping for a while: queue_changes_ moves on with every submission and
+                // every completed batch, so the mutex is taken only when there is something new to look at
+                const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(spin_microseconds_);
+                uint64_t seen = queue_changes_.load(std::memory_order_acquire) - 1;
+                while (batch.requests.empty() && std::chrono::steady_clock::now() < give_up)
+                {
+                    const uint64_t now = queue_changes_.load(std::memory_order_acquire);
+                    if (now == seen)
+                        continue;
+                    seen = now;
+                    const std::lock_guard<std::mutex> lock(mutex_);
+                    if (stopping_)
+                        break;
+                    take_runnable_locked(batch);
+                }
+            }
+            if (batch.requests.empty())
             {
                 std::unique_lock<std::mutex> lock(mutex_);
                 work_ready_.wait(lock, [&] { return take_runnable_locked(batch) || (stopping_ && queue_.empty() && singles_.empty() && !collecting_); });
@@ -743,9 +944,16 @@ private:
             Results results;
             try
             {
+                // a device-resident batch runs on the sampler that holds its rows; a batch of host logits on the
+                // next sampler in turn, so that batches which different workers run at once meet on different ones
                 const bool resident = batch.requests.front().logits == nullptr;
-                results = resident ? SessionBatchSampler::sample_resident(sampler_, batch.requests)
-                                   : SessionBatchSampler::sample(sampler_, batch.requests);
+                const size_t lane = resident ? batch.requests.front().resident_sampler
+                                             : host_lane(next_host_lane_.fetch_add(1, std::memory_order_relaxed));
+                if (running_calls_.fetch_add(1, std::memory_order_acq_rel) != 0)
+                    overlapped_calls_.fetch_add(1, std::memory_order_relaxed);
+                results = resident ? SessionBatchSampler::sample_resident(samplers_[lane], batch.requests)
+                                   : SessionBatchSampler::sample(samplers_[lane], batch.requests);
+                running_calls_.fetch_sub(1, std::memory_order_acq_rel);
                 device_calls_.fetch_add(1, std::memory_order_relaxed);
             }
             catch (const std::exception& error)
@@ -762,6 +970,7 @@ private:
                     if (order->second.empty())
                         session_order_.erase(order);
                 }
+                queue_changes_.fetch_add(1, std::memory_order_release);
             }
             work_ready_.notify_all(); // a batch that waited for one of these Sessions may run now
             if (batch.single_promises.empty())
@@ -812,8 +1021,13 @@ private:
                 for (auto single = singles_.begin(); single != singles_.end() && batch.requests.size() < max_collected_;)
                 {
                     const bool resident = single->request.logits == nullptr;
-                    const bool same_kind = batch.requests.empty() || resident == (batch.requests.front().logits == nullptr);
-                    if (!same_kind || std::find(taken.begin(), taken.end(), single->request.session) != taken.end())
+                    const bool same_kind = batch.requests.empty() ||
+                        (resident == (batch.requests.front().logits == nullptr) &&
+                         (!resident || single->request.resident_sampler == batch.requests.front().resident_sampler));
+                    bool row_taken = false;
+                    for (const SampleBatchRequest& other : batch.requests)
+                        row_taken = row_taken || (resident && other.device_row == single->request.device_row);
+                    if (!same_kind || row_taken || std::find(taken.begin(), taken.end(), single->request.session) != taken.end())
                     {
                         ++single;
                         continue;
@@ -833,13 +1047,19 @@ private:
                 else
                     collection_timeouts_.fetch_add(1, std::memory_order_relaxed);
                 queue_.push_back(std::move(batch));
+                queue_changes_.fetch_add(1, std::memory_order_release);
                 collecting_ = !singles_.empty();
             }
             work_ready_.notify_one();
         }
     }
 
-    HipSamplerPtr sampler_;
+    std::vector<HipSamplerPtr> samplers_;
+    std::atomic<uint64_t> next_host_lane_{0};
+    std::atomic<uint64_t> queue_changes_{1};
+    uint32_t spin_microseconds_ = 0;
+    std::atomic<uint32_t> running_calls_{0};
+    std::atomic<uint64_t> overlapped_calls_{0};
     uint32_t window_ = 0;
     uint32_t worker_count_ = 1;
     size_t max_collected_ = 1;
@@ -860,8 +1080,23 @@ private:
 };
 
 BatchSampleScheduler::BatchSampleScheduler(HipSamplerPtr sampler, const SampleSchedulerOptions& options)
-    : implementation_(std::make_unique<Implementation>(std::move(sampler), options))
+    : implementation_(std::make_unique<Implementation>(std::vector<HipSamplerPtr>{std::move(sampler)}, options))
 {
+}
+
+BatchSampleScheduler::BatchSampleScheduler(std::vector<HipSamplerPtr> samplers, const SampleSchedulerOptions& options)
+    : implementation_(std::make_unique<Implementation>(std::move(samplers), options))
+{
+}
+
+size_t BatchSampleScheduler::sampler_count() const noexcept
+{
+    return implementation_->sampler_count();
+}
+
+HipSamplerPtr BatchSampleScheduler::sampler(size_t index) const
+{
+    return implementation_->sampler(index);
 }
 
 BatchSampleScheduler::~BatchSampleScheduler() = default;

@@ -213,12 +213,21 @@ public:
     Result<DeviceLogitsRows> device_logits(uint32_t rows, uint32_t vocab, bool bf16 = false);
 
     // sample() over the rows last laid out by device_logits(); the rows must be complete in device
-    // memory when this is called.
+    // memory when this is called.  device_rows empty: entry i of the operands samples row i (as many
+    // entries as rows were laid out).  Otherwise entry i samples row device_rows[i], in any order and for
+    // any subset of the rows; the rows that no entry names are left alone.  A sample() of host logits in
+    // between overwrites the buffer: the next sample_resident() is then refused until device_logits() has
+    // laid the rows out again.
     std::vector<Result<BatchSampledToken>> sample_resident(
         std::span<const SamplingOptions> options,
         std::span<const float> uniforms,
         std::span<const std::vector<int32_t>> stop_tokens,
-        std::vector<uint8_t>& draw_consumed);
+        std::vector<uint8_t>& draw_consumed,
+        std::span<const uint32_t> device_rows = {});
+
+    // Copies host rows into the buffer and lays it out for them, as a decode step that runs on the CPU would
+    // hand its logits over (ncnn_moe_hip_sampler_upload_logits): sample_resident() then samples them.
+    Result<DeviceLogitsRows> upload_resident(std::span<const std::span<const float>> logits);
 
     // sampling_distribution for one row.
     Result<std::vector<TokenProbability>> distribution(std::span<const float> logits, const SamplingOptions& options);
@@ -234,7 +243,22 @@ public:
         const SamplingOptions& options,
         std::span<const float> uniforms,
         uint32_t& draws_consumed,
-        uint32_t* accept_draws = nullptr); // of draws_consumed, those of the accept tests (the rest is the last token's draw)
+        uint32_t* accept_draws = nullptr, // of draws_consumed, those of the accept tests (the rest is the last token's draw)
+        // set when the step failed only after its accept loop had ended with nothing accepted, i.e. while the
+        // next token was drawn: a caller without cache transactions leaves speculative mode in front of that
+        // draw (src/engine/session.cpp:843-857) and never sees the failure
+        bool* failed_behind_an_empty_accept_loop = nullptr);
+
+    // The same over rows that are already in the sampler's buffer: rows 0 .. D the target's logits after the
+    // anchor and after each of the D proposed tokens, rows D + 1 .. 2 D the draft rows those tokens were
+    // sampled from (laid out by device_logits(2 D + 1, vocab)).
+    Result<SpeculativeVerification> verify_speculative_resident(
+        std::span<const int32_t> proposed_token_ids,
+        const SamplingOptions& options,
+        std::span<const float> uniforms,
+        uint32_t& draws_consumed,
+        uint32_t* accept_draws = nullptr,
+        bool* failed_behind_an_empty_accept_loop = nullptr);
 
 private:
     HipSampler();
@@ -317,10 +341,19 @@ Result<SamplingSessionPtr> create_sampling_session(const HipSamplerPtr& sampler,
 
 struct SampleBatchRequest
 {
+    static constexpr uint32_t kRowByPosition = UINT32_MAX;
+
     SamplingSession* session = nullptr;
     const LogitsOutput* logits = nullptr; // null for a Session in SampledToken mode: its row is in the device buffer
     SamplingOptions sampling;
     std::vector<int32_t> stop_tokens; // GenerationOptions::stop_tokens
+    // SampledToken mode: the row of the device buffer that holds this Session's logits (the place the decode
+    // step gave it).  kRowByPosition: request i of a batch samples row i, which fits a batch that is
+    // submitted whole, in the decode step's order.  A request that travels alone (one serving thread per
+    // Session, collected across calls by the scheduler) names its row.
+    uint32_t device_row = kRowByPosition;
+    // ... and, for a scheduler over several samplers, the one whose buffer holds the row
+    uint32_t resident_sampler = 0;
 };
 
 class SessionBatchSampler
@@ -331,8 +364,9 @@ public:
     // rows of different lengths with InvalidArgument for every row.
     static std::vector<Result<BatchSampledToken>> sample(const HipSamplerPtr& sampler, std::span<const SampleBatchRequest> requests);
 
-    // The same for Sessions in SampledToken mode: request i samples row i of the rows last laid out by
-    // HipSampler::device_logits (the decode step wrote them there); every request's logits must be null.
+    // The same for Sessions in SampledToken mode: a request samples its device_row (or, with kRowByPosition in
+    // every request, request i row i) of the rows last laid out by HipSampler::device_logits (the decode
+    // step wrote them there); every request's logits must be null.
     static std::vector<Result<BatchSampledToken>> sample_resident(const HipSamplerPtr& sampler, std::span<const SampleBatchRequest> requests);
 };
 
@@ -342,6 +376,10 @@ struct SampleSchedulerOptions
     uint32_t worker_count = 0;                     // 0: min(4, hardware threads), src/engine/scheduler.cpp:87
     uint32_t cross_call_window_microseconds = 200; // zero disables cross-call collection
     uint32_t cross_call_max_batch_size = 0;        // 0: the sampler's max_rows
+    // An idle worker looks for work this long before it goes to sleep on the queue's condition variable: waking a
+    // sleeping thread costs more than a whole device call of the select path (tens of microseconds against 15 to
+    // 30), so a serving loop that submits batch after batch keeps its workers awake in between.  0: sleep at once.
+    uint32_t worker_spin_microseconds = 100;
 };
 
 struct SampleSchedulerStatistics
@@ -356,6 +394,7 @@ struct SampleSchedulerStatistics
     uint64_t cross_call_collected_requests = 0;
     uint64_t cross_call_collection_timeouts = 0;
     uint64_t device_calls = 0;
+    uint64_t overlapped_device_calls = 0; // device calls that began while another one of this scheduler was running
     uint32_t worker_count = 0;
 };
 
@@ -370,12 +409,20 @@ class BatchSampleScheduler
 {
 public:
     explicit BatchSampleScheduler(HipSamplerPtr sampler, const SampleSchedulerOptions& options = {});
+    // Several samplers, each with device buffers and a stream of its own: batches that different workers
+    // run at the same time go to different samplers and overlap on the GPU (the scheduler's workers run
+    // batches concurrently, src/engine/scheduler.cpp:87-104, :257-270).  A batch of host logits takes the
+    // next sampler in turn; a device-resident batch runs on the sampler its requests name
+    // (SampleBatchRequest::resident_sampler: the one into whose buffer the decode step wrote).
+    explicit BatchSampleScheduler(std::vector<HipSamplerPtr> samplers, const SampleSchedulerOptions& options = {});
     ~BatchSampleScheduler();
     BatchSampleScheduler(const BatchSampleScheduler&) = delete;
     BatchSampleScheduler& operator=(const BatchSampleScheduler&) = delete;
 
     [[nodiscard]] std::future<std::vector<Result<BatchSampledToken>>> submit_sample(std::vector<SampleBatchRequest> requests);
     [[nodiscard]] SampleSchedulerStatistics statistics() const noexcept;
+    [[nodiscard]] size_t sampler_count() const noexcept;
+    [[nodiscard]] HipSamplerPtr sampler(size_t index) const; // null beyond sampler_count()
 
 private:
     class Implementation;

@@ -692,10 +692,13 @@ static void test_sampled_token_mode(const HipSamplerPtr& sampler)
             requests.push_back(SampleBatchRequest{resident[i].get(), nullptr, options, {}});
             full_requests.push_back(SampleBatchRequest{full[i].get(), &host_rows[i], options, {}});
         }
-        auto expected = SessionBatchSampler::sample(sampler, full_requests);
-        // the upload of the full-logits batch replaced the buffer's rows with the same values
         auto got = SessionBatchSampler::sample_resident(sampler, requests);
+        auto expected = SessionBatchSampler::sample(sampler, full_requests);
         check(got.size() == count && expected.size() == count);
+        // that sample() of host logits used the buffer: the rows laid out before are gone, and say so
+        auto stale = SessionBatchSampler::sample_resident(sampler, requests);
+        check(stale.size() == count && !stale[0] && stale[0].error().code == ErrorCode::InvalidArgument &&
+              stale[0].error().message.find("overwritten") != std::string::npos);
         for (uint32_t i = 0; i < count; ++i)
         {
             check(static_cast<bool>(got[i]) && static_cast<bool>(expected[i]));
@@ -709,6 +712,217 @@ static void test_sampled_token_mode(const HipSamplerPtr& sampler)
     check(mixed.size() == 1 && !mixed[0] && mixed[0].error().code == ErrorCode::InvalidArgument);
     auto wrong = SessionBatchSampler::sample_resident(sampler, std::vector<SampleBatchRequest>{SampleBatchRequest{full[0].get(), nullptr, options, {}}});
     check(wrong.size() == 1 && !wrong[0] && wrong[0].error().code == ErrorCode::InvalidArgument);
+}
+
+// SampledToken-mode requests that travel alone through the scheduler, one serving thread per Session, in an
+// order that has nothing to do with the decode step's: each names the device row that holds its logits.  Tokens
+// per Session against SessionBatchSampler::sample_resident on the whole batch in layout order.
+static void test_resident_requests_through_the_scheduler(const HipSamplerPtr& sampler)
+{
+    const uint32_t vocab = 4001, count = 8;
+    SamplingOptions options;
+    options.temperature = 0.9f;
+    options.top_k = 30;
+    options.top_p = 0.95f;
+    std::vector<SamplingSessionPtr> scheduled, direct;
+    for (uint32_t i = 0; i < count; ++i)
+    {
+        scheduled.push_back(create_sampling_session(sampler, SamplingSessionOptions{900 + i, LogitsOutputMode::SampledToken}).value());
+        direct.push_back(create_sampling_session(sampler, SamplingSessionOptions{900 + i, LogitsOutputMode::SampledToken}).value());
+    }
+    SampleSchedulerOptions scheduler_options;
+    scheduler_options.worker_count = 4;
+    scheduler_options.cross_call_window_microseconds = 3000;
+    BatchSampleScheduler scheduler(sampler, scheduler_options);
+    for (uint32_t step = 0; step < 4; ++step)
+    {
+        auto rows = sampler->device_logits(count, vocab);
+        check(static_cast<bool>(rows));
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            const std::vector<float> values = synthetic_logits(vocab, i, step, 17);
+            check(hipMemcpy(static_cast<float*>(rows.value().data) + static_cast<size_t>(i) * rows.value().row_stride, values.data(),
+                            vocab * sizeof(float), hipMemcpyHostToDevice) == hipSuccess);
+        }
+        std::vector<SampleBatchRequest> whole;
+        for (uint32_t i = 0; i < count; ++i)
+            whole.push_back(SampleBatchRequest{direct[i].get(), nullptr, options, {}});
+        auto expected = SessionBatchSampler::sample_resident(sampler, whole);
+        std::vector<std::future<std::vector<Result<BatchSampledToken>>>> futures(count);
+        std::vector<std::thread> threads;
+        for (uint32_t k = 0; k < count; ++k)
+        {
+            const uint32_t i = (k * 5 + step) % count; // Session i's thread starts k-th
+            threads.emplace_back([&, i] {
+                SampleBatchRequest request{scheduled[i].get(), nullptr, options, {}};
+                request.device_row = i;
+                futures[i] = scheduler.submit_sample(std::vector<SampleBatchRequest>{request});
+            });
+        }
+        for (std::thread& thread : threads)
+            thread.join();
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            auto got = futures[i].get();
+            check(got.size() == 1 && static_cast<bool>(got[0]) && static_cast<bool>(expected[i]));
+            check(got[0].value().token.token_id == expected[i].value().token.token_id);
+            check(std::bit_cast<uint32_t>(got[0].value().token.probability) == std::bit_cast<uint32_t>(expected[i].value().token.probability));
+        }
+    }
+    check(scheduler.statistics().cross_call_collected_requests > 0);
+    // a subset of the rows, named in descending order, directly
+    {
+        std::vector<SampleBatchRequest> whole, some;
+        for (uint32_t i = 0; i < count; ++i)
+            whole.push_back(SampleBatchRequest{direct[i].get(), nullptr, options, {}});
+        for (uint32_t i : {6u, 3u, 1u})
+        {
+            SampleBatchRequest request{scheduled[i].get(), nullptr, options, {}};
+            request.device_row = i;
+            some.push_back(request);
+        }
+        auto got = SessionBatchSampler::sample_resident(sampler, some);
+        auto expected = SessionBatchSampler::sample_resident(sampler, whole);
+        const uint32_t named[3] = {6, 3, 1};
+        for (size_t j = 0; j < 3; ++j)
+        {
+            check(static_cast<bool>(got[j]) && got[j].value().token.token_id == expected[named[j]].value().token.token_id);
+            check(std::bit_cast<uint32_t>(got[j].value().token.probability) == std::bit_cast<uint32_t>(expected[named[j]].value().token.probability));
+        }
+        // (the Sessions of `scheduled` that were not named keep their generators: bring them level again)
+        std::vector<SampleBatchRequest> rest;
+        for (uint32_t i : {0u, 2u, 4u, 5u, 7u})
+        {
+            SampleBatchRequest request{scheduled[i].get(), nullptr, options, {}};
+            request.device_row = i;
+            rest.push_back(request);
+        }
+        auto level = SessionBatchSampler::sample_resident(sampler, rest);
+        check(level.size() == 5 && static_cast<bool>(level[0]));
+        // a row named twice, a row beyond the layout, rows named for some requests only
+        some[1].device_row = 6;
+        auto twice = SessionBatchSampler::sample_resident(sampler, some);
+        check(!twice[0] && twice[0].error().message.find("twice") != std::string::npos);
+        some[1].device_row = count;
+        auto beyond = SessionBatchSampler::sample_resident(sampler, some);
+        check(!beyond[0] && beyond[0].error().message.find("beyond") != std::string::npos);
+        some[1].device_row = SampleBatchRequest::kRowByPosition;
+        auto partly = SessionBatchSampler::sample_resident(sampler, some);
+        check(!partly[0] && partly[0].error().code == ErrorCode::InvalidArgument);
+    }
+    // a request that names no row and travels alone is a batch of one: row 0 of a one-row layout, never merged
+    {
+        auto one = sampler->device_logits(1, vocab);
+        check(static_cast<bool>(one));
+        const std::vector<float> values = synthetic_logits(vocab, 3, 9, 17);
+        check(hipMemcpy(one.value().data, values.data(), vocab * sizeof(float), hipMemcpyHostToDevice) == hipSuccess);
+        const uint64_t collected_before = scheduler.statistics().cross_call_collected_requests;
+        auto alone = scheduler.submit_sample(std::vector<SampleBatchRequest>{SampleBatchRequest{scheduled[0].get(), nullptr, options, {}}}).get();
+        auto same = SessionBatchSampler::sample_resident(sampler, std::vector<SampleBatchRequest>{SampleBatchRequest{direct[0].get(), nullptr, options, {}}});
+        check(alone.size() == 1 && static_cast<bool>(alone[0]) && alone[0].value().token.token_id == same[0].value().token.token_id);
+        check(scheduler.statistics().cross_call_collected_requests == collected_before);
+    }
+    // the two kinds in one batch, and a sampler the scheduler does not have
+    {
+        const LogitsOutput row = logits_of({1.0f, 2.0f, 3.0f});
+        SamplingSession host_session(sampler, SamplingSessionOptions{5});
+        std::vector<SampleBatchRequest> mixed = {SampleBatchRequest{scheduled[0].get(), nullptr, options, {}},
+                                                 SampleBatchRequest{&host_session, &row, options, {}}};
+        auto rejected = scheduler.submit_sample(mixed).get();
+        check(rejected.size() == 2 && !rejected[0] && rejected[0].error().message.find("mixes") != std::string::npos);
+        SampleBatchRequest elsewhere{scheduled[0].get(), nullptr, options, {}};
+        elsewhere.resident_sampler = 3;
+        auto missing = scheduler.submit_sample(std::vector<SampleBatchRequest>{elsewhere}).get();
+        check(missing.size() == 1 && !missing[0] && missing[0].error().code == ErrorCode::InvalidArgument);
+    }
+}
+
+// A scheduler over three samplers: batches of host logits that its workers run at the same time go to
+// different samplers (buffers and streams of their own) and overlap on the GPU, while a device-resident batch
+// runs on the sampler that holds its rows.  Every batch bit-equal to the same batch sampled alone.
+static void test_scheduler_over_several_samplers(const HipSamplerPtr& first)
+{
+    const uint32_t vocab = 6007, batches = 18, per_batch = 5;
+    std::vector<HipSamplerPtr> samplers = {first, HipSampler::create(0, 64, 8192), HipSampler::create(0, 64, 8192)};
+    check(samplers[1] != nullptr && samplers[2] != nullptr);
+    SamplingOptions options;
+    options.temperature = 0.8f;
+    options.top_k = 40;
+    options.top_p = 0.9f;
+    std::deque<SamplingSession> through, alone;
+    std::vector<std::vector<LogitsOutput>> rows(batches);
+    for (uint32_t b = 0; b < batches; ++b)
+    {
+        for (uint32_t i = 0; i < per_batch; ++i)
+        {
+            through.emplace_back(first, SamplingSessionOptions{3000 + b * per_batch + i});
+            alone.emplace_back(first, SamplingSessionOptions{3000 + b * per_batch + i});
+            rows[b].push_back(logits_of(synthetic_logits(vocab, b * per_batch + i, 2, 41)));
+        }
+    }
+    SampleSchedulerOptions scheduler_options;
+    scheduler_options.worker_count = 3;
+    scheduler_options.cross_call_window_microseconds = 0;
+    BatchSampleScheduler scheduler(samplers, scheduler_options);
+    check(scheduler.sampler_count() == 3 && scheduler.sampler(0) == first && scheduler.sampler(3) == nullptr);
+    // rows on the first sampler's buffer, for a resident batch in the middle of the host batches
+    std::deque<SamplingSession> resident_through, resident_alone;
+    auto laid_out = scheduler.sampler(0)->device_logits(4, vocab);
+    check(static_cast<bool>(laid_out));
+    for (uint32_t i = 0; i < 4; ++i)
+    {
+        resident_through.emplace_back(first, SamplingSessionOptions{7000 + i, LogitsOutputMode::SampledToken});
+        resident_alone.emplace_back(first, SamplingSessionOptions{7000 + i, LogitsOutputMode::SampledToken});
+        const std::vector<float> values = synthetic_logits(vocab, 100 + i, 0, 41);
+        check(hipMemcpy(static_cast<float*>(laid_out.value().data) + static_cast<size_t>(i) * laid_out.value().row_stride, values.data(),
+                        vocab * sizeof(float), hipMemcpyHostToDevice) == hipSuccess);
+    }
+    std::vector<std::future<std::vector<Result<BatchSampledToken>>>> futures;
+    std::future<std::vector<Result<BatchSampledToken>>> resident_future;
+    for (uint32_t b = 0; b < batches; ++b)
+    {
+        std::vector<SampleBatchRequest> requests;
+        for (uint32_t i = 0; i < per_batch; ++i)
+            requests.push_back(SampleBatchRequest{&through[b * per_batch + i], &rows[b][i], options, {}});
+        futures.push_back(scheduler.submit_sample(std::move(requests)));
+        if (b == batches / 2)
+        {
+            std::vector<SampleBatchRequest> resident;
+            for (uint32_t i = 0; i < 4; ++i)
+                resident.push_back(SampleBatchRequest{&resident_through[i], nullptr, options, {}});
+            resident_future = scheduler.submit_sample(std::move(resident));
+        }
+    }
+    for (uint32_t b = 0; b < batches; ++b)
+    {
+        auto got = futures[b].get();
+        std::vector<SampleBatchRequest> requests;
+        for (uint32_t i = 0; i < per_batch; ++i)
+            requests.push_back(SampleBatchRequest{&alone[b * per_batch + i], &rows[b][i], options, {}});
+        auto expected = SessionBatchSampler::sample(samplers[1], requests);
+        check(got.size() == per_batch);
+        for (uint32_t i = 0; i < per_batch; ++i)
+        {
+            check(static_cast<bool>(got[i]) && static_cast<bool>(expected[i]));
+            check(got[i].value().token.token_id == expected[i].value().token.token_id);
+            check(std::bit_cast<uint32_t>(got[i].value().token.probability) == std::bit_cast<uint32_t>(expected[i].value().token.probability));
+        }
+    }
+    // no host batch ran on the first sampler: its rows are still there, for the scheduler's batch and for this one
+    auto resident_got = resident_future.get();
+    std::vector<SampleBatchRequest> resident;
+    for (uint32_t i = 0; i < 4; ++i)
+        resident.push_back(SampleBatchRequest{&resident_alone[i], nullptr, options, {}});
+    auto resident_expected = SessionBatchSampler::sample_resident(first, resident);
+    for (uint32_t i = 0; i < 4; ++i)
+    {
+        check(static_cast<bool>(resident_got[i]) && static_cast<bool>(resident_expected[i]));
+        check(resident_got[i].value().token.token_id == resident_expected[i].value().token.token_id);
+    }
+    const SampleSchedulerStatistics statistics = scheduler.statistics();
+    check(statistics.device_calls == batches + 1 && statistics.completed_requests == batches * per_batch + 4);
+    std::printf("scheduler over 3 samplers: %llu of %llu device calls began while another was running\n",
+                static_cast<unsigned long long>(statistics.overlapped_device_calls), static_cast<unsigned long long>(statistics.device_calls));
 }
 
 // A state without cache transactions: a step in which nothing is accepted falls back before the next token
@@ -1218,8 +1432,105 @@ static int generation_bench(uint32_t session_count, uint32_t vocab, uint32_t ste
     return 0;
 }
 
+// --scheduler-bench ROWS VOCAB SAMPLERS STEPS: batches of ROWS device-resident rows through BatchSampleScheduler
+// over SAMPLERS samplers (a worker each), as many batches in flight as there are samplers, every batch one
+// synchronous device call of the worker that runs it.  Prints one line; the tokens of the first batch are there
+// for a check against the CPU oracle (row i of sampler 0: synthetic_logits(VOCAB, i, 0, -1), seed 5000 + i).
+static int scheduler_bench(uint32_t rows, uint32_t vocab, uint32_t sampler_count, uint32_t steps)
+{
+    std::vector<HipSamplerPtr> samplers;
+    std::deque<SamplingSession> sessions;
+    for (uint32_t lane = 0; lane < sampler_count; ++lane)
+    {
+        samplers.push_back(HipSampler::create(0, rows, vocab));
+        if (!samplers.back())
+        {
+            std::fprintf(stderr, "HipSampler::create failed: no usable GPU\n");
+            return 2;
+        }
+        std::vector<std::vector<float>> values;
+        std::vector<std::span<const float>> spans;
+        for (uint32_t i = 0; i < rows; ++i)
+            values.push_back(synthetic_logits(vocab, i, lane, -1));
+        for (const std::vector<float>& row : values)
+            spans.emplace_back(row);
+        auto uploaded = samplers.back()->upload_resident(spans);
+        if (!uploaded)
+        {
+            std::fprintf(stderr, "upload_resident failed: %s\n", uploaded.error().message.c_str());
+            return 1;
+        }
+        for (uint32_t i = 0; i < rows; ++i)
+            sessions.emplace_back(samplers.back(), SamplingSessionOptions{5000 + lane * rows + i, LogitsOutputMode::SampledToken});
+    }
+    SamplingOptions options{0.7f, 20, 0.8f, 0.0f};
+    SampleSchedulerOptions scheduler_options;
+    scheduler_options.worker_count = sampler_count;
+    scheduler_options.cross_call_window_microseconds = 0;
+    BatchSampleScheduler scheduler(samplers, scheduler_options);
+    const auto batch_of = [&](uint32_t lane) {
+        std::vector<SampleBatchRequest> requests;
+        for (uint32_t i = 0; i < rows; ++i)
+        {
+            SampleBatchRequest request{&sessions[lane * rows + i], nullptr, options, {}};
+            request.resident_sampler = lane;
+            requests.push_back(std::move(request));
+        }
+        return requests;
+    };
+    std::vector<std::future<std::vector<Result<BatchSampledToken>>>> in_flight(sampler_count);
+    std::vector<Result<BatchSampledToken>> first_batch;
+    double seconds = 0.0;
+    for (int pass = 0; pass < 2; ++pass) // the first pass warms up (and keeps the first batch's tokens)
+    {
+        const uint32_t count = pass == 0 ? 4 * sampler_count : steps;
+        const auto started = std::chrono::steady_clock::now();
+        for (uint32_t step = 0; step < count; ++step)
+        {
+            const uint32_t lane = step % sampler_count;
+            if (in_flight[lane].valid())
+            {
+                while (in_flight[lane].wait_for(std::chrono::seconds(0)) != std::future_status::ready)
+                {
+                } // (the serving thread keeps awake as well)
+                auto done = in_flight[lane].get();
+                if (first_batch.empty())
+                    first_batch = std::move(done);
+            }
+            in_flight[lane] = scheduler.submit_sample(batch_of(lane));
+        }
+        for (auto& future : in_flight)
+        {
+            if (future.valid())
+            {
+                auto done = future.get();
+                for (const auto& row : done)
+                {
+                    if (!row)
+                    {
+                        std::fprintf(stderr, "a row failed: %s\n", row.error().message.c_str());
+                        return 1;
+                    }
+                }
+            }
+        }
+        seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - started).count();
+    }
+    const SampleSchedulerStatistics statistics = scheduler.statistics();
+    std::printf("scheduler_bench rows %u vocab %u samplers %u steps %u seconds %.6f device_calls %llu overlapped_device_calls %llu first_batch",
+                rows, vocab, sampler_count, steps, seconds, static_cast<unsigned long long>(statistics.device_calls),
+                static_cast<unsigned long long>(statistics.overlapped_device_calls));
+    for (const auto& row : first_batch)
+        std::printf(" %d:%u", row ? row.value().token.token_id : -1, row ? std::bit_cast<uint32_t>(row.value().token.probability) : 0u);
+    std::printf("\n");
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
+    if (argc == 6 && std::strcmp(argv[1], "--scheduler-bench") == 0)
+        return scheduler_bench(static_cast<uint32_t>(std::atoi(argv[2])), static_cast<uint32_t>(std::atoi(argv[3])),
+                               static_cast<uint32_t>(std::atoi(argv[4])), static_cast<uint32_t>(std::atoi(argv[5])));
     if (argc == 5 && std::strcmp(argv[1], "--generation-bench") == 0)
         return generation_bench(static_cast<uint32_t>(std::atoi(argv[2])), static_cast<uint32_t>(std::atoi(argv[3])),
                                 static_cast<uint32_t>(std::atoi(argv[4])));
@@ -1259,6 +1570,8 @@ int main(int argc, char** argv)
         test_scheduler_collects_across_calls(sampler);
         test_scheduler_keeps_a_sessions_order(sampler);
         test_sampled_token_mode(sampler);
+        test_resident_requests_through_the_scheduler(sampler);
+        test_scheduler_over_several_samplers(sampler);
         test_generation_loop_equals_serial(sampler);
         test_generation_loop_callback_and_errors(sampler);
     }
