@@ -1113,7 +1113,7 @@ SampleSchedulerStatistics BatchSampleScheduler::statistics() const noexcept
 
 Result<std::vector<GenerationResult>> BatchGenerationLoop::generate(
     const HipSamplerPtr& sampler, std::span<SamplingSession* const> sessions, IDeviceLogitsSource& source,
-    std::span<const GenerationOptions> options, const BatchTokenCallback& on_token)
+    std::span<const GenerationOptions> options, const BatchTokenCallback& on_token, const TokenTextDecoder& decode_text)
 {
     const size_t count = sessions.size();
     if (count == 0)
@@ -1140,90 +1140,256 @@ Result<std::vector<GenerationResult>> BatchGenerationLoop::generate(
         // Session::generate checks these before it decodes anything (src/engine/session.cpp:461-473)
         if (options_of(i).max_new_tokens == 0)
             return invalid_argument("max_new_tokens must be non-zero");
+        const float threshold = options_of(i).speculative_confidence_threshold;
+        if (!std::isfinite(threshold) || threshold < 0.0f || threshold > 1.0f)
+            return invalid_argument("speculative_confidence_threshold must be in the range [0, 1]");
         auto valid = validate_sampling_options(options_of(i).sampling);
         if (!valid)
             return valid.error();
     }
+    auto* const speculative = dynamic_cast<ISpeculativeLogitsSource*>(&source);
+    const uint32_t block_size = speculative != nullptr ? std::min<uint32_t>(speculative->speculative_block_size(), NCNN_MOE_MAX_DRAFT_TOKENS) : 0u;
+    const bool state_cache_transactions = speculative != nullptr && speculative->state_cache_transactions();
+    if (block_size != 0 && 2u * block_size + 1u > sampler->max_rows())
+        return invalid_argument("speculative verification exceeds the sampler's max_rows");
 
     std::vector<GenerationResult> results(count);
-    // the Sessions that sample at this token index, in Session order; row i of the device buffer is theirs
-    std::vector<uint32_t> active(count);
+    // enable_speculative_context of session.cpp:503-506, and whether the Session is still in speculative mode
+    std::vector<uint8_t> speculative_context(count, 0), speculative_active(count, 0), finished(count, 0);
     for (size_t i = 0; i < count; ++i)
-        active[i] = static_cast<uint32_t>(i);
-    auto rows = sampler->device_logits(static_cast<uint32_t>(count), vocab, bf16);
-    if (!rows)
-        return rows.error();
-    auto prefilled = source.prefill(active, rows.value());
-    if (!prefilled)
-        return prefilled.error();
+        speculative_context[i] = speculative_active[i] = (block_size != 0 && options_of(i).enable_speculative) ? 1 : 0;
+
+    // One token of Session i goes out: text, callback, and the three reasons to stop in the order of
+    // src/engine/session.cpp:1000-1013 (callback, stop token, token budget).  False: the Session has finished.
+    const auto emit = [&](uint32_t i, int32_t token_id, float probability, bool is_stop_token) {
+        StreamToken token;
+        token.index = static_cast<uint32_t>(results[i].tokens.size());
+        token.token_id = token_id;
+        token.probability = probability;
+        token.is_stop_token = is_stop_token;
+        if (decode_text)
+            token.text = decode_text(token.token_id);
+        const bool continue_generation = !on_token || on_token(i, token);
+        results[i].tokens.push_back(std::move(token));
+        if (!continue_generation)
+            results[i].stopped_by_callback = true;
+        else if (results[i].tokens.back().is_stop_token)
+            results[i].stopped_by_stop_token = true;
+        else if (results[i].tokens.size() < options_of(i).max_new_tokens)
+            return true;
+        finished[i] = 1;
+        return false;
+    };
+    const auto is_stop = [&](uint32_t i, int32_t token_id) {
+        const std::vector<int32_t>& stops = options_of(i).stop_tokens;
+        return std::find(stops.begin(), stops.end(), token_id) != stops.end();
+    };
 
     std::vector<SamplingOptions> row_options;
     std::vector<float> uniforms;
     std::vector<std::vector<int32_t>> stop_tokens;
     std::vector<uint8_t> draw_consumed;
-    std::vector<DecodeSlot> slots;
-    std::vector<uint32_t> next_active;
-    for (uint32_t index = 0; !active.empty(); ++index)
-    {
+    // Samples the rows the buffer holds, row r for Session members[r], consuming each Session's draw where the
+    // sampler took it.  A row that failed fails the call before anything of the step is committed: no draw is
+    // taken from a generator, no callback runs and no token is appended for the Sessions in front of it.
+    const auto sample_members = [&](const std::vector<uint32_t>& members, bool with_stop_tokens) -> Result<std::vector<BatchSampledToken>> {
         row_options.clear();
         uniforms.clear();
-        stop_tokens.resize(active.size());
-        for (size_t row = 0; row < active.size(); ++row)
+        stop_tokens.resize(with_stop_tokens ? members.size() : 0);
+        for (size_t row = 0; row < members.size(); ++row)
         {
-            const uint32_t i = active[row];
+            const uint32_t i = members[row];
             row_options.push_back(options_of(i).sampling);
             uniforms.push_back(sessions[i]->uniform_ahead(0));
-            stop_tokens[row] = options_of(i).stop_tokens; // assignment reuses the row's storage from the last step
+            if (with_stop_tokens)
+                stop_tokens[row] = options_of(i).stop_tokens; // assignment reuses the row's storage from the last step
         }
         const SampleTimer timer;
         auto sampled = sampler->sample_resident(row_options, uniforms, stop_tokens, draw_consumed);
-        slots.clear();
-        next_active.clear();
-        // a row that failed fails the call before anything of this step is committed: no draw is taken
-        // from a generator, no callback runs and no token is appended for the Sessions in front of it
-        for (size_t row = 0; row < active.size(); ++row)
+        std::vector<BatchSampledToken> tokens;
+        tokens.reserve(members.size());
+        for (size_t row = 0; row < members.size(); ++row)
         {
             if (!sampled[row])
                 return sampled[row].error();
         }
-        for (size_t row = 0; row < active.size(); ++row)
+        for (size_t row = 0; row < members.size(); ++row)
         {
-            const uint32_t i = active[row];
-            timer.charge(sessions[i]->statistics_, 1);
+            timer.charge(sessions[members[row]]->statistics_, 1);
             if (draw_consumed[row])
-                sessions[i]->consume_uniforms(1);
-            StreamToken token;
-            token.index = index;
-            token.token_id = sampled[row].value().token.token_id;
-            token.probability = sampled[row].value().token.probability;
-            token.is_stop_token = sampled[row].value().is_stop_token;
-            const bool continue_generation = !on_token || on_token(i, token);
-            results[i].tokens.push_back(std::move(token));
-            // the order of src/engine/session.cpp:1000-1013: callback, stop token, token budget
-            if (!continue_generation)
-            {
-                results[i].stopped_by_callback = true;
-                continue;
-            }
-            if (results[i].tokens.back().is_stop_token)
-            {
-                results[i].stopped_by_stop_token = true;
-                continue;
-            }
-            if (index + 1 == options_of(i).max_new_tokens)
-                continue;
-            slots.push_back(DecodeSlot{i, results[i].tokens.back().token_id});
-            next_active.push_back(i);
+                sessions[members[row]]->consume_uniforms(1);
+            tokens.push_back(sampled[row].value());
         }
-        active.swap(next_active);
-        if (active.empty())
+        return tokens;
+    };
+
+    // ---- token 0 of every Session, from the prefill's logits
+    std::vector<uint32_t> everyone(count);
+    for (size_t i = 0; i < count; ++i)
+        everyone[i] = static_cast<uint32_t>(i);
+    auto rows = sampler->device_logits(static_cast<uint32_t>(count), vocab, bf16);
+    if (!rows)
+        return rows.error();
+    auto prefilled = source.prefill(everyone, rows.value());
+    if (!prefilled)
+        return prefilled.error();
+    {
+        auto first = sample_members(everyone, true);
+        if (!first)
+            return first.error();
+        for (uint32_t i : everyone)
+            emit(i, first.value()[i].token.token_id, first.value()[i].token.probability, first.value()[i].is_stop_token);
+    }
+
+    std::vector<uint32_t> stepping, proposing;
+    std::vector<DecodeSlot> slots;
+    std::vector<std::vector<int32_t>> proposals(count);
+    for (;;)
+    {
+        // The Sessions that take a plain step now (decode the last token, sample the next): those outside
+        // speculative mode and those with one token left (session.cpp:586).  The others propose.
+        stepping.clear();
+        proposing.clear();
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            if (finished[i])
+                continue;
+            const size_t remaining = options_of(i).max_new_tokens - results[i].tokens.size();
+            if (speculative_context[i] && speculative_active[i] && remaining > 1)
+                proposing.push_back(i);
+            else
+                stepping.push_back(i);
+        }
+        if (stepping.empty() && proposing.empty())
             break;
-        rows = sampler->device_logits(static_cast<uint32_t>(active.size()), vocab, bf16);
-        if (!rows)
-            return rows.error();
-        auto decoded = source.decode(slots, rows.value());
-        if (!decoded)
-            return decoded.error();
+        if (!stepping.empty())
+        {
+            slots.clear();
+            for (uint32_t i : stepping)
+                slots.push_back(DecodeSlot{i, results[i].tokens.back().token_id});
+            rows = sampler->device_logits(static_cast<uint32_t>(stepping.size()), vocab, bf16);
+            if (!rows)
+                return rows.error();
+            auto decoded = source.decode(slots, rows.value());
+            if (!decoded)
+                return decoded.error();
+            auto sampled = sample_members(stepping, true);
+            if (!sampled)
+                return sampled.error();
+            for (size_t row = 0; row < stepping.size(); ++row)
+            {
+                const uint32_t i = stepping[row];
+                emit(i, sampled.value()[row].token.token_id, sampled.value()[row].token.probability, sampled.value()[row].is_stop_token);
+            }
+        }
+        if (proposing.empty())
+            continue;
+
+        // ---- propose: the block's draft tokens, each sampled with the Session's own options and generator as
+        // the executor's sampler callback does (session.cpp:634-652), one device call per draft index
+        for (uint32_t i : proposing)
+            proposals[i].clear();
+        for (uint32_t draft_index = 0; draft_index < block_size; ++draft_index)
+        {
+            slots.clear();
+            for (uint32_t i : proposing)
+                slots.push_back(DecodeSlot{i, draft_index == 0 ? results[i].tokens.back().token_id : proposals[i].back()});
+            rows = sampler->device_logits(static_cast<uint32_t>(proposing.size()), vocab, bf16);
+            if (!rows)
+                return rows.error();
+            auto drafted = speculative->draft(slots, draft_index, rows.value());
+            if (!drafted)
+                return drafted.error();
+            auto sampled = sample_members(proposing, false);
+            if (!sampled)
+                return sampled.error();
+            for (size_t row = 0; row < proposing.size(); ++row)
+                proposals[proposing[row]].push_back(sampled.value()[row].token.token_id);
+        }
+
+        // ---- cut and verify, Session by Session
+        for (uint32_t i : proposing)
+        {
+            const GenerationOptions& session_options = options_of(i);
+            const size_t remaining = session_options.max_new_tokens - results[i].tokens.size();
+            size_t draft_count = std::min<size_t>(proposals[i].size(), remaining - 1);
+            if (session_options.speculative_max_draft_tokens != 0)
+                draft_count = std::min<size_t>(draft_count, session_options.speculative_max_draft_tokens);
+            if (session_options.speculative_confidence_threshold > 0.0f)
+            {
+                for (size_t index = 0; index < draft_count; ++index)
+                {
+                    const float confidence = 1.0f / (1.0f + std::exp(-speculative->confidence_logit(i, static_cast<uint32_t>(index))));
+                    if (confidence < session_options.speculative_confidence_threshold)
+                    {
+                        draft_count = index;
+                        break;
+                    }
+                }
+            }
+            if (draft_count == 0)
+            {
+                // nothing worth verifying: the proposal is dropped and the Session leaves speculative mode (session.cpp:690-694)
+                auto dropped = speculative->commit(i, {});
+                if (!dropped)
+                    return dropped.error();
+                speculative_active[i] = 0;
+                continue;
+            }
+            const int32_t anchor = results[i].tokens.back().token_id;
+            const std::span<const int32_t> proposed(proposals[i].data(), draft_count);
+            rows = sampler->device_logits(static_cast<uint32_t>(2 * draft_count + 1), vocab, bf16);
+            if (!rows)
+                return rows.error();
+            auto written = speculative->verify(i, anchor, proposed, rows.value());
+            if (!written)
+                return written.error();
+            uniforms.resize(draft_count + 1);
+            for (size_t k = 0; k <= draft_count; ++k)
+                uniforms[k] = sessions[i]->uniform_ahead(k);
+            uint32_t draws_consumed = 0, accept_draws = 0;
+            bool failed_behind_an_empty_accept_loop = false;
+            const SampleTimer timer;
+            auto verified = sampler->verify_speculative_resident(proposed, session_options.sampling, uniforms, draws_consumed, &accept_draws,
+                                                                 &failed_behind_an_empty_accept_loop);
+            SamplingStatistics& statistics = sessions[i]->statistics_;
+            statistics.speculative_steps += 1;
+            statistics.speculative_verify_time_microseconds += static_cast<uint64_t>(
+                std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - timer.started).count());
+            if (!state_cache_transactions && ((verified && verified.value().accepted.empty()) || failed_behind_an_empty_accept_loop))
+            {
+                // session.cpp:843-857: roll the step back, leave speculative mode; only the accept test's draw is gone
+                sessions[i]->consume_uniforms(accept_draws);
+                auto rolled_back = speculative->commit(i, {});
+                if (!rolled_back)
+                    return rolled_back.error();
+                speculative_active[i] = 0;
+                continue;
+            }
+            if (!verified)
+                return verified.error();
+            sessions[i]->consume_uniforms(draws_consumed);
+            std::vector<int32_t> emitted;
+            bool continues = true;
+            for (const SampledToken& accepted : verified.value().accepted)
+            {
+                emitted.push_back(accepted.token_id);
+                continues = emit(i, accepted.token_id, accepted.probability, is_stop(i, accepted.token_id));
+                if (!continues)
+                    break;
+            }
+            if (continues)
+            {
+                const SampledToken& next = verified.value().next;
+                emitted.push_back(next.token_id);
+                emit(i, next.token_id, next.probability, is_stop(i, next.token_id));
+            }
+            statistics.sampled_tokens += emitted.size();
+            statistics.speculative_accepted_tokens += emitted.size() - 1;
+            auto committed = speculative->commit(i, emitted);
+            if (!committed)
+                return committed.error();
+        }
     }
     return results;
 }

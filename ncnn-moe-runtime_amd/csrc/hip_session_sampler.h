@@ -103,14 +103,13 @@ struct SampledToken
     float probability = 0.0f;
 };
 
-// StreamToken, GenerationOptions and GenerationResult of include/ncnn/moe/session.h:63-91 (without the
-// speculative switches, which belong to Session::generate's draft model).
+// StreamToken, GenerationOptions, GenerationResult and TokenTextDecoder of include/ncnn/moe/session.h:63-96.
 struct StreamToken
 {
     uint32_t index = 0;
     int32_t token_id = -1;
     float probability = 0.0f;
-    std::string text; // left empty: callers decode token ids themselves
+    std::string text; // what the caller's TokenTextDecoder returned for the token; empty without one
     bool is_stop_token = false;
 };
 
@@ -119,7 +118,12 @@ struct GenerationOptions
     uint32_t max_new_tokens = 1;
     SamplingOptions sampling;
     std::vector<int32_t> stop_tokens;
+    bool enable_speculative = true;
+    float speculative_confidence_threshold = 0.5f;
+    uint32_t speculative_max_draft_tokens = 0;
 };
+
+using TokenTextDecoder = std::function<std::string(int32_t token_id)>;
 
 struct GenerationResult
 {
@@ -276,6 +280,11 @@ struct SamplingStatistics
     uint64_t sampled_tokens = 0;           // tokens this Session's sampler returned
     uint64_t sample_calls = 0;             // device calls the Session took part in
     uint64_t sample_time_microseconds = 0; // wall time of those calls (a batched call counts in full for each of its Sessions)
+    // SessionStatistics::speculative_accepted_tokens and ::speculative_verify_time_microseconds (the share of the
+    // verification's device call), plus the steps themselves
+    uint64_t speculative_steps = 0;
+    uint64_t speculative_accepted_tokens = 0;
+    uint64_t speculative_verify_time_microseconds = 0;
 };
 
 struct SamplingSessionOptions
@@ -449,6 +458,30 @@ public:
     virtual Result<bool> decode(std::span<const DecodeSlot> slots, const DeviceLogitsRows& rows) = 0;
 };
 
+// The draft side of a model that can speculate: what CpuExecutor::propose_speculative and the verification pass of
+// Session::generate do (src/engine/cpu_executor.cpp:2105-2160, :2270-2312; src/engine/session.cpp:630-760), writing
+// device rows.  A source that implements it is recognised by BatchGenerationLoop::generate.
+class ISpeculativeLogitsSource : public IDeviceLogitsSource
+{
+public:
+    // Tokens of one proposal (CompiledModel::speculative.block_size); 0: the model has no draft head.
+    virtual uint32_t speculative_block_size() const = 0;
+    // SpeculativeModelKind::Mtp: the model state can keep part of a step (state cache transactions); without them
+    // a step that accepts nothing is rolled back and the Session leaves speculative mode (session.cpp:843-857).
+    virtual bool state_cache_transactions() const = 0;
+    // Draft row `draft_index` of every listed Session: the draft head's logits after slot.token_id was fed (the
+    // anchor for index 0, the Session's previous draft after that).  Row i belongs to slots[i].
+    virtual Result<bool> draft(std::span<const DecodeSlot> slots, uint32_t draft_index, const DeviceLogitsRows& rows) = 0;
+    // CpuSpeculativeProposal::confidence_logits of the Session's current proposal (+infinity where the model has none).
+    virtual float confidence_logit(uint32_t session_index, uint32_t draft_index) const = 0;
+    // The verification rows of one Session's step: rows 0 .. D the target's logits after the anchor and after each
+    // of the D proposed tokens, rows D + 1 .. 2 D the draft rows those tokens were sampled from.
+    virtual Result<bool> verify(uint32_t session_index, int32_t anchor, std::span<const int32_t> proposed, const DeviceLogitsRows& rows) = 0;
+    // The step's outcome: the tokens that were emitted (the accepted ones and the one after them), none when the
+    // step was rolled back.  The state moves on by them (finish_cache_transaction, session.cpp:931-935).
+    virtual Result<bool> commit(uint32_t session_index, std::span<const int32_t> emitted) = 0;
+};
+
 // Called for every token as it is sampled; returning false stops that Session (GenerationResult::stopped_by_callback).
 using BatchTokenCallback = std::function<bool(uint32_t session_index, const StreamToken& token)>;
 
@@ -462,9 +495,18 @@ public:
     // declined, and decode the others' tokens for the next step.  `options` holds one entry for all
     // Sessions or one per Session.  Token ids, probabilities, stop flags and generator states end up
     // as Session::generate (src/engine/session.cpp:978-1020) leaves them for each Session alone.
+    //
+    // With a source that can speculate (ISpeculativeLogitsSource with a block size above zero) a Session whose
+    // options enable it runs the speculative loop of Session::generate (src/engine/session.cpp:522-977): after its
+    // first token, rounds of propose (the block's draft tokens, each sampled with the Session's own generator, one
+    // device call per draft index for all such Sessions) - cut the proposal (token budget,
+    // speculative_max_draft_tokens, confidence threshold) - verify (one device pass per Session: accept loop and
+    // the token after it) - stream the accepted tokens and that one.  A step that proposes or, without cache
+    // transactions, accepts nothing leaves speculative mode for good, and the Session goes on token by token.
+    // decode_text fills StreamToken::text in front of the callback (TokenTextDecoder, session.h:96).
     static Result<std::vector<GenerationResult>> generate(
         const HipSamplerPtr& sampler, std::span<SamplingSession* const> sessions, IDeviceLogitsSource& source,
-        std::span<const GenerationOptions> options, const BatchTokenCallback& on_token = {});
+        std::span<const GenerationOptions> options, const BatchTokenCallback& on_token = {}, const TokenTextDecoder& decode_text = {});
 };
 
 // validate_sampling_options (src/engine/session.cpp:65-74) on the host, with the same messages.

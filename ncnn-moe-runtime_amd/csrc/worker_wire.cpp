@@ -408,6 +408,11 @@ GenerateRequest parse_generate_request(std::string_view line)
         parsed.options.sampling.top_p = static_cast<float>(*top_p);
     if (const auto min_p = fields.number("min_p"))
         parsed.options.sampling.min_p = static_cast<float>(*min_p);
+    // the speculative switches of examples/ncnn_moe_worker.cpp:1040, :1053-1055
+    parsed.options.enable_speculative = fields.boolean("enable_speculative").value_or(true);
+    if (const auto confidence = fields.number("speculative_confidence"))
+        parsed.options.speculative_confidence_threshold = static_cast<float>(*confidence);
+    parsed.options.speculative_max_draft_tokens = request_uint(fields, "speculative_max_draft", 0);
     return parsed;
 }
 

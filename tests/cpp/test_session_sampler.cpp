@@ -1143,6 +1143,133 @@ private:
     std::vector<uint32_t> positions_;
 };
 
+// The same model with a draft head: a proposal's row k predicts the token k places behind the anchor from the
+// row the target will have there, shifted by 0.75 at every fifth token (exact in fp32), so that proposals are
+// mostly but not always accepted; its confidence logit is low at some positions.  The verification rows are the
+// target's rows for the anchor and the proposed tokens and the draft rows the tokens were sampled from.
+inline std::vector<float> synthetic_draft_logits(uint32_t vocab, uint32_t session, uint32_t position, int32_t fed_token, uint32_t draft_index)
+{
+    std::vector<float> row = synthetic_logits(vocab, session, position, fed_token);
+    for (uint32_t v = (session + draft_index) % 5u; v < vocab; v += 5u)
+        row[v] += 0.75f;
+    return row;
+}
+
+inline float synthetic_confidence_logit(uint32_t session, uint32_t position)
+{
+    return (session * 7u + position * 3u) % 11u == 0u ? -0.5f : 2.0f;
+}
+
+class SyntheticSpeculativeSource : public ISpeculativeLogitsSource
+{
+public:
+    SyntheticSpeculativeSource(uint32_t vocab, uint32_t sessions, uint32_t block_size, bool transactions)
+        : vocab_(vocab), block_size_(block_size), transactions_(transactions), positions_(sessions, 0), proposal_rows_(sessions)
+    {
+    }
+
+    uint32_t vocabulary_size() const override { return vocab_; }
+    uint32_t speculative_block_size() const override { return block_size_; }
+    bool state_cache_transactions() const override { return transactions_; }
+
+    Result<bool> prefill(std::span<const uint32_t> session_indices, const DeviceLogitsRows& rows) override
+    {
+        for (size_t row = 0; row < session_indices.size(); ++row)
+        {
+            positions_[session_indices[row]] = 0;
+            auto written = write_row(rows, row, synthetic_logits(vocab_, session_indices[row], 0, -1));
+            if (!written)
+                return written;
+        }
+        return true;
+    }
+
+    Result<bool> decode(std::span<const DecodeSlot> slots, const DeviceLogitsRows& rows) override
+    {
+        for (size_t row = 0; row < slots.size(); ++row)
+        {
+            const uint32_t position = ++positions_[slots[row].session_index];
+            auto written = write_row(rows, row, synthetic_logits(vocab_, slots[row].session_index, position, slots[row].token_id));
+            if (!written)
+                return written;
+        }
+        ++decode_calls;
+        return true;
+    }
+
+    Result<bool> draft(std::span<const DecodeSlot> slots, uint32_t draft_index, const DeviceLogitsRows& rows) override
+    {
+        for (size_t row = 0; row < slots.size(); ++row)
+        {
+            const uint32_t session = slots[row].session_index;
+            if (draft_index == 0)
+                proposal_rows_[session].clear();
+            if (proposal_rows_[session].size() != draft_index)
+                return Error{ErrorCode::InternalError, "synthetic source: draft rows out of order"};
+            proposal_rows_[session].push_back(
+                synthetic_draft_logits(vocab_, session, positions_[session] + 1 + draft_index, slots[row].token_id, draft_index));
+            auto written = write_row(rows, row, proposal_rows_[session].back());
+            if (!written)
+                return written;
+        }
+        ++draft_calls;
+        return true;
+    }
+
+    float confidence_logit(uint32_t session_index, uint32_t draft_index) const override
+    {
+        return synthetic_confidence_logit(session_index, positions_[session_index] + 1 + draft_index);
+    }
+
+    Result<bool> verify(uint32_t session_index, int32_t anchor, std::span<const int32_t> proposed, const DeviceLogitsRows& rows) override
+    {
+        const uint32_t drafts = static_cast<uint32_t>(proposed.size());
+        if (rows.rows != 2 * drafts + 1 || proposal_rows_[session_index].size() < drafts)
+            return Error{ErrorCode::InternalError, "synthetic source: unexpected verification rows"};
+        for (uint32_t k = 0; k <= drafts; ++k)
+        {
+            auto written = write_row(rows, k, synthetic_logits(vocab_, session_index, positions_[session_index] + 1 + k, k == 0 ? anchor : proposed[k - 1]));
+            if (!written)
+                return written;
+        }
+        for (uint32_t k = 0; k < drafts; ++k)
+        {
+            auto written = write_row(rows, drafts + 1 + k, proposal_rows_[session_index][k]);
+            if (!written)
+                return written;
+        }
+        ++verify_calls;
+        return true;
+    }
+
+    Result<bool> commit(uint32_t session_index, std::span<const int32_t> emitted) override
+    {
+        positions_[session_index] += static_cast<uint32_t>(emitted.size());
+        committed_tokens += static_cast<uint32_t>(emitted.size());
+        rolled_back_steps += emitted.empty() ? 1u : 0u;
+        return true;
+    }
+
+    uint32_t decode_calls = 0, draft_calls = 0, verify_calls = 0, committed_tokens = 0, rolled_back_steps = 0;
+
+private:
+    Result<bool> write_row(const DeviceLogitsRows& rows, size_t row, const std::vector<float>& values)
+    {
+        if (rows.bf16 || rows.vocab != vocab_ || row >= rows.rows || rows.row_stride < vocab_)
+            return Error{ErrorCode::InternalError, "synthetic source: unexpected device rows"};
+        float* target = static_cast<float*>(rows.data) + row * rows.row_stride;
+        if (hipMemcpy(target, values.data(), values.size() * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
+            return Error{ErrorCode::InternalError, "synthetic source: hipMemcpy failed"};
+        return true;
+    }
+
+    uint32_t vocab_;
+    uint32_t block_size_;
+    bool transactions_;
+    std::vector<uint32_t> positions_;
+    std::vector<std::vector<std::vector<float>>> proposal_rows_;
+};
+
 struct LoopCase
 {
     uint64_t seed;
@@ -1322,6 +1449,162 @@ static void test_generation_loop_callback_and_errors(const HipSamplerPtr& sample
         auto failed = BatchGenerationLoop::generate(sampler, pointers, source, options);
         check(!failed && failed.error().message == "synthetic decode failure");
     }
+}
+
+constexpr uint32_t kSpeculativeBlock = 4;
+
+static std::vector<LoopCase> speculative_cases()
+{
+    std::vector<LoopCase> cases;
+    const auto add = [&](uint64_t seed, uint32_t max_new_tokens, float temperature, uint32_t top_k, float top_p, float min_p,
+                         std::vector<int32_t> stop_tokens, bool enable, float confidence, uint32_t max_draft) {
+        LoopCase entry;
+        entry.seed = seed;
+        entry.options.max_new_tokens = max_new_tokens;
+        entry.options.sampling = SamplingOptions{temperature, top_k, top_p, min_p};
+        entry.options.stop_tokens = std::move(stop_tokens);
+        entry.options.enable_speculative = enable;
+        entry.options.speculative_confidence_threshold = confidence;
+        entry.options.speculative_max_draft_tokens = max_draft;
+        cases.push_back(std::move(entry));
+    };
+    std::vector<int32_t> many_stops;
+    for (int32_t id = 0; id < 3000; id += 11)
+        many_stops.push_back(id);
+    add(31, 30, 0.0f, 0, 1.0f, 0.0f, {}, true, 0.5f, 0);            // greedy: proposals stand while they are the target's choice
+    add(32, 30, 0.7f, 20, 0.8f, 0.0f, {}, true, 0.5f, 0);           // the headline options: ratio tests, residual draws
+    add(33, 30, 0.7f, 20, 0.8f, 0.0f, {}, false, 0.5f, 0);          // speculation switched off for this Session
+    add(34, 23, 1.0f, 50, 0.95f, 0.0f, {}, true, 0.0f, 2);          // no confidence cut, two drafts a step at most
+    add(35, 30, 0.9f, 40, 0.9f, 0.0f, many_stops, true, 0.3f, 0);   // stops on a stop token, possibly an accepted one
+    add(36, 2, 0.8f, 8, 1.0f, 0.0f, {}, true, 0.5f, 0);             // two tokens: the second by a plain step (one token left)
+    add(37, 30, 0.5f, 1, 1.0f, 0.0f, {}, true, 0.5f, 0);            // single survivor: ratio 1, no residual, few draws
+    add(38, 17, 1.2f, 64, 0.6f, 0.02f, {}, true, 1.0f, 0);          // threshold 1: every finite confidence falls short, nothing is ever verified
+    return cases;
+}
+
+static std::vector<GenerationResult> run_speculative(const HipSamplerPtr& sampler, const std::vector<LoopCase>& cases, bool transactions,
+                                                     SyntheticSpeculativeSource** source_out = nullptr, const TokenTextDecoder& decode_text = {})
+{
+    static std::deque<SyntheticSpeculativeSource> sources; // (kept for the caller to read the counters)
+    std::deque<SamplingSession> sessions;
+    make_sessions(sampler, cases, sessions);
+    sources.emplace_back(kLoopVocab, static_cast<uint32_t>(cases.size()), kSpeculativeBlock, transactions);
+    if (source_out != nullptr)
+        *source_out = &sources.back();
+    std::vector<SamplingSession*> pointers;
+    std::vector<GenerationOptions> options;
+    for (size_t i = 0; i < cases.size(); ++i)
+    {
+        pointers.push_back(&sessions[i]);
+        options.push_back(cases[i].options);
+    }
+    auto generated = BatchGenerationLoop::generate(sampler, pointers, sources.back(), options, {}, decode_text);
+    if (!generated)
+        throw std::runtime_error("speculative generation failed: " + generated.error().message);
+    if (source_out != nullptr)
+    {
+        const SamplingStatistics statistics = sessions[1].statistics();
+        check(statistics.speculative_steps > 0 && statistics.speculative_verify_time_microseconds > 0);
+    }
+    return std::move(generated).value();
+}
+
+// The speculative loop: structure (every Session gets its tokens, budgets and stop tokens hold, a Session with
+// speculation off equals the plain loop), the text decoder, option errors.  The tokens themselves are checked by
+// tests/test_gpu_generation_loop.py, which replays every Session with the CPU oracle.
+static void test_speculative_generation_loop(const HipSamplerPtr& sampler)
+{
+    const std::vector<LoopCase> cases = speculative_cases();
+    for (const bool transactions : {true, false})
+    {
+        SyntheticSpeculativeSource* source = nullptr;
+        uint32_t decoded = 0;
+        const std::vector<GenerationResult> results = run_speculative(sampler, cases, transactions, &source, [&](int32_t token_id) {
+            ++decoded;
+            return "<" + std::to_string(token_id) + ">";
+        });
+        check(results.size() == cases.size());
+        size_t tokens = 0;
+        for (size_t i = 0; i < results.size(); ++i)
+        {
+            check(!results[i].tokens.empty() && results[i].tokens.size() <= cases[i].options.max_new_tokens);
+            check(results[i].stopped_by_stop_token || results[i].tokens.size() == cases[i].options.max_new_tokens);
+            for (size_t k = 0; k < results[i].tokens.size(); ++k)
+            {
+                const StreamToken& token = results[i].tokens[k];
+                check(token.index == k && token.text == "<" + std::to_string(token.token_id) + ">");
+                const bool stop = std::find(cases[i].options.stop_tokens.begin(), cases[i].options.stop_tokens.end(), token.token_id) != cases[i].options.stop_tokens.end();
+                check(token.is_stop_token == stop && (!stop || k + 1 == results[i].tokens.size()));
+            }
+            tokens += results[i].tokens.size();
+        }
+        check(decoded == tokens);
+        check(source->verify_calls > 0 && source->draft_calls > 0 && source->committed_tokens > 0);
+        check(transactions || source->rolled_back_steps > 0);
+        // the Session with speculation off generates what the plain loop generates
+        std::deque<SamplingSession> plain_sessions;
+        plain_sessions.emplace_back(sampler, SamplingSessionOptions{cases[2].seed});
+        SyntheticSource plain(kLoopVocab, 3);
+        // (Session index 2 of the synthetic model: two idle Sessions in front keep its index)
+        std::deque<SamplingSession> idle;
+        idle.emplace_back(sampler, SamplingSessionOptions{1});
+        idle.emplace_back(sampler, SamplingSessionOptions{2});
+        std::vector<SamplingSession*> pointers = {&idle[0], &idle[1], &plain_sessions[0]};
+        GenerationOptions one_token;
+        one_token.sampling.temperature = 0.0f;
+        std::vector<GenerationOptions> options = {one_token, one_token, cases[2].options};
+        auto alone = BatchGenerationLoop::generate(sampler, pointers, plain, options);
+        check(static_cast<bool>(alone) && alone.value()[2].tokens.size() == results[2].tokens.size());
+        for (size_t k = 0; k < results[2].tokens.size(); ++k)
+        {
+            check(alone.value()[2].tokens[k].token_id == results[2].tokens[k].token_id);
+            check(std::bit_cast<uint32_t>(alone.value()[2].tokens[k].probability) == std::bit_cast<uint32_t>(results[2].tokens[k].probability));
+        }
+    }
+    // the threshold is checked before anything runs (src/engine/session.cpp:462-470)
+    std::deque<SamplingSession> sessions;
+    sessions.emplace_back(sampler, SamplingSessionOptions{1});
+    std::vector<SamplingSession*> pointers = {&sessions[0]};
+    SyntheticSpeculativeSource source(kLoopVocab, 1, kSpeculativeBlock, true);
+    GenerationOptions bad;
+    bad.speculative_confidence_threshold = 1.5f;
+    auto rejected = BatchGenerationLoop::generate(sampler, pointers, source, std::vector<GenerationOptions>{bad});
+    check(!rejected && rejected.error().code == ErrorCode::InvalidArgument &&
+          rejected.error().message == "speculative_confidence_threshold must be in the range [0, 1]");
+    check(source.draft_calls == 0);
+}
+
+static void print_trace_lines(const std::vector<LoopCase>& cases, const std::vector<GenerationResult>& results)
+{
+    for (size_t i = 0; i < results.size(); ++i)
+    {
+        const GenerationOptions& options = cases[i].options;
+        std::printf("session %zu seed %llu max_new_tokens %u temperature_bits %u top_k %u top_p_bits %u min_p_bits %u "
+                    "speculative %d confidence_bits %u max_draft %u stops",
+                    i, static_cast<unsigned long long>(cases[i].seed), options.max_new_tokens,
+                    std::bit_cast<uint32_t>(options.sampling.temperature), options.sampling.top_k,
+                    std::bit_cast<uint32_t>(options.sampling.top_p), std::bit_cast<uint32_t>(options.sampling.min_p),
+                    options.enable_speculative ? 1 : 0, std::bit_cast<uint32_t>(options.speculative_confidence_threshold),
+                    options.speculative_max_draft_tokens);
+        for (int32_t id : options.stop_tokens)
+            std::printf(" %d", id);
+        std::printf("\n");
+        for (const StreamToken& token : results[i].tokens)
+            std::printf("token %zu %u %d %u %d\n", i, token.index, token.token_id, std::bit_cast<uint32_t>(token.probability),
+                        token.is_stop_token ? 1 : 0);
+        std::printf("result %zu tokens %zu stopped_by_stop_token %d stopped_by_callback %d\n", i, results[i].tokens.size(),
+                    results[i].stopped_by_stop_token ? 1 : 0, results[i].stopped_by_callback ? 1 : 0);
+    }
+}
+
+// --speculative-trace 0|1: the speculative loop without / with state cache transactions, printed like --generation-trace
+static int print_speculative_trace(const HipSamplerPtr& sampler, bool transactions)
+{
+    const std::vector<LoopCase> cases = speculative_cases();
+    const std::vector<GenerationResult> results = run_speculative(sampler, cases, transactions);
+    print_trace_lines(cases, results);
+    std::printf("vocab %u\nblock %u\ntransactions %d\n", kLoopVocab, kSpeculativeBlock, transactions ? 1 : 0);
+    return 0;
 }
 
 // Prints "session index token_id probability_bits is_stop" per emitted token and a summary line per
@@ -1536,6 +1819,7 @@ int main(int argc, char** argv)
                                 static_cast<uint32_t>(std::atoi(argv[4])));
     const bool host_only = argc > 1 && std::strcmp(argv[1], "--host") == 0;
     const bool trace_only = argc > 1 && std::strcmp(argv[1], "--generation-trace") == 0;
+    const bool speculative_trace = argc > 2 && std::strcmp(argv[1], "--speculative-trace") == 0;
     try
     {
         test_option_validation_messages();
@@ -1559,6 +1843,8 @@ int main(int argc, char** argv)
         }
         if (trace_only)
             return print_generation_trace(sampler);
+        if (speculative_trace)
+            return print_speculative_trace(sampler, std::atoi(argv[2]) != 0);
         test_sampling_like_the_runtime_test(sampler);
         test_rng_bookkeeping(sampler);
         test_distribution_known_answers(sampler);
@@ -1574,6 +1860,7 @@ int main(int argc, char** argv)
         test_scheduler_over_several_samplers(sampler);
         test_generation_loop_equals_serial(sampler);
         test_generation_loop_callback_and_errors(sampler);
+        test_speculative_generation_loop(sampler);
     }
     catch (const std::exception& error)
     {
