@@ -423,6 +423,29 @@ def bench_scheduler(args):
     print(json.dumps(line))
 
 
+def bench_geometry_sweep(args):
+    """The select path over batch sizes, row lengths and both logits types at configuration 2's options (T 0.7,
+    Top-K 20, Top-P 0.8): one run of this script per shape (--rows, --vocab, --logits-dtype; one rotated buffer
+    checked against the CPU oracle), one table line each: microseconds per step, share of the 8 TB/s roofline,
+    the kernel variant that served the shape, token mismatches."""
+    import subprocess
+    print("%5s %8s %5s  %-58s %9s %8s %11s" % ("rows", "vocab", "type", "kernel, grid", "us/step", "% peak", "mismatches"), flush=True)
+    for dtype in ((args.logits_dtype,) if args.logits_dtype else ("f32", "bf16")):
+        for vocab in (32000, 129280, 151936, 201088, 262144):
+            for rows in (1, 8, 32, 64, 128, 192, 256, 384, 512):
+                steps = max(60, min(600, int(3e9 / (rows * vocab * (4 if dtype == "f32" else 2)))))
+                done = subprocess.run([sys.executable, os.path.abspath(__file__), "--workload", "cfg2_topk_topp", "--rows", str(rows),
+                                       "--vocab", str(vocab), "--logits-dtype", dtype, "--steps", str(steps), "--warmup", "10",
+                                       "--no-cpu-baseline", "--parity-buffers", "1"], capture_output=True, text=True, timeout=600)
+                if done.returncode != 0:
+                    sys.exit("shape %d x %d %s failed: %s" % (rows, vocab, dtype, done.stderr[-600:]))
+                line = json.loads(done.stdout.strip().splitlines()[-1])
+                parity = line["parity"]
+                print("%5d %8d %5s  %-58s %9.2f %8.1f %11d" % (
+                    rows, vocab, dtype, line["roofline"]["kernel"][:58], line["ms_per_step"] * 1e3, 100.0 * line["roofline"]["frac"],
+                    parity["token_mismatches"] + parity["probability_bit_mismatches"] + parity["status_mismatches"]), flush=True)
+
+
 def bench_timeline(args):
     """Where the time of a split-row launch goes: the library built with wall-clock stamps in the split
     kernel (make -C ncnn-moe-runtime_amd timeline) runs bursts of 12 launches over rotated logits buffers;
@@ -573,6 +596,13 @@ def main():
     parser.add_argument("--warmup", type=int, default=200)
     parser.add_argument("--workload", default="cfg2_topk_topp")
     parser.add_argument("--rows", type=int, default=0, help="batch rows (0: the configuration's own)")
+    parser.add_argument("--vocab", type=int, default=0, help="row length (0: the configuration's own)")
+    parser.add_argument("--logits-dtype", default="", choices=["", "f32", "bf16"],
+                        help="store the configuration's logits as fp32 or bf16 instead of its own type")
+    parser.add_argument("--parity-buffers", type=int, default=0,
+                        help="rotated buffers checked against the CPU oracle (0: every one; a sweep over large shapes checks one)")
+    parser.add_argument("--geometry-sweep", action="store_true",
+                        help="the select path at B x V x {fp32, bf16}, K = 20 (configuration 2's options): one table line per shape")
     parser.add_argument("--batches-in-flight", action="store_true",
                         help="also time 2 and 4 independent batches in flight (detail only; their launches overlap, "
                              "so leave it off under a kernel trace)")
@@ -597,6 +627,9 @@ def main():
 
     load_package()
     from ncnn_moe_runtime_amd import hip_sampler, workloads
+    if args.geometry_sweep:
+        bench_geometry_sweep(args)
+        return
     if args.timeline:
         if args.workload in ("cfg3_full_nucleus", "cfg4_service_mix"):
             bench_full_order_timeline(args)
@@ -621,7 +654,14 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    workload = workloads.make_workload(args.workload, rows=args.rows if args.rows > 0 else None)
+    workload = workloads.make_workload(args.workload, rows=args.rows if args.rows > 0 else None, vocab=args.vocab if args.vocab > 0 else None)
+    if args.logits_dtype and args.logits_dtype != workload["dtype"]:
+        if args.logits_dtype == "bf16":
+            workload["logits"] = workloads.float32_to_bf16_bits(workload["logits"])
+        else:
+            workload["logits"] = workloads.bf16_bits_to_float32(workload["logits"])
+        workload["dtype"] = args.logits_dtype
+        workload["description"] += " [logits stored as %s]" % args.logits_dtype
     rows, vocab = workload["rows"], workload["vocab"]
     element_bytes = 4 if workload["dtype"] == "f32" else 2
     dtype_code = hip_sampler.LOGITS_F32 if workload["dtype"] == "f32" else hip_sampler.LOGITS_BF16
@@ -798,7 +838,8 @@ def main():
     import parity_util
     host_threads = min(16, os.cpu_count() or 1)
     parity = None
-    for index in range(buffers):
+    checked_buffers = buffers if args.parity_buffers <= 0 else min(buffers, args.parity_buffers)
+    for index in range(checked_buffers):
         host_buffer = workload["logits"] if index == 0 else logits[index].cpu().numpy().view(workload["logits"].dtype)
         cpu = oracle_lib.oracle_sample_batch(host_buffer, workload["params"], workload["uniforms"],
                                              workload["stop_ids"], threads=host_threads)
@@ -810,11 +851,12 @@ def main():
         else:
             for key, value in counters.items():
                 parity[key] += value
-    parity["buffers_checked"] = buffers
+    parity["buffers_checked"] = checked_buffers
 
     bytes_per_launch = algorithmic_bytes(rows, vocab, element_bytes)
     achieved = bytes_per_launch / seconds_per_step
-    traffic, traffic_file = measured_traffic(workload["name"]) if args.rows == 0 else (None, None)
+    own_shape = args.rows == 0 and args.vocab == 0 and not args.logits_dtype
+    traffic, traffic_file = measured_traffic(workload["name"]) if own_shape else (None, None)
     segments, chunks, variant = hip_sampler.select_geometry(dtype_code, rows, vocab)
     kernel = {hip_sampler.GEOMETRY_WHOLE_ROW: "scan_select_kernel (one workgroup per row)",
               hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK: "split_select_kernel (%d one-chunk workgroups per row)" % segments,
@@ -822,8 +864,8 @@ def main():
     if may_need_full_order:
         kernel += " + the later passes for rows without a Top-K window of at most 64 (wide select, sort, replay)"
     metric = METRICS.get(workload["name"], "sampled rows/sec + HBM GB/s (% peak), " + workload["name"])
-    if args.rows > 0:
-        metric += " [rows overridden: %d]" % rows
+    if not own_shape:
+        metric += " [shape overridden: %d x %d %s]" % (rows, vocab, workload["dtype"])
     line = {
         "metric": metric,
         "value": rows / seconds_per_step,

@@ -30,6 +30,9 @@ int ncnn_moe_hip_sampler_debug_chunk_steps(ncnn_moe_hip_sampler* sampler, int en
 /* spread_sort (on by default): the radix sort of a long full-order row runs on several workgroups; off,
  * every row is sorted by one workgroup. */
 int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* sampler, int enabled);
+/* fused_bf16 (on by default): a bf16 full-order row is counted and walked by one kernel, its runs staying in LDS; off,
+ * by the counting kernel and the replay kernel, with the runs in device memory between them.  Same results either way. */
+int ncnn_moe_hip_sampler_debug_fused_bf16(ncnn_moe_hip_sampler* sampler, int enabled);
 /* Sets the per-row launch numbers (epochs, 1 .. 16383) that tag the split kernel's hand-over records: of the
  * handle, or with a null handle of the static scratch of `device` (after it has served a call).  Tests start a
  * few launches in front of the point where the epochs start over. */

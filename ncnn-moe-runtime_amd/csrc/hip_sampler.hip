@@ -28,6 +28,7 @@ struct ncnn_moe_hip_sampler
     int force_general = 0;
     int scatter_segments = 0;
     int spread_sort = 1; // a long row's radix sort runs on several workgroups
+    int fused_bf16 = 1;  // bf16 full-order rows are counted and walked by one kernel
     // a call with rows for the wide select and rows for the full-order kernels runs the two side by side
     hipStream_t side_stream = nullptr;
     hipEvent_t side_fork = nullptr;
@@ -378,7 +379,11 @@ int launch_sampler(
         };
         using F32 = std::integral_constant<int, NCNN_MOE_LOGITS_F32>;
         using BF16 = std::integral_constant<int, NCNN_MOE_LOGITS_BF16>;
-        if (runs)
+        // (bf16 rows that need no exported distribution: counted and walked by one kernel, unless a test asks for the two)
+        const bool fused_runs = runs && s->fused_bf16 != 0;
+        if (fused_runs)
+            hipLaunchKernelGGL(bf16_counting_replay_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
+        else if (runs)
             hipLaunchKernelGGL(bf16_counting_sort_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
         else if (dtype == NCNN_MOE_LOGITS_F32 && want_distribution)
             sort_rows(F32{}, std::true_type{});
@@ -398,6 +403,8 @@ int launch_sampler(
                 a.chunk_steps_ready = 1;
             }
         }
+        if (fused_runs)
+            return;
         if (runs)
             hipLaunchKernelGGL((general_replay_kernel<NCNN_MOE_LOGITS_BF16, true>), dim3(rows), dim3(kReplayThreads), 0, stream, a);
         else if (dtype == NCNN_MOE_LOGITS_F32)
@@ -1157,6 +1164,14 @@ int ncnn_moe_hip_sampler_debug_set_row_epochs(ncnn_moe_hip_sampler* s, int devic
         hipMemsetD32(reinterpret_cast<hipDeviceptr_t>(epochs), static_cast<int>(epoch), count) != hipSuccess ||
         hipDeviceSynchronize() != hipSuccess)
         return NCNN_MOE_SAMPLER_HIP_ERROR;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+int ncnn_moe_hip_sampler_debug_fused_bf16(ncnn_moe_hip_sampler* s, int enabled)
+{
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    s->fused_bf16 = enabled ? 1 : 0;
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

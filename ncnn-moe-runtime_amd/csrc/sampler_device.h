@@ -344,6 +344,16 @@ __device__ __forceinline__ void lds_barrier()
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// A 16-byte load from device memory through a pointer whose address space the compiler cannot see (an argument
+// of a function that is not inlined): as a global load it counts against the vector-memory counter only, where a
+// flat load also counts as an LDS operation and is waited for by lds_barrier().
+__device__ __forceinline__ uint4 load_global_uint4(const void* address)
+{
+    typedef uint32_t NativeVector __attribute__((ext_vector_type(4)));
+    const NativeVector loaded = *(const __attribute__((address_space(1))) NativeVector*)(address);
+    return make_uint4(loaded.x, loaded.y, loaded.z, loaded.w);
+}
+
 // Agent-scope relaxed accesses: they write through / read around the per-XCD L2, so data handed from
 // one workgroup to another needs no L2 write-back or invalidate, only a wait for the stores to land.
 __device__ __forceinline__ void store_agent(uint32_t* address, uint32_t value)

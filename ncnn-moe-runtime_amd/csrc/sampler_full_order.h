@@ -749,66 +749,108 @@ __device__ __forceinline__ bool fold_special_bf16_counts(uint32_t* bins, int tid
     return fits;
 }
 
+constexpr int kCountBlocks = kCountWords / kWaveSize; // blocks of 64 consecutive counter words
+
 struct CountScratch
 {
-    uint32_t wave_totals[kSortWaves];
-    uint32_t wave_runs[kSortWaves];
+    alignas(16) uint32_t block_totals[kCountBlocks]; // elements counted in each block
+    alignas(16) uint32_t block_runs[kCountBlocks];   // counters above zero in each block
 };
 
-// Turns the counters into runs.  Wave w owns words [2048 w, 2048 (w + 1)) and reads them 64 consecutive
-// words at a time (lane l of trip j: word 2048 w + 64 j + l: no bank conflicts), so the order of the keys
-// inside the wave is (trip, lane, half).  Returns false (and writes nothing) when PACKED counters have
-// overflowed.  key_base: key16 of word 0's first counter; written / runs_written: totals of an earlier round.
+// Turns the counters into runs.  The words are taken 64 consecutive ones at a time (a block: lane l reads word
+// 64 b + l, no bank conflicts), and block b belongs to wave b % 16: the keys in use lie close together (a row of
+// logits between -8 and 16 touches four of sixteen equal stretches of the key space), and dealt out this way every
+// wave gets its share of them.  The order of the keys is (block, lane, half).  Returns false (and writes nothing)
+// when PACKED counters have overflowed.  key_base: key16 of word 0's first counter; written / runs_written: totals
+// of an earlier round.
+// in_place != nullptr (PACKED only, first round): when the row's runs fit `in_place_capacity`, they are written over
+// the counters themselves (every counter is in a register by then), keys from bins[0] on and ends from
+// bins[in_place_capacity] on, instead of to run_keys / run_ends; *in_place tells which.
 template <bool PACKED>
 __device__ __forceinline__ bool write_runs_of_counts(
-    const uint32_t* bins, uint32_t expected, uint32_t key_base, uint32_t& written, uint32_t& runs_written,
-    uint32_t* run_keys, uint32_t* run_ends, CountScratch& scratch, int tid)
+    uint32_t* bins, uint32_t expected, uint32_t key_base, uint32_t& written, uint32_t& runs_written,
+    uint32_t* run_keys, uint32_t* run_ends, CountScratch& scratch, int tid, bool* in_place = nullptr, uint32_t in_place_capacity = 0)
 {
-    constexpr int kTrips = kCountWords / kSortWaves / kWaveSize; // 32
+    constexpr int kTrips = kCountBlocks / kSortWaves; // 32
+    static_assert(kTrips == 32 && kSortWaves == 16, "a wave's block totals fill lanes 0..31; eight blocks a lane in the scan");
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
-    const uint32_t wave_first_word = static_cast<uint32_t>(wave) * (kTrips * kWaveSize);
     uint32_t words[kTrips];
-    uint32_t lane_total = 0, lane_runs = 0;
+    uint32_t my_total = 0, my_runs = 0; // lane j: the totals of the wave's trip j
+#pragma unroll
+    for (int j = 0; j < kTrips; ++j)
+        words[j] = bins[static_cast<uint32_t>((j * kSortWaves + wave) * kWaveSize + lane)];
 #pragma unroll
     for (int j = 0; j < kTrips; ++j)
     {
-        words[j] = bins[wave_first_word + static_cast<uint32_t>(j * kWaveSize + lane)];
+        if (__ballot(words[j] != 0u) == 0ull)
+            continue; // most blocks are empty
+        const uint32_t low = PACKED ? (words[j] & 0xffffu) : words[j];
+        const uint32_t high = PACKED ? (words[j] >> 16) : 0u;
+        const uint32_t lane_runs = (low != 0u ? 1u : 0u) + (high != 0u ? 1u : 0u);
+        uint32_t block_total, block_runs;
         if (PACKED)
         {
-            lane_total += (words[j] & 0xffffu) + (words[j] >> 16);
-            lane_runs += ((words[j] & 0xffffu) != 0u ? 1u : 0u) + ((words[j] >> 16) != 0u ? 1u : 0u);
+            // one sum for both: a block's 16-bit counters sum to less than 2^23, its runs to at most 128
+            const uint32_t both = static_cast<uint32_t>(
+                __builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(((low + high) << 8) | lane_runs)), 63));
+            block_total = both >> 8;
+            block_runs = both & 0xffu;
         }
         else
         {
-            lane_total += words[j];
-            lane_runs += words[j] != 0u ? 1u : 0u;
+            block_total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(low)), 63));
+            block_runs = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(lane_runs)), 63));
         }
+        my_total = lane == j ? block_total : my_total;
+        my_runs = lane == j ? block_runs : my_runs;
     }
-    const uint32_t wave_total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(lane_total)), 63));
-    const uint32_t wave_run_total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(lane_runs)), 63));
-    if (lane == 0)
+    if (lane < kTrips)
     {
-        scratch.wave_totals[wave] = wave_total;
-        scratch.wave_runs[wave] = wave_run_total;
+        scratch.block_totals[lane * kSortWaves + wave] = my_total;
+        scratch.block_runs[lane * kSortWaves + wave] = my_runs;
     }
-    __syncthreads();
-    uint32_t position = written;      // elements before the keys this wave looks at next
-    uint32_t run = runs_written;      // runs before them
-    uint32_t all = 0, all_runs = 0;
+    __syncthreads(); // every counter is in a register now, every block total in the scratch
+    // Every wave scans the 512 block totals: lane l takes blocks 8 l .. 8 l + 7.  The wave's trip j is block
+    // 16 j + wave: lane 2 j + wave / 8, slot wave % 8.
+    uint32_t first_element, first_run; // of this lane's block of slot wave % 8, before `written` / `runs_written`
+    uint32_t all, all_runs;
+    {
+        const uint4 t0 = *reinterpret_cast<const uint4*>(&scratch.block_totals[8 * lane]);
+        const uint4 t1 = *reinterpret_cast<const uint4*>(&scratch.block_totals[8 * lane + 4]);
+        const uint4 r0 = *reinterpret_cast<const uint4*>(&scratch.block_runs[8 * lane]);
+        const uint4 r1 = *reinterpret_cast<const uint4*>(&scratch.block_runs[8 * lane + 4]);
+        const uint32_t totals[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+        const uint32_t runs[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+        uint32_t lane_total = 0, lane_runs = 0;
+        uint32_t slot_total = 0, slot_runs = 0; // of the slots in front of slot wave % 8
 #pragma unroll
-    for (int w = 0; w < kSortWaves; ++w)
-    {
-        const uint32_t t = scratch.wave_totals[w];
-        const uint32_t r = scratch.wave_runs[w];
-        position += w < wave ? t : 0u;
-        run += w < wave ? r : 0u;
-        all += t;
-        all_runs += r;
+        for (int i = 0; i < 8; ++i)
+        {
+            slot_total = i == (wave & 7) ? lane_total : slot_total;
+            slot_runs = i == (wave & 7) ? lane_runs : slot_runs;
+            lane_total += totals[i];
+            lane_runs += runs[i];
+        }
+        const uint32_t inclusive_total = wave_prefix_sum_u32(lane_total);
+        const uint32_t inclusive_runs = wave_prefix_sum_u32(lane_runs);
+        first_element = inclusive_total - lane_total + slot_total;
+        first_run = inclusive_runs - lane_runs + slot_runs;
+        all = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive_total), 63));
+        all_runs = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive_runs), 63));
     }
     __syncthreads(); // the scratch is written again by a later call
     if (PACKED && all != expected)
         return false;
+    if (in_place != nullptr)
+    {
+        *in_place = runs_written == 0u && all_runs <= in_place_capacity;
+        if (*in_place)
+        {
+            run_keys = bins;
+            run_ends = bins + in_place_capacity;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < kTrips; ++j)
     {
@@ -818,10 +860,13 @@ __device__ __forceinline__ bool write_runs_of_counts(
         const uint64_t has_high = PACKED ? __ballot(high != 0u) : 0ull;
         if ((has_low | has_high) == 0ull)
             continue;
+        const uint32_t source = static_cast<uint32_t>(2 * j + (wave >> 3));
+        const uint32_t position = written + static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(first_element), source));
+        const uint32_t run = runs_written + static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(first_run), source));
         const uint32_t inclusive = wave_prefix_sum_u32(low + high);
         const uint32_t before = position + inclusive - (low + high);
         uint32_t slot = run + static_cast<uint32_t>(lanes_below(has_low) + lanes_below(has_high));
-        const uint32_t word = wave_first_word + static_cast<uint32_t>(j * kWaveSize + lane);
+        const uint32_t word = static_cast<uint32_t>((j * kSortWaves + wave) * kWaveSize + lane);
         const uint32_t first_key16 = key_base + (PACKED ? 2u * word : word);
         // the lower half of a key is all ones for a non-negative logit and for NaN, else zero
         const auto full_key = [](uint32_t key16) {
@@ -838,8 +883,6 @@ __device__ __forceinline__ bool write_runs_of_counts(
             run_keys[slot] = full_key(first_key16 + 1u);
             run_ends[slot] = before + low + high;
         }
-        position += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive), 63));
-        run += static_cast<uint32_t>(__popcll(has_low) + __popcll(has_high));
     }
     written += all;
     runs_written += all_runs;
@@ -916,31 +959,36 @@ struct RecoverScratch
 // Every thread of the workgroup must call it.
 template <int DTYPE>
 __device__ __noinline__ int32_t recover_token_of_key(
-    const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, RecoverScratch& scratch, int tid);
+    const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, uint32_t occurrences, RecoverScratch& scratch, int tid);
 
 template <int DTYPE>
 __device__ __forceinline__ int32_t recover_token_index(
     const void* row_pointer, uint32_t vocab, const uint32_t* keys, uint32_t rank, RecoverScratch& scratch, int tid)
 {
     const uint32_t key = keys[rank];
-    // first position holding this key
+    // first position holding this key, and the first behind it
     const uint32_t low = wave_partition_point(rank, [keys, key](uint32_t position) { return keys[position] < key; });
-    return recover_token_of_key<DTYPE>(row_pointer, vocab, key, rank - low, scratch, tid);
+    const uint32_t high = rank + 1u +
+        wave_partition_point(vocab - rank - 1u, [keys, key, rank](uint32_t position) { return keys[rank + 1u + position] <= key; });
+    return recover_token_of_key<DTYPE>(row_pointer, vocab, key, rank - low, high - low, scratch, tid);
 }
 
-// The ordinal-th element of the row, in index order, whose key equals `key`.  The workgroup reads the row
-// front to back in trips of sixteen consecutive slices, one per wave (16-byte loads, eight per lane in
-// flight); after each trip the waves' match counts tell whether the wanted match lies in it, and the wave
-// whose slice holds it locates the element from the masks it still has in registers.  The row is read
-// once, and only as far as the match.  Every thread of the workgroup must call it.
+// The ordinal-th of the `occurrences` elements of the row, in index order, whose key equals `key`.  The workgroup
+// reads the row from the end that is nearer in occurrences (front to back for the first half of them, back to front
+// for the rest: a quarter of the row on average instead of half, half of it at most), in trips of sixteen
+// consecutive slices, one per wave; the 16-byte loads of the next trip are in flight while this one's matches are
+// counted (the barrier between trips does not wait for them).  After each trip the waves' match counts tell whether
+// the wanted match lies in it, and the wave whose slice holds it locates the element from the masks it still has in
+// registers.  Every thread of the workgroup must call it.
 template <int DTYPE>
 __device__ __noinline__ int32_t recover_token_of_key(
-    const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, RecoverScratch& scratch, int tid)
+    const void* row_pointer, uint32_t vocab, uint32_t key, uint32_t ordinal, uint32_t occurrences, RecoverScratch& scratch, int tid)
 {
     using Vector = LogitsVector<DTYPE>;
     constexpr uint32_t kWidth = Vector::kWidth;
-    constexpr int kLoads = 8;
+    constexpr int kLoads = 4;
     constexpr uint32_t kSlice = kLoads * kWaveSize * kWidth; // positions a wave looks at per trip
+    constexpr uint32_t kTrip = kSlice * kReplayWaves;
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
     // positions count from the 16-byte boundary below the row: [misalignment, end) hold the row
@@ -948,51 +996,78 @@ __device__ __noinline__ int32_t recover_token_of_key(
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row_pointer) & 15u) / Vector::kElementBytes;
     const char* aligned_base = static_cast<const char*>(row_pointer) - static_cast<size_t>(misalignment) * Vector::kElementBytes;
     const uint32_t end = misalignment + vocab;
+    const uint32_t trips = (end + kTrip - 1u) / kTrip;
 
     // An element matches when its key equals `key`.  Keys are one-to-one with the logits' bit patterns except
     // that the two zeros share a key, and all NaNs another: the raw bits are compared (with the sign masked for
-    // zero), which takes a third of the instructions of building every element's key.
+    // zero), which takes a third of the instructions of building every element's key.  One test without a branch
+    // serves all three cases, with constants that are the same in every lane:
+    //   ((bits & kept) ^ flipped) - floor <= room     (unsigned; a difference below zero wraps far above `room`)
+    // a value: kept = every bit (no sign for zero), flipped = its pattern, floor = room = 0: equality;
+    // NaN: kept = the bits without the sign, flipped = 0, floor = infinity + 1, room = the patterns above that.
+    // A bf16 logit is tested where it lies in its 32-bit word, the constants shifted to the upper half for the odd ones.
     constexpr uint32_t kAbsoluteBits = DTYPE == NCNN_MOE_LOGITS_F32 ? 0x7fffffffu : 0x7fffu;
+    constexpr uint32_t kEveryBit = DTYPE == NCNN_MOE_LOGITS_F32 ? 0xffffffffu : 0xffffu;
     constexpr uint32_t kInfinityBits = DTYPE == NCNN_MOE_LOGITS_F32 ? 0x7f800000u : 0x7f80u;
     const bool wants_nan = key == 0xffffffffu;
     const uint32_t value_bits = __float_as_uint(value_from_descending_key(key));
     const uint32_t pattern = DTYPE == NCNN_MOE_LOGITS_F32 ? value_bits : value_bits >> 16;
-    const uint32_t compared = (pattern & kAbsoluteBits) == 0u ? kAbsoluteBits : 0xffffffffu;
-    const auto matches_key = [&](uint32_t bits) {
-        const bool is_nan = (bits & kAbsoluteBits) > kInfinityBits;
-        return wants_nan ? is_nan : ((bits ^ pattern) & compared) == 0u;
+    const uint32_t kept = wants_nan || (pattern & kAbsoluteBits) == 0u ? kAbsoluteBits : kEveryBit;
+    const uint32_t flipped = wants_nan ? 0u : pattern & kept;
+    const uint32_t floor = wants_nan ? kInfinityBits + 1u : 0u;
+    const uint32_t room = wants_nan ? kAbsoluteBits - (kInfinityBits + 1u) : 0u;
+    const uint32_t kept_high = kept << 16, flipped_high = flipped << 16, floor_high = floor << 16, room_high = room << 16;
+    // the matches among the kWidth logits of one 16-byte load, bit c for the c-th
+    const auto matches_of = [&](const uint4& loaded) {
+        const uint32_t words[4] = {loaded.x, loaded.y, loaded.z, loaded.w};
+        uint32_t mask = 0;
+#pragma unroll
+        for (uint32_t c = 0; c < kWidth; ++c)
+        {
+            bool match;
+            if (DTYPE == NCNN_MOE_LOGITS_F32)
+                match = ((words[c] & kept) ^ flipped) - floor <= room;
+            else if ((c & 1u) == 0u)
+                match = ((words[c >> 1] & kept) ^ flipped) - floor <= room;
+            else
+                match = ((words[c >> 1] & kept_high) ^ flipped_high) - floor_high <= room_high;
+            mask |= match ? 1u << c : 0u;
+        }
+        return mask;
     };
+
+    // backward: the wanted match is the target-th counted from the row's end, and everything below counts from there
+    const bool backward = ordinal < occurrences && ordinal >= occurrences - ordinal;
+    const uint32_t target = backward ? occurrences - 1u - ordinal : ordinal;
 
     if (tid == 0)
         scratch.found = -1;
-    uint32_t seen = 0; // matches in the trips before this one
-    uint32_t parity = 0;
-    for (uint32_t trip = 0; trip < end; trip += kSlice * kReplayWaves, parity ^= 1u)
-    {
-        const uint32_t first = trip + static_cast<uint32_t>(wave) * kSlice;
-        // per load k: the lane's matches among the kWidth positions from first + (k * 64 + lane) * kWidth
-        uint4 raw[kLoads];
+    const auto load_trip = [&](uint32_t trip, uint4 (&raw)[kLoads]) {
+        const uint32_t first = trip * kTrip + static_cast<uint32_t>(wave) * kSlice;
 #pragma unroll
         for (int k = 0; k < kLoads; ++k)
         {
             const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth;
-            raw[k] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(position < end ? position : 0u) * Vector::kElementBytes);
+            raw[k] = load_global_uint4(aligned_base + static_cast<size_t>(position < end ? position : 0u) * Vector::kElementBytes);
         }
+    };
+    uint32_t seen = 0; // matches in the trips before this one
+    // One trip: starts the loads of the next into `next`, counts the matches of `raw`.  True when the search is over.
+    const auto search_trip = [&](uint32_t step, uint4 (&raw)[kLoads], uint4 (&next)[kLoads]) -> bool {
+        const uint32_t trip = backward ? trips - 1u - step : step;
+        // (the last step loads its own trip again: a load under a condition would make the wait below one for every
+        // load in flight, the new ones included)
+        load_trip(step + 1u < trips ? (backward ? trip - 1u : trip + 1u) : trip, next);
+        const uint32_t parity = step & 1u;
+        const uint32_t first = trip * kTrip + static_cast<uint32_t>(wave) * kSlice;
+        // per load k: the lane's matches among the kWidth positions from first + (k * 64 + lane) * kWidth
         uint32_t masks[kLoads];
         uint32_t lane_matches = 0;
 #pragma unroll
         for (int k = 0; k < kLoads; ++k)
         {
             const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth;
-            const uint32_t words[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
-            uint32_t mask = 0;
-#pragma unroll
-            for (uint32_t c = 0; c < kWidth; ++c)
-            {
-                const uint32_t bits = DTYPE == NCNN_MOE_LOGITS_F32 ? words[c]
-                                                                   : ((c & 1u) ? words[c >> 1] >> 16 : words[c >> 1] & 0xffffu);
-                mask |= matches_key(bits) ? 1u << c : 0u;
-            }
+            const uint32_t mask = matches_of(raw[k]);
             // positions in front of the row's first element and behind its last are no elements of it
             const uint32_t below = position < misalignment ? min(misalignment - position, kWidth) : 0u;
             const uint32_t inside = position < end ? min(end - position, kWidth) : 0u;
@@ -1003,50 +1078,65 @@ __device__ __noinline__ int32_t recover_token_of_key(
             static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(lane_matches)), kWaveSize - 1));
         if (lane == 0)
             scratch.wave_counts[parity][wave] = wave_matches;
-        __syncthreads();
-        uint32_t before = seen; // matches in front of this wave's slice
-        uint32_t trip_matches = 0;
-#pragma unroll
-        for (int w = 0; w < kReplayWaves; ++w)
+        lds_barrier();
+        // lane w holds wave w's count; a prefix sum over the lanes gives every wave the matches on either side of it
+        const uint32_t count_of_lane = lane < kReplayWaves ? scratch.wave_counts[parity][lane] : 0u;
+        const uint32_t through_lane = wave_prefix_sum_u32(count_of_lane);
+        const uint32_t trip_matches = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(through_lane), kReplayWaves - 1));
+        const uint32_t through_wave = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(through_lane), wave));
+        // matches between the end the search started from and this wave's slice
+        const uint32_t skipped = seen + (backward ? trip_matches - through_wave : through_wave - wave_matches);
+        if (target >= seen + trip_matches)
         {
-            const uint32_t count = scratch.wave_counts[parity][w];
-            before += w < wave ? count : 0u;
-            trip_matches += count;
+            seen += trip_matches;
+            return step + 1u >= trips;
         }
-        if (ordinal < seen + trip_matches)
+        if (target >= skipped && target < skipped + wave_matches)
         {
-            if (ordinal >= before && ordinal < before + wave_matches)
+            uint32_t remaining = target - skipped; // matches of this slice still to skip
+            bool done = false;
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i)
             {
-                uint32_t remaining = ordinal - before; // matches of this slice still to skip
-                bool done = false;
-#pragma unroll
-                for (int k = 0; k < kLoads; ++k)
+                // (static indices either way: the loads are looked at in the search's direction)
+                const uint32_t load_mask = backward ? masks[kLoads - 1 - i] : masks[i];
+                const uint32_t k = backward ? static_cast<uint32_t>(kLoads - 1 - i) : static_cast<uint32_t>(i);
+                if (done || __ballot(load_mask != 0u) == 0)
+                    continue; // most loads hold no match at all: no scan for them
+                const uint32_t count = static_cast<uint32_t>(__popc(load_mask));
+                const uint32_t inclusive = wave_prefix_sum_u32(count); // matches in lanes 0..lane of this load
+                const uint32_t total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive), kWaveSize - 1));
+                if (remaining < total)
                 {
-                    if (done || __ballot(masks[k] != 0u) == 0)
-                        continue; // most loads hold no match at all: no scan for them
-                    const uint32_t count = static_cast<uint32_t>(__popc(masks[k]));
-                    const uint32_t inclusive = wave_prefix_sum_u32(count); // matches in lanes 0..lane of this load
-                    const uint32_t total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(inclusive), kWaveSize - 1));
-                    if (remaining < total)
+                    // matches of this load that the search passes before it reaches this lane's
+                    const uint32_t passed = backward ? total - inclusive : inclusive - count;
+                    if (remaining >= passed && remaining < passed + count)
                     {
-                        if (remaining >= inclusive - count && remaining < inclusive)
-                        {
-                            uint32_t mask = masks[k];
-                            for (uint32_t skipped = inclusive - count; skipped < remaining; ++skipped)
-                                mask &= mask - 1u;
-                            const uint32_t position = first + static_cast<uint32_t>(k * kWaveSize + lane) * kWidth +
-                                static_cast<uint32_t>(__builtin_ctz(mask));
-                            scratch.found = static_cast<int32_t>(position - misalignment);
-                        }
-                        done = true;
+                        uint32_t mask = load_mask;
+                        for (uint32_t dropped = passed; dropped < remaining; ++dropped)
+                            mask = backward ? mask & ~(0x80000000u >> __builtin_clz(mask)) : mask & (mask - 1u);
+                        const uint32_t bit = backward ? 31u - static_cast<uint32_t>(__builtin_clz(mask))
+                                                      : static_cast<uint32_t>(__builtin_ctz(mask));
+                        const uint32_t position = first + (k * kWaveSize + static_cast<uint32_t>(lane)) * kWidth + bit;
+                        scratch.found = static_cast<int32_t>(position - misalignment);
                     }
-                    else
-                        remaining -= total;
+                    done = true;
                 }
+                else
+                    remaining -= total;
             }
-            break;
         }
-        seen += trip_matches;
+        return true;
+    };
+    // two sets of registers take turns, so that no set is copied (a copy would wait for the loads it copies)
+    uint4 even[kLoads], odd[kLoads];
+    load_trip(backward ? trips - 1u : 0u, even);
+    for (uint32_t step = 0;; step += 2u)
+    {
+        if (search_trip(step, even, odd))
+            break;
+        if (search_trip(step + 1u, odd, even))
+            break;
     }
     __syncthreads();
     const int32_t found = scratch.found;
@@ -1057,74 +1147,19 @@ __device__ __noinline__ int32_t recover_token_of_key(
 // Full-order rows: walks the sorted row as the CPU sampler does (src/engine/session.cpp:84-134,
 // :429-442).  One workgroup per row.  With RUNS the row comes from bf16_counting_sort_kernel as runs
 // of equal keys; otherwise sort_keys[1] holds one key per element.
+// The walk over one sorted row, from the sorted keys (or runs) and their terms to the row's result.  Every thread
+// of the workgroup (kReplayThreads) calls it.
 template <int DTYPE, bool RUNS>
-__global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerArgs a)
+__device__ __forceinline__ void replay_row(
+    const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p, const uint32_t* keys, const uint32_t* run_ends,
+    uint32_t run_total, const float* terms0, int tid)
 {
-    const uint32_t row = blockIdx.x;
-    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
-        return;
-    const int tid = threadIdx.x;
-    NCNN_MOE_STAMP(blockIdx.x, 15, 0);
-    const ncnn_moe_sample_params p = a.params[row];
-    const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
-    const uint32_t* run_ends = RUNS ? a.sort_keys[0] + row * a.sort_stride : nullptr;
-    // exp(logit/T - maximum) of every item, computed once for the three sums that use it (greedy rows add nothing)
-    const float* terms0 = nullptr;
-    const auto term_of_key = [&p](uint32_t key, float maximum) {
-        return expf_libm(value_from_descending_key(key) / p.temperature - maximum);
-    };
-    if constexpr (RUNS)
-    {
-        // a row of few runs is walked from LDS; the terms of a longer one go to the sort's spare index buffer
-        __shared__ uint32_t cached_keys[kCachedRuns];
-        __shared__ uint32_t cached_ends[kCachedRuns];
-        __shared__ __align__(16) float cached_terms[kCachedRuns];
-        const uint32_t run_total = a.sort_indices[0][row * a.sort_stride];
-        const float maximum = value_from_descending_key(keys[0]) / p.temperature;
-        if (run_total <= static_cast<uint32_t>(kCachedRuns))
-        {
-            for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
-            {
-                const uint32_t key = keys[i];
-                cached_keys[i] = key;
-                cached_ends[i] = run_ends[i];
-                cached_terms[i] = term_of_key(key, maximum);
-            }
-            __syncthreads();
-            keys = cached_keys;
-            run_ends = cached_ends;
-            terms0 = cached_terms;
-        }
-        else
-        {
-            float* terms = reinterpret_cast<float*>(a.sort_indices[1] + row * a.sort_stride);
-            if (p.temperature != 0.0f)
-            {
-                for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
-                    terms[i] = term_of_key(keys[i], maximum);
-            }
-            __syncthreads();
-            terms0 = terms;
-        }
-    }
-    else
-    {
-        float* terms = reinterpret_cast<float*>(a.sort_keys[0] + row * a.sort_stride);
-        if (a.terms_precomputed == 0 && p.temperature != 0.0f)
-        {
-            const float maximum = value_from_descending_key(keys[0]) / p.temperature;
-            for (uint32_t i = threadIdx.x; i < a.vocab; i += kReplayThreads)
-                terms[i] = term_of_key(keys[i], maximum);
-            __syncthreads();
-        }
-        terms0 = terms;
-    }
     NCNN_MOE_STAMP(blockIdx.x, 15, 1);
     const bool have_indices = !RUNS && a.distribution_count != nullptr; // the pair sort ran: indices are valid
     const uint32_t* indices = have_indices ? a.sort_indices[1] + row * a.sort_stride : nullptr;
     const uint32_t vocab = a.vocab;
     // items: what `keys` holds one entry of (an element, or a run of equal keys)
-    const uint32_t items = RUNS ? a.sort_indices[0][row * a.sort_stride] : vocab;
+    const uint32_t items = RUNS ? run_total : vocab;
     const char* row_pointer = static_cast<const char*>(a.logits) +
         static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
 
@@ -1160,7 +1195,8 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
         if constexpr (RUNS)
         {
             const uint32_t run = run_of_element(layout, rank);
-            return recover_token_of_key<DTYPE>(row_pointer, vocab, keys[run], rank - run_first_element(layout, run), recover_scratch, tid);
+            const uint32_t run_first = run_first_element(layout, run);
+            return recover_token_of_key<DTYPE>(row_pointer, vocab, keys[run], rank - run_first, run_ends[run] - run_first, recover_scratch, tid);
         }
         else
             return recover_token_index<DTYPE>(row_pointer, vocab, keys, rank, recover_scratch, tid);
@@ -1217,6 +1253,187 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
             chunk_steps = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity;
     }
     replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0, chunk_steps, a.vocab);
+}
+
+template <int DTYPE, bool RUNS>
+__global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerArgs a)
+{
+    const uint32_t row = blockIdx.x;
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+        return;
+    const int tid = threadIdx.x;
+    NCNN_MOE_STAMP(blockIdx.x, 15, 0);
+    const ncnn_moe_sample_params p = a.params[row];
+    const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
+    uint32_t run_total_of_row = 0;
+    const uint32_t* run_ends = RUNS ? a.sort_keys[0] + row * a.sort_stride : nullptr;
+    // exp(logit/T - maximum) of every item, computed once for the three sums that use it (greedy rows add nothing)
+    const float* terms0 = nullptr;
+    const auto term_of_key = [&p](uint32_t key, float maximum) {
+        return expf_libm(value_from_descending_key(key) / p.temperature - maximum);
+    };
+    if constexpr (RUNS)
+    {
+        // a row of few runs is walked from LDS; the terms of a longer one go to the sort's spare index buffer
+        __shared__ uint32_t cached_keys[kCachedRuns];
+        __shared__ uint32_t cached_ends[kCachedRuns];
+        __shared__ __align__(16) float cached_terms[kCachedRuns];
+        const uint32_t run_total = a.sort_indices[0][row * a.sort_stride];
+        run_total_of_row = run_total;
+        const float maximum = value_from_descending_key(keys[0]) / p.temperature;
+        if (run_total <= static_cast<uint32_t>(kCachedRuns))
+        {
+            for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
+            {
+                const uint32_t key = keys[i];
+                cached_keys[i] = key;
+                cached_ends[i] = run_ends[i];
+                cached_terms[i] = term_of_key(key, maximum);
+            }
+            __syncthreads();
+            keys = cached_keys;
+            run_ends = cached_ends;
+            terms0 = cached_terms;
+        }
+        else
+        {
+            float* terms = reinterpret_cast<float*>(a.sort_indices[1] + row * a.sort_stride);
+            if (p.temperature != 0.0f)
+            {
+                for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
+                    terms[i] = term_of_key(keys[i], maximum);
+            }
+            __syncthreads();
+            terms0 = terms;
+        }
+    }
+    else
+    {
+        float* terms = reinterpret_cast<float*>(a.sort_keys[0] + row * a.sort_stride);
+        if (a.terms_precomputed == 0 && p.temperature != 0.0f)
+        {
+            const float maximum = value_from_descending_key(keys[0]) / p.temperature;
+            for (uint32_t i = threadIdx.x; i < a.vocab; i += kReplayThreads)
+                terms[i] = term_of_key(keys[i], maximum);
+            __syncthreads();
+        }
+        terms0 = terms;
+    }
+    replay_row<DTYPE, RUNS>(a, row, p, keys, run_ends, run_total_of_row, terms0, tid);
+}
+
+// bf16 full-order rows in ONE kernel: bf16_counting_sort_kernel and general_replay_kernel<BF16, runs> back to
+// back in one workgroup per row, which both are.  The runs never leave the compute unit: once every counter
+// sits in a register they are written over the counters themselves (keys, ends and, behind them, the terms: a
+// third of the 128 KB each), which saves the runs' trip through device memory and a launch.  A row with more
+// runs than that, or one whose counters overflowed 16 bits, writes its runs to device memory as the two
+// kernels do, and walks them from there.
+constexpr uint32_t kRunsInPlace = kCountWords / 3; // 10,922 runs with their ends and terms in the counters' LDS
+
+__global__ __launch_bounds__(kSortThreads) void bf16_counting_replay_kernel(SamplerArgs a)
+{
+    static_assert(kSortThreads == kReplayThreads, "the count and the walk share a workgroup");
+    const uint32_t row = blockIdx.x;
+    if (a.row_state[row] != kRowNeedsGeneral || left_to_the_wide_select(a, row))
+        return;
+    const int tid = threadIdx.x;
+    const uint32_t n = a.vocab;
+
+    __shared__ uint32_t arena[kCountWords];
+    __shared__ CountScratch scratch;
+    __shared__ uint32_t specials_fit;
+
+    const uint16_t* logits = reinterpret_cast<const uint16_t*>(
+        static_cast<const char*>(a.logits) + static_cast<size_t>(row) * a.row_stride * 2u);
+    uint32_t* global_keys = a.sort_keys[1] + row * a.sort_stride;
+    uint32_t* global_ends = a.sort_keys[0] + row * a.sort_stride;
+    const uint32_t misalignment = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(logits) & 15u) / 2u;
+    const uint16_t* aligned_logits = logits - misalignment;
+    const uint32_t aligned_end = misalignment + n;
+
+    const auto clear_bins = [&]() {
+        uint4* wide = reinterpret_cast<uint4*>(arena);
+#pragma unroll
+        for (int j = 0; j < kCountWords / 4 / kSortThreads; ++j)
+            wide[j * kSortThreads + tid] = uint4{0u, 0u, 0u, 0u};
+        __syncthreads();
+    };
+    uint32_t runs_written = 0;
+    uint32_t written = 0;
+    NCNN_MOE_STAMP(blockIdx.x, 14, 0);
+    clear_bins();
+    count_bf16_keys<true>(aligned_logits, misalignment, aligned_end, 0u, arena, tid);
+    __syncthreads();
+    {
+        const bool fits = fold_special_bf16_counts(arena, tid);
+        if (tid == 0)
+            specials_fit = fits ? 1u : 0u;
+    }
+    __syncthreads();
+    NCNN_MOE_STAMP(blockIdx.x, 14, 1);
+    bool in_place = false;
+    const bool packed_sound = write_runs_of_counts<true>(
+        arena, specials_fit != 0u ? n : 0xffffffffu, 0u, written, runs_written, global_keys, global_ends, scratch, tid, &in_place, kRunsInPlace);
+    NCNN_MOE_STAMP(blockIdx.x, 14, 2);
+    if (!packed_sound)
+    {
+        in_place = false;
+        for (uint32_t round = 0; round < 2; ++round)
+        {
+            __syncthreads();
+            clear_bins();
+            count_bf16_keys<false>(aligned_logits, misalignment, aligned_end, round, arena, tid);
+            __syncthreads();
+            write_runs_of_counts<false>(arena, 0u, round << 15, written, runs_written, global_keys, global_ends, scratch, tid);
+        }
+    }
+    __syncthreads(); // the runs are where the walk reads them (LDS, or device memory written by this workgroup)
+    NCNN_MOE_STAMP(blockIdx.x, 15, 0);
+
+    const ncnn_moe_sample_params p = a.params[row];
+    const uint32_t run_total = runs_written;
+    uint32_t* const cached_keys = arena;
+    uint32_t* const cached_ends = arena + kRunsInPlace;
+    float* const cached_terms = reinterpret_cast<float*>(arena + 2 * kRunsInPlace);
+    const uint32_t* keys = global_keys;
+    const uint32_t* run_ends = global_ends;
+    const float* terms0 = nullptr;
+    const auto term_of_key = [&p](uint32_t key, float maximum) {
+        return expf_libm(value_from_descending_key(key) / p.temperature - maximum);
+    };
+    if (in_place || run_total <= kRunsInPlace)
+    {
+        if (!in_place)
+        {
+            // (a row that was counted in two rounds: its runs come back from device memory, the counters are dead)
+            for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
+            {
+                cached_keys[i] = global_keys[i];
+                cached_ends[i] = global_ends[i];
+            }
+            __syncthreads();
+        }
+        const float maximum = value_from_descending_key(cached_keys[0]) / p.temperature;
+        for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
+            cached_terms[i] = term_of_key(cached_keys[i], maximum);
+        __syncthreads();
+        keys = cached_keys;
+        run_ends = cached_ends;
+        terms0 = cached_terms;
+    }
+    else
+    {
+        float* terms = reinterpret_cast<float*>(a.sort_indices[1] + row * a.sort_stride);
+        if (p.temperature != 0.0f)
+        {
+            const float maximum = value_from_descending_key(global_keys[0]) / p.temperature;
+            for (uint32_t i = threadIdx.x; i < run_total; i += kReplayThreads)
+                terms[i] = term_of_key(global_keys[i], maximum);
+        }
+        __syncthreads();
+        terms0 = terms;
+    }
+    replay_row<NCNN_MOE_LOGITS_BF16, true>(a, row, p, keys, run_ends, run_total, terms0, tid);
 }
 
 // exp(logit/T - maximum) of every element of the sorted full-order rows, written over the sort's other key

@@ -72,6 +72,7 @@ TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_force_general",
     "ncnn_moe_hip_sampler_debug_scatter_segments",
     "ncnn_moe_hip_sampler_debug_spread_sort",
+    "ncnn_moe_hip_sampler_debug_fused_bf16",
     "ncnn_moe_hip_sampler_debug_chunk_steps",
     "ncnn_moe_hip_sampler_debug_stream_only",
     "ncnn_moe_hip_sampler_debug_set_row_epochs",
@@ -117,6 +118,7 @@ def _bind(lib, testing):
     lib.ncnn_moe_hip_sampler_debug_force_general.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_scatter_segments.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_spread_sort.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_fused_bf16.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_chunk_steps.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_stream_only.argtypes = [vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp]
     lib.ncnn_moe_hip_sampler_debug_set_row_epochs.argtypes = [vp, ctypes.c_int, ctypes.c_uint32]
@@ -327,6 +329,10 @@ class HipSampler:
     def spread_sort(self, enabled):
         """Test hook: the radix sort of long full-order rows on several workgroups (default) or on one."""
         self._check(self._hooks().ncnn_moe_hip_sampler_debug_spread_sort(self._handle, 1 if enabled else 0))
+
+    def fused_bf16(self, enabled):
+        """Test hook: bf16 full-order rows counted and walked by one kernel (default) or by two."""
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_fused_bf16(self._handle, 1 if enabled else 0))
 
     def set_row_epochs(self, epoch):
         """Test hook: the launch number that tags the split kernel's hand-over records, for every row (1 .. LAST_EPOCH)."""

@@ -547,8 +547,10 @@ def test_full_order_rows_listed_in_a_batch_of_many_rows():
     assert np.array_equal(np.nonzero(served_in_full_order)[0], full_order)
 
 
-def test_bf16_counters_that_overflow_sixteen_bits(batch_sampler):
-    """bf16 full-order rows are counted in 16-bit counters, two to a word; a row in which one value occurs
+@pytest.mark.parametrize("fused", [True, False])
+def test_bf16_counters_that_overflow_sixteen_bits(batch_sampler, fused):
+    """(fused: the count and the walk in one kernel, the shipped path, or in the two kernels it replaces.)
+    bf16 full-order rows are counted in 16-bit counters, two to a word; a row in which one value occurs
     65536 times or more is counted again in 32-bit counters.  Rows just below and at the limit, in the lower
     and in the upper half of a word (neighbouring bf16 values), in both, a constant row, and rows whose NaN
     or zeros add up to the limit."""
@@ -576,32 +578,68 @@ def test_bf16_counters_that_overflow_sixteen_bits(batch_sampler):
     params = hip_sampler.make_params(rows, 1.0, 0, 0.95, 0.0)
     params["temperature"] = rng.uniform(0.5, 1.4, size=rows).astype(np.float32)
     params["top_p"][::2] = 1.0
-    for trial in range(3):
-        uniforms = rng.random(rows, dtype=np.float32)
-        gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", vocab=vocab,
-                             context="bf16 counters at the 16-bit limit, draw %d" % trial)
-        assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+    batch_sampler.fused_bf16(fused)
+    try:
+        for trial in range(3):
+            uniforms = rng.random(rows, dtype=np.float32)
+            gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", vocab=vocab,
+                                 context="bf16 counters at the 16-bit limit, draw %d, fused %s" % (trial, fused))
+            assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+    finally:
+        batch_sampler.fused_bf16(True)
 
 
-def test_bf16_rows_of_many_runs(batch_sampler):
-    """bf16 full-order rows with more distinct values than the replay keeps in LDS (6144 runs): the runs and
-    their exp terms are then walked from device memory.  Logits spread over sixty binades."""
+@pytest.mark.parametrize("fused", [True, False])
+def test_bf16_rows_of_many_runs(batch_sampler, fused):
+    """bf16 full-order rows with more distinct values than the walk keeps in LDS (10,922 runs in the one kernel
+    that counts and walks, 6,144 in the replay kernel of the two-kernel path): the runs and their exp terms are then
+    walked from device memory.  Logits spread over sixty binades."""
     rng = np.random.default_rng(515)
     rows, vocab = 40, 109999
     magnitude = np.exp2(rng.uniform(-40.0, 4.0, size=(rows, vocab)))
     logits = (rng.standard_normal((rows, vocab)) * magnitude).astype(np.float32)
     bits = workloads.float32_to_bf16_bits(logits)
     distinct = [np.unique(bits[row]).size for row in range(rows)]
-    assert min(distinct) > 6144, distinct
+    assert min(distinct) > 10922, distinct
     params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
     params["temperature"] = rng.uniform(0.5, 3.0, size=rows).astype(np.float32)
     params["top_p"] = np.where(np.arange(rows) % 3 == 0, 1.0, rng.uniform(0.6, 0.999, size=rows)).astype(np.float32)
     params["min_p"][1::5] = 0.001
-    for trial in range(2):
-        uniforms = rng.random(rows, dtype=np.float32)
-        gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", vocab=vocab,
-                             context="bf16 rows of more than 6144 runs, draw %d" % trial)
-        assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+    batch_sampler.fused_bf16(fused)
+    try:
+        for trial in range(2):
+            uniforms = rng.random(rows, dtype=np.float32)
+            gpu, _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", vocab=vocab,
+                                 context="bf16 rows of more than 10922 runs, draw %d, fused %s" % (trial, fused))
+            assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+    finally:
+        batch_sampler.fused_bf16(True)
+
+
+def test_bf16_rows_counted_and_walked_by_one_kernel_or_two(batch_sampler):
+    """Full-nucleus bf16 rows (the shape of configuration 3, and rows of 6,145 to 10,922 runs, which only the one
+    kernel keeps in LDS): byte-identical results from the fused kernel and from the two it replaces, and the oracle's."""
+    rng = np.random.default_rng(616)
+    rows, vocab = 48, 109999
+    mix = (rng.gumbel(0.0, 1.0, size=(rows, vocab)) + rng.standard_normal((rows, vocab))).astype(np.float32)
+    magnitude = np.exp2(rng.uniform(-18.0, 3.0, size=(rows // 2, vocab)))
+    mix[rows // 2:] = (rng.standard_normal((rows // 2, vocab)) * magnitude).astype(np.float32)
+    bits = workloads.float32_to_bf16_bits(mix)
+    distinct = [np.unique(bits[row]).size for row in range(rows // 2, rows)]
+    assert 6144 < min(distinct) and max(distinct) <= 10922, distinct
+    params = hip_sampler.make_params(rows, 1.0, 0, 0.95, 0.0)
+    params["temperature"][1::3] = 0.7
+    params["min_p"][2::7] = 0.01
+    uniforms = rng.random(rows, dtype=np.float32)
+    results = {}
+    for fused in (True, False):
+        batch_sampler.fused_bf16(fused)
+        try:
+            results[fused], _ = _check_rows(batch_sampler, bits, params, uniforms, dtype="bf16", vocab=vocab,
+                                            context="bf16 full nucleus, fused %s" % fused)
+        finally:
+            batch_sampler.fused_bf16(True)
+    assert results[True].tobytes() == results[False].tobytes()
 
 
 @pytest.mark.parametrize("tied", [0, 700, 1500, 2600])
