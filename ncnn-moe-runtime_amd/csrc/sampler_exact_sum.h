@@ -236,6 +236,8 @@ struct SortedRow
     const uint32_t* keys;     // one key per element, or one per run of equal keys
     const uint32_t* run_ends; // runs only: position behind the last element of each run (null otherwise)
     uint32_t run_count;
+    uint32_t known_runs;      // runs only, 0 = unknown: the first known_runs runs hold ...
+    uint32_t known_elements;  // ... exactly this many elements
     const float* terms0;      // exp(logit/T - maximum) of every item (element or run), computed beforehand
     const uint4* chunk_steps; // elements only, may be null: (exponent, even step, odd step, valid) of every chunk of terms0 ...
     uint32_t chunk_steps_cover; // ... up to this element (the last chunk may be a partial one)
@@ -350,17 +352,41 @@ __device__ __forceinline__ RoundFront begin_round(
     RoundFront front{0u, false, false};
     if (summing)
     {
-        // every wave's total is read at once (independent LDS loads); the composition stays in registers
-        ParityStep totals[WAVES];
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w)
-            totals[w] = scratch.wave_totals[slot][w];
         ParityStep before{0u, 0u};
-#pragma unroll
-        for (int w = 0; w < WAVES - 1; ++w)
+        if constexpr (WAVES > 8)
         {
-            const ParityStep with = compose_steps(before, totals[w]);
-            before = ParityStep{w < wave ? with.even : before.even, w < wave ? with.odd : before.odd};
+            // many waves: lane w takes wave w's total, and four DPP stages (the lanes share a row of sixteen)
+            // compose them in order; the waves in front of this one end at lane wave - 1
+            static_assert(WAVES <= 16, "the waves' totals must fit one DPP row");
+            ParityStep v = lane < WAVES ? scratch.wave_totals[slot][lane] : ParityStep{0u, 0u};
+#define NCNN_MOE_SCAN_STAGE(CONTROL)                                                                         \
+    {                                                                                                        \
+        const ParityStep earlier{dpp_source<CONTROL, 0xf>(v.even), dpp_source<CONTROL, 0xf>(v.odd)};         \
+        v = compose_steps(earlier, v);                                                                       \
+    }
+            NCNN_MOE_SCAN_STAGE(0x111) // row_shr:1
+            NCNN_MOE_SCAN_STAGE(0x112) // row_shr:2
+            NCNN_MOE_SCAN_STAGE(0x114) // row_shr:4
+            NCNN_MOE_SCAN_STAGE(0x118) // row_shr:8
+#undef NCNN_MOE_SCAN_STAGE
+            const int source = wave > 0 ? wave - 1 : 0;
+            const uint32_t even_there = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v.even), source));
+            const uint32_t odd_there = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v.odd), source));
+            before = ParityStep{wave > 0 ? even_there : 0u, wave > 0 ? odd_there : 0u};
+        }
+        else
+        {
+            // every wave's total is read at once (independent LDS loads); the composition stays in registers
+            ParityStep totals[WAVES];
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w)
+                totals[w] = scratch.wave_totals[slot][w];
+#pragma unroll
+            for (int w = 0; w < WAVES - 1; ++w)
+            {
+                const ParityStep with = compose_steps(before, totals[w]);
+                before = ParityStep{w < wave ? with.even : before.even, w < wave ? with.odd : before.odd};
+            }
         }
         before = compose_steps(before, exclusive);
         front.current = apply_step(mantissa, before);
@@ -695,6 +721,7 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
     // FIRST: the terms as they are (they never grow: the sum also stops once it no longer moves); else
     // divided by the two divisors, one after the other (a divisor of one leaves a term as it is)
     const float* const terms0 = row.terms0;
+    const uint32_t* const run_ends = row.run_ends;
     const auto term_of_run = [terms0, divisor, second_divisor](uint32_t run) {
         const float t = terms0[run];
         return FIRST ? t : (t / divisor) / second_divisor;
@@ -703,8 +730,11 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
     float sum = 0.0f;
     if (count == 0u)
         return RunningSum{sum, 0u, false};
-    const uint32_t runs = run_of_element_uniform(row, count - 1u) + 1u;
+    // runs that hold the elements in front of `count` (the caller may know it for its whole row)
+    const uint32_t runs = (row.known_runs != 0u && count == row.known_elements) ? row.known_runs
+                                                                               : run_of_element_uniform(row, count - 1u) + 1u;
     uint32_t start = 0; // elements before this one have been added
+    uint32_t first_run; // the run that holds element `start`
 
     // The first kSequentialHeadOfRuns elements are added in order, as the CPU does, an element per lane (every
     // wave does the same): the sum climbs through most of its binades here, each of which would cost the
@@ -714,16 +744,16 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
         const uint32_t head_runs = min(runs, static_cast<uint32_t>(kWaveSize));
         const float head_term = static_cast<uint32_t>(lane) < head_runs ? term_of_run(static_cast<uint32_t>(lane)) : 0.0f;
         // (a lane without a run: an end that no element lies behind)
-        const uint32_t head_end = static_cast<uint32_t>(lane) < head_runs ? min(row.run_ends[lane], count) : 0xffffffffu;
+        const uint32_t head_end = static_cast<uint32_t>(lane) < head_runs ? min(run_ends[lane], count) : 0xffffffffu;
         const uint32_t head_limit = min(count, static_cast<uint32_t>(kSequentialHeadOfRuns));
-        // the run of element `lane`: the number of runs that end at or in front of it (the ends ascend with the lanes)
-        uint32_t run = 0;
-#pragma unroll
-        for (uint32_t step = kWaveSize / 2; step > 0u; step >>= 1)
-        {
-            const uint32_t end_there = static_cast<uint32_t>(__shfl(static_cast<int>(head_end), static_cast<int>(run + step - 1u), kWaveSize));
-            run += end_there <= static_cast<uint32_t>(lane) ? step : 0u;
-        }
+        // Bit b of `last_elements`: a run ends with element b.  The run of element `lane` is the number of runs that
+        // end in front of it: the bits below `lane`.  (The ends ascend, one run per lane: no bit is set twice.)
+        const bool ends_in_head = head_end <= static_cast<uint32_t>(kWaveSize);
+        const uint32_t last_element = head_end - 1u;
+        const uint32_t low_bits = wave_or_u32(ends_in_head && last_element < 32u ? 1u << last_element : 0u);
+        const uint32_t high_bits = wave_or_u32(ends_in_head && last_element >= 32u ? 1u << (last_element - 32u) : 0u);
+        const uint64_t last_elements = (static_cast<uint64_t>(high_bits) << 32) | low_bits;
+        const uint32_t run = static_cast<uint32_t>(__popcll(last_elements & ((1ull << lane) - 1ull)));
         const float term_there = __shfl(head_term, static_cast<int>(run), kWaveSize);
         const float own = static_cast<uint32_t>(lane) < head_limit ? term_there : 0.0f;
         const float sums = wave_sequential_sums(own); // (lanes behind the head add zero: they hold the head's sum)
@@ -739,12 +769,24 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
         start = head_limit;
         if (start >= count)
             return RunningSum{sum, 0u, false};
+        // (start is 64 here: every run that ends inside the head ends in front of it)
+        first_run = static_cast<uint32_t>(__popcll(last_elements));
     }
-    const uint32_t first_run = run_of_element_uniform(row, start);
     if (tid == 0)
         scratch.first_event[0] = 0xffffffffu;
     uint32_t round = 0;
-    for (uint32_t base = first_run; base < runs; base += kRunsChunk)
+    // A thread takes kRunsPerThread consecutive runs and the workgroup kRunsChunk; a chunk costs a round, and one
+    // more for each binade the sum leaves inside it (measured on 256 rows of 201,088 bf16 logits, ~5,500 runs each:
+    // 2 runs x 8 waves 67.3 us, 2 x 4 68.5, 4 x 8 69.5, 1 x 16 69.7, 4 x 16 69.9, 2 x 16 70.1, 1 x 8 71.1, 8 x 16 74.3:
+    // a round over a long chunk repeats more work after every event than the rounds of short chunks cost).
+    // The chunks start at a multiple of kRunsPerThread, so that a thread's runs are whole groups of the arrays
+    // (runs in front of `start` add nothing: their elements are clipped away below).
+    static_assert((kRunsPerThread & (kRunsPerThread - 1)) == 0, "the chunks start at a multiple of a thread's runs");
+    constexpr bool kGroups = kRunsPerThread % 4 == 0; // a thread's runs are loaded in groups of four
+    const uint32_t first_base = first_run & ~static_cast<uint32_t>(kRunsPerThread - 1);
+    const bool groups_aligned = kGroups &&
+        ((reinterpret_cast<uintptr_t>(terms0) | reinterpret_cast<uintptr_t>(run_ends)) & 15u) == 0u;
+    for (uint32_t base = first_base; base < runs; base += kRunsChunk)
     {
         const uint32_t chunk_end = min(runs, base + static_cast<uint32_t>(kRunsChunk));
         const uint32_t thread_first = base + static_cast<uint32_t>(tid) * kRunsPerThread;
@@ -752,14 +794,38 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
         uint32_t firsts[kRunsPerThread]; // first and one-past-last element of each run, clipped to count
         uint32_t lasts[kRunsPerThread];
         const bool summing = tid < kRunsWaves * kWaveSize;
-#pragma unroll
-        for (int j = 0; j < kRunsPerThread; ++j)
+        if (groups_aligned && summing && thread_first + kRunsPerThread <= chunk_end)
         {
-            const uint32_t i = thread_first + j;
-            const bool valid = summing && i < chunk_end;
-            terms[j] = valid ? term_of_run(i) : 0.0f;
-            firsts[j] = valid ? run_first_element(row, i) : 0u;
-            lasts[j] = valid ? min(row.run_ends[i], count) : 0u;
+            float loaded[kRunsPerThread];
+            uint32_t ends[kRunsPerThread];
+#pragma unroll
+            for (int g = 0; g + 4 <= kRunsPerThread; g += 4)
+            {
+                const float4 t = *reinterpret_cast<const float4*>(terms0 + thread_first + g);
+                const uint4 e = *reinterpret_cast<const uint4*>(run_ends + thread_first + g);
+                loaded[g + 0] = t.x, loaded[g + 1] = t.y, loaded[g + 2] = t.z, loaded[g + 3] = t.w;
+                ends[g + 0] = e.x, ends[g + 1] = e.y, ends[g + 2] = e.z, ends[g + 3] = e.w;
+            }
+            const uint32_t before = thread_first == 0u ? 0u : run_ends[thread_first - 1u];
+#pragma unroll
+            for (int j = 0; j < kRunsPerThread; ++j)
+            {
+                terms[j] = FIRST ? loaded[j] : (loaded[j] / divisor) / second_divisor;
+                firsts[j] = j == 0 ? before : ends[j - 1];
+                lasts[j] = min(ends[j], count);
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int j = 0; j < kRunsPerThread; ++j)
+            {
+                const uint32_t i = thread_first + j;
+                const bool valid = summing && i < chunk_end;
+                terms[j] = valid ? term_of_run(i) : 0.0f;
+                firsts[j] = valid ? run_first_element(row, i) : 0u;
+                lasts[j] = valid ? min(run_ends[i], count) : 0u;
+            }
         }
         bool fresh = true; // no event in this chunk yet
         while (true)
@@ -774,13 +840,21 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
             NCNN_MOE_COUNT(blockIdx.x, 15, 13);
 
             // A run of m equal terms moves the mantissa m times by the term's step - unless the term ends exactly
-            // half an ulp above a multiple of the ulp (its two steps differ): a wave that holds such a term
-            // composes its totals again the long way.
+            // half an ulp above a multiple of the ulp (its two steps differ): where a lane of the wave holds such
+            // a run, the wave works that run's two totals out the long way.  A wave none of whose runs has an
+            // element left (all in front of `start`, or behind `count`) composes nothing.
             ParityStep thread_total{0u, 0u};
-            bool tie = false;
+            ParityStep run_totals[kRunsPerThread]; // of each run's additions, for the search for an event
             ParityStep first_single{0u, 0u};
             uint32_t first_multiplicity = 0;
-            if (summing)
+            bool live = false;
+#pragma unroll
+            for (int j = 0; j < kRunsPerThread; ++j)
+                run_totals[j] = ParityStep{0u, 0u};
+#pragma unroll
+            for (int j = 0; j < kRunsPerThread; ++j)
+                live = live || lasts[j] > max(firsts[j], start);
+            if (__builtin_amdgcn_ballot_w64(live) != 0ull)
             {
 #pragma unroll
                 for (int j = 0; j < kRunsPerThread; ++j)
@@ -793,25 +867,13 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
                         first_single = single;
                         first_multiplicity = multiplicity;
                     }
-                    tie = tie || (single.even != single.odd && multiplicity != 0u);
                     const uint64_t product = static_cast<uint64_t>(single.even) * multiplicity;
                     const uint32_t repeated = product > kStepCap ? kStepCap : static_cast<uint32_t>(product);
-                    thread_total = compose_steps(thread_total, ParityStep{repeated, repeated});
-                }
-                if (__builtin_amdgcn_ballot_w64(tie) != 0ull)
-                {
-                    thread_total = ParityStep{0u, 0u};
-                    const uint32_t last_run = min(thread_first + static_cast<uint32_t>(kRunsPerThread), chunk_end);
-#pragma unroll 1
-                    for (uint32_t run = thread_first; run < last_run; ++run)
-                    {
-                        const uint32_t low = max(run_first_element(row, run), start);
-                        const uint32_t high = min(row.run_ends[run], count);
-                        const uint32_t multiplicity = high > low ? high - low : 0u;
-                        const ParityStep single = step_of_term(term_of_run(run), exponent);
-                        thread_total = compose_steps(
-                            thread_total, ParityStep{repeated_step(false, single, multiplicity), repeated_step(true, single, multiplicity)});
-                    }
+                    ParityStep run_total{repeated, repeated};
+                    if (__builtin_amdgcn_ballot_w64(single.even != single.odd && multiplicity != 0u) != 0ull)
+                        run_total = ParityStep{repeated_step(false, single, multiplicity), repeated_step(true, single, multiplicity)};
+                    run_totals[j] = run_total;
+                    thread_total = compose_steps(thread_total, run_total);
                 }
             }
             if (FIRST)
@@ -819,45 +881,61 @@ __device__ __noinline__ RunningSum exact_running_sum_runs_scaled(
                 // the largest remaining term of the row does not move the sum: nothing later can
                 if (tid == 0)
                     scratch.absorbed[slot] =
-                        (fresh && base > first_run && (first_multiplicity == 0u || (first_single.even == 0u && first_single.odd == 0u))) ? 1 : 0;
+                        (fresh && base > first_base && (first_multiplicity == 0u || (first_single.even == 0u && first_single.odd == 0u))) ? 1 : 0;
             }
             const auto find_event = [&](uint32_t current, RoundEvent& found) -> bool {
-                // (one thread of a round, in few rounds: a short loop that reads the runs again)
-                const uint32_t last_run = min(thread_first + static_cast<uint32_t>(kRunsPerThread), chunk_end);
-#pragma unroll 1
-                for (uint32_t run = thread_first; run < last_run; ++run)
+                // The thread's first run whose additions take the mantissa to the limit (from the registers: no
+                // branch, no load), then the first such addition of that run.
+                bool hit = false;
+                uint32_t hit_low = 0, hit_multiplicity = 0, hit_current = 0;
+                float hit_term = 0.0f;
+#pragma unroll
+                for (int j = 0; j < kRunsPerThread; ++j)
                 {
-                    const uint32_t low = max(run_first_element(row, run), start);
-                    const uint32_t high = min(row.run_ends[run], count);
-                    const uint32_t multiplicity = high > low ? high - low : 0u;
-                    const float term = term_of_run(run);
-                    const ParityStep single = step_of_term(term, exponent);
-                    const bool odd = (current & 1u) != 0u;
-                    const uint32_t next = current + repeated_step(odd, single, multiplicity);
-                    if (multiplicity > 0u && next >= limit)
-                    {
-                        // the first addition of the run after which the mantissa reaches the limit
-                        uint32_t none = 0u, some = multiplicity; // repeated additions: `none` stay below, `some` reach it
-                        while (some - none > 1u)
-                        {
-                            const uint32_t middle = none + ((some - none) >> 1);
-                            if (current + repeated_step(odd, single, middle) >= limit)
-                                some = middle;
-                            else
-                                none = middle;
-                        }
-                        const uint32_t before_event = current + repeated_step(odd, single, none);
-                        const uint32_t after_event = apply_step(before_event, single);
-                        const uint32_t element = low + none;
-                        if (after_event >= kBinadeFull)
-                            found = RoundEvent{element << 1, before_event, term};
-                        else
-                            found = RoundEvent{(element << 1) | 1u, after_event, 0.0f};
-                        return true;
-                    }
+                    const uint32_t low = max(firsts[j], start);
+                    const uint32_t multiplicity = lasts[j] > low ? lasts[j] - low : 0u;
+                    const uint32_t next = apply_step(current, run_totals[j]);
+                    const bool here = !hit && multiplicity > 0u && next >= limit;
+                    hit_low = here ? low : hit_low;
+                    hit_multiplicity = here ? multiplicity : hit_multiplicity;
+                    hit_current = here ? current : hit_current;
+                    hit_term = here ? terms[j] : hit_term;
+                    hit = hit || here;
                     current = next;
                 }
-                return false;
+                if (!hit)
+                    return false;
+                const ParityStep single = step_of_term(hit_term, exponent);
+                const bool odd = (hit_current & 1u) != 0u;
+                // repeated additions: `none` of them stay below the limit, one more reaches it
+                uint32_t none = 0u;
+                if (single.even == single.odd)
+                {
+                    // every addition moves the mantissa by the same step: a division finds the first that arrives
+                    // (a mantissa at the limit already - a stop bound of zero - has its event at the first addition)
+                    if (hit_current < limit && single.even != 0u)
+                        none = (limit - 1u - hit_current) / single.even;
+                }
+                else
+                {
+                    uint32_t some = hit_multiplicity; // this many reach it
+                    while (some - none > 1u)
+                    {
+                        const uint32_t middle = none + ((some - none) >> 1);
+                        if (hit_current + repeated_step(odd, single, middle) >= limit)
+                            some = middle;
+                        else
+                            none = middle;
+                    }
+                }
+                const uint32_t before_event = hit_current + repeated_step(odd, single, none);
+                const uint32_t after_event = apply_step(before_event, single);
+                const uint32_t element = hit_low + none;
+                if (after_event >= kBinadeFull)
+                    found = RoundEvent{element << 1, before_event, hit_term};
+                else
+                    found = RoundEvent{(element << 1) | 1u, after_event, 0.0f};
+                return true;
             };
             uint32_t event = 0;
             const RoundOutcome outcome =
@@ -899,7 +977,8 @@ __device__ __forceinline__ void replay_sorted_window(
     const SamplerArgs& a, uint32_t row, const ncnn_moe_sample_params& p,
     const uint32_t* keys, const uint32_t* run_ends, uint32_t run_count, uint32_t n,
     const uint32_t* sorted_indices, uint8_t flags, ReplayScratch& scratch, int tid, TokenAt token_at,
-    const float* terms0 = nullptr, const uint4* chunk_steps = nullptr, uint32_t chunk_steps_cover = 0u)
+    const float* terms0 = nullptr, const uint4* chunk_steps = nullptr, uint32_t chunk_steps_cover = 0u,
+    uint32_t known_runs = 0u, uint32_t known_elements = 0u)
 {
 #ifdef NCNN_MOE_TIMELINE
     const uint32_t stamp_row = a.only_pending ? 0xffffffffu : row; // the full-order rows' stamps (not the wide select's)
@@ -908,6 +987,8 @@ __device__ __forceinline__ void replay_sorted_window(
     sorted.keys = keys;
     sorted.run_ends = run_ends;
     sorted.run_count = run_count;
+    sorted.known_runs = RUNS ? known_runs : 0u;
+    sorted.known_elements = known_elements;
     sorted.terms0 = terms0;
     sorted.chunk_steps = RUNS ? nullptr : chunk_steps;
     sorted.chunk_steps_cover = chunk_steps_cover;

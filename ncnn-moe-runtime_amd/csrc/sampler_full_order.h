@@ -1242,7 +1242,8 @@ __device__ __forceinline__ void replay_row(
     }
     // first item whose key is not finite
     const uint32_t low = wave_partition_point(items, [keys](uint32_t item) { return keys[item] <= kLastFiniteKey; });
-    uint32_t n = first_element(low);
+    const uint32_t finite_elements = first_element(low);
+    uint32_t n = finite_elements;
     if (p.top_k > 0 && p.top_k < vocab && n > p.top_k)
         n = p.top_k;
     NCNN_MOE_STAMP(blockIdx.x, 15, 2);
@@ -1252,7 +1253,9 @@ __device__ __forceinline__ void replay_row(
         if (a.chunk_steps_ready != 0)
             chunk_steps = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity;
     }
-    replay_sorted_window<RUNS>(a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0, chunk_steps, a.vocab);
+    // (the finite runs and the elements they hold: a sum over all of them need not look for its last run)
+    replay_sorted_window<RUNS>(
+        a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0, chunk_steps, a.vocab, RUNS ? low : 0u, finite_elements);
 }
 
 template <int DTYPE, bool RUNS>
@@ -1276,7 +1279,7 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     {
         // a row of few runs is walked from LDS; the terms of a longer one go to the sort's spare index buffer
         __shared__ uint32_t cached_keys[kCachedRuns];
-        __shared__ uint32_t cached_ends[kCachedRuns];
+        __shared__ __align__(16) uint32_t cached_ends[kCachedRuns];
         __shared__ __align__(16) float cached_terms[kCachedRuns];
         const uint32_t run_total = a.sort_indices[0][row * a.sort_stride];
         run_total_of_row = run_total;
@@ -1328,7 +1331,7 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
 // third of the 128 KB each), which saves the runs' trip through device memory and a launch.  A row with more
 // runs than that, or one whose counters overflowed 16 bits, writes its runs to device memory as the two
 // kernels do, and walks them from there.
-constexpr uint32_t kRunsInPlace = kCountWords / 3; // 10,922 runs with their ends and terms in the counters' LDS
+constexpr uint32_t kRunsInPlace = (kCountWords / 3) & ~3u; // 10,920 runs with their ends and terms in the counters' LDS (each array on a 16-byte boundary)
 
 __global__ __launch_bounds__(kSortThreads) void bf16_counting_replay_kernel(SamplerArgs a)
 {
