@@ -33,6 +33,13 @@ int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* sampler, int en
 /* fused_bf16 (on by default): a bf16 full-order row is counted and walked by one kernel, its runs staying in LDS; off,
  * by the counting kernel and the replay kernel, with the runs in device memory between them.  Same results either way. */
 int ncnn_moe_hip_sampler_debug_fused_bf16(ncnn_moe_hip_sampler* sampler, int enabled);
+/* partial_sort (on by default): a full-order fp32 row whose sort is spread over the GPU is sorted only as far as its
+ * terms can move one of the sampler's sums (a kernel guesses how far, the walk checks the guess against its exact sums
+ * and has a row whose guess was too short sorted whole by a second launch); off, every row is sorted whole.  Same
+ * results either way.  sort_lengths copies out, for the first `rows` rows of the last call, the number of elements that
+ * were sorted (0xffffffff: the whole row; only rows that took the spread sort with partial_sort on are written). */
+int ncnn_moe_hip_sampler_debug_partial_sort(ncnn_moe_hip_sampler* sampler, int enabled);
+int ncnn_moe_hip_sampler_debug_sort_lengths(ncnn_moe_hip_sampler* sampler, uint32_t* lengths, uint32_t rows);
 /* Sets the per-row launch numbers (epochs, 1 .. 16383) that tag the split kernel's hand-over records: of the
  * handle, or with a null handle of the static scratch of `device` (after it has served a call).  Tests start a
  * few launches in front of the point where the epochs start over. */

@@ -67,6 +67,8 @@ struct ncnn_moe_hip_sampler
     uint32_t* sort_indices[2] = {nullptr, nullptr};
     uint64_t sort_stride = 0;
     uint32_t* row_list = nullptr;         // [1 + rows], see SamplerArgs::row_list
+    uint32_t* sort_cuts = nullptr;        // [3][rows]: SamplerArgs::sort_lengths, sort_last_keys, finite_counts
+    int partial_sort = 1;                 // full-order fp32 rows are sorted only as far as their terms can move a sum
     uint32_t* sort_part_counts = nullptr; // [rows][kMaxSortParts][256]
     double* term_sums = nullptr;          // [rows][term_sum_parts]: fp64 sums of the terms kernel's blocks
     uint4* chunk_steps = nullptr;         // [rows][chunk_capacity]: composed step of every whole chunk of a sorted row's terms
@@ -359,6 +361,17 @@ int launch_sampler(
     };
     // `leftovers`: the launch behind the wide select, for the few rows (usually none) that it could not
     // finish; it is kept to two kernels, because every launch costs its few microseconds even with no row to serve.
+    // fp32 rows whose sort is spread over the GPU are sorted only as far as their terms can move a sum
+    // (full_order_cut_kernel); a row whose replay finds that guess too short stays pending, and a second launch of
+    // the full-order kernels, behind the first, sorts it whole.
+    const bool partial_sort = passes.full_order && dtype == NCNN_MOE_LOGITS_F32 && !want_distribution && sort_tiles >= 4 &&
+        s->spread_sort != 0 && s->partial_sort != 0;
+    if (partial_sort)
+    {
+        a.sort_lengths = s->sort_cuts;
+        a.sort_last_keys = s->sort_cuts + s->max_rows;
+        a.finite_counts = s->sort_cuts + 2 * static_cast<size_t>(s->max_rows);
+    }
     const auto launch_full_order = [&](SamplerArgs a, bool leftovers) {
         const bool spread_sort = sort_tiles >= 4 && s->spread_sort != 0 && !leftovers;
         const bool runs = dtype == NCNN_MOE_LOGITS_BF16 && !want_distribution;
@@ -368,6 +381,8 @@ int launch_sampler(
             hipLaunchKernelGGL(full_order_row_list_kernel, dim3(1), dim3(kSortThreads), 0, stream, a, rows, s->row_list);
             a.row_list = s->row_list;
         }
+        if (!leftovers && partial_sort)
+            hipLaunchKernelGGL(full_order_cut_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
         // the token indices ride along with the keys only when the whole distribution is exported
         const auto sort_rows = [&](auto dtype_tag, auto pairs_tag) {
             constexpr int kType = decltype(dtype_tag)::value;
@@ -441,6 +456,8 @@ int launch_sampler(
             launch_wide(stream, 1);
         if (passes.full_order)
             launch_full_order(a, false);
+        if (partial_sort)
+            launch_full_order(a, true);
     }
     SAMPLER_HIP_CHECK(s, hipGetLastError());
     return NCNN_MOE_SAMPLER_SUCCESS;
@@ -608,6 +625,7 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
         CREATE_CHECK(hipMalloc(&s->sort_indices[i], rows * s->sort_stride * sizeof(uint32_t)));
     }
     CREATE_CHECK(hipMalloc(&s->row_list, (static_cast<size_t>(rows) + 1) * sizeof(uint32_t)));
+    CREATE_CHECK(hipMalloc(&s->sort_cuts, 3 * static_cast<size_t>(rows) * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->sort_part_counts, rows * kMaxSortParts * 256 * sizeof(uint32_t)));
     s->term_sum_parts = (max_vocab + kTermsThreads * kTermsPerThread - 1) / (kTermsThreads * kTermsPerThread);
     s->chunk_capacity = max_vocab / kReplayChunk + 1;
@@ -664,7 +682,7 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
     void* buffers[] = {
         s->logits, s->params, s->uniforms, s->results, s->segment_values, s->segment_indices,
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->split_records, s->row_epoch, s->sort_keys[0], s->sort_keys[1],
-        s->sort_indices[0], s->sort_indices[1], s->sort_part_counts, s->row_list, s->term_sums, s->chunk_steps, s->distribution_ids, s->distribution_probabilities,
+        s->sort_indices[0], s->sort_indices[1], s->sort_part_counts, s->row_list, s->sort_cuts, s->term_sums, s->chunk_steps, s->distribution_ids, s->distribution_probabilities,
         s->distribution_count, s->single_params, s->single_uniform, s->single_result, s->verify_ids,
         s->verify_probabilities, s->verify_counts, s->verify_long_ids, s->verify_long_probabilities, s->verify_dense};
     for (void* buffer : buffers)
@@ -1133,6 +1151,33 @@ int ncnn_moe_hip_sampler_debug_spread_sort(ncnn_moe_hip_sampler* s, int enabled)
     if (s == nullptr)
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     s->spread_sort = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+// Full-order fp32 rows sorted only as far as their terms can move a sum (the default), or always whole.
+int ncnn_moe_hip_sampler_debug_partial_sort(ncnn_moe_hip_sampler* s, int enabled)
+{
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    s->partial_sort = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+// The rows' sort lengths of the last call (0xffffffff: the row was, or is to be, sorted whole).
+int ncnn_moe_hip_sampler_debug_sort_lengths(ncnn_moe_hip_sampler* s, uint32_t* lengths, uint32_t rows)
+{
+    if (s == nullptr || lengths == nullptr || rows > s->max_rows)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
+    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    std::vector<uint32_t> last_keys(rows);
+    SAMPLER_HIP_CHECK(s, hipMemcpy(lengths, s->sort_cuts, rows * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    SAMPLER_HIP_CHECK(s, hipMemcpy(last_keys.data(), s->sort_cuts + s->max_rows, rows * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    for (uint32_t row = 0; row < rows; ++row)
+    {
+        if (last_keys[row] == 0xffffffffu)
+            lengths[row] = 0xffffffffu;
+    }
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

@@ -73,7 +73,22 @@ struct SamplerArgs
     // the rows in ascending order.  Kernels over a (parts, rows) grid look their row up here (null: in row_state).
     // (The struct's last member: what the select kernels read keeps its place among the kernel's arguments.)
     const uint32_t* row_list;
+
+    // Full-order fp32 rows sorted only as far as their terms can move a sum (full_order_cut_kernel), all [rows]
+    // (null: every row is sorted whole): the last key among the elements that are sorted (every element with a
+    // larger key is left out; 0xffffffff: none is), their number, and the row's finite logits (with kRowHoldsNan).
+    uint32_t* sort_lengths;
+    uint32_t* sort_last_keys;
+    uint32_t* finite_counts;
 };
+
+// Elements of the row that the full-order sort orders (the row's first ones in sorted order).
+__device__ __forceinline__ uint32_t sorted_length(const SamplerArgs& a, uint32_t row)
+{
+    return a.sort_lengths == nullptr ? a.vocab : a.sort_lengths[row];
+}
+
+constexpr uint32_t kRowHoldsNan = 0x80000000u; // in finite_counts: the row holds a NaN (a row has fewer than 2^31 logits)
 
 __device__ __forceinline__ uint8_t stop_flag(const SamplerArgs& a, const ncnn_moe_sample_params& p, int32_t token)
 {

@@ -978,7 +978,8 @@ __device__ __forceinline__ void replay_sorted_window(
     const uint32_t* keys, const uint32_t* run_ends, uint32_t run_count, uint32_t n,
     const uint32_t* sorted_indices, uint8_t flags, ReplayScratch& scratch, int tid, TokenAt token_at,
     const float* terms0 = nullptr, const uint4* chunk_steps = nullptr, uint32_t chunk_steps_cover = 0u,
-    uint32_t known_runs = 0u, uint32_t known_elements = 0u)
+    uint32_t known_runs = 0u, uint32_t known_elements = 0u, uint32_t sorted_elements = 0xffffffffu, uint32_t tail_key = 0u,
+    bool* tail_matters = nullptr)
 {
 #ifdef NCNN_MOE_TIMELINE
     const uint32_t stamp_row = a.only_pending ? 0xffffffffu : row; // the full-order rows' stamps (not the wide select's)
@@ -996,12 +997,43 @@ __device__ __forceinline__ void replay_sorted_window(
     sorted.maximum = value_from_descending_key(keys[0]) / p.temperature;
     sorted.normalizer = 1.0f;
     sorted.renormalizer = 1.0f;
+    // A row sorted in part (elements only): `keys` holds its first sorted_elements elements in sorted order, and
+    // every element behind them has a key of tail_key or more, a term of at most tail_term.  A sum that runs
+    // past the sorted elements is the sum over those, as long as the largest term of the tail does not move it
+    // (neither does any smaller one, and a sum that does not move meets no stop condition that it has not met);
+    // where it could, *tail_matters is set and the caller has the row sorted whole.
+    const bool sorted_in_part = !RUNS && sorted_elements < n;
+    // (the exp may be off its neighbours' by an ulp: the bound is taken a little above it)
+    const float tail_term =
+        sorted_in_part ? expf_libm(value_from_descending_key(tail_key) / p.temperature - sorted.maximum) * 1.00001f : 0.0f;
+    bool tail_moves = false;
     auto running_sum = [&](auto phase, uint32_t count, int mode, float bound) -> RunningSum {
         constexpr int kPhase = decltype(phase)::value;
         if constexpr (RUNS)
             return exact_running_sum_runs<kPhase>(sorted, count, mode, bound, scratch, tid);
         else
-            return exact_running_sum<kPhase>(sorted, count, mode, bound, scratch, tid);
+        {
+            const uint32_t covered = min(count, sorted_elements);
+            const RunningSum result = exact_running_sum<kPhase>(sorted, covered, mode, bound, scratch, tid);
+            if (covered < count && !result.stopped)
+            {
+                float largest = tail_term;
+                if (kPhase >= 1)
+                    largest = largest / sorted.normalizer;
+                if (kPhase >= 2)
+                    largest = largest / sorted.renormalizer;
+                int exponent;
+                uint32_t mantissa;
+                decode_sum(result.sum, exponent, mantissa);
+                const ParityStep step = step_of_term(largest, exponent);
+                tail_moves = tail_moves || step.even != 0u || step.odd != 0u || !is_finite_f32(result.sum);
+            }
+            return result;
+        }
+    };
+    const auto leave_to_whole_sort = [&]() {
+        if (tail_matters != nullptr)
+            *tail_matters = true;
     };
     // the item (element, or run) that holds an element
     auto item_of = [&](uint32_t element) -> uint32_t { // for an element that the whole wave asks for
@@ -1022,6 +1054,8 @@ __device__ __forceinline__ void replay_sorted_window(
     }
     else
         normalizer = running_sum(std::integral_constant<int, 0>{}, n, kStopNever, 0.0f).sum; // (checks the first term itself)
+    if (tail_moves)
+        return leave_to_whole_sort();
     if (!is_finite_f32(normalizer) || !(normalizer > 0.0f))
     {
         if (tid == 0)
@@ -1038,16 +1072,24 @@ __device__ __forceinline__ void replay_sorted_window(
         const float threshold = row_term<1>(sorted, 0) * p.min_p;
         // first item whose probability is below the threshold
         const uint32_t first = wave_partition_point(
-            RUNS ? item_of(n - 1u) + 1u : n, [&sorted, threshold](uint32_t item) { return row_term<1>(sorted, item) >= threshold; });
+            RUNS ? item_of(n - 1u) + 1u : min(n, sorted_elements),
+            [&sorted, threshold](uint32_t item) { return row_term<1>(sorted, item) >= threshold; });
         if constexpr (RUNS)
             candidates = min(n, run_first_element(sorted, first));
         else
+        {
             candidates = first;
+            // every sorted element survives: the cut lies in the tail unless the tail's largest term is below it
+            if (sorted_in_part && first == sorted_elements && tail_term / sorted.normalizer >= threshold)
+                return leave_to_whole_sort();
+        }
     }
 
     NCNN_MOE_STAMP(stamp_row, 15, 4);
     // ---- Top-P (session.cpp:119-128) and the renormaliser (:130-132), which adds the same values
     const RunningSum nucleus = running_sum(std::integral_constant<int, 1>{}, candidates, kStopAtOrAbove, p.top_p);
+    if (tail_moves)
+        return leave_to_whole_sort();
     const uint32_t kept = nucleus.stopped ? nucleus.stop_index + 1u : candidates;
     sorted.renormalizer = nucleus.sum;
     NCNN_MOE_STAMP(stamp_row, 15, 5);
@@ -1076,6 +1118,9 @@ __device__ __forceinline__ void replay_sorted_window(
     // ---- inverse-CDF draw over the kept prefix (session.cpp:432-442)
     const RunningSum draw = running_sum(std::integral_constant<int, 2>{}, kept, kStopAbove, a.uniforms[row]);
     const uint32_t selected = draw.stopped ? draw.stop_index : kept - 1u;
+    // (a draw that no partial sum exceeds takes the last kept element, which a row sorted in part may not hold)
+    if (tail_moves || (sorted_in_part && selected >= sorted_elements))
+        return leave_to_whole_sort();
     NCNN_MOE_STAMP(stamp_row, 15, 6);
     const int32_t token = token_at(selected);
     NCNN_MOE_STAMP(stamp_row, 15, 7);

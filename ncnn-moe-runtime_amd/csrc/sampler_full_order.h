@@ -40,6 +40,15 @@ __device__ __forceinline__ bool spread_grid_row(const SamplerArgs& a, uint32_t& 
     return a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
 }
 
+// The largest key that pass `pass` of a row's spread sort keeps: the first pass of a row that is sorted in part
+// leaves out the elements behind the row's cut; every other pass keeps what it reads.
+__device__ __forceinline__ uint32_t sort_last_key(const SamplerArgs& a, uint32_t row, int pass)
+{
+    if (pass != 0 || a.sort_lengths == nullptr)
+        return 0xffffffffu;
+    return a.sort_last_keys[row];
+}
+
 // Lists the rows that the full-order kernels serve (see SamplerArgs::row_list).  One workgroup.
 __global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(SamplerArgs a, uint32_t rows, uint32_t* list)
 {
@@ -71,6 +80,186 @@ __global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(Sampl
     }
     if (tid == 0)
         list[0] = listed;
+}
+
+// How much of a full-order fp32 row needs sorting.  The sampler's sums add the row's terms exp(logit/T - max)
+// in descending order, and a term below half an ulp of the sum it meets leaves that sum as it is: behind some
+// point of the sorted row nothing moves any sum, and what lies there need not be in order (nor be sorted at
+// all) - only counted.  For a temperature of 1 and logits spread like N(0, 4) that point lies past most of the
+// row; at 0.5 it lies behind the first tenth.
+// One workgroup per row looks at a sample of the row (16,384 logits, evenly spaced groups of four): counts of
+// the keys' upper twelve bits (4,096 buckets: sign, exponent and three bits of the mantissa).  With the terms of
+// the buckets' lower and upper ends it looks for the first bucket whose largest possible term is below 2^-27 of
+// the least the buckets in front of it add up to (the sums' half ulp is 2^-25 to 2^-24 of them), and has the sort
+// keep the buckets in front of it: sort_last_keys.  This is a guess that costs or saves time, never exactness:
+// the replay checks against its exact sums that the largest term left out moves none of them, and otherwise has
+// the row sorted whole.  The exact counts that go with a cut (elements kept, finite logits, NaN seen) are taken
+// by the sort's first counting pass, which reads the whole row; this kernel clears them.  Rows it does not cut
+// get a last key of 0xffffffff and the row's length.
+constexpr int kCutBuckets = 4096;
+constexpr int kCutCopies = 4;                   // of the counters: a lane uses copy lane % 4 (few buckets hold most of a row)
+constexpr int kCutStride = kCutBuckets + 1;     // (the copies of a counter lie in different banks)
+constexpr uint32_t kCutSample = 4096;           // 16-byte groups of the row that are looked at
+constexpr float kCutMinimum = 4096.0f;          // rows are not cut shorter than about this
+
+__global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArgs a)
+{
+    static_assert(kCutSample == 4u * kSortThreads && kCutBuckets == 4 * kSortThreads, "four loads and four buckets a thread");
+    const uint32_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid >> 6;
+    const bool served = a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
+    const float temperature = a.params[row].temperature;
+    const auto sort_whole_row = [&]() {
+        if (tid == 0)
+        {
+            a.sort_last_keys[row] = 0xffffffffu;
+            a.sort_lengths[row] = a.vocab;
+        }
+    };
+    if (!served || !(temperature > 0.0f))
+        return sort_whole_row();
+    __shared__ uint32_t counts[kCutCopies * kCutStride];
+    __shared__ uint32_t wave_keys[kSortWaves];
+    __shared__ float wave_counts[kSortWaves];
+    __shared__ float wave_masses[kSortWaves];
+    __shared__ uint32_t cut_bucket;
+
+    // ---- the sample: group g of kCutSample lies at 16-byte group g * groups / kCutSample of the row
+    const float* logits = static_cast<const float*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
+    const uint32_t misalignment = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(logits) & 15u) / 4u;
+    const float* aligned_logits = logits - misalignment;
+    const uint32_t aligned_end = misalignment + a.vocab; // positions [misalignment, aligned_end) hold the row
+    const uint32_t groups = (aligned_end + 3u) / 4u;
+    const uint32_t sampled = min(groups, kCutSample);
+    uint4 raw[4];
+    uint32_t positions[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        const uint32_t g = static_cast<uint32_t>(k * kSortThreads + tid);
+        const uint32_t group = static_cast<uint32_t>(static_cast<uint64_t>(g) * groups / kCutSample);
+        positions[k] = g < sampled || groups >= kCutSample ? group * 4u : aligned_end;
+        if (groups < kCutSample)
+            positions[k] = g < groups ? g * 4u : aligned_end; // a short row is looked at whole
+        raw[k] = *reinterpret_cast<const uint4*>(aligned_logits + (positions[k] < aligned_end ? positions[k] : 0u));
+    }
+    for (int i = tid; i < kCutCopies * kCutStride; i += kSortThreads)
+        counts[i] = 0u;
+    if (tid == 0)
+        cut_bucket = kCutBuckets;
+    __syncthreads();
+    uint32_t* const my_counts = counts + (lane & (kCutCopies - 1)) * kCutStride;
+    uint32_t smallest_key = 0xffffffffu;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        const uint32_t words[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
+#pragma unroll
+        for (uint32_t c = 0; c < 4u; ++c)
+        {
+            const uint32_t key = descending_key(__uint_as_float(words[c]));
+            if (positions[k] + c >= misalignment && positions[k] + c < aligned_end)
+            {
+                atomicAdd(&my_counts[key >> 20], 1u);
+                smallest_key = key > kPositiveInfinityKey ? min(smallest_key, key) : smallest_key;
+            }
+        }
+    }
+    smallest_key = ~wave_max_u32(~smallest_key);
+    if (lane == 0)
+        wave_keys[wave] = smallest_key;
+    __syncthreads();
+    uint32_t first_key = 0xffffffffu; // of the sample in sorted order, +inf aside: the largest logit's
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w)
+        first_key = min(first_key, wave_keys[w]);
+    if (first_key > kLastFiniteKey)
+        return sort_whole_row(); // (no finite logit in the sample)
+    // every sampled element stands for this many of the row
+    const float weight = static_cast<float>(groups) / static_cast<float>(min(groups, kCutSample));
+
+    // ---- thread t: buckets 4 t .. 4 t + 3; the terms are taken relative to the sample's largest logit (the
+    // comparison below is one of ratios: any reference would do)
+    constexpr uint32_t kFirstFiniteBucket = 0x008u, kLastFiniteBucket = 0xff7u; // keys 0x00800000 .. 0xff7fffff
+    float bucket_counts[4];
+    float bucket_least[4]; // the least that the bucket's elements add up to
+    float lane_count = 0.0f, lane_mass = 0.0f;
+    const float maximum = value_from_descending_key(first_key);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        const uint32_t bucket = static_cast<uint32_t>(4 * tid + j);
+        uint32_t count = 0;
+#pragma unroll
+        for (int copy = 0; copy < kCutCopies; ++copy)
+            count += counts[copy * kCutStride + bucket];
+        const bool finite = bucket >= kFirstFiniteBucket && bucket <= kLastFiniteBucket;
+        bucket_counts[j] = static_cast<float>(count) * weight;
+        const float lowest = value_from_descending_key((bucket << 20) | 0xfffffu);
+        bucket_least[j] = finite && count != 0u ? bucket_counts[j] * __expf(fminf((lowest - maximum) / temperature, 0.0f)) : 0.0f;
+        lane_count += bucket_counts[j];
+        lane_mass += bucket_least[j];
+    }
+    // sums over the buckets in front of this thread's
+    float count_through = lane_count, mass_through = lane_mass;
+#pragma unroll
+    for (int step = 1; step < kWaveSize; step <<= 1)
+    {
+        const float count_up = __shfl_up(count_through, step, kWaveSize);
+        const float mass_up = __shfl_up(mass_through, step, kWaveSize);
+        if (lane >= step)
+        {
+            count_through += count_up;
+            mass_through += mass_up;
+        }
+    }
+    if (lane == kWaveSize - 1)
+    {
+        wave_counts[wave] = count_through;
+        wave_masses[wave] = mass_through;
+    }
+    __syncthreads();
+    float count_before = count_through - lane_count;
+    float mass_before = mass_through - lane_mass;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w)
+    {
+        count_before += w < wave ? wave_counts[w] : 0.0f;
+        mass_before += w < wave ? wave_masses[w] : 0.0f;
+    }
+    // the first bucket that can be left out, with all behind it
+    uint32_t candidate = kCutBuckets;
+#pragma unroll
+    for (int j = 3; j >= 0; --j)
+    {
+        const uint32_t bucket = static_cast<uint32_t>(4 * tid + j);
+        float count_here = count_before, mass_here = mass_before;
+#pragma unroll
+        for (int i = 0; i < j; ++i)
+        {
+            count_here += bucket_counts[i];
+            mass_here += bucket_least[i];
+        }
+        const float highest = value_from_descending_key(bucket << 20);
+        const float largest_term = __expf(fminf((highest - maximum) / temperature, 0.0f));
+        if (bucket > kFirstFiniteBucket && bucket <= kLastFiniteBucket && count_here >= kCutMinimum &&
+            largest_term < mass_here * 7.450580596923828e-09f) // 2^-27
+            candidate = bucket;
+    }
+    if (candidate < static_cast<uint32_t>(kCutBuckets))
+        atomicMin(&cut_bucket, candidate);
+    __syncthreads();
+    const uint32_t cut = cut_bucket;
+    if (cut >= static_cast<uint32_t>(kCutBuckets))
+        return sort_whole_row();
+    if (tid == 0)
+    {
+        a.sort_last_keys[row] = (cut << 20) - 1u;
+        a.sort_lengths[row] = 0u;   // counted by sort_part_histogram_kernel's first pass
+        a.finite_counts[row] = 0u;  // ... with the row's finite logits and whether it holds a NaN
+    }
 }
 
 template <int DTYPE>
@@ -391,13 +580,19 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(Sampl
     if (!spread_grid_row(a, row))
         return;
     const int tid = threadIdx.x;
-    const uint32_t n = a.vocab;
     const int pass = static_cast<int>(a.sort_pass);
+    // the first pass reads the whole row and keeps the elements that are sorted; the others read those
+    const uint32_t n = pass == 0 ? a.vocab : sorted_length(a, row);
+    const uint32_t last_key = sort_last_key(a, row, pass);
     const int shift = 8 * (pass + kFirstDigit);
     __shared__ uint32_t counts[kHistogramParts][8][257]; // (257: the copies of a digit's counter lie in eight different banks)
     for (int i = tid; i < kHistogramParts * 8 * 257; i += kSortThreads)
         (&counts[0][0][0])[i] = 0;
     __syncthreads();
+    // The first pass of a row that is sorted in part also takes the row's exact counts: the elements that are
+    // kept (the sum of the digits' counts), the finite logits and whether there is a NaN among all of them.
+    const bool counting = pass == 0 && last_key != 0xffffffffu;
+    uint32_t finite_seen = 0, nan_seen = 0;
     const uint32_t part_span = a.sort_tiles_per_part * kSortTile;
     for (uint32_t offset = 0; offset < part_span; offset += kSortTile)
     {
@@ -418,12 +613,54 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(Sampl
             {
                 // (eight copies of the counters, a lane using copy lane % 8: the uppermost digit of a row's keys
                 // takes few values, and 64 atomics on one address take as many turns)
-                if (tile + static_cast<uint32_t>(e * kSortThreads + tid) < n)
+                const bool inside = tile + static_cast<uint32_t>(e * kSortThreads + tid) < n;
+                if (inside && keys[q][e] <= last_key)
                     atomicAdd(&counts[q][tid & 7][(keys[q][e] >> shift) & 255u], 1u);
+                if (counting)
+                {
+                    finite_seen += inside && keys[q][e] > kPositiveInfinityKey && keys[q][e] <= kLastFiniteKey ? 1u : 0u;
+                    nan_seen |= inside && keys[q][e] == 0xffffffffu ? 1u : 0u;
+                }
             }
         }
     }
     __syncthreads();
+    if (counting)
+    {
+        __shared__ uint32_t wave_finite[kSortWaves], wave_kept[kSortWaves], wave_nan[kSortWaves];
+        uint32_t kept = 0;
+        if (tid < 256 * kHistogramParts)
+        {
+#pragma unroll
+            for (int copy = 0; copy < 8; ++copy)
+                kept += counts[tid >> 8][copy][tid & 255];
+        }
+        const uint32_t wave_index = static_cast<uint32_t>(tid) >> 6;
+        const uint32_t finite_total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(finite_seen)), 63));
+        const uint32_t kept_total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_prefix_sum_u32(kept)), 63));
+        const uint32_t nan_total = wave_or_u32(nan_seen);
+        if ((tid & 63) == 0)
+        {
+            wave_finite[wave_index] = finite_total;
+            wave_kept[wave_index] = kept_total;
+            wave_nan[wave_index] = nan_total;
+        }
+        __syncthreads();
+        if (tid == 0)
+        {
+            uint32_t finite_all = 0, kept_all = 0, nan_all = 0;
+            for (int w = 0; w < kSortWaves; ++w)
+            {
+                finite_all += wave_finite[w];
+                kept_all += wave_kept[w];
+                nan_all |= wave_nan[w];
+            }
+            atomicAdd(&a.sort_lengths[row], kept_all);
+            atomicAdd(&a.finite_counts[row], finite_all);
+            if (nan_all != 0u)
+                atomicOr(&a.finite_counts[row], kRowHoldsNan);
+        }
+    }
     {
         const int q = tid >> 8; // kSortThreads / 256 == kHistogramParts
         const int digit = tid & 255;
@@ -454,8 +691,10 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
-    const uint32_t n = a.vocab;
     const int pass = static_cast<int>(a.sort_pass);
+    // the first pass reads the whole row and keeps the elements that are sorted; the others read those
+    const uint32_t n = pass == 0 ? a.vocab : sorted_length(a, row);
+    const uint32_t last_key = sort_last_key(a, row, pass);
     const int shift = 8 * (pass + kFirstDigit);
 
     __shared__ uint32_t digit_base[256];          // output position of the next key of each digit
@@ -469,18 +708,34 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
     uint32_t* target_keys = a.sort_keys[pass & 1] + row * a.sort_stride;
     uint32_t* target_indices = a.sort_indices[pass & 1] + row * a.sort_stride;
 
+    // the first tile is asked for before the parts' counts: the two trips to memory overlap
+    const uint32_t first_tile = part * a.sort_tiles_per_part * kSortTile;
+    const uint32_t end = min(n, first_tile + a.sort_tiles_per_part * kSortTile);
+    if (first_tile >= end)
+        return;
+    uint32_t tile_keys[kSortPerThread];
+    uint32_t tile_indices[kSortPerThread];
+    load_sort_keys<DTYPE, PAIRS>(a, row, pass, first_tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread), n, lane, kWaveSize,
+                                 tile_keys, tile_indices);
+
     // where this part's keys of every digit go: behind the row's smaller digits and behind the same
     // digit's keys of the parts before this one
     {
         uint32_t row_total = 0, before = 0, inclusive = 0;
         if (tid < 256)
         {
+            // (every part's count is asked for before the first is used: a loop of the parts' real number would
+            // wait for each load in turn, sixteen trips to memory one behind the other)
             const uint32_t* counts = a.sort_part_counts + static_cast<size_t>(row) * a.sort_parts * 256 + tid;
-            for (uint32_t g = 0; g < a.sort_parts; ++g)
+            uint32_t part_counts[kMaxSortParts];
+#pragma unroll
+            for (uint32_t g = 0; g < static_cast<uint32_t>(kMaxSortParts); ++g)
+                part_counts[g] = g < a.sort_parts ? counts[static_cast<size_t>(g) * 256] : 0u;
+#pragma unroll
+            for (uint32_t g = 0; g < static_cast<uint32_t>(kMaxSortParts); ++g)
             {
-                const uint32_t c = counts[static_cast<size_t>(g) * 256];
-                row_total += c;
-                before += g < part ? c : 0u;
+                row_total += part_counts[g];
+                before += g < part ? part_counts[g] : 0u;
             }
             inclusive = row_total;
 #pragma unroll
@@ -505,19 +760,14 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
         __syncthreads();
     }
 
-    const uint32_t first_tile = part * a.sort_tiles_per_part * kSortTile;
-    const uint32_t end = min(n, first_tile + a.sort_tiles_per_part * kSortTile);
-    if (first_tile >= end)
-        return;
     // A wave owns 512 consecutive keys of a tile and ranks them in 8 rounds of 64, so that the order
     // inside the wave is the input order (see general_sort_kernel).
-    // (no tile is fetched ahead: a workgroup has one tile or few, and two workgroups share a compute unit)
+    // (no later tile is fetched ahead: a workgroup has one tile or few, and two workgroups share a compute unit)
     for (uint32_t tile = first_tile; tile < end; tile += kSortTile)
     {
-        uint32_t tile_keys[kSortPerThread];
-        uint32_t tile_indices[kSortPerThread];
-        load_sort_keys<DTYPE, PAIRS>(a, row, pass, tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread), n, lane, kWaveSize,
-                                     tile_keys, tile_indices);
+        if (tile != first_tile)
+            load_sort_keys<DTYPE, PAIRS>(a, row, pass, tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread), n, lane, kWaveSize,
+                                         tile_keys, tile_indices);
         for (int i = tid; i < kSortWaves * 256; i += kSortThreads)
             (&wave_counts[0][0])[i] = 0;
         uint32_t tile_ranks[kSortPerThread];
@@ -527,7 +777,7 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
         for (int e = 0; e < kSortPerThread; ++e)
         {
             const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
-            const bool valid = i < n;
+            const bool valid = i < n && tile_keys[e] <= last_key;
             const uint32_t digit = (tile_keys[e] >> shift) & 255u;
             if (ANY_ORDER)
             {
@@ -580,13 +830,16 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
             tile_start[tid] = start;
             global_offset[tid] = digit_base[tid] - start;
             digit_base[tid] += digit_total;
+            if (tid == 255)
+                scan_partial[3] = start + digit_total; // the tile's keys that are kept (read behind the next barrier;
+                                                       // its readers as a wave's total are in front of this one)
         }
         lds_barrier();
 #pragma unroll
         for (int e = 0; e < kSortPerThread; ++e)
         {
             const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
-            if (i < n)
+            if (i < n && tile_keys[e] <= last_key)
             {
                 const uint32_t digit = (tile_keys[e] >> shift) & 255u;
                 const uint32_t slot = tile_start[digit] + wave_counts[wave][digit] + tile_ranks[e];
@@ -596,7 +849,7 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
             }
         }
         lds_barrier();
-        const uint32_t tile_count = min(static_cast<uint32_t>(kSortTile), n - tile);
+        const uint32_t tile_count = scan_partial[3];
 #pragma unroll
         for (int e = 0; e < kSortPerThread; ++e)
         {
@@ -963,13 +1216,14 @@ __device__ __noinline__ int32_t recover_token_of_key(
 
 template <int DTYPE>
 __device__ __forceinline__ int32_t recover_token_index(
-    const void* row_pointer, uint32_t vocab, const uint32_t* keys, uint32_t rank, RecoverScratch& scratch, int tid)
+    const void* row_pointer, uint32_t vocab, const uint32_t* keys, uint32_t sorted, uint32_t rank, RecoverScratch& scratch, int tid)
 {
     const uint32_t key = keys[rank];
-    // first position holding this key, and the first behind it
+    // first position holding this key, and the first behind it (`sorted` keys are there; a row sorted in part ends
+    // between two different keys)
     const uint32_t low = wave_partition_point(rank, [keys, key](uint32_t position) { return keys[position] < key; });
     const uint32_t high = rank + 1u +
-        wave_partition_point(vocab - rank - 1u, [keys, key, rank](uint32_t position) { return keys[rank + 1u + position] <= key; });
+        wave_partition_point(sorted - rank - 1u, [keys, key, rank](uint32_t position) { return keys[rank + 1u + position] <= key; });
     return recover_token_of_key<DTYPE>(row_pointer, vocab, key, rank - low, high - low, scratch, tid);
 }
 
@@ -1158,8 +1412,10 @@ __device__ __forceinline__ void replay_row(
     const bool have_indices = !RUNS && a.distribution_count != nullptr; // the pair sort ran: indices are valid
     const uint32_t* indices = have_indices ? a.sort_indices[1] + row * a.sort_stride : nullptr;
     const uint32_t vocab = a.vocab;
+    // a row of elements may be sorted in part: its first elements in sorted order, all finite, and counts of the rest
+    const bool sorted_in_part = !RUNS && a.sort_lengths != nullptr && a.sort_last_keys[row] != 0xffffffffu;
     // items: what `keys` holds one entry of (an element, or a run of equal keys)
-    const uint32_t items = RUNS ? run_total : vocab;
+    const uint32_t items = RUNS ? run_total : sorted_length(a, row);
     const char* row_pointer = static_cast<const char*>(a.logits) +
         static_cast<size_t>(row) * a.row_stride * LogitsVector<DTYPE>::kElementBytes;
 
@@ -1173,7 +1429,7 @@ __device__ __forceinline__ void replay_row(
         if (resolve_row_mode(p, vocab, a.max_select_top_k, 0, effective_k, status) != kModeGeneral)
             flags |= NCNN_MOE_ROW_FLAG_FALLBACK;
     }
-    if (keys[items - 1] == 0xffffffffu)
+    if (sorted_in_part ? (a.finite_counts[row] & kRowHoldsNan) != 0u : keys[items - 1] == 0xffffffffu)
         flags |= NCNN_MOE_ROW_FLAG_HAS_NAN;
     if (tid == 0)
         a.row_state[row] = kRowDone;
@@ -1199,7 +1455,7 @@ __device__ __forceinline__ void replay_row(
             return recover_token_of_key<DTYPE>(row_pointer, vocab, keys[run], rank - run_first, run_ends[run] - run_first, recover_scratch, tid);
         }
         else
-            return recover_token_index<DTYPE>(row_pointer, vocab, keys, rank, recover_scratch, tid);
+            return recover_token_index<DTYPE>(row_pointer, vocab, keys, items, rank, recover_scratch, tid);
     };
 
     if (p.temperature == 0.0f)
@@ -1242,7 +1498,7 @@ __device__ __forceinline__ void replay_row(
     }
     // first item whose key is not finite
     const uint32_t low = wave_partition_point(items, [keys](uint32_t item) { return keys[item] <= kLastFiniteKey; });
-    const uint32_t finite_elements = first_element(low);
+    const uint32_t finite_elements = sorted_in_part ? a.finite_counts[row] & ~kRowHoldsNan : first_element(low);
     uint32_t n = finite_elements;
     if (p.top_k > 0 && p.top_k < vocab && n > p.top_k)
         n = p.top_k;
@@ -1254,8 +1510,18 @@ __device__ __forceinline__ void replay_row(
             chunk_steps = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity;
     }
     // (the finite runs and the elements they hold: a sum over all of them need not look for its last run)
+    bool tail_matters = false;
     replay_sorted_window<RUNS>(
-        a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0, chunk_steps, a.vocab, RUNS ? low : 0u, finite_elements);
+        a, row, p, keys, run_ends, items, n, indices, flags, scratch, tid, token_at, terms0, chunk_steps, RUNS ? vocab : items,
+        RUNS ? low : 0u, finite_elements, sorted_in_part ? items : 0xffffffffu, sorted_in_part ? a.sort_last_keys[row] + 1u : 0u, &tail_matters);
+    // An element that was left out of the sort could have moved a sum, or been the one drawn: the row stays
+    // pending, and the launch behind this one sorts it whole.
+    if (tail_matters && tid == 0)
+    {
+        a.sort_last_keys[row] = 0xffffffffu;
+        a.sort_lengths[row] = vocab;
+        a.row_state[row] = kRowNeedsGeneral;
+    }
 }
 
 template <int DTYPE, bool RUNS>
@@ -1316,7 +1582,8 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
         if (a.terms_precomputed == 0 && p.temperature != 0.0f)
         {
             const float maximum = value_from_descending_key(keys[0]) / p.temperature;
-            for (uint32_t i = threadIdx.x; i < a.vocab; i += kReplayThreads)
+            const uint32_t sorted = sorted_length(a, row);
+            for (uint32_t i = threadIdx.x; i < sorted; i += kReplayThreads)
                 terms[i] = term_of_key(keys[i], maximum);
             __syncthreads();
         }
@@ -1454,6 +1721,9 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
     __shared__ uint64_t exp2_table[32]; // a copy in LDS: the lookups of a wave are 64 different addresses
     if (threadIdx.x < 32)
         exp2_table[threadIdx.x] = kExp2Table[threadIdx.x];
+    const uint32_t n = sorted_length(a, row);
+    if (blockIdx.x * (kTermsThreads * kTermsPerThread) >= n)
+        return; // (behind the row's sorted elements: no chunk reads this block's sum)
     const float temperature = a.params[row].temperature;
     const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
     float* terms = reinterpret_cast<float*>(a.sort_keys[0] + row * a.sort_stride);
@@ -1464,7 +1734,7 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
     for (int j = 0; j < kTermsPerThread; ++j)
     {
         const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
-        loaded[j] = i < a.vocab ? keys[i] : 0u;
+        loaded[j] = i < n ? keys[i] : 0u;
     }
     __syncthreads();
     double sum = 0.0;
@@ -1472,7 +1742,7 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
     for (int j = 0; j < kTermsPerThread; ++j)
     {
         const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
-        if (i < a.vocab)
+        if (i < n)
         {
             const float term = expf_libm(value_from_descending_key(loaded[j]) / temperature - maximum, exp2_table);
             terms[i] = term;
@@ -1525,6 +1795,9 @@ __global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kern
     const float* terms = reinterpret_cast<const float*>(a.sort_keys[0] + row * a.sort_stride);
     uint4* const out = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity + chunk;
     const uint32_t base = chunk * kReplayChunk;
+    const uint32_t n = sorted_length(a, row);
+    if (base >= n)
+        return; // (behind the row's sorted elements: the replay does not look at this chunk)
     // the chunk's terms are asked for first: the estimate below is a chain of loads, a reduction and a barrier
     // (the row's last chunk may be a partial one: the terms behind the row count as zero)
     const uint32_t first = base + static_cast<uint32_t>(tid) * kChunkStepPerThread;
@@ -1533,11 +1806,11 @@ __global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kern
     for (int j = 0; j < kChunkStepPerThread / 4; ++j)
     {
         const uint32_t at = first + 4u * static_cast<uint32_t>(j);
-        if (at + 4u <= a.vocab)
+        if (at + 4u <= n)
             loaded[j] = *reinterpret_cast<const float4*>(terms + at);
         else
-            loaded[j] = float4{at < a.vocab ? terms[at] : 0.0f, at + 1u < a.vocab ? terms[at + 1u] : 0.0f,
-                               at + 2u < a.vocab ? terms[at + 2u] : 0.0f, 0.0f};
+            loaded[j] = float4{at < n ? terms[at] : 0.0f, at + 1u < n ? terms[at + 1u] : 0.0f,
+                               at + 2u < n ? terms[at + 2u] : 0.0f, 0.0f};
     }
     // the sum in front of the chunk: the blocks of the terms kernel before it, or (first chunk) the head of
     // terms that every running sum adds one by one

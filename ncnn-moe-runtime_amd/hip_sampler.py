@@ -73,6 +73,8 @@ TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_scatter_segments",
     "ncnn_moe_hip_sampler_debug_spread_sort",
     "ncnn_moe_hip_sampler_debug_fused_bf16",
+    "ncnn_moe_hip_sampler_debug_partial_sort",
+    "ncnn_moe_hip_sampler_debug_sort_lengths",
     "ncnn_moe_hip_sampler_debug_chunk_steps",
     "ncnn_moe_hip_sampler_debug_stream_only",
     "ncnn_moe_hip_sampler_debug_set_row_epochs",
@@ -118,6 +120,8 @@ def _bind(lib, testing):
     lib.ncnn_moe_hip_sampler_debug_force_general.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_scatter_segments.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_spread_sort.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_partial_sort.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_sort_lengths.argtypes = [vp, vp, ctypes.c_uint32]
     lib.ncnn_moe_hip_sampler_debug_fused_bf16.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_chunk_steps.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_stream_only.argtypes = [vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp]
@@ -330,6 +334,16 @@ class HipSampler:
         """Test hook: the radix sort of long full-order rows on several workgroups (default) or on one."""
         self._check(self._hooks().ncnn_moe_hip_sampler_debug_spread_sort(self._handle, 1 if enabled else 0))
 
+    def partial_sort(self, enabled):
+        """Test hook: full-order fp32 rows sorted only as far as their terms can move a sum (default) or whole."""
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_partial_sort(self._handle, 1 if enabled else 0))
+
+    def sort_lengths(self, rows):
+        """Test hook: elements sorted of each of the last call's first `rows` rows (SORT_WHOLE_ROW: all of them)."""
+        out = np.empty(rows, dtype=np.uint32)
+        self._check(self._hooks(True).ncnn_moe_hip_sampler_debug_sort_lengths(self._handle, out.ctypes.data, rows))
+        return out
+
     def fused_bf16(self, enabled):
         """Test hook: bf16 full-order rows counted and walked by one kernel (default) or by two."""
         self._check(self._hooks().ncnn_moe_hip_sampler_debug_fused_bf16(self._handle, 1 if enabled else 0))
@@ -347,6 +361,7 @@ class HipSampler:
 
 STATIC_MAX_ROWS = 1024
 LAST_EPOCH = 16383  # the launch numbers of the split kernel's records run 1 .. LAST_EPOCH and start over
+SORT_WHOLE_ROW = 0xFFFFFFFF  # sort_lengths(): the row is sorted whole
 
 
 def set_static_row_epochs(device, epoch):

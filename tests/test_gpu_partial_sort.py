@@ -1,0 +1,126 @@
+"""Full-order fp32 rows that are sorted only in part (GPU): a kernel guesses how far down the sorted row a term
+can still move one of the sampler's sums, only that much of the row is sorted, and the walk checks the guess
+against its exact sums.  The results must be the oracle's, byte for byte those of the whole sort, and a row whose
+guess turns out too short must come back from the second launch that sorts it whole."""
+import numpy as np
+import pytest
+
+import parity_util
+from ncnn_moe_runtime_amd import hip_sampler
+
+pytestmark = pytest.mark.gpu
+
+ROWS, VOCAB = 40, 70001  # nine tiles of 8,192 keys: the sort is spread over several workgroups
+
+
+def _announce(text):
+    print("[case] " + text, flush=True)
+
+
+@pytest.fixture(scope="module")
+def sampler():
+    handle = hip_sampler.HipSampler(ROWS, VOCAB, testing=True)
+    yield handle
+    handle.close()
+
+
+def _rows(seed, spread=2.0):
+    rng = np.random.default_rng(seed)
+    logits = (rng.standard_normal((ROWS, VOCAB)) * spread).astype(np.float32)
+    params = hip_sampler.make_params(ROWS, 1.0, 0, 1.0, 0.0)
+    params["temperature"] = np.linspace(0.05, 1.5, ROWS).astype(np.float32)
+    return rng, logits, params
+
+
+def _sample_both_ways(sampler, logits, params, uniforms, context):
+    """The oracle's results, from the partial sort and from the whole sort; returns the partial sort's results and
+    how many elements of each row it sorted in the end."""
+    _announce(context)
+    sampler.upload_logits(logits)
+    partial = sampler.sample(params, uniforms, None)
+    lengths = sampler.sort_lengths(ROWS)
+    sampler.partial_sort(False)
+    try:
+        whole = sampler.sample(params, uniforms, None)
+    finally:
+        sampler.partial_sort(True)
+    cpu = parity_util.run_oracle(logits, params, uniforms)
+    parity_util.assert_results_match(partial, cpu, "f32", context)
+    assert partial.tobytes() == whole.tobytes(), context
+    return partial, lengths
+
+
+def test_rows_are_sorted_as_far_as_their_terms_matter(sampler):
+    """Temperatures from 0.05 to 1.5 over N(0, 4) logits: the cold rows are sorted a few thousand elements deep, the
+    warm ones whole; Top-P and Min-P cuts on some rows, a wide Top-K on others."""
+    rng, logits, params = _rows(4100)
+    params["top_p"] = np.where(np.arange(ROWS) % 3 == 0, 1.0, rng.uniform(0.5, 0.999, size=ROWS)).astype(np.float32)
+    params["min_p"] = np.where(np.arange(ROWS) % 4 == 1, rng.uniform(0.0, 0.05, size=ROWS), 0.0).astype(np.float32)
+    params["top_k"][6::9] = 3000  # wider than the select kernels take, narrower than some rows' sorted part
+    for trial in range(3):
+        uniforms = rng.random(ROWS, dtype=np.float32)
+        gpu, lengths = _sample_both_ways(sampler, logits, params, uniforms, "partial sort, draw %d" % trial)
+        assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+    shortened = lengths < VOCAB
+    assert shortened[:ROWS // 3].all(), lengths        # cold rows: a small part
+    assert (lengths[:ROWS // 4] < VOCAB // 4).all(), lengths
+    assert not shortened[-3:].any(), lengths           # T around 1.5 over N(0, 4): every term matters
+    assert (lengths[shortened] >= 4096).all(), lengths
+
+
+def test_rows_whose_guess_is_too_short_are_sorted_whole(sampler):
+    """A draw that no partial sum exceeds takes the row's last element, and a Min-P threshold below every term
+    keeps the whole row: neither can be served from the sorted part, and the rows come back from the second
+    launch."""
+    rng, logits, params = _rows(4200)
+    ordinary = rng.random(ROWS, dtype=np.float32)
+    _, lengths_before = _sample_both_ways(sampler, logits, params, ordinary, "partial sort, ordinary draws")
+    shortened = lengths_before < VOCAB
+    assert shortened.sum() >= ROWS // 2
+    # the largest uniform below one: the renormalised probabilities of about half the rows add up to no more
+    last = np.full(ROWS, np.float32(1.0) - np.float32(2.0 ** -24), dtype=np.float32)
+    gpu, lengths = _sample_both_ways(sampler, logits, params, last, "partial sort, draws at the top of [0, 1)")
+    sent_back = shortened & (lengths == hip_sampler.SORT_WHOLE_ROW)
+    assert sent_back.any(), lengths
+    assert (gpu["kept_count"][sent_back] == VOCAB).all()
+    # a Min-P threshold far below the smallest probability
+    params["min_p"] = np.float32(1e-30)
+    _, lengths = _sample_both_ways(sampler, logits, params, ordinary, "partial sort, Min-P below every probability")
+    # (but for the coldest rows, whose smallest terms are zero and stay below any threshold)
+    assert (lengths[shortened][-5:] == hip_sampler.SORT_WHOLE_ROW).all(), lengths
+
+
+def test_rows_with_logits_that_are_not_finite(sampler):
+    """-inf and NaN lie behind the sorted part of a row (they are counted, and NaN is flagged); +inf rejects the
+    row; a row of few finite logits is sorted whole."""
+    rng, logits, params = _rows(4300)
+    params["temperature"] = np.float32(0.4)
+    logits[0, 100:5000] = -np.inf
+    logits[1, ::7] = np.nan
+    logits[2, 17] = np.inf
+    logits[3, :] = -np.inf
+    logits[3, 5:2000] = rng.standard_normal(1995).astype(np.float32)
+    logits[4, 9::2] = np.nan
+    logits[4, 8::2] = -np.inf
+    logits[5, :] = -np.inf
+    logits[6, :] = np.nan
+    params["top_p"][7:] = rng.uniform(0.7, 1.0, size=ROWS - 7).astype(np.float32)
+    uniforms = rng.random(ROWS, dtype=np.float32)
+    gpu, lengths = _sample_both_ways(sampler, logits, params, uniforms, "partial sort, infinities and NaN")
+    assert gpu["status"][2] != 0 and gpu["status"][5] != 0 and gpu["status"][6] != 0
+    assert lengths[0] < VOCAB and lengths[1] < VOCAB
+    assert (gpu["flags"][1] & hip_sampler.FLAG_HAS_NAN) != 0
+
+
+def test_heavy_ties_and_narrow_rows(sampler):
+    """Rows of a few dozen distinct values (a bucket of the guess holds thousands of equal keys), rows whose logits
+    all lie in one bucket, and rows at a temperature so low that the sorted part is the minimum."""
+    rng, logits, params = _rows(4400)
+    logits[0:8] = np.round(logits[0:8])
+    logits[8:12] = (1.0 + rng.random((4, VOCAB)) * 0.05).astype(np.float32)  # one bucket holds the row
+    logits[12:16] = (rng.integers(0, 3, size=(4, VOCAB)) * 8.0).astype(np.float32)
+    params["temperature"][16:20] = np.float32(0.01)
+    params["top_p"] = rng.uniform(0.6, 1.0, size=ROWS).astype(np.float32)
+    for trial in range(2):
+        uniforms = rng.random(ROWS, dtype=np.float32)
+        _sample_both_ways(sampler, logits, params, uniforms, "partial sort, ties and narrow rows, draw %d" % trial)
