@@ -157,7 +157,7 @@ int ncnn_moe_hip_sampler_sample_device(
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  The select pass of
  * ncnn_moe_hip_sampler_sample_device (may_need_full_order = 0) without a handle: the call allocates
  * nothing, on the device or through any library; its scratch (the segments' candidate records and the
- * per-row hand-over words, 13.6 MB) is a static device array that every GPU the library runs on holds
+ * per-row hand-over words, 18.8 MB) is a static device array that every GPU the library runs on holds
  * from its first call until the process ends.  Greedy rows and rows with 1 <= top_k <= 64 are final;
  * any other row comes back NCNN_MOE_ROW_NEEDS_FULL_ORDER.  Limits: rows <= NCNN_MOE_STATIC_MAX_ROWS,
  * any vocab; a larger batch is rejected with NCNN_MOE_SAMPLER_INVALID_ARGUMENT and the reason is

@@ -40,7 +40,7 @@ int ncnn_moe_hip_sampler_debug_fused_bf16(ncnn_moe_hip_sampler* sampler, int ena
  * were sorted (0xffffffff: the whole row; only rows that took the spread sort with partial_sort on are written). */
 int ncnn_moe_hip_sampler_debug_partial_sort(ncnn_moe_hip_sampler* sampler, int enabled);
 int ncnn_moe_hip_sampler_debug_sort_lengths(ncnn_moe_hip_sampler* sampler, uint32_t* lengths, uint32_t rows);
-/* Sets the per-row launch numbers (epochs, 1 .. 16383) that tag the split kernel's hand-over records: of the
+/* Sets the per-row launch numbers (epochs, 1 .. 8191) that tag the split kernel's hand-over records: of the
  * handle, or with a null handle of the static scratch of `device` (after it has served a call).  Tests start a
  * few launches in front of the point where the epochs start over. */
 int ncnn_moe_hip_sampler_debug_set_row_epochs(ncnn_moe_hip_sampler* sampler, int device, uint32_t epoch);

@@ -173,9 +173,9 @@ SelectGeometry select_geometry(int dtype, uint64_t span, uint32_t rows, bool wid
     SelectGeometry g;
     g.wide = wide;
     const uint64_t total_chunks = std::max<uint64_t>(1, (span + chunk_values(dtype) - 1) / chunk_values(dtype));
-    auto split = [&](int workgroups) {
+    auto split = [&](int workgroups, int most) {
         const uint64_t wanted = (static_cast<uint64_t>(workgroups) + rows - 1) / rows;
-        uint64_t segments = std::min<uint64_t>(std::min<uint64_t>(wanted, total_chunks), static_cast<uint64_t>(kMaxSegments));
+        uint64_t segments = std::min<uint64_t>(std::min<uint64_t>(wanted, total_chunks), static_cast<uint64_t>(most));
         const uint64_t chunks_per_segment = (total_chunks + segments - 1) / segments;
         segments = (total_chunks + chunks_per_segment - 1) / chunks_per_segment;
         g.segments = static_cast<uint32_t>(segments);
@@ -188,9 +188,13 @@ SelectGeometry select_geometry(int dtype, uint64_t span, uint32_t rows, bool wid
     }
     else
     {
-        split(kSingleChunkWorkgroups);
-        if (g.chunks_per_segment > 1)
-            split(kLoopedWorkgroups); // the looped kernel keeps two workgroups per CU resident
+        split(kSingleChunkWorkgroups, kSplitMaxSegments);
+        // (bf16 rows of more than 16 chunks: from about 2,300 one-chunk workgroups on the looped kernel is as fast or
+        // faster - 128 x 262,144: 27.6 us against 31.1; fp32 rows are faster in one-chunk workgroups at every batch size)
+        const bool long_bf16_rows = dtype == NCNN_MOE_LOGITS_BF16 && g.segments > static_cast<uint32_t>(kMaxSegments) &&
+            static_cast<uint64_t>(rows) * g.segments > 2304u;
+        if (g.chunks_per_segment > 1 || long_bf16_rows)
+            split(kLoopedWorkgroups, kMaxSegments); // the looped kernel keeps two workgroups per CU resident
     }
     g.looped = g.chunks_per_segment > 1 || g.segments == 1;
     return g;
@@ -243,8 +247,10 @@ void launch_select(const SelectGeometry& g, uint32_t rows, hipStream_t stream, S
         hipLaunchKernelGGL((scan_select_kernel<DTYPE, true, true>), grid, dim3(kScanThreads), 0, stream, a);
     else if (g.looped)
         hipLaunchKernelGGL((scan_select_kernel<DTYPE, true, false>), grid, dim3(kScanThreads), 0, stream, a);
+    else if (g.segments > static_cast<uint32_t>(kMaxSegments))
+        hipLaunchKernelGGL((split_select_kernel<DTYPE, kSplitMaxSegments>), grid, dim3(kScanThreads), 0, stream, a);
     else if (g.segments > 1)
-        hipLaunchKernelGGL((split_select_kernel<DTYPE>), grid, dim3(kScanThreads), 0, stream, a);
+        hipLaunchKernelGGL((split_select_kernel<DTYPE, 16>), grid, dim3(kScanThreads), 0, stream, a);
     else
         hipLaunchKernelGGL((scan_select_kernel<DTYPE, false, false>), grid, dim3(kScanThreads), 0, stream, a);
 }
@@ -308,7 +314,7 @@ int launch_sampler(
         a.distribution_count = export_to.count;
     }
     const SelectGeometry batch_geometry = select_geometry(dtype, span, rows, false);
-    if (batch_geometry.segments > s->max_segments)
+    if (batch_geometry.looped && batch_geometry.segments > s->max_segments)
         return fail(s, NCNN_MOE_SAMPLER_INVALID_ARGUMENT, "vocab exceeds the handle's max_vocab");
 
     // only_pending: 1 = the rows an earlier launch left pending, 2 = the rows whose options ask for a wide window
@@ -498,7 +504,7 @@ struct StaticScratchLayout
     unsigned long long row_counter[kStaticMaxRows];
     uint32_t row_flags[kStaticMaxRows];
     uint32_t row_state[kStaticMaxRows];
-    unsigned long long split_records[static_cast<size_t>(kStaticSplitRows) * kMaxSegments * kSplitRecordSlots];
+    unsigned long long split_records[static_cast<size_t>(kStaticSplitRows) * kSplitMaxSegments * kSplitRecordSlots];
     uint32_t row_epoch[kStaticMaxRows];
 };
 static_assert(kStaticMaxRows >= kStaticSplitRows, "a split batch must fit the per-row words");
@@ -527,8 +533,9 @@ __global__ void static_scratch_clear_kernel(StaticScratchLayout* layout)
         layout->row_epoch[i] = 1u;
     }
     if (i < kStaticSplitRows * kMaxSegments)
-    {
         layout->segment_counts[i] = 0u;
+    if (i < kStaticSplitRows * kSplitMaxSegments)
+    {
         for (uint32_t entry = 0; entry < static_cast<uint32_t>(kSplitRecordSlots); ++entry)
             layout->split_records[static_cast<size_t>(i) * kSplitRecordSlots + entry] = 0ull; // epoch 0 tags nothing
     }
@@ -611,8 +618,8 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipMalloc(&s->row_state, rows * sizeof(uint32_t)));
     // split path: records start untagged (epoch 0 tags nothing), every row at epoch 1
     const size_t split_rows = std::min<size_t>(rows, static_cast<size_t>(kWholeRowBatch) - 1);
-    CREATE_CHECK(hipMalloc(&s->split_records, split_rows * kMaxSegments * kSplitRecordSlots * sizeof(unsigned long long)));
-    CREATE_CHECK(hipMemset(s->split_records, 0, split_rows * kMaxSegments * kSplitRecordSlots * sizeof(unsigned long long)));
+    CREATE_CHECK(hipMalloc(&s->split_records, split_rows * kSplitMaxSegments * kSplitRecordSlots * sizeof(unsigned long long)));
+    CREATE_CHECK(hipMemset(s->split_records, 0, split_rows * kSplitMaxSegments * kSplitRecordSlots * sizeof(unsigned long long)));
     CREATE_CHECK(hipMalloc(&s->row_epoch, rows * sizeof(uint32_t)));
     CREATE_CHECK(hipMemsetD32(reinterpret_cast<hipDeviceptr_t>(s->row_epoch), 1, rows));
     CREATE_CHECK(hipMemset(s->segment_counts, 0, slots * sizeof(uint32_t)));
@@ -895,7 +902,7 @@ int ncnn_moe_hip_sampler_sample_device_static(
             if (error != hipSuccess || address == nullptr)
                 return static_fail(NCNN_MOE_SAMPLER_HIP_ERROR, "hipGetSymbolAddress(scratch)", hipGetErrorString(error));
             constexpr uint32_t kClearThreads = 256;
-            constexpr uint32_t kClearWords = std::max<uint32_t>(kStaticSplitRows * kMaxSegments, kStaticMaxRows);
+            constexpr uint32_t kClearWords = std::max<uint32_t>(kStaticSplitRows * kSplitMaxSegments, kStaticMaxRows);
             hipLaunchKernelGGL(static_scratch_clear_kernel, dim3((kClearWords + kClearThreads - 1) / kClearThreads), dim3(kClearThreads), 0, on,
                                static_cast<StaticScratchLayout*>(address));
             error = hipGetLastError();

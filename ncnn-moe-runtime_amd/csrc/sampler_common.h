@@ -36,8 +36,8 @@ struct SamplerArgs
     uint32_t xcd_grouped;      // the grid is one-dimensional and puts the segments of a row on one XCD
     uint32_t* row_flags;       // [rows], zero between launches
     uint32_t* row_state;       // [rows], written by every launch
-    // split path: [rows][kMaxSegments][kSplitRecordSlots] entries of (key, epoch | token index), and the
-    // row's epoch (1 .. 16383; the row's last workgroup moves it on in every launch)
+    // split path: [rows][kSplitMaxSegments][kSplitRecordSlots] entries of (key, epoch | token index), and the
+    // row's epoch (1 .. 8191; the row's last workgroup moves it on in every launch)
     unsigned long long* split_records;
     uint32_t* row_epoch;
 

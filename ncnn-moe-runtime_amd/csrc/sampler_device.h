@@ -30,9 +30,10 @@ constexpr int kNarrowListCap = 512;      // candidate list for Top-K windows up 
 constexpr int kWideListCap = 4096;       // candidate list for Top-K windows up to kSelectTopK
 constexpr int kSegmentRecordSlots = 256; // candidate slots of a segment's record in HBM
 constexpr int kMaxSegments = 16;
+constexpr int kSplitMaxSegments = 32;   // ... of one chunk each, on the split path
 constexpr int kSplitRecordSlots = 160;   // 8-byte entries of a segment's record on the split path: 2 header entries + up to 2 * 64 + 16 candidates
 constexpr int kWholeRowBatch = 256;          // from this many rows on, one workgroup streams a whole row
-constexpr int kSingleChunkWorkgroups = 4096;  // a smaller batch is split into one-chunk workgroups up to this many (several rounds of 4 per CU beat fewer, looped ones)
+constexpr int kSingleChunkWorkgroups = 8192;  // a smaller batch is split into one-chunk workgroups up to this many (several rounds of 4 per CU beat fewer, looped ones)
 constexpr int kLoopedWorkgroups = 512;        // ... and when each streams several chunks (2 per CU)
          // segments per row the row merge can stage in one trip
 constexpr int kMergeStageSlots = 4096;   // record slots of a row loaded in one trip (8 per thread)
@@ -133,7 +134,7 @@ __device__ unsigned long long g_timeline_rows[kTimelineRows * kTimelineSlots];
 #define NCNN_MOE_LSTAMP_FLUSH(row, segment, first, last)                                                     \
     do                                                                                                       \
     {                                                                                                        \
-        if (threadIdx.x == 0 && (row) < static_cast<uint32_t>(kTimelineRows))                                \
+        if (threadIdx.x == 0 && (row) < static_cast<uint32_t>(kTimelineRows) && (segment) < static_cast<uint32_t>(kMaxSegments)) \
         {                                                                                                    \
             for (int slot_ = (first); slot_ <= (last); ++slot_)                                              \
                 g_timeline[((row) * kMaxSegments + (segment)) * kTimelineSlots + slot_] = timeline_staging[slot_]; \

@@ -26,17 +26,17 @@
 namespace ncnn_moe_hip {
 
 constexpr int kSplitHeaderEntries = 2;  // (segment bound, count | flags) and (segment maximum, 0)
-constexpr int kSplitLanesPerSegment = kScanThreads / kMaxSegments; // 32 lanes read one segment's record
-constexpr int kSplitSlotsPerLane = (kSplitRecordSlots + kSplitLanesPerSegment - 1) / kSplitLanesPerSegment;
-constexpr uint32_t kSplitIndexBits = 18; // a split row holds at most 16 chunks of 12,288 logits
+// The kernel comes in two shapes: rows of up to 16 one-chunk workgroups, whose merge reads a segment's record with
+// 32 lanes, and rows of 17 to kSplitMaxSegments (fp32 rows beyond 163,840 logits, bf16 rows beyond 196,608), read
+// with 16 lanes a segment.  A record's place in memory is the same for both: a row's records lie kSplitMaxSegments apart.
+constexpr uint32_t kSplitIndexBits = 19; // a split row holds at most 32 chunks of 12,288 logits
 constexpr uint32_t kSplitIndexMask = (1u << kSplitIndexBits) - 1u;
-constexpr uint32_t kSplitLastEpoch = (1u << (32 - kSplitIndexBits)) - 1u; // epochs run 1 .. 16383; 0 never tags an entry
+constexpr uint32_t kSplitLastEpoch = (1u << (32 - kSplitIndexBits)) - 1u; // epochs run 1 .. 8191; 0 never tags an entry
 constexpr int kSplitBins = kWaveSize;    // one histogram bin per lane of the scanning wave
 constexpr int kSplitBinCapacity = 16;    // candidates of one bin that the merge orders in place (more: the list and its rankings)
 constexpr uint32_t kSplitRetryLimit = 1u << 16;
-static_assert(kMaxSegments * kSegmentValuesBF16 + 8 <= (1 << kSplitIndexBits), "token indices of a split row fit the entry");
+static_assert(kSplitMaxSegments * kSegmentValuesBF16 + 8 <= (1 << kSplitIndexBits), "token indices of a split row fit the entry");
 static_assert(kSplitHeaderEntries + 2 * kFastTopK + 16 <= kSplitRecordSlots, "a record holds the widest hand-over");
-static_assert(kSplitLanesPerSegment * 2 == kWaveSize, "a wave reads the records of two segments");
 
 struct SplitSegmentInfo
 {
@@ -48,7 +48,6 @@ struct SplitSegmentInfo
 struct SplitShared
 {
     SelectShared<false> select;
-    SplitSegmentInfo segments[kMaxSegments];
     uint32_t histogram[kSplitBins];
     alignas(16) uint32_t bin_keys[kSplitBins * kSplitBinCapacity];   // the candidates of a bin, in the order the histogram's atomics placed them
     alignas(16) uint32_t bin_indices[kSplitBins * kSplitBinCapacity];
@@ -84,9 +83,18 @@ __device__ __forceinline__ unsigned long long load_entry(const unsigned long lon
                      : __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-template <int DTYPE>
+template <int DTYPE, int SEGMENTS = 16>
 __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4) void split_select_kernel(SamplerArgs a)
 {
+    static_assert(SEGMENTS == 16 || SEGMENTS == kSplitMaxSegments, "a wave reads the headers of all segments: 2 x 16 or 2 x 32 lanes");
+    constexpr int kSplitLanesPerSegment = kScanThreads / SEGMENTS; // lanes that read one segment's record: 32 or 16
+    // entries of a record that a lane reads: all 160 of it with 32 lanes a segment; with 16 lanes six each, and a
+    // segment hands over at most 94 candidates (a longer list is cut to its exact window first): ten entries a lane
+    // would take the merge past the registers that eight waves a SIMD leave it
+    constexpr int kSplitSlotsPerLane = SEGMENTS == 16 ? (kSplitRecordSlots + kSplitLanesPerSegment - 1) / kSplitLanesPerSegment : 6;
+    constexpr uint32_t kRecordCap = static_cast<uint32_t>(kSplitLanesPerSegment * kSplitSlotsPerLane - kSplitHeaderEntries);
+    static_assert(kRecordCap + kSplitHeaderEntries <= kSplitRecordSlots && kRecordCap >= static_cast<uint32_t>(kFastTopK) + 16u, "a record holds a window and its ties");
+    constexpr int kSegmentsPerWave = kWaveSize / kSplitLanesPerSegment; // 2 or 4
     using Vector = LogitsVector<DTYPE>;
     constexpr int kWidth = Vector::kWidth;
     constexpr int kVectors = Vector::kVectorsPerLane;
@@ -176,7 +184,7 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     }
     const bool greedy = mode == kModeGreedy;
     const int top_k = static_cast<int>(effective_k);
-    const uint32_t record_entries = segment_record_entries(effective_k);
+    const uint32_t record_entries = min(segment_record_entries(effective_k), kRecordCap);
     if (tid == 0)
     {
         select.block_flags = 0;
@@ -343,7 +351,7 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     const uint32_t own_count = overflow ? 0u : handed;
 
     // ---- hand-over: the entries go out, nothing waits for them
-    unsigned long long* const row_records = a.split_records + static_cast<size_t>(row) * kMaxSegments * kSplitRecordSlots;
+    unsigned long long* const row_records = a.split_records + static_cast<size_t>(row) * kSplitMaxSegments * kSplitRecordSlots;
     unsigned long long* const own_record = row_records + static_cast<size_t>(segment) * kSplitRecordSlots;
     const uint32_t tag = epoch << kSplitIndexBits;
     for (uint32_t j = tid; j < own_count; j += kScanThreads)
@@ -358,7 +366,7 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     // stays in LDS.  (Issuing these loads before the counter's atomic, so that they travel beside it, does
     // not pay: two times out of three an entry of a workgroup that counted itself a moment earlier has
     // not landed yet, and the second trip costs more than the first saved.)
-    const uint32_t read_segment = static_cast<uint32_t>(2 * wave + (lane >> 5));
+    const uint32_t read_segment = static_cast<uint32_t>(kSegmentsPerWave * wave + lane / kSplitLanesPerSegment);
     const int read_lane = lane & (kSplitLanesPerSegment - 1);
     const uint32_t entries_to_read = static_cast<uint32_t>(kSplitHeaderEntries) + record_entries;
     const unsigned long long* const read_record = row_records + static_cast<size_t>(read_segment) * kSplitRecordSlots;
@@ -417,10 +425,11 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     // Every wave reads the headers of all the row's segments for itself (lane s the first entry of segment s,
     // lane 16 + s the second): the row's bound, maximum and flags then come from exchanges inside the wave,
     // without a trip through LDS and a barrier behind the records' arrival.
-    const uint32_t header_segment = static_cast<uint32_t>(lane & (kMaxSegments - 1));
-    const bool header_lane = lane < 2 * kMaxSegments && header_segment < a.segments;
+    const uint32_t header_segment = static_cast<uint32_t>(lane & (SEGMENTS - 1));
+    const bool header_lane = lane < 2 * SEGMENTS && header_segment < a.segments;
     const bool own_header = header_segment == segment;
-    const unsigned long long* const header_address = row_records + static_cast<size_t>(header_segment) * kSplitRecordSlots + ((lane >> 4) & 1);
+    const unsigned long long* const header_address =
+        row_records + static_cast<size_t>(header_segment) * kSplitRecordSlots + (lane >= SEGMENTS ? 1 : 0);
     unsigned long long header = 0ull;
     const auto load_headers = [&](bool around_l2) {
         if (header_lane && !own_header)
@@ -438,24 +447,35 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
         attempts = attempt + 1u;
         uint32_t word = static_cast<uint32_t>(header);
         uint32_t tag_word = static_cast<uint32_t>(header >> 32);
-        if (lane < 2 * kMaxSegments && own_header)
+        if (lane < 2 * SEGMENTS && own_header)
         {
-            word = lane < kMaxSegments ? bound_key : shared.segment_maximum;
-            tag_word = lane < kMaxSegments ? (tag | own_count | (segment_flags << 8)) : tag;
+            word = lane < SEGMENTS ? bound_key : shared.segment_maximum;
+            tag_word = lane < SEGMENTS ? (tag | own_count | (segment_flags << 8)) : tag;
         }
         bool valid = !header_lane || (tag_word >> kSplitIndexBits) == epoch;
-        // rows of 16 lanes: the first holds the segments' bounds, counts and flags, the second their maxima
+        // rows of 16 lanes: the first (two, of 32 segments) hold the segments' bounds, counts and flags, the next their maxima
         const auto larger = [](uint32_t x, uint32_t y) { return max(x, y); };
         const uint32_t extremes = row16_reduce_u32(header_lane ? word : 0u, larger);
-        lower = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(extremes), 0));
-        upper = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(extremes), kMaxSegments));
-        const uint32_t flag_bits = row16_reduce_u32((header_lane && lane < kMaxSegments) ? ((tag_word >> 8) & 7u) : 0u,
+        const uint32_t flag_bits = row16_reduce_u32((header_lane && lane < SEGMENTS) ? ((tag_word >> 8) & 7u) : 0u,
                                                     [](uint32_t x, uint32_t y) { return x | y; });
+        lower = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(extremes), 0));
+        upper = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(extremes), SEGMENTS));
         row_flags = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(flag_bits), 0));
-        const uint32_t count_word = (header_lane && lane < kMaxSegments) ? (tag_word & 0xffu) : 0u;
-        const uint32_t count_low = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(count_word), 2 * wave));
-        const uint32_t count_high = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(count_word), 2 * wave + 1));
-        my_count = lane >= kSplitLanesPerSegment ? count_high : count_low;
+        if (SEGMENTS == 32)
+        {
+            lower = max(lower, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(extremes), 16)));
+            upper = max(upper, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(extremes), 48)));
+            row_flags |= static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(flag_bits), 16));
+        }
+        // the count of the segment whose record this lane reads: lane s of the first rows holds segment s's
+        const uint32_t count_word = (header_lane && lane < SEGMENTS) ? (tag_word & 0xffu) : 0u;
+        my_count = 0;
+#pragma unroll
+        for (int g = 0; g < kSegmentsPerWave; ++g)
+        {
+            const uint32_t count_there = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(count_word), kSegmentsPerWave * wave + g));
+            my_count = lane / kSplitLanesPerSegment == g ? count_there : my_count;
+        }
         if (reads_any)
         {
 #pragma unroll
@@ -520,7 +540,7 @@ __global__ __launch_bounds__(kScanThreads, DTYPE == NCNN_MOE_LOGITS_F32 ? 8 : 4)
     if (epoch == kSplitLastEpoch)
     {
         // the epochs start over: nothing that the old ones tagged may be left (the records are read)
-        for (uint32_t j = tid; j < static_cast<uint32_t>(kMaxSegments * kSplitRecordSlots); j += kScanThreads)
+        for (uint32_t j = tid; j < static_cast<uint32_t>(kSplitMaxSegments * kSplitRecordSlots); j += kScanThreads)
             store_entry(&row_records[j], 0u, 0u);
     }
     NCNN_MOE_LSTAMP(5);

@@ -360,7 +360,7 @@ class HipSampler:
 
 
 STATIC_MAX_ROWS = 1024
-LAST_EPOCH = 16383  # the launch numbers of the split kernel's records run 1 .. LAST_EPOCH and start over
+LAST_EPOCH = 8191  # the launch numbers of the split kernel's records run 1 .. LAST_EPOCH and start over
 SORT_WHOLE_ROW = 0xFFFFFFFF  # sort_lengths(): the row is sorted whole
 
 

@@ -50,18 +50,51 @@ def long_sampler():
     sampler.close()
 
 
-@pytest.mark.parametrize("vocab", [163841, 262144])
-@pytest.mark.parametrize("rows", [8, 64, 130, 200, 255])
-def test_fp32_workgroups_that_stream_several_chunks(long_sampler, rows, vocab):
-    """fp32 rows longer than 16 chunks in batches below 256 rows: several workgroups per row, several
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("vocab", [163841, 201088, 262144])
+@pytest.mark.parametrize("rows", [1, 8, 64, 130, 255])
+def test_rows_of_seventeen_to_thirty_two_one_chunk_workgroups(long_sampler, rows, vocab, dtype):
+    """Rows longer than 16 chunks in batches below 256 rows (fp32 from 163,841 logits on, bf16 from 196,609):
+    the one-chunk kernel in its shape for up to 32 segments, whose merge reads a segment's record with 16 lanes."""
+    code = hip_sampler.LOGITS_F32 if dtype == "f32" else hip_sampler.LOGITS_BF16
+    segments, chunks, variant = hip_sampler.select_geometry(code, rows, vocab)
+    if dtype == "bf16" and vocab <= 196608:
+        assert variant == hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK and segments <= 16
+        pytest.skip("a bf16 row of %d logits is 16 chunks or fewer" % vocab)
+    if dtype == "bf16" and rows * ((vocab + 12287) // 12288) > 2304:
+        # (large batches of long bf16 rows keep the looped kernel, which is as fast there)
+        assert variant == hip_sampler.GEOMETRY_SPLIT_LOOPED and segments > 1 and chunks > 1
+    else:
+        assert variant == hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK and 16 < segments <= 32 and chunks == 1
+    logits, params, uniforms = _batch(rows * 1000 + vocab, rows, vocab)
+    data = workloads.float32_to_bf16_bits(logits) if dtype == "bf16" else logits
+    plain = np.ones(rows, dtype=bool)
+    plain[1::7] = False  # heavy ties may overflow the lists and take the full-order kernels
+    plain[2::11] = False  # ... and so may a row whose first third is -inf (a segment that starts without a bound)
+    for repeat in range(2):  # the same handle again: stale records and counts of the launch before are in place
+        _check(long_sampler, data, params, uniforms, "%d segments, %d x %d %s, launch %d" % (segments, rows, vocab, dtype, repeat),
+               dtype=dtype, scattered=repeat == 1 and rows == 64, must_select=plain)
+
+
+@pytest.fixture(scope="module")
+def longest_sampler():
+    sampler = hip_sampler.HipSampler(130, 340000, testing=True)
+    yield sampler
+    sampler.close()
+
+
+@pytest.mark.parametrize("rows", [8, 64, 130])
+def test_fp32_workgroups_that_stream_several_chunks(longest_sampler, rows):
+    """fp32 rows longer than 32 chunks in batches below 256 rows: several workgroups per row, several
     chunks per workgroup, hand-over through the segments' records."""
+    vocab = 340000
     segments, chunks, variant = hip_sampler.select_geometry(hip_sampler.LOGITS_F32, rows, vocab)
     assert variant == hip_sampler.GEOMETRY_SPLIT_LOOPED and segments > 1 and chunks > 1
     logits, params, uniforms = _batch(rows * 1000 + vocab, rows, vocab)
     plain = np.ones(rows, dtype=bool)
     plain[1::7] = False  # heavy ties may overflow the lists and take the full-order kernels
     plain[2::11] = False  # ... and so may a row whose first third is -inf (a segment that starts without a bound)
-    _check(long_sampler, logits, params, uniforms, "looped split, %d x %d fp32 (%d segments x %d chunks)" % (rows, vocab, segments, chunks),
+    _check(longest_sampler, logits, params, uniforms, "looped split, %d x %d fp32 (%d segments x %d chunks)" % (rows, vocab, segments, chunks),
            must_select=plain)
 
 
@@ -105,7 +138,7 @@ def test_many_launches_on_one_handle():
 
 
 def test_launch_numbers_start_over():
-    """The per-row launch numbers (epochs) that tag the hand-over records run 1 .. 16383 and start over; a
+    """The per-row launch numbers (epochs) that tag the hand-over records run 1 .. 8191 and start over; a
     serving loop gets there within minutes.  A handle that has records of its first launches in place is
     set three launches in front of that point and runs eight launches of changing shape, data and window
     across it: the launch at the last number clears the rows' records, so that what the first launches
