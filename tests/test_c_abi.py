@@ -51,10 +51,17 @@ def test_select_geometry_of_the_benchmark_shapes():
     assert hip_sampler.select_geometry(f32, 1, 32000) == (4, 1, hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK)
     assert hip_sampler.select_geometry(f32, 512, 129280)[2] == hip_sampler.GEOMETRY_WHOLE_ROW
     assert hip_sampler.select_geometry(bf16, 1024, 262144)[2] == hip_sampler.GEOMETRY_WHOLE_ROW
-    for rows in (8, 64, 130, 200, 255):
-        for vocab in (163841, 262144):
-            segments, chunks, variant = hip_sampler.select_geometry(f32, rows, vocab)
-            assert variant == hip_sampler.GEOMETRY_SPLIT_LOOPED and chunks > 1 and segments > 1
+    for rows in (1, 8, 64, 130, 200, 255):
+        # rows of 17 to 32 chunks: one-chunk workgroups (fp32 always, bf16 up to 2,304 of them); longer rows: looped
+        assert hip_sampler.select_geometry(f32, rows, 163841) == (17, 1, hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK)
+        assert hip_sampler.select_geometry(f32, rows, 262144) == (26, 1, hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK)
+        segments, chunks, variant = hip_sampler.select_geometry(bf16, rows, 262144)
+        if rows * 22 <= 2304:
+            assert (segments, chunks, variant) == (22, 1, hip_sampler.GEOMETRY_SPLIT_ONE_CHUNK)
+        else:
+            assert variant == hip_sampler.GEOMETRY_SPLIT_LOOPED and chunks > 1 and 1 < segments <= 16
+        segments, chunks, variant = hip_sampler.select_geometry(f32, rows, 340000)
+        assert variant == hip_sampler.GEOMETRY_SPLIT_LOOPED and chunks > 1 and 1 < segments <= 16
 
 
 def test_router_header_and_binding_agree():
