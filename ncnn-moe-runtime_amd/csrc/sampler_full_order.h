@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(Sampl
 // point of the sorted row nothing moves any sum, and what lies there need not be in order (nor be sorted at
 // all) - only counted.  For a temperature of 1 and logits spread like N(0, 4) that point lies past most of the
 // row; at 0.5 it lies behind the first tenth.
-// One workgroup per row looks at a sample of the row (16,384 logits, evenly spaced groups of four): counts of
+// One workgroup per row looks at a sample of the row (16,384 logits, 256 evenly spaced runs of 64): counts of
 // the keys' upper twelve bits (4,096 buckets: sign, exponent and three bits of the mantissa).  With the terms of
 // the buckets' lower and upper ends it looks for the first bucket whose largest possible term is below 2^-27 of
 // the least the buckets in front of it add up to (the sums' half ulp is 2^-25 to 2^-24 of them), and has the sort
@@ -132,15 +132,16 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
     const float* aligned_logits = logits - misalignment;
     const uint32_t aligned_end = misalignment + a.vocab; // positions [misalignment, aligned_end) hold the row
     const uint32_t groups = (aligned_end + 3u) / 4u;
-    const uint32_t sampled = min(groups, kCutSample);
     uint4 raw[4];
     uint32_t positions[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k)
     {
+        // (runs of sixteen groups, 256 bytes: device memory is fetched by the line, and single groups spread over
+        // the row would fetch all of it)
         const uint32_t g = static_cast<uint32_t>(k * kSortThreads + tid);
-        const uint32_t group = static_cast<uint32_t>(static_cast<uint64_t>(g) * groups / kCutSample);
-        positions[k] = g < sampled || groups >= kCutSample ? group * 4u : aligned_end;
+        const uint32_t run_first = static_cast<uint32_t>(static_cast<uint64_t>(g >> 4) * groups / (kCutSample >> 4));
+        positions[k] = min((run_first + (g & 15u)) * 4u, aligned_end);
         if (groups < kCutSample)
             positions[k] = g < groups ? g * 4u : aligned_end; // a short row is looked at whole
         raw[k] = *reinterpret_cast<const uint4*>(aligned_logits + (positions[k] < aligned_end ? positions[k] : 0u));
