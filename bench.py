@@ -50,15 +50,16 @@ def algorithmic_bytes(rows, vocab, element_bytes):
 
 
 def measured_traffic(workload_name):
-    """HBM bytes per launch of the dominant kernel as measured with rocprofv3 --pmc FETCH_SIZE and
+    """HBM bytes per launch of the dominant kernel (per step of all the step's kernels, for a workload whose step is
+    several) as measured with rocprofv3 --pmc FETCH_SIZE and
     WRITE_SIZE (each scaled by the reading of a 256 MiB copy), recorded beside the profile summaries:
     a stored figure from those counter runs, not something this run measures.  Returns (bytes, file)."""
-    name = "split_select_%s_traffic.json" % workload_name
-    path = os.path.join(ROOT, "profiles", name)
-    if not os.path.exists(path):
-        return None, None
-    with open(path) as handle:
-        return json.load(handle).get("hbm_bytes_per_launch"), "profiles/" + name
+    for name in ("%s_hbm_traffic.json" % workload_name, "split_select_%s_traffic.json" % workload_name):
+        path = os.path.join(ROOT, "profiles", name)
+        if os.path.exists(path):
+            with open(path) as handle:
+                return json.load(handle).get("hbm_bytes_per_launch"), "profiles/" + name
+    return None, None
 
 
 def host_description():
@@ -171,6 +172,11 @@ def bench_speculative_verify(args, hip_sampler):
         sys.exit("bench.py needs a GPU: no HIP device is visible")
     drafts, vocab = args.drafts, 151936
     options = dict(temperature=0.7, top_k=20, top_p=0.8, min_p=0.0)
+    if args.dense_verify:
+        # no Top-K window: the filtered distributions are longer than the verification's lists, and the step takes the
+        # dense path (full-order kernels that export every row's distribution, the accept loop over dense rows)
+        options = dict(temperature=1.0, top_k=0, top_p=0.95, min_p=0.0)
+    options_text = "T %.1f, Top-K %d, Top-P %.2f" % (options["temperature"], options["top_k"], options["top_p"])
     rng = np.random.Generator(np.random.PCG64(77))
     target = (rng.standard_normal((drafts + 1, vocab), dtype=np.float32) * np.float32(3.0))
     draft = target[:drafts] + rng.standard_normal((drafts, vocab), dtype=np.float32) * np.float32(0.5)
@@ -201,16 +207,17 @@ def bench_speculative_verify(args, hip_sampler):
     cpu_seconds = (time.perf_counter() - cpu_start) / cpu_steps
     bytes_per_step = (2 * drafts + 1) * vocab * 4
     line = {
-        "metric": "speculative verification steps/sec, D=%d V=151936 fp32 temp+topk+topp" % drafts,
+        "metric": "speculative verification steps/sec, D=%d V=151936 fp32 %s" % (drafts, "full-vocabulary nucleus (dense path)" if args.dense_verify else "temp+topk+topp"),
         "value": 1.0 / seconds_per_step, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": seconds_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "speculative verification, %d drafted tokens, %d x %d fp32 logits resident in HBM; "
-                               "T 0.7, Top-K 20, Top-P 0.8" % (drafts, 2 * drafts + 1, vocab),
+                               "%s" % (drafts, 2 * drafts + 1, vocab, options_text),
                    "entry_point": "ncnn_moe_hip_sampler_speculative_verify (host operands, synchronous)"},
         "roofline": {"bound": "hbm", "achieved": bytes_per_step / seconds_per_step / 1e9, "peak": HBM_PEAK_BYTES_PER_S / 1e9,
                      "unit": "GB/s", "frac": bytes_per_step / seconds_per_step / HBM_PEAK_BYTES_PER_S, "traffic": None,
-                     "kernel": "scan_select_kernel + speculative_verify_kernel, wall clock of the synchronous call",
+                     "kernel": ("full-order kernels with exported distributions + speculative_verify_dense_kernel" if args.dense_verify
+                                else "scan_select_kernel + speculative_verify_kernel") + ", wall clock of the synchronous call",
                      "algorithmic_bytes_per_launch": bytes_per_step},
         "parity": {"steps_checked": 16, "step_mismatches": mismatches, "mean_accepted": accepted_total / 16.0},
         "cpu_baseline": {"value": 1.0 / cpu_seconds, "unit": "steps/s", "cores": 1, "kind": "port",
@@ -462,7 +469,7 @@ def bench_timeline(args):
     lib.ncnn_moe_hip_sampler_debug_timeline.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
     lib.ncnn_moe_hip_sampler_debug_timeline_rows.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
     names = ["entered", "logits arrived", "bound", "collected", "counted itself"]
-    merge_names = ["counted itself", "records read and checked", "cut and list", "result written"]
+    merge_names = ["counted itself", "records read, checked, candidates placed in their bins", "bins scanned, window ordered", "result written"]
     device = torch.device("cuda:0")
     for rows in sorted({1, args.rows if args.rows > 0 else 64}):
         workload = workloads.make_workload(args.workload, rows=rows)
@@ -514,9 +521,9 @@ def bench_timeline(args):
         d, dm, df = np.diff(seg, axis=-1), np.diff(mer, axis=-1), np.diff(fin, axis=-1)
         print("  phases of a workgroup (medians): wait for the logits %.2f | maxima + bound %.2f | collect %.2f | entries out + counter atomic %.2f" % tuple(
             np.median(d[..., k]) for k in range(4)))
-        print("  phases of the merge (medians): read + check records %.2f | histogram cut + list %.2f | rank + epilogue %.2f" % tuple(
+        print("  phases of the merge (medians): records read, checked, placed %.2f | bins scanned, window ordered %.2f | epilogue %.2f" % tuple(
             np.median(dm[..., k]) for k in range(3)))
-        print("  inside rank + epilogue (medians): rank %.2f | divide + expf %.2f | normaliser %.2f | divide + Min-P + Top-P %.2f | export %.2f | draw %.2f | "
+        print("  inside the epilogue (medians): last ordering %.2f | divide + expf %.2f | normaliser %.2f | divide + Min-P + Top-P %.2f | export %.2f | draw %.2f | "
               "result store %.2f | exit %.2f" % tuple(np.median(df[..., k]) for k in range(8)))
         print("  last result of a launch (median over launches) %.2f us; last logits of a launch %.2f us; re-reads of records per merge: mean %.2f" % (
             np.median(mer[..., 3].max(axis=1)), np.median(seg[..., 1].reshape(len(segment_times), -1).max(axis=1)), np.concatenate(retries).mean()))
@@ -577,9 +584,10 @@ def bench_full_order_timeline(args):
 
     if full_order.size:
         if workload["dtype"] != "f32":
-            table("bf16_counting_sort_kernel, one workgroup per row, after its entry:", after[full_order, 14, :3],
-                  ["entered", "row counted (one pass, 16-bit counters)", "runs written"])
-        table("general_replay_kernel, one workgroup per row, after its entry:", after[full_order, 15, :8],
+            table("bf16_counting_replay_kernel, one workgroup per row: the count, after the kernel's entry:", after[full_order, 14, :3],
+                  ["entered", "row counted (one pass, 16-bit counters)", "runs written (into the counters' LDS)"])
+        table("general_replay_kernel, one workgroup per row, after its entry:" if workload["dtype"] == "f32" else
+              "bf16_counting_replay_kernel: the walk, after the count:", after[full_order, 15, :8],
               ["entered", "exp terms of the row ready", "finite prefix found", "normaliser (exact running sum)", "Min-P cut",
                "Top-P walk (exact running sum)", "draw (exact running sum)", "token index recovered from the logits"])
         rounds = (after - before)[full_order, 15, 12:14].sum(axis=1)
@@ -610,6 +618,8 @@ def main():
                         help="score function of --workload router_dispatch")
     parser.add_argument("--samplers", type=int, default=2, help="samplers (and workers) of --workload scheduler")
     parser.add_argument("--drafts", type=int, default=5, help="drafted tokens per step of --workload speculative_verify")
+    parser.add_argument("--dense-verify", action="store_true",
+                        help="--workload speculative_verify without a Top-K window (T 1.0, Top-P 0.95): the dense path")
     parser.add_argument("--buffers", type=int, default=0, help="distinct logits buffers (0: enough to exceed 320 MB)")
     parser.add_argument("--cpu-rows", type=int, default=64)
     parser.add_argument("--no-cpu-baseline", action="store_true")
