@@ -111,6 +111,8 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
     const int wave = tid >> 6;
     const bool served = a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
     const float temperature = a.params[row].temperature;
+    const uint32_t top_k = a.params[row].top_k;
+    const float window = top_k > 0u && top_k < a.vocab ? static_cast<float>(top_k) : 0.0f;
     const auto sort_whole_row = [&]() {
         if (tid == 0)
         {
@@ -245,8 +247,10 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
         }
         const float highest = value_from_descending_key(bucket << 20);
         const float largest_term = __expf(fminf((highest - maximum) / temperature, 0.0f));
+        // (a Top-K window ends the row's sums at K elements: a few times K, by the sample's count, are kept)
+        const bool behind_the_window = window != 0.0f && count_here >= 2.0f * window + kCutMinimum;
         if (bucket > kFirstFiniteBucket && bucket <= kLastFiniteBucket && count_here >= kCutMinimum &&
-            largest_term < mass_here * 7.450580596923828e-09f) // 2^-27
+            (largest_term < mass_here * 7.450580596923828e-09f || behind_the_window)) // 2^-27
             candidate = bucket;
     }
     if (candidate < static_cast<uint32_t>(kCutBuckets))
