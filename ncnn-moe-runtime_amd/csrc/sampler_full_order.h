@@ -90,7 +90,8 @@ __global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(Sampl
 // One workgroup per row looks at a sample of the row (16,384 logits, 256 evenly spaced runs of 64): counts of
 // the keys' upper twelve bits (4,096 buckets: sign, exponent and three bits of the mantissa).  With the terms of
 // the buckets' lower and upper ends it looks for the first bucket whose largest possible term is below 2^-27 of
-// the least the buckets in front of it add up to (the sums' half ulp is 2^-25 to 2^-24 of them), and has the sort
+// the least the buckets in front of it add up to (the sums' half ulp is 2^-25 to 2^-24 of them) - or, under a Top-K
+// window, the first bucket behind twice the window by the sample's count - and has the sort
 // keep the buckets in front of it: sort_last_keys.  This is a guess that costs or saves time, never exactness:
 // the replay checks against its exact sums that the largest term left out moves none of them, and otherwise has
 // the row sorted whole.  The exact counts that go with a cut (elements kept, finite logits, NaN seen) are taken
