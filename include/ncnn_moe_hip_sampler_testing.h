@@ -40,6 +40,13 @@ int ncnn_moe_hip_sampler_debug_fused_bf16(ncnn_moe_hip_sampler* sampler, int ena
  * were sorted (0xffffffff: the whole row; only rows that took the spread sort with partial_sort on are written). */
 int ncnn_moe_hip_sampler_debug_partial_sort(ncnn_moe_hip_sampler* sampler, int enabled);
 int ncnn_moe_hip_sampler_debug_sort_lengths(ncnn_moe_hip_sampler* sampler, uint32_t* lengths, uint32_t rows);
+/* skip_low_digit (on by default, with partial_sort): that sort takes three passes, over the keys' upper 24 bits, and
+ * the kernel that computes the terms puts the neighbours that agree in those bits in order; a row in which it cannot
+ * (more such keys in a row than it looks at, and out of order) is sorted whole by the second launch.  Off: four passes.
+ * Same results either way.  disordered_rows copies out, for the first `rows` rows of the last call, 1 for a row that
+ * was handed to the second launch for this reason (written for the rows that partial_sort serves). */
+int ncnn_moe_hip_sampler_debug_skip_low_digit(ncnn_moe_hip_sampler* sampler, int enabled);
+int ncnn_moe_hip_sampler_debug_disordered_rows(ncnn_moe_hip_sampler* sampler, uint32_t* flags, uint32_t rows);
 /* Sets the per-row launch numbers (epochs, 1 .. 8191) that tag the split kernel's hand-over records: of the
  * handle, or with a null handle of the static scratch of `device` (after it has served a call).  Tests start a
  * few launches in front of the point where the epochs start over. */

@@ -67,8 +67,9 @@ struct ncnn_moe_hip_sampler
     uint32_t* sort_indices[2] = {nullptr, nullptr};
     uint64_t sort_stride = 0;
     uint32_t* row_list = nullptr;         // [1 + rows], see SamplerArgs::row_list
-    uint32_t* sort_cuts = nullptr;        // [3][rows]: SamplerArgs::sort_lengths, sort_last_keys, finite_counts
+    uint32_t* sort_cuts = nullptr;        // [4][rows]: SamplerArgs::sort_lengths, sort_last_keys, finite_counts, disordered_rows
     int partial_sort = 1;                 // full-order fp32 rows are sorted only as far as their terms can move a sum
+    int skip_low_digit = 1;               // ... by three passes over the keys' upper 24 bits, the lowest byte put in order by the terms kernel
     uint32_t* sort_part_counts = nullptr; // [rows][kMaxSortParts][256]
     double* term_sums = nullptr;          // [rows][term_sum_parts]: fp64 sums of the terms kernel's blocks
     uint4* chunk_steps = nullptr;         // [rows][chunk_capacity]: composed step of every whole chunk of a sorted row's terms
@@ -354,7 +355,7 @@ int launch_sampler(
         constexpr bool kPairs = decltype(pairs_tag)::value;
         spread.sort_parts = sort_parts;
         spread.sort_tiles_per_part = sort_tiles_per_part;
-        const int passes = kType == NCNN_MOE_LOGITS_F32 ? 4 : 2;
+        const int passes = kType == NCNN_MOE_LOGITS_F32 ? 4 - static_cast<int>(spread.sort_low_digit_skipped) : 2;
         for (int pass = 0; pass < passes; ++pass)
         {
             spread.sort_pass = static_cast<uint32_t>(pass);
@@ -377,10 +378,13 @@ int launch_sampler(
         a.sort_lengths = s->sort_cuts;
         a.sort_last_keys = s->sort_cuts + s->max_rows;
         a.finite_counts = s->sort_cuts + 2 * static_cast<size_t>(s->max_rows);
+        a.disordered_rows = s->sort_cuts + 3 * static_cast<size_t>(s->max_rows);
     }
     const auto launch_full_order = [&](SamplerArgs a, bool leftovers) {
         const bool spread_sort = sort_tiles >= 4 && s->spread_sort != 0 && !leftovers;
         const bool runs = dtype == NCNN_MOE_LOGITS_BF16 && !want_distribution;
+        // (keys alone, sorted in part or whole by the spread sort: its pass over the lowest byte is left out)
+        a.sort_low_digit_skipped = !leftovers && partial_sort && s->skip_low_digit != 0 ? 1u : 0u;
         if (!leftovers && !runs)
         {
             // (the kernels over a (parts, rows) grid find their rows in a list)
@@ -632,7 +636,7 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
         CREATE_CHECK(hipMalloc(&s->sort_indices[i], rows * s->sort_stride * sizeof(uint32_t)));
     }
     CREATE_CHECK(hipMalloc(&s->row_list, (static_cast<size_t>(rows) + 1) * sizeof(uint32_t)));
-    CREATE_CHECK(hipMalloc(&s->sort_cuts, 3 * static_cast<size_t>(rows) * sizeof(uint32_t)));
+    CREATE_CHECK(hipMalloc(&s->sort_cuts, 4 * static_cast<size_t>(rows) * sizeof(uint32_t)));
     CREATE_CHECK(hipMalloc(&s->sort_part_counts, rows * kMaxSortParts * 256 * sizeof(uint32_t)));
     s->term_sum_parts = (max_vocab + kTermsThreads * kTermsPerThread - 1) / (kTermsThreads * kTermsPerThread);
     s->chunk_capacity = max_vocab / kReplayChunk + 1;
@@ -1167,6 +1171,26 @@ int ncnn_moe_hip_sampler_debug_partial_sort(ncnn_moe_hip_sampler* s, int enabled
     if (s == nullptr)
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     s->partial_sort = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+// The spread sort of full-order fp32 rows in three passes and a touch-up of the lowest byte (the default), or in four.
+int ncnn_moe_hip_sampler_debug_skip_low_digit(ncnn_moe_hip_sampler* s, int enabled)
+{
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    s->skip_low_digit = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+// Which rows of the last call the touch-up of the lowest byte could not put in order (1; they were sorted whole).
+int ncnn_moe_hip_sampler_debug_disordered_rows(ncnn_moe_hip_sampler* s, uint32_t* flags, uint32_t rows)
+{
+    if (s == nullptr || flags == nullptr || rows > s->max_rows)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
+    SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
+    SAMPLER_HIP_CHECK(s, hipMemcpy(flags, s->sort_cuts + 3 * static_cast<size_t>(s->max_rows), rows * sizeof(uint32_t), hipMemcpyDeviceToHost));
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

@@ -80,7 +80,21 @@ struct SamplerArgs
     uint32_t* sort_lengths;
     uint32_t* sort_last_keys;
     uint32_t* finite_counts;
+    // The spread sort of such rows may leave out the keys' lowest byte (sort_low_digit_skipped = 1: three passes,
+    // over bits 8 to 31, which end in sort_keys[0]).  full_order_terms_kernel then puts the few neighbours that
+    // agree in their upper 24 bits in order on its way through the keys (into sort_keys[1]; the terms go to
+    // sort_indices[0]), and notes in disordered_rows [rows] a row in which it cannot (such keys too many in a
+    // row to see them all, and out of order): that row is sorted whole by the launch behind this one.
+    uint32_t* disordered_rows;
+    uint32_t sort_low_digit_skipped;
 };
+
+// Where the terms of the sorted rows' elements are kept (see sort_low_digit_skipped).
+__device__ __forceinline__ float* sorted_terms(const SamplerArgs& a, uint32_t row)
+{
+    uint32_t* const base = a.sort_low_digit_skipped != 0u ? a.sort_indices[0] : a.sort_keys[0];
+    return reinterpret_cast<float*>(base + row * a.sort_stride);
+}
 
 // Elements of the row that the full-order sort orders (the row's first ones in sorted order).
 __device__ __forceinline__ uint32_t sorted_length(const SamplerArgs& a, uint32_t row)

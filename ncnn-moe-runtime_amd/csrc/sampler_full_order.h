@@ -119,6 +119,7 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
         {
             a.sort_last_keys[row] = 0xffffffffu;
             a.sort_lengths[row] = a.vocab;
+            a.disordered_rows[row] = 0u;
         }
     };
     if (!served || !(temperature > 0.0f))
@@ -265,6 +266,7 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
         a.sort_last_keys[row] = (cut << 20) - 1u;
         a.sort_lengths[row] = 0u;   // counted by sort_part_histogram_kernel's first pass
         a.finite_counts[row] = 0u;  // ... with the row's finite logits and whether it holds a NaN
+        a.disordered_rows[row] = 0u;
     }
 }
 
@@ -590,7 +592,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(Sampl
     // the first pass reads the whole row and keeps the elements that are sorted; the others read those
     const uint32_t n = pass == 0 ? a.vocab : sorted_length(a, row);
     const uint32_t last_key = sort_last_key(a, row, pass);
-    const int shift = 8 * (pass + kFirstDigit);
+    const int shift = 8 * (pass + kFirstDigit + static_cast<int>(a.sort_low_digit_skipped));
     __shared__ uint32_t counts[kHistogramParts][8][257]; // (257: the copies of a digit's counter lie in eight different banks)
     for (int i = tid; i < kHistogramParts * 8 * 257; i += kSortThreads)
         (&counts[0][0][0])[i] = 0;
@@ -701,7 +703,7 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
     // the first pass reads the whole row and keeps the elements that are sorted; the others read those
     const uint32_t n = pass == 0 ? a.vocab : sorted_length(a, row);
     const uint32_t last_key = sort_last_key(a, row, pass);
-    const int shift = 8 * (pass + kFirstDigit);
+    const int shift = 8 * (pass + kFirstDigit + static_cast<int>(a.sort_low_digit_skipped));
 
     __shared__ uint32_t digit_base[256];          // output position of the next key of each digit
     __shared__ uint32_t wave_counts[kSortWaves][256];
@@ -1584,7 +1586,17 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     }
     else
     {
-        float* terms = reinterpret_cast<float*>(a.sort_keys[0] + row * a.sort_stride);
+        // (a row whose keys the terms kernel could not put in order: the launch behind this one sorts it whole)
+        if (a.sort_low_digit_skipped != 0u && a.disordered_rows[row] != 0u)
+        {
+            if (tid == 0)
+            {
+                a.sort_last_keys[row] = 0xffffffffu;
+                a.sort_lengths[row] = a.vocab;
+            }
+            return;
+        }
+        float* terms = sorted_terms(a, row);
         if (a.terms_precomputed == 0 && p.temperature != 0.0f)
         {
             const float maximum = value_from_descending_key(keys[0]) / p.temperature;
@@ -1716,8 +1728,94 @@ __global__ __launch_bounds__(kSortThreads) void bf16_counting_replay_kernel(Samp
 // buffer: the replay that follows adds these terms one workgroup per row, and computing them there would
 // put a few dozen instructions per element on that workgroup's path; here the whole GPU shares them.
 // grid (parts, rows).
+//
+// After a sort that left out the keys' lowest byte (SamplerArgs::sort_low_digit_skipped) the keys arrive ordered
+// by their upper 24 bits, and the keys that agree in those - neighbours, one to three of them where a row's
+// logits are spread over the floats, because 256 consecutive floats rarely hold two - are put in order here: an
+// element looks at up to kTouchUpReach neighbours on either side as far as they share its upper 24 bits, counts
+// those in front of it that belong behind it and those behind it that belong in front, and moves by the
+// difference (equal keys keep their places).  That is the element's place in the sorted row whenever it has seen
+// all of its group.  A group that reaches further is harmless if it is in order already (a run of equal keys: a
+// row of rounded logits, a padded vocabulary), and whether it is shows between neighbours: a group longer than
+// the reach that holds two adjacent keys out of order has an element that sees them without seeing the group's
+// end (the group's first or last element if they lie within reach of it, else the first of the two), and that
+// element marks the row in disordered_rows: the replay leaves such a row to the launch that sorts it whole.
 constexpr int kTermsThreads = 256;
 constexpr int kTermsPerThread = 8;
+constexpr int kTermsTile = kTermsThreads * kTermsPerThread;
+constexpr int kTouchUpReach = 16;
+constexpr int kTouchUpNear = 4; // neighbours on either side that every element looks at, without a branch
+
+// The place in the sorted row of the element at position i, whose key is `key` and lies at mine[0] among its
+// neighbours' keys (positions outside the row hold keys that share their upper 24 bits with no element next to
+// them).  A group of up to kTouchUpNear + 1 keys is seen whole within kTouchUpNear steps, by straight-line code: an
+// instruction costs this kernel as much as a byte (its time is the instructions its waves issue), and a loop
+// that ends where the group does is some fifty of them a step.  `lost`: see full_order_terms_kernel.
+__device__ __forceinline__ uint32_t touched_up_place(const uint32_t* mine, uint32_t key, uint32_t i, bool& further)
+{
+    uint32_t belong_behind = 0, belong_in_front = 0;
+    bool same = true;
+#pragma unroll
+    for (int d = 1; d <= kTouchUpNear; ++d)
+    {
+        const uint32_t other = mine[-d];
+        same = same & ((other ^ key) < 256u);
+        belong_behind += same & (other > key) ? 1u : 0u;
+    }
+    further = same;
+    same = true;
+#pragma unroll
+    for (int d = 1; d <= kTouchUpNear; ++d)
+    {
+        const uint32_t other = mine[d];
+        same = same & ((other ^ key) < 256u);
+        belong_in_front += same & (other < key) ? 1u : 0u;
+    }
+    further = further | same;
+    return i - belong_behind + belong_in_front;
+}
+
+// The same for an element of a longer group (rare among spread logits; every element of a row of rounded ones),
+// one step at a time up to kTouchUpReach on either side.
+__device__ __forceinline__ uint32_t touched_up_place_of_long_group(const uint32_t* mine, uint32_t i, uint32_t& lost)
+{
+    const uint32_t key = mine[0];
+    uint32_t belong_behind = 0, belong_in_front = 0;
+    uint32_t previous = key;
+    bool out_of_order = false, end_seen = false;
+#pragma nounroll
+    for (int d = 1; d <= kTouchUpReach; ++d)
+    {
+        const uint32_t other = mine[-d];
+        if ((other ^ key) >= 256u)
+        {
+            end_seen = true;
+            break;
+        }
+        belong_behind += other > key ? 1u : 0u;
+        out_of_order |= other > previous;
+        previous = other;
+    }
+    bool all_seen = end_seen;
+    end_seen = false;
+    previous = key;
+#pragma nounroll
+    for (int d = 1; d <= kTouchUpReach; ++d)
+    {
+        const uint32_t other = mine[d];
+        if ((other ^ key) >= 256u)
+        {
+            end_seen = true;
+            break;
+        }
+        belong_in_front += other < key ? 1u : 0u;
+        out_of_order |= previous > other;
+        previous = other;
+    }
+    all_seen = all_seen && end_seen;
+    lost |= !all_seen && out_of_order ? 1u : 0u;
+    return i - belong_behind + belong_in_front;
+}
 
 __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(SamplerArgs a)
 {
@@ -1725,24 +1823,91 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
     if (!spread_grid_row(a, row))
         return;
     __shared__ uint64_t exp2_table[32]; // a copy in LDS: the lookups of a wave are 64 different addresses
+    __shared__ uint32_t tile_keys[kTermsTile + 2 * kTouchUpReach];
     if (threadIdx.x < 32)
         exp2_table[threadIdx.x] = kExp2Table[threadIdx.x];
     const uint32_t n = sorted_length(a, row);
-    if (blockIdx.x * (kTermsThreads * kTermsPerThread) >= n)
+    const uint32_t tile_first = blockIdx.x * kTermsTile;
+    if (tile_first >= n)
         return; // (behind the row's sorted elements: no chunk reads this block's sum)
+    const bool touch_up = a.sort_low_digit_skipped != 0u;
     const float temperature = a.params[row].temperature;
-    const uint32_t* keys = a.sort_keys[1] + row * a.sort_stride;
-    float* terms = reinterpret_cast<float*>(a.sort_keys[0] + row * a.sort_stride);
-    const float maximum = value_from_descending_key(keys[0]) / temperature;
-    const uint32_t first = blockIdx.x * (kTermsThreads * kTermsPerThread) + threadIdx.x;
+    const uint32_t* keys = a.sort_keys[touch_up ? 0 : 1] + row * a.sort_stride;
+    uint32_t* const ordered_keys = a.sort_keys[1] + row * a.sort_stride;
+    float* terms = sorted_terms(a, row);
+    const uint32_t first = tile_first + threadIdx.x;
+    // (in place of the keys behind the row's end: one that shares its upper 24 bits with no key next to it)
+    const uint32_t behind_the_row = touch_up ? ~keys[n - 1u] : 0u;
     uint32_t loaded[kTermsPerThread];
 #pragma unroll
     for (int j = 0; j < kTermsPerThread; ++j)
     {
         const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
-        loaded[j] = i < n ? keys[i] : 0u;
+        loaded[j] = i < n ? keys[i] : behind_the_row;
     }
-    __syncthreads();
+    uint32_t smallest_key;
+    uint32_t places[kTermsPerThread];
+    if (!touch_up)
+    {
+        smallest_key = keys[0];
+#pragma unroll
+        for (int j = 0; j < kTermsPerThread; ++j)
+            places[j] = first + static_cast<uint32_t>(j * kTermsThreads);
+        __syncthreads();
+    }
+    else
+    {
+        // the row's smallest key is in the first group: the first of the row if that group is in order, and
+        // within reach of the row's first element if it is not (or the row is marked)
+        const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+        const uint32_t front = lane <= static_cast<uint32_t>(kTouchUpReach) && lane < n ? keys[lane] : 0xffffffffu;
+        smallest_key = ~wave_max_u32(~front);
+        // the tile's keys, with kTouchUpReach of the tiles on either side, at tile_keys[position - tile_first + reach]
+#pragma unroll
+        for (int j = 0; j < kTermsPerThread; ++j)
+            tile_keys[kTouchUpReach + j * kTermsThreads + static_cast<int>(threadIdx.x)] = loaded[j];
+        if (threadIdx.x < 2 * kTouchUpReach)
+        {
+            const bool left = threadIdx.x < static_cast<uint32_t>(kTouchUpReach);
+            const int64_t position = left ? static_cast<int64_t>(tile_first) - kTouchUpReach + threadIdx.x
+                                          : static_cast<int64_t>(tile_first) + kTermsTile + (threadIdx.x - kTouchUpReach);
+            const uint32_t slot = left ? threadIdx.x : static_cast<uint32_t>(kTermsTile) + threadIdx.x;
+            uint32_t key = behind_the_row;
+            if (position < 0)
+                key = ~keys[0];
+            else if (position < static_cast<int64_t>(n))
+                key = keys[position];
+            tile_keys[slot] = key;
+        }
+        __syncthreads();
+        uint32_t long_groups = 0;
+#pragma unroll
+        for (int j = 0; j < kTermsPerThread; ++j)
+        {
+            const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
+            bool further = false;
+            places[j] = touched_up_place(tile_keys + kTouchUpReach + j * kTermsThreads + static_cast<int>(threadIdx.x), loaded[j], i, further);
+            long_groups |= further && i < n ? 1u << j : 0u;
+        }
+        if (long_groups != 0u)
+        {
+            uint32_t lost = 0;
+#pragma nounroll
+            for (int j = 0; j < kTermsPerThread; ++j)
+            {
+                if ((long_groups >> j & 1u) == 0u)
+                    continue;
+                const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
+                const uint32_t place = touched_up_place_of_long_group(tile_keys + kTouchUpReach + j * kTermsThreads + static_cast<int>(threadIdx.x), i, lost);
+#pragma unroll
+                for (int at = 0; at < kTermsPerThread; ++at)
+                    places[at] = at == j ? place : places[at];
+            }
+            if (lost != 0u)
+                atomicOr(&a.disordered_rows[row], 1u);
+        }
+    }
+    const float maximum = value_from_descending_key(smallest_key) / temperature;
     double sum = 0.0;
 #pragma unroll
     for (int j = 0; j < kTermsPerThread; ++j)
@@ -1751,7 +1916,9 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
         if (i < n)
         {
             const float term = expf_libm(value_from_descending_key(loaded[j]) / temperature - maximum, exp2_table);
-            terms[i] = term;
+            terms[places[j]] = term;
+            if (touch_up)
+                ordered_keys[places[j]] = loaded[j];
             sum += static_cast<double>(term);
         }
     }
@@ -1798,7 +1965,7 @@ __global__ __launch_bounds__(kChunkStepThreads) void full_order_chunk_steps_kern
     constexpr int kWaves = kChunkStepThreads / kWaveSize;
     __shared__ double wave_sums[kWaves];
     __shared__ ParityStep wave_totals[kWaves];
-    const float* terms = reinterpret_cast<const float*>(a.sort_keys[0] + row * a.sort_stride);
+    const float* terms = sorted_terms(a, row);
     uint4* const out = a.chunk_steps + static_cast<size_t>(row) * a.chunk_capacity + chunk;
     const uint32_t base = chunk * kReplayChunk;
     const uint32_t n = sorted_length(a, row);

@@ -75,6 +75,8 @@ TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_fused_bf16",
     "ncnn_moe_hip_sampler_debug_partial_sort",
     "ncnn_moe_hip_sampler_debug_sort_lengths",
+    "ncnn_moe_hip_sampler_debug_skip_low_digit",
+    "ncnn_moe_hip_sampler_debug_disordered_rows",
     "ncnn_moe_hip_sampler_debug_chunk_steps",
     "ncnn_moe_hip_sampler_debug_stream_only",
     "ncnn_moe_hip_sampler_debug_set_row_epochs",
@@ -122,6 +124,8 @@ def _bind(lib, testing):
     lib.ncnn_moe_hip_sampler_debug_spread_sort.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_partial_sort.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_sort_lengths.argtypes = [vp, vp, ctypes.c_uint32]
+    lib.ncnn_moe_hip_sampler_debug_skip_low_digit.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_disordered_rows.argtypes = [vp, vp, ctypes.c_uint32]
     lib.ncnn_moe_hip_sampler_debug_fused_bf16.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_chunk_steps.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_stream_only.argtypes = [vp, vp, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vp]
@@ -342,6 +346,18 @@ class HipSampler:
         """Test hook: elements sorted of each of the last call's first `rows` rows (SORT_WHOLE_ROW: all of them)."""
         out = np.empty(rows, dtype=np.uint32)
         self._check(self._hooks(True).ncnn_moe_hip_sampler_debug_sort_lengths(self._handle, out.ctypes.data, rows))
+        return out
+
+    def skip_low_digit(self, enabled):
+        """Test hook: the spread sort of full-order fp32 rows in three passes over the keys' upper 24 bits, the lowest
+        byte put in order on the way to the terms (default), or in four passes."""
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_skip_low_digit(self._handle, 1 if enabled else 0))
+
+    def disordered_rows(self, rows):
+        """Test hook: which of the last call's first `rows` rows the three-pass sort could not finish (1: the row was
+        sorted whole by the launch behind it)."""
+        out = np.empty(rows, dtype=np.uint32)
+        self._check(self._hooks(True).ncnn_moe_hip_sampler_debug_disordered_rows(self._handle, out.ctypes.data, rows))
         return out
 
     def fused_bf16(self, enabled):

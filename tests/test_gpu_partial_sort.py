@@ -124,3 +124,68 @@ def test_heavy_ties_and_narrow_rows(sampler):
     for trial in range(2):
         uniforms = rng.random(ROWS, dtype=np.float32)
         _sample_both_ways(sampler, logits, params, uniforms, "partial sort, ties and narrow rows, draw %d" % trial)
+
+
+def _sample_with_three_passes_and_four(sampler, logits, params, uniforms, context):
+    """The oracle's results from the sort in three passes (with the lowest byte put in order on the way to the
+    terms) and from the sort in four; returns the former's results and which rows it handed to the second launch."""
+    _announce(context)
+    sampler.upload_logits(logits)
+    three = sampler.sample(params, uniforms, None)
+    disordered = sampler.disordered_rows(ROWS)
+    sampler.skip_low_digit(False)
+    try:
+        four = sampler.sample(params, uniforms, None)
+    finally:
+        sampler.skip_low_digit(True)
+    cpu = parity_util.run_oracle(logits, params, uniforms)
+    parity_util.assert_results_match(three, cpu, "f32", context)
+    assert three.tobytes() == four.tobytes(), context
+    return three, disordered
+
+
+def test_three_passes_leave_the_lowest_byte_to_the_terms_kernel(sampler):
+    """Logits spread over the floats: keys that agree in their upper 24 bits are one to three neighbours, which the
+    terms kernel orders; no row goes to the second launch for it.  Cold rows (sorted in part) and warm ones (whole)."""
+    rng, logits, params = _rows(4500)
+    params["top_p"] = rng.uniform(0.5, 1.0, size=ROWS).astype(np.float32)
+    logits[5] = (4.0 + rng.random(VOCAB) * 4.0).astype(np.float32)  # every 256 floats of [4, 8) hold two of these
+    logits[6] = (2.0 + rng.random(VOCAB)).astype(np.float32)        # ... and of [2, 3) four
+    params["temperature"][5:7] = np.float32(1.0)
+    for trial in range(2):
+        uniforms = rng.random(ROWS, dtype=np.float32)
+        gpu, disordered = _sample_with_three_passes_and_four(sampler, logits, params, uniforms, "three passes, draw %d" % trial)
+        assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+        assert not disordered.any(), np.nonzero(disordered)[0]
+
+
+def _grouped_row(rng, group, vocab=VOCAB):
+    """A row of positive logits in groups of `group` keys that share their upper 24 bits and differ in the lowest byte
+    (drawn without replacement where 256 values allow it), in random places of the row."""
+    groups = (vocab + group - 1) // group
+    cells = rng.choice(np.arange(0x3F8000, 0x410000, dtype=np.uint32), size=groups, replace=False)  # floats in [1, 8)
+    low = np.concatenate([rng.permutation(256)[:group] if group <= 256 else rng.integers(0, 256, size=group) for _ in range(groups)])
+    bits = (np.repeat(cells, group).astype(np.uint32) << np.uint32(8)) | low.astype(np.uint32)
+    return rng.permutation(bits[:vocab]).view(np.float32)
+
+
+def test_groups_of_keys_that_differ_in_the_lowest_byte_only(sampler):
+    """Groups of up to 16 such keys are within the terms kernel's reach and come out in order; longer ones that are
+    not in order send the row to the second launch; long runs of equal keys (and a row of few distinct values)
+    are in order as they are."""
+    rng, logits, params = _rows(4600)
+    params["temperature"] = np.float32(1.0)
+    params["top_p"] = rng.uniform(0.3, 1.0, size=ROWS).astype(np.float32)
+    sizes = {0: 2, 1: 3, 2: 7, 3: 15, 4: 16, 5: 17, 6: 18, 7: 31, 8: 33, 9: 64, 10: 300, 11: 5000}
+    for row, group in sizes.items():
+        logits[row] = _grouped_row(rng, group)
+    logits[12] = np.round(logits[12] * 2) / 2                     # a few dozen values, thousands of times each
+    logits[13, 1000:40000] = np.float32(1.25)                     # a padded stretch of equal logits among spread ones
+    logits[14] = _grouped_row(rng, 40)
+    logits[14] = -np.sort(-logits[14])                            # long groups, in order already (descending logits)
+    for trial in range(2):
+        uniforms = rng.random(ROWS, dtype=np.float32)
+        _, disordered = _sample_with_three_passes_and_four(sampler, logits, params, uniforms, "groups in the lowest byte, draw %d" % trial)
+        expected = np.zeros(ROWS, dtype=bool)
+        expected[[row for row, group in sizes.items() if group > 16]] = True
+        assert (disordered.astype(bool) == expected).all(), (np.nonzero(disordered)[0], np.nonzero(expected)[0])
