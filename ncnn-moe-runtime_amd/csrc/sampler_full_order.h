@@ -1744,35 +1744,28 @@ constexpr int kTermsThreads = 256;
 constexpr int kTermsPerThread = 8;
 constexpr int kTermsTile = kTermsThreads * kTermsPerThread;
 constexpr int kTouchUpReach = 16;
-constexpr int kTouchUpNear = 4; // neighbours on either side that every element looks at, without a branch
+constexpr int kTouchUpNear = 6; // neighbours on either side that every element looks at, without a branch
 
 // The place in the sorted row of the element at position i, whose key is `key` and lies at mine[0] among its
-// neighbours' keys (positions outside the row hold keys that share their upper 24 bits with no element next to
-// them).  A group of up to kTouchUpNear + 1 keys is seen whole within kTouchUpNear steps, by straight-line code: an
-// instruction costs this kernel as much as a byte (its time is the instructions its waves issue), and a loop
-// that ends where the group does is some fifty of them a step.  `lost`: see full_order_terms_kernel.
+// neighbours' keys (positions in front of the row hold 0, positions behind it 0xffffffff: neither is ever counted,
+// and neither is out of order where it stands).  A group of up to kTouchUpNear keys is seen whole within
+// kTouchUpNear steps, by straight-line code: an instruction costs this kernel as much as a byte (its time is the
+// instructions its waves issue), and a loop that ends where the group does is some fifty of them a step.  A key
+// in front belongs behind this one if it lies in (key, key | 255], one behind belongs in front if it lies in
+// [key & ~255, key): a subtraction and a compare each.  `further`: the group may reach beyond what was looked at.
 __device__ __forceinline__ uint32_t touched_up_place(const uint32_t* mine, uint32_t key, uint32_t i, bool& further)
 {
-    uint32_t belong_behind = 0, belong_in_front = 0;
-    bool same = true;
+    const uint32_t low = key & 255u;
+    const uint32_t room_above = 255u - low;
+    uint32_t place = i;
 #pragma unroll
     for (int d = 1; d <= kTouchUpNear; ++d)
     {
-        const uint32_t other = mine[-d];
-        same = same & ((other ^ key) < 256u);
-        belong_behind += same & (other > key) ? 1u : 0u;
+        place -= mine[-d] - key - 1u < room_above ? 1u : 0u;
+        place += key - mine[d] - 1u < low ? 1u : 0u;
     }
-    further = same;
-    same = true;
-#pragma unroll
-    for (int d = 1; d <= kTouchUpNear; ++d)
-    {
-        const uint32_t other = mine[d];
-        same = same & ((other ^ key) < 256u);
-        belong_in_front += same & (other < key) ? 1u : 0u;
-    }
-    further = further | same;
-    return i - belong_behind + belong_in_front;
+    further = ((mine[-kTouchUpNear] ^ key) < 256u) | ((mine[kTouchUpNear] ^ key) < 256u);
+    return place;
 }
 
 // The same for an element of a longer group (rare among spread logits; every element of a row of rounded ones),
@@ -1836,8 +1829,7 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
     uint32_t* const ordered_keys = a.sort_keys[1] + row * a.sort_stride;
     float* terms = sorted_terms(a, row);
     const uint32_t first = tile_first + threadIdx.x;
-    // (in place of the keys behind the row's end: one that shares its upper 24 bits with no key next to it)
-    const uint32_t behind_the_row = touch_up ? ~keys[n - 1u] : 0u;
+    const uint32_t behind_the_row = 0xffffffffu; // (in place of the keys behind the row's end; see touched_up_place)
     uint32_t loaded[kTermsPerThread];
 #pragma unroll
     for (int j = 0; j < kTermsPerThread; ++j)
@@ -1872,10 +1864,8 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
             const int64_t position = left ? static_cast<int64_t>(tile_first) - kTouchUpReach + threadIdx.x
                                           : static_cast<int64_t>(tile_first) + kTermsTile + (threadIdx.x - kTouchUpReach);
             const uint32_t slot = left ? threadIdx.x : static_cast<uint32_t>(kTermsTile) + threadIdx.x;
-            uint32_t key = behind_the_row;
-            if (position < 0)
-                key = ~keys[0];
-            else if (position < static_cast<int64_t>(n))
+            uint32_t key = position < 0 ? 0u : behind_the_row;
+            if (position >= 0 && position < static_cast<int64_t>(n))
                 key = keys[position];
             tile_keys[slot] = key;
         }
