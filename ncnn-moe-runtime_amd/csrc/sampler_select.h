@@ -429,7 +429,7 @@ __device__ __forceinline__ void load_chunk(
 // LOOPED: a workgroup streams several chunks (double-buffered).  WIDE: Top-K windows up to kSelectTopK
 // (a long candidate list, more registers and LDS); otherwise up to kFastTopK.
 template <int DTYPE, bool LOOPED, bool WIDE>
-__global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_F32) ? 8 : (WIDE ? 1 : 4)) void scan_select_kernel(SamplerArgs a)
+__global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_F32) ? 8 : 4) void scan_select_kernel(SamplerArgs a)
 {
     using Vector = LogitsVector<DTYPE>;
     static_assert(LOOPED || !WIDE, "wide windows are served by whole-row workgroups");

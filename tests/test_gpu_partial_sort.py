@@ -189,3 +189,24 @@ def test_groups_of_keys_that_differ_in_the_lowest_byte_only(sampler):
         expected = np.zeros(ROWS, dtype=bool)
         expected[[row for row, group in sizes.items() if group > 16]] = True
         assert (disordered.astype(bool) == expected).all(), (np.nonzero(disordered)[0], np.nonzero(expected)[0])
+
+
+def test_parts_of_several_tiles():
+    """Rows longer than sixteen tiles: a part of the spread sort holds several tiles (three here), and the row's
+    cut, its three passes and the touch-up of the lowest byte work across them."""
+    rows, vocab = 6, 300007
+    rng = np.random.default_rng(4800)
+    logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+    params["temperature"] = np.array([0.3, 0.6, 0.9, 1.1, 1.3, 1.5], dtype=np.float32)
+    params["top_p"] = np.array([0.9, 0.95, 0.99, 1.0, 0.8, 0.999], dtype=np.float32)
+    with hip_sampler.HipSampler(rows, vocab, testing=True) as handle:
+        for trial in range(2):
+            uniforms = rng.random(rows, dtype=np.float32)
+            _announce("parts of three tiles, %d x %d, draw %d" % (rows, vocab, trial))
+            handle.upload_logits(logits)
+            gpu = handle.sample(params, uniforms, None)
+            assert not handle.disordered_rows(rows).any()
+            cpu = parity_util.run_oracle(logits, params, uniforms)
+            parity_util.assert_results_match(gpu, cpu, "f32", "parts of three tiles, draw %d" % trial)
+            assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
