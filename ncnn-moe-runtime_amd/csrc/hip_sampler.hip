@@ -33,6 +33,7 @@ struct ncnn_moe_hip_sampler
     hipStream_t side_stream = nullptr;
     hipEvent_t side_fork = nullptr;
     hipEvent_t side_join = nullptr;
+    hipEvent_t cut_done = nullptr;
     hipStream_t stream = nullptr;
 
     void* logits = nullptr;
@@ -326,15 +327,47 @@ int launch_sampler(
         else
             launch_select<NCNN_MOE_LOGITS_BF16>(row_geometry, rows, on, a, only_pending, s->scatter_segments != 0);
     };
+    // A long row's radix sort is spread over several workgroups (two tiles each, at most kMaxSortParts):
+    // two launches per pass over a (parts, rows) grid.  Short rows keep the one-workgroup kernel.
+    const uint32_t sort_tiles = static_cast<uint32_t>((static_cast<uint64_t>(vocab) + kSortTile - 1) / kSortTile);
+    const uint32_t sort_tiles_per_part = std::max<uint32_t>(1, (sort_tiles + kMaxSortParts - 1) / kMaxSortParts);
+    const uint32_t sort_parts = std::max<uint32_t>(1, (sort_tiles + sort_tiles_per_part - 1) / sort_tiles_per_part);
+    // fp32 rows whose sort is spread over the GPU are sorted only as far as their terms can move a sum
+    // (full_order_cut_kernel); a row whose replay finds that guess too short stays pending, and a second launch of
+    // the full-order kernels, behind the first, sorts it whole.
+    const bool partial_sort = passes.full_order && dtype == NCNN_MOE_LOGITS_F32 && !want_distribution && sort_tiles >= 4 &&
+        s->spread_sort != 0 && s->partial_sort != 0;
+    if (partial_sort)
+    {
+        a.sort_lengths = s->sort_cuts;
+        a.sort_last_keys = s->sort_cuts + s->max_rows;
+        a.finite_counts = s->sort_cuts + 2 * static_cast<size_t>(s->max_rows);
+        a.disordered_rows = s->sort_cuts + 3 * static_cast<size_t>(s->max_rows);
+    }
     // Side by side (see below) with the first select in the call: the wide select is forked off in front of it
     // and picks its rows by their options, and the first select leaves those rows alone.
     const bool side_by_side = passes.side_by_side && passes.wide_select && passes.full_order && s->side_stream != nullptr;
     const bool early_wide = side_by_side && passes.select;
-    if (early_wide)
+    // The kernel that guesses the rows' cuts needs the logits and the options only: it runs on the second stream
+    // beside the first select, for the rows whose options no select pass serves (a row that a select pass hands
+    // on, its window overflowing with ties, is sorted whole).
+    const bool early_cut = partial_sort && passes.select && s->side_stream != nullptr;
+    if (early_wide || early_cut)
     {
         if (hipEventRecord(s->side_fork, stream) != hipSuccess || hipStreamWaitEvent(s->side_stream, s->side_fork, 0) != hipSuccess)
             return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
-        launch_wide(s->side_stream, 2);
+        if (early_cut)
+        {
+            SamplerArgs cut = a;
+            cut.leave_wide_rows = 0;
+            cut.cut_by_options = 1;
+            cut.max_select_top_k = passes.wide_select || batch_geometry.wide ? kSelectTopK : kFastTopK;
+            hipLaunchKernelGGL(full_order_cut_kernel, dim3(rows), dim3(kSortThreads), 0, s->side_stream, cut);
+            if (hipEventRecord(s->cut_done, s->side_stream) != hipSuccess)
+                return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
+        }
+        if (early_wide)
+            launch_wide(s->side_stream, 2);
     }
     if (passes.select)
     {
@@ -345,11 +378,6 @@ int launch_sampler(
         else
             launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, first, 0, s->scatter_segments != 0);
     }
-    // A long row's radix sort is spread over several workgroups (two tiles each, at most kMaxSortParts):
-    // two launches per pass over a (parts, rows) grid.  Short rows keep the one-workgroup kernel.
-    const uint32_t sort_tiles = static_cast<uint32_t>((static_cast<uint64_t>(vocab) + kSortTile - 1) / kSortTile);
-    const uint32_t sort_tiles_per_part = std::max<uint32_t>(1, (sort_tiles + kMaxSortParts - 1) / kMaxSortParts);
-    const uint32_t sort_parts = std::max<uint32_t>(1, (sort_tiles + sort_tiles_per_part - 1) / sort_tiles_per_part);
     const auto launch_spread_sort = [&](SamplerArgs spread, auto dtype_tag, auto pairs_tag) {
         constexpr int kType = decltype(dtype_tag)::value;
         constexpr bool kPairs = decltype(pairs_tag)::value;
@@ -368,18 +396,6 @@ int launch_sampler(
     };
     // `leftovers`: the launch behind the wide select, for the few rows (usually none) that it could not
     // finish; it is kept to two kernels, because every launch costs its few microseconds even with no row to serve.
-    // fp32 rows whose sort is spread over the GPU are sorted only as far as their terms can move a sum
-    // (full_order_cut_kernel); a row whose replay finds that guess too short stays pending, and a second launch of
-    // the full-order kernels, behind the first, sorts it whole.
-    const bool partial_sort = passes.full_order && dtype == NCNN_MOE_LOGITS_F32 && !want_distribution && sort_tiles >= 4 &&
-        s->spread_sort != 0 && s->partial_sort != 0;
-    if (partial_sort)
-    {
-        a.sort_lengths = s->sort_cuts;
-        a.sort_last_keys = s->sort_cuts + s->max_rows;
-        a.finite_counts = s->sort_cuts + 2 * static_cast<size_t>(s->max_rows);
-        a.disordered_rows = s->sort_cuts + 3 * static_cast<size_t>(s->max_rows);
-    }
     const auto launch_full_order = [&](SamplerArgs a, bool leftovers) {
         const bool spread_sort = sort_tiles >= 4 && s->spread_sort != 0 && !leftovers;
         const bool runs = dtype == NCNN_MOE_LOGITS_BF16 && !want_distribution;
@@ -391,7 +407,9 @@ int launch_sampler(
             hipLaunchKernelGGL(full_order_row_list_kernel, dim3(1), dim3(kSortThreads), 0, stream, a, rows, s->row_list);
             a.row_list = s->row_list;
         }
-        if (!leftovers && partial_sort)
+        if (!leftovers && partial_sort && early_cut)
+            (void)hipStreamWaitEvent(stream, s->cut_done, 0);
+        else if (!leftovers && partial_sort)
             hipLaunchKernelGGL(full_order_cut_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
         // the token indices ride along with the keys only when the whole distribution is exported
         const auto sort_rows = [&](auto dtype_tag, auto pairs_tag) {
@@ -599,6 +617,7 @@ int ncnn_moe_hip_sampler_create(int device, uint32_t max_rows, uint32_t max_voca
     CREATE_CHECK(hipStreamCreateWithFlags(&s->side_stream, hipStreamNonBlocking));
     CREATE_CHECK(hipEventCreateWithFlags(&s->side_fork, hipEventDisableTiming));
     CREATE_CHECK(hipEventCreateWithFlags(&s->side_join, hipEventDisableTiming));
+    CREATE_CHECK(hipEventCreateWithFlags(&s->cut_done, hipEventDisableTiming));
     const size_t rows = max_rows;
     const size_t slots = rows * s->max_segments;
     CREATE_CHECK(hipMalloc(&s->logits, rows * s->logits_stride_f32 * sizeof(float)));
@@ -690,6 +709,8 @@ void ncnn_moe_hip_sampler_destroy(ncnn_moe_hip_sampler* s)
         (void)hipEventDestroy(s->side_fork);
     if (s->side_join != nullptr)
         (void)hipEventDestroy(s->side_join);
+    if (s->cut_done != nullptr)
+        (void)hipEventDestroy(s->cut_done);
     void* buffers[] = {
         s->logits, s->params, s->uniforms, s->results, s->segment_values, s->segment_indices,
         s->segment_counts, s->row_counter, s->row_flags, s->row_state, s->split_records, s->row_epoch, s->sort_keys[0], s->sort_keys[1],

@@ -87,6 +87,9 @@ struct SamplerArgs
     // row to see them all, and out of order): that row is sorted whole by the launch behind this one.
     uint32_t* disordered_rows;
     uint32_t sort_low_digit_skipped;
+    // full_order_cut_kernel runs beside the first select: it takes the rows that no select pass serves by their
+    // options (widest window: max_select_top_k), not by row_state, which that select is still writing
+    uint32_t cut_by_options;
 };
 
 // Where the terms of the sorted rows' elements are kept (see sort_low_digit_skipped).

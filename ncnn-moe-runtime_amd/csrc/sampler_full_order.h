@@ -110,7 +110,15 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
-    const bool served = a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
+    bool served;
+    if (a.cut_by_options != 0u)
+    {
+        uint32_t effective_k = 0;
+        int status = NCNN_MOE_ROW_OK;
+        served = resolve_row_mode(a.params[row], a.vocab, a.max_select_top_k, a.force_general, effective_k, status) == kModeGeneral;
+    }
+    else
+        served = a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
     const float temperature = a.params[row].temperature;
     const uint32_t top_k = a.params[row].top_k;
     const float window = top_k > 0u && top_k < a.vocab ? static_cast<float>(top_k) : 0.0f;
