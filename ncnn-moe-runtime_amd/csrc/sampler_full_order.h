@@ -1878,14 +1878,33 @@ __global__ __launch_bounds__(kTermsThreads) void full_order_terms_kernel(Sampler
             tile_keys[slot] = key;
         }
         __syncthreads();
-        uint32_t long_groups = 0;
+        // A tile that is in order as it stands, with the neighbours its elements would look at, needs nothing
+        // (every tile of a row whose keys end in the same byte: logits that were rounded to bf16 or fp16, whose
+        // groups are long runs of equal keys): no pair of keys within reach of an element is out of order unless
+        // two adjacent keys between them are.
+        bool out_of_order = false;
 #pragma unroll
         for (int j = 0; j < kTermsPerThread; ++j)
         {
-            const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
-            bool further = false;
-            places[j] = touched_up_place(tile_keys + kTouchUpReach + j * kTermsThreads + static_cast<int>(threadIdx.x), loaded[j], i, further);
-            long_groups |= further && i < n ? 1u << j : 0u;
+            places[j] = first + static_cast<uint32_t>(j * kTermsThreads);
+            out_of_order |= tile_keys[kTouchUpReach + j * kTermsThreads + static_cast<int>(threadIdx.x) + 1] < loaded[j];
+        }
+        if (threadIdx.x < static_cast<uint32_t>(kTouchUpReach))
+            out_of_order |= tile_keys[threadIdx.x + 1u] < tile_keys[threadIdx.x];
+        else if (threadIdx.x < 2u * kTouchUpReach - 1u)
+            out_of_order |= tile_keys[kTermsTile + threadIdx.x + 1u] < tile_keys[kTermsTile + threadIdx.x];
+        const bool touch_tile = __syncthreads_or(out_of_order ? 1 : 0) != 0;
+        uint32_t long_groups = 0;
+        if (touch_tile)
+        {
+#pragma unroll
+            for (int j = 0; j < kTermsPerThread; ++j)
+            {
+                const uint32_t i = first + static_cast<uint32_t>(j * kTermsThreads);
+                bool further = false;
+                places[j] = touched_up_place(tile_keys + kTouchUpReach + j * kTermsThreads + static_cast<int>(threadIdx.x), loaded[j], i, further);
+                long_groups |= further && i < n ? 1u << j : 0u;
+            }
         }
         if (long_groups != 0u)
         {

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import parity_util
-from ncnn_moe_runtime_amd import hip_sampler
+from ncnn_moe_runtime_amd import hip_sampler, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -183,6 +183,8 @@ def test_groups_of_keys_that_differ_in_the_lowest_byte_only(sampler):
     logits[13, 1000:40000] = np.float32(1.25)                     # a padded stretch of equal logits among spread ones
     logits[14] = _grouped_row(rng, 40)
     logits[14] = -np.sort(-logits[14])                            # long groups, in order already (descending logits)
+    # logits that were rounded to bf16 on their way (an LM head in bf16, its output widened): every key ends in the same bytes
+    logits[15] = workloads.bf16_bits_to_float32(workloads.float32_to_bf16_bits(logits[15]))
     for trial in range(2):
         uniforms = rng.random(ROWS, dtype=np.float32)
         _, disordered = _sample_with_three_passes_and_four(sampler, logits, params, uniforms, "groups in the lowest byte, draw %d" % trial)
