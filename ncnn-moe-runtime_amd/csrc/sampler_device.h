@@ -337,6 +337,23 @@ __device__ __forceinline__ void narrow_digit_peers(uint32_t digit, uint32_t& low
     high = __builtin_amdgcn_bitop3_b32(high, static_cast<uint32_t>(set >> 32), mine, kKeepWhereEqual);
 }
 
+__device__ __forceinline__ void wave_digit_peers(uint32_t digit, bool valid, uint32_t& low, uint32_t& high);
+
+// (every lane of the wave is valid)
+__device__ __forceinline__ void wave_digit_peers(uint32_t digit, uint32_t& low, uint32_t& high)
+{
+    low = 0xffffffffu;
+    high = 0xffffffffu;
+    narrow_digit_peers<0>(digit, low, high);
+    narrow_digit_peers<1>(digit, low, high);
+    narrow_digit_peers<2>(digit, low, high);
+    narrow_digit_peers<3>(digit, low, high);
+    narrow_digit_peers<4>(digit, low, high);
+    narrow_digit_peers<5>(digit, low, high);
+    narrow_digit_peers<6>(digit, low, high);
+    narrow_digit_peers<7>(digit, low, high);
+}
+
 __device__ __forceinline__ void wave_digit_peers(uint32_t digit, bool valid, uint32_t& low, uint32_t& high)
 {
     const uint64_t all = __builtin_amdgcn_ballot_w64(valid);

@@ -789,27 +789,41 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
         uint32_t tile_ranks[kSortPerThread];
         const uint32_t wave_first = tile + static_cast<uint32_t>(wave) * (kWaveSize * kSortPerThread);
         lds_barrier();
+        // (a tile that lies inside the row and keeps every key - all tiles but a row's last in the passes behind
+        // the first - is ranked and staged by code without the tests of each key: the pass's time is the
+        // instructions it issues)
+        const bool whole_tile = tile + kSortTile <= n && last_key == 0xffffffffu;
+        const auto rank_tile = [&](auto whole_tag) {
+            constexpr bool kWhole = decltype(whole_tag)::value;
 #pragma unroll
-        for (int e = 0; e < kSortPerThread; ++e)
-        {
-            const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
-            const bool valid = i < n && tile_keys[e] <= last_key;
-            const uint32_t digit = (tile_keys[e] >> shift) & 255u;
-            if (ANY_ORDER)
+            for (int e = 0; e < kSortPerThread; ++e)
             {
-                tile_ranks[e] = valid ? atomicAdd(&wave_counts[wave][digit], 1u) : 0u;
-                continue;
+                const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+                const bool valid = kWhole || (i < n && tile_keys[e] <= last_key);
+                const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+                if (ANY_ORDER)
+                {
+                    tile_ranks[e] = valid ? atomicAdd(&wave_counts[wave][digit], 1u) : 0u;
+                    continue;
+                }
+                uint32_t peers_low, peers_high;
+                if constexpr (kWhole)
+                    wave_digit_peers(digit, peers_low, peers_high);
+                else
+                    wave_digit_peers(digit, valid, peers_low, peers_high);
+                const uint32_t rank_in_round = __builtin_amdgcn_mbcnt_hi(peers_high, __builtin_amdgcn_mbcnt_lo(peers_low, 0u));
+                uint32_t seen = 0;
+                if (valid)
+                    seen = wave_counts[wave][digit];
+                tile_ranks[e] = seen + rank_in_round;
+                if (valid && rank_in_round == 0)
+                    wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popc(peers_low) + __popc(peers_high));
             }
-            uint32_t peers_low, peers_high;
-            wave_digit_peers(digit, valid, peers_low, peers_high);
-            const uint32_t rank_in_round = __builtin_amdgcn_mbcnt_hi(peers_high, __builtin_amdgcn_mbcnt_lo(peers_low, 0u));
-            uint32_t seen = 0;
-            if (valid)
-                seen = wave_counts[wave][digit];
-            tile_ranks[e] = seen + rank_in_round;
-            if (valid && rank_in_round == 0)
-                wave_counts[wave][digit] = seen + static_cast<uint32_t>(__popc(peers_low) + __popc(peers_high));
-        }
+        };
+        if (whole_tile)
+            rank_tile(std::true_type{});
+        else
+            rank_tile(std::false_type{});
         lds_barrier();
         uint32_t digit_total = 0;
         uint32_t inclusive = 0;
@@ -851,34 +865,48 @@ __global__ __launch_bounds__(kSortThreads) __attribute__((amdgpu_waves_per_eu(8,
                                                        // its readers as a wave's total are in front of this one)
         }
         lds_barrier();
+        const auto stage_tile = [&](auto whole_tag) {
+            constexpr bool kWhole = decltype(whole_tag)::value;
 #pragma unroll
-        for (int e = 0; e < kSortPerThread; ++e)
-        {
-            const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
-            if (i < n && tile_keys[e] <= last_key)
+            for (int e = 0; e < kSortPerThread; ++e)
             {
-                const uint32_t digit = (tile_keys[e] >> shift) & 255u;
-                const uint32_t slot = tile_start[digit] + wave_counts[wave][digit] + tile_ranks[e];
-                staged_keys[slot] = tile_keys[e];
-                if (PAIRS)
-                    staged_indices[slot] = tile_indices[e];
+                const uint32_t i = wave_first + static_cast<uint32_t>(e * kWaveSize + lane);
+                if (kWhole || (i < n && tile_keys[e] <= last_key))
+                {
+                    const uint32_t digit = (tile_keys[e] >> shift) & 255u;
+                    const uint32_t slot = tile_start[digit] + wave_counts[wave][digit] + tile_ranks[e];
+                    staged_keys[slot] = tile_keys[e];
+                    if (PAIRS)
+                        staged_indices[slot] = tile_indices[e];
+                }
             }
-        }
+        };
+        if (whole_tile)
+            stage_tile(std::true_type{});
+        else
+            stage_tile(std::false_type{});
         lds_barrier();
         const uint32_t tile_count = scan_partial[3];
+        const auto write_tile = [&](auto whole_tag) {
+            constexpr bool kWhole = decltype(whole_tag)::value;
 #pragma unroll
-        for (int e = 0; e < kSortPerThread; ++e)
-        {
-            const uint32_t slot = static_cast<uint32_t>(e * kSortThreads + tid);
-            if (slot < tile_count)
+            for (int e = 0; e < kSortPerThread; ++e)
             {
-                const uint32_t key = staged_keys[slot];
-                const uint32_t position = global_offset[(key >> shift) & 255u] + slot;
-                target_keys[position] = key;
-                if (PAIRS)
-                    target_indices[position] = staged_indices[slot];
+                const uint32_t slot = static_cast<uint32_t>(e * kSortThreads + tid);
+                if (kWhole || slot < tile_count)
+                {
+                    const uint32_t key = staged_keys[slot];
+                    const uint32_t position = global_offset[(key >> shift) & 255u] + slot;
+                    target_keys[position] = key;
+                    if (PAIRS)
+                        target_indices[position] = staged_indices[slot];
+                }
             }
-        }
+        };
+        if (whole_tile)
+            write_tile(std::true_type{});
+        else
+            write_tile(std::false_type{});
         lds_barrier();
     }
 }
