@@ -212,3 +212,36 @@ def test_parts_of_several_tiles():
             cpu = parity_util.run_oracle(logits, params, uniforms)
             parity_util.assert_results_match(gpu, cpu, "f32", "parts of three tiles, draw %d" % trial)
             assert (gpu["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+
+
+@pytest.mark.parametrize("vocab", [24577, 32768, 32769, 65543, 131072, 131073, 200003])
+def test_row_lengths_around_the_tiles_and_parts_of_the_sort(vocab):
+    """Rows that end at, just behind and just in front of a tile of the spread sort (8,192 keys) and of the terms
+    kernel (2,048), and rows of one tile and of two tiles per part: the cut, the three passes and the touch-up of
+    the lowest byte at the row's end, against the oracle and the four-pass sort."""
+    rows = 5
+    rng = np.random.default_rng(4900 + vocab)
+    logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    logits[3] = workloads.bf16_bits_to_float32(workloads.float32_to_bf16_bits(logits[3]))
+    logits[4, -3000:] = logits[4, -1]  # a run of equal logits at the row's end (in index order)
+    params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+    params["temperature"] = np.array([0.2, 0.7, 1.2, 1.0, 1.5], dtype=np.float32)
+    params["top_p"] = np.array([0.9, 0.97, 1.0, 0.95, 0.999], dtype=np.float32)
+    with hip_sampler.HipSampler(rows, vocab, testing=True) as handle:
+        handle.upload_logits(logits)
+        for trial in range(2):
+            uniforms = rng.random(rows, dtype=np.float32)
+            _announce("rows of %d logits, draw %d" % (vocab, trial))
+            three = handle.sample(params, uniforms, None)
+            # (row 4 may go to the second launch: a spread logit that shares its upper 24 bits with the run's value and
+            # has a larger lowest byte would have to cross the whole run)
+            assert not handle.disordered_rows(rows)[:4].any()
+            handle.skip_low_digit(False)
+            try:
+                four = handle.sample(params, uniforms, None)
+            finally:
+                handle.skip_low_digit(True)
+            cpu = parity_util.run_oracle(logits, params, uniforms)
+            parity_util.assert_results_match(three, cpu, "f32", "rows of %d logits, draw %d" % (vocab, trial))
+            assert three.tobytes() == four.tobytes()
+            assert (three["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
