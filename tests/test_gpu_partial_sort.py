@@ -245,3 +245,40 @@ def test_row_lengths_around_the_tiles_and_parts_of_the_sort(vocab):
             parity_util.assert_results_match(three, cpu, "f32", "rows of %d logits, draw %d" % (vocab, trial))
             assert three.tobytes() == four.tobytes()
             assert (three["flags"] & hip_sampler.FLAG_GENERAL_PATH != 0).all()
+
+
+def test_random_rows_three_passes_and_four():
+    """Thirty random batches (row length, spread, offset, quantisation, infinities, options drawn at random): the
+    three-pass sort against the oracle and, byte for byte, against the four-pass sort."""
+    rng = np.random.default_rng(5000)
+    for case in range(30):
+        rows = int(rng.integers(1, 9))
+        vocab = int(rng.integers(24577, 150000))
+        spread = float(rng.choice([0.05, 0.5, 2.0, 6.0]))
+        logits = (rng.standard_normal((rows, vocab)) * spread + float(rng.choice([0.0, -30.0, 100.0]))).astype(np.float32)
+        kind = case % 5
+        if kind == 1:
+            logits = np.round(logits * 8) / 8                              # few distinct values
+        elif kind == 2:
+            logits = workloads.bf16_bits_to_float32(workloads.float32_to_bf16_bits(logits))
+        elif kind == 3:
+            logits[:, rng.integers(0, vocab, vocab // 3)] = -np.inf
+            logits[0, rng.integers(0, vocab, 3)] = np.nan
+        elif kind == 4:
+            logits[:, vocab // 2:] = logits[:, :1]                         # half of every row one value
+        params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+        params["temperature"] = rng.choice(np.array([0.1, 0.5, 0.9, 1.3, 2.0], dtype=np.float32), size=rows)
+        params["top_p"] = rng.choice(np.array([0.3, 0.9, 0.99, 1.0], dtype=np.float32), size=rows)
+        params["min_p"] = rng.choice(np.array([0.0, 0.0, 0.01], dtype=np.float32), size=rows)
+        params["top_k"] = rng.choice(np.array([0, 0, 2000, 70000], dtype=np.uint32), size=rows)
+        uniforms = rng.random(rows, dtype=np.float32)
+        context = "random case %d: %d x %d, spread %.2f, kind %d" % (case, rows, vocab, spread, kind)
+        _announce(context)
+        with hip_sampler.HipSampler(rows, vocab, testing=True) as handle:
+            handle.upload_logits(logits)
+            three = handle.sample(params, uniforms, None)
+            handle.skip_low_digit(False)
+            four = handle.sample(params, uniforms, None)
+        cpu = parity_util.run_oracle(logits, params, uniforms)
+        parity_util.assert_results_match(three, cpu, "f32", context)
+        assert three.tobytes() == four.tobytes(), context
