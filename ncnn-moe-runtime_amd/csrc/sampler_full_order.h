@@ -584,8 +584,10 @@ __device__ __forceinline__ void load_sort_keys(
 
 // One workgroup counts kHistogramParts consecutive parts of a row, with the loads of all of them in flight
 // together: a workgroup's time is one trip to memory and the hand-over of its counts, whatever it counts,
-// so a part per workgroup would only add rounds of workgroups.  grid (parts / kHistogramParts rounded up, rows).
-constexpr int kHistogramParts = 4;
+// so a part per workgroup only adds rounds of workgroups (configuration 4: 384 us a step with one part a
+// workgroup, 374 with two, 379 with four, which leave half of the GPU's workgroup slots empty in the passes
+// that read the kept keys).  grid (parts / kHistogramParts rounded up, rows).
+constexpr int kHistogramParts = 2;
 
 template <int DTYPE>
 __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(SamplerArgs a)
@@ -678,10 +680,10 @@ __global__ __launch_bounds__(kSortThreads) void sort_part_histogram_kernel(Sampl
         }
     }
     {
-        const int q = tid >> 8; // kSortThreads / 256 == kHistogramParts
+        const int q = tid >> 8; // (the first 256 * kHistogramParts threads)
         const int digit = tid & 255;
-        static_assert(kSortThreads == 256 * kHistogramParts, "a thread per part and digit");
-        if (first_part + q < a.sort_parts)
+        static_assert(kSortThreads >= 256 * kHistogramParts, "a thread per part and digit");
+        if (q < kHistogramParts && first_part + q < a.sort_parts)
         {
             uint32_t total = 0;
 #pragma unroll
