@@ -89,7 +89,7 @@ __global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(Sampl
 // row; at 0.5 it lies behind the first tenth.
 // One workgroup per row looks at a sample of the row (16,384 logits, 256 evenly spaced runs of 64): counts of
 // the keys' upper twelve bits (4,096 buckets: sign, exponent and three bits of the mantissa).  With the terms of
-// the buckets' lower and upper ends it looks for the first bucket whose largest possible term is below 2^-27 of
+// the buckets' lower and upper ends it looks for the first bucket whose largest possible term is below 2^-26 of
 // the least the buckets in front of it add up to (the sums' half ulp is 2^-25 to 2^-24 of them) - or, under a Top-K
 // window, the first bucket behind twice the window by the sample's count - and has the sort
 // keep the buckets in front of it: sort_last_keys.  This is a guess that costs or saves time, never exactness:
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
         // (a Top-K window ends the row's sums at K elements: a few times K, by the sample's count, are kept)
         const bool behind_the_window = window != 0.0f && count_here >= 2.0f * window + kCutMinimum;
         if (bucket > kFirstFiniteBucket && bucket <= kLastFiniteBucket && count_here >= kCutMinimum &&
-            (largest_term < mass_here * 7.450580596923828e-09f || behind_the_window)) // 2^-27
+            (largest_term < mass_here * 1.4901161193847656e-08f || behind_the_window)) // 2^-26
             candidate = bucket;
     }
     if (candidate < static_cast<uint32_t>(kCutBuckets))
