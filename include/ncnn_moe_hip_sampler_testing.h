@@ -47,6 +47,10 @@ int ncnn_moe_hip_sampler_debug_sort_lengths(ncnn_moe_hip_sampler* sampler, uint3
  * was handed to the second launch for this reason (written for the rows that partial_sort serves). */
 int ncnn_moe_hip_sampler_debug_skip_low_digit(ncnn_moe_hip_sampler* sampler, int enabled);
 int ncnn_moe_hip_sampler_debug_disordered_rows(ncnn_moe_hip_sampler* sampler, uint32_t* flags, uint32_t rows);
+/* wide_sampled_bound (on by default): a row of four chunks or more whose Top-K window is wider than 512 gets the bound
+ * under which the wide select collects its candidates from a sample of the whole row (a row whose list then ends short
+ * of the window is handed to the full-order kernels); off, from the row's first chunk.  Same results either way. */
+int ncnn_moe_hip_sampler_debug_wide_sampled_bound(ncnn_moe_hip_sampler* sampler, int enabled);
 /* Sets the per-row launch numbers (epochs, 1 .. 8191) that tag the split kernel's hand-over records: of the
  * handle, or with a null handle of the static scratch of `device` (after it has served a call).  Tests start a
  * few launches in front of the point where the epochs start over. */

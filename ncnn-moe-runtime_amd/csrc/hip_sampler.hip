@@ -71,6 +71,7 @@ struct ncnn_moe_hip_sampler
     uint32_t* sort_cuts = nullptr;        // [4][rows]: SamplerArgs::sort_lengths, sort_last_keys, finite_counts, disordered_rows
     int partial_sort = 1;                 // full-order fp32 rows are sorted only as far as their terms can move a sum
     int skip_low_digit = 1;               // ... by three passes over the keys' upper 24 bits, the lowest byte put in order by the terms kernel
+    int wide_sampled_bound = 1;           // the wide select bounds its widest windows from a sample of the whole row
     uint32_t* sort_part_counts = nullptr; // [rows][kMaxSortParts][256]
     double* term_sums = nullptr;          // [rows][term_sum_parts]: fp64 sums of the terms kernel's blocks
     uint4* chunk_steps = nullptr;         // [rows][chunk_capacity]: composed step of every whole chunk of a sorted row's terms
@@ -292,6 +293,7 @@ int launch_sampler(
     a.vocab = vocab;
     const uint64_t span = logits_span(vocab, dtype, logits, row_stride);
     a.force_general = s->force_general;
+    a.wide_sampled_bound = s->wide_sampled_bound != 0 ? 1u : 0u;
     a.params = params;
     a.uniforms = uniforms;
     a.stop_ids = stop_ids;
@@ -1201,6 +1203,15 @@ int ncnn_moe_hip_sampler_debug_skip_low_digit(ncnn_moe_hip_sampler* s, int enabl
     if (s == nullptr)
         return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
     s->skip_low_digit = enabled ? 1 : 0;
+    return NCNN_MOE_SAMPLER_SUCCESS;
+}
+
+// The wide select's bound for windows wider than 512: from a sample of the whole row (the default) or from the first chunk.
+int ncnn_moe_hip_sampler_debug_wide_sampled_bound(ncnn_moe_hip_sampler* s, int enabled)
+{
+    if (s == nullptr)
+        return NCNN_MOE_SAMPLER_INVALID_ARGUMENT;
+    s->wide_sampled_bound = enabled ? 1 : 0;
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

@@ -90,6 +90,9 @@ struct SamplerArgs
     // full_order_cut_kernel runs beside the first select: it takes the rows that no select pass serves by their
     // options (widest window: max_select_top_k), not by row_state, which that select is still writing
     uint32_t cut_by_options;
+    // The wide select takes the bound of a window wider than kTwoKeyBoundTopK from a sample of the whole row (1)
+    // or from the row's first chunk alone (0); same results either way.
+    uint32_t wide_sampled_bound;
 };
 
 // Where the terms of the sorted rows' elements are kept (see sort_low_digit_skipped).

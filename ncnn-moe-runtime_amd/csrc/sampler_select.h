@@ -516,7 +516,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     if (WIDE && a.only_pending == 2 && (greedy || effective_k <= static_cast<uint32_t>(kFastTopK)))
         return; // the first select's row
     // the list is tightened when it grows past this; a wide list keeps room for a chunk's additions
-    const uint32_t tighten_limit = WIDE ? static_cast<uint32_t>(2 * top_k + 64) : static_cast<uint32_t>(kNarrowListCap - 192);
+    uint32_t tighten_limit = WIDE ? static_cast<uint32_t>(2 * top_k + 64) : static_cast<uint32_t>(kNarrowListCap - 192);
     uint32_t next_check = 0;      // chunk at which the list is looked at next
     uint32_t count_at_check = 0;  // list length at the last look
     uint32_t chunk_at_check = first_chunk;  // first chunk after the last look
@@ -525,6 +525,63 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
     {
         shared.block_flags = 0;
         shared.list_count = 0;
+    }
+
+    // ---- a window wider than kTwoKeyBoundTopK over a long row: the bound comes from a sample of the whole row.
+    // The K-th largest value of the first chunk is reached by a tenth of that chunk, and the bounds that the list's
+    // cuts give after c chunks are still reached by K / c values of the next one: some 4 K candidates in all for a
+    // row of thirteen chunks, and two or three cuts of the list on the way.  A sample of one chunk's size, in runs of
+    // 64 bytes spread evenly over the row, says where the K-th largest of the row lies: with r = vocab / sample size,
+    // the sample's m-th largest is reached by about m r values of the row, give or take r sqrt(m), and m is chosen
+    // so that m r - kSampleSigmas r sqrt(m) = K.  For K = 1000 in 129,280 logits m = 146: some 1,840 candidates in
+    // all (give or take 150), no cut on the way, and no bound to work out from the first chunk.  The sample can mislead (values in an
+    // order that the runs' spacing resonates with): a list that ends with fewer than K candidates under such a
+    // bound proves nothing, and the row is handed to the full-order kernels like a row whose list overflowed.
+    bool sampled_bound = false;
+    if constexpr (WIDE)
+    {
+        constexpr uint32_t kRunVectors = 4; // 64 bytes
+        constexpr uint32_t kRuns = static_cast<uint32_t>(kScanThreads) * kVectors / kRunVectors;
+        constexpr uint32_t kSampledBoundMinChunks = 4;
+        constexpr float kSampleSigmas = 5.5f;
+        static_assert(static_cast<uint32_t>(kScanThreads) * kVectors % kRunVectors == 0, "whole runs");
+        if (a.wide_sampled_bound != 0u && top_k > kTwoKeyBoundTopK && total_chunks >= kSampledBoundMinChunks)
+        {
+            // vectors that lie inside the row as a whole: at least (kSampledBoundMinChunks - 1) chunks' worth - 2
+            const uint32_t first_whole = (valid_begin + kWidth - 1) / kWidth;
+            const uint32_t whole_vectors = valid_end / kWidth - first_whole;
+            const uint32_t spacing = whole_vectors / kRuns; // >= 2 * kRunVectors
+            uint32_t sample_keys[kLaneValues];
+            uint4 sample[kVectors];
+#pragma unroll
+            for (int v = 0; v < kVectors; ++v)
+            {
+                const uint32_t g = static_cast<uint32_t>(v * kScanThreads + tid);
+                const uint32_t vector = first_whole + (g / kRunVectors) * spacing + g % kRunVectors;
+                // (an ordinary load: the line stays in the cache for the chunk that holds it)
+                sample[v] = *reinterpret_cast<const uint4*>(aligned_base + static_cast<size_t>(vector) * 16u);
+            }
+#pragma unroll
+            for (int v = 0; v < kVectors; ++v)
+            {
+                float x[kWidth];
+                Vector::unpack(sample[v], x);
+#pragma unroll
+                for (int c = 0; c < kWidth; ++c)
+                    sample_keys[v * kWidth + c] = x[c] > -__builtin_inff() ? ascending_key(x[c]) : 0u; // false for NaN as well
+            }
+            const float ratio = static_cast<float>(a.vocab) / static_cast<float>(kChunk);
+            const float root = 0.5f * (kSampleSigmas + sqrtf(kSampleSigmas * kSampleSigmas + 4.0f * static_cast<float>(top_k) / ratio));
+            const int sample_rank = static_cast<int>(root * root) + 1;
+            const uint32_t sample_bound = workgroup_kth_of_keys_by_digits(sample_keys, sample_rank, tid, shared.bound);
+            if (sample_bound != 0u)
+            {
+                bound_key = sample_bound;
+                sampled_bound = true;
+                // under such a bound a chunk adds a few hundred candidates at most: the list may grow further
+                tighten_limit = max(tighten_limit, static_cast<uint32_t>(kWideListCap - 1024));
+            }
+        }
     }
 
     __syncthreads();
@@ -606,7 +663,7 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         // the row is no smaller.
         // (also a later chunk while there is no bound yet: a row that begins with a stretch of -inf, a masked
         // part of the vocabulary, must not pour its first chunk of finite logits into the list unfiltered)
-        if (first_of_segment || (LOOPED && bound_key == 0u))
+        if ((first_of_segment && !sampled_bound) || (LOOPED && bound_key == 0u))
         {
             if (WIDE && top_k > kTwoKeyBoundTopK)
             {
@@ -743,6 +800,8 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
         __syncthreads();
         if (shared.list_count > static_cast<uint32_t>(Shared::kListCap))
             overflow = true;
+        if (sampled_bound && shared.list_count < static_cast<uint32_t>(top_k))
+            overflow = true; // the sample misled: the list holds a part of the window only
     }
     else
     {

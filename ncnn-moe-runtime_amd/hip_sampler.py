@@ -76,6 +76,7 @@ TESTING_SYMBOLS = [
     "ncnn_moe_hip_sampler_debug_partial_sort",
     "ncnn_moe_hip_sampler_debug_sort_lengths",
     "ncnn_moe_hip_sampler_debug_skip_low_digit",
+    "ncnn_moe_hip_sampler_debug_wide_sampled_bound",
     "ncnn_moe_hip_sampler_debug_disordered_rows",
     "ncnn_moe_hip_sampler_debug_chunk_steps",
     "ncnn_moe_hip_sampler_debug_stream_only",
@@ -125,6 +126,7 @@ def _bind(lib, testing):
     lib.ncnn_moe_hip_sampler_debug_partial_sort.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_sort_lengths.argtypes = [vp, vp, ctypes.c_uint32]
     lib.ncnn_moe_hip_sampler_debug_skip_low_digit.argtypes = [vp, ctypes.c_int]
+    lib.ncnn_moe_hip_sampler_debug_wide_sampled_bound.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_disordered_rows.argtypes = [vp, vp, ctypes.c_uint32]
     lib.ncnn_moe_hip_sampler_debug_fused_bf16.argtypes = [vp, ctypes.c_int]
     lib.ncnn_moe_hip_sampler_debug_chunk_steps.argtypes = [vp, ctypes.c_int]
@@ -352,6 +354,11 @@ class HipSampler:
         """Test hook: the spread sort of full-order fp32 rows in three passes over the keys' upper 24 bits, the lowest
         byte put in order on the way to the terms (default), or in four passes."""
         self._check(self._hooks().ncnn_moe_hip_sampler_debug_skip_low_digit(self._handle, 1 if enabled else 0))
+
+    def wide_sampled_bound(self, enabled):
+        """Test hook: the wide select bounds a window wider than 512 from a sample of the whole row (default) or from
+        the row's first chunk."""
+        self._check(self._hooks().ncnn_moe_hip_sampler_debug_wide_sampled_bound(self._handle, 1 if enabled else 0))
 
     def disordered_rows(self, rows):
         """Test hook: which of the last call's first `rows` rows the three-pass sort could not finish (1: the row was
