@@ -172,3 +172,42 @@ def test_distribution_under_a_sampled_bound(sampler):
         assert np.array_equal(ids[:count], oracle_ids)
         assert np.array_equal(probabilities[:count].view(np.uint32),
                               np.asarray(oracle_probabilities, dtype=np.float32).view(np.uint32))
+
+
+def test_random_rows_under_a_sampled_bound(sampler):
+    """Thirty random batches (row length, type, spread, quantisation, masked parts, infinities, NaN, sorted rows, options
+    and windows drawn at random; windows from 400, below where the sample is used, to 1100, beyond the wide select):
+    against the oracle under both bounds, and the two results byte for byte."""
+    rng = np.random.default_rng(6006)
+    for case in range(30):
+        dtype = "bf16" if case % 3 == 2 else "f32"
+        rows = int(rng.integers(1, 13))
+        vocab = int(rng.integers(30000, VOCAB_BF16))
+        spread = float(rng.choice([0.05, 0.5, 2.0, 6.0]))
+        logits = (rng.standard_normal((rows, vocab)) * spread + float(rng.choice([0.0, -30.0, 100.0]))).astype(np.float32)
+        kind = case % 6
+        if kind == 1:
+            logits = np.round(logits * 8) / 8                              # few distinct values
+        elif kind == 2:
+            logits[:, rng.integers(0, vocab, vocab // 3)] = -np.inf
+            logits[0, rng.integers(0, vocab, 3)] = np.nan
+        elif kind == 3:
+            logits[:, vocab // 2:] = logits[:, :1]                         # half of every row one value
+        elif kind == 4:
+            logits = np.sort(logits, axis=1)                               # the window at the row's end
+            logits[rows // 2:] = logits[rows // 2:, ::-1]                  # ... or at its start
+        elif kind == 5:
+            logits[:, :int(rng.integers(1, vocab))] = -np.inf              # a masked head of any length
+            logits[-1, rng.integers(0, vocab)] = np.inf
+        data = workloads.float32_to_bf16_bits(logits) if dtype == "bf16" else logits
+        params = hip_sampler.make_params(rows, 1.0, 0, 1.0, 0.0)
+        params["temperature"] = rng.choice(np.array([0.1, 0.5, 0.9, 1.3, 2.0], dtype=np.float32), size=rows)
+        params["top_p"] = rng.choice(np.array([0.3, 0.9, 0.99, 1.0], dtype=np.float32), size=rows)
+        params["min_p"] = rng.choice(np.array([0.0, 0.0, 0.01], dtype=np.float32), size=rows)
+        params["top_k"] = rng.choice(np.array([400, 513, 600, 777, 1000, 1024, 1100], dtype=np.uint32), size=rows)
+        uniforms = rng.random(rows, dtype=np.float32)
+        context = "random case %d: %d x %d, spread %.2f, kind %d" % (case, rows, vocab, spread, kind)
+        with_sample, without = _both_ways(sampler, data, params, uniforms, dtype, context)
+        # (the flags differ where one bound lets the select serve a row that the other hands on)
+        for field in ("token_id", "probability", "kept_count", "status", "is_stop", "draw_consumed"):
+            assert with_sample[field].tobytes() == without[field].tobytes(), "%s: %s" % (context, field)
