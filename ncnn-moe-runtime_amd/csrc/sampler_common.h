@@ -538,16 +538,19 @@ __device__ __forceinline__ uint32_t workgroup_kth_of_keys(
 // digit down).  A tenth of the barriers of the bit-by-bit search above.  The keys of a candidate list
 // share their upper digits: a wave first counts the lanes that hold its first lane's digit and adds them
 // with one atomic (twice), and only what is left goes to the histogram lane by lane.
+// LEVELS < 4: only the upper LEVELS digits are worked out, the rest left at zero: a lower bound that at least
+// top_k keys reach (and only as many more as share those digits with the top_k-th largest).
 // All threads of the workgroup must call it.
-template <int N>
+template <int N, int LEVELS = 4>
 __device__ __forceinline__ uint32_t workgroup_kth_of_keys_by_digits(
     const uint32_t (&keys)[N], int top_k, int tid, BoundScratch& scratch)
 {
+    static_assert(LEVELS >= 1 && LEVELS <= 4, "a key has four digits");
     const int lane = tid & (kWaveSize - 1);
     uint32_t prefix = 0;     // the digits found so far, in place
     uint32_t determined = 0; // the bits they occupy
     uint32_t wanted = static_cast<uint32_t>(top_k); // rank among the keys that share those digits
-    for (int level = 0; level < 4; ++level)
+    for (int level = 0; level < LEVELS; ++level)
     {
         const int shift = 24 - 8 * level;
         uint32_t* const bins = scratch.hot_keys + 256 * (level & 1); // alternate levels, alternate bins: one barrier less

@@ -573,7 +573,9 @@ __global__ __launch_bounds__(kScanThreads, (!LOOPED && DTYPE == NCNN_MOE_LOGITS_
             const float ratio = static_cast<float>(a.vocab) / static_cast<float>(kChunk);
             const float root = 0.5f * (kSampleSigmas + sqrtf(kSampleSigmas * kSampleSigmas + 4.0f * static_cast<float>(top_k) / ratio));
             const int sample_rank = static_cast<int>(root * root) + 1;
-            const uint32_t sample_bound = workgroup_kth_of_keys_by_digits(sample_keys, sample_rank, tid, shared.bound);
+            // (the upper 16 bits of the sample's m-th largest: half the selection's rounds, and the few dozen values of
+            // the row that share those bits with it are nothing beside the estimate's own spread)
+            const uint32_t sample_bound = workgroup_kth_of_keys_by_digits<kLaneValues, 2>(sample_keys, sample_rank, tid, shared.bound);
             if (sample_bound != 0u)
             {
                 bound_key = sample_bound;
