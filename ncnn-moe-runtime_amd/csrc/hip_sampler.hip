@@ -360,11 +360,20 @@ int launch_sampler(
             return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
         if (early_cut)
         {
+            // the rows' list, their cuts and the sort's first counting pass: all three need the logits and the options only
             SamplerArgs cut = a;
             cut.leave_wide_rows = 0;
             cut.cut_by_options = 1;
             cut.max_select_top_k = passes.wide_select || batch_geometry.wide ? kSelectTopK : kFastTopK;
+            hipLaunchKernelGGL(full_order_row_list_kernel, dim3(1), dim3(kSortThreads), 0, s->side_stream, cut, rows, s->row_list);
             hipLaunchKernelGGL(full_order_cut_kernel, dim3(rows), dim3(kSortThreads), 0, s->side_stream, cut);
+            cut.row_list = s->row_list;
+            cut.sort_low_digit_skipped = s->skip_low_digit != 0 ? 1u : 0u;
+            cut.sort_parts = sort_parts;
+            cut.sort_tiles_per_part = sort_tiles_per_part;
+            cut.sort_pass = 0;
+            hipLaunchKernelGGL((sort_part_histogram_kernel<NCNN_MOE_LOGITS_F32>), dim3((sort_parts + kHistogramParts - 1) / kHistogramParts, rows),
+                               dim3(kSortThreads), 0, s->side_stream, cut);
             if (hipEventRecord(s->cut_done, s->side_stream) != hipSuccess)
                 return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
         }
@@ -380,7 +389,8 @@ int launch_sampler(
         else
             launch_select<NCNN_MOE_LOGITS_BF16>(batch_geometry, rows, stream, first, 0, s->scatter_segments != 0);
     }
-    const auto launch_spread_sort = [&](SamplerArgs spread, auto dtype_tag, auto pairs_tag) {
+    // first_counted: the first pass's counting kernel has run on the second stream (see early_cut)
+    const auto launch_spread_sort = [&](SamplerArgs spread, auto dtype_tag, auto pairs_tag, bool first_counted) {
         constexpr int kType = decltype(dtype_tag)::value;
         constexpr bool kPairs = decltype(pairs_tag)::value;
         spread.sort_parts = sort_parts;
@@ -389,7 +399,8 @@ int launch_sampler(
         for (int pass = 0; pass < passes; ++pass)
         {
             spread.sort_pass = static_cast<uint32_t>(pass);
-            hipLaunchKernelGGL((sort_part_histogram_kernel<kType>), dim3((sort_parts + kHistogramParts - 1) / kHistogramParts, rows), dim3(kSortThreads), 0, stream, spread);
+            if (pass != 0 || !first_counted)
+                hipLaunchKernelGGL((sort_part_histogram_kernel<kType>), dim3((sort_parts + kHistogramParts - 1) / kHistogramParts, rows), dim3(kSortThreads), 0, stream, spread);
             if (pass == 0 && !kPairs) // (keys alone: the first pass need not keep the order of equal digits)
                 hipLaunchKernelGGL((sort_part_scatter_kernel<kType, kPairs, true>), dim3(sort_parts, rows), dim3(kSortThreads), 0, stream, spread);
             else
@@ -403,22 +414,28 @@ int launch_sampler(
         const bool runs = dtype == NCNN_MOE_LOGITS_BF16 && !want_distribution;
         // (keys alone, sorted in part or whole by the spread sort: its pass over the lowest byte is left out)
         a.sort_low_digit_skipped = !leftovers && partial_sort && s->skip_low_digit != 0 ? 1u : 0u;
-        if (!leftovers && !runs)
+        const bool listed_early = !leftovers && partial_sort && early_cut;
+        if (listed_early)
+        {
+            // (listed, cut and counted for the first pass on the second stream)
+            a.row_list = s->row_list;
+            a.rows_listed_by_options = 1;
+            (void)hipStreamWaitEvent(stream, s->cut_done, 0);
+        }
+        else if (!leftovers && !runs)
         {
             // (the kernels over a (parts, rows) grid find their rows in a list)
             hipLaunchKernelGGL(full_order_row_list_kernel, dim3(1), dim3(kSortThreads), 0, stream, a, rows, s->row_list);
             a.row_list = s->row_list;
         }
-        if (!leftovers && partial_sort && early_cut)
-            (void)hipStreamWaitEvent(stream, s->cut_done, 0);
-        else if (!leftovers && partial_sort)
+        if (!leftovers && partial_sort && !early_cut)
             hipLaunchKernelGGL(full_order_cut_kernel, dim3(rows), dim3(kSortThreads), 0, stream, a);
         // the token indices ride along with the keys only when the whole distribution is exported
         const auto sort_rows = [&](auto dtype_tag, auto pairs_tag) {
             constexpr int kType = decltype(dtype_tag)::value;
             constexpr bool kPairs = decltype(pairs_tag)::value;
             if (spread_sort)
-                launch_spread_sort(a, dtype_tag, pairs_tag);
+                launch_spread_sort(a, dtype_tag, pairs_tag, listed_early);
             else
                 hipLaunchKernelGGL((general_sort_kernel<kType, kPairs>), dim3(rows), dim3(kSortThreads), 0, stream, a);
         };
@@ -1223,6 +1240,8 @@ int ncnn_moe_hip_sampler_debug_disordered_rows(ncnn_moe_hip_sampler* s, uint32_t
     SAMPLER_HIP_CHECK(s, hipSetDevice(s->device));
     SAMPLER_HIP_CHECK(s, hipStreamSynchronize(s->stream));
     SAMPLER_HIP_CHECK(s, hipMemcpy(flags, s->sort_cuts + 3 * static_cast<size_t>(s->max_rows), rows * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    for (uint32_t row = 0; row < rows; ++row)
+        flags[row] &= 1u; // (bit 1 marks the rows that were in no list of the call)
     return NCNN_MOE_SAMPLER_SUCCESS;
 }
 

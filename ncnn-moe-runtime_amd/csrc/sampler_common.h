@@ -87,9 +87,13 @@ struct SamplerArgs
     // row to see them all, and out of order): that row is sorted whole by the launch behind this one.
     uint32_t* disordered_rows;
     uint32_t sort_low_digit_skipped;
-    // full_order_cut_kernel runs beside the first select: it takes the rows that no select pass serves by their
-    // options (widest window: max_select_top_k), not by row_state, which that select is still writing
+    // full_order_row_list_kernel, full_order_cut_kernel and the sort's first counting pass run beside the first
+    // select: they take the rows that no select pass serves by their options (widest window: max_select_top_k),
+    // not by row_state, which that select is still writing.  The cut kernel then marks every other row in
+    // disordered_rows (bit 1): should a select kernel hand such a row on after all (ties beyond its list), it is in
+    // no list, and the replay (rows_listed_by_options = 1) leaves it to the launch behind it like a disordered one.
     uint32_t cut_by_options;
+    uint32_t rows_listed_by_options;
     // The wide select takes the bound of a window wider than kTwoKeyBoundTopK from a sample of the whole row (1)
     // or from the row's first chunk alone (0); same results either way.
     uint32_t wide_sampled_bound;

@@ -60,7 +60,15 @@ __global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(Sampl
     for (uint32_t first = 0; first < rows; first += kSortThreads)
     {
         const uint32_t row = first + static_cast<uint32_t>(tid);
-        const bool mine = row < rows && a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
+        bool mine = false;
+        if (row < rows && a.cut_by_options != 0u)
+        {
+            uint32_t effective_k = 0;
+            int status = NCNN_MOE_ROW_OK;
+            mine = resolve_row_mode(a.params[row], a.vocab, a.max_select_top_k, a.force_general, effective_k, status) == kModeGeneral;
+        }
+        else if (row < rows)
+            mine = a.row_state[row] == kRowNeedsGeneral && !left_to_the_wide_select(a, row);
         const uint64_t mask = __builtin_amdgcn_ballot_w64(mine);
         if (lane == 0)
             wave_totals[wave] = static_cast<uint32_t>(__popcll(mask));
@@ -127,7 +135,7 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
         {
             a.sort_last_keys[row] = 0xffffffffu;
             a.sort_lengths[row] = a.vocab;
-            a.disordered_rows[row] = 0u;
+            a.disordered_rows[row] = (a.cut_by_options != 0u && !served) ? 2u : 0u; // (2: in no list of this call)
         }
     };
     if (!served || !(temperature > 0.0f))
@@ -1624,8 +1632,10 @@ __global__ __launch_bounds__(kReplayThreads) void general_replay_kernel(SamplerA
     }
     else
     {
-        // (a row whose keys the terms kernel could not put in order: the launch behind this one sorts it whole)
-        if (a.sort_low_digit_skipped != 0u && a.disordered_rows[row] != 0u)
+        // (a row whose keys the terms kernel could not put in order, or one that a select kernel handed on after the
+        // rows were listed by their options: the launch behind this one sorts it whole)
+        const uint32_t unordered = (a.sort_low_digit_skipped != 0u || a.rows_listed_by_options != 0u) ? a.disordered_rows[row] : 0u;
+        if ((a.sort_low_digit_skipped != 0u && (unordered & 1u) != 0u) || (a.rows_listed_by_options != 0u && (unordered & 2u) != 0u))
         {
             if (tid == 0)
             {
