@@ -282,3 +282,35 @@ def test_random_rows_three_passes_and_four():
         cpu = parity_util.run_oracle(logits, params, uniforms)
         parity_util.assert_results_match(three, cpu, "f32", context)
         assert three.tobytes() == four.tobytes(), context
+
+
+def test_rows_that_a_select_hands_on_beside_listed_rows():
+    """The rows of the partial sort are listed, cut and counted by their options while the first select is still
+    running.  A row with a Top-K window whose select kernel cannot finish it (hundreds or thousands of equal logits at
+    the window's edge, more than its list holds) is pending afterwards and in no list: the walk leaves it to the
+    second launch, which sorts it whole.  Rows of every kind in one call, 300 rows (whole-row select) and 40 (split)."""
+    rng = np.random.default_rng(8128)
+    vocab = 129280
+    for rows in (300, 40):
+        logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+        kind = np.arange(rows) % 5   # 0, 1: no window (listed) | 2: window 20 | 3: window 1000 | 4: window 50 with ties
+        logits[kind == 4] = np.round(logits[kind == 4] / 2.0) * 2.0  # hundreds of equal logits at the window's edge
+        logits[3::10] = np.round(logits[3::10] * 2.0) / 2.0        # ... also for half of the wide windows
+        params = hip_sampler.make_params(rows, 1.0, 0, 0.95, 0.0)
+        params["temperature"] = rng.uniform(0.3, 1.4, size=rows).astype(np.float32)
+        params["top_k"] = np.array([0, 0, 20, 1000, 50], dtype=np.uint32)[kind]
+        uniforms = rng.random(rows, dtype=np.float32)
+        context = "rows handed on beside listed rows, %d rows" % rows
+        _announce(context)
+        with hip_sampler.HipSampler(rows, vocab, testing=True) as handle:
+            handle.upload_logits(logits)
+            early = handle.sample(params, uniforms, None)
+            flagged = handle.disordered_rows(rows)
+            again = handle.sample(params, uniforms, None)
+        cpu = parity_util.run_oracle(logits, params, uniforms)
+        parity_util.assert_results_match(early, cpu, "f32", context)
+        assert early.tobytes() == again.tobytes(), context
+        general = (early["flags"] & hip_sampler.FLAG_GENERAL_PATH) != 0
+        assert general[kind <= 1].all() and general[kind == 4].all(), context      # listed rows and rows handed on
+        assert not general[kind == 2].any(), context
+        assert not flagged[kind >= 2].any(), context                               # (the hook names disordered rows only)
