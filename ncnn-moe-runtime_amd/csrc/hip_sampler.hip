@@ -6,6 +6,7 @@
 #include "sampler_verify.h"
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <algorithm>
 #include <cmath>
@@ -372,10 +373,20 @@ int launch_sampler(
             cut.sort_parts = sort_parts;
             cut.sort_tiles_per_part = sort_tiles_per_part;
             cut.sort_pass = 0;
-            hipLaunchKernelGGL((sort_part_histogram_kernel<NCNN_MOE_LOGITS_F32>), dim3((sort_parts + kHistogramParts - 1) / kHistogramParts, rows),
-                               dim3(kSortThreads), 0, s->side_stream, cut);
-            if (hipEventRecord(s->cut_done, s->side_stream) != hipSuccess)
-                return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
+            // (the event rides on the kernel's own completion signal where the stream is not being captured: a record
+            // of its own is one more packet for the caller's stream to wait behind)
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            (void)hipStreamIsCapturing(stream, &capturing);
+            if (capturing == hipStreamCaptureStatusNone)
+                hipExtLaunchKernelGGL((sort_part_histogram_kernel<NCNN_MOE_LOGITS_F32>), dim3((sort_parts + kHistogramParts - 1) / kHistogramParts, rows),
+                                      dim3(kSortThreads), 0, s->side_stream, nullptr, s->cut_done, 0, cut);
+            else
+            {
+                hipLaunchKernelGGL((sort_part_histogram_kernel<NCNN_MOE_LOGITS_F32>), dim3((sort_parts + kHistogramParts - 1) / kHistogramParts, rows),
+                                   dim3(kSortThreads), 0, s->side_stream, cut);
+                if (hipEventRecord(s->cut_done, s->side_stream) != hipSuccess)
+                    return fail(s, NCNN_MOE_SAMPLER_HIP_ERROR, "fork to the second stream failed");
+            }
         }
         if (early_wide)
             launch_wide(s->side_stream, 2);
