@@ -366,8 +366,8 @@ int launch_sampler(
             cut.leave_wide_rows = 0;
             cut.cut_by_options = 1;
             cut.max_select_top_k = passes.wide_select || batch_geometry.wide ? kSelectTopK : kFastTopK;
-            hipLaunchKernelGGL(full_order_row_list_kernel, dim3(1), dim3(kSortThreads), 0, s->side_stream, cut, rows, s->row_list);
-            hipLaunchKernelGGL(full_order_cut_kernel, dim3(rows), dim3(kSortThreads), 0, s->side_stream, cut);
+            cut.row_list_out = s->row_list; // (one more workgroup, which lists the rows)
+            hipLaunchKernelGGL(full_order_cut_kernel, dim3(rows + 1), dim3(kSortThreads), 0, s->side_stream, cut);
             cut.row_list = s->row_list;
             cut.sort_low_digit_skipped = s->skip_low_digit != 0 ? 1u : 0u;
             cut.sort_parts = sort_parts;

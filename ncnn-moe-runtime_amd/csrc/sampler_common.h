@@ -94,6 +94,8 @@ struct SamplerArgs
     // no list, and the replay (rows_listed_by_options = 1) leaves it to the launch behind it like a disordered one.
     uint32_t cut_by_options;
     uint32_t rows_listed_by_options;
+    // ... and the list is written by one more workgroup of full_order_cut_kernel (the one behind the rows'), beside the others
+    uint32_t* row_list_out;
     // The wide select takes the bound of a window wider than kTwoKeyBoundTopK from a sample of the whole row (1)
     // or from the row's first chunk alone (0); same results either way.
     uint32_t wide_sampled_bound;

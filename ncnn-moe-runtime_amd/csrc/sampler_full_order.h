@@ -50,7 +50,7 @@ __device__ __forceinline__ uint32_t sort_last_key(const SamplerArgs& a, uint32_t
 }
 
 // Lists the rows that the full-order kernels serve (see SamplerArgs::row_list).  One workgroup.
-__global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(SamplerArgs a, uint32_t rows, uint32_t* list)
+__device__ __forceinline__ void list_full_order_rows(const SamplerArgs& a, uint32_t rows, uint32_t* list)
 {
     __shared__ uint32_t wave_totals[kSortWaves];
     const int tid = threadIdx.x;
@@ -90,6 +90,11 @@ __global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(Sampl
         list[0] = listed;
 }
 
+__global__ __launch_bounds__(kSortThreads) void full_order_row_list_kernel(SamplerArgs a, uint32_t rows, uint32_t* list)
+{
+    list_full_order_rows(a, rows, list);
+}
+
 // How much of a full-order fp32 row needs sorting.  The sampler's sums add the row's terms exp(logit/T - max)
 // in descending order, and a term below half an ulp of the sum it meets leaves that sum as it is: behind some
 // point of the sorted row nothing moves any sum, and what lies there need not be in order (nor be sorted at
@@ -115,6 +120,8 @@ __global__ __launch_bounds__(kSortThreads) void full_order_cut_kernel(SamplerArg
 {
     static_assert(kCutSample == 4u * kSortThreads && kCutBuckets == 4 * kSortThreads, "four loads and four buckets a thread");
     const uint32_t row = blockIdx.x;
+    if (row == a.rows)
+        return list_full_order_rows(a, a.rows, a.row_list_out); // (the workgroup behind the rows', where the host asks for one)
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
     const int wave = tid >> 6;
